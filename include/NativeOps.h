@@ -1,0 +1,145 @@
+// class NativeOps - the drop-in surface of the legacy op-execution path.
+//
+// Same class name, member names, argument order and POD argument types as the reference's
+// blas/NativeOps.h, restricted to the members on the hot path (transform, pairwise, broadcast, reduce,
+// index-reduce, summary-stats, random) and the lifecycle members a host needs around them.  A JavaCPP
+// binding generated against the reference header resolves these members to the same Itanium-mangled
+// symbols in libnd4j_amd.so.  Members of the reference class that are outside this path are not
+// declared here.
+//
+// Calling convention = the reference's CUDA backend (blas/cuda/NativeOps.cu):
+//   * data pointers, shapeInfo arguments, `dimension` and `extraParams` are DEVICE pointers;
+//   * extraPointers[0] host xShapeInfo, [1] the HIP stream handle by value, [2] device id,
+//     [3] allocation scratch (unused here), [4] reduction scratch (unused here), [5] host-visible scalar
+//     result (unused: scalars are returned by value after a stream synchronise), [7] host yShapeInfo,
+//     [8] host zShapeInfo, [9] host TAD shapeInfo, [10] device TAD shapeInfo, [11] device TAD offsets,
+//     [12]/[13] device TAD shapeInfo/offsets of the result (broadcast);
+//   * array results are enqueued on the stream and the call returns; scalar-returning members
+//     synchronise the stream.
+//   Missing host copies ([0],[7],[8],[9] null) are fetched from the device pointers, and missing TAD
+//   tables are computed and cached by the library, at the price of a stream synchronise.
+#pragma once
+
+#include "nd4j_types.h"
+
+#ifndef ND4J_EXPORT
+#define ND4J_EXPORT __attribute__((visibility("default")))
+#endif
+
+// One block of members per data type: SUFFIX in {Float, Half, Double}, T in {float, float16, double},
+// R the scalar return type (float for Float and Half, double for Double).
+#define ND4J_EXEC_MEMBERS(SUFFIX, T, R)                                                                         \
+    /* reference: blas/NativeOps.h:544-602 (Float/Half), 80-113 (Double) */                                      \
+    R execIndexReduceScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,          \
+                                    T *extraParams);                                                             \
+    void execIndexReduce##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,             \
+                                 T *extraParams, T *result, Nd4jLong *resultShapeInfoBuffer, int *dimension,     \
+                                 int dimensionLength);                                                           \
+    /* reference: blas/NativeOps.h:615-649, 115-139 */                                                           \
+    void execBroadcast##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *y,         \
+                               Nd4jLong *yShapeInfo, T *result, Nd4jLong *resultShapeInfo, int *dimension,       \
+                               int dimensionLength);                                                             \
+    /* reference: blas/NativeOps.h:665-798, 141-210: strided, indexed (a no-op in both reference back ends:    \
+       blas/cuda/NativeOps.cu:1928-1960) and shaped overloads */                                                 \
+    void execPairwiseTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong xStride, T *y,    \
+                                       Nd4jLong yStride, T *result, Nd4jLong resultStride, T *extraParams,       \
+                                       Nd4jLong n);                                                              \
+    void execPairwiseTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong *xShapeInfo,      \
+                                       T *y, Nd4jLong *yShapeInfo, T *result, Nd4jLong *resultShapeInfo,         \
+                                       T *extraParams, Nd4jLong *xIndexes, Nd4jLong *yIndexes,                   \
+                                       Nd4jLong *resultIndexes);                                                 \
+    void execPairwiseTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong *xShapeInfo,      \
+                                       T *y, Nd4jLong *yShapeInfo, T *result, Nd4jLong *resultShapeInfo,         \
+                                       T *extraParams);                                                          \
+    /* reference: blas/NativeOps.h:809-906, 212-250 */                                                           \
+    void execReduce##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *extraParams,  \
+                            T *result, Nd4jLong *resultShapeInfo);                                               \
+    void execReduce##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *extraParams,  \
+                            T *result, Nd4jLong *resultShapeInfo, int *dimension, int dimensionLength);          \
+    R execReduceScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,               \
+                               T *extraParams);                                                                  \
+    /* reference: blas/NativeOps.h:1223-1325, 438-490 */                                                         \
+    R execSummaryStatsScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,         \
+                                     T *extraParams, bool biasCorrected);                                        \
+    void execSummaryStats##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,            \
+                                  T *extraParams, T *result, Nd4jLong *resultShapeInfo, bool biasCorrected);     \
+    void execSummaryStats##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,            \
+                                  T *extraParams, T *result, Nd4jLong *resultShapeInfoBuffer, int *dimension,    \
+                                  int dimensionLength, bool biasCorrected);                                      \
+    /* reference: blas/NativeOps.h:1337-1443, 492-542: strided, shaped and indexed (no-op:                      \
+       blas/cuda/NativeOps.cu:3598-3612) overloads */                                                            \
+    void execTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong xStride, T *result,       \
+                               Nd4jLong resultStride, T *extraParams, Nd4jLong n);                               \
+    void execTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong *xShapeInfo, T *result,   \
+                               Nd4jLong *resultShapeInfo, T *extraParams);                                       \
+    void execTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong *xShapeInfo, T *result,   \
+                               Nd4jLong *resultShapeInfo, T *extraParams, Nd4jLong *xIndexes,                    \
+                               Nd4jLong *resultIndexes);                                                         \
+    /* reference: blas/NativeOps.h:2327-2498: (z), (x,y,z) and (x,z) overloads; `state` is the pointer        \
+       returned by initRandom */                                                                                 \
+    void execRandom##SUFFIX(Nd4jPointer *extraPointers, int opNum, Nd4jPointer state, T *z,                     \
+                            Nd4jLong *zShapeBuffer, T *extraArguments);                                          \
+    void execRandom##SUFFIX(Nd4jPointer *extraPointers, int opNum, Nd4jPointer state, T *x,                     \
+                            Nd4jLong *xShapeBuffer, T *y, Nd4jLong *yShapeBuffer, T *z, Nd4jLong *zShapeBuffer,  \
+                            T *extraArguments);                                                                  \
+    void execRandom##SUFFIX(Nd4jPointer *extraPointers, int opNum, Nd4jPointer state, T *x,                     \
+                            Nd4jLong *xShapeBuffer, T *z, Nd4jLong *zShapeBuffer, T *extraArguments);
+
+class ND4J_EXPORT NativeOps {
+public:
+    ND4J_EXEC_MEMBERS(Float, float, float)
+    ND4J_EXEC_MEMBERS(Half, float16, float)
+    ND4J_EXEC_MEMBERS(Double, double, double)
+
+    // ---- RNG lifecycle, reference: blas/NativeOps.h:2510-2539 ------------------------------------
+    // extraPointers[0] = host u64 buffer (bufferSize entries), ptrToBuffer = device u64 buffer
+    // (blas/cuda/NativeOps.cu:5384-5407).
+    Nd4jPointer initRandom(Nd4jPointer *extraPointers, long seed, long bufferSize, Nd4jPointer ptrToBuffer);
+    void refreshBuffer(Nd4jPointer *extraPointers, long seed, Nd4jPointer ptrRandom);
+    void reSeedBuffer(Nd4jPointer *extraPointers, long seed, Nd4jPointer ptrRandom);
+    void destroyRandom(Nd4jPointer ptrRandom);
+
+    // ---- shape service, reference: blas/NativeOps.h:1880-1884 (host side in both back ends) -------
+    void tadOnlyShapeInfo(Nd4jLong *xShapeInfo, int *dimension, int dimensionLength, Nd4jLong *targetBuffer,
+                          Nd4jLong *offsetsBuffer);
+
+    // ---- device / stream / memory lifecycle, reference: blas/NativeOps.h:1607-1864 ----------------
+    void initializeDevicesAndFunctions();
+    Nd4jPointer mallocHost(Nd4jLong memorySize, int flags);
+    Nd4jPointer mallocDevice(Nd4jLong memorySize, Nd4jPointer ptrToDeviceId, int flags);
+    int freeHost(Nd4jPointer pointer);
+    int freeDevice(Nd4jPointer pointer, Nd4jPointer ptrToDeviceId);
+    int ompGetMaxThreads();
+    int ompGetNumThreads();
+    void setOmpNumThreads(int threads);
+    void setOmpMinThreads(int threads);
+    Nd4jPointer createContext();
+    Nd4jPointer createStream();
+    Nd4jPointer createEvent();
+    int registerEvent(Nd4jPointer event, Nd4jPointer stream);
+    int destroyEvent(Nd4jPointer event);
+    int setDevice(Nd4jPointer ptrToDeviceId);
+    int getDevice();
+    int streamSynchronize(Nd4jPointer stream);
+    int eventSynchronize(Nd4jPointer event);
+    Nd4jLong getDeviceFreeMemory(Nd4jPointer ptrToDeviceId);
+    Nd4jLong getDeviceTotalMemory(Nd4jPointer ptrToDeviceId);
+    int getDeviceMajor(Nd4jPointer ptrToDeviceId);
+    int getDeviceMinor(Nd4jPointer ptrToDeviceId);
+    const char *getDeviceName(Nd4jPointer ptrToDeviceId);
+    // flags: 0 host-to-host, 1 host-to-device, 2 device-to-host, 3 device-to-device; `reserved` is the stream
+    int memcpy(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved);
+    int memcpyAsync(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved);
+    int memset(Nd4jPointer dst, int value, Nd4jLong size, int flags, Nd4jPointer reserved);
+    int memsetAsync(Nd4jPointer dst, int value, Nd4jLong size, int flags, Nd4jPointer reserved);
+    int memcpyConstantAsync(Nd4jLong dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved);
+    Nd4jPointer getConstantSpace();
+    int getAvailableDevices();
+    void enableDebugMode(bool reallyEnable);
+    void enableVerboseMode(bool reallyEnable);
+    void setGridLimit(int gridSize);
+    void setElementThreshold(int num);
+    void setTADThreshold(int num);
+};
+
+#undef ND4J_EXEC_MEMBERS

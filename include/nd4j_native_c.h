@@ -1,0 +1,157 @@
+/* C ABI of libnd4j_amd.so: one extern "C" entry point per NativeOps member on the legacy op-execution
+ * path, for bindings that cannot call C++ members (ctypes, cgo, N-API ...).  Each function forwards to
+ * the member of the same name in include/NativeOps.h; where the C++ class overloads a name, the C name
+ * carries a suffix (Strided / Indexed / Full / XZ / XYZ).  Arguments are plain pointers and integers;
+ * their meaning, the extraPointers convention and the synchronisation behaviour are those documented in
+ * include/NativeOps.h.
+ *
+ * Reference declarations replaced (blas/NativeOps.h, Float / Half / Double):
+ *   execIndexReduceScalar*  544-573, 80-94        execIndexReduce*      576-602, 96-113
+ *   execBroadcast*          615-649, 115-139      execPairwiseTransform* 665-798, 141-210
+ *   execReduce*             809-876, 212-244      execReduceScalar*     886-906, 246-250
+ *   execSummaryStatsScalar* 1223-1242, 438-451    execSummaryStats*     1253-1325, 453-490
+ *   execTransform*          1337-1443, 492-542    execRandom*           2327-2498
+ *   initRandom/refreshBuffer/reSeedBuffer/destroyRandom 2510-2539        tadOnlyShapeInfo 1880-1884
+ *   device, stream, event and memory members 1607-1864
+ *
+ * Error convention: the reference throws std::runtime_error on device failures; a C ABI cannot, so a
+ * failed call records a message retrievable with nd4j_lastError() (empty string when the last call on
+ * this thread succeeded) and returns 0 / NULL / leaves the output untouched.
+ */
+#ifndef ND4J_NATIVE_C_H
+#define ND4J_NATIVE_C_H
+
+#include "nd4j_types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
+const char *nd4j_lastError(void);
+
+#define ND4J_C_EXEC(SUFFIX, T, R)                                                                                 \
+    R nd4j_execIndexReduceScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,       \
+                                         T *extraParams);                                                         \
+    void nd4j_execIndexReduce##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,          \
+                                      T *extraParams, T *result, Nd4jLong *resultShapeInfoBuffer, int *dimension, \
+                                      int dimensionLength);                                                       \
+    void nd4j_execBroadcast##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *y,      \
+                                    Nd4jLong *yShapeInfo, T *result, Nd4jLong *resultShapeInfo, int *dimension,   \
+                                    int dimensionLength);                                                         \
+    void nd4j_execPairwiseTransform##SUFFIX##Strided(Nd4jPointer *extraPointers, int opNum, T *dx,                \
+                                                     Nd4jLong xStride, T *y, Nd4jLong yStride, T *result,         \
+                                                     Nd4jLong resultStride, T *extraParams, Nd4jLong n);          \
+    void nd4j_execPairwiseTransform##SUFFIX##Indexed(Nd4jPointer *extraPointers, int opNum, T *dx,                \
+                                                     Nd4jLong *xShapeInfo, T *y, Nd4jLong *yShapeInfo, T *result, \
+                                                     Nd4jLong *resultShapeInfo, T *extraParams,                   \
+                                                     Nd4jLong *xIndexes, Nd4jLong *yIndexes,                      \
+                                                     Nd4jLong *resultIndexes);                                    \
+    void nd4j_execPairwiseTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong *xShapeInfo,   \
+                                            T *y, Nd4jLong *yShapeInfo, T *result, Nd4jLong *resultShapeInfo,     \
+                                            T *extraParams);                                                      \
+    void nd4j_execReduce##SUFFIX##Full(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,         \
+                                       T *extraParams, T *result, Nd4jLong *resultShapeInfo);                     \
+    void nd4j_execReduce##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,               \
+                                 T *extraParams, T *result, Nd4jLong *resultShapeInfo, int *dimension,            \
+                                 int dimensionLength);                                                            \
+    R nd4j_execReduceScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,            \
+                                    T *extraParams);                                                              \
+    R nd4j_execSummaryStatsScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,      \
+                                          T *extraParams, int biasCorrected);                                     \
+    void nd4j_execSummaryStats##SUFFIX##Full(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,   \
+                                             T *extraParams, T *result, Nd4jLong *resultShapeInfo,                \
+                                             int biasCorrected);                                                  \
+    void nd4j_execSummaryStats##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,         \
+                                       T *extraParams, T *result, Nd4jLong *resultShapeInfoBuffer,                \
+                                       int *dimension, int dimensionLength, int biasCorrected);                   \
+    void nd4j_execTransform##SUFFIX##Strided(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong xStride,      \
+                                             T *result, Nd4jLong resultStride, T *extraParams, Nd4jLong n);       \
+    void nd4j_execTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong *xShapeInfo,           \
+                                    T *result, Nd4jLong *resultShapeInfo, T *extraParams);                        \
+    void nd4j_execTransform##SUFFIX##Indexed(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong *xShapeInfo,  \
+                                             T *result, Nd4jLong *resultShapeInfo, T *extraParams,                \
+                                             Nd4jLong *xIndexes, Nd4jLong *resultIndexes);                        \
+    void nd4j_execRandom##SUFFIX(Nd4jPointer *extraPointers, int opNum, Nd4jPointer state, T *z,                  \
+                                 Nd4jLong *zShapeBuffer, T *extraArguments);                                      \
+    void nd4j_execRandom##SUFFIX##XYZ(Nd4jPointer *extraPointers, int opNum, Nd4jPointer state, T *x,             \
+                                      Nd4jLong *xShapeBuffer, T *y, Nd4jLong *yShapeBuffer, T *z,                 \
+                                      Nd4jLong *zShapeBuffer, T *extraArguments);                                 \
+    void nd4j_execRandom##SUFFIX##XZ(Nd4jPointer *extraPointers, int opNum, Nd4jPointer state, T *x,              \
+                                     Nd4jLong *xShapeBuffer, T *z, Nd4jLong *zShapeBuffer, T *extraArguments);
+
+ND4J_C_EXEC(Float, float, float)
+ND4J_C_EXEC(Half, float16, float)
+ND4J_C_EXEC(Double, double, double)
+#undef ND4J_C_EXEC
+
+Nd4jPointer nd4j_initRandom(Nd4jPointer *extraPointers, long seed, long bufferSize, Nd4jPointer ptrToBuffer);
+void nd4j_refreshBuffer(Nd4jPointer *extraPointers, long seed, Nd4jPointer ptrRandom);
+void nd4j_reSeedBuffer(Nd4jPointer *extraPointers, long seed, Nd4jPointer ptrRandom);
+void nd4j_destroyRandom(Nd4jPointer ptrRandom);
+
+void nd4j_tadOnlyShapeInfo(Nd4jLong *xShapeInfo, int *dimension, int dimensionLength, Nd4jLong *targetBuffer,
+                           Nd4jLong *offsetsBuffer);
+
+void nd4j_initializeDevicesAndFunctions(void);
+Nd4jPointer nd4j_mallocHost(Nd4jLong memorySize, int flags);
+Nd4jPointer nd4j_mallocDevice(Nd4jLong memorySize, Nd4jPointer ptrToDeviceId, int flags);
+int nd4j_freeHost(Nd4jPointer pointer);
+int nd4j_freeDevice(Nd4jPointer pointer, Nd4jPointer ptrToDeviceId);
+int nd4j_ompGetMaxThreads(void);
+int nd4j_ompGetNumThreads(void);
+void nd4j_setOmpNumThreads(int threads);
+void nd4j_setOmpMinThreads(int threads);
+Nd4jPointer nd4j_createContext(void);
+Nd4jPointer nd4j_createStream(void);
+Nd4jPointer nd4j_createEvent(void);
+int nd4j_registerEvent(Nd4jPointer event, Nd4jPointer stream);
+int nd4j_destroyEvent(Nd4jPointer event);
+int nd4j_setDevice(Nd4jPointer ptrToDeviceId);
+int nd4j_getDevice(void);
+int nd4j_streamSynchronize(Nd4jPointer stream);
+int nd4j_eventSynchronize(Nd4jPointer event);
+Nd4jLong nd4j_getDeviceFreeMemory(Nd4jPointer ptrToDeviceId);
+Nd4jLong nd4j_getDeviceTotalMemory(Nd4jPointer ptrToDeviceId);
+int nd4j_getDeviceMajor(Nd4jPointer ptrToDeviceId);
+int nd4j_getDeviceMinor(Nd4jPointer ptrToDeviceId);
+const char *nd4j_getDeviceName(Nd4jPointer ptrToDeviceId);
+int nd4j_memcpy(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved);
+int nd4j_memcpyAsync(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved);
+int nd4j_memset(Nd4jPointer dst, int value, Nd4jLong size, int flags, Nd4jPointer reserved);
+int nd4j_memsetAsync(Nd4jPointer dst, int value, Nd4jLong size, int flags, Nd4jPointer reserved);
+int nd4j_memcpyConstantAsync(Nd4jLong dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved);
+Nd4jPointer nd4j_getConstantSpace(void);
+int nd4j_getAvailableDevices(void);
+void nd4j_enableDebugMode(int reallyEnable);
+void nd4j_enableVerboseMode(int reallyEnable);
+void nd4j_setGridLimit(int gridSize);
+void nd4j_setElementThreshold(int num);
+void nd4j_setTADThreshold(int num);
+
+/* ---- measurement and parity aids: no counterpart in the reference ---------------------------------- */
+/* out[i] = RandomBuffer::getElement(start + i) for the generator `ptrRandom`, computed on the device with
+ * the state as it stands (reference for the values: include/helpers/helper_generator.h:185-220). `out` is
+ * a device pointer. */
+void nd4j_amd_rngDump(Nd4jPointer *extraPointers, Nd4jPointer ptrRandom, Nd4jLong start, Nd4jLong n,
+                      unsigned long long *out);
+/* state[0..4] = size, offset, seed, generation, amplifier of the generator */
+void nd4j_amd_rngState(Nd4jPointer ptrRandom, Nd4jLong *state);
+/* HIP events with timing enabled, to time work on the stream the ops are launched on */
+Nd4jPointer nd4j_amd_timerCreate(void);
+int nd4j_amd_timerRecord(Nd4jPointer timer, Nd4jPointer stream);
+float nd4j_amd_timerElapsedMs(Nd4jPointer start, Nd4jPointer stop);
+int nd4j_amd_timerDestroy(Nd4jPointer timer);
+/* plain device-to-device copy kernel of `bytes` bytes (16-byte vectors): the yardstick against which
+ * hardware traffic counters are scaled */
+void nd4j_amd_copyKernel(Nd4jPointer *extraPointers, void *dst, const void *src, Nd4jLong bytes);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
+#ifdef __cplusplus
+}
+#endif
+#endif

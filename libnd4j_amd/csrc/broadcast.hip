@@ -1,0 +1,59 @@
+// Broadcast family: z[tad][f] = op(x[tad][f], y[f]).  Reference loop: include/loops/cpu/broadcasting.cpp:42-156.
+#include "elementwise.cuh"
+#include "launch.h"
+
+namespace nd4j_amd {
+
+template <typename T> struct BroadcastBody {
+    template <int KIND> struct Run {
+        static bool run(hipStream_t s, const T *x, const T *y, T *z, const BroadcastPlan &pl) {
+            typedef Broadcast2F<KIND> F;
+            if (pl.numTads <= 0 || pl.tadLength <= 0) return true;
+            if (pl.kind == BroadcastPlan::ROW) {
+                constexpr int VEC = Pack<T>::N;
+                Long vecsPerTad = (pl.tadLength + VEC - 1) / VEC;
+                int gx = (int)((vecsPerTad + kBlock - 1) / kBlock);
+                Long wantY = (Long)kGridCap / gx;
+                if (wantY < 1) wantY = 1;
+                // at least 4 TADs per block so the y registers are reused
+                Long gy = pl.numTads / 4;
+                if (gy < 1) gy = 1;
+                if (gy > wantY) gy = wantY;
+                if (gy > 65535) gy = 65535;
+                int aligned = (((uintptr_t)x | (uintptr_t)z) & 15) == 0 ? 1 : 0;
+                hipLaunchKernelGGL((bcRowKernel<T, F>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
+                                   pl.zOffsets, pl.tadLength, pl.numTads, aligned);
+            } else if (pl.kind == BroadcastPlan::COL) {
+                int gx = (int)((pl.numTads + kBlock - 1) / kBlock);
+                Long gy = (Long)kGridCap / gx;
+                if (gy < 1) gy = 1;
+                if (gy > pl.tadLength) gy = pl.tadLength;
+                if (gy > 65535) gy = 65535;
+                hipLaunchKernelGGL((bcColKernel<T, F>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
+                                   pl.zOffsets, pl.tadLength, pl.numTads, pl.tadEws, pl.yEws, pl.zEws);
+            } else {
+                int grid = gridFor(pl.numTads, 1, kGridCap);
+                hipLaunchKernelGGL((bcGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, pl.xm, y, pl.ym, z, pl.zm,
+                                   pl.xOffsets, pl.zOffsets, pl.tadLength, pl.numTads);
+            }
+            return true;
+        }
+    };
+};
+
+template <typename T>
+bool launchBroadcast(hipStream_t s, int opNum, const T *x, const T *y, T *z, const BroadcastPlan &plan) {
+    int kind = broadcastKind(opNum);
+    if (kind == B_Invalid) return false;
+    // only kinds that appear in the broadcast table are instantiated (B_Add .. B_TruncateDiv)
+    return dispatchSeq<BroadcastBody<T>::template Run>(kind, std::make_integer_sequence<int, B_TruncateDiv + 1>{}, s, x, y,
+                                                       z, plan);
+}
+
+#define INST(T) template bool launchBroadcast<T>(hipStream_t, int, const T *, const T *, T *, const BroadcastPlan &);
+INST(float)
+INST(float16)
+INST(double)
+#undef INST
+
+}  // namespace nd4j_amd

@@ -1,0 +1,23 @@
+#!/bin/bash
+# Builds libnd4j_amd.so (gfx950) in-tree from the sources in this directory.  Usage: build.sh [-jN]
+set -e
+cd "$(dirname "$0")"
+JOBS=${1:--j8}
+OUT=../libnd4j_amd.so
+OBJ=build
+mkdir -p $OBJ
+HIPFLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -ffp-contract=off -fvisibility=hidden -Xclang -target-feature -Xclang -packed-fp32-ops -Wno-unused-command-line-argument"
+SRCS="transform.hip pairwise.hip broadcast.hip reduce.hip indexreduce.hip summarystats.hip random.hip native_ops.cpp native_reduce.cpp native_random.cpp runtime.cpp c_api.cpp"
+cat > $OBJ/Makefile <<MK
+OBJS := \$(addsuffix .o,\$(basename $SRCS))
+all: ../$OUT
+../$OUT: \$(OBJS)
+	hipcc --offload-arch=gfx950 -shared -fPIC -o \$@ \$(OBJS)
+%.o: ../%.hip \$(wildcard ../*.h ../*.cuh ../../../include/*.h)
+	hipcc $HIPFLAGS -c \$< -o \$@ 2>&1 | grep -v "packed-fp32-ops' is not a recognized feature" || true
+	test -f \$@
+%.o: ../%.cpp \$(wildcard ../*.h ../*.cuh ../../../include/*.h)
+	hipcc $HIPFLAGS -x hip -c \$< -o \$@ 2>&1 | grep -v "packed-fp32-ops' is not a recognized feature" || true
+	test -f \$@
+MK
+make -C $OBJ $JOBS all

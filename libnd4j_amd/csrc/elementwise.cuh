@@ -1,0 +1,294 @@
+// Elementwise kernels shared by the transform, pairwise and broadcast families.
+//
+//   ewVecKernel      all operands contiguous: 16-byte loads/stores, 4 vectors in flight per thread.
+//   ewGeneralKernel  arbitrary views: each operand has its own index -> offset map (DimMap).
+//   bcRowKernel      broadcast over contiguous TADs: the y vector stays in registers while the thread
+//                    walks down the TADs at a fixed column.
+//   bcColKernel      broadcast over strided TADs: one thread per TAD, neighbouring TADs coalesce.
+//   bcGeneralKernel  broadcast with per-element coordinate maps.
+//
+// All of them are HBM-bound: algorithmic bytes are (inputs + 1) * sizeof(T) per element.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <utility>
+
+#include "ops_elementwise.cuh"
+#include "types.h"
+#include "view.h"
+
+namespace nd4j_amd {
+
+static constexpr int kBlock = 256;
+static constexpr int kUnroll = 4;
+
+template <typename T> struct alignas(16) Pack {
+    static constexpr int N = 16 / sizeof(T);
+    T v[N];
+};
+
+// Functor adapters: apply(a, b, params)
+template <int OP> struct TransformF {
+    static constexpr int nin = 1;
+    template <typename C, typename P> static __device__ __forceinline__ C apply(C a, C, P p) {
+        return TransformOp<OP>::template op<C, P>(a, p);
+    }
+};
+template <int KIND> struct Pairwise3F {
+    static constexpr int nin = 2;
+    template <typename C, typename P> static __device__ __forceinline__ C apply(C a, C b, P p) {
+        return BinaryOp<KIND>::template op3<C, P>(a, b, p);
+    }
+};
+template <int KIND> struct Broadcast2F {
+    static constexpr int nin = 2;
+    template <typename C, typename P> static __device__ __forceinline__ C apply(C a, C b, P) {
+        return BinaryOp<KIND>::template op2<C>(a, b);
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------
+// z[i] = F(x[i], y[i or 0]) over n contiguous elements.  `head` leading elements are done one by one so
+// that the vector part starts on a 16-byte boundary (the host guarantees all operands share the same
+// misalignment); yScalar selects y[0] for every element.
+template <typename T, typename F>
+__global__ void __launch_bounds__(kBlock) ewVecKernel(const T *x, const T *y, T *z, Params<T> p, Long n, int head,
+                                                      int yScalar) {
+    typedef typename Compute<T>::type C;
+    constexpr int VEC = Pack<T>::N;
+    const Long body = n - head;
+    const Long nvec = body / VEC;
+    const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x + head);
+    const Pack<T> *yv = reinterpret_cast<const Pack<T> *>(y + head);
+    Pack<T> *zv = reinterpret_cast<Pack<T> *>(z + head);
+    C ys = (C)0;
+    if (F::nin == 2 && yScalar) ys = toCompute(y[0]);
+
+    const Long chunk = (Long)kBlock * kUnroll;
+    for (Long base = (Long)blockIdx.x * chunk; base < nvec; base += (Long)gridDim.x * chunk) {
+        Pack<T> a[kUnroll], b[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            Long j = base + u * kBlock + threadIdx.x;
+            if (j < nvec) {
+                a[u] = xv[j];
+                if (F::nin == 2 && !yScalar) b[u] = yv[j];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            Long j = base + u * kBlock + threadIdx.x;
+            if (j < nvec) {
+                Pack<T> r;
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
+                    C bv = (F::nin == 2) ? (yScalar ? ys : toCompute(b[u].v[e])) : (C)0;
+                    r.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a[u].v[e]), bv, p));
+                }
+                zv[j] = r;
+            }
+        }
+    }
+    // head and tail elements
+    const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
+    const Long tailStart = head + nvec * VEC;
+    const Long nScalar = head + (n - tailStart);
+    if (gtid < nScalar) {
+        Long i = gtid < head ? gtid : tailStart + (gtid - head);
+        C bv = (F::nin == 2) ? (yScalar ? ys : toCompute(y[i])) : (C)0;
+        z[i] = fromCompute<T>(F::template apply<C>(toCompute(x[i]), bv, p));
+    }
+}
+
+// C-order linear index -> element offset through a DimMap.
+__device__ __forceinline__ Long mapOffset32(const DimMap &m, unsigned idx) {
+    if (m.rank == 1) return (Long)idx * m.stride[0];
+    Long off = 0;
+    for (int d = m.rank - 1; d > 0; d--) {
+        unsigned q = idx / m.shape[d];
+        unsigned c = idx - q * m.shape[d];
+        off += (Long)c * m.stride[d];
+        idx = q;
+    }
+    return off + (Long)idx * m.stride[0];
+}
+__device__ __forceinline__ Long mapOffset64(const DimMap &m, unsigned long long idx) {
+    if (m.rank == 1) return (Long)idx * m.stride[0];
+    Long off = 0;
+    for (int d = m.rank - 1; d > 0; d--) {
+        unsigned long long q = idx / m.shape[d];
+        unsigned long long c = idx - q * m.shape[d];
+        off += (Long)c * m.stride[d];
+        idx = q;
+    }
+    return off + (Long)idx * m.stride[0];
+}
+
+template <typename T, typename F>
+__global__ void __launch_bounds__(kBlock) ewGeneralKernel(const T *x, DimMap xm, const T *y, DimMap ym, T *z,
+                                                          DimMap zm, Params<T> p, Long n) {
+    typedef typename Compute<T>::type C;
+    const Long stride = (Long)gridDim.x * kBlock;
+    if (n <= 0xffffffffLL) {
+        for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+            Long ox = mapOffset32(xm, (unsigned)i);
+            Long oz = mapOffset32(zm, (unsigned)i);
+            C bv = (C)0;
+            if (F::nin == 2) bv = toCompute(y[mapOffset32(ym, (unsigned)i)]);
+            z[oz] = fromCompute<T>(F::template apply<C>(toCompute(x[ox]), bv, p));
+        }
+    } else {
+        for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+            Long ox = mapOffset64(xm, (unsigned long long)i);
+            Long oz = mapOffset64(zm, (unsigned long long)i);
+            C bv = (C)0;
+            if (F::nin == 2) bv = toCompute(y[mapOffset64(ym, (unsigned long long)i)]);
+            z[oz] = fromCompute<T>(F::template apply<C>(toCompute(x[ox]), bv, p));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Broadcast over contiguous TADs (tadEWS == yEWS == zEWS == 1).  blockIdx.x picks a column chunk of
+// kBlock vectors, blockIdx.y strides over TADs.  TADs whose offsets (or the base pointers) are not
+// 16-byte aligned fall back to scalar accesses for that TAD only.
+template <typename T, typename F>
+__global__ void __launch_bounds__(kBlock) bcRowKernel(const T *x, const T *y, T *z, const Long *xOffsets,
+                                                      const Long *zOffsets, Long tadLength, Long numTads,
+                                                      int basesAligned) {
+    typedef typename Compute<T>::type C;
+    constexpr int VEC = Pack<T>::N;
+    const Long col = ((Long)blockIdx.x * kBlock + threadIdx.x) * VEC;
+    if (col >= tadLength) return;
+    const bool full = col + VEC <= tadLength;
+    Params<T> p{nullptr};
+    C yv[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) yv[e] = (col + e < tadLength) ? toCompute(y[col + e]) : (C)0;
+
+    for (Long r = blockIdx.y; r < numTads; r += gridDim.y) {
+        const Long xo = xOffsets[r];
+        const Long zo = zOffsets[r];
+        const T *xr = x + xo + col;
+        T *zr = z + zo + col;
+        if (full && basesAligned && ((xo | zo) % VEC) == 0) {
+            Pack<T> a = *reinterpret_cast<const Pack<T> *>(xr);
+            Pack<T> o;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) o.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), yv[e], p));
+            *reinterpret_cast<Pack<T> *>(zr) = o;
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; e++)
+                if (col + e < tadLength) zr[e] = fromCompute<T>(F::template apply<C>(toCompute(xr[e]), yv[e], p));
+        }
+    }
+}
+
+// Broadcast over strided TADs: thread <-> TAD, loop over the TAD's elements.  When neighbouring TADs
+// are neighbours in memory (a column of a c-order matrix) each wave reads and writes full lines.
+template <typename T, typename F>
+__global__ void __launch_bounds__(kBlock) bcColKernel(const T *x, const T *y, T *z, const Long *xOffsets,
+                                                      const Long *zOffsets, Long tadLength, Long numTads,
+                                                      Long tadEws, Long yEws, Long zEws) {
+    typedef typename Compute<T>::type C;
+    const Long t = (Long)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= numTads) return;
+    Params<T> p{nullptr};
+    const T *xr = x + xOffsets[t];
+    T *zr = z + zOffsets[t];
+    const Long f0 = (Long)blockIdx.y;
+    for (Long f = f0; f < tadLength; f += gridDim.y) {
+        C bv = toCompute(y[f * yEws]);
+        zr[f * zEws] = fromCompute<T>(F::template apply<C>(toCompute(xr[f * tadEws]), bv, p));
+    }
+}
+
+template <typename T, typename F>
+__global__ void __launch_bounds__(kBlock) bcGeneralKernel(const T *x, DimMap xm, const T *y, DimMap ym, T *z,
+                                                          DimMap zm, const Long *xOffsets, const Long *zOffsets,
+                                                          Long tadLength, Long numTads) {
+    typedef typename Compute<T>::type C;
+    Params<T> p{nullptr};
+    for (Long r = blockIdx.x; r < numTads; r += gridDim.x) {
+        const Long xo = xOffsets[r];
+        const Long zo = zOffsets[r];
+        for (Long f = threadIdx.x; f < tadLength; f += kBlock) {
+            Long ox = xo + mapOffset32(xm, (unsigned)f);
+            Long oz = zo + mapOffset32(zm, (unsigned)f);
+            Long oy = mapOffset32(ym, (unsigned)f);
+            z[oz] = fromCompute<T>(F::template apply<C>(toCompute(x[ox]), toCompute(y[oy]), p));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Host-side launch helpers.
+
+inline int gridFor(Long work, Long perBlock, int cap) {
+    Long g = (work + perBlock - 1) / perBlock;
+    if (g < 1) g = 1;
+    if (g > cap) g = cap;
+    return (int)g;
+}
+
+static constexpr int kGridCap = 256 * 32;  // 32 blocks of 256 threads per CU
+
+// Returns the number of leading scalar elements that brings every pointer to a 16-byte boundary, or -1
+// when the pointers do not share one misalignment.
+template <typename T> inline int commonHead(const void *a, const void *b, const void *c) {
+    uintptr_t pa = (uintptr_t)a, pb = b ? (uintptr_t)b : pa, pc = c ? (uintptr_t)c : pa;
+    if ((pa & 15) != (pb & 15) || (pa & 15) != (pc & 15)) return -1;
+    if ((pa & (sizeof(T) - 1)) != 0) return -1;
+    return (int)(((16 - (pa & 15)) & 15) / sizeof(T));
+}
+
+template <typename T, typename F>
+inline void launchStrided(hipStream_t s, const T *x, Long xs, const T *y, Long ys, T *z, Long zs, const T *extra, Long n) {
+    if (n <= 0) return;
+    Params<T> p{extra};
+    const bool two = F::nin == 2;
+    const bool contig = xs == 1 && zs == 1 && (!two || ys == 1 || ys == 0);
+    if (contig) {
+        int head = commonHead<T>(x, (two && ys == 1) ? (const void *)y : nullptr, z);
+        if (head >= 0) {
+            if (head > n) head = (int)n;
+            Long nvec = (n - head) / Pack<T>::N;
+            int grid = gridFor(nvec > 0 ? nvec : 1, (Long)kBlock * kUnroll, kGridCap);
+            hipLaunchKernelGGL((ewVecKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, two ? y : x, z, p, n, head,
+                               (two && ys == 0) ? 1 : 0);
+            return;
+        }
+    }
+    DimMap xm, ym, zm;
+    xm.rank = ym.rank = zm.rank = 1;
+    xm.shape[0] = ym.shape[0] = zm.shape[0] = (unsigned)(n > 0xffffffffLL ? 0xffffffffu : n);
+    xm.stride[0] = xs; ym.stride[0] = ys; zm.stride[0] = zs;
+    int grid = gridFor(n, kBlock * 4, kGridCap);
+    hipLaunchKernelGGL((ewGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, xm, two ? y : x, ym, z, zm, p, n);
+}
+
+template <typename T, typename F>
+inline void launchGeneral(hipStream_t s, const T *x, const DimMap &xm, const T *y, const DimMap &ym, T *z,
+                          const DimMap &zm, const T *extra, Long n) {
+    if (n <= 0) return;
+    const bool two = F::nin == 2;
+    if (xm.rank == 1 && zm.rank == 1 && (!two || ym.rank == 1)) {
+        launchStrided<T, F>(s, x, xm.stride[0], y, two ? ym.stride[0] : 0, z, zm.stride[0], extra, n);
+        return;
+    }
+    Params<T> p{extra};
+    int grid = gridFor(n, kBlock * 4, kGridCap);
+    hipLaunchKernelGGL((ewGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, xm, two ? y : x, two ? ym : xm, z, zm,
+                       p, n);
+}
+
+// Compile-time opNum dispatch: calls Body<I>::run(args...) for I == op, returns false if no I matches
+// or the op has no functor.
+template <template <int> class Body, int... Is, typename... A>
+inline bool dispatchSeq(int op, std::integer_sequence<int, Is...>, A &&...a) {
+    return ((op == Is ? Body<Is>::run(std::forward<A>(a)...) : false) || ...);
+}
+
+}  // namespace nd4j_amd

@@ -1,0 +1,115 @@
+// Interface between the host boundary (native_ops.cpp) and the kernel translation units.
+// Every launcher enqueues on `stream` and returns false when opNum has no functor (the caller then
+// reports it the way the reference does, op_boilerplate.h:1148: a printed error, output untouched).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "types.h"
+#include "view.h"
+
+namespace nd4j_amd {
+
+// ---- elementwise -----------------------------------------------------------------------------------
+template <typename T>
+bool launchTransformStrided(hipStream_t stream, int opNum, const T *x, Long xs, T *z, Long zs, const T *extra, Long n);
+template <typename T>
+bool launchTransformGeneral(hipStream_t stream, int opNum, const T *x, const DimMap &xm, T *z, const DimMap &zm,
+                            const T *extra, Long n);
+// ys == 0 broadcasts y[0]
+template <typename T>
+bool launchPairwiseStrided(hipStream_t stream, int opNum, const T *x, Long xs, const T *y, Long ys, T *z, Long zs,
+                           const T *extra, Long n);
+template <typename T>
+bool launchPairwiseGeneral(hipStream_t stream, int opNum, const T *x, const DimMap &xm, const T *y, const DimMap &ym,
+                           T *z, const DimMap &zm, const T *extra, Long n);
+
+struct BroadcastPlan {
+    enum Kind { ROW, COL, GENERAL } kind;
+    Long tadLength, numTads;
+    Long tadEws, yEws, zEws;     // ROW / COL
+    DimMap xm, ym, zm;           // GENERAL: element index inside the TAD -> offset
+    const Long *xOffsets;        // device, numTads entries
+    const Long *zOffsets;        // device, numTads entries
+};
+template <typename T>
+bool launchBroadcast(hipStream_t stream, int opNum, const T *x, const T *y, T *z, const BroadcastPlan &plan);
+
+// ---- reductions ------------------------------------------------------------------------------------
+// How the elements of one TAD are addressed and how TADs relate to each other.
+struct TadPlan {
+    enum Kind {
+        ROW,      // tadEws == 1: lanes cooperate along a contiguous TAD
+        COL,      // tadEws  > 1: one lane per TAD, rows of adjacent TADs coalesce
+        GENERAL   // no element-wise stride: per-element coordinate map
+    } kind;
+    Long tadLength, numTads, tadEws;
+    DimMap tm;               // GENERAL
+    const Long *offsets;     // device, numTads entries
+};
+
+// Scratch for multi-block stages.  `bytes` is what the pointer is known to hold.
+struct Workspace {
+    void *ptr;
+    size_t bytes;
+};
+
+// Full-array view for scalar reductions: either 1-D strided (ews >= 1) or a C-order coordinate map.
+struct FlatPlan {
+    Long n;
+    bool strided;
+    Long ews;
+    DimMap xm;
+};
+
+template <typename T>
+bool launchReduceTad(hipStream_t stream, int opNum, const T *x, const T *extra, T *z, const TadPlan &plan,
+                     Workspace ws);
+// writes the post-processed scalar to z[0] (device) and, if hostResult != nullptr, leaves it there for
+// the caller to read after synchronising (hostResult must be device-visible pinned memory or null)
+template <typename T>
+bool launchReduceScalar(hipStream_t stream, int opNum, const T *x, const T *extra, T *z, const FlatPlan &plan,
+                        Workspace ws);
+
+template <typename T>
+bool launchIndexReduceTad(hipStream_t stream, int opNum, const T *x, const T *extra, T *z, const TadPlan &plan,
+                          Workspace ws);
+template <typename T>
+bool launchIndexReduceScalar(hipStream_t stream, int opNum, const T *x, const T *extra, T *z, const FlatPlan &plan,
+                             Workspace ws);
+
+template <typename T>
+bool launchSummaryStatsTad(hipStream_t stream, int opNum, bool biasCorrected, bool phantomZero, const T *x, T *z,
+                           const TadPlan &plan, Workspace ws);
+template <typename T>
+bool launchSummaryStatsScalar(hipStream_t stream, int opNum, bool biasCorrected, const T *x, T *z,
+                              const FlatPlan &plan, Workspace ws);
+
+// ---- random ----------------------------------------------------------------------------------------
+// Device image of the generator state that getElement() needs (reference: helper_generator.h:61-74,
+// 185-220).  Passed by value, so one op sees one consistent state.
+struct RngState {
+    const unsigned long long *buffer;  // device copy of the u64 buffer
+    Long size;
+    Long position;    // currentPosition
+    Long generation;
+    Long seed;
+    Long amplifier;
+};
+struct RandomPlan {
+    Long n;
+    // each operand: 1-D strided (ews >= 1 for all) or Fortran-order coordinate maps (cpu/random.cpp:46-76)
+    bool strided;
+    Long xEws, yEws, zEws;
+    DimMap xm, ym, zm;
+    Long yLength;  // Choice
+};
+template <typename T>
+bool launchRandom(hipStream_t stream, int opNum, const RngState &rng, const T *x, const T *y, T *z, const T *args,
+                  const RandomPlan &plan, int operands /* 1: z, 2: x,z, 3: x,y,z */, bool yIsZ);
+// debugging / parity aid: out[i] = getElement(start + i)
+void launchRngDump(hipStream_t stream, const RngState &rng, Long start, Long n, unsigned long long *out);
+// plain copy with 16-byte vectors (bytes is rounded down to a multiple of 16 plus a byte tail)
+void launchCopy(hipStream_t stream, void *dst, const void *src, Long bytes);
+
+}  // namespace nd4j_amd

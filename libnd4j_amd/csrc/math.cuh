@@ -1,0 +1,90 @@
+// Device math for the op functors.
+//
+// The reference evaluates every op through libm: nd4j_tanh<float> is tanhf, nd4j_exp<float> is expf and
+// so on (include/templatemath.h:537-1100).  To stay within 2 ULP of those float routines without
+// re-deriving each of them, the float overloads evaluate the double-precision routine and round once,
+// which is within 0.5 ULP of the exact value (+ a negligible double-rounding term).  Operations that
+// are exact or correctly rounded in IEEE arithmetic (sqrt, floor, fmod ...) stay in float.
+//
+// Device code is compiled with -ffp-contract=off: the reference build targets plain x86-64 without
+// FMA, so a*b+c there rounds twice.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace nd4j_amd {
+namespace m {
+
+#define ND4J_VIA_DOUBLE(name, fn)                                                       \
+    __device__ __forceinline__ float name(float v) { return (float)::fn((double)v); }   \
+    __device__ __forceinline__ double name(double v) { return ::fn(v); }
+
+ND4J_VIA_DOUBLE(cos_, cos)
+ND4J_VIA_DOUBLE(sin_, sin)
+ND4J_VIA_DOUBLE(tan_, tan)
+ND4J_VIA_DOUBLE(cosh_, cosh)
+ND4J_VIA_DOUBLE(sinh_, sinh)
+ND4J_VIA_DOUBLE(tanh_, tanh)
+ND4J_VIA_DOUBLE(acos_, acos)
+ND4J_VIA_DOUBLE(asin_, asin)
+ND4J_VIA_DOUBLE(atan_, atan)
+ND4J_VIA_DOUBLE(acosh_, acosh)
+ND4J_VIA_DOUBLE(atanh_, atanh)
+ND4J_VIA_DOUBLE(exp_, exp)
+ND4J_VIA_DOUBLE(log_, log)
+ND4J_VIA_DOUBLE(erf_, erf)
+ND4J_VIA_DOUBLE(erfc_, erfc)
+#undef ND4J_VIA_DOUBLE
+
+__device__ __forceinline__ float pow_(float a, float b) { return (float)::pow((double)a, (double)b); }
+__device__ __forceinline__ double pow_(double a, double b) { return ::pow(a, b); }
+__device__ __forceinline__ float atan2_(float a, float b) { return (float)::atan2((double)a, (double)b); }
+__device__ __forceinline__ double atan2_(double a, double b) { return ::atan2(a, b); }
+
+__device__ __forceinline__ float sqrt_(float v) { return __fsqrt_rn(v); }
+__device__ __forceinline__ double sqrt_(double v) { return __dsqrt_rn(v); }
+__device__ __forceinline__ float abs_(float v) { return ::fabsf(v); }
+__device__ __forceinline__ double abs_(double v) { return ::fabs(v); }
+__device__ __forceinline__ float floor_(float v) { return ::floorf(v); }
+__device__ __forceinline__ double floor_(double v) { return ::floor(v); }
+__device__ __forceinline__ float ceil_(float v) { return ::ceilf(v); }
+__device__ __forceinline__ double ceil_(double v) { return ::ceil(v); }
+__device__ __forceinline__ float round_(float v) { return ::roundf(v); }
+__device__ __forceinline__ double round_(double v) { return ::round(v); }
+__device__ __forceinline__ float rint_(float v) { return ::rintf(v); }
+__device__ __forceinline__ double rint_(double v) { return ::rint(v); }
+__device__ __forceinline__ float fmod_(float a, float b) { return ::fmodf(a, b); }
+__device__ __forceinline__ double fmod_(double a, double b) { return ::fmod(a, b); }
+__device__ __forceinline__ float remainder_(float a, float b) { return ::remainderf(a, b); }
+__device__ __forceinline__ double remainder_(double a, double b) { return ::remainder(a, b); }
+
+template <typename C> __device__ __forceinline__ bool isnan_(C v) { return v != v; }
+__device__ __forceinline__ bool isinf_(float v) { return ::fabsf(v) == __builtin_inff(); }
+__device__ __forceinline__ bool isinf_(double v) { return ::fabs(v) == __builtin_inf(); }
+
+// nd4j_max / nd4j_min (templatemath.h:447-470): plain comparisons, so NaN handling is positional.
+template <typename C> __device__ __forceinline__ C max_(C a, C b) { return a > b ? a : b; }
+template <typename C> __device__ __forceinline__ C min_(C a, C b) { return a < b ? a : b; }
+template <typename C> __device__ __forceinline__ C sgn_(C v) { return v < (C)0 ? (C)-1 : (v > (C)0 ? (C)1 : (C)0); }
+
+// nd4j_sigmoid (templatemath.h:147-150): 1 / (1 + exp(-x)) evaluated step by step in the compute type.
+template <typename C> __device__ __forceinline__ C sigmoid_(C v) { return (C)1 / ((C)1 + exp_(-v)); }
+
+// nd4j_re (templatemath.h): relative error |a-b| / (|a|+|b|), 0 when both are 0.
+template <typename C> __device__ __forceinline__ C re_(C a, C b) {
+    if (a == (C)0 && b == (C)0) return (C)0;
+    return abs_(a - b) / (abs_(a) + abs_(b));
+}
+
+// (T)(int) casts as x86 performs them: out-of-range and NaN become INT_MIN (cvttss2si).
+__device__ __forceinline__ int toIntX86(float v) {
+    if (!(v > -2147483904.0f && v < 2147483648.0f)) return (int)0x80000000;
+    return (int)v;
+}
+__device__ __forceinline__ int toIntX86(double v) {
+    if (!(v > -2147483649.0 && v < 2147483648.0)) return (int)0x80000000;
+    return (int)v;
+}
+
+}  // namespace m
+}  // namespace nd4j_amd

@@ -1,0 +1,379 @@
+// NativeOps boundary, part 1: lifecycle members and the elementwise families (transform, pairwise,
+// broadcast).  Branch selection follows the reference's CPU loops, which are the parity oracle:
+//   transform  include/loops/cpu/transform.cpp:28-89
+//   pairwise   include/loops/pairwise_transform.h:154-366
+//   broadcast  include/loops/cpu/broadcasting.cpp:42-156
+// extraPointers are decoded as the reference's CUDA back end does (blas/cuda/NativeOps.cu:1813-1823,
+// 3100-3131).
+#include <cstring>
+
+#include "../../include/NativeOps.h"
+#include "runtime.h"
+
+using namespace nd4j_amd;
+
+namespace {
+
+inline bool sameShape(const Long *a, const Long *b) {
+    if (siRank(a) != siRank(b)) return false;
+    for (int i = 0; i < siRank(a); i++)
+        if (siShape(a)[i] != siShape(b)[i]) return false;
+    return true;
+}
+
+// Index -> offset map of one operand walked by its own linear index, in C order or Fortran order.
+void linearMap(const Long *shape, const Long *stride, int rank, char order, DimMap &out) {
+    if (order == 'c') {
+        ownCanon(rank, shape, stride, out);
+        return;
+    }
+    Long rs[kMaxRank], rt[kMaxRank];
+    for (int i = 0; i < rank; i++) { rs[i] = shape[rank - 1 - i]; rt[i] = stride[rank - 1 - i]; }
+    ownCanon(rank, rs, rt, out);
+}
+
+template <typename T>
+void transformStrided(Nd4jPointer *extra, int opNum, T *x, Long xs, T *z, Long zs, T *params, Long n) {
+    hipStream_t s = streamOf(extra);
+    if (!launchTransformStrided<T>(s, opNum, x, xs, z, zs, params, n)) { reportUnknownOp("transform", opNum); return; }
+    checkLaunch("execTransform(strided)", s);
+}
+
+template <typename T>
+void transformShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, Long *zInfo, T *params) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx, sz;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    const Long *hz = hostShapeInfo(extra, X_HOST_Z_SHAPE, zInfo, sz, s);
+    if (hx == nullptr || hz == nullptr) return;
+    Long n = siNumel(hx);
+    Long xe = siEws(hx), ze = siEws(hz);
+    bool ok;
+    if (xe >= 1 && ze >= 1 && siOrder(hx) == siOrder(hz)) {
+        ok = launchTransformStrided<T>(s, opNum, x, xe, z, ze, params, n);
+    } else {
+        // same logical coordinates on both sides (raw iteration over x's shape)
+        const Long *strides[3] = {siStride(hx), nullptr, siStride(hz)};
+        DimMap maps[3];
+        jointCanon(siRank(hx), siShape(hx), strides, maps);
+        ok = launchTransformGeneral<T>(s, opNum, x, maps[0], z, maps[2], params, n);
+    }
+    if (!ok) { reportUnknownOp("transform", opNum); return; }
+    checkLaunch("execTransform", s);
+}
+
+template <typename T>
+void pairwiseStrided(Nd4jPointer *extra, int opNum, T *x, Long xs, T *y, Long ys, T *z, Long zs, T *params, Long n) {
+    hipStream_t s = streamOf(extra);
+    bool ok;
+    if (ys == 0) {
+        // a literal zero stride is a valid (if unusual) request: every element pairs with y[0]
+        DimMap xm, ym, zm;
+        xm.rank = ym.rank = zm.rank = 1;
+        xm.shape[0] = ym.shape[0] = zm.shape[0] = (unsigned)n;
+        xm.stride[0] = xs; ym.stride[0] = 0; zm.stride[0] = zs;
+        ok = launchPairwiseGeneral<T>(s, opNum, x, xm, y, ym, z, zm, params, n);
+    } else {
+        ok = launchPairwiseStrided<T>(s, opNum, x, xs, y, ys, z, zs, params, n);
+    }
+    if (!ok) { reportUnknownOp("pairwise", opNum); return; }
+    checkLaunch("execPairwiseTransform(strided)", s);
+}
+
+template <typename T>
+void pairwiseShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Long *yInfo, T *z, Long *zInfo, T *params) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx, sy, sz;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    const Long *hy = hostShapeInfo(extra, X_HOST_Y_SHAPE, yInfo, sy, s);
+    const Long *hz = hostShapeInfo(extra, X_HOST_Z_SHAPE, zInfo, sz, s);
+    if (hx == nullptr || hy == nullptr || hz == nullptr) return;
+    Long n = siNumel(hx);
+    Long xe = siEws(hx), ye = siEws(hy), ze = siEws(hz);
+    bool ok;
+    if (siIsScalar(hy)) {
+        if (xe == 1 && ze == 1) {
+            ok = launchPairwiseStrided<T>(s, opNum, x, 1, y, 0, z, 1, params, n);
+        } else {
+            DimMap xm, ym, zm;
+            linearMap(siShape(hx), siStride(hx), siRank(hx), 'c', xm);
+            linearMap(siShape(hz), siStride(hz), siRank(hz), 'c', zm);
+            ym.rank = 1; ym.shape[0] = 1; ym.stride[0] = 0;
+            ok = launchPairwiseGeneral<T>(s, opNum, x, xm, y, ym, z, zm, params, n);
+        }
+    } else {
+        bool same = sameShape(hx, hy);
+        bool ordersEqual = siOrder(hx) == siOrder(hy) && siOrder(hz) == siOrder(hx);
+        bool ewsOk = xe >= 1 && ye >= 1 && ze >= 1 && xe == ye;
+        if (ewsOk && ordersEqual) {
+            // same shape: n elements; different shapes: length(y) elements (pairwise_transform.h:209-239)
+            Long count = same ? n : siNumel(hy);
+            ok = launchPairwiseStrided<T>(s, opNum, x, xe, y, ye, z, ze, params, count);
+        } else if (same) {
+            const Long *strides[3] = {siStride(hx), siStride(hy), siStride(hz)};
+            DimMap maps[3];
+            jointCanon(siRank(hx), siShape(hx), strides, maps);
+            ok = launchPairwiseGeneral<T>(s, opNum, x, maps[0], y, maps[1], z, maps[2], params, n);
+        } else {
+            DimMap xm, ym, zm;
+            linearMap(siShape(hx), siStride(hx), siRank(hx), 'c', xm);
+            linearMap(siShape(hy), siStride(hy), siRank(hy), 'c', ym);
+            if (x == z) zm = xm;
+            else linearMap(siShape(hz), siStride(hz), siRank(hz), 'c', zm);
+            ok = launchPairwiseGeneral<T>(s, opNum, x, xm, y, ym, z, zm, params, n);
+        }
+    }
+    if (!ok) { reportUnknownOp("pairwise", opNum); return; }
+    checkLaunch("execPairwiseTransform", s);
+}
+
+template <typename T>
+void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Long *yInfo, T *z, Long *zInfo,
+                     int *dimension, int dimLen) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx, sy, sz, szt;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    const Long *hy = hostShapeInfo(extra, X_HOST_Y_SHAPE, yInfo, sy, s);
+    const Long *hz = hostShapeInfo(extra, X_HOST_Z_SHAPE, zInfo, sz, s);
+    if (hx == nullptr || hy == nullptr || hz == nullptr) return;
+
+    ResolvedTad tx;
+    if (!resolveTad(extra, X_HOST_TAD_SHAPE, X_DEV_TAD_OFFSETS, hx, dimension, dimLen, tx, s)) return;
+
+    // TADs of the result: the caller's tables when given, else those of x (cpu/broadcasting.cpp:79-82).
+    const Long *zTadInfo = tx.hostInfo;
+    const Long *zOffsets = tx.devOffsets;
+    const Long *devZTad = reinterpret_cast<const Long *>(slotOf(extra, X_DEV_TAD_SHAPE_Z));
+    const Long *devZOff = reinterpret_cast<const Long *>(slotOf(extra, X_DEV_TAD_OFFSETS_Z));
+    if (devZTad != nullptr && devZOff != nullptr) {
+        zOffsets = devZOff;
+        bool zLikeX = siRank(hx) == siRank(hz) &&
+                      std::memcmp(hx, hz, sizeof(Long) * siLength(siRank(hx))) == 0;
+        if (!zLikeX) {
+            zTadInfo = hostShapeInfo(nullptr, 0, devZTad, szt, s);
+            if (zTadInfo == nullptr) return;
+        }
+    }
+
+    BroadcastPlan pl;
+    pl.tadLength = tx.tadLength;
+    pl.numTads = tx.numTads;
+    pl.xOffsets = tx.devOffsets;
+    pl.zOffsets = zOffsets;
+    pl.tadEws = siEws(tx.hostInfo);
+    pl.yEws = siEws(hy);
+    pl.zEws = siEws(zTadInfo);
+    if (pl.tadEws > 0 && pl.yEws > 0 && pl.zEws > 0 && dimLen == 1) {
+        pl.kind = (pl.tadEws == 1 && pl.yEws == 1 && pl.zEws == 1) ? BroadcastPlan::ROW : BroadcastPlan::COL;
+    } else {
+        pl.kind = BroadcastPlan::GENERAL;
+        char xo = siOrder(tx.hostInfo) == 'c' ? 'c' : 'f';
+        char zo = siOrder(zTadInfo) == 'c' ? 'c' : 'f';
+        linearMap(siShape(tx.hostInfo), siStride(tx.hostInfo), siRank(tx.hostInfo), xo, pl.xm);
+        linearMap(siShape(hy), siStride(hy), siRank(hy), xo, pl.ym);
+        linearMap(siShape(zTadInfo), siStride(zTadInfo), siRank(zTadInfo), zo, pl.zm);
+    }
+    if (!launchBroadcast<T>(s, opNum, x, y, z, pl)) { reportUnknownOp("broadcast", opNum); return; }
+    checkLaunch("execBroadcast", s);
+}
+
+}  // namespace
+
+// ---- per-type members ---------------------------------------------------------------------------------
+#define ND4J_ELEMENTWISE_MEMBERS(SUFFIX, T)                                                                      \
+    void NativeOps::execTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong xStride,        \
+                                          T *result, Nd4jLong resultStride, T *extraParams, Nd4jLong n) {        \
+        transformStrided<T>(extraPointers, opNum, dx, xStride, result, resultStride, extraParams, n);            \
+    }                                                                                                            \
+    void NativeOps::execTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong *xShapeInfo,    \
+                                          T *result, Nd4jLong *resultShapeInfo, T *extraParams) {                \
+        transformShaped<T>(extraPointers, opNum, dx, xShapeInfo, result, resultShapeInfo, extraParams);          \
+    }                                                                                                            \
+    void NativeOps::execTransform##SUFFIX(Nd4jPointer *, int, T *, Nd4jLong *, T *, Nd4jLong *, T *, Nd4jLong *, \
+                                          Nd4jLong *) {                                                          \
+        /* indexed variant: empty in the reference too (blas/cuda/NativeOps.cu:3598-3612) */                     \
+    }                                                                                                            \
+    void NativeOps::execPairwiseTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx,                  \
+                                                  Nd4jLong xStride, T *y, Nd4jLong yStride, T *result,           \
+                                                  Nd4jLong resultStride, T *extraParams, Nd4jLong n) {           \
+        pairwiseStrided<T>(extraPointers, opNum, dx, xStride, y, yStride, result, resultStride, extraParams, n); \
+    }                                                                                                            \
+    void NativeOps::execPairwiseTransform##SUFFIX(Nd4jPointer *, int, T *, Nd4jLong *, T *, Nd4jLong *, T *,     \
+                                                  Nd4jLong *, T *, Nd4jLong *, Nd4jLong *, Nd4jLong *) {         \
+        /* indexed variant: empty in the reference's CUDA back end (blas/cuda/NativeOps.cu:1928-1960) */         \
+    }                                                                                                            \
+    void NativeOps::execPairwiseTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx,                  \
+                                                  Nd4jLong *xShapeInfo, T *y, Nd4jLong *yShapeInfo, T *result,   \
+                                                  Nd4jLong *resultShapeInfo, T *extraParams) {                   \
+        pairwiseShaped<T>(extraPointers, opNum, dx, xShapeInfo, y, yShapeInfo, result, resultShapeInfo,          \
+                          extraParams);                                                                          \
+    }                                                                                                            \
+    void NativeOps::execBroadcast##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,     \
+                                          T *y, Nd4jLong *yShapeInfo, T *result, Nd4jLong *resultShapeInfo,      \
+                                          int *dimension, int dimensionLength) {                                 \
+        broadcastShaped<T>(extraPointers, opNum, x, xShapeInfo, y, yShapeInfo, result, resultShapeInfo,          \
+                           dimension, dimensionLength);                                                          \
+    }
+
+ND4J_ELEMENTWISE_MEMBERS(Float, float)
+ND4J_ELEMENTWISE_MEMBERS(Half, float16)
+ND4J_ELEMENTWISE_MEMBERS(Double, double)
+
+// ---- shape service -------------------------------------------------------------------------------------
+void NativeOps::tadOnlyShapeInfo(Nd4jLong *xShapeInfo, int *dimension, int dimensionLength, Nd4jLong *targetBuffer,
+                                 Nd4jLong *offsetsBuffer) {
+    TadPack pack;
+    computeTad(xShapeInfo, dimension, dimensionLength, pack, offsetsBuffer != nullptr);
+    std::memcpy(targetBuffer, pack.shapeInfo.data(), pack.shapeInfo.size() * sizeof(Long));
+    if (offsetsBuffer != nullptr) std::memcpy(offsetsBuffer, pack.offsets.data(), pack.offsets.size() * sizeof(Long));
+}
+
+// ---- lifecycle (reference: blas/cuda/NativeOps.cu:3946-4390) ---------------------------------------------
+static int deviceIdOf(Nd4jPointer p) { return (int)(intptr_t)p; }
+
+void NativeOps::initializeDevicesAndFunctions() {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) (void)hipGetLastError();
+}
+
+Nd4jPointer NativeOps::mallocHost(Nd4jLong memorySize, int) {
+    void *p = nullptr;
+    if (hipHostMalloc(&p, (size_t)memorySize, hipHostMallocDefault) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    return p;
+}
+Nd4jPointer NativeOps::mallocDevice(Nd4jLong memorySize, Nd4jPointer, int) {
+    void *p = nullptr;
+    if (hipMalloc(&p, (size_t)memorySize) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    return p;
+}
+int NativeOps::freeHost(Nd4jPointer pointer) { return hipHostFree(pointer) == hipSuccess ? 1 : 0; }
+int NativeOps::freeDevice(Nd4jPointer pointer, Nd4jPointer) { return hipFree(pointer) == hipSuccess ? 1 : 0; }
+
+int NativeOps::ompGetMaxThreads() { return environment().maxThreads.load(); }
+int NativeOps::ompGetNumThreads() { return environment().maxThreads.load(); }
+void NativeOps::setOmpNumThreads(int threads) {
+    // on the GPU back end this is the maximum block size, clamped to 32..1024 (blas/cuda/NativeOps.cu:4380-4390)
+    if (threads < 32) threads = 32;
+    if (threads > 1024) threads = 1024;
+    environment().maxThreads.store(threads);
+}
+void NativeOps::setOmpMinThreads(int) {}
+Nd4jPointer NativeOps::createContext() { return nullptr; }
+Nd4jPointer NativeOps::createStream() {
+    hipStream_t s = nullptr;
+    if (hipStreamCreate(&s) != hipSuccess) throw std::runtime_error("createStream failed");
+    return reinterpret_cast<Nd4jPointer>(s);  // the handle itself (blas/cuda/NativeOps.cu:4166-4177)
+}
+Nd4jPointer NativeOps::createEvent() {
+    hipEvent_t e = nullptr;
+    if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) throw std::runtime_error("createEvent failed");
+    return reinterpret_cast<Nd4jPointer>(e);
+}
+int NativeOps::registerEvent(Nd4jPointer event, Nd4jPointer stream) {
+    if (hipEventRecord(reinterpret_cast<hipEvent_t>(event), reinterpret_cast<hipStream_t>(stream)) != hipSuccess)
+        throw std::runtime_error("registerEvent failed");
+    return 1;
+}
+int NativeOps::destroyEvent(Nd4jPointer event) {
+    if (hipEventDestroy(reinterpret_cast<hipEvent_t>(event)) != hipSuccess) throw std::runtime_error("destroyEvent failed");
+    return 1;
+}
+int NativeOps::setDevice(Nd4jPointer ptrToDeviceId) {
+    if (hipSetDevice(deviceIdOf(ptrToDeviceId)) != hipSuccess) throw std::runtime_error("setDevice failed");
+    return 1;
+}
+int NativeOps::getDevice() {
+    int d = 0;
+    (void)hipGetDevice(&d);
+    return d;
+}
+int NativeOps::streamSynchronize(Nd4jPointer stream) {
+    if (hipStreamSynchronize(reinterpret_cast<hipStream_t>(stream)) != hipSuccess)
+        throw std::runtime_error("streamSynchronize failed");
+    return 1;
+}
+int NativeOps::eventSynchronize(Nd4jPointer event) {
+    if (hipEventSynchronize(reinterpret_cast<hipEvent_t>(event)) != hipSuccess)
+        throw std::runtime_error("eventSynchronize failed");
+    return 1;
+}
+Nd4jLong NativeOps::getDeviceFreeMemory(Nd4jPointer ptrToDeviceId) {
+    int prev = getDevice(), want = deviceIdOf(ptrToDeviceId);
+    if (want >= 0 && want != prev) (void)hipSetDevice(want);
+    size_t f = 0, t = 0;
+    (void)hipMemGetInfo(&f, &t);
+    if (want >= 0 && want != prev) (void)hipSetDevice(prev);
+    return (Nd4jLong)f;
+}
+Nd4jLong NativeOps::getDeviceTotalMemory(Nd4jPointer ptrToDeviceId) {
+    int prev = getDevice(), want = deviceIdOf(ptrToDeviceId);
+    if (want >= 0 && want != prev) (void)hipSetDevice(want);
+    size_t f = 0, t = 0;
+    (void)hipMemGetInfo(&f, &t);
+    if (want >= 0 && want != prev) (void)hipSetDevice(prev);
+    return (Nd4jLong)t;
+}
+static hipDeviceProp_t &propsOf(int dev) {
+    static hipDeviceProp_t props[64];
+    static bool have[64] = {false};
+    if (dev < 0 || dev >= 64) dev = 0;
+    if (!have[dev]) {
+        if (hipGetDeviceProperties(&props[dev], dev) != hipSuccess) { (void)hipGetLastError(); std::memset(&props[dev], 0, sizeof(props[dev])); }
+        have[dev] = true;
+    }
+    return props[dev];
+}
+int NativeOps::getDeviceMajor(Nd4jPointer ptrToDeviceId) { return propsOf(deviceIdOf(ptrToDeviceId)).major; }
+int NativeOps::getDeviceMinor(Nd4jPointer ptrToDeviceId) { return propsOf(deviceIdOf(ptrToDeviceId)).minor; }
+const char *NativeOps::getDeviceName(Nd4jPointer ptrToDeviceId) { return propsOf(deviceIdOf(ptrToDeviceId)).name; }
+
+static hipMemcpyKind kindOf(int flags) {
+    switch (flags) {
+        case 0: return hipMemcpyHostToHost;
+        case 1: return hipMemcpyHostToDevice;
+        case 2: return hipMemcpyDeviceToHost;
+        case 3: return hipMemcpyDeviceToDevice;
+        default: return hipMemcpyDefault;
+    }
+}
+int NativeOps::memcpy(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer) {
+    return hipMemcpy(dst, src, (size_t)size, kindOf(flags)) == hipSuccess ? 1 : 0;
+}
+int NativeOps::memcpyAsync(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved) {
+    return hipMemcpyAsync(dst, src, (size_t)size, kindOf(flags), reinterpret_cast<hipStream_t>(reserved)) == hipSuccess ? 1 : 0;
+}
+int NativeOps::memset(Nd4jPointer dst, int value, Nd4jLong size, int, Nd4jPointer) {
+    return hipMemset(dst, value, (size_t)size) == hipSuccess ? 1 : 0;
+}
+int NativeOps::memsetAsync(Nd4jPointer dst, int value, Nd4jLong size, int, Nd4jPointer reserved) {
+    return hipMemsetAsync(dst, value, (size_t)size, reinterpret_cast<hipStream_t>(reserved)) == hipSuccess ? 1 : 0;
+}
+
+// The reference keeps a 48 KiB __constant__ arena that ND4J fills with shapeInfo buffers
+// (blas/cuda/NativeOps.cu:87, 4793-4835).  Plain device memory serves the same purpose here.
+static void *constantSpace() {
+    static void *space = nullptr;
+    if (space == nullptr && hipMalloc(&space, 49152) != hipSuccess) { (void)hipGetLastError(); space = nullptr; }
+    return space;
+}
+int NativeOps::memcpyConstantAsync(Nd4jLong dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved) {
+    char *base = reinterpret_cast<char *>(constantSpace());
+    if (base == nullptr || dst < 0 || dst + size > 49152) return 0;
+    hipMemcpyKind k = flags == 3 ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice;
+    return hipMemcpyAsync(base + dst, src, (size_t)size, k, reinterpret_cast<hipStream_t>(reserved)) == hipSuccess ? 1 : 0;
+}
+Nd4jPointer NativeOps::getConstantSpace() { return constantSpace(); }
+int NativeOps::getAvailableDevices() {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; }
+    return n;
+}
+void NativeOps::enableDebugMode(bool reallyEnable) { environment().debug.store(reallyEnable); }
+void NativeOps::enableVerboseMode(bool reallyEnable) { environment().verbose.store(reallyEnable); }
+void NativeOps::setGridLimit(int gridSize) {
+    if (gridSize > 8192) gridSize = 8192;
+    if (gridSize < 1) gridSize = 1;
+    environment().gridLimit.store(gridSize);
+}
+void NativeOps::setElementThreshold(int num) { if (num > 0) environment().elementThreshold.store(num); }
+void NativeOps::setTADThreshold(int num) { if (num > 0) environment().tadThreshold.store(num); }

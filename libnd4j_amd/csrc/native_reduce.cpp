@@ -1,0 +1,324 @@
+// NativeOps boundary, part 2: reduce, index-reduce and summary-stats members.
+// Branch selection follows the reference's CPU loops (the parity oracle):
+//   reduce         include/loops/cpu/reduce.cpp:91-193, scalar 14-64 / 206-323; LogSumExp pre-pass
+//                  blas/cpu/NativeOpExcutioner.cpp:122-147
+//   index-reduce   include/loops/cpu/indexreduce.cpp:36-129, 131-228
+//   summary stats  include/loops/cpu/summarystatsreduce.cpp:24-196
+// extraPointers decoding follows blas/cuda/NativeOps.cu:2098-2139 and 1600-1643.
+#include <cstring>
+
+#include "../../include/NativeOps.h"
+#include "runtime.h"
+
+using namespace nd4j_amd;
+
+namespace {
+
+static const size_t kScalarArea = 4096;          // first bytes of the workspace: scalar results
+static const size_t kWorkspaceBytes = 8u << 20;  // default size; grows on demand
+
+struct Scratch {
+    void *scalars;   // kScalarArea bytes
+    Workspace rest;  // partial accumulators
+};
+Scratch scratchFor(hipStream_t s, size_t wantRest = 0) {
+    size_t want = kScalarArea + (wantRest > 0 ? wantRest : kWorkspaceBytes - kScalarArea);
+    Workspace w = workspaceFor(s, want);
+    Scratch sc;
+    sc.scalars = w.ptr;
+    sc.rest.ptr = reinterpret_cast<char *>(w.ptr) + kScalarArea;
+    sc.rest.bytes = w.bytes - kScalarArea;
+    return sc;
+}
+
+void cLinearMap(const Long *info, DimMap &out) { ownCanon(siRank(info), siShape(info), siStride(info), out); }
+
+// Order-independent full-array walk: 1-D strided when the EWS field says so, otherwise the view with its
+// dimensions sorted by stride and merged (a dense f-order array becomes one contiguous run).
+FlatPlan flatAnyOrder(const Long *hx) {
+    FlatPlan pl;
+    pl.n = siNumel(hx);
+    Long ews = siEws(hx);
+    if (ews >= 1) { pl.strided = true; pl.ews = ews; pl.xm.rank = 0; return pl; }
+    const Long *strides[3] = {siStride(hx), nullptr, nullptr};
+    DimMap maps[3];
+    jointCanon(siRank(hx), siShape(hx), strides, maps);
+    if (maps[0].rank == 1) { pl.strided = true; pl.ews = maps[0].stride[0]; pl.xm.rank = 0; return pl; }
+    pl.strided = false;
+    pl.ews = 0;
+    pl.xm = maps[0];
+    return pl;
+}
+// Full-array walk that keeps the element numbering of the reference: memory-linear i*ews when EWS >= 1,
+// C-order logical index otherwise (cpu/indexreduce.cpp:43-75).
+FlatPlan flatIndexed(const Long *hx) {
+    FlatPlan pl;
+    pl.n = siNumel(hx);
+    Long ews = siEws(hx);
+    if (ews >= 1) { pl.strided = true; pl.ews = ews; pl.xm.rank = 0; return pl; }
+    pl.strided = false;
+    pl.ews = 0;
+    cLinearMap(hx, pl.xm);
+    return pl;
+}
+
+TadPlan tadPlanFrom(const ResolvedTad &t) {
+    TadPlan pl;
+    pl.tadLength = t.tadLength;
+    pl.numTads = t.numTads;
+    pl.offsets = t.devOffsets;
+    pl.tadEws = siEws(t.hostInfo);
+    pl.tm.rank = 0;
+    if (pl.tadEws == 1) pl.kind = TadPlan::ROW;
+    else if (pl.tadEws > 1) pl.kind = TadPlan::COL;
+    else { pl.kind = TadPlan::GENERAL; cLinearMap(t.hostInfo, pl.tm); }
+    return pl;
+}
+
+float halfBitsToFloatHost(unsigned short h) {
+    unsigned sign = (h >> 15) & 1u, exp = (h >> 10) & 0x1fu, man = h & 0x3ffu;
+    unsigned bits;
+    if (exp == 0x1f) bits = man ? 0x7fffffffu : ((sign << 31) | 0x7f800000u);
+    else if (exp == 0) {
+        if (man == 0) bits = sign << 31;
+        else {
+            int e = -1;
+            do { e++; man <<= 1; } while ((man & 0x400u) == 0);
+            bits = (sign << 31) | ((unsigned)(127 - 15 - e) << 23) | ((man & 0x3ffu) << 13);
+        }
+    } else bits = (sign << 31) | ((exp + 112u) << 23) | (man << 13);
+    float f;
+    std::memcpy(&f, &bits, 4);
+    return f;
+}
+template <typename T> struct ScalarOut;
+template <> struct ScalarOut<float> { typedef float R; static R get(float v) { return v; } };
+template <> struct ScalarOut<double> { typedef double R; static R get(double v) { return v; } };
+template <> struct ScalarOut<float16> { typedef float R; static R get(float16 v) { return halfBitsToFloatHost(v.x); } };
+
+template <typename T> typename ScalarOut<T>::R readScalar(const void *devSlot, hipStream_t s, const char *what) {
+    T v;
+    std::memset(&v, 0, sizeof(T));
+    hipError_t e = hipMemcpyAsync(&v, devSlot, sizeof(T), hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+    syncAndCheck(what, s);
+    return ScalarOut<T>::get(v);
+}
+
+// ---- reduce -----------------------------------------------------------------------------------------
+template <typename T> bool reduceScalarTo(hipStream_t s, int opNum, const T *x, const Long *hx, const T *extra, T *zDev) {
+    Scratch sc = scratchFor(s);
+    FlatPlan pl = flatAnyOrder(hx);
+    if (opNum == 19) {
+        // LogSumExp: maximum first, then exp(x - max) summed (NativeOpExcutioner.cpp:138-141)
+        T *maxSlot = reinterpret_cast<T *>(reinterpret_cast<char *>(sc.scalars) + 64);
+        if (!launchReduceScalar<T>(s, 3, x, extra, maxSlot, pl, sc.rest)) return false;
+        return launchReduceScalar<T>(s, 19, x, maxSlot, zDev, pl, sc.rest);
+    }
+    return launchReduceScalar<T>(s, opNum, x, extra, zDev, pl, sc.rest);
+}
+
+template <typename T> typename ScalarOut<T>::R reduceScalar(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    if (hx == nullptr) return 0;
+    Scratch sc = scratchFor(s);
+    T *slot = reinterpret_cast<T *>(sc.scalars);
+    if (!reduceScalarTo<T>(s, opNum, x, hx, params, slot)) { reportUnknownOp("reduce", opNum); return 0; }
+    return readScalar<T>(slot, s, "execReduceScalar");
+}
+
+template <typename T> void reduceFull(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *z) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    if (hx == nullptr) return;
+    if (!reduceScalarTo<T>(s, opNum, x, hx, params, z)) { reportUnknownOp("reduce", opNum); return; }
+    // the reference blocks here (blas/cuda/NativeOps.cu:2049)
+    syncAndCheck("execReduce", s);
+}
+
+template <typename T>
+void reduceDims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *z, int *dimension, int dimLen) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    if (hx == nullptr) return;
+    if (dimension == nullptr || dimLen == siRank(hx)) {
+        if (!reduceScalarTo<T>(s, opNum, x, hx, params, z)) { reportUnknownOp("reduce", opNum); return; }
+        checkLaunch("execReduce", s);
+        return;
+    }
+    ResolvedTad t;
+    if (!resolveTad(extra, X_HOST_TAD_SHAPE, X_DEV_TAD_OFFSETS, hx, dimension, dimLen, t, s)) return;
+    if (t.numTads == 1) {
+        if (!reduceScalarTo<T>(s, opNum, x, hx, params, z)) { reportUnknownOp("reduce", opNum); return; }
+        checkLaunch("execReduce", s);
+        return;
+    }
+    Scratch sc = scratchFor(s);
+    TadPlan pl = tadPlanFrom(t);
+    bool ok = true;
+    if (opNum == 19) ok = launchReduceTad<T>(s, 3, x, params, z, pl, sc.rest);  // maxima into z first
+    ok = ok && launchReduceTad<T>(s, opNum, x, params, z, pl, sc.rest);
+    if (!ok) { reportUnknownOp("reduce", opNum); return; }
+    checkLaunch("execReduce", s);
+}
+
+// ---- index reduce -----------------------------------------------------------------------------------
+template <typename T> bool indexScalarTo(hipStream_t s, int opNum, const T *x, const Long *hx, const T *extra, T *zDev) {
+    Scratch sc = scratchFor(s);
+    FlatPlan pl = flatIndexed(hx);
+    return launchIndexReduceScalar<T>(s, opNum, x, extra, zDev, pl, sc.rest);
+}
+
+template <typename T> typename ScalarOut<T>::R indexReduceScalar(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    if (hx == nullptr) return 0;
+    Scratch sc = scratchFor(s);
+    T *slot = reinterpret_cast<T *>(sc.scalars);
+    if (!indexScalarTo<T>(s, opNum, x, hx, params, slot)) { reportUnknownOp("indexreduce", opNum); return 0; }
+    return readScalar<T>(slot, s, "execIndexReduceScalar");
+}
+
+template <typename T>
+void indexReduceDims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *z, Long *zInfo, int *dimension,
+                     int dimLen) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    if (hx == nullptr) return;
+    const Long *hz = reinterpret_cast<const Long *>(slotOf(extra, X_HOST_Z_SHAPE));
+    bool scalarResult = hz != nullptr ? siIsScalar(hz) : false;
+    ResolvedTad t;
+    if (!scalarResult) {
+        if (dimension == nullptr || dimLen < 1) scalarResult = true;
+        else if (!resolveTad(extra, X_HOST_TAD_SHAPE, X_DEV_TAD_OFFSETS, hx, dimension, dimLen, t, s)) return;
+        else if (hz == nullptr && t.numTads == 1) scalarResult = true;
+    }
+    if (scalarResult) {
+        if (!indexScalarTo<T>(s, opNum, x, hx, params, z)) { reportUnknownOp("indexreduce", opNum); return; }
+        checkLaunch("execIndexReduce", s);
+        return;
+    }
+    Scratch sc = scratchFor(s);
+    TadPlan pl = tadPlanFrom(t);
+    if (!launchIndexReduceTad<T>(s, opNum, x, params, z, pl, sc.rest)) { reportUnknownOp("indexreduce", opNum); return; }
+    checkLaunch("execIndexReduce", s);
+}
+
+// ---- summary stats ----------------------------------------------------------------------------------
+template <typename T> bool statsScalarTo(hipStream_t s, int opNum, bool bias, const T *x, const Long *hx, T *zDev) {
+    Scratch sc = scratchFor(s);
+    FlatPlan pl = flatAnyOrder(hx);
+    // the reference walks EWS == 1 arrays linearly and everything else by C-order coordinates
+    // (cpu/summarystatsreduce.cpp:31-62); the moments do not depend on the visiting order
+    return launchSummaryStatsScalar<T>(s, opNum, bias, x, zDev, pl, sc.rest);
+}
+
+template <typename T>
+typename ScalarOut<T>::R statsScalar(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, bool bias) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    if (hx == nullptr) return 0;
+    Scratch sc = scratchFor(s);
+    T *slot = reinterpret_cast<T *>(sc.scalars);
+    if (!statsScalarTo<T>(s, opNum, bias, x, hx, slot)) { reportUnknownOp("summarystats", opNum); return 0; }
+    return readScalar<T>(slot, s, "execSummaryStatsScalar");
+}
+
+template <typename T> void statsFull(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, bool bias) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    if (hx == nullptr) return;
+    if (!statsScalarTo<T>(s, opNum, bias, x, hx, z)) { reportUnknownOp("summarystats", opNum); return; }
+    checkLaunch("execSummaryStats", s);
+}
+
+template <typename T>
+void statsDims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, Long *zInfo, int *dimension, int dimLen, bool bias) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    if (hx == nullptr) return;
+    const Long *hz = reinterpret_cast<const Long *>(slotOf(extra, X_HOST_Z_SHAPE));
+    bool scalarResult = hz != nullptr && siIsScalar(hz);
+    ResolvedTad t;
+    if (!scalarResult) {
+        if (dimension == nullptr || dimLen < 1) scalarResult = true;
+        else if (!resolveTad(extra, X_HOST_TAD_SHAPE, X_DEV_TAD_OFFSETS, hx, dimension, dimLen, t, s)) return;
+        else {
+            // resultLength == 1, all dimensions, or a TAD that is "the whole thing" (TAD.h:337-352) fall back
+            // to the scalar routine writing result[0] (cpu/summarystatsreduce.cpp:82-90)
+            Long n = siNumel(hx);
+            bool whole = false;
+            if (!siIsVector(hx))
+                whole = t.numTads == 1 || ((dimLen == siRank(hx) || (t.numTads == n && siOrder(hx) == 'c')) && siEws(hx) == 1);
+            else if (siIsScalar(hx))
+                whole = true;
+            Long resultLength = hz != nullptr ? siNumel(hz) : t.numTads;
+            if (resultLength == 1 || dimLen == siRank(hx) || whole) scalarResult = true;
+        }
+    }
+    if (scalarResult) {
+        if (!statsScalarTo<T>(s, opNum, bias, x, hx, z)) { reportUnknownOp("summarystats", opNum); return; }
+        checkLaunch("execSummaryStats", s);
+        return;
+    }
+    Scratch sc = scratchFor(s);
+    TadPlan pl = tadPlanFrom(t);
+    // single-dimension TADs without an element-wise stride start from a zero sample in the reference
+    // (cpu/summarystatsreduce.cpp:92-146, `comp.initWithValue(0.0)`)
+    bool phantomZero = dimLen == 1 && siEws(t.hostInfo) < 1;
+    if (!launchSummaryStatsTad<T>(s, opNum, bias, phantomZero, x, z, pl, sc.rest)) { reportUnknownOp("summarystats", opNum); return; }
+    checkLaunch("execSummaryStats", s);
+}
+
+}  // namespace
+
+#define ND4J_REDUCE_MEMBERS(SUFFIX, T, R)                                                                            \
+    R NativeOps::execReduceScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,         \
+                                          T *extraParams) {                                                          \
+        return reduceScalar<T>(extraPointers, opNum, x, xShapeInfo, extraParams);                                    \
+    }                                                                                                                \
+    void NativeOps::execReduce##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,            \
+                                       T *extraParams, T *result, Nd4jLong *) {                                      \
+        reduceFull<T>(extraPointers, opNum, x, xShapeInfo, extraParams, result);                                     \
+    }                                                                                                                \
+    void NativeOps::execReduce##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,            \
+                                       T *extraParams, T *result, Nd4jLong *, int *dimension, int dimensionLength) { \
+        reduceDims<T>(extraPointers, opNum, x, xShapeInfo, extraParams, result, dimension, dimensionLength);         \
+    }                                                                                                                \
+    R NativeOps::execIndexReduceScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,    \
+                                               T *extraParams) {                                                     \
+        return indexReduceScalar<T>(extraPointers, opNum, x, xShapeInfo, extraParams);                               \
+    }                                                                                                                \
+    void NativeOps::execIndexReduce##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,       \
+                                            T *extraParams, T *result, Nd4jLong *resultShapeInfoBuffer,              \
+                                            int *dimension, int dimensionLength) {                                   \
+        indexReduceDims<T>(extraPointers, opNum, x, xShapeInfo, extraParams, result, resultShapeInfoBuffer,          \
+                           dimension, dimensionLength);                                                              \
+    }                                                                                                                \
+    R NativeOps::execSummaryStatsScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,   \
+                                                T *, bool biasCorrected) {                                           \
+        return statsScalar<T>(extraPointers, opNum, x, xShapeInfo, biasCorrected);                                   \
+    }                                                                                                                \
+    void NativeOps::execSummaryStats##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *, \
+                                             T *result, Nd4jLong *, bool biasCorrected) {                            \
+        statsFull<T>(extraPointers, opNum, x, xShapeInfo, result, biasCorrected);                                    \
+    }                                                                                                                \
+    void NativeOps::execSummaryStats##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *, \
+                                             T *result, Nd4jLong *resultShapeInfoBuffer, int *dimension,             \
+                                             int dimensionLength, bool biasCorrected) {                              \
+        statsDims<T>(extraPointers, opNum, x, xShapeInfo, result, resultShapeInfoBuffer, dimension,                  \
+                     dimensionLength, biasCorrected);                                                                \
+    }
+
+ND4J_REDUCE_MEMBERS(Float, float, float)
+ND4J_REDUCE_MEMBERS(Half, float16, float)
+ND4J_REDUCE_MEMBERS(Double, double, double)

@@ -1,0 +1,397 @@
+// Random family: z[i] = op([x[i], [y[i],]] i, length, generator, args), a counter-based generator.
+// Reference loops: include/loops/cpu/random.cpp:11-199; ops include/ops/random_ops.h:36-197 and
+// include/ops/special_random_ops.h (Choice 14-238, Gaussian 246-397, Binomial 405-520, BinomialEx 531-650,
+// TruncatedNormal 654-815, LogNormal 818-969); generator include/helpers/helper_generator.h:185-242.
+// opNum table: include/loops/legacy_ops.h:225-239.
+//
+// Element i of a draw depends only on (state, i), so every lane computes its own elements; the host
+// advances the state afterwards (rewindH).  The integer stream is reproduced bit for bit: all 64-bit
+// wrap-around products, the `x / y + 11` branch of safeShift and the `% 2147483647` of next64.
+#include "elementwise.cuh"
+#include "launch.h"
+
+namespace nd4j_amd {
+
+typedef unsigned long long u64;
+
+__device__ __forceinline__ u64 rotl64(u64 x, int k) { return (x << k) | (x >> (64 - k)); }
+
+__device__ __forceinline__ u64 seedConvDev(u64 x) {
+    u64 z = (x += 0x9E3779B97F4A7C15ULL);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+    return z ^ (z >> 31);
+}
+
+// x mod (2^31 - 1): 2^31 == 1 (mod M), so the three 31-bit digits of x are summed and folded.
+__device__ __forceinline__ u64 modMersenne31(u64 x) {
+    const u64 M = 2147483647ULL;
+    u64 s = (x & M) + ((x >> 31) & M) + (x >> 62);
+    s = (s & M) + (s >> 31);
+    if (s >= M) s -= M;
+    return s;
+}
+
+// RandomBuffer::next64 (helper_generator.h:222-232)
+__device__ __forceinline__ u64 next64Dev(u64 s0) {
+    u64 s1 = modMersenne31(s0) + 11;
+    s1 ^= s0;
+    u64 r0 = rotl64(s0, 55) ^ s1 ^ (s1 << 14);
+    u64 r1 = rotl64(s1, 36);
+    return r0 + r1;
+}
+
+// floor(n / y) for n < y * 2^32 (so the quotient fits 32 bits), through a double estimate that is then
+// corrected with the exact remainder.  ry approximates 1/y to ~2^-52.
+__device__ __forceinline__ unsigned quot32(u64 n, unsigned y, double ry) {
+    double qd = (double)n * ry;
+    if (qd > 4294967295.0) qd = 4294967295.0;
+    unsigned q = (unsigned)qd;
+    long long rem = (long long)(n - (u64)q * (u64)y);
+    if (rem < 0) { q--; }
+    else if ((u64)rem >= (u64)y) { q++; }
+    return q;
+}
+
+// floor(x / y), y >= 1.
+__device__ __forceinline__ u64 divU64(u64 x, u64 y) {
+    if ((y >> 32) != 0) return x / y;
+    const unsigned ys = (unsigned)y;
+    double yd = (double)ys;
+    double ry = __builtin_amdgcn_rcp(yd);
+    ry = ry * (2.0 - yd * ry);
+    ry = ry * (2.0 - yd * ry);
+    const unsigned hi = (unsigned)(x >> 32);
+    const unsigned qhi = quot32((u64)hi, ys, ry);
+    const unsigned r = hi - qhi * ys;
+    const u64 n2 = ((u64)r << 32) | (x & 0xffffffffULL);
+    const unsigned qlo = quot32(n2, ys, ry);
+    return ((u64)qhi << 32) | qlo;
+}
+
+// RandomBuffer::safeShift (helper_generator.h:238-242)
+__device__ __forceinline__ u64 safeShiftDev(u64 x, u64 y) {
+    if (y != 0 && x > divU64(0xffffffffffffffffULL, y)) return divU64(x, y) + 11;
+    return x * y + 11;
+}
+
+// RandomBuffer::getElement (helper_generator.h:185-220)
+__device__ __forceinline__ u64 rngElement(const RngState &st, Long position) {
+    Long p = st.position + position;
+    Long tempGen = st.generation;
+    if (p >= st.size) {
+        u64 q = divU64((u64)p, (u64)st.size);
+        tempGen += (Long)q;
+        p = p - (Long)q * st.size;
+    }
+    u64 r = st.buffer[p];
+    const bool genDiffers = tempGen != st.generation;
+    if (genDiffers) r = safeShiftDev(r, (u64)tempGen);
+    if (st.generation > 1) r = safeShiftDev(r, (u64)st.generation);
+    if (st.amplifier != st.seed) r = safeShiftDev(r, (u64)st.amplifier);
+    if (st.amplifier != st.seed || st.generation > 1 || genDiffers) r = next64Dev(seedConvDev(r));
+    return r;
+}
+
+// relativeT<T>(index): u64 -> [0, 1] (helper_generator.h:481-486).  (T)MAX_UINT is exactly 2^64.
+template <typename C> __device__ __forceinline__ C toUnit(u64 r);
+template <> __device__ __forceinline__ float toUnit<float>(u64 r) { return (float)r * 5.42101086242752217e-20f; }
+template <> __device__ __forceinline__ double toUnit<double>(u64 r) { return (double)r * 5.42101086242752217e-20; }
+
+template <typename TT> struct RandomCtx {
+    typedef typename Compute<TT>::type C;
+    RngState st;
+    Params<TT> args;
+    Long length;
+    __device__ __forceinline__ C unit(Long i) const {
+        C u = toUnit<C>(rngElement(st, i));
+        // storage types narrower than float round the draw to the storage type first (481-484)
+        if (sizeof(TT) < 4) u = toCompute(fromCompute<TT>(u));
+        return u;
+    }
+    __device__ __forceinline__ C unit(Long i, C from, C to) const { return from + (unit(i) * (to - from)); }
+};
+
+// Plain (non-special) ops.  nOperands: 1 = (z), 2 = (x, z), 3 = (x, y, z).  Overloads an op does not define
+// return the reference's marker values -1 / -2 / -3 (random_ops.h:15-17).
+template <int OP, typename TT>
+__device__ __forceinline__ typename Compute<TT>::type randomOp(const RandomCtx<TT> &c, int nOperands,
+                                                               typename Compute<TT>::type x,
+                                                               typename Compute<TT>::type y, Long i) {
+    typedef typename Compute<TT>::type C;
+    const C undefinedValue = nOperands == 1 ? (C)-1 : (nOperands == 2 ? (C)-2 : (C)-3);
+    switch (OP) {
+        case 0:  // UniformDistribution
+            if (nOperands != 1) return undefinedValue;
+            return c.unit(i, c.args[0], c.args[1]);
+        case 1:  // DropOut
+            if (nOperands != 2) return undefinedValue;
+            return c.unit(i) >= c.args[0] ? (C)0 : x;
+        case 2: {  // DropOutInverted
+            if (nOperands != 2) return undefinedValue;
+            C prob = c.args[0];
+            return c.unit(i) >= prob ? (C)0 : x / prob;
+        }
+        case 3:  // ProbablisticMerge
+            if (nOperands != 3) return undefinedValue;
+            return c.unit(i) <= c.args[0] ? y : x;
+        case 4: {  // Linspace
+            if (nOperands != 1) return undefinedValue;
+            C from = c.args[0];
+            C to = c.args[1];
+            C step = (C)i / ((C)c.length - (C)1);
+            return from * ((C)1 - step) + step * to;
+        }
+        case 7:  // BernoulliDistribution
+            if (nOperands == 1) return c.args[0] >= c.unit(i) ? (C)1 : (C)0;
+            if (nOperands == 2) return x >= c.unit(i) ? (C)1 : (C)0;
+            return undefinedValue;
+        case 12: {  // AlphaDropOut: args = p, a, b, alphaPrime
+            if (nOperands != 2) return undefinedValue;
+            C u = c.unit(i);
+            return u >= c.args[0] ? c.args[1] * c.args[3] + c.args[2] : c.args[1] * x + c.args[2];
+        }
+        case 13: {  // ExponentialDistribution
+            C lambda = c.args[0];
+            if (nOperands == 1) {
+                // DataTypeUtils::min<T>(): smallest positive normal of the data type
+                C lo = sizeof(TT) == 8 ? (C)2.2250738585072014e-308 : (sizeof(TT) == 4 ? (C)1.175494e-38f : (C)6.1035e-05f);
+                C v = c.unit(i, lo, (C)1);
+                return (C)1 - m::pow_((C)2.718281828459045, -(lambda * v));
+            }
+            if (nOperands == 2) return x <= (C)0 ? (C)0 : (C)1 - m::pow_((C)2.718281828459045, -(lambda * x));
+            return undefinedValue;
+        }
+        default:
+            // special ops reached through an overload without specialOp: marker values
+            return undefinedValue;
+    }
+}
+
+template <typename TT, int OP>
+__global__ void __launch_bounds__(kBlock) randomPlainKernel(RandomCtx<TT> c, const TT *x, const TT *y, TT *z, int nOperands,
+                                                            int strided, Long xEws, Long yEws, Long zEws, DimMap xm,
+                                                            DimMap ym, DimMap zm) {
+    typedef typename Compute<TT>::type C;
+    const Long stride = (Long)gridDim.x * kBlock;
+    for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < c.length; i += stride) {
+        Long ox, oy, oz;
+        if (strided) {
+            ox = i * xEws; oy = i * yEws; oz = i * zEws;
+        } else {
+            ox = nOperands >= 2 ? mapOffset32(xm, (unsigned)i) : 0;
+            oy = nOperands >= 3 ? mapOffset32(ym, (unsigned)i) : 0;
+            oz = mapOffset32(zm, (unsigned)i);
+        }
+        C xv = nOperands >= 2 ? toCompute(x[ox]) : (C)0;
+        C yv = nOperands >= 3 ? toCompute(y[oy]) : (C)0;
+        z[oz] = fromCompute<TT>(randomOp<OP, TT>(c, nOperands, xv, yv, i));
+    }
+}
+
+// Box-Muller pairs (2k, 2k+1) sharing u0 = draw(2k), u1 = draw(2k+1) (special_random_ops.h:333-396):
+// z[2k] = sqrt(-2 ln u0) cos(2 pi u1) * stddev + mean, z[2k+1] = ... sin(...).  EXP applies exp() on top
+// (LogNormal, 900-969).
+template <typename TT, bool EXP>
+__global__ void __launch_bounds__(kBlock) gaussianKernel(RandomCtx<TT> c, const TT *y, TT *z, int yIsZ, Long yEws, Long zEws) {
+    typedef typename Compute<TT>::type C;
+    const C twoPi = (C)(2.0 * 3.14159265358979323846);
+    const C mean = c.args[0];
+    const C stddev = c.args[1];
+    const Long pairs = (c.length + 1) / 2;
+    const Long stride = (Long)gridDim.x * kBlock;
+    for (Long k = (Long)blockIdx.x * kBlock + threadIdx.x; k < pairs; k += stride) {
+        const Long e = 2 * k;
+        C u0 = c.unit(e, (C)1e-5f, (C)1);
+        C u1 = c.unit(e + 1, (C)1e-5f, (C)1);
+        C r = m::sqrt_((C)-2 * m::log_(u0));
+        C ang = twoPi * u1;
+        C z0 = r * m::cos_(ang);
+        C z1 = r * m::sin_(ang);
+        C m0 = yIsZ ? mean : toCompute(y[e * yEws]);
+        C v0 = z0 * stddev + m0;
+        z[e * zEws] = fromCompute<TT>(EXP ? m::exp_(v0) : v0);
+        if (e + 1 < c.length) {
+            C m1 = yIsZ ? mean : toCompute(y[(e + 1) * yEws]);
+            C v1 = z1 * stddev + m1;
+            z[(e + 1) * zEws] = fromCompute<TT>(EXP ? m::exp_(v1) : v1);
+        }
+    }
+}
+
+// TruncatedNormal (special_random_ops.h:731-790): pairs (e, e + middle), redrawn with the index advanced
+// by zLength until both lie within two standard deviations.
+template <typename TT>
+__global__ void __launch_bounds__(kBlock) truncatedNormalKernel(RandomCtx<TT> c, const TT *y, TT *z, int yIsZ, Long yEws,
+                                                                Long zEws) {
+    typedef typename Compute<TT>::type C;
+    const C twoPi = (C)(2.0 * 3.14159265358979323846);
+    const C mean = c.args[0];
+    const C stddev = c.args[1];
+    const Long n = c.length;
+    const Long middle = (n % 2 == 0) ? n / 2 : n / 2 + 1;
+    const C ds = m::abs_(stddev) * (C)2;
+    const Long stride = (Long)gridDim.x * kBlock;
+    for (Long e = (Long)blockIdx.x * kBlock + threadIdx.x; e < middle; e += stride) {
+        C m0 = yIsZ ? mean : toCompute(y[e * yEws]);
+        C m1 = (yIsZ || e + middle >= n) ? (yIsZ ? mean : (C)0) : toCompute(y[(e + middle) * yEws]);
+        C r0 = (C)0, r1 = (C)0;
+        Long gen = 0;
+        // the acceptance probability per round is about 0.91; the bound only guarantees termination
+        for (int tries = 0; tries < 4096; tries++) {
+            C u0 = c.unit(e + gen, (C)1e-6f, (C)1);
+            C u1 = c.unit(e + middle + gen, (C)1e-6f, (C)1);
+            C l = m::sqrt_((C)-2 * m::log_(u0));
+            C ang = twoPi * u1;
+            r0 = (l * m::cos_(ang)) * stddev + m0;
+            r1 = (l * m::sin_(ang)) * stddev + m1;
+            gen += n;
+            if (!(m::abs_(m0) + m::abs_(r0) > ds || m::abs_(m1) + m::abs_(r1) > ds)) break;
+        }
+        z[e * zEws] = fromCompute<TT>(r0);
+        if (e + middle < n) z[(e + middle) * zEws] = fromCompute<TT>(r1);
+    }
+}
+
+// Binomial (405-520): trials draws at index (e+1)*t; probabilities args[1] or y[t-1] (EX: y[e], 531-650).
+template <typename TT, bool EX>
+__global__ void __launch_bounds__(kBlock) binomialKernel(RandomCtx<TT> c, const TT *y, TT *z, int yIsZ, Long yEws, Long zEws) {
+    typedef typename Compute<TT>::type C;
+    const int trials = m::toIntX86(c.args[0]);
+    const Long stride = (Long)gridDim.x * kBlock;
+    for (Long e = (Long)blockIdx.x * kBlock + threadIdx.x; e < c.length; e += stride) {
+        C prob = c.args[1];
+        int success = 0;
+        for (int t = 1; t <= trials; t++) {
+            C v = c.unit((e + 1) * t);
+            if (!yIsZ) prob = toCompute(y[(EX ? e : (Long)(t - 1)) * yEws]);
+            if (v < prob) success++;
+        }
+        z[e * zEws] = fromCompute<TT>((C)success);
+    }
+}
+
+// Choice (145-238): inverse CDF over probabilities y, values x.
+template <typename TT>
+__global__ void __launch_bounds__(kBlock) choiceKernel(RandomCtx<TT> c, const TT *x, const TT *y, TT *z, int strided,
+                                                       Long xEws, Long yEws, Long zEws, DimMap xm, DimMap ym, DimMap zm,
+                                                       Long yLength) {
+    typedef typename Compute<TT>::type C;
+    const Long stride = (Long)gridDim.x * kBlock;
+    for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < c.length; i += stride) {
+        C prob = c.unit(i);
+        C cum = (C)0;
+        Long oz = strided ? i * zEws : mapOffset32(zm, (unsigned)i);
+        for (Long f = 0; f < yLength; f++) {
+            // in the coordinate branch the reference indexes the probabilities with the OUTPUT index i
+            Long oy = strided ? f * yEws : mapOffset32(ym, (unsigned)i);
+            cum = toCompute(fromCompute<TT>(cum + toCompute(y[oy])));
+            if (prob <= cum || f == yLength - 1) {
+                Long ox = strided ? f * xEws : mapOffset32(xm, (unsigned)f);
+                z[oz] = x[ox];
+                break;
+            }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(kBlock) rngDumpKernel(RngState st, Long start, Long n, u64 *out) {
+    const Long stride = (Long)gridDim.x * kBlock;
+    for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) out[i] = rngElement(st, start + i);
+}
+
+__global__ void __launch_bounds__(kBlock) copyKernel(uint4 *dst, const uint4 *src, Long nvec, unsigned char *dtail,
+                                                     const unsigned char *stail, int tail) {
+    const Long stride = (Long)gridDim.x * kBlock;
+    for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += stride) dst[i] = src[i];
+    if (blockIdx.x == 0 && (int)threadIdx.x < tail) dtail[threadIdx.x] = stail[threadIdx.x];
+}
+
+template <typename T> struct RandomPlainBody {
+    template <int OP> struct Run {
+        static bool run(hipStream_t s, const RandomCtx<T> &c, const T *x, const T *y, T *z, const RandomPlan &pl,
+                        int operands) {
+            int grid = gridFor(pl.n, kBlock * 4, kGridCap);
+            hipLaunchKernelGGL((randomPlainKernel<T, OP>), dim3(grid), dim3(kBlock), 0, s, c, x, y, z, operands,
+                               pl.strided ? 1 : 0, pl.xEws, pl.yEws, pl.zEws, pl.xm, pl.ym, pl.zm);
+            return true;
+        }
+    };
+};
+
+template <typename T>
+bool launchRandom(hipStream_t s, int opNum, const RngState &rng, const T *x, const T *y, T *z, const T *args,
+                  const RandomPlan &pl, int operands, bool yIsZ) {
+    if (opNum < 0 || opNum > 13) return false;
+    if (pl.n <= 0) return true;
+    RandomCtx<T> c;
+    c.st = rng;
+    c.args.p = args;
+    c.length = pl.n;
+    const bool special = opNum == 5 || opNum == 6 || (opNum >= 8 && opNum <= 11);
+    if (special && operands == 3) {
+        int yz = yIsZ ? 1 : 0;
+        switch (opNum) {
+            case 5: {
+                int grid = gridFor(pl.n, kBlock, kGridCap);
+                hipLaunchKernelGGL((choiceKernel<T>), dim3(grid), dim3(kBlock), 0, s, c, x, y, z, pl.strided ? 1 : 0, pl.xEws,
+                                   pl.yEws, pl.zEws, pl.xm, pl.ym, pl.zm, pl.yLength);
+                break;
+            }
+            case 6: {
+                int grid = gridFor((pl.n + 1) / 2, kBlock * 2, kGridCap);
+                hipLaunchKernelGGL((gaussianKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                break;
+            }
+            case 10: {
+                int grid = gridFor((pl.n + 1) / 2, kBlock * 2, kGridCap);
+                hipLaunchKernelGGL((gaussianKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                break;
+            }
+            case 8: {
+                int grid = gridFor(pl.n, kBlock, kGridCap);
+                hipLaunchKernelGGL((binomialKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                break;
+            }
+            case 9: {
+                int grid = gridFor(pl.n, kBlock, kGridCap);
+                hipLaunchKernelGGL((binomialKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                break;
+            }
+            case 11: {
+                int grid = gridFor((pl.n + 1) / 2, kBlock, kGridCap);
+                hipLaunchKernelGGL((truncatedNormalKernel<T>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                break;
+            }
+        }
+        return true;
+    }
+    return dispatchSeq<RandomPlainBody<T>::template Run>(opNum, std::make_integer_sequence<int, 14>{}, s, c, x, y, z, pl,
+                                                         operands);
+}
+
+void launchRngDump(hipStream_t s, const RngState &rng, Long start, Long n, unsigned long long *out) {
+    if (n <= 0) return;
+    int grid = gridFor(n, kBlock * 4, kGridCap);
+    hipLaunchKernelGGL(rngDumpKernel, dim3(grid), dim3(kBlock), 0, s, rng, start, n, out);
+}
+
+void launchCopy(hipStream_t s, void *dst, const void *src, Long bytes) {
+    if (bytes <= 0) return;
+    Long nvec = bytes / 16;
+    int tail = (int)(bytes - nvec * 16);
+    int grid = gridFor(nvec > 0 ? nvec : 1, kBlock * 4, kGridCap);
+    hipLaunchKernelGGL(copyKernel, dim3(grid), dim3(kBlock), 0, s, reinterpret_cast<uint4 *>(dst),
+                       reinterpret_cast<const uint4 *>(src), nvec, reinterpret_cast<unsigned char *>(dst) + nvec * 16,
+                       reinterpret_cast<const unsigned char *>(src) + nvec * 16, tail);
+}
+
+#define INST(T)                                                                                                   \
+    template bool launchRandom<T>(hipStream_t, int, const RngState &, const T *, const T *, T *, const T *,        \
+                                  const RandomPlan &, int, bool);
+INST(float)
+INST(float16)
+INST(double)
+#undef INST
+
+}  // namespace nd4j_amd

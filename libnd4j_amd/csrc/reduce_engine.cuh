@@ -1,0 +1,297 @@
+// Reduction skeletons shared by the reduce, index-reduce and summary-stats families.
+//
+// A policy `Pol` supplies the accumulator and its algebra:
+//     typedef T (storage), C (compute), Acc
+//     Acc  init(const T *first)            starting accumulator (may read the first element of the run)
+//     void accumulate(Acc &, C v, Long i)  fold element i (its position inside the TAD / array)
+//     Acc  combine(Acc a, Acc b)           merge two partial accumulators
+//     T    finalize(Acc, Long n)           post-process into the stored result
+//     void setTad(Long r)                  per-TAD hook (LogSumExp reads its shift from the result array)
+//
+// Kernels:
+//   tadRowKernel<Pol, GROUP>  contiguous TADs (tadEws == 1): GROUP lanes walk one TAD with 16-byte loads,
+//                             wave64 cross-lane merge, LDS only across waves.
+//   tadColKernel<Pol>         strided TADs: one lane per TAD so that a row of adjacent TADs is one
+//                             coalesced request; the TAD length is split over blockIdx.y and merged by
+//                             tadColFinish when split.
+//   tadGeneralKernel<Pol>     block per TAD with a coordinate map.
+//   flatKernel<Pol> + flatFinish<Pol>  two-stage grid reduction over the whole array.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "elementwise.cuh"
+#include "types.h"
+#include "view.h"
+
+namespace nd4j_amd {
+
+static constexpr int kWave = 64;
+
+template <typename A> __device__ __forceinline__ A shflDownAny(A v, int delta) {
+    static_assert(sizeof(A) % 4 == 0, "accumulator must be a multiple of 4 bytes");
+    constexpr int W = sizeof(A) / 4;
+    struct Words { int w[W]; };
+    Words in = __builtin_bit_cast(Words, v);
+    Words out;
+#pragma unroll
+    for (int i = 0; i < W; i++) out.w[i] = __shfl_down(in.w[i], delta, kWave);
+    return __builtin_bit_cast(A, out);
+}
+
+// Merge over the lanes of one wave; lane 0 (of each WIDTH-lane segment) ends up with the result.
+template <class Pol, int WIDTH = kWave>
+__device__ __forceinline__ typename Pol::Acc waveMerge(const Pol &pol, typename Pol::Acc a) {
+#pragma unroll
+    for (int d = WIDTH / 2; d >= 1; d >>= 1) {
+        typename Pol::Acc o = shflDownAny(a, d);
+        a = pol.combine(a, o);
+    }
+    return a;
+}
+
+// Merge over a whole 256-thread block; thread 0 gets the result.  `smem` holds kBlock/kWave accumulators.
+template <class Pol>
+__device__ __forceinline__ typename Pol::Acc blockMerge(const Pol &pol, typename Pol::Acc a, typename Pol::Acc *smem) {
+    a = waveMerge<Pol>(pol, a);
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    __syncthreads();  // smem may still be read from a previous round
+    if (lane == 0) smem[wave] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < kBlock / kWave; w++) a = pol.combine(a, smem[w]);
+    }
+    return a;
+}
+
+// Folds n contiguous elements starting at `p` (element positions base.. in the run) using `lanes`
+// cooperating lanes, this lane being `lane`.
+template <class Pol>
+__device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc &acc, const typename Pol::T *p, Long n,
+                                               int lane, int lanes) {
+    typedef typename Pol::T T;
+    constexpr int VEC = Pack<T>::N;
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
+    Long head = 0;
+    if ((addr & (sizeof(T) - 1)) == 0) head = (Long)(((16 - (addr & 15)) & 15) / sizeof(T));
+    else head = n;  // cannot be vectorised
+    if (head > n) head = n;
+    for (Long i = lane; i < head; i += lanes) pol.accumulate(acc, toCompute(p[i]), i);
+    const Long nvec = (n - head) / VEC;
+    const Pack<T> *pv = reinterpret_cast<const Pack<T> *>(p + head);
+#pragma unroll 4
+    for (Long v = lane; v < nvec; v += lanes) {
+        Pack<T> pk = pv[v];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk.v[e]), head + v * VEC + e);
+    }
+    for (Long i = head + nvec * VEC + lane; i < n; i += lanes) pol.accumulate(acc, toCompute(p[i]), i);
+}
+
+template <class Pol, int GROUP>
+__global__ void __launch_bounds__(kBlock) tadRowKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
+                                                       const Long *offsets, Long tadLength, Long numTads) {
+    typedef typename Pol::Acc Acc;
+    constexpr int GROUPS = kBlock / GROUP;
+    __shared__ Acc smem[kBlock / kWave];
+    const int g = threadIdx.x / GROUP, lane = threadIdx.x % GROUP;
+    // GROUP == kBlock: every thread of the block runs the same trip count, so blockMerge may synchronise
+    for (Long r0 = (Long)blockIdx.x * GROUPS; r0 < numTads; r0 += (Long)gridDim.x * GROUPS) {
+        const Long r = r0 + g;
+        const bool live = r < numTads;
+        Acc acc;
+        if (live) {
+            pol.setTad(r, z);
+            const typename Pol::T *tx = x + offsets[r];
+            acc = pol.init(tx);
+            foldContiguous<Pol>(pol, acc, tx, tadLength, lane, GROUP);
+        }
+        if (GROUP == kBlock) {
+            acc = blockMerge<Pol>(pol, acc, smem);
+        } else {
+            if (live) acc = waveMerge<Pol, GROUP>(pol, acc);
+        }
+        if (live && lane == 0) z[r] = pol.finalize(acc, tadLength);
+    }
+}
+
+// Strided TADs: thread t <-> TAD t, rows [rowsPerSplit * blockIdx.y, ...) of each TAD.
+template <class Pol>
+__global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
+                                                       typename Pol::Acc *partials, const Long *offsets, Long tadLength,
+                                                       Long numTads, Long tadEws, Long rowsPerSplit) {
+    typedef typename Pol::Acc Acc;
+    const Long t = (Long)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= numTads) return;
+    pol.setTad(t, z);
+    const typename Pol::T *base = x + offsets[t];
+    Acc acc = pol.init(base);
+    const Long j0 = (Long)blockIdx.y * rowsPerSplit;
+    Long j1 = j0 + rowsPerSplit;
+    if (j1 > tadLength) j1 = tadLength;
+    Long j = j0;
+    for (; j + 8 <= j1; j += 8) {
+        typename Pol::T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = base[(j + u) * tadEws];
+#pragma unroll
+        for (int u = 0; u < 8; u++) pol.accumulate(acc, toCompute(v[u]), j + u);
+    }
+    for (; j < j1; j++) pol.accumulate(acc, toCompute(base[j * tadEws]), j);
+    if (gridDim.y == 1) z[t] = pol.finalize(acc, tadLength);
+    else partials[(Long)blockIdx.y * numTads + t] = acc;
+}
+
+template <class Pol>
+__global__ void __launch_bounds__(kBlock) tadColFinish(Pol pol, typename Pol::T *z, const typename Pol::Acc *partials,
+                                                       Long tadLength, Long numTads, int splits) {
+    const Long t = (Long)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= numTads) return;
+    pol.setTad(t, z);
+    typename Pol::Acc acc = partials[t];
+    for (int s = 1; s < splits; s++) acc = pol.combine(acc, partials[(Long)s * numTads + t]);
+    z[t] = pol.finalize(acc, tadLength);
+}
+
+template <class Pol>
+__global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
+                                                           const Long *offsets, DimMap tm, Long tadLength, Long numTads) {
+    typedef typename Pol::Acc Acc;
+    __shared__ Acc smem[kBlock / kWave];
+    for (Long r = blockIdx.x; r < numTads; r += gridDim.x) {
+        pol.setTad(r, z);
+        const typename Pol::T *tx = x + offsets[r];
+        Acc acc = pol.init(tx);
+        for (Long f = threadIdx.x; f < tadLength; f += kBlock)
+            pol.accumulate(acc, toCompute(tx[mapOffset32(tm, (unsigned)f)]), f);
+        acc = blockMerge<Pol>(pol, acc, smem);
+        if (threadIdx.x == 0) z[r] = pol.finalize(acc, tadLength);
+    }
+}
+
+// Stage 1 of the full-array reduction: block b folds the chunks b, b+grid, ... of kBlock*kUnroll vectors.
+template <class Pol>
+__global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol::T *x, typename Pol::Acc *partials,
+                                                     Long n, int strided, Long ews, DimMap xm) {
+    typedef typename Pol::T T;
+    typedef typename Pol::Acc Acc;
+    __shared__ Acc smem[kBlock / kWave];
+    pol.setTad(0, nullptr);
+    Acc acc = pol.init(x);
+    if (strided && ews == 1) {
+        constexpr int VEC = Pack<T>::N;
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
+        Long head = ((addr & (sizeof(T) - 1)) == 0) ? (Long)(((16 - (addr & 15)) & 15) / sizeof(T)) : n;
+        if (head > n) head = n;
+        const Long nvec = (n - head) / VEC;
+        const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x + head);
+        const Long chunk = (Long)kBlock * kUnroll;
+        for (Long b = (Long)blockIdx.x * chunk; b < nvec; b += (Long)gridDim.x * chunk) {
+            Pack<T> pk[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                Long v = b + u * kBlock + threadIdx.x;
+                if (v < nvec) pk[u] = xv[v];
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                Long v = b + u * kBlock + threadIdx.x;
+                if (v < nvec) {
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[u].v[e]), head + v * VEC + e);
+                }
+            }
+        }
+        if (blockIdx.x == 0) {
+            for (Long i = threadIdx.x; i < head; i += kBlock) pol.accumulate(acc, toCompute(x[i]), i);
+            for (Long i = head + nvec * VEC + threadIdx.x; i < n; i += kBlock) pol.accumulate(acc, toCompute(x[i]), i);
+        }
+    } else if (strided) {
+        for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock)
+            pol.accumulate(acc, toCompute(x[i * ews]), i);
+    } else {
+        for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock)
+            pol.accumulate(acc, toCompute(x[mapOffset32(xm, (unsigned)i)]), i);
+    }
+    acc = blockMerge<Pol>(pol, acc, smem);
+    if (threadIdx.x == 0) partials[blockIdx.x] = acc;
+}
+
+template <class Pol>
+__global__ void __launch_bounds__(kBlock) flatFinish(Pol pol, const typename Pol::T *x, typename Pol::T *z,
+                                                     const typename Pol::Acc *partials, int count, Long n) {
+    typedef typename Pol::Acc Acc;
+    __shared__ Acc smem[kBlock / kWave];
+    pol.setTad(0, nullptr);
+    Acc acc = pol.init(x);
+    for (int i = threadIdx.x; i < count; i += kBlock) acc = pol.combine(acc, partials[i]);
+    acc = blockMerge<Pol>(pol, acc, smem);
+    if (threadIdx.x == 0) z[0] = pol.finalize(acc, n);
+}
+
+// ---- host launch logic shared by the three families ---------------------------------------------------
+template <class Pol>
+inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typename Pol::T *z, const TadPlan &pl,
+                         Workspace ws) {
+    typedef typename Pol::Acc Acc;
+    if (pl.numTads <= 0) return;
+    if (pl.kind == TadPlan::ROW && pl.tadLength >= 32) {
+        if (pl.tadLength >= 8192) {
+            int grid = gridFor(pl.numTads, 1, kGridCap);
+            hipLaunchKernelGGL((tadRowKernel<Pol, kBlock>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets,
+                               pl.tadLength, pl.numTads);
+        } else if (pl.tadLength >= 256) {
+            int grid = gridFor(pl.numTads, kBlock / 64, kGridCap);
+            hipLaunchKernelGGL((tadRowKernel<Pol, 64>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets,
+                               pl.tadLength, pl.numTads);
+        } else {
+            int grid = gridFor(pl.numTads, kBlock / 16, kGridCap);
+            hipLaunchKernelGGL((tadRowKernel<Pol, 16>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets,
+                               pl.tadLength, pl.numTads);
+        }
+        return;
+    }
+    if (pl.kind == TadPlan::ROW || pl.kind == TadPlan::COL) {
+        // one lane per TAD; split the TAD length so that the grid fills the chip
+        int gx = (int)((pl.numTads + kBlock - 1) / kBlock);
+        Long splits = 2048 / gx;
+        if (splits < 1) splits = 1;
+        Long maxSplitsByRows = (pl.tadLength + 31) / 32;  // at least 32 rows per split
+        if (splits > maxSplitsByRows) splits = maxSplitsByRows;
+        size_t need = (size_t)splits * (size_t)pl.numTads * sizeof(Acc);
+        while (splits > 1 && need > ws.bytes) { splits /= 2; need = (size_t)splits * (size_t)pl.numTads * sizeof(Acc); }
+        if (splits < 1) splits = 1;
+        Long rowsPerSplit = (pl.tadLength + splits - 1) / splits;
+        splits = (pl.tadLength + rowsPerSplit - 1) / rowsPerSplit;
+        if (splits < 1) splits = 1;
+        Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+        hipLaunchKernelGGL((tadColKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
+                           pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit);
+        if (splits > 1)
+            hipLaunchKernelGGL((tadColFinish<Pol>), dim3(gx), dim3(kBlock), 0, s, pol, z, partials, pl.tadLength,
+                               pl.numTads, (int)splits);
+        return;
+    }
+    int grid = gridFor(pl.numTads, 1, kGridCap);
+    hipLaunchKernelGGL((tadGeneralKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets, pl.tm, pl.tadLength,
+                       pl.numTads);
+}
+
+template <class Pol>
+inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typename Pol::T *z, const FlatPlan &pl,
+                          Workspace ws) {
+    typedef typename Pol::Acc Acc;
+    typedef typename Pol::T T;
+    Long perBlock = (Long)kBlock * kUnroll * Pack<T>::N;
+    int grid = gridFor(pl.n, perBlock, 2048);
+    size_t maxByWs = ws.bytes / sizeof(Acc);
+    if ((size_t)grid > maxByWs) grid = (int)maxByWs;
+    if (grid < 1) grid = 1;
+    Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+    hipLaunchKernelGGL((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
+                       pl.ews, pl.xm);
+    hipLaunchKernelGGL((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n);
+}
+
+}  // namespace nd4j_amd

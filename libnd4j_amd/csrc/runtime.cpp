@@ -1,0 +1,162 @@
+#include "runtime.h"
+
+#include <map>
+#include <mutex>
+#include <utility>
+
+namespace nd4j_amd {
+
+Environment &environment() {
+    static Environment env;
+    return env;
+}
+
+bool isDeviceMemory(const void *p) {
+    if (p == nullptr) return false;
+    hipPointerAttribute_t attr;
+    hipError_t e = hipPointerGetAttributes(&attr, p);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();  // plain (unregistered) host memory reports an error: clear it
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice;
+}
+
+static void throwHip(const char *what, hipError_t e) {
+    throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+const Long *hostShapeInfo(Nd4jPointer *extra, int slot, const Long *arg, std::vector<Long> &storage, hipStream_t s) {
+    if (void *h = slotOf(extra, slot)) return reinterpret_cast<const Long *>(h);
+    if (arg == nullptr) return nullptr;
+    if (!isDeviceMemory(arg)) return arg;
+    Long rank = 0;
+    hipError_t e = hipMemcpyAsync(&rank, arg, sizeof(Long), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) throwHip("fetching shapeInfo rank", e);
+    if (rank < 0 || rank > kMaxRank) throw std::runtime_error("shapeInfo rank out of range");
+    storage.resize(siLength((int)rank));
+    e = hipMemcpyAsync(storage.data(), arg, storage.size() * sizeof(Long), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) throwHip("fetching shapeInfo", e);
+    return storage.data();
+}
+
+bool hostInts(const int *arg, int count, std::vector<int> &out, hipStream_t s) {
+    out.clear();
+    if (arg == nullptr || count <= 0) return false;
+    out.resize(count);
+    if (!isDeviceMemory(arg)) {
+        for (int i = 0; i < count; i++) out[i] = arg[i];
+        return true;
+    }
+    hipError_t e = hipMemcpyAsync(out.data(), arg, count * sizeof(int), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) throwHip("fetching dimension", e);
+    return true;
+}
+
+void checkLaunch(const char *what, hipStream_t s) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) throwHip(what, e);
+    if (environment().debug.load()) {
+        e = hipStreamSynchronize(s);
+        if (e != hipSuccess) throwHip(what, e);
+    }
+}
+
+void syncAndCheck(const char *what, hipStream_t s) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) throwHip(what, e);
+    e = hipStreamSynchronize(s);
+    if (e != hipSuccess) throwHip(what, e);
+}
+
+void reportUnknownOp(const char *family, int opNum) {
+    // the reference prints and carries on without touching the output (op_boilerplate.h:1148)
+    printf("[ERROR] Unknown opNum=%d for %s on %s:%d\n", opNum, family, __FILE__, __LINE__);
+    fflush(stdout);
+}
+
+namespace {
+std::mutex gMutex;
+std::map<std::pair<int, hipStream_t>, Workspace> gWorkspaces;
+
+struct CachedTad {
+    TadPack pack;
+    Long *devOffsets = nullptr;
+    Long tadLength = 0;
+};
+std::map<std::vector<Long>, CachedTad *> gTadCache;
+}  // namespace
+
+Workspace workspaceFor(hipStream_t s, size_t minBytes) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    std::lock_guard<std::mutex> lock(gMutex);
+    Workspace &w = gWorkspaces[std::make_pair(dev, s)];
+    if (w.ptr != nullptr && w.bytes >= minBytes) return w;
+    size_t want = minBytes < (size_t)(8u << 20) ? (size_t)(8u << 20) : minBytes;
+    if (w.ptr != nullptr) {
+        // earlier work on this stream may still use the old block
+        (void)hipStreamSynchronize(s);
+        (void)hipFree(w.ptr);
+        w.ptr = nullptr;
+        w.bytes = 0;
+    }
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, want);
+    if (e != hipSuccess) throwHip("workspace allocation", e);
+    w.ptr = p;
+    w.bytes = want;
+    return w;
+}
+
+bool resolveTad(Nd4jPointer *extra, int hostSlot, int offsetSlot, const Long *hostXInfo, const int *dimension,
+                int dimLen, ResolvedTad &out, hipStream_t s) {
+    const Long *hostTad = reinterpret_cast<const Long *>(slotOf(extra, hostSlot));
+    const Long *devOff = reinterpret_cast<const Long *>(slotOf(extra, offsetSlot));
+    if (hostTad != nullptr && devOff != nullptr) {
+        out.hostInfo = hostTad;
+        out.devOffsets = devOff;
+        out.tadLength = siNumel(hostTad);
+        out.numTads = out.tadLength > 0 ? siNumel(hostXInfo) / out.tadLength : 0;
+        return true;
+    }
+    std::vector<int> dims;
+    if (!hostInts(dimension, dimLen, dims, s)) return false;
+    int rank = siRank(hostXInfo);
+    for (int &d : dims) {
+        if (d < 0) d += rank;
+        if (d < 0 || d >= rank) return false;
+    }
+    std::vector<Long> key(hostXInfo, hostXInfo + siLength(rank));
+    key.push_back(-777);
+    for (int d : dims) key.push_back(d);
+
+    std::lock_guard<std::mutex> lock(gMutex);
+    auto it = gTadCache.find(key);
+    CachedTad *c = nullptr;
+    if (it != gTadCache.end()) {
+        c = it->second;
+    } else {
+        c = new CachedTad();
+        computeTad(hostXInfo, dims.data(), dimLen, c->pack, true);
+        c->tadLength = tadLengthOf(hostXInfo, dims.data(), dimLen);
+        size_t bytes = c->pack.offsets.size() * sizeof(Long);
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&c->devOffsets), bytes ? bytes : sizeof(Long));
+        if (e != hipSuccess) { delete c; throwHip("TAD offsets allocation", e); }
+        if (bytes) {
+            e = hipMemcpy(c->devOffsets, c->pack.offsets.data(), bytes, hipMemcpyHostToDevice);
+            if (e != hipSuccess) { (void)hipFree(c->devOffsets); delete c; throwHip("TAD offsets upload", e); }
+        }
+        gTadCache[key] = c;
+    }
+    out.hostInfo = c->pack.shapeInfo.data();
+    out.devOffsets = c->devOffsets;
+    out.numTads = c->pack.numTads;
+    out.tadLength = c->tadLength;
+    return true;
+}
+
+}  // namespace nd4j_amd

@@ -1,0 +1,86 @@
+// Host runtime shared by the boundary translation units: environment switches, extraPointers decoding,
+// shapeInfo fetching, the per-stream workspace and the TAD cache.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdio>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "launch.h"
+#include "shape_host.h"
+#include "types.h"
+
+namespace nd4j_amd {
+
+// Runtime switches, the counterpart of nd4j::Environment (reference: blas/Environment.cpp:13-33).
+struct Environment {
+    std::atomic<bool> debug{false};
+    std::atomic<bool> verbose{false};
+    std::atomic<int> elementThreshold{1024};
+    std::atomic<int> tadThreshold{8};
+    std::atomic<int> gridLimit{8192};
+    std::atomic<int> maxThreads{512};
+};
+Environment &environment();
+
+// extraPointers slots of the reference's CUDA convention (blas/cuda/NativeOps.cu:1609-1624,1813-1823).
+enum ExtraSlot {
+    X_HOST_X_SHAPE = 0,
+    X_STREAM = 1,
+    X_DEVICE_ID = 2,
+    X_ALLOCATION = 3,
+    X_REDUCTION = 4,
+    X_RESULT = 5,
+    X_SPECIAL = 6,
+    X_HOST_Y_SHAPE = 7,
+    X_HOST_Z_SHAPE = 8,
+    X_HOST_TAD_SHAPE = 9,
+    X_DEV_TAD_SHAPE = 10,
+    X_DEV_TAD_OFFSETS = 11,
+    X_DEV_TAD_SHAPE_Z = 12,
+    X_DEV_TAD_OFFSETS_Z = 13,
+};
+
+inline hipStream_t streamOf(Nd4jPointer *extra) { return extra ? reinterpret_cast<hipStream_t>(extra[X_STREAM]) : nullptr; }
+inline void *slotOf(Nd4jPointer *extra, int slot) { return extra ? extra[slot] : nullptr; }
+
+// true when the pointer refers to device memory that the host must not dereference
+bool isDeviceMemory(const void *p);
+
+// Returns a host-readable shapeInfo: the host copy in extraPointers[slot] when present, else the
+// argument itself when it is host memory, else a copy fetched from the device into `storage` (this
+// last case synchronises the stream).  Null when there is nothing to read.
+const Long *hostShapeInfo(Nd4jPointer *extra, int slot, const Long *arg, std::vector<Long> &storage, hipStream_t s);
+
+// Host copy of a small int array argument (`dimension`), which is a device pointer on this convention.
+bool hostInts(const int *arg, int count, std::vector<int> &out, hipStream_t s);
+
+// Throws std::runtime_error when the launch failed; in debug mode also synchronises the stream and
+// reports asynchronous errors (reference: include/helpers/DebugHelper.h:31-57, op_boilerplate.h:96-97).
+void checkLaunch(const char *what, hipStream_t s);
+// Synchronise + check, for scalar-returning members.
+void syncAndCheck(const char *what, hipStream_t s);
+
+void reportUnknownOp(const char *family, int opNum);
+
+// Device scratch owned by the library, one per (device, stream), allocated on first use and kept.
+Workspace workspaceFor(hipStream_t s, size_t minBytes);
+
+// TAD tables resolved for a call: host shapeInfo of one TAD + device offsets.
+struct ResolvedTad {
+    const Long *hostInfo = nullptr;
+    const Long *devOffsets = nullptr;
+    Long numTads = 0;
+    Long tadLength = 0;
+};
+// Uses extraPointers[hostSlot]/[offsetSlot] when both are present; otherwise computes the TAD from the
+// host xShapeInfo and `dimension` (fetched from the device if needed), uploads the offsets once and caches
+// them by (shapeInfo, dimension).
+bool resolveTad(Nd4jPointer *extra, int hostSlot, int offsetSlot, const Long *hostXInfo, const int *dimension,
+                int dimLen, ResolvedTad &out, hipStream_t s);
+
+}  // namespace nd4j_amd
