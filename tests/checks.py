@@ -1,0 +1,363 @@
+"""Parity checks that take a backend (tests/backends.py), so the CPU oracle and the HIP path are held to the
+same known answers:
+
+  * the golden values of the reference's own unit tests (tests/golden/reference_fixtures.json);
+  * vectors produced by the compiled reference (tests/golden/ref_vectors.json);
+  * closed forms that do not come from the code under test (numpy / brute force).
+
+Tolerances (from the task statement): bit-exact for indices and the generator's integer stream, at most 2 ULP
+for fp32 elementwise results, relative error 1e-5 for fp32 reductions, 1e-2 for fp16.
+"""
+import json
+import os
+
+import numpy as np
+
+from golden_inputs import (BROADCAST_OPS, INDEX_OPS, PAIRWISE_OPS, REDUCE_OPS, TRANSFORM_OPS, from_hexbits, op_extra,
+                           pairwise_inputs, reduce_input, shape_info_np, transform_input, ulp_distance)
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ELEMENTWISE_ULP = 2
+REDUCE_RTOL = 1e-5
+HALF_RTOL = 1e-2
+
+
+def load_json(name):
+    with open(os.path.join(HERE, "golden", name)) as f:
+        return json.load(f)
+
+
+def assert_ulp(got, want, max_ulp, what):
+    got = np.asarray(got)
+    want = np.asarray(want)
+    assert got.shape == want.shape, "%s: shape %s vs %s" % (what, got.shape, want.shape)
+    d = ulp_distance(got, want)
+    nan_mismatch = np.isnan(got) != np.isnan(want)
+    assert not nan_mismatch.any(), "%s: NaN pattern differs at %s" % (what, np.nonzero(nan_mismatch)[0][:5])
+    worst = int(d.max()) if d.size else 0
+    assert worst <= max_ulp, "%s: %d ULP at index %d (got %r, want %r)" % (
+        what, worst, int(d.argmax()), got.flat[int(d.argmax())], want.flat[int(d.argmax())])
+
+
+def assert_reduction_close(got, want, scale, what, rtol=REDUCE_RTOL):
+    """|got - want| <= rtol * max(|want|, scale).  `scale` is the natural magnitude of the accumulation (for a
+    sum: the sum of magnitudes over sqrt(n)), which keeps the bound meaningful where a sum cancels to ~0."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    assert np.array_equal(np.isnan(got), np.isnan(want)), "%s: NaN pattern differs" % what
+    bound = rtol * np.maximum(np.abs(want), scale)
+    err = np.abs(got - want)
+    ok = (err <= bound) | (np.isnan(want)) | (got == want)
+    assert ok.all(), "%s: |err| %g > bound %g at %d (got %r want %r)" % (
+        what, err[~ok].max(), bound[~ok][0], int(np.nonzero(~ok)[0][0]), got[~ok][0], want[~ok][0])
+
+
+# ---------------------------------------------------------------------------------------------------------
+# fixtures of the reference's own tests
+
+def check_reference_fixtures(be):
+    fx = load_json("reference_fixtures.json")
+    f32 = np.float32
+    for c in fx["transform"]:
+        shape = c["shape"]
+        n = int(np.prod(shape))
+        x = np.array(c["x"], f32) if "x" in c else np.full(n, c["fill"], f32)
+        want = np.array(c["expected"], f32) if "expected" in c else np.full(n, c["expected_fill"], f32)
+        extra = np.array(c["extra"], f32) if "extra" in c else None
+        info = shape_info_np(shape)
+        got = be.transform(c["opNum"], x, info, info, extra)
+        assert np.array_equal(got, want), c["source"]
+    for c in fx["pairwise"]:
+        n = int(np.prod(c["shape"]))
+        info = shape_info_np(c["shape"])
+        got = be.pairwise(c["opNum"], np.full(n, c["x_fill"], f32), info, np.full(n, c["y_fill"], f32), info, info)
+        assert np.array_equal(got, np.full(n, c["expected_fill"], f32)), c["source"]
+    for c in fx["broadcast"]:
+        xi = np.array(c["x_info"], np.int64)
+        got = be.broadcast(c["opNum"], np.array(c["x"], f32), xi, np.array(c["y"], f32), np.array(c["y_info"], np.int64),
+                           xi, c["dims"])
+        assert np.array_equal(got, np.array(c["expected"], f32)), c["source"]
+    for c in fx["reduce"]:
+        shape = c["shape"]
+        if "row_pattern" in c:
+            k = np.arange(1, shape[0] + 1, dtype=f32)[:, None]
+            x = (k * np.array(c["row_pattern"], f32)[None, :]).reshape(-1)
+        else:
+            x = np.array(c["x"], f32)
+        got = be.reduce(c["opNum"], x, shape_info_np(shape), None, c["dims"], len(c["expected"]))
+        assert np.array_equal(got, np.array(c["expected"], f32)), c["source"]
+    for c in fx["reduce_scalar"]:
+        got = be.reduce_scalar(c["opNum"], np.array(c["x"], f32), shape_info_np(c["shape"]))
+        assert float(got) == c["expected"], c["source"]
+    for c in fx["index_reduce"]:
+        xi = np.array(c["x_info"], np.int64)
+        x = np.array(c["x"], f32) if "x" in c else np.linspace(c["linspace"][0], c["linspace"][1], int(np.prod(xi[1:1 + xi[0]]))).astype(f32)
+        got = be.indexreduce(c["opNum"], x, xi, None, c["dims"], len(c["expected"]))
+        assert np.array_equal(got, np.array(c["expected"], f32)), c["source"]
+    for c in fx["index_reduce_scalar"]:
+        xi = np.array(c["x_info"], np.int64)
+        x = np.linspace(c["linspace"][0], c["linspace"][1], 25).astype(f32)
+        assert float(be.indexreduce_scalar(c["opNum"], x, xi)) == c["expected"], c["source"]
+    for c in fx["summary_stats"]:
+        got = be.summarystats(c["opNum"], c["bias"], np.array(c["x"], f32), shape_info_np(c["shape"]), c["dims"],
+                              len(c["expected"]))
+        assert np.allclose(got, c["expected"], atol=c["tol"], rtol=0), c["source"]
+    for c in fx["summary_stats_scalar"]:
+        if "x" in c:
+            x = np.array(c["x"], f32)
+            shape = c["shape"]
+        else:
+            n = c["n"]
+            base, amp = c["alternating"]
+            x = (f32(base) + np.where(np.arange(n) % 2 == 1, f32(amp), -f32(amp))).astype(f32)
+            shape = [1, n]
+        got = be.summarystats_scalar(c["opNum"], c["bias"], x, shape_info_np(shape))
+        assert abs(float(got) - c["expected"]) <= c["tol"], "%s: %r" % (c["source"], got)
+
+
+def check_tad_fixtures(tad_fn):
+    """tad_fn(x_info, dims) -> (tadShapeInfo, offsets)."""
+    fx = load_json("reference_fixtures.json")
+    for c in fx["tad_shape_info"]:
+        ti, _ = tad_fn(np.array(c["x_info"], np.int64), c["dims"])
+        assert [int(v) for v in ti] == c["tad_info"], "%s: %s" % (c["source"], list(ti))
+    for c in fx["tad_offsets"]:
+        _, off = tad_fn(np.array(c["x_info"], np.int64), c["dims"])
+        assert [int(v) for v in off] == c["offsets"], c["source"]
+    for c in fx["tad_ews"]:
+        info = shape_info_np(c["shape"], c["order"])
+        ti, off = tad_fn(info, c["dims"])
+        r = int(ti[0])
+        assert int(ti[2 * r + 2]) == c["ews"], c["source"]
+        assert len(off) == c["result_length"], c["source"]
+    for c in fx["shape_info"]:
+        info = shape_info_np(c["shape"], c["order"])
+        r = len(c["shape"])
+        assert [int(v) for v in info[1 + r:1 + 2 * r]] == c["strides"], c["source"]
+    vec = load_json("ref_vectors.json")
+    for c in vec["tad"]:
+        info = shape_info_np(c["shape"], c["order"])
+        assert [int(v) for v in info] == c["x_info"], "shapeInfo of %s %s" % (c["shape"], c["order"])
+        ti, off = tad_fn(info, c["dims"])
+        assert [int(v) for v in ti] == c["tad_info"], "TAD shapeInfo %s %s %s" % (c["shape"], c["order"], c["dims"])
+        assert len(off) == c["num_tads"]
+        assert [int(v) for v in off[:8]] == c["offsets_head"] and [int(v) for v in off[-3:]] == c["offsets_tail"]
+        assert int(np.sum(off)) == c["offsets_sum"]
+
+
+# ---------------------------------------------------------------------------------------------------------
+# vectors of the compiled reference
+
+def check_op_vectors(be, max_ulp=ELEMENTWISE_ULP):
+    vec = load_json("ref_vectors.json")["ops"]
+    f32 = np.float32
+    x = transform_input()
+    xi = shape_info_np([1, x.size])
+    for op in TRANSFORM_OPS:
+        want = from_hexbits(vec["transform_f32"][str(op)], f32)
+        got = be.transform(op, x, xi, xi, op_extra("transform", op))
+        assert_ulp(got, want, max_ulp, "transform op %d" % op)
+    a, b = pairwise_inputs()
+    ai = shape_info_np([1, a.size])
+    for op in PAIRWISE_OPS:
+        want = from_hexbits(vec["pairwise_f32"][str(op)], f32)
+        got = be.pairwise(op, a, ai, b, ai, ai, op_extra("pairwise", op))
+        # LogPoisonLossFull (94) is a five-term float sum that the reference's -fassociative-math build is free to
+        # reorder; its vectors are reproduced to a few ULP only
+        assert_ulp(got, want, 8 if op == 94 else max_ulp, "pairwise op %d" % op)
+    bxi = shape_info_np([12, 8])
+    for op in BROADCAST_OPS:
+        want = from_hexbits(vec["broadcast_f32_12x8"][str(op)]["dim1"], f32)
+        got = be.broadcast(op, a, bxi, b[:8].copy(), shape_info_np([1, 8]), bxi, [1])
+        assert_ulp(got, want, max_ulp, "broadcast op %d dim 1" % op)
+        want = from_hexbits(vec["broadcast_f32_12x8"][str(op)]["dim0"], f32)
+        got = be.broadcast(op, a, bxi, b[8:20].copy(), shape_info_np([12, 1]), bxi, [0])
+        assert_ulp(got, want, max_ulp, "broadcast op %d dim 0" % op)
+    m = reduce_input()
+    mi = shape_info_np([12, 10])
+    scale = float(np.abs(m).sum())
+    for op in REDUCE_OPS:
+        e = op_extra("reduce", op)
+        w = vec["reduce_f32_12x10"][str(op)]
+        assert_reduction_close(be.reduce(op, m, mi, e, [1], 12), from_hexbits(w["dim1"], f32), scale * 1e-2, "reduce op %d dim 1" % op)
+        assert_reduction_close(be.reduce(op, m, mi, e, [0], 10), from_hexbits(w["dim0"], f32), scale * 1e-2, "reduce op %d dim 0" % op)
+        assert_reduction_close([be.reduce_scalar(op, m, mi, e)], from_hexbits(w["scalar"], f32), scale * 1e-2, "reduce op %d scalar" % op)
+    for op in INDEX_OPS:
+        e = op_extra("indexreduce", op)
+        w = vec["indexreduce_f32_12x10"][str(op)]
+        assert np.array_equal(be.indexreduce(op, m, mi, e, [1], 12), from_hexbits(w["dim1"], f32)), "index op %d dim 1" % op
+        assert np.array_equal(be.indexreduce(op, m, mi, e, [0], 10), from_hexbits(w["dim0"], f32)), "index op %d dim 0" % op
+        assert f32(be.indexreduce_scalar(op, m, mi, e)) == from_hexbits(w["scalar"], f32)[0], "index op %d scalar" % op
+    for op in (0, 1):
+        for bias in (0, 1):
+            w = vec["summarystats_f32_12x10"]["%d_%d" % (op, bias)]
+            assert_reduction_close(be.summarystats(op, bias, m, mi, [1], 12), from_hexbits(w["dim1"], f32), 0, "stats %d/%d dim 1" % (op, bias))
+            assert_reduction_close(be.summarystats(op, bias, m, mi, [0], 10), from_hexbits(w["dim0"], f32), 0, "stats %d/%d dim 0" % (op, bias))
+            assert_reduction_close([be.summarystats_scalar(op, bias, m, mi)], from_hexbits(w["scalar"], f32), 0, "stats %d/%d scalar" % (op, bias))
+
+
+def check_half_vectors(be, exact):
+    """fp16 known answers of the reference's float16 loops.  `exact`: the CPU checkers reproduce them bit for
+    bit (same per-operation rounding); the HIP path computes in fp32 and rounds once, so it is held to 1e-2."""
+    vec = load_json("ref_vectors.json")["ops"]["f16_2x4"]
+    h = np.float16
+    xh = (0.1 * (np.arange(8, dtype=np.float32) + 1)).astype(h)
+    yh = (1000 + np.arange(8, dtype=np.float32)).astype(h)
+    hi = shape_info_np([2, 4])
+    rowh = (0.333 * np.arange(4, dtype=np.float32)).astype(h)
+
+    def cmp(got, key):
+        want = from_hexbits(vec[key], h)
+        if exact:
+            assert np.array_equal(np.asarray(got).view(np.uint16), want.view(np.uint16)), key
+        else:
+            g, w = np.asarray(got, np.float64), want.astype(np.float64)
+            assert np.all(np.abs(g - w) <= HALF_RTOL * np.abs(w)), key
+
+    cmp(be.pairwise(0, xh, hi, yh, hi, hi), "pairwise_add")
+    cmp(be.pairwise(6, xh, hi, yh, hi, hi), "pairwise_multiply")
+    cmp(be.transform(15, xh, hi, hi), "transform_tanh")
+    cmp(be.broadcast(0, xh, hi, rowh, shape_info_np([1, 4]), hi, [1]), "broadcast_add_row")
+    cmp(np.array([be.reduce_scalar(1, yh, hi)], h), "reduce_sum_y")
+
+
+def check_rng_vectors(be, float_ulp=ELEMENTWISE_ULP, big=True):
+    vec = load_json("ref_vectors.json")["rng"]
+    u64 = np.uint64
+    for c in vec["small"]:
+        g = be.rng(c["seed"], c["size"])
+        for kind, v in c["ops"]:
+            if kind == "rewind":
+                g.rewind(v)
+            elif kind == "reseed":
+                g.reseed(v)
+        assert list(g.state()) == c["state"], "state %s" % c
+        got = g.elements(0, 400)
+        assert np.array_equal(got, np.array(c["elements_0_400"], u64)), "stream seed %d size %d ops %s" % (c["seed"], c["size"], c["ops"])
+        g.destroy()
+    if big:
+        c = vec["seed119_size2p20"]
+        g = be.rng(119, 1 << 20)
+        assert [int(v) for v in g.buffer[:8]] == c["buffer_head"] and [int(v) for v in g.buffer[-2:]] == c["buffer_tail"]
+        probe = c["probe_index"]
+        assert [int(g.elements(i, 1)[0]) for i in probe] == c["fresh"]
+        g.destroy()
+    seq = vec["float_sequence_seed119_size4096"]
+    g = be.rng(119, 4096)
+    f32 = np.float32
+    for s in seq:
+        n = s["n"]
+        want = from_hexbits(s["out"], f32)
+        x = np.arange(n, dtype=f32) + 1
+        if s["overload"] == "z":
+            got = g.random_z(s["op"], n, s["args"])
+        elif s["overload"] == "xz_inplace":
+            got = g.random_xz(s["op"], x, s["args"], inplace=True)
+        elif s["overload"] == "xz":
+            got = g.random_xz(s["op"], x, s["args"], inplace=False)
+        elif s["overload"] == "xyz_inplace":
+            got = g.random_xyz(s["op"], None, None, s["args"], mode="inplace_all", n=n)
+        else:
+            got = g.random_xyz(s["op"], x, -np.arange(n, dtype=f32), s["args"])
+        exact_ops = (1, 2, 3, 4, 7, 8, 12)  # selections, integer counts, plain arithmetic
+        assert_ulp(got, want, 0 if s["op"] in exact_ops else float_ulp, "random op %d (%s)" % (s["op"], s["overload"]))
+        assert list(g.state()) == s["state"], "state after random op %d: %s vs %s" % (s["op"], g.state(), s["state"])
+    g.destroy()
+
+
+# ---------------------------------------------------------------------------------------------------------
+# closed forms independent of the code under test
+
+def check_closed_forms(be):
+    f32 = np.float32
+    rs = np.random.RandomState(5)
+    # elementwise: the mathematical function evaluated in float64 and rounded once; the C library's float
+    # routines are within 2 ULP of that
+    x = rs.uniform(-4, 4, 4099).astype(f32)
+    xi = shape_info_np([1, x.size])
+    for op, fn in ((15, np.tanh), (3, np.exp), (0, np.abs), (12, np.sin), (2, np.cos), (6, np.negative), (4, np.floor)):
+        assert_ulp(be.transform(op, x, xi, xi), fn(x.astype(np.float64)).astype(f32), 2, "transform %d vs float64" % op)
+    pos = np.abs(x) + f32(0.01)
+    assert_ulp(be.transform(5, pos, xi, xi), np.log(pos.astype(np.float64)).astype(f32), 2, "log vs float64")
+    assert_ulp(be.transform(14, pos, xi, xi), np.sqrt(pos), 0, "sqrt vs numpy")
+    y = rs.randn(4099).astype(f32)
+    for op, fn in ((0, np.add), (6, np.multiply), (9, np.subtract), (2, np.divide)):
+        assert np.array_equal(be.pairwise(op, x, xi, y, xi, xi), fn(x, y)), "pairwise %d vs numpy" % op
+    # broadcast of a row / a column
+    R, C = 37, 53
+    m = rs.randn(R * C).astype(f32)
+    mi = shape_info_np([R, C])
+    row = rs.randn(C).astype(f32)
+    col = rs.randn(R).astype(f32)
+    assert np.array_equal(be.broadcast(0, m, mi, row, shape_info_np([1, C]), mi, [1]).reshape(R, C), m.reshape(R, C) + row[None, :])
+    assert np.array_equal(be.broadcast(1, m, mi, col, shape_info_np([R, 1]), mi, [0]).reshape(R, C), m.reshape(R, C) - col[:, None])
+    # reductions against float64 ground truth
+    M = m.reshape(R, C).astype(np.float64)
+    scale1 = np.abs(M).sum(axis=1) / np.sqrt(C)
+    scale0 = np.abs(M).sum(axis=0) / np.sqrt(R)
+    assert_reduction_close(be.reduce(1, m, mi, None, [1], R), M.sum(axis=1), scale1, "sum dim1")
+    assert_reduction_close(be.reduce(1, m, mi, None, [0], C), M.sum(axis=0), scale0, "sum dim0")
+    assert_reduction_close(be.reduce(0, m, mi, None, [1], R), M.mean(axis=1), scale1 / C, "mean dim1")
+    assert np.array_equal(be.reduce(3, m, mi, None, [1], R), m.reshape(R, C).max(axis=1))
+    assert np.array_equal(be.reduce(3, m, mi, None, [0], C), m.reshape(R, C).max(axis=0))
+    assert np.array_equal(be.reduce(4, m, mi, None, [0], C), m.reshape(R, C).min(axis=0))
+    assert_reduction_close([be.reduce_scalar(1, m, mi)], [M.sum()], np.abs(M).sum() / np.sqrt(M.size), "sum all")
+    assert f32(be.reduce_scalar(3, m, mi)) == m.max()
+    ones = np.ones(R * C, f32)
+    assert float(be.reduce_scalar(1, ones, mi)) == R * C
+    # argmax with ties: first maximum wins
+    t = np.array([1, 7, 7, 3, 7, 0], f32)
+    assert float(be.indexreduce_scalar(0, t, shape_info_np([1, 6]))) == 1.0
+    tie = m.reshape(R, C).copy()
+    tie[:, 10] = 50
+    tie[:, 20] = 50
+    tie[3, :] = 60
+    assert np.array_equal(be.indexreduce(0, tie.reshape(-1), mi, None, [1], R), np.argmax(tie, axis=1).astype(f32))
+    assert np.array_equal(be.indexreduce(0, tie.reshape(-1), mi, None, [0], C), np.argmax(tie, axis=0).astype(f32))
+    assert np.array_equal(be.indexreduce(1, tie.reshape(-1), mi, None, [1], R), np.argmin(tie, axis=1).astype(f32))
+    assert float(be.indexreduce_scalar(0, tie.reshape(-1), mi)) == float(np.argmax(tie))
+    # all values below the start value -1e37: index 0 (the reference starts from -1e37, not -inf)
+    low = np.full(8, -np.inf, f32)
+    assert float(be.indexreduce_scalar(0, low, shape_info_np([1, 8]))) == 0.0
+    # variance / standard deviation: two-pass float64
+    for bias in (0, 1):
+        assert_reduction_close(be.summarystats(0, bias, m, mi, [1], R), M.var(axis=1, ddof=bias), 0, "var dim1 bias %d" % bias)
+        assert_reduction_close(be.summarystats(1, bias, m, mi, [0], C), M.std(axis=0, ddof=bias), 0, "std dim0 bias %d" % bias)
+        assert_reduction_close([be.summarystats_scalar(0, bias, m, mi)], [M.var(ddof=bias)], 0, "var all bias %d" % bias)
+    shifted = (m + f32(1000)).astype(f32)
+    assert_reduction_close(be.summarystats(0, 0, shifted, mi, [1], R), shifted.reshape(R, C).astype(np.float64).var(axis=1), 0,
+                           "var of shifted data")
+
+
+def check_rng_closed_forms(be):
+    """The buffer fill is textbook xoroshiro128+ seeded through splitmix64: recomputed here from the published
+    recurrences; and the first `size` draws of a fresh generator are the buffer itself."""
+    mask = (1 << 64) - 1
+
+    def splitmix(x):
+        x = (x + 0x9E3779B97F4A7C15) & mask
+        z = x
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
+        return z ^ (z >> 31)
+
+    def rotl(x, k):
+        return ((x << k) | (x >> (64 - k))) & mask
+
+    for seed, size in ((119, 64), (1, 33), (-7, 20)):
+        s0 = splitmix(seed & mask)
+        s1 = splitmix((seed * 119 + 3) & mask)
+        want = []
+        for _ in range(size):
+            want.append((s0 + s1) & mask)
+            s1 ^= s0
+            s0 = rotl(s0, 55) ^ s1 ^ ((s1 << 14) & mask)
+            s1 = rotl(s1, 36)
+        g = be.rng(seed, size)
+        assert [int(v) for v in g.buffer] == want, "buffer fill seed %d" % seed
+        assert [int(v) for v in g.elements(0, size)] == want, "fresh draws are the buffer"
+        # uniform [0,1): float(u64) / 2^64
+        u = g.random_z(0, size, [0, 1])
+        assert np.array_equal(u, (np.array(want, np.uint64).astype(np.float32) * np.float32(2.0 ** -64)))
+        assert g.state()[1] == 0 and g.state()[3] == 2  # offset wrapped exactly once: generation 1 -> 2
+        g.destroy()

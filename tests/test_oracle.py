@@ -1,0 +1,150 @@
+"""Pins the CPU oracle (oracle/nd4j_oracle.cpp) without a GPU: the reference's own golden values, vectors of
+the compiled reference, closed forms - and, when oracle/_ref was built, the compiled reference itself on
+seeded inputs."""
+import numpy as np
+import pytest
+
+import backends
+import checks
+from golden_inputs import (BROADCAST_OPS, INDEX_OPS, PAIRWISE_OPS, REDUCE_OPS, TRANSFORM_OPS, op_extra, shape_info_np,
+                           ulp_distance)
+
+
+@pytest.fixture(scope="module")
+def oracle(oracle_lib):
+    return backends.CpuBackend(oracle_lib)
+
+
+def test_reference_fixtures(oracle):
+    checks.check_reference_fixtures(oracle)
+
+
+def test_op_vectors_bit_exact(oracle):
+    # same compiler, flags and libm as the compiled reference: elementwise results must be identical
+    checks.check_op_vectors(oracle, max_ulp=0)
+
+
+def test_half_vectors(oracle):
+    checks.check_half_vectors(oracle, exact=True)
+
+
+def test_rng_vectors(oracle):
+    checks.check_rng_vectors(oracle, float_ulp=0)
+
+
+def test_closed_forms(oracle):
+    checks.check_closed_forms(oracle)
+
+
+def test_rng_closed_forms(oracle):
+    checks.check_rng_closed_forms(oracle)
+
+
+def test_tad_fixtures(oracle):
+    checks.check_tad_fixtures(oracle.tad)
+
+
+def test_index_is_stored_in_the_data_type(oracle):
+    # 2^24 + 1 is not representable in fp32: the reference returns (float) index
+    n = (1 << 24) + 2
+    x = np.zeros(n, np.float32)
+    x[(1 << 24) + 1] = 5.0
+    assert float(oracle.indexreduce_scalar(0, x, shape_info_np([1, n]))) == 16777216.0
+
+
+# ---- against the compiled reference on seeded inputs -------------------------------------------------
+def _views():
+    """(name, shape, order, strides or None, ews or None): dense c / f arrays and strided views."""
+    return [("c", [6, 7], "c", None, None), ("f", [6, 7], "f", None, None), ("c3", [3, 4, 5], "c", None, None),
+            ("f3", [3, 4, 5], "f", None, None), ("strided", [5, 6], "c", [12, 2], None),
+            ("permuted", [4, 5, 3], "c", [3, 12, 1], None), ("vec", [1, 9], "c", [1, 3], 3)]
+
+
+def _mk(view, rs):
+    from libnd4j_amd.harness import shape_info, span_of
+    name, shape, order, strides, ews = view
+    info = shape_info(shape, order, strides=strides, ews=ews)
+    return rs.uniform(-3, 3, span_of(info)).astype(np.float32), info
+
+
+def test_matches_compiled_reference_on_views(oracle, reference_lib):
+    ref = backends.CpuBackend(reference_lib)
+    rs = np.random.RandomState(11)
+    for vx in _views():
+        x, xi = _mk(vx, rs)
+        for vz in _views():
+            if np.prod(vz[1]) != np.prod(vx[1]) or len(vz[1]) != len(vx[1]) or vz[1] != vx[1]:
+                continue
+            _, zi = _mk(vz, rs)
+            for op in (15, 3, 0, 6):
+                assert np.array_equal(oracle.transform(op, x, xi, zi), ref.transform(op, x, xi, zi)), (vx[0], vz[0], op)
+            y, yi = _mk(vx, rs)
+            for op in (0, 6, 9):
+                assert np.array_equal(oracle.pairwise(op, x, xi, y, yi, zi), ref.pairwise(op, x, xi, y, yi, zi)), (vx[0], vz[0], op)
+        rank = len(vx[1])
+        import itertools
+        for k in range(1, rank + (0 if rank > 1 else 1)):
+            for dims in itertools.combinations(range(rank), k):
+                dims = list(dims)
+                out_len = int(np.prod(vx[1]) // np.prod([vx[1][d] for d in dims]))
+                if out_len < 1:
+                    continue
+                for op in (1, 3, 0, 8):
+                    a, b = oracle.reduce(op, x, xi, None, dims, out_len), ref.reduce(op, x, xi, None, dims, out_len)
+                    assert np.allclose(a, b, rtol=1e-6, atol=1e-6), (vx[0], dims, op)
+                assert np.array_equal(oracle.indexreduce(0, x, xi, None, dims, out_len), ref.indexreduce(0, x, xi, None, dims, out_len)), (vx[0], dims)
+                for bias in (0, 1):
+                    a = oracle.summarystats(0, bias, x, xi, dims, out_len)
+                    b = ref.summarystats(0, bias, x, xi, dims, out_len)
+                    assert np.allclose(a, b, rtol=1e-6, atol=1e-7), (vx[0], dims, bias)
+        assert np.isclose(float(oracle.reduce_scalar(1, x, xi)), float(ref.reduce_scalar(1, x, xi)), rtol=1e-6)
+        assert float(oracle.indexreduce_scalar(0, x, xi)) == float(ref.indexreduce_scalar(0, x, xi))
+        assert np.isclose(float(oracle.summarystats_scalar(1, 1, x, xi)), float(ref.summarystats_scalar(1, 1, x, xi)), rtol=1e-6)
+
+
+def test_broadcast_matches_compiled_reference(oracle, reference_lib):
+    ref = backends.CpuBackend(reference_lib)
+    rs = np.random.RandomState(12)
+    from libnd4j_amd.harness import shape_info
+    for shape, order, dims in (([5, 6], "c", [1]), ([5, 6], "c", [0]), ([5, 6], "f", [0]), ([5, 6], "f", [1]),
+                               ([3, 4, 5], "c", [0, 2]), ([3, 4, 5], "c", [1]), ([3, 4, 5], "f", [1, 2]), ([2, 3, 4, 5], "c", [1, 3])):
+        xi = shape_info(shape, order)
+        x = rs.uniform(1.5, 4, int(np.prod(shape))).astype(np.float32)
+        yshape = [shape[d] for d in dims]
+        yi = shape_info(yshape if len(yshape) > 1 else [1, yshape[0]], order if len(yshape) > 1 else "c")
+        y = rs.uniform(1.5, 4, int(np.prod(yshape))).astype(np.float32)
+        for op in BROADCAST_OPS:
+            assert np.array_equal(oracle.broadcast(op, x, xi, y, yi, xi, dims), ref.broadcast(op, x, xi, y, yi, xi, dims)), (shape, order, dims, op)
+
+
+def test_rng_matches_compiled_reference(oracle, reference_lib):
+    ref = backends.CpuBackend(reference_lib)
+    for seed, size, pre in ((119, 1 << 12, 0), (3, 777, 5000), (-11, 64, 63)):
+        a, b = oracle.rng(seed, size), ref.rng(seed, size)
+        a.rewind(pre)
+        b.rewind(pre)
+        assert np.array_equal(a.elements(0, 5000), b.elements(0, 5000))
+        a.reseed(424242)
+        b.reseed(424242)
+        assert np.array_equal(a.elements(100, 3000), b.elements(100, 3000))
+        for op, args in ((0, [0, 1]), (0, [-1, 3]), (7, [0.4]), (4, [2, 5]), (13, [0.7])):
+            assert np.array_equal(a.random_z(op, 1001, args), b.random_z(op, 1001, args)), op
+            assert a.state() == b.state()
+        x = np.linspace(-2, 2, 999).astype(np.float32)
+        for op, args in ((1, [0.5]), (2, [0.3]), (7, [0]), (12, [0.5, 1.1, 0.2, -1.7]), (13, [2.0])):
+            assert np.array_equal(a.random_xz(op, x, args), b.random_xz(op, x, args)), op
+        for op, args in ((6, [1.5, 2.0]), (10, [0.1, 0.3]), (11, [0.0, 1.0]), (8, [3, 0.5])):
+            assert np.array_equal(a.random_xyz(op, None, None, args, mode="inplace_all", n=777),
+                                  b.random_xyz(op, None, None, args, mode="inplace_all", n=777)), op
+            assert a.state() == b.state()
+        y = np.linspace(0, 1, 999).astype(np.float32)
+        assert np.array_equal(a.random_xyz(3, x, y, [0.5]), b.random_xyz(3, x, y, [0.5]))
+        assert np.array_equal(a.random_xyz(6, x, y, [0, 0.5]), b.random_xyz(6, x, y, [0, 0.5]))
+        probs = np.array([0.1, 0.2, 0.3, 0.4], np.float32)
+        vals = np.array([10, 20, 30, 40], np.float32)
+        za, zb = np.zeros(500, np.float32), np.zeros(500, np.float32)
+        a.g.random_xyz(5, vals, shape_info_np([1, 4]), probs, shape_info_np([1, 4]), za, shape_info_np([1, 500]), np.zeros(1, np.float32))
+        b.g.random_xyz(5, vals, shape_info_np([1, 4]), probs, shape_info_np([1, 4]), zb, shape_info_np([1, 500]), np.zeros(1, np.float32))
+        assert np.array_equal(za, zb)
+        a.destroy()
+        b.destroy()
