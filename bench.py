@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the legacy op-execution path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--families] [--no-cpu]
+
+A step is one pass of the headline workload: execPairwiseTransformFloat Add, execPairwiseTransformFloat
+Multiply and execBroadcastFloat Add of a row vector on fp32 [65536,1024] c-order operands that are already
+resident in HBM.  The line printed at the end is one JSON object:
+
+  value      algorithmic GB/s of the whole step loop (host clock around K steps, device idle before and after)
+  roofline   the dominant kernel (the 16-byte-vector elementwise kernel running pairwise Add): algorithmic
+             bytes per launch / average launch duration from HIP events recorded on the launch stream inside
+             the timed loop, against 8 TB/s
+  cpu_baseline  the same step on the host cores (compiled reference loops when oracle/_ref is present, else
+             this repository's CPU restatement), a bounded sample
+  families   (with --families) every op family of the other configurations, each timed with HIP events over
+             K back-to-back launches, with its CPU time next to it
+
+Inputs are synthetic (seeded numpy generators); nothing is read from disk.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--families", action="store_true", help="also time every op family of the other configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU sample of the headline step")
+    ap.add_argument("--traffic", default=None, help="JSON file with measured HBM bytes per launch of the dominant kernel")
+    return ap.parse_args()
+
+
+class EventTimer(object):
+    """HIP events on the stream the library launches on."""
+
+    def __init__(self, dev, count):
+        self.dev = dev
+        self.ev = [dev.ops.amd_timerCreate() for _ in range(count)]
+        if not all(self.ev):
+            raise RuntimeError("hipEventCreate failed")
+
+    def record(self, i):
+        if self.dev.ops.amd_timerRecord(self.ev[i], self.dev.stream) != 1:
+            raise RuntimeError("hipEventRecord failed")
+
+    def ms(self, i, j):
+        return float(self.dev.ops.amd_timerElapsedMs(self.ev[i], self.ev[j]))
+
+    def destroy(self):
+        for e in self.ev:
+            self.dev.ops.amd_timerDestroy(e)
+
+
+def time_case(dev, case, steps, warmup):
+    """Average device time of one launch of `case`, HIP events around `steps` back-to-back launches."""
+    t = EventTimer(dev, 2)
+    for _ in range(warmup):
+        case.gpu()
+    dev.sync()
+    t.record(0)
+    for _ in range(steps):
+        case.gpu()
+    t.record(1)
+    dev.sync()
+    ms = t.ms(0, 1) / steps
+    t.destroy()
+    return ms
+
+
+def load_cpu():
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import cpu_ref
+    lib = cpu_ref.load_reference()
+    if lib is None:
+        lib = cpu_ref.load_oracle()
+    return lib, ("reference" if lib.kind == "reference" else "port")
+
+
+def cpu_time(fn, lib, budget_s, min_runs=3, max_runs=200):
+    fn(lib)  # warm-up (page faults of the output buffer, OpenMP pool start)
+    times = []
+    start = time.perf_counter()
+    while len(times) < max_runs and (len(times) < min_runs or time.perf_counter() - start < budget_s):
+        t0 = time.perf_counter()
+        fn(lib)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2], len(times)
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (one process, one device, no collectives); "
+              "--gpus %d is not supported, run with --gpus 1" % args.gpus, file=sys.stderr)
+        return 2
+    from libnd4j_amd import harness, workloads
+
+    dev = harness.Device()  # raises when the HIP library or the GPU is missing: there is no CPU fallback
+    K, W = args.steps, args.warmup
+
+    # ---- headline: configs[1] ---------------------------------------------------------------------
+    w = workloads.pairwise_broadcast(dev)
+    add, mul, bca = w.case("pairwise_add"), w.case("pairwise_multiply"), w.case("broadcast_add_row")
+    step_cases = (add, mul, bca)
+    step_bytes = sum(c.bytes for c in step_cases)
+    step_elems = sum(c.elements for c in step_cases)
+    for _ in range(W):
+        for c in step_cases:
+            c.gpu()
+    dev.sync()
+    ev = EventTimer(dev, 4 * K)
+    t0 = time.perf_counter()
+    for s in range(K):
+        ev.record(4 * s)
+        add.gpu()
+        ev.record(4 * s + 1)
+        mul.gpu()
+        ev.record(4 * s + 2)
+        bca.gpu()
+        ev.record(4 * s + 3)
+    dev.sync()
+    wall = time.perf_counter() - t0
+    per_kernel_ms = [sum(ev.ms(4 * s + k, 4 * s + k + 1) for s in range(K)) / K for k in range(3)]
+    ev.destroy()
+    ms_per_step = wall * 1e3 / K
+    value = step_bytes / (wall / K) / 1e9
+
+    traffic = None
+    if args.traffic and os.path.exists(args.traffic):
+        with open(args.traffic) as f:
+            traffic = json.load(f).get("bytes_per_launch")
+    achieved = add.bytes / (per_kernel_ms[0] * 1e-3) / 1e9
+    out = {
+        "metric": "achieved HBM GB/s (algorithmic bytes) of the legacy op path: pairwise add + pairwise multiply + broadcast add row",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: " + w.name + ", seed 7", "elements_per_step": step_elems,
+                   "bytes_per_step": step_bytes},
+        "elements_per_sec": round(step_elems / (wall / K), 1),
+        "pct_of_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "kernels": {c.name: {"ms": round(ms, 4), "GB/s": round(c.bytes / ms / 1e6, 1),
+                             "frac": round(c.bytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+                    for c, ms in zip(step_cases, per_kernel_ms)},
+        "roofline": {"bound": "hbm", "kernel": "ewVecKernel (pairwise Add, fp32, 16-byte vectors)",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "bytes_per_launch": add.bytes, "avg_launch_ms": round(per_kernel_ms[0], 4)},
+    }
+
+    cpu_lib = None
+    if not args.no_cpu:
+        cpu_lib, kind = load_cpu()
+        cores = cpu_lib.lib.nd4j_cpu_get_threads()
+
+        def cpu_step(lib):
+            for c in step_cases:
+                c.cpu(lib)
+
+        med, runs = cpu_time(cpu_step, cpu_lib, args.cpu_seconds)
+        out["cpu_baseline"] = {"value": round(step_bytes / med / 1e9, 2), "unit": "GB/s", "cores": int(cores), "kind": kind,
+                               "sample": "%d full passes of the same step (all 3 calls on the full [65536,1024] operands), "
+                                         "median; %.1f ms per step, %.3g elements/s" % (runs, med * 1e3, step_elems / med),
+                               "elements_per_sec": round(step_elems / med, 1)}
+    else:
+        out["cpu_baseline"] = None
+    w.free()
+
+    # ---- every other family ---------------------------------------------------------------------------
+    if args.families:
+        fam = []
+        builders = [workloads.transform_tanh, lambda d: workloads.pairwise_broadcast(d, dtype="float16"),
+                    workloads.reductions, workloads.stats_softmax, workloads.random_fills]
+        for build in builders:
+            wl = build(dev)
+            for c in wl.cases:
+                ms = time_case(dev, c, max(3, min(K, 20)), 2)
+                row = {"config": wl.name, "case": c.name, "family": c.family, "contiguous": c.contiguous,
+                       "ms": round(ms, 4), "GB/s": round(c.bytes / ms / 1e6, 1),
+                       "frac": round(c.bytes / ms / 1e6 / HBM_PEAK_GBS, 4), "elements_per_sec": round(c.elements / ms * 1e3, 1)}
+                if cpu_lib is not None and not (c.name.endswith("float16")):
+                    med, runs = cpu_time(c.cpu, cpu_lib, 1.0, min_runs=2, max_runs=10)
+                    row["cpu_ms"] = round(med * 1e3, 3)
+                    row["cpu_GB/s"] = round(c.bytes / med / 1e9, 2)
+                fam.append(row)
+                print("%-22s %-12s %9.4f ms %8.1f GB/s %5.1f%%%s" % (
+                    c.name, c.family, ms, row["GB/s"], 100 * row["frac"],
+                    "   cpu %9.2f ms" % row["cpu_ms"] if "cpu_ms" in row else ""), file=sys.stderr, flush=True)
+            wl.free()
+        out["families"] = fam
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -139,7 +139,8 @@ void nd4j_amd_rngDump(Nd4jPointer *extraPointers, Nd4jPointer ptrRandom, Nd4jLon
                       unsigned long long *out);
 /* state[0..4] = size, offset, seed, generation, amplifier of the generator */
 void nd4j_amd_rngState(Nd4jPointer ptrRandom, Nd4jLong *state);
-/* HIP events with timing enabled, to time work on the stream the ops are launched on */
+/* HIP events with timing enabled, to time work on the stream the ops are launched on; Record and Destroy
+ * return 1 on success and 0 on failure, ElapsedMs waits for `stop` and returns -1 on failure */
 Nd4jPointer nd4j_amd_timerCreate(void);
 int nd4j_amd_timerRecord(Nd4jPointer timer, Nd4jPointer stream);
 float nd4j_amd_timerElapsedMs(Nd4jPointer start, Nd4jPointer stop);

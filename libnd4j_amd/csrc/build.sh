@@ -1,12 +1,20 @@
 #!/bin/bash
-# Builds libnd4j_amd.so (gfx950) in-tree from the sources in this directory.  Usage: build.sh [-jN]
+# Builds libnd4j_amd.so (gfx950) in-tree from the sources in this directory.  Usage: build.sh [--force] [-jN]
+# (--force recompiles every object; otherwise make rebuilds what is out of date)
 set -e
 cd "$(dirname "$0")"
-JOBS=${1:--j8}
+JOBS=-j8
+FORCE=
+for a in "$@"; do
+  case "$a" in
+    --force) FORCE=-B ;;
+    -j*) JOBS=$a ;;
+  esac
+done
 OUT=../libnd4j_amd.so
 OBJ=build
 mkdir -p $OBJ
-HIPFLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -ffp-contract=off -fvisibility=hidden -Xclang -target-feature -Xclang -packed-fp32-ops -Wno-unused-command-line-argument"
+HIPFLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -ffp-contract=off -fhip-fp32-correctly-rounded-divide-sqrt -fvisibility=hidden -Xclang -target-feature -Xclang -packed-fp32-ops -Wno-unused-command-line-argument"
 SRCS="transform.hip pairwise.hip broadcast.hip reduce.hip indexreduce.hip summarystats.hip random.hip native_ops.cpp native_reduce.cpp native_random.cpp runtime.cpp c_api.cpp"
 cat > $OBJ/Makefile <<MK
 OBJS := \$(addsuffix .o,\$(basename $SRCS))
@@ -20,4 +28,4 @@ all: ../$OUT
 	hipcc $HIPFLAGS -x hip -c \$< -o \$@ 2>&1 | grep -v "packed-fp32-ops' is not a recognized feature" || true
 	test -f \$@
 MK
-make -C $OBJ $JOBS all
+make -C $OBJ $JOBS $FORCE all

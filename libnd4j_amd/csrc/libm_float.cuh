@@ -1,10 +1,11 @@
-// Single-precision exp / log / sin / cos / expm1 / tanh that follow, step for step, the algorithms of the
+// Single-precision exp / log / pow / sin / cos / expm1 / tanh that follow, step for step, the algorithms of the
 // C library the reference calls them from: the reference's nd4j_exp<float> etc. are expf, logf, sinf, cosf,
 // tanhf of the host libm (include/templatemath.h:537-847), which is not part of the reference tree.  On the
 // image this was built for that is glibc 2.35:
 //   expf   sysdeps/ieee754/flt-32/e_expf.c    (2^(k/32) table + cubic in double, one rounding to float)
 //   logf   sysdeps/ieee754/flt-32/e_logf.c    (16-entry 1/c, log c table + cubic in double)
 //   sinf / cosf   sysdeps/ieee754/flt-32/s_sincosf.h (pi/2 reduction in double, degree 7/8 polynomials)
+//   powf   sysdeps/ieee754/flt-32/e_powf.c    (log2 table + degree-5 polynomial, y log2 x, 2^t; all in double)
 //   expm1f sysdeps/ieee754/flt-32/s_expm1f.c, tanhf sysdeps/ieee754/flt-32/s_tanhf.c (fdlibm, float ops)
 // Restating them (instead of rounding a double-precision result) reproduces the library's own rounding
 // decisions, so transforms built from these functions agree with the CPU path bit for bit in all but a
@@ -226,6 +227,102 @@ __device__ __forceinline__ float tanhf_(float x) {
         z = one - tiny;
     }
     return jx >= 0 ? z : -z;
+}
+
+// powf: sysdeps/ieee754/flt-32/e_powf.c.  log2(x) from a 16-entry 1/c, log2 c table and a degree-5 polynomial
+// in double, y * log2(x) in double, then 2^t through the 2^(k/32) table and a cubic: one rounding to float.
+__device__ static const double kPowLog2Tab[16][2] = {
+    {0x1.661ec79f8f3bep+0, -0x1.efec65b963019p-2}, {0x1.571ed4aaf883dp+0, -0x1.b0b6832d4fca4p-2},
+    {0x1.49539f0f010bp+0, -0x1.7418b0a1fb77bp-2},  {0x1.3c995b0b80385p+0, -0x1.39de91a6dcf7bp-2},
+    {0x1.30d190c8864a5p+0, -0x1.01d9bf3f2b631p-2}, {0x1.25e227b0b8eap+0, -0x1.97c1d1b3b7afp-3},
+    {0x1.1bb4a4a1a343fp+0, -0x1.2f9e393af3c9fp-3}, {0x1.12358f08ae5bap+0, -0x1.960cbbf788d5cp-4},
+    {0x1.0953f419900a7p+0, -0x1.a6f9db6475fcep-5}, {0x1p+0, 0x0p+0},
+    {0x1.e608cfd9a47acp-1, 0x1.338ca9f24f53dp-4},  {0x1.ca4b31f026aap-1, 0x1.476a9543891bap-3},
+    {0x1.b2036576afce6p-1, 0x1.e840b4ac4e4d2p-3},  {0x1.9c2d163a1aa2dp-1, 0x1.40645f0c6651cp-2},
+    {0x1.886e6037841edp-1, 0x1.88e9c2c1b9ff8p-2},  {0x1.767dcf5534862p-1, 0x1.ce0a44eb17bccp-2},
+};
+
+__device__ __forceinline__ bool zeroInfNan(unsigned i) { return 2 * i - 1 >= 2u * 0x7f800000u - 1; }
+
+// 0: y is not an integer, 1: odd integer, 2: even integer
+__device__ __forceinline__ int checkInt(unsigned iy) {
+    const int e = (iy >> 23) & 0xff;
+    if (e < 0x7f) return 0;
+    if (e > 0x7f + 23) return 2;
+    if (iy & ((1u << (0x7f + 23 - e)) - 1)) return 0;
+    if (iy & (1u << (0x7f + 23 - e))) return 1;
+    return 2;
+}
+
+__device__ __forceinline__ float powf_(float x, float y) {
+    unsigned signBias = 0;
+    unsigned ix = asU32(x);
+    const unsigned iy = asU32(y);
+    if (ix - 0x00800000u >= 0x7f800000u - 0x00800000u || zeroInfNan(iy)) {
+        if (zeroInfNan(iy)) {
+            const bool xSignalling = 2 * (ix ^ 0x00400000u) > 2u * 0x7fc00000u;
+            if (2 * iy == 0) return xSignalling ? x + y : 1.0f;
+            if (ix == 0x3f800000u) return (2 * (iy ^ 0x00400000u) > 2u * 0x7fc00000u) ? x + y : 1.0f;
+            if (2 * ix > 2u * 0x7f800000u || 2 * iy > 2u * 0x7f800000u) return x + y;
+            if (2 * ix == 2 * 0x3f800000u) return 1.0f;
+            if ((2 * ix < 2 * 0x3f800000u) == !(iy & 0x80000000u)) return 0.0f;
+            return y * y;
+        }
+        if (zeroInfNan(ix)) {
+            float x2 = x * x;
+            if ((ix & 0x80000000u) && checkInt(iy) == 1) {
+                x2 = -x2;
+                signBias = 1;
+            }
+            if (2 * ix == 0 && (iy & 0x80000000u)) return signBias ? -__builtin_inff() : __builtin_inff();
+            return (iy & 0x80000000u) ? 1 / x2 : x2;
+        }
+        if (ix & 0x80000000u) {  // finite x < 0
+            const int yint = checkInt(iy);
+            if (yint == 0) return __builtin_nanf("");
+            if (yint == 1) signBias = 1u << (5 + 11);
+            ix &= 0x7fffffffu;
+        }
+        if (ix < 0x00800000u) {  // subnormal x
+            ix = asU32(x * 0x1p23f);
+            ix &= 0x7fffffffu;
+            ix -= 23u << 23;
+        }
+    }
+    // log2(x) = log1p(z / c - 1) / ln2 + log2(c) + k
+    const unsigned tmp = ix - 0x3f330000u;
+    const int i = (tmp >> (23 - 4)) % 16;
+    const unsigned top = tmp & 0xff800000u;
+    const int k = (int)top >> 23;
+    const double z = (double)asF32(ix - top);
+    const double r = z * kPowLog2Tab[i][0] - 1;
+    const double y0 = kPowLog2Tab[i][1] + (double)k;
+    const double r2 = r * r;
+    double yy = 0x1.27616c9496e0bp-2 * r + -0x1.71969a075c67ap-2;
+    const double p = 0x1.ec70a6ca7baddp-2 * r + -0x1.7154748bef6c8p-1;
+    const double r4 = r2 * r2;
+    double q = 0x1.71547652ab82bp0 * r + y0;
+    q = p * r2 + q;
+    yy = yy * r4 + q;
+    const double ylogx = (double)y * yy;
+    if (((asU64(ylogx) >> 47) & 0xffff) >= (asU64(126.0) >> 47)) {  // |y log2 x| >= 126
+        if (ylogx > 0x1.fffffffd1d571p+6) return signBias ? -__builtin_inff() : __builtin_inff();
+        if (ylogx <= -150.0) return signBias ? -0.0f : 0.0f;
+    }
+    const double shift = 0x1.8p+52 / 32;
+    double kd = ylogx + shift;
+    const unsigned long long ki = asU64(kd);
+    kd -= shift;
+    const double rr = ylogx - kd;
+    unsigned long long t = kExp2Tab[ki % 32];
+    t += (ki + signBias) << (52 - 5);
+    const double s = asF64(t);
+    const double zz = 0x1.c6af84b912394p-5 * rr + 0x1.ebfce50fac4f3p-3;
+    const double rr2 = rr * rr;
+    double out = 0x1.62e42ff0c52d6p-1 * rr + 1;
+    out = zz * rr2 + out;
+    out = out * s;
+    return (float)out;
 }
 
 }  // namespace lm

@@ -53,13 +53,15 @@ ND4J_VIA_DOUBLE(erf_, erf)
 ND4J_VIA_DOUBLE(erfc_, erfc)
 #undef ND4J_VIA_DOUBLE
 
-__device__ __forceinline__ float pow_(float a, float b) { return (float)::pow((double)a, (double)b); }
+__device__ __forceinline__ float pow_(float a, float b) { return lm::powf_(a, b); }
 __device__ __forceinline__ double pow_(double a, double b) { return ::pow(a, b); }
 __device__ __forceinline__ float atan2_(float a, float b) { return (float)::atan2((double)a, (double)b); }
 __device__ __forceinline__ double atan2_(double a, double b) { return ::atan2(a, b); }
 
-__device__ __forceinline__ float sqrt_(float v) { return __fsqrt_rn(v); }
-__device__ __forceinline__ double sqrt_(double v) { return __dsqrt_rn(v); }
+// sqrtf under -fhip-fp32-correctly-rounded-divide-sqrt is the IEEE square root (__fsqrt_rn is not: it maps to
+// the native approximate instruction)
+__device__ __forceinline__ float sqrt_(float v) { return sqrtf(v); }
+__device__ __forceinline__ double sqrt_(double v) { return sqrt(v); }
 __device__ __forceinline__ float abs_(float v) { return ::fabsf(v); }
 __device__ __forceinline__ double abs_(double v) { return ::fabs(v); }
 __device__ __forceinline__ float floor_(float v) { return ::floorf(v); }

@@ -313,19 +313,20 @@ Nd4jLong NativeOps::getDeviceTotalMemory(Nd4jPointer ptrToDeviceId) {
     if (want >= 0 && want != prev) (void)hipSetDevice(prev);
     return (Nd4jLong)t;
 }
-static hipDeviceProp_t &propsOf(int dev) {
-    static hipDeviceProp_t props[64];
-    static bool have[64] = {false};
-    if (dev < 0 || dev >= 64) dev = 0;
-    if (!have[dev]) {
-        if (hipGetDeviceProperties(&props[dev], dev) != hipSuccess) { (void)hipGetLastError(); std::memset(&props[dev], 0, sizeof(props[dev])); }
-        have[dev] = true;
-    }
-    return props[dev];
+static int attributeOf(Nd4jPointer ptrToDeviceId, hipDeviceAttribute_t attr) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, attr, deviceIdOf(ptrToDeviceId)) != hipSuccess) { (void)hipGetLastError(); return 0; }
+    return v;
 }
-int NativeOps::getDeviceMajor(Nd4jPointer ptrToDeviceId) { return propsOf(deviceIdOf(ptrToDeviceId)).major; }
-int NativeOps::getDeviceMinor(Nd4jPointer ptrToDeviceId) { return propsOf(deviceIdOf(ptrToDeviceId)).minor; }
-const char *NativeOps::getDeviceName(Nd4jPointer ptrToDeviceId) { return propsOf(deviceIdOf(ptrToDeviceId)).name; }
+int NativeOps::getDeviceMajor(Nd4jPointer ptrToDeviceId) { return attributeOf(ptrToDeviceId, hipDeviceAttributeComputeCapabilityMajor); }
+int NativeOps::getDeviceMinor(Nd4jPointer ptrToDeviceId) { return attributeOf(ptrToDeviceId, hipDeviceAttributeComputeCapabilityMinor); }
+const char *NativeOps::getDeviceName(Nd4jPointer ptrToDeviceId) {
+    static char names[64][256];
+    int dev = deviceIdOf(ptrToDeviceId);
+    if (dev < 0 || dev >= 64) dev = 0;
+    if (names[dev][0] == 0 && hipDeviceGetName(names[dev], 255, dev) != hipSuccess) { (void)hipGetLastError(); names[dev][0] = 0; }
+    return names[dev];
+}
 
 static hipMemcpyKind kindOf(int flags) {
     switch (flags) {

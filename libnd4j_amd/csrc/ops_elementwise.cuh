@@ -152,14 +152,16 @@ ND4J_TRANSFORM(50, CubeDerivative, return (C)3 * d1 * d1;)
 ND4J_TRANSFORM(51, HardSigmoid, return m::min_((C)1, m::max_((C)0, (C)0.2f * d1 + (C)0.5f));)
 ND4J_TRANSFORM(52, HardSigmoidDerivative, return (d1 < (C)-2.5f || d1 > (C)2.5f) ? (C)0 : (C)0.2f;)
 ND4J_TRANSFORM(53, RationalTanh, {
+    // the four-term sum is added with the constant last, the order the reference's -fassociative-math build
+    // settles on; 1 - 1/(1 + a) amplifies a last-place difference of that sum
     C dis = ((C)2 / (C)3) * d1;
-    C t = m::sgn_(dis) *
-          ((C)1 - ((C)1 / ((C)1 + m::abs_(dis) + m::pow_(dis, (C)2) + (C)1.41645f * m::pow_(dis, (C)4))));
+    C a = ((m::abs_(dis) + m::pow_(dis, (C)2)) + (C)1.41645f * m::pow_(dis, (C)4)) + (C)1;
+    C t = m::sgn_(dis) * ((C)1 - ((C)1 / a));
     return (C)1.7159f * t;
 })
 ND4J_TRANSFORM(54, RationalTanhDerivative, {
     C dis = ((C)2 / (C)3) * d1;
-    C a = (C)1 + m::abs_(dis) + m::pow_(dis, (C)2) + (C)1.41645f * m::pow_(dis, (C)4);
+    C a = ((m::abs_(dis) + m::pow_(dis, (C)2)) + (C)1.41645f * m::pow_(dis, (C)4)) + (C)1;
     C tDeriv = ((C)1 + m::sgn_(dis) * ((C)2 * dis + (C)4 * (C)1.41645f * m::pow_(dis, (C)3))) / (a * a);
     return (C)1.7159f * ((C)2 / (C)3) * tDeriv;
 })
@@ -179,7 +181,9 @@ ND4J_TRANSFORM(67, SELU, {
     // SELU_ALPHA / SELU_LAMBDA (ops.h:47-48), each rounded to the compute type first as (T) casts do
     const C alpha = (C)1.6732632423543772848170429916717;
     const C lambda = (C)1.0507009873554804934193349852946;
-    return d1 > (C)0 ? lambda * d1 : lambda * (alpha * m::exp_(d1) - alpha);
+    // alpha * e - alpha is evaluated as alpha * (e - 1): the reference's release flags (-fassociative-math) let
+    // GCC factor it, and for small |d1| the two forms differ by far more than rounding (e - 1 is exact)
+    return d1 > (C)0 ? lambda * d1 : lambda * (alpha * (m::exp_(d1) - (C)1));
 })
 ND4J_TRANSFORM(68, SELUDerivative, {
     const C alpha = (C)1.6732632423543772848170429916717;

@@ -139,7 +139,8 @@ __device__ __forceinline__ typename Compute<TT>::type randomOp(const RandomCtx<T
             if (nOperands != 1) return undefinedValue;
             C from = c.args[0];
             C to = c.args[1];
-            C step = (C)i / ((C)c.length - (C)1);
+            // the reference's release flags (-freciprocal-math) hoist 1 / (length - 1) out of its loop
+            C step = (C)i * ((C)1 / ((C)c.length - (C)1));
             return from * ((C)1 - step) + step * to;
         }
         case 7:  // BernoulliDistribution

@@ -1,0 +1,342 @@
+"""Parity of the HIP path, driven through the C ABI of libnd4j_amd.so, against the CPU checkers.
+
+Sizes: the vector / fixture replays are tiny; the seeded comparisons use shapes the CPU checker finishes in
+seconds; BASELINE-size runs are in test_gpu_configs.py.  Tolerances are those of tests/checks.py.
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+import backends
+import checks
+from golden_inputs import BROADCAST_OPS, shape_info_np, ulp_distance
+from libnd4j_amd import harness
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def cpu(cpu_checker):
+    return backends.CpuBackend(cpu_checker)
+
+
+def test_native_library_is_the_one_running(gpu):
+    import os
+    from libnd4j_amd import native
+    assert os.path.exists(native.LIBRARY_PATH)
+    maps = open("/proc/self/maps").read()
+    assert "libnd4j_amd.so" in maps
+    assert gpu.ops.getAvailableDevices() >= 1
+    assert gpu.ops.getDeviceTotalMemory(None) > (1 << 30)
+    assert gpu.ops.getDeviceMajor(None) >= 9
+
+
+def test_reference_fixtures(gpu):
+    checks.check_reference_fixtures(gpu)
+
+
+def test_op_vectors(gpu):
+    checks.check_op_vectors(gpu)
+
+
+def test_half_vectors(gpu):
+    checks.check_half_vectors(gpu, exact=False)
+
+
+def test_rng_vectors(gpu):
+    checks.check_rng_vectors(gpu)
+
+
+def test_closed_forms(gpu):
+    checks.check_closed_forms(gpu)
+
+
+def test_rng_closed_forms(gpu):
+    checks.check_rng_closed_forms(gpu)
+
+
+def test_index_is_stored_in_the_data_type(gpu):
+    n = (1 << 24) + 2
+    x = np.zeros(n, np.float32)
+    x[(1 << 24) + 1] = 5.0
+    assert float(gpu.indexreduce_scalar(0, x, shape_info_np([1, n]))) == 16777216.0
+
+
+# ---- views: dense c / f, strided, permuted -------------------------------------------------------------
+VIEWS = [("c", [33, 65], "c", None, None), ("f", [33, 65], "f", None, None), ("c3", [5, 6, 7], "c", None, None),
+         ("f3", [5, 6, 7], "f", None, None), ("strided", [9, 10], "c", [20, 2], None),
+         ("permuted", [4, 5, 3], "c", [3, 12, 1], None), ("vec", [1, 19], "c", [1, 3], 3),
+         ("c4", [3, 2, 4, 5], "c", None, None)]
+
+
+def _mk(view, rs, lo=-3, hi=3):
+    name, shape, order, strides, ews = view
+    info = harness.shape_info(shape, order, strides=strides, ews=ews)
+    return rs.uniform(lo, hi, harness.span_of(info)).astype(np.float32), info
+
+
+def _touched(info):
+    return harness.element_offsets(info)
+
+
+def test_transform_and_pairwise_on_views(gpu, cpu):
+    rs = np.random.RandomState(21)
+    for vx in VIEWS:
+        x, xi = _mk(vx, rs)
+        for vz in VIEWS:
+            if vz[1] != vx[1]:
+                continue
+            _, zi = _mk(vz, rs)
+            sel = _touched(zi)
+            for op in (15, 3, 6, 10):
+                g, c = gpu.transform(op, x, xi, zi), cpu.transform(op, x, xi, zi)
+                assert ulp_distance(g[sel], c[sel]).max() <= 2, (vx[0], vz[0], op)
+                untouched = np.setdiff1d(np.arange(g.size), sel)
+                assert np.all(g[untouched] == 0), "wrote outside the view"
+            y, yi = _mk(vx, rs)
+            for op in (0, 6, 2, 13):
+                g, c = gpu.pairwise(op, x, xi, y, yi, zi), cpu.pairwise(op, x, xi, y, yi, zi)
+                assert np.array_equal(g[sel], c[sel]), (vx[0], vz[0], op)
+        # in place
+        g, c = gpu.transform_inplace(15, x, xi), cpu.transform_inplace(15, x, xi)
+        assert ulp_distance(g, c).max() <= 2, vx[0]
+
+
+def test_pairwise_branches(gpu, cpu):
+    rs = np.random.RandomState(22)
+    # scalar y
+    x, xi = _mk(VIEWS[0], rs)
+    ys = np.array([1.75], np.float32)
+    for zi in (xi, harness.shape_info([33, 65], "f")):
+        assert np.array_equal(gpu.pairwise(0, x, xi, ys, shape_info_np([1, 1]), zi), cpu.pairwise(0, x, xi, ys, shape_info_np([1, 1]), zi))
+    # different shapes, same length, all c order with EWS 1: walks length(y) elements linearly
+    a = rs.randn(60).astype(np.float32)
+    b = rs.randn(60).astype(np.float32)
+    ai, bi = shape_info_np([6, 10]), shape_info_np([10, 6])
+    assert np.array_equal(gpu.pairwise(6, a, ai, b, bi, ai), cpu.pairwise(6, a, ai, b, bi, ai))
+    # different shapes and orders: every operand by its own C-order index
+    bf = harness.shape_info([10, 6], "f")
+    assert np.array_equal(gpu.pairwise(0, a, ai, b, bf, ai), cpu.pairwise(0, a, ai, b, bf, ai))
+    # strided overloads, including negative-free odd strides and a tail that is not a multiple of the vector
+    for n, xs, ys_, zs in ((1000, 1, 1, 1), (1001, 1, 1, 1), (7, 1, 1, 1), (333, 2, 3, 1), (333, 1, 1, 4), (0, 1, 1, 1)):
+        xx = rs.randn(max(1, n * xs)).astype(np.float32)
+        yy = rs.randn(max(1, n * ys_)).astype(np.float32)
+        assert np.array_equal(gpu.pairwise_strided(0, xx, xs, yy, ys_, zs, None, n), cpu.pairwise_strided(0, xx, xs, yy, ys_, zs, None, n))
+        g, c = gpu.transform_strided(15, xx, xs, zs, None, n), cpu.transform_strided(15, xx, xs, zs, None, n)
+        assert ulp_distance(g, c).max() <= 2
+
+
+def test_misaligned_buffers(gpu, cpu):
+    # operands that start 4, 8 and 12 bytes past a 16-byte boundary, equal and unequal misalignment
+    rs = np.random.RandomState(23)
+    n = 4099
+    base = rs.randn(n + 8).astype(np.float32)
+    dev = gpu.dev
+    X = dev.upload(base)
+    Z = dev.upload(np.zeros(n + 8, np.float32))
+    for xo, zo in ((1, 1), (2, 2), (3, 3), (1, 2), (0, 3)):
+        gpu.ops.memset(Z.ptr, 0, (n + 8) * 4, 0, None)
+        gpu.ops.execTransformFloat(dev.extra(), 0, X.ptr + 4 * xo, 1, Z.ptr + 4 * zo, 1, None, n)
+        got = Z.download(np.float32)
+        assert np.array_equal(got[zo:zo + n], np.abs(base[xo:xo + n])), (xo, zo)
+        assert np.all(got[:zo] == 0) and np.all(got[zo + n:] == 0), (xo, zo)
+    X.free()
+    Z.free()
+    dev.release()
+
+
+def _dims_of(rank):
+    for k in range(1, rank):
+        for dims in itertools.combinations(range(rank), k):
+            yield list(dims)
+
+
+def test_reductions_on_views(gpu, cpu):
+    rs = np.random.RandomState(24)
+    for vx in VIEWS:
+        x, xi = _mk(vx, rs)
+        shape = vx[1]
+        rank = len(shape)
+        absx = float(np.abs(x).sum())
+        for dims in _dims_of(rank) if rank > 1 else []:
+            out_len = int(np.prod(shape) // np.prod([shape[d] for d in dims]))
+            tad_len = int(np.prod(shape)) // out_len
+            for op in (1, 0, 3, 4, 6, 8, 19):
+                if op == 19 and out_len == 1:
+                    # the reference hands a one-element result to its whole-array loop with the caller's
+                    # extraParams, and LogSumExp reads extraParams[0] there (reduce.cpp exec -> execScalar):
+                    # with extraParams == null that is a null read in the reference itself, so no oracle exists
+                    continue
+                g, c = gpu.reduce(op, x, xi, None, dims, out_len), cpu.reduce(op, x, xi, None, dims, out_len)
+                checks.assert_reduction_close(g, c, absx / out_len / np.sqrt(tad_len) if op in (1,) else 0, "%s reduce %d dims %s" % (vx[0], op, dims),
+                                              rtol=1e-5 if op != 8 else 1e-4)
+            for op in range(4):
+                assert np.array_equal(gpu.indexreduce(op, x, xi, None, dims, out_len), cpu.indexreduce(op, x, xi, None, dims, out_len)), (vx[0], op, dims)
+            for op in (0, 1):
+                for bias in (0, 1):
+                    g = gpu.summarystats(op, bias, x, xi, dims, out_len)
+                    c = cpu.summarystats(op, bias, x, xi, dims, out_len)
+                    checks.assert_reduction_close(g, c, 0, "%s stats %d/%d dims %s" % (vx[0], op, bias, dims))
+        checks.assert_reduction_close([gpu.reduce_scalar(1, x, xi)], [cpu.reduce_scalar(1, x, xi)], absx / np.sqrt(x.size), vx[0] + " sum")
+        assert float(gpu.reduce_scalar(3, x, xi)) == float(cpu.reduce_scalar(3, x, xi))
+        checks.assert_reduction_close([gpu.reduce_scalar(19, x, xi)], [cpu.reduce_scalar(19, x, xi)], 0, vx[0] + " logsumexp")
+        for op in range(4):
+            assert float(gpu.indexreduce_scalar(op, x, xi)) == float(cpu.indexreduce_scalar(op, x, xi)), (vx[0], op)
+        checks.assert_reduction_close([gpu.summarystats_scalar(1, 1, x, xi)], [cpu.summarystats_scalar(1, 1, x, xi)], 0, vx[0] + " std")
+
+
+def test_reductions_without_caller_tad_tables(gpu, cpu):
+    # extraPointers without TAD slots: the library computes and caches the tables itself
+    rs = np.random.RandomState(25)
+    x, xi = _mk(VIEWS[2], rs)
+    for dims in ([1], [0, 2]):
+        out_len = int(np.prod(VIEWS[2][1]) // np.prod([VIEWS[2][1][d] for d in dims]))
+        for _ in range(2):  # second call hits the cache
+            g = gpu.reduce(3, x, xi, None, dims, out_len, pass_tads=False)
+            assert np.array_equal(g, cpu.reduce(3, x, xi, None, dims, out_len))
+            assert np.array_equal(gpu.indexreduce(0, x, xi, None, dims, out_len, pass_tads=False), cpu.indexreduce(0, x, xi, None, dims, out_len))
+    y = rs.randn(6).astype(np.float32)
+    assert np.array_equal(gpu.broadcast(0, x, xi, y, shape_info_np([1, 6]), xi, [1], pass_tads=False),
+                          cpu.broadcast(0, x, xi, y, shape_info_np([1, 6]), xi, [1]))
+
+
+def test_tad_shapes_of_every_kernel_variant(gpu, cpu):
+    # contiguous TADs of length 5 .. 20000 (sub-wave, wave, block kernels), strided TADs with and without splits
+    rs = np.random.RandomState(26)
+    for rows, cols in ((300, 5), (64, 31), (40, 64), (33, 300), (7, 4100), (3, 20011), (2000, 3), (5, 1), (1, 17)):
+        x = rs.randn(rows * cols).astype(np.float32)
+        xi = shape_info_np([rows, cols])
+        scale1 = np.abs(x).reshape(rows, cols).sum(axis=1) / np.sqrt(cols)
+        scale0 = np.abs(x).reshape(rows, cols).sum(axis=0) / np.sqrt(rows)
+        if cols > 1 and rows > 1:
+            checks.assert_reduction_close(gpu.reduce(1, x, xi, None, [1], rows), cpu.reduce(1, x, xi, None, [1], rows), scale1, "sum rows %dx%d" % (rows, cols))
+            checks.assert_reduction_close(gpu.reduce(1, x, xi, None, [0], cols), cpu.reduce(1, x, xi, None, [0], cols), scale0, "sum cols %dx%d" % (rows, cols))
+            assert np.array_equal(gpu.reduce(3, x, xi, None, [1], rows), cpu.reduce(3, x, xi, None, [1], rows))
+            assert np.array_equal(gpu.indexreduce(0, x, xi, None, [1], rows), cpu.indexreduce(0, x, xi, None, [1], rows))
+            assert np.array_equal(gpu.indexreduce(0, x, xi, None, [0], cols), cpu.indexreduce(0, x, xi, None, [0], cols))
+            checks.assert_reduction_close(gpu.summarystats(0, 1, x, xi, [1], rows), cpu.summarystats(0, 1, x, xi, [1], rows), 0, "var rows")
+            checks.assert_reduction_close(gpu.summarystats(0, 1, x, xi, [0], cols), cpu.summarystats(0, 1, x, xi, [0], cols), 0, "var cols")
+            y = rs.randn(cols).astype(np.float32)
+            assert np.array_equal(gpu.broadcast(0, x, xi, y, shape_info_np([1, cols]), xi, [1]), cpu.broadcast(0, x, xi, y, shape_info_np([1, cols]), xi, [1]))
+            yc = rs.randn(rows).astype(np.float32)
+            assert np.array_equal(gpu.broadcast(2, x, xi, yc, shape_info_np([rows, 1]), xi, [0]), cpu.broadcast(2, x, xi, yc, shape_info_np([rows, 1]), xi, [0]))
+        assert float(gpu.indexreduce_scalar(0, x, xi)) == float(cpu.indexreduce_scalar(0, x, xi))
+
+
+def test_broadcast_on_views_all_ops(gpu, cpu):
+    rs = np.random.RandomState(27)
+    for shape, order, dims in (([17, 33], "c", [1]), ([17, 33], "c", [0]), ([17, 33], "f", [0]), ([17, 33], "f", [1]),
+                               ([3, 4, 5], "c", [0, 2]), ([3, 4, 5], "c", [1]), ([3, 4, 5], "f", [1, 2]), ([2, 3, 4, 5], "c", [1, 3])):
+        xi = harness.shape_info(shape, order)
+        x = rs.uniform(1.5, 4, int(np.prod(shape))).astype(np.float32)
+        yshape = [shape[d] for d in dims]
+        yi = harness.shape_info(yshape if len(yshape) > 1 else [1, yshape[0]], order if len(yshape) > 1 else "c")
+        y = rs.uniform(1.5, 4, int(np.prod(yshape))).astype(np.float32)
+        for op in BROADCAST_OPS:
+            g, c = gpu.broadcast(op, x, xi, y, yi, xi, dims), cpu.broadcast(op, x, xi, y, yi, xi, dims)
+            assert ulp_distance(g, c).max() <= 2, (shape, order, dims, op)
+
+
+def test_nan_and_special_values(gpu, cpu):
+    x = np.array([np.nan, 1.0, -np.inf, np.inf, 0.0, -0.0, 3.0, np.nan, 2.0, -1e38, 1e38, 5.0], np.float32)
+    xi = shape_info_np([1, x.size])
+    for op in (79, 80, 81, 0, 6, 46):
+        g, c = gpu.transform(op, x, xi, xi, np.array([7, 0, 0, 0], np.float32)), cpu.transform(op, x, xi, xi, np.array([7, 0, 0, 0], np.float32))
+        assert ulp_distance(g, c).max() == 0 and np.array_equal(np.isnan(g), np.isnan(c)), op
+    # NaN never wins an index reduction; IndexMax over the finite part
+    assert float(gpu.indexreduce_scalar(0, x, xi)) == float(cpu.indexreduce_scalar(0, x, xi)) == 3.0
+    assert float(gpu.indexreduce_scalar(1, x, xi)) == float(cpu.indexreduce_scalar(1, x, xi))
+
+
+def test_unknown_op_leaves_output_untouched(gpu, capfd):
+    x = np.ones(64, np.float32)
+    xi = shape_info_np([1, 64])
+    got = gpu.transform(500, x, xi, xi, z=np.full(64, 9.0, np.float32))
+    assert np.all(got == 9.0)
+    got = gpu.transform(38, x, xi, xi, z=np.full(64, 9.0, np.float32))  # SoftMax: whole-array op, not on this path
+    assert np.all(got == 9.0)
+    assert float(gpu.reduce_scalar(2, x, xi)) == 0.0  # opNum 2 is a gap in the reduce table
+
+
+def test_half_families(gpu, cpu):
+    rs = np.random.RandomState(28)
+    h = np.float16
+    R, C = 64, 96
+    x = rs.randn(R * C).astype(h)
+    y = rs.randn(R * C).astype(h)
+    xi = shape_info_np([R, C])
+
+    def close(g, c, what):
+        g64, c64 = g.astype(np.float64), c.astype(np.float64)
+        assert np.all(np.abs(g64 - c64) <= 1e-2 * np.maximum(np.abs(c64), 1e-2)), what
+
+    for op in (0, 6, 9):
+        close(gpu.pairwise(op, x, xi, y, xi, xi), cpu.pairwise(op, x, xi, y, xi, xi), "half pairwise %d" % op)
+    for op in (15, 3, 10):
+        close(gpu.transform(op, x, xi, xi), cpu.transform(op, x, xi, xi), "half transform %d" % op)
+    row = rs.randn(C).astype(h)
+    close(gpu.broadcast(0, x, xi, row, shape_info_np([1, C]), xi, [1]), cpu.broadcast(0, x, xi, row, shape_info_np([1, C]), xi, [1]), "half broadcast")
+    # reductions: the reference accumulates in fp16, this path in fp32; compare with the exact value instead
+    exact = x.astype(np.float64).reshape(R, C)
+    g = gpu.reduce(1, x, xi, None, [1], R).astype(np.float64)
+    assert np.all(np.abs(g - exact.sum(axis=1)) <= 1e-2 * np.maximum(np.abs(exact.sum(axis=1)), 1.0))
+    assert np.array_equal(gpu.reduce(3, x, xi, None, [0], C), exact.max(axis=0).astype(h))
+    assert np.array_equal(gpu.indexreduce(0, x, xi, None, [1], R), np.argmax(exact, axis=1).astype(h))
+    g = gpu.summarystats(0, 1, x, xi, [0], C).astype(np.float64)
+    assert np.all(np.abs(g - exact.var(axis=0, ddof=1)) <= 1e-2 * exact.var(axis=0, ddof=1))
+    # NaN is stored as 0x7fff
+    nan_in = np.array([np.nan, 1.0], h)
+    out = gpu.transform(6, nan_in, shape_info_np([1, 2]), shape_info_np([1, 2]))
+    assert out.view(np.uint16)[0] == 0x7fff
+
+
+def test_double_family_smoke(gpu, cpu):
+    rs = np.random.RandomState(29)
+    x = rs.randn(1000).astype(np.float64)
+    xi = shape_info_np([10, 100])
+    g, c = gpu.transform(15, x, xi, xi), cpu.transform(15, x, xi, xi)
+    assert np.allclose(g, c, rtol=1e-14, atol=0)
+    assert np.allclose(gpu.reduce(1, x, xi, None, [1], 10), cpu.reduce(1, x, xi, None, [1], 10), rtol=1e-13)
+    assert float(gpu.indexreduce_scalar(0, x, xi)) == float(cpu.indexreduce_scalar(0, x, xi))
+
+
+def test_random_ops_against_cpu(gpu, cpu):
+    for seed, size, pre in ((119, 1 << 12, 0), (3, 777, 5000), (-11, 64, 63)):
+        a, b = gpu.rng(seed, size), cpu.rng(seed, size)
+        a.rewind(pre)
+        b.rewind(pre)
+        assert a.state() == b.state()
+        assert np.array_equal(a.elements(0, 5000), b.elements(0, 5000))
+        a.reseed(424242)
+        b.reseed(424242)
+        assert np.array_equal(a.elements(100, 3000), b.elements(100, 3000))
+        for op, args in ((0, [0, 1]), (0, [-1, 3]), (7, [0.4]), (4, [2, 5]), (13, [0.7])):
+            assert ulp_distance(a.random_z(op, 1001, args), b.random_z(op, 1001, args)).max() <= (2 if op == 13 else 0), op
+            assert a.state() == b.state()
+        x = np.linspace(-2, 2, 999).astype(np.float32)
+        for op, args in ((1, [0.5]), (2, [0.3]), (7, [0]), (12, [0.5, 1.1, 0.2, -1.7]), (13, [2.0])):
+            assert ulp_distance(a.random_xz(op, x, args), b.random_xz(op, x, args)).max() <= (2 if op == 13 else 0), op
+        for op, args in ((6, [1.5, 2.0]), (10, [0.1, 0.3]), (11, [0.0, 1.0]), (8, [3, 0.5]), (9, [2, 0.7])):
+            g = a.random_xyz(op, None, None, args, mode="inplace_all", n=777)
+            c = b.random_xyz(op, None, None, args, mode="inplace_all", n=777)
+            assert ulp_distance(g, c).max() <= 2, op
+            assert a.state() == b.state(), op
+        y = np.linspace(0, 1, 999).astype(np.float32)
+        assert np.array_equal(a.random_xyz(3, x, y, [0.5]), b.random_xyz(3, x, y, [0.5]))
+        assert ulp_distance(a.random_xyz(6, x, y, [0, 0.5]), b.random_xyz(6, x, y, [0, 0.5])).max() <= 2
+        a.refresh(99)
+        b.refresh(99)
+        assert a.state() == b.state() and np.array_equal(a.elements(0, 300), b.elements(0, 300))
+        a.destroy()
+        b.destroy()
+
+
+def test_random_on_strided_output(gpu, cpu):
+    # a non-EWS output is filled in Fortran order of its shape (the reference's ind2sub branch)
+    zi = harness.shape_info([7, 9], "f")  # EWS -1
+    a, b = gpu.rng(5, 128), cpu.rng(5, 128)
+    assert np.array_equal(a.random_z(0, zi, [0, 1]), b.random_z(0, zi, [0, 1]))
+    assert a.state() == b.state()
+    a.destroy()
+    b.destroy()

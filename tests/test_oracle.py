@@ -21,7 +21,7 @@ def test_reference_fixtures(oracle):
 
 def test_op_vectors_bit_exact(oracle):
     # same compiler, flags and libm as the compiled reference: elementwise results must be identical
-    checks.check_op_vectors(oracle, max_ulp=0)
+    checks.check_op_vectors(oracle, max_ulp=0, exact_composites=True)
 
 
 def test_half_vectors(oracle):
