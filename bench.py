@@ -5,7 +5,8 @@
 
 A step is one pass of the headline workload: execPairwiseTransformFloat Add, execPairwiseTransformFloat
 Multiply and execBroadcastFloat Add of a row vector on fp32 [65536,1024] c-order operands that are already
-resident in HBM.  The line printed at the end is one JSON object:
+resident in HBM (in two device copies used in turn, so that no pass finds its operands in the 256 MiB
+last-level cache).  The line printed at the end is one JSON object:
 
   value      algorithmic GB/s of the whole step loop (host clock around K steps, device idle before and after)
   roofline   the dominant kernel (the 16-byte-vector elementwise kernel running pairwise Add): algorithmic
@@ -38,6 +39,9 @@ def parse():
     ap.add_argument("--families", action="store_true", help="also time every op family of the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU sample of the headline step")
+    ap.add_argument("--counters", action="store_true",
+                    help="for hardware-counter runs: launch the yardstick copy kernel (256 MiB) and each headline kernel "
+                         "3 times and exit")
     ap.add_argument("--traffic", default=None, help="JSON file with measured HBM bytes per launch of the dominant kernel")
     return ap.parse_args()
 
@@ -66,12 +70,12 @@ class EventTimer(object):
 def time_case(dev, case, steps, warmup):
     """Average device time of one launch of `case`, HIP events around `steps` back-to-back launches."""
     t = EventTimer(dev, 2)
-    for _ in range(warmup):
-        case.gpu()
+    for k in range(warmup):
+        case.gpu(k)
     dev.sync()
     t.record(0)
-    for _ in range(steps):
-        case.gpu()
+    for k in range(steps):
+        case.gpu(warmup + k)
     t.record(1)
     dev.sync()
     ms = t.ms(0, 1) / steps
@@ -117,19 +121,30 @@ def main():
     step_cases = (add, mul, bca)
     step_bytes = sum(c.bytes for c in step_cases)
     step_elems = sum(c.elements for c in step_cases)
-    for _ in range(W):
+    if args.counters:
+        src, dst = dev.empty(1 << 28), dev.empty(1 << 28)
+        for _ in range(3):
+            dev.ops.amd_copyKernel(dev.extra(), dst.ptr, src.ptr, 1 << 28)
         for c in step_cases:
-            c.gpu()
+            for _ in range(3):
+                c.gpu()
+        dev.sync()
+        print(json.dumps({"counters_run": {"copy_bytes_read": 1 << 28, "copy_bytes_written": 1 << 28,
+                                           "kernels": {c.name: c.bytes for c in step_cases}}}))
+        return 0
+    for k in range(W):
+        for c in step_cases:
+            c.gpu(k)
     dev.sync()
     ev = EventTimer(dev, 4 * K)
     t0 = time.perf_counter()
     for s in range(K):
         ev.record(4 * s)
-        add.gpu()
+        add.gpu(W + s)
         ev.record(4 * s + 1)
-        mul.gpu()
+        mul.gpu(W + s)
         ev.record(4 * s + 2)
-        bca.gpu()
+        bca.gpu(W + s)
         ev.record(4 * s + 3)
     dev.sync()
     wall = time.perf_counter() - t0

@@ -12,17 +12,15 @@ template <typename T> struct BroadcastBody {
             if (pl.kind == BroadcastPlan::ROW) {
                 constexpr int VEC = Pack<T>::N;
                 Long vecsPerTad = (pl.tadLength + VEC - 1) / VEC;
-                int gx = (int)((vecsPerTad + kBlock - 1) / kBlock);
-                Long wantY = (Long)kGridCap / gx;
-                if (wantY < 1) wantY = 1;
-                // at least 4 TADs per block so the y registers are reused
-                Long gy = pl.numTads / 4;
-                if (gy < 1) gy = 1;
-                if (gy > wantY) gy = wantY;
+                int colShift = 0;
+                while ((1 << colShift) < kBlock && (1LL << colShift) < vecsPerTad) colShift++;
+                const int colThreads = 1 << colShift, rowsPerBlock = kBlock >> colShift;
+                Long gy = (vecsPerTad + colThreads - 1) / colThreads;
                 if (gy > 65535) gy = 65535;
+                int gx = gridFor(pl.numTads, (Long)rowsPerBlock * kBcRows, kMaxGrid);
                 int aligned = (((uintptr_t)x | (uintptr_t)z) & 15) == 0 ? 1 : 0;
                 hipLaunchKernelGGL((bcRowKernel<T, F>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
-                                   pl.zOffsets, pl.tadLength, pl.numTads, aligned);
+                                   pl.zOffsets, pl.tadLength, pl.numTads, aligned, colShift);
             } else if (pl.kind == BroadcastPlan::COL) {
                 int gx = (int)((pl.numTads + kBlock - 1) / kBlock);
                 Long gy = (Long)kGridCap / gx;

@@ -95,6 +95,11 @@ struct RngState {
     Long generation;
     Long seed;
     Long amplifier;
+    // Host-computed helpers for the divisions by launch-wide constants: 1 / size in double (quotient estimate
+    // that the device corrects with the exact remainder) and floor((2^64 - 1) / d) for d = generation and
+    // d = amplifier (0 when d < 1), which turn x / d into a 64-bit high multiplication plus one correction.
+    double rSize;
+    unsigned long long mGeneration, mAmplifier;
 };
 struct RandomPlan {
     Long n;

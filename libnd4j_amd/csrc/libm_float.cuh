@@ -216,13 +216,12 @@ __device__ __forceinline__ float tanhf_(float x) {
     if (ix < 0x41b00000) {  // |x| < 22
         if (ix == 0) return x;
         if (ix < 0x24000000) return x * (one + x);
-        if (ix >= 0x3f800000) {
-            t = expm1f_(two * __builtin_fabsf(x));
-            z = one - two / (t + two);
-        } else {
-            t = expm1f_(-two * __builtin_fabsf(x));
-            z = -t / (t + two);
-        }
+        // |x| >= 1: t = expm1(2|x|), z = 1 - 2 / (t + 2); else t = expm1(-2|x|), z = -t / (t + 2).  One expm1f and
+        // one division serve both cases, so lanes of a wave that fall on either side do not run the routine twice.
+        const bool big = ix >= 0x3f800000;
+        t = expm1f_((big ? two : -two) * __builtin_fabsf(x));
+        const float q = (big ? two : -t) / (t + two);
+        z = big ? one - q : q;
     } else {
         z = one - tiny;
     }

@@ -42,7 +42,7 @@ __device__ __forceinline__ u64 next64Dev(u64 s0) {
 }
 
 // floor(n / y) for n < y * 2^32 (so the quotient fits 32 bits), through a double estimate that is then
-// corrected with the exact remainder.  ry approximates 1/y to ~2^-52.
+// corrected with the exact remainder.  ry approximates 1/y to ~2^-52, so the estimate is off by at most one.
 __device__ __forceinline__ unsigned quot32(u64 n, unsigned y, double ry) {
     double qd = (double)n * ry;
     if (qd > 4294967295.0) qd = 4294967295.0;
@@ -53,44 +53,93 @@ __device__ __forceinline__ unsigned quot32(u64 n, unsigned y, double ry) {
     return q;
 }
 
-// floor(x / y), y >= 1.
-__device__ __forceinline__ u64 divU64(u64 x, u64 y) {
-    if ((y >> 32) != 0) return x / y;
-    const unsigned ys = (unsigned)y;
-    double yd = (double)ys;
+// 1 / y in double for 1 <= y < 2^32: hardware estimate plus two Newton steps
+__device__ __forceinline__ double recip32(unsigned y) {
+    const double yd = (double)y;
     double ry = __builtin_amdgcn_rcp(yd);
     ry = ry * (2.0 - yd * ry);
     ry = ry * (2.0 - yd * ry);
+    return ry;
+}
+
+// floor(x / y) for 1 <= y < 2^32, ry ~ 1 / y: schoolbook division with two 32-bit quotient digits
+__device__ __forceinline__ u64 divU64By32(u64 x, unsigned y, double ry) {
     const unsigned hi = (unsigned)(x >> 32);
-    const unsigned qhi = quot32((u64)hi, ys, ry);
-    const unsigned r = hi - qhi * ys;
+    const unsigned qhi = quot32((u64)hi, y, ry);
+    const unsigned r = hi - qhi * y;
     const u64 n2 = ((u64)r << 32) | (x & 0xffffffffULL);
-    const unsigned qlo = quot32(n2, ys, ry);
+    const unsigned qlo = quot32(n2, y, ry);
     return ((u64)qhi << 32) | qlo;
 }
 
-// RandomBuffer::safeShift (helper_generator.h:238-242)
-__device__ __forceinline__ u64 safeShiftDev(u64 x, u64 y) {
-    if (y != 0 && x > divU64(0xffffffffffffffffULL, y)) return divU64(x, y) + 11;
+// floor((2^64 - 1) / y) for 1 <= y < 2^32: the multiplier that turns x / y into a high multiplication
+__device__ __forceinline__ u64 magicFor(u64 y) {
+    if (y == 0 || (y >> 32) != 0) return 0;
+    return divU64By32(0xffffffffffffffffULL, (unsigned)y, recip32((unsigned)y));
+}
+
+// RandomBuffer::safeShift (helper_generator.h:238-242): x > MAX / y ? x / y + 11 : x * y + 11.
+// For y < 2^32, "x > floor((2^64 - 1) / y)" is "x * y does not fit 64 bits", read off the 96-bit product, and
+// with m = floor((2^64 - 1) / y) the quotient is mulhi(x, m) or one more (x / y - x m / 2^64 lies in [0, 1)).
+__device__ __forceinline__ u64 safeShiftDev(u64 x, u64 y, u64 m) {
+    if (y == 0) return 11;
+    if ((y >> 32) == 0) {
+        const unsigned ys = (unsigned)y;
+        const u64 lo = (u64)(unsigned)x * ys;
+        const u64 hi = (x >> 32) * ys + (lo >> 32);
+        if ((hi >> 32) != 0) {
+            u64 q = __umul64hi(x, m);
+            if (x - q * (u64)ys >= (u64)ys) q++;
+            return q + 11;
+        }
+        return ((hi << 32) | (lo & 0xffffffffULL)) + 11;
+    }
+    if (x > 0xffffffffffffffffULL / y) return x / y + 11;
     return x * y + 11;
 }
 
+// Per-thread memory between the elements a thread draws: the quotient / remainder of the last position by
+// the buffer size (positions that advance by less than `size` need no division) and the multiplier of the
+// last generation divisor.
+struct RngWalk {
+    Long lastP, q, rem;
+    u64 y, m;
+    bool valid;
+    __device__ __forceinline__ RngWalk() : lastP(0), q(0), rem(0), y(0), m(0), valid(false) {}
+};
+
 // RandomBuffer::getElement (helper_generator.h:185-220)
-__device__ __forceinline__ u64 rngElement(const RngState &st, Long position) {
-    Long p = st.position + position;
-    Long tempGen = st.generation;
-    if (p >= st.size) {
-        u64 q = divU64((u64)p, (u64)st.size);
-        tempGen += (Long)q;
-        p = p - (Long)q * st.size;
+__device__ __forceinline__ u64 rngElement(const RngState &st, Long position, RngWalk &w) {
+    const Long p = st.position + position;
+    Long q, r;
+    if (w.valid && p >= w.lastP && p - w.lastP < st.size) {
+        q = w.q;
+        r = w.rem + (p - w.lastP);
+        if (r >= st.size) { r -= st.size; q++; }
+    } else if (p < st.size) {
+        q = 0;
+        r = p;
+    } else {
+        if ((u64)st.size < (1ULL << 32) && ((u64)p >> 32) < (u64)st.size) q = (Long)quot32((u64)p, (unsigned)st.size, st.rSize);
+        else q = (Long)((u64)p / (u64)st.size);
+        r = p - q * st.size;
     }
-    u64 r = st.buffer[p];
-    const bool genDiffers = tempGen != st.generation;
-    if (genDiffers) r = safeShiftDev(r, (u64)tempGen);
-    if (st.generation > 1) r = safeShiftDev(r, (u64)st.generation);
-    if (st.amplifier != st.seed) r = safeShiftDev(r, (u64)st.amplifier);
-    if (st.amplifier != st.seed || st.generation > 1 || genDiffers) r = next64Dev(seedConvDev(r));
-    return r;
+    w.lastP = p; w.q = q; w.rem = r; w.valid = true;
+    u64 x = st.buffer[r];
+    const bool genDiffers = q != 0;
+    if (genDiffers) {
+        const u64 tempGen = (u64)(st.generation + q);
+        if (tempGen != w.y) { w.y = tempGen; w.m = magicFor(tempGen); }
+        x = safeShiftDev(x, tempGen, w.m);
+    }
+    if (st.generation > 1) x = safeShiftDev(x, (u64)st.generation, st.mGeneration);
+    if (st.amplifier != st.seed) x = safeShiftDev(x, (u64)st.amplifier, st.mAmplifier);
+    if (st.amplifier != st.seed || st.generation > 1 || genDiffers) x = next64Dev(seedConvDev(x));
+    return x;
+}
+__device__ __forceinline__ u64 rngElement(const RngState &st, Long position) {
+    RngWalk w;
+    return rngElement(st, position, w);
 }
 
 // relativeT<T>(index): u64 -> [0, 1] (helper_generator.h:481-486).  (T)MAX_UINT is exactly 2^64.
@@ -103,12 +152,17 @@ template <typename TT> struct RandomCtx {
     RngState st;
     Params<TT> args;
     Long length;
-    __device__ __forceinline__ C unit(Long i) const {
-        C u = toUnit<C>(rngElement(st, i));
+    __device__ __forceinline__ C unit(Long i, RngWalk &w) const {
+        C u = toUnit<C>(rngElement(st, i, w));
         // storage types narrower than float round the draw to the storage type first (481-484)
         if (sizeof(TT) < 4) u = toCompute(fromCompute<TT>(u));
         return u;
     }
+    __device__ __forceinline__ C unit(Long i) const {
+        RngWalk w;
+        return unit(i, w);
+    }
+    __device__ __forceinline__ C unit(Long i, C from, C to, RngWalk &w) const { return from + (unit(i, w) * (to - from)); }
     __device__ __forceinline__ C unit(Long i, C from, C to) const { return from + (unit(i) * (to - from)); }
 };
 
@@ -117,24 +171,24 @@ template <typename TT> struct RandomCtx {
 template <int OP, typename TT>
 __device__ __forceinline__ typename Compute<TT>::type randomOp(const RandomCtx<TT> &c, int nOperands,
                                                                typename Compute<TT>::type x,
-                                                               typename Compute<TT>::type y, Long i) {
+                                                               typename Compute<TT>::type y, Long i, RngWalk &w) {
     typedef typename Compute<TT>::type C;
     const C undefinedValue = nOperands == 1 ? (C)-1 : (nOperands == 2 ? (C)-2 : (C)-3);
     switch (OP) {
         case 0:  // UniformDistribution
             if (nOperands != 1) return undefinedValue;
-            return c.unit(i, c.args[0], c.args[1]);
+            return c.unit(i, c.args[0], c.args[1], w);
         case 1:  // DropOut
             if (nOperands != 2) return undefinedValue;
-            return c.unit(i) >= c.args[0] ? (C)0 : x;
+            return c.unit(i, w) >= c.args[0] ? (C)0 : x;
         case 2: {  // DropOutInverted
             if (nOperands != 2) return undefinedValue;
             C prob = c.args[0];
-            return c.unit(i) >= prob ? (C)0 : x / prob;
+            return c.unit(i, w) >= prob ? (C)0 : x / prob;
         }
         case 3:  // ProbablisticMerge
             if (nOperands != 3) return undefinedValue;
-            return c.unit(i) <= c.args[0] ? y : x;
+            return c.unit(i, w) <= c.args[0] ? y : x;
         case 4: {  // Linspace
             if (nOperands != 1) return undefinedValue;
             C from = c.args[0];
@@ -144,12 +198,12 @@ __device__ __forceinline__ typename Compute<TT>::type randomOp(const RandomCtx<T
             return from * ((C)1 - step) + step * to;
         }
         case 7:  // BernoulliDistribution
-            if (nOperands == 1) return c.args[0] >= c.unit(i) ? (C)1 : (C)0;
-            if (nOperands == 2) return x >= c.unit(i) ? (C)1 : (C)0;
+            if (nOperands == 1) return c.args[0] >= c.unit(i, w) ? (C)1 : (C)0;
+            if (nOperands == 2) return x >= c.unit(i, w) ? (C)1 : (C)0;
             return undefinedValue;
         case 12: {  // AlphaDropOut: args = p, a, b, alphaPrime
             if (nOperands != 2) return undefinedValue;
-            C u = c.unit(i);
+            C u = c.unit(i, w);
             return u >= c.args[0] ? c.args[1] * c.args[3] + c.args[2] : c.args[1] * x + c.args[2];
         }
         case 13: {  // ExponentialDistribution
@@ -157,7 +211,7 @@ __device__ __forceinline__ typename Compute<TT>::type randomOp(const RandomCtx<T
             if (nOperands == 1) {
                 // DataTypeUtils::min<T>(): smallest positive normal of the data type
                 C lo = sizeof(TT) == 8 ? (C)2.2250738585072014e-308 : (sizeof(TT) == 4 ? (C)1.175494e-38f : (C)6.1035e-05f);
-                C v = c.unit(i, lo, (C)1);
+                C v = c.unit(i, lo, (C)1, w);
                 return (C)1 - m::pow_((C)2.718281828459045, -(lambda * v));
             }
             if (nOperands == 2) return x <= (C)0 ? (C)0 : (C)1 - m::pow_((C)2.718281828459045, -(lambda * x));
@@ -169,24 +223,33 @@ __device__ __forceinline__ typename Compute<TT>::type randomOp(const RandomCtx<T
     }
 }
 
+// Elements per thread of the two hot kernels: a block takes kRngIter * kBlock consecutive elements, so the
+// positions one thread visits advance by kBlock and its RngWalk state stays valid across them.
+static constexpr int kRngIter = 8;
+
 template <typename TT, int OP>
 __global__ void __launch_bounds__(kBlock) randomPlainKernel(RandomCtx<TT> c, const TT *x, const TT *y, TT *z, int nOperands,
                                                             int strided, Long xEws, Long yEws, Long zEws, DimMap xm,
                                                             DimMap ym, DimMap zm) {
     typedef typename Compute<TT>::type C;
-    const Long stride = (Long)gridDim.x * kBlock;
-    for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < c.length; i += stride) {
-        Long ox, oy, oz;
-        if (strided) {
-            ox = i * xEws; oy = i * yEws; oz = i * zEws;
-        } else {
-            ox = nOperands >= 2 ? mapOffset32(xm, (unsigned)i) : 0;
-            oy = nOperands >= 3 ? mapOffset32(ym, (unsigned)i) : 0;
-            oz = mapOffset32(zm, (unsigned)i);
+    const Long chunk = (Long)kBlock * kRngIter;
+    RngWalk w;
+    for (Long base = (Long)blockIdx.x * chunk; base < c.length; base += (Long)gridDim.x * chunk) {
+        for (int k = 0; k < kRngIter; k++) {
+            const Long i = base + (Long)k * kBlock + threadIdx.x;
+            if (i >= c.length) break;
+            Long ox, oy, oz;
+            if (strided) {
+                ox = i * xEws; oy = i * yEws; oz = i * zEws;
+            } else {
+                ox = nOperands >= 2 ? mapOffset32(xm, (unsigned)i) : 0;
+                oy = nOperands >= 3 ? mapOffset32(ym, (unsigned)i) : 0;
+                oz = mapOffset32(zm, (unsigned)i);
+            }
+            C xv = nOperands >= 2 ? toCompute(x[ox]) : (C)0;
+            C yv = nOperands >= 3 ? toCompute(y[oy]) : (C)0;
+            z[oz] = fromCompute<TT>(randomOp<OP, TT>(c, nOperands, xv, yv, i, w));
         }
-        C xv = nOperands >= 2 ? toCompute(x[ox]) : (C)0;
-        C yv = nOperands >= 3 ? toCompute(y[oy]) : (C)0;
-        z[oz] = fromCompute<TT>(randomOp<OP, TT>(c, nOperands, xv, yv, i));
     }
 }
 
@@ -200,11 +263,15 @@ __global__ void __launch_bounds__(kBlock) gaussianKernel(RandomCtx<TT> c, const 
     const C mean = c.args[0];
     const C stddev = c.args[1];
     const Long pairs = (c.length + 1) / 2;
-    const Long stride = (Long)gridDim.x * kBlock;
-    for (Long k = (Long)blockIdx.x * kBlock + threadIdx.x; k < pairs; k += stride) {
+    const Long chunk = (Long)kBlock * kRngIter;
+    RngWalk w;
+    for (Long base = (Long)blockIdx.x * chunk; base < pairs; base += (Long)gridDim.x * chunk)
+    for (int it = 0; it < kRngIter; it++) {
+        const Long k = base + (Long)it * kBlock + threadIdx.x;
+        if (k >= pairs) break;
         const Long e = 2 * k;
-        C u0 = c.unit(e, (C)1e-5f, (C)1);
-        C u1 = c.unit(e + 1, (C)1e-5f, (C)1);
+        C u0 = c.unit(e, (C)1e-5f, (C)1, w);
+        C u1 = c.unit(e + 1, (C)1e-5f, (C)1, w);
         C r = m::sqrt_((C)-2 * m::log_(u0));
         C ang = twoPi * u1;
         C z0 = r * m::cos_(ang);
@@ -312,7 +379,7 @@ template <typename T> struct RandomPlainBody {
     template <int OP> struct Run {
         static bool run(hipStream_t s, const RandomCtx<T> &c, const T *x, const T *y, T *z, const RandomPlan &pl,
                         int operands) {
-            int grid = gridFor(pl.n, kBlock * 4, kGridCap);
+            int grid = gridFor(pl.n, kBlock * kRngIter, kMaxGrid);
             hipLaunchKernelGGL((randomPlainKernel<T, OP>), dim3(grid), dim3(kBlock), 0, s, c, x, y, z, operands,
                                pl.strided ? 1 : 0, pl.xEws, pl.yEws, pl.zEws, pl.xm, pl.ym, pl.zm);
             return true;
@@ -340,12 +407,12 @@ bool launchRandom(hipStream_t s, int opNum, const RngState &rng, const T *x, con
                 break;
             }
             case 6: {
-                int grid = gridFor((pl.n + 1) / 2, kBlock * 2, kGridCap);
+                int grid = gridFor((pl.n + 1) / 2, kBlock * kRngIter, kMaxGrid);
                 hipLaunchKernelGGL((gaussianKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
                 break;
             }
             case 10: {
-                int grid = gridFor((pl.n + 1) / 2, kBlock * 2, kGridCap);
+                int grid = gridFor((pl.n + 1) / 2, kBlock * kRngIter, kMaxGrid);
                 hipLaunchKernelGGL((gaussianKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
                 break;
             }

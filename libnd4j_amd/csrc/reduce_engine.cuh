@@ -82,7 +82,7 @@ __device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc
     const Pack<T> *pv = reinterpret_cast<const Pack<T> *>(p + head);
 #pragma unroll 4
     for (Long v = lane; v < nvec; v += lanes) {
-        Pack<T> pk = pv[v];
+        Pack<T> pk = loadPack(pv + v);
 #pragma unroll
         for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk.v[e]), head + v * VEC + e);
     }
@@ -143,15 +143,31 @@ __global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename P
     else partials[(Long)blockIdx.y * numTads + t] = acc;
 }
 
+// Merges the `splits` partial accumulators of each TAD: 64 TADs per block, the four waves of the block take
+// every fourth split (independent loads, several in flight), then merge through LDS.
 template <class Pol>
-__global__ void __launch_bounds__(kBlock) tadColFinish(Pol pol, typename Pol::T *z, const typename Pol::Acc *partials,
-                                                       Long tadLength, Long numTads, int splits) {
-    const Long t = (Long)blockIdx.x * kBlock + threadIdx.x;
-    if (t >= numTads) return;
-    pol.setTad(t, z);
-    typename Pol::Acc acc = partials[t];
-    for (int s = 1; s < splits; s++) acc = pol.combine(acc, partials[(Long)s * numTads + t]);
-    z[t] = pol.finalize(acc, tadLength);
+__global__ void __launch_bounds__(kBlock) tadColFinish(Pol pol, typename Pol::T *z,
+                                                       const typename Pol::Acc *__restrict__ partials, Long tadLength,
+                                                       Long numTads, int splits) {
+    typedef typename Pol::Acc Acc;
+    constexpr int GROUPS = kBlock / kWave;
+    __shared__ Acc smem[kBlock];
+    const int lane = threadIdx.x % kWave, grp = threadIdx.x / kWave;
+    const Long t = (Long)blockIdx.x * kWave + lane;
+    const bool live = t < numTads && grp < splits;
+    Acc acc;
+    if (live) {
+        acc = partials[(Long)grp * numTads + t];
+#pragma unroll 4
+        for (int s = grp + GROUPS; s < splits; s += GROUPS) acc = pol.combine(acc, partials[(Long)s * numTads + t]);
+        smem[threadIdx.x] = acc;
+    }
+    __syncthreads();
+    if (live && grp == 0) {
+        pol.setTad(t, z);
+        for (int g = 1; g < GROUPS && g < splits; g++) acc = pol.combine(acc, smem[g * kWave + lane]);
+        z[t] = pol.finalize(acc, tadLength);
+    }
 }
 
 template <class Pol>
@@ -192,7 +208,7 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
                 Long v = b + u * kBlock + threadIdx.x;
-                if (v < nvec) pk[u] = xv[v];
+                if (v < nvec) pk[u] = loadPack(xv + v);
             }
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
@@ -269,8 +285,8 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         hipLaunchKernelGGL((tadColKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
                            pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit);
         if (splits > 1)
-            hipLaunchKernelGGL((tadColFinish<Pol>), dim3(gx), dim3(kBlock), 0, s, pol, z, partials, pl.tadLength,
-                               pl.numTads, (int)splits);
+            hipLaunchKernelGGL((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kWave - 1) / kWave)), dim3(kBlock), 0, s, pol,
+                               z, partials, pl.tadLength, pl.numTads, (int)splits);
         return;
     }
     int grid = gridFor(pl.numTads, 1, kGridCap);

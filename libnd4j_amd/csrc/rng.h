@@ -64,6 +64,9 @@ struct RandomBuffer {
         st.generation = generation;
         st.seed = seed;
         st.amplifier = amplifier;
+        st.rSize = size > 0 ? 1.0 / (double)size : 0.0;
+        st.mGeneration = generation > 0 ? ~0ULL / (unsigned long long)generation : 0ULL;
+        st.mAmplifier = amplifier > 0 ? ~0ULL / (unsigned long long)amplifier : 0ULL;
         return st;
     }
 };

@@ -24,16 +24,38 @@ S_VAR, S_STD = 0, 1
 RND_UNIFORM, RND_DROPOUT, RND_GAUSSIAN = 0, 1, 6
 
 
+ROTATE_BYTES = 3 << 29  # device copies of the operands are made until they span 1.5 GiB
+
+
 class Case(object):
+    """One call of the library.  The operands exist in several device copies ("sets") and ``gpu(k)`` runs the
+    call on set ``k % sets``: a timing loop that passes its iteration counter never finds its operands in the
+    256 MiB last-level cache left there by the previous iteration, so what it measures is HBM traffic."""
+
     def __init__(self, name, family, elements, nbytes, gpu, cpu, contiguous, result=None):
         self.name = name
         self.family = family
         self.elements = int(elements)
         self.bytes = int(nbytes)
-        self.gpu = gpu
+        self._gpu = [gpu]
+        self._result = [result]
         self.cpu = cpu
         self.contiguous = contiguous
-        self.result = result  # () -> numpy array of what the last gpu() call wrote
+
+    @property
+    def sets(self):
+        return len(self._gpu)
+
+    def gpu(self, k=0):
+        self._gpu[k % len(self._gpu)]()
+
+    def result(self, k=0):
+        """numpy array of what the last gpu(k) call wrote"""
+        return self._result[k % len(self._result)]()
+
+    def add_set(self, other):
+        self._gpu += other._gpu
+        self._result += other._result
 
 
 class Workload(object):
@@ -74,6 +96,20 @@ def _vec(n):
     return harness.shape_info([1, int(n)])
 
 
+def _replicated(dev, name, set_bytes, host, device_set, copies=None):
+    """Builds a Workload from ``device_set(w) -> [Case]``, called once per device copy of the operands."""
+    w = Workload(dev, name)
+    w.host.update(host)
+    if copies is None:
+        copies = max(2, -(-ROTATE_BYTES // int(set_bytes)))
+    w.cases = device_set(w)
+    for _ in range(copies - 1):
+        for c, extra in zip(w.cases, device_set(w)):
+            c.add_set(extra)
+    w.copies = copies
+    return w
+
+
 def _normal(rs, n, dtype):
     return rs.standard_normal(n, dtype=F32).astype(dtype, copy=False)
 
@@ -87,189 +123,191 @@ def _suffix(dtype):
 
 
 # ---- configs[0]: tanh over 2^24 ------------------------------------------------------------------------
-def transform_tanh(dev, n=1 << 24, seed=42):
-    w = Workload(dev, "transform tanh fp32 1-D 2^%d" % int(np.log2(n)))
+def transform_tanh(dev, n=1 << 24, seed=42, copies=None):
     x = _uniform(np.random.default_rng(seed), n, -4, 4)
     xi = _vec(n)
-    X, Z = w.operand(x, xi), w.operand(np.zeros(n, F32), xi)
-    ex = dev.extra(xi, z_info=xi)
-    ops = dev.ops
-    w.host.update(x=x, xi=xi)
-
-    def gpu():
-        ops.execTransformFloat(ex, T_TANH, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, None)
-
     zc = np.zeros(n, F32)
-    w.host["z_cpu"] = zc
-    w.cases.append(Case("transform_tanh", "transform", n, 8 * n, gpu,
-                        lambda lib: lib.transform(T_TANH, x, xi, zc, xi, None), True, Z.get))
-    return w
+    ops = dev.ops
+
+    def device_set(w):
+        X, Z = w.operand(x, xi), w.operand(np.zeros(n, F32), xi)
+        ex = dev.extra(xi, z_info=xi)
+        return [Case("transform_tanh", "transform", n, 8 * n,
+                     lambda: ops.execTransformFloat(ex, T_TANH, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, None),
+                     lambda lib: lib.transform(T_TANH, x, xi, zc, xi, None), True, Z.get)]
+
+    return _replicated(dev, "transform tanh fp32 1-D 2^%d" % int(np.log2(n)), 8 * n, dict(x=x, xi=xi, z_cpu=zc),
+                       device_set, copies)
 
 
 # ---- configs[1]: pairwise add / multiply and broadcast add of a row ----------------------------------
-def pairwise_broadcast(dev, rows=65536, cols=1024, seed=7, dtype=F32):
+def pairwise_broadcast(dev, rows=65536, cols=1024, seed=7, dtype=F32, copies=None):
     dtype = np.dtype(dtype)
-    w = Workload(dev, "pairwise add+multiply, broadcast add row; %s [%d,%d] c-order" % (dtype.name, rows, cols))
     rs = np.random.default_rng(seed)
     n = rows * cols
     x, y = _normal(rs, n, dtype), _normal(rs, n, dtype)
     bias = _uniform(rs, cols, -1, 1, dtype)
     xi, bi = harness.shape_info([rows, cols]), _vec(cols)
-    X, Y, Z, B = w.operand(x, xi), w.operand(y, xi), w.operand(np.zeros(n, dtype), xi), w.operand(bias, bi)
     ops, suf, sz = dev.ops, _suffix(dtype), dtype.itemsize
     pw, bc = getattr(ops, "execPairwiseTransform" + suf), getattr(ops, "execBroadcast" + suf)
-    ex_p = dev.extra(xi, xi, xi)
     tad = dev.tad(xi, [1])
-    ex_b = dev.extra(xi, bi, xi, tad=tad, tad_z=tad)
-    D = w.raw(np.array([1], np.int32))
-    w.host.update(x=x, y=y, bias=bias, xi=xi, bi=bi)
     zc = np.zeros(n, dtype)
-    w.host["z_cpu"] = zc
-
-    def mk_pw(op):
-        return lambda: pw(ex_p, op, X.ptr, X.info_ptr, Y.ptr, Y.info_ptr, Z.ptr, Z.info_ptr, None)
-
-    def gpu_bc():
-        bc(ex_b, B_ADD, X.ptr, X.info_ptr, B.ptr, B.info_ptr, Z.ptr, Z.info_ptr, D.ptr, 1)
-
     tag = "" if dtype == F32 else "_" + dtype.name
-    w.cases.append(Case("pairwise_add" + tag, "pairwise", n, 3 * sz * n, mk_pw(P_ADD),
-                        lambda lib: lib.pairwise(P_ADD, x, xi, y, xi, zc, xi, None), True, Z.get))
-    w.cases.append(Case("pairwise_multiply" + tag, "pairwise", n, 3 * sz * n, mk_pw(P_MUL),
-                        lambda lib: lib.pairwise(P_MUL, x, xi, y, xi, zc, xi, None), True, Z.get))
-    w.cases.append(Case("broadcast_add_row" + tag, "broadcast", n, 2 * sz * n + sz * cols, gpu_bc,
-                        lambda lib: lib.broadcast(B_ADD, x, xi, bias, bi, zc, xi, [1]), True, Z.get))
-    return w
+
+    def device_set(w):
+        X, Y, Z, B = w.operand(x, xi), w.operand(y, xi), w.operand(np.zeros(n, dtype), xi), w.operand(bias, bi)
+        ex_p = dev.extra(xi, xi, xi)
+        ex_b = dev.extra(xi, bi, xi, tad=tad, tad_z=tad)
+        D = w.raw(np.array([1], np.int32))
+
+        def mk_pw(op):
+            return lambda: pw(ex_p, op, X.ptr, X.info_ptr, Y.ptr, Y.info_ptr, Z.ptr, Z.info_ptr, None)
+
+        def gpu_bc():
+            bc(ex_b, B_ADD, X.ptr, X.info_ptr, B.ptr, B.info_ptr, Z.ptr, Z.info_ptr, D.ptr, 1)
+
+        return [Case("pairwise_add" + tag, "pairwise", n, 3 * sz * n, mk_pw(P_ADD),
+                     lambda lib: lib.pairwise(P_ADD, x, xi, y, xi, zc, xi, None), True, Z.get),
+                Case("pairwise_multiply" + tag, "pairwise", n, 3 * sz * n, mk_pw(P_MUL),
+                     lambda lib: lib.pairwise(P_MUL, x, xi, y, xi, zc, xi, None), True, Z.get),
+                Case("broadcast_add_row" + tag, "broadcast", n, 2 * sz * n + sz * cols, gpu_bc,
+                     lambda lib: lib.broadcast(B_ADD, x, xi, bias, bi, zc, xi, [1]), True, Z.get)]
+
+    return _replicated(dev, "pairwise add+multiply, broadcast add row; %s [%d,%d] c-order" % (dtype.name, rows, cols),
+                       3 * sz * n, dict(x=x, y=y, bias=bias, xi=xi, bi=bi, z_cpu=zc), device_set, copies)
 
 
 # ---- configs[2]: reduce sum / max / mean and argmax along rows, columns and over everything ----------
-def reductions(dev, rows=16384, cols=4096, seed=11):
-    w = Workload(dev, "reduce sum/max/mean + argmax; fp32 [%d,%d] c-order; dim 1, dim 0, full" % (rows, cols))
+def reductions(dev, rows=16384, cols=4096, seed=11, copies=None):
     n = rows * cols
     x = _normal(np.random.default_rng(seed), n, F32)
     xi = harness.shape_info([rows, cols])
-    X = w.operand(x, xi)
     ops = dev.ops
-    w.host.update(x=x, xi=xi)
-    scalar_out = {}
-    for dim, out_len in ((1, rows), (0, cols)):
-        zi = _vec(out_len)
-        Z = w.operand(np.zeros(out_len, F32), zi)
-        D = w.raw(np.array([dim], np.int32))
-        ex = dev.extra(xi, z_info=zi, tad=dev.tad(xi, [dim]))
-        zc = np.zeros(out_len, F32)
-        for fam, member, cpu_name, op, opname in (("reduce", ops.execReduceFloat, "reduce", R_SUM, "sum"),
-                                                  ("reduce", ops.execReduceFloat, "reduce", R_MAX, "max"),
-                                                  ("reduce", ops.execReduceFloat, "reduce", R_MEAN, "mean"),
-                                                  ("indexreduce", ops.execIndexReduceFloat, "indexreduce", I_MAX, "argmax")):
-            def gpu(member=member, op=op, Z=Z, D=D, ex=ex):
-                member(ex, op, X.ptr, X.info_ptr, None, Z.ptr, Z.info_ptr, D.ptr, 1)
+    tads = {1: dev.tad(xi, [1]), 0: dev.tad(xi, [0])}
+    host_out = {(dim, out_len): np.zeros(out_len, F32) for dim, out_len in ((1, rows), (0, cols))}
 
-            def cpu(lib, cpu_name=cpu_name, op=op, zc=zc, zi=zi, dim=dim):
-                getattr(lib, cpu_name)(op, x, xi, None, zc, zi, [dim])
+    def device_set(w):
+        cases = []
+        X = w.operand(x, xi)
+        scalar_out = {}
+        for dim, out_len in ((1, rows), (0, cols)):
+            zi = _vec(out_len)
+            Z = w.operand(np.zeros(out_len, F32), zi)
+            D = w.raw(np.array([dim], np.int32))
+            ex = dev.extra(xi, z_info=zi, tad=tads[dim])
+            zc = host_out[(dim, out_len)]
+            for fam, member, cpu_name, op, opname in (("reduce", ops.execReduceFloat, "reduce", R_SUM, "sum"),
+                                                      ("reduce", ops.execReduceFloat, "reduce", R_MAX, "max"),
+                                                      ("reduce", ops.execReduceFloat, "reduce", R_MEAN, "mean"),
+                                                      ("indexreduce", ops.execIndexReduceFloat, "indexreduce", I_MAX, "argmax")):
+                def gpu(member=member, op=op, Z=Z, D=D, ex=ex):
+                    member(ex, op, X.ptr, X.info_ptr, None, Z.ptr, Z.info_ptr, D.ptr, 1)
 
-            w.cases.append(Case("%s_dim%d" % (opname, dim), fam, n, 4 * n + 4 * out_len, gpu, cpu, dim == 1, Z.get))
-    ex_s = dev.extra(xi)
-    for fam, member, cpu_name, op, opname in (("reduce", ops.execReduceScalarFloat, "reduce_scalar", R_SUM, "sum"),
-                                              ("reduce", ops.execReduceScalarFloat, "reduce_scalar", R_MAX, "max"),
-                                              ("reduce", ops.execReduceScalarFloat, "reduce_scalar", R_MEAN, "mean"),
-                                              ("indexreduce", ops.execIndexReduceScalarFloat, "indexreduce_scalar", I_MAX, "argmax")):
-        def gpu(member=member, op=op, opname=opname):
-            scalar_out[opname] = member(ex_s, op, X.ptr, X.info_ptr, None)
+                def cpu(lib, cpu_name=cpu_name, op=op, zc=zc, zi=zi, dim=dim):
+                    getattr(lib, cpu_name)(op, x, xi, None, zc, zi, [dim])
 
-        def cpu(lib, cpu_name=cpu_name, op=op):
-            return getattr(lib, cpu_name)(op, x, xi, None)
+                cases.append(Case("%s_dim%d" % (opname, dim), fam, n, 4 * n + 4 * out_len, gpu, cpu, dim == 1, Z.get))
+        ex_s = dev.extra(xi)
+        for fam, member, cpu_name, op, opname in (("reduce", ops.execReduceScalarFloat, "reduce_scalar", R_SUM, "sum"),
+                                                  ("reduce", ops.execReduceScalarFloat, "reduce_scalar", R_MAX, "max"),
+                                                  ("reduce", ops.execReduceScalarFloat, "reduce_scalar", R_MEAN, "mean"),
+                                                  ("indexreduce", ops.execIndexReduceScalarFloat, "indexreduce_scalar", I_MAX, "argmax")):
+            def gpu(member=member, op=op, opname=opname):
+                scalar_out[opname] = member(ex_s, op, X.ptr, X.info_ptr, None)
 
-        w.cases.append(Case("%s_full" % opname, fam, n, 4 * n + 4, gpu, cpu, True,
-                            lambda opname=opname: np.array([scalar_out[opname]], F32)))
-    return w
+            def cpu(lib, cpu_name=cpu_name, op=op):
+                return getattr(lib, cpu_name)(op, x, xi, None)
+
+            cases.append(Case("%s_full" % opname, fam, n, 4 * n + 4, gpu, cpu, True,
+                              lambda opname=opname: np.array([scalar_out[opname]], F32)))
+        return cases
+
+    return _replicated(dev, "reduce sum/max/mean + argmax; fp32 [%d,%d] c-order; dim 1, dim 0, full" % (rows, cols),
+                       4 * n, dict(x=x, xi=xi), device_set, copies)
 
 
 # ---- configs[3]: summary statistics and a softmax-style chain on an f-order matrix ---------------------
-def stats_softmax(dev, rows=32768, cols=2048, seed=23):
-    w = Workload(dev, "summary stats var/std + softmax-style chain; fp32 [%d,%d] f-order" % (rows, cols))
+def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
     n = rows * cols
     x = _uniform(np.random.default_rng(seed), n, -10, 10)  # memory order of the f-order matrix
     xi = harness.shape_info([rows, cols], "f")
-    X = w.operand(x, xi)
     ops = dev.ops
-    w.host.update(x=x, xi=xi)
-    for dim, out_len in ((1, rows), (0, cols)):
-        zi = _vec(out_len)
-        Z = w.operand(np.zeros(out_len, F32), zi)
-        D = w.raw(np.array([dim], np.int32))
-        ex = dev.extra(xi, z_info=zi, tad=dev.tad(xi, [dim]))
-        zc = np.zeros(out_len, F32)
-        for op, opname in ((S_VAR, "variance"), (S_STD, "std")):
-            def gpu(op=op, Z=Z, D=D, ex=ex):
-                ops.execSummaryStatsFloat(ex, op, X.ptr, X.info_ptr, None, Z.ptr, Z.info_ptr, D.ptr, 1, 1)
-
-            def cpu(lib, op=op, zc=zc, zi=zi, dim=dim):
-                lib.summarystats(op, 1, x, xi, zc, zi, [dim])
-
-            # dim 0 TADs are the contiguous columns of the f-order matrix, dim 1 TADs have stride `rows`
-            w.cases.append(Case("%s_dim%d" % (opname, dim), "summarystats", n, 4 * n + 4 * out_len, gpu, cpu, dim == 0, Z.get))
-
-    # softmax along dimension 1 as five calls: m = max(x, 1); t = x - m; t = exp(t); s = sum(t, 1); t = t / s
+    tad1, tad0 = dev.tad(xi, [1]), dev.tad(xi, [0])
     ri = _vec(rows)
     ci = harness.shape_info([rows, 1])
-    M, S, T = w.operand(np.zeros(rows, F32), ri), w.operand(np.zeros(rows, F32), ri), w.operand(np.zeros(n, F32), xi)
-    D1, D0 = w.raw(np.array([1], np.int32)), w.raw(np.array([0], np.int32))
-    tad1, tad0 = dev.tad(xi, [1]), dev.tad(xi, [0])
-    ex_r = dev.extra(xi, z_info=ri, tad=tad1)
-    ex_b = dev.extra(xi, ci, xi, tad=tad0, tad_z=tad0)
-    ex_t = dev.extra(xi, z_info=xi)
     mc, sc, tc = np.zeros(rows, F32), np.zeros(rows, F32), np.zeros(n, F32)
-    w.host.update(softmax_cpu=tc)
-    steps = [
-        ("softmax_1_max", "reduce", 4 * n + 4 * rows,
-         lambda: ops.execReduceFloat(ex_r, R_MAX, X.ptr, X.info_ptr, None, M.ptr, M.info_ptr, D1.ptr, 1),
-         lambda lib: lib.reduce(R_MAX, x, xi, None, mc, ri, [1])),
-        ("softmax_2_subtract", "broadcast", 8 * n + 4 * rows,
-         lambda: ops.execBroadcastFloat(ex_b, B_SUB, X.ptr, X.info_ptr, M.ptr, M.info_ptr, T.ptr, T.info_ptr, D0.ptr, 1),
-         lambda lib: lib.broadcast(B_SUB, x, xi, mc, ci, tc, xi, [0])),
-        ("softmax_3_exp", "transform", 8 * n,
-         lambda: ops.execTransformFloat(ex_t, T_EXP, T.ptr, T.info_ptr, T.ptr, T.info_ptr, None),
-         lambda lib: lib.transform(T_EXP, tc, xi, tc, xi, None)),
-        ("softmax_4_sum", "reduce", 4 * n + 4 * rows,
-         lambda: ops.execReduceFloat(ex_r, R_SUM, T.ptr, T.info_ptr, None, S.ptr, S.info_ptr, D1.ptr, 1),
-         lambda lib: lib.reduce(R_SUM, tc, xi, None, sc, ri, [1])),
-        ("softmax_5_divide", "broadcast", 8 * n + 4 * rows,
-         lambda: ops.execBroadcastFloat(ex_b, B_DIV, T.ptr, T.info_ptr, S.ptr, S.info_ptr, T.ptr, T.info_ptr, D0.ptr, 1),
-         lambda lib: lib.broadcast(B_DIV, tc, xi, sc, ci, tc, xi, [0])),
-    ]
-    for name, fam, nbytes, gpu, cpu in steps:
-        w.cases.append(Case(name, fam, n, nbytes, gpu, cpu, False, T.get))
+    host_out = {(dim, out_len): np.zeros(out_len, F32) for dim, out_len in ((1, rows), (0, cols))}
 
-    def chain_gpu():
-        for _, _, _, g, _ in steps:
-            g()
+    def device_set(w):
+        cases = []
+        X = w.operand(x, xi)
+        for dim, out_len, tad in ((1, rows, tad1), (0, cols, tad0)):
+            zi = _vec(out_len)
+            Z = w.operand(np.zeros(out_len, F32), zi)
+            D = w.raw(np.array([dim], np.int32))
+            ex = dev.extra(xi, z_info=zi, tad=tad)
+            zc = host_out[(dim, out_len)]
+            for op, opname in ((S_VAR, "variance"), (S_STD, "std")):
+                def gpu(op=op, Z=Z, D=D, ex=ex):
+                    ops.execSummaryStatsFloat(ex, op, X.ptr, X.info_ptr, None, Z.ptr, Z.info_ptr, D.ptr, 1, 1)
 
-    def chain_cpu(lib):
-        for _, _, _, _, c in steps:
-            c(lib)
+                def cpu(lib, op=op, zc=zc, zi=zi, dim=dim):
+                    lib.summarystats(op, 1, x, xi, zc, zi, [dim])
 
-    w.cases.append(Case("softmax_chain", "chain", n, sum(s[2] for s in steps), chain_gpu, chain_cpu, False, T.get))
-    return w
+                # dim 0 TADs are the contiguous columns of the f-order matrix, dim 1 TADs have stride `rows`
+                cases.append(Case("%s_dim%d" % (opname, dim), "summarystats", n, 4 * n + 4 * out_len, gpu, cpu, dim == 0, Z.get))
+
+        # softmax along dimension 1 as five calls: m = max(x, 1); t = x - m; t = exp(t); s = sum(t, 1); t = t / s
+        M, S, T = w.operand(np.zeros(rows, F32), ri), w.operand(np.zeros(rows, F32), ri), w.operand(np.zeros(n, F32), xi)
+        D1, D0 = w.raw(np.array([1], np.int32)), w.raw(np.array([0], np.int32))
+        ex_r = dev.extra(xi, z_info=ri, tad=tad1)
+        ex_b = dev.extra(xi, ci, xi, tad=tad0, tad_z=tad0)
+        ex_t = dev.extra(xi, z_info=xi)
+        steps = [
+            ("softmax_1_max", "reduce", 4 * n + 4 * rows,
+             lambda: ops.execReduceFloat(ex_r, R_MAX, X.ptr, X.info_ptr, None, M.ptr, M.info_ptr, D1.ptr, 1),
+             lambda lib: lib.reduce(R_MAX, x, xi, None, mc, ri, [1])),
+            ("softmax_2_subtract", "broadcast", 8 * n + 4 * rows,
+             lambda: ops.execBroadcastFloat(ex_b, B_SUB, X.ptr, X.info_ptr, M.ptr, M.info_ptr, T.ptr, T.info_ptr, D0.ptr, 1),
+             lambda lib: lib.broadcast(B_SUB, x, xi, mc, ci, tc, xi, [0])),
+            ("softmax_3_exp", "transform", 8 * n,
+             lambda: ops.execTransformFloat(ex_t, T_EXP, T.ptr, T.info_ptr, T.ptr, T.info_ptr, None),
+             lambda lib: lib.transform(T_EXP, tc, xi, tc, xi, None)),
+            ("softmax_4_sum", "reduce", 4 * n + 4 * rows,
+             lambda: ops.execReduceFloat(ex_r, R_SUM, T.ptr, T.info_ptr, None, S.ptr, S.info_ptr, D1.ptr, 1),
+             lambda lib: lib.reduce(R_SUM, tc, xi, None, sc, ri, [1])),
+            ("softmax_5_divide", "broadcast", 8 * n + 4 * rows,
+             lambda: ops.execBroadcastFloat(ex_b, B_DIV, T.ptr, T.info_ptr, S.ptr, S.info_ptr, T.ptr, T.info_ptr, D0.ptr, 1),
+             lambda lib: lib.broadcast(B_DIV, tc, xi, sc, ci, tc, xi, [0])),
+        ]
+        for name, fam, nbytes, gpu, cpu in steps:
+            cases.append(Case(name, fam, n, nbytes, gpu, cpu, False, T.get))
+
+        def chain_gpu():
+            for st in steps:
+                st[3]()
+
+        def chain_cpu(lib):
+            for st in steps:
+                st[4](lib)
+
+        cases.append(Case("softmax_chain", "chain", n, sum(st[2] for st in steps), chain_gpu, chain_cpu, False, T.get))
+        return cases
+
+    return _replicated(dev, "summary stats var/std + softmax-style chain; fp32 [%d,%d] f-order" % (rows, cols), 8 * n,
+                       dict(x=x, xi=xi, softmax_cpu=tc), device_set, copies)
 
 
 # ---- configs[4]: random fills and dropout ---------------------------------------------------------------
-def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data_seed=5):
-    w = Workload(dev, "random uniform / gaussian fill 2^%d fp32, dropout p=0.5 in place [%d,%d]" % (int(np.log2(n)), side, side))
+def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data_seed=5, copies=None):
     ops = dev.ops
     host_buf = np.zeros(buffer_longs, np.uint64)
-    dev_buf = w.raw(np.zeros(buffer_longs, np.uint64))
+    dev_buf = dev.upload(np.zeros(buffer_longs, np.uint64))
     gen = ops.initRandom(dev.extra(host_buffer=host_buf.ctypes.data), seed, buffer_longs, dev_buf.ptr)
-    w.host.update(rng_buffer=host_buf, generator=gen, seed=seed, buffer_longs=buffer_longs)
     zi = _vec(n)
-    Z = w.operand(np.zeros(n, F32), zi)
-    a_uni, a_gau, a_drop = w.raw(np.array([0, 1], F32)), w.raw(np.array([0, 1], F32)), w.raw(np.array([0.5], F32))
-    ex = dev.extra()
     m = side * side
     di = harness.shape_info([side, side])
     xd = _normal(np.random.default_rng(data_seed), m, F32)
-    Xd = w.operand(xd, di)
-    w.host.update(dropout_x=xd, di=di, zi=zi)
     cpu_state = {}
 
     def cpu_gen(lib):
@@ -279,22 +317,33 @@ def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data
             cpu_state["x"] = xd.copy()
         return cpu_state["g"]
 
-    w.cases.append(Case("uniform_fill", "random", n, 4 * n,
-                        lambda: ops.execRandomFloat(ex, RND_UNIFORM, gen, Z.ptr, Z.info_ptr, a_uni.ptr),
-                        lambda lib: cpu_gen(lib).random_z(RND_UNIFORM, cpu_state["z"], zi, np.array([0, 1], F32)), True, Z.get))
-    w.cases.append(Case("gaussian_fill", "random", n, 4 * n,
-                        lambda: ops.execRandomFloat(ex, RND_GAUSSIAN, gen, Z.ptr, Z.info_ptr, Z.ptr, Z.info_ptr, Z.ptr, Z.info_ptr, a_gau.ptr),
-                        lambda lib: cpu_gen(lib).random_xyz(RND_GAUSSIAN, cpu_state["z"], zi, cpu_state["z"], zi, cpu_state["z"], zi,
-                                                            np.array([0, 1], F32)), True, Z.get))
-    w.cases.append(Case("dropout_inplace", "random", m, 8 * m,
-                        lambda: ops.execRandomFloat(ex, RND_DROPOUT, gen, Xd.ptr, Xd.info_ptr, Xd.ptr, Xd.info_ptr, a_drop.ptr),
-                        lambda lib: cpu_gen(lib).random_xz(RND_DROPOUT, cpu_state["x"], di, cpu_state["x"], di, np.array([0.5], F32)),
-                        True, Xd.get))
+    def device_set(w):
+        Z = w.operand(np.zeros(n, F32), zi)
+        a_uni, a_gau, a_drop = w.raw(np.array([0, 1], F32)), w.raw(np.array([0, 1], F32)), w.raw(np.array([0.5], F32))
+        ex = dev.extra()
+        Xd = w.operand(xd, di)
+        return [
+            Case("uniform_fill", "random", n, 4 * n,
+                 lambda: ops.execRandomFloat(ex, RND_UNIFORM, gen, Z.ptr, Z.info_ptr, a_uni.ptr),
+                 lambda lib: cpu_gen(lib).random_z(RND_UNIFORM, cpu_state["z"], zi, np.array([0, 1], F32)), True, Z.get),
+            Case("gaussian_fill", "random", n, 4 * n,
+                 lambda: ops.execRandomFloat(ex, RND_GAUSSIAN, gen, Z.ptr, Z.info_ptr, Z.ptr, Z.info_ptr, Z.ptr, Z.info_ptr, a_gau.ptr),
+                 lambda lib: cpu_gen(lib).random_xyz(RND_GAUSSIAN, cpu_state["z"], zi, cpu_state["z"], zi, cpu_state["z"], zi,
+                                                     np.array([0, 1], F32)), True, Z.get),
+            Case("dropout_inplace", "random", m, 8 * m,
+                 lambda: ops.execRandomFloat(ex, RND_DROPOUT, gen, Xd.ptr, Xd.info_ptr, Xd.ptr, Xd.info_ptr, a_drop.ptr),
+                 lambda lib: cpu_gen(lib).random_xz(RND_DROPOUT, cpu_state["x"], di, cpu_state["x"], di, np.array([0.5], F32)),
+                 True, Xd.get)]
+
+    w = _replicated(dev, "random uniform / gaussian fill 2^%d fp32, dropout p=0.5 in place [%d,%d]" % (int(np.log2(n)), side, side),
+                    4 * n + 4 * m, dict(rng_buffer=host_buf, generator=gen, seed=seed, buffer_longs=buffer_longs,
+                                        dropout_x=xd, di=di, zi=zi), device_set, copies)
     free0 = w.free
 
     def free():
         dev.sync()
         ops.destroyRandom(gen)
+        dev_buf.free()
         free0()
 
     w.free = free
