@@ -167,12 +167,19 @@ __global__ void __launch_bounds__(kBlock) bcRowKernel(const T *x, const T *y, T 
     const int rowsPerBlock = kBlock >> colShift;
     const int cIdx = threadIdx.x & (colThreads - 1);
     const int rIdx = threadIdx.x >> colShift;
+    const bool yAligned = (reinterpret_cast<uintptr_t>(y) & 15) == 0;
     Params<T> p{nullptr};
     for (Long col = ((Long)blockIdx.y * colThreads + cIdx) * VEC; col < tadLength; col += (Long)gridDim.y * colThreads * VEC) {
         const bool full = col + VEC <= tadLength;
         C yv[VEC];
+        if (full && yAligned) {
+            const Pack<T> yp = *reinterpret_cast<const Pack<T> *>(y + col);  // through the caches: every TAD re-reads it
 #pragma unroll
-        for (int e = 0; e < VEC; e++) yv[e] = (col + e < tadLength) ? toCompute(y[col + e]) : (C)0;
+            for (int e = 0; e < VEC; e++) yv[e] = toCompute(yp.v[e]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) yv[e] = (col + e < tadLength) ? toCompute(y[col + e]) : (C)0;
+        }
         const Long rowsPerPass = (Long)rowsPerBlock * kBcRows;
         for (Long r0 = (Long)blockIdx.x * rowsPerPass + rIdx; r0 < numTads; r0 += (Long)gridDim.x * rowsPerPass) {
             Long xo[kBcRows], zo[kBcRows];

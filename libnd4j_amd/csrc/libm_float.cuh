@@ -140,7 +140,9 @@ __device__ __forceinline__ float sincosCore(float y, bool wantCos) {
     return sincosPoly(x * s, x * x, wantCos ? (n ^ 1) : n, neg);
 }
 
-__device__ __forceinline__ float expm1f_(float x) {
+// expm1f exactly as fdlibm branches it; the branch-free expm1f_ below covers 2^-25 <= |x| < 27 ln2 and
+// leaves the rest (tiny, huge, infinite, NaN arguments) to this one.
+static __device__ __noinline__ float expm1fSlow_(float x) {
     const float one = 1.0f, tiny = 1.0e-30f, hugev = 1.0e30f, o_threshold = 8.8721679688e+01f,
                 ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f,
                 Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f, Q4 = 4.0082177293e-06f,
@@ -207,25 +209,68 @@ __device__ __forceinline__ float expm1f_(float x) {
     return y;
 }
 
+// The same arithmetic with the case distinctions turned into selects: every lane of a wave runs one
+// instruction stream whatever case its argument falls in.  fdlibm's cases differ only in k (0, +-1 near
+// +-ln2, round(x / ln2) otherwise - with t = k the reduction x - t ln2_hi, t ln2_lo is the same expression in
+// all of them) and in how the result is put together from the shared polynomial.
+__device__ __forceinline__ float expm1f_(float x0) {
+    const float one = 1.0f, ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f,
+                Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f, Q4 = 4.0082177293e-06f,
+                Q5 = -2.0109921195e-07f;
+    unsigned hx = asU32(x0);
+    const bool neg = (hx >> 31) != 0;
+    hx &= 0x7fffffffu;
+    if (__builtin_expect(hx >= 0x4195b844u || hx < 0x33000000u, 0)) return expm1fSlow_(x0);
+    const bool red = hx > 0x3eb17218u, nearLn2 = hx < 0x3F851592u;
+    const int kg = (int)(invln2 * x0 + (neg ? -0.5f : 0.5f));
+    const int k = red ? (nearLn2 ? (neg ? -1 : 1) : kg) : 0;
+    float t = (float)k;
+    const float hi = x0 - t * ln2_hi, lo = t * ln2_lo;
+    const float x = hi - lo;
+    const float c = (hi - x) - lo;
+    const float hfx = 0.5f * x, hxs = x * hfx;
+    const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    t = 3.0f - r1 * hfx;
+    const float e = hxs * ((r1 - t) / (6.0f - x * t));
+    const float res0 = x - (x * e - hxs);  // k == 0
+    float e2 = (x * (e - c) - c);
+    e2 -= hxs;
+    const float resM1 = 0.5f * (x - e2) - 0.5f;  // k == -1
+    const float resP1 = x < -0.25f ? -2.0f * (e2 - (x + 0.5f)) : one + 2.0f * (x - e2);  // k == 1
+    const unsigned sh = (unsigned)k << 23;
+    float yn = one - (e2 - x);  // k <= -2
+    yn = asF32(asU32(yn) + sh) - one;
+    const int kk = k < 0 ? 0 : (k > 31 ? 31 : k);
+    float ya = asF32(0x3f800000u - (0x1000000u >> kk)) - (e2 - x);  // 2 <= k < 23
+    ya = asF32(asU32(ya) + sh);
+    float yb = x - (e2 + asF32((unsigned)(0x7f - k) << 23));  // 23 <= k
+    yb += one;
+    yb = asF32(asU32(yb) + sh);
+    float r = k < 23 ? ya : yb;
+    r = k <= -2 ? yn : r;
+    r = k == 1 ? resP1 : r;
+    r = k == -1 ? resM1 : r;
+    r = k == 0 ? res0 : r;
+    return r;
+}
+
+// tanhf (s_tanhf.c): |x| >= 1: 1 - 2 / (expm1(2|x|) + 2); |x| < 1: -t / (t + 2) with t = expm1(-2|x|); |x| >= 22: 1;
+// |x| < 2^-55: x (1 + x).  One expm1f and one division serve all lanes.
 __device__ __forceinline__ float tanhf_(float x) {
     const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
-    float t, z;
     const int jx = (int)asU32(x);
     const int ix = jx & 0x7fffffff;
-    if (ix >= 0x7f800000) return jx >= 0 ? one / x + one : one / x - one;
-    if (ix < 0x41b00000) {  // |x| < 22
-        if (ix == 0) return x;
-        if (ix < 0x24000000) return x * (one + x);
-        // |x| >= 1: t = expm1(2|x|), z = 1 - 2 / (t + 2); else t = expm1(-2|x|), z = -t / (t + 2).  One expm1f and
-        // one division serve both cases, so lanes of a wave that fall on either side do not run the routine twice.
-        const bool big = ix >= 0x3f800000;
-        t = expm1f_((big ? two : -two) * __builtin_fabsf(x));
-        const float q = (big ? two : -t) / (t + two);
-        z = big ? one - q : q;
-    } else {
-        z = one - tiny;
-    }
-    return jx >= 0 ? z : -z;
+    if (__builtin_expect(ix >= 0x7f800000, 0)) return jx >= 0 ? one / x + one : one / x - one;
+    const bool big = ix >= 0x3f800000, sat = ix >= 0x41b00000;
+    float arg = (big ? two : -two) * __builtin_fabsf(x);
+    if (sat) arg = one;  // result unused; keeps expm1f_ on its main path
+    const float t = expm1f_(arg);
+    const float q = (big ? two : -t) / (t + two);
+    float z = big ? one - q : q;
+    z = sat ? one - tiny : z;
+    float r = jx >= 0 ? z : -z;
+    r = ix < 0x24000000 ? x * (one + x) : r;
+    return r;
 }
 
 // powf: sysdeps/ieee754/flt-32/e_powf.c.  log2(x) from a 16-entry 1/c, log2 c table and a degree-5 polynomial
