@@ -52,6 +52,7 @@ template <typename TT, int OP> struct IndexPol {
             }
         }
     }
+    __device__ __forceinline__ void checkpoint(Acc &) const {}
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const {
         if (OP <= 3) {
             return better(b.value, b.index, a.value, a.index) ? b : a;

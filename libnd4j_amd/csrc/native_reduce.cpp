@@ -96,12 +96,10 @@ template <> struct ScalarOut<float> { typedef float R; static R get(float v) { r
 template <> struct ScalarOut<double> { typedef double R; static R get(double v) { return v; } };
 template <> struct ScalarOut<float16> { typedef float R; static R get(float16 v) { return halfBitsToFloatHost(v.x); } };
 
-template <typename T> typename ScalarOut<T>::R readScalar(const void *devSlot, hipStream_t s, const char *what) {
-    T v;
-    std::memset(&v, 0, sizeof(T));
-    hipError_t e = hipMemcpyAsync(&v, devSlot, sizeof(T), hipMemcpyDeviceToHost, s);
-    if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+template <typename T> typename ScalarOut<T>::R readScalar(const void *pinnedSlot, hipStream_t s, const char *what) {
     syncAndCheck(what, s);
+    T v;
+    std::memcpy(&v, pinnedSlot, sizeof(T));
     return ScalarOut<T>::get(v);
 }
 
@@ -124,7 +122,7 @@ template <typename T> typename ScalarOut<T>::R reduceScalar(Nd4jPointer *extra, 
     const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
     if (hx == nullptr) return 0;
     Scratch sc = scratchFor(s);
-    T *slot = reinterpret_cast<T *>(sc.scalars);
+    T *slot = reinterpret_cast<T *>(pinnedScalarFor(s));
     if (!reduceScalarTo<T>(s, opNum, x, hx, params, slot)) { reportUnknownOp("reduce", opNum); return 0; }
     return readScalar<T>(slot, s, "execReduceScalar");
 }
@@ -179,7 +177,7 @@ template <typename T> typename ScalarOut<T>::R indexReduceScalar(Nd4jPointer *ex
     const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
     if (hx == nullptr) return 0;
     Scratch sc = scratchFor(s);
-    T *slot = reinterpret_cast<T *>(sc.scalars);
+    T *slot = reinterpret_cast<T *>(pinnedScalarFor(s));
     if (!indexScalarTo<T>(s, opNum, x, hx, params, slot)) { reportUnknownOp("indexreduce", opNum); return 0; }
     return readScalar<T>(slot, s, "execIndexReduceScalar");
 }
@@ -226,7 +224,7 @@ typename ScalarOut<T>::R statsScalar(Nd4jPointer *extra, int opNum, T *x, Long *
     const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
     if (hx == nullptr) return 0;
     Scratch sc = scratchFor(s);
-    T *slot = reinterpret_cast<T *>(sc.scalars);
+    T *slot = reinterpret_cast<T *>(pinnedScalarFor(s));
     if (!statsScalarTo<T>(s, opNum, bias, x, hx, slot)) { reportUnknownOp("summarystats", opNum); return 0; }
     return readScalar<T>(slot, s, "execSummaryStatsScalar");
 }

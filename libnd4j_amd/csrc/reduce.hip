@@ -93,6 +93,7 @@ template <typename TT, int OP> struct ReducePol {
     __device__ __forceinline__ void accumulate(Acc &a, C v, Long) const {
         a = ReduceOp<OP>::template update<C>(a, ReduceOp<OP>::template op<C>(v, p, shift));
     }
+    __device__ __forceinline__ void checkpoint(Acc &) const {}
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const { return ReduceOp<OP>::template update<C>(a, b); }
     __device__ __forceinline__ TT finalize(Acc a, Long n) const {
         return fromCompute<TT>(ReduceOp<OP>::template post<C>(a, n, p, shift));

@@ -6,14 +6,16 @@
 //     void accumulate(Acc &, C v, Long i)  fold element i (its position inside the TAD / array)
 //     Acc  combine(Acc a, Acc b)           merge two partial accumulators
 //     T    finalize(Acc, Long n)           post-process into the stored result
+//     void checkpoint(Acc &a)              called between groups of accumulate() calls; a policy may renormalise
 //     void setTad(Long r)                  per-TAD hook (LogSumExp reads its shift from the result array)
 //
 // Kernels:
 //   tadRowKernel<Pol, GROUP>  contiguous TADs (tadEws == 1): GROUP lanes walk one TAD with 16-byte loads,
 //                             wave64 cross-lane merge, LDS only across waves.
-//   tadColKernel<Pol>         strided TADs: one lane per TAD so that a row of adjacent TADs is one
-//                             coalesced request; the TAD length is split over blockIdx.y and merged by
-//                             tadColFinish when split.
+//   tadColVecKernel<Pol>      strided TADs that are adjacent in memory: one lane per 16 bytes' worth of TADs,
+//                             rows split over the waves of a block and over blockIdx.y (tadColFinish merges).
+//   tadColKernel<Pol>         other strided TADs and short contiguous ones: one lane per TAD; the TAD length
+//                             is split over blockIdx.y and merged by tadColFinish when split.
 //   tadGeneralKernel<Pol>     block per TAD with a coordinate map.
 //   flatKernel<Pol> + flatFinish<Pol>  two-stage grid reduction over the whole array.
 #pragma once
@@ -77,16 +79,29 @@ __device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc
     if ((addr & (sizeof(T) - 1)) == 0) head = (Long)(((16 - (addr & 15)) & 15) / sizeof(T));
     else head = n;  // cannot be vectorised
     if (head > n) head = n;
-    for (Long i = lane; i < head; i += lanes) pol.accumulate(acc, toCompute(p[i]), i);
+    for (Long i = lane; i < head; i += lanes) { pol.accumulate(acc, toCompute(p[i]), i); pol.checkpoint(acc); }
     const Long nvec = (n - head) / VEC;
     const Pack<T> *pv = reinterpret_cast<const Pack<T> *>(p + head);
-#pragma unroll 4
-    for (Long v = lane; v < nvec; v += lanes) {
+    Long v = lane;
+    // four independent 16-byte loads in flight per lane, then the arithmetic
+    for (; v + 3 * (Long)lanes < nvec; v += 4 * (Long)lanes) {
+        Pack<T> pk[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) pk[u] = loadPack(pv + v + u * (Long)lanes);
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[u].v[e]), head + (v + u * (Long)lanes) * VEC + e);
+            pol.checkpoint(acc);
+        }
+    }
+    for (; v < nvec; v += lanes) {
         Pack<T> pk = loadPack(pv + v);
 #pragma unroll
         for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk.v[e]), head + v * VEC + e);
+        pol.checkpoint(acc);
     }
-    for (Long i = head + nvec * VEC + lane; i < n; i += lanes) pol.accumulate(acc, toCompute(p[i]), i);
+    for (Long i = head + nvec * VEC + lane; i < n; i += lanes) { pol.accumulate(acc, toCompute(p[i]), i); pol.checkpoint(acc); }
 }
 
 template <class Pol, int GROUP>
@@ -137,10 +152,90 @@ __global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename P
         for (int u = 0; u < 8; u++) v[u] = base[(j + u) * tadEws];
 #pragma unroll
         for (int u = 0; u < 8; u++) pol.accumulate(acc, toCompute(v[u]), j + u);
+        pol.checkpoint(acc);
     }
-    for (; j < j1; j++) pol.accumulate(acc, toCompute(base[j * tadEws]), j);
+    for (; j < j1; j++) { pol.accumulate(acc, toCompute(base[j * tadEws]), j); pol.checkpoint(acc); }
     if (gridDim.y == 1) z[t] = pol.finalize(acc, tadLength);
     else partials[(Long)blockIdx.y * numTads + t] = acc;
+}
+
+// Strided TADs whose neighbours are neighbours in memory (columns of a c-order matrix, rows of an f-order
+// one): every lane owns Pack<T>::N adjacent TADs and reads them with one 16-byte load per row, so a wave
+// covers a contiguous kilobyte per row.  The four waves of a block take every fourth row of the block's row
+// range [rowsPerSplit * blockIdx.y, ...) and merge through LDS; row ranges are merged by tadColFinish.
+// Lanes whose TADs are not adjacent / aligned (checked against the offsets table) walk them one by one.
+template <class Pol>
+__global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
+                                                          typename Pol::Acc *partials, const Long *offsets, Long tadLength,
+                                                          Long numTads, Long tadEws, Long rowsPerSplit) {
+    typedef typename Pol::T T;
+    typedef typename Pol::Acc Acc;
+    constexpr int VEC = Pack<T>::N;
+    constexpr int WAVES = kBlock / kWave;
+    __shared__ Acc smem[(WAVES - 1) * kWave];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const Long t0 = ((Long)blockIdx.x * kWave + lane) * VEC;
+    const bool live = t0 < numTads;
+    const Long j0 = (Long)blockIdx.y * rowsPerSplit;
+    Long j1 = j0 + rowsPerSplit;
+    if (j1 > tadLength) j1 = tadLength;
+    Acc acc[VEC];
+    Pol pe[VEC];
+    if (live) {
+        Long off[VEC];
+        bool vec = t0 + VEC <= numTads;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            off[e] = (t0 + e < numTads) ? offsets[t0 + e] : 0;
+            pe[e] = pol;
+            if (t0 + e < numTads) pe[e].setTad(t0 + e, z);
+            acc[e] = pe[e].init(x + off[e]);
+            if (e > 0 && off[e] != off[0] + e) vec = false;
+        }
+        if ((reinterpret_cast<uintptr_t>(x + off[0]) & 15) != 0 || (tadEws % VEC) != 0) vec = false;
+        if (vec) {
+            const T *base = x + off[0];
+            Long j = j0 + wave;
+            for (; j + 3 * WAVES < j1; j += 4 * WAVES) {
+                Pack<T> pk[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) pk[u] = loadPack(reinterpret_cast<const Pack<T> *>(base + (j + u * WAVES) * tadEws));
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) pe[e].accumulate(acc[e], toCompute(pk[u].v[e]), j + u * WAVES);
+                }
+#pragma unroll
+                for (int e = 0; e < VEC; e++) pe[e].checkpoint(acc[e]);
+            }
+            for (; j < j1; j += WAVES) {
+                Pack<T> pk = loadPack(reinterpret_cast<const Pack<T> *>(base + j * tadEws));
+#pragma unroll
+                for (int e = 0; e < VEC; e++) { pe[e].accumulate(acc[e], toCompute(pk.v[e]), j); pe[e].checkpoint(acc[e]); }
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                if (t0 + e >= numTads) continue;
+                const T *base = x + off[e];
+                for (Long j = j0 + wave; j < j1; j += WAVES) { pe[e].accumulate(acc[e], toCompute(base[j * tadEws]), j); pe[e].checkpoint(acc[e]); }
+            }
+        }
+    }
+    // merge the four waves, one owned TAD at a time (keeps the LDS footprint at three waves of accumulators)
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        __syncthreads();
+        if (wave > 0) smem[(wave - 1) * kWave + lane] = acc[e];
+        __syncthreads();
+        if (wave == 0 && live && t0 + e < numTads) {
+            Acc a = acc[e];
+#pragma unroll
+            for (int w = 0; w < WAVES - 1; w++) a = pe[e].combine(a, smem[w * kWave + lane]);
+            if (gridDim.y == 1) z[t0 + e] = pe[e].finalize(a, tadLength);
+            else partials[(Long)blockIdx.y * numTads + t0 + e] = a;
+        }
+    }
 }
 
 // Merges the `splits` partial accumulators of each TAD: 64 TADs per block, the four waves of the block take
@@ -180,7 +275,7 @@ __global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typena
         const typename Pol::T *tx = x + offsets[r];
         Acc acc = pol.init(tx);
         for (Long f = threadIdx.x; f < tadLength; f += kBlock)
-            pol.accumulate(acc, toCompute(tx[mapOffset32(tm, (unsigned)f)]), f);
+            { pol.accumulate(acc, toCompute(tx[mapOffset32(tm, (unsigned)f)]), f); pol.checkpoint(acc); }
         acc = blockMerge<Pol>(pol, acc, smem);
         if (threadIdx.x == 0) z[r] = pol.finalize(acc, tadLength);
     }
@@ -216,24 +311,28 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
                 if (v < nvec) {
 #pragma unroll
                     for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[u].v[e]), head + v * VEC + e);
+                    pol.checkpoint(acc);
                 }
             }
         }
         if (blockIdx.x == 0) {
-            for (Long i = threadIdx.x; i < head; i += kBlock) pol.accumulate(acc, toCompute(x[i]), i);
-            for (Long i = head + nvec * VEC + threadIdx.x; i < n; i += kBlock) pol.accumulate(acc, toCompute(x[i]), i);
+            for (Long i = threadIdx.x; i < head; i += kBlock) { pol.accumulate(acc, toCompute(x[i]), i); pol.checkpoint(acc); }
+            for (Long i = head + nvec * VEC + threadIdx.x; i < n; i += kBlock) { pol.accumulate(acc, toCompute(x[i]), i); pol.checkpoint(acc); }
         }
     } else if (strided) {
         for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock)
-            pol.accumulate(acc, toCompute(x[i * ews]), i);
+            { pol.accumulate(acc, toCompute(x[i * ews]), i); pol.checkpoint(acc); }
     } else {
         for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock)
-            pol.accumulate(acc, toCompute(x[mapOffset32(xm, (unsigned)i)]), i);
+            { pol.accumulate(acc, toCompute(x[mapOffset32(xm, (unsigned)i)]), i); pol.checkpoint(acc); }
     }
     acc = blockMerge<Pol>(pol, acc, smem);
     if (threadIdx.x == 0) partials[blockIdx.x] = acc;
 }
 
+// Stage 2: one block merges the per-block partials.  (Doing this in the first launch, by the block that
+// arrives last at a ticket counter, needs a device-scope fence in every block; on this chip those fences cost
+// the streaming kernel more than twice its run time, a second launch costs a few microseconds.)
 template <class Pol>
 __global__ void __launch_bounds__(kBlock) flatFinish(Pol pol, const typename Pol::T *x, typename Pol::T *z,
                                                      const typename Pol::Acc *partials, int count, Long n) {
@@ -266,6 +365,29 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
             hipLaunchKernelGGL((tadRowKernel<Pol, 16>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets,
                                pl.tadLength, pl.numTads);
         }
+        return;
+    }
+    if (pl.kind == TadPlan::COL && pl.numTads >= 2 * kWave * Pack<typename Pol::T>::N) {
+        // lane per Pack::N adjacent TADs, 64 lanes per block column, rows split over the block's waves and blockIdx.y
+        constexpr int VEC = Pack<typename Pol::T>::N;
+        int gx = (int)((pl.numTads + (Long)kWave * VEC - 1) / ((Long)kWave * VEC));
+        Long splits = 2048 / gx;
+        if (splits < 1) splits = 1;
+        Long maxSplitsByRows = (pl.tadLength + 63) / 64;  // at least 16 rows per wave
+        if (splits > maxSplitsByRows) splits = maxSplitsByRows;
+        if (splits > 65535) splits = 65535;
+        size_t need = (size_t)splits * (size_t)pl.numTads * sizeof(Acc);
+        while (splits > 1 && need > ws.bytes) { splits /= 2; need = (size_t)splits * (size_t)pl.numTads * sizeof(Acc); }
+        if (splits < 1) splits = 1;
+        Long rowsPerSplit = (pl.tadLength + splits - 1) / splits;
+        splits = (pl.tadLength + rowsPerSplit - 1) / rowsPerSplit;
+        if (splits < 1) splits = 1;
+        Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+        hipLaunchKernelGGL((tadColVecKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
+                           pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit);
+        if (splits > 1)
+            hipLaunchKernelGGL((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kWave - 1) / kWave)), dim3(kBlock), 0, s, pol,
+                               z, partials, pl.tadLength, pl.numTads, (int)splits);
         return;
     }
     if (pl.kind == TadPlan::ROW || pl.kind == TadPlan::COL) {

@@ -1,5 +1,7 @@
 #include "runtime.h"
 
+#include <cstring>
+
 #include <map>
 #include <mutex>
 #include <utility>
@@ -110,6 +112,20 @@ Workspace workspaceFor(hipStream_t s, size_t minBytes) {
     w.ptr = p;
     w.bytes = want;
     return w;
+}
+
+void *pinnedScalarFor(hipStream_t s) {
+    static std::map<std::pair<int, hipStream_t>, void *> slots;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    std::lock_guard<std::mutex> lock(gMutex);
+    void *&p = slots[std::make_pair(dev, s)];
+    if (p == nullptr) {
+        hipError_t e = hipHostMalloc(&p, 256, hipHostMallocDefault);
+        if (e != hipSuccess) { p = nullptr; throwHip("pinned scalar slot", e); }
+        std::memset(p, 0, 256);
+    }
+    return p;
 }
 
 bool resolveTad(Nd4jPointer *extra, int hostSlot, int offsetSlot, const Long *hostXInfo, const int *dimension,

@@ -69,6 +69,9 @@ void reportUnknownOp(const char *family, int opNum);
 
 // Device scratch owned by the library, one per (device, stream), allocated on first use and kept.
 Workspace workspaceFor(hipStream_t s, size_t minBytes);
+// 256 bytes of pinned, device-visible host memory per (device, stream): the kernels of the scalar-returning
+// entry points write their result there, so the host reads it after the stream synchronisation without a copy.
+void *pinnedScalarFor(hipStream_t s);
 
 // TAD tables resolved for a call: host shapeInfo of one TAD + device offsets.
 struct ResolvedTad {

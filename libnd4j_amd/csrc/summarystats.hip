@@ -57,7 +57,11 @@ template <typename TT, int OP> struct StatsPol {
         a.cs1 += e;
         a.cs2 += e * e;
         a.cn += 1.0;
-        if (a.cn == kStatsRun) statsFlush(a);
+    }
+    // closes the current run once it holds kStatsRun samples or more (kept out of accumulate() so that the
+    // per-sample code is straight-line)
+    __device__ __forceinline__ void checkpoint(Acc &a) const {
+        if (a.cn >= kStatsRun) statsFlush(a);
     }
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const {
         statsFlush(a);

@@ -204,7 +204,8 @@ def test_reductions_without_caller_tad_tables(gpu, cpu):
 def test_tad_shapes_of_every_kernel_variant(gpu, cpu):
     # contiguous TADs of length 5 .. 20000 (sub-wave, wave, block kernels), strided TADs with and without splits
     rs = np.random.RandomState(26)
-    for rows, cols in ((300, 5), (64, 31), (40, 64), (33, 300), (7, 4100), (3, 20011), (2000, 3), (5, 1), (1, 17)):
+    for rows, cols in ((300, 5), (64, 31), (40, 64), (33, 300), (7, 4100), (3, 20011), (2000, 3), (5, 1), (1, 17),
+                       (1500, 1028), (130, 2050), (515, 516)):
         x = rs.randn(rows * cols).astype(np.float32)
         xi = shape_info_np([rows, cols])
         scale1 = np.abs(x).reshape(rows, cols).sum(axis=1) / np.sqrt(cols)
@@ -285,6 +286,15 @@ def test_half_families(gpu, cpu):
     assert np.array_equal(gpu.indexreduce(0, x, xi, None, [1], R), np.argmax(exact, axis=1).astype(h))
     g = gpu.summarystats(0, 1, x, xi, [0], C).astype(np.float64)
     assert np.all(np.abs(g - exact.var(axis=0, ddof=1)) <= 1e-2 * exact.var(axis=0, ddof=1))
+    # wide enough for the kernel that gives each lane eight adjacent strided TADs
+    R2, C2 = 200, 2056
+    x2 = rs.randn(R2 * C2).astype(h)
+    e2 = x2.astype(np.float64).reshape(R2, C2)
+    xi2 = shape_info_np([R2, C2])
+    assert np.array_equal(gpu.reduce(3, x2, xi2, None, [0], C2), e2.max(axis=0).astype(h))
+    assert np.array_equal(gpu.indexreduce(1, x2, xi2, None, [0], C2), np.argmin(e2, axis=0).astype(h))
+    g = gpu.reduce(1, x2, xi2, None, [0], C2).astype(np.float64)
+    assert np.all(np.abs(g - e2.sum(axis=0)) <= 1e-2 * np.maximum(np.abs(e2.sum(axis=0)), 1.0))
     # NaN is stored as 0x7fff
     nan_in = np.array([np.nan, 1.0], h)
     out = gpu.transform(6, nan_in, shape_info_np([1, 2]), shape_info_np([1, 2]))
@@ -299,6 +309,11 @@ def test_double_family_smoke(gpu, cpu):
     assert np.allclose(g, c, rtol=1e-14, atol=0)
     assert np.allclose(gpu.reduce(1, x, xi, None, [1], 10), cpu.reduce(1, x, xi, None, [1], 10), rtol=1e-13)
     assert float(gpu.indexreduce_scalar(0, x, xi)) == float(cpu.indexreduce_scalar(0, x, xi))
+    x = rs.randn(300 * 600).astype(np.float64)
+    xi = shape_info_np([300, 600])
+    assert np.allclose(gpu.reduce(1, x, xi, None, [0], 600), cpu.reduce(1, x, xi, None, [0], 600), rtol=1e-13)
+    assert np.array_equal(gpu.indexreduce(0, x, xi, None, [0], 600), cpu.indexreduce(0, x, xi, None, [0], 600))
+    assert np.allclose(gpu.summarystats(0, 1, x, xi, [0], 600), cpu.summarystats(0, 1, x, xi, [0], 600), rtol=1e-12)
 
 
 def test_random_ops_against_cpu(gpu, cpu):
