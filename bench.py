@@ -42,7 +42,8 @@ def parse():
     ap.add_argument("--counters", action="store_true",
                     help="for hardware-counter runs: launch the yardstick copy kernel (256 MiB) and each headline kernel "
                          "3 times and exit")
-    ap.add_argument("--traffic", default=None, help="JSON file with measured HBM bytes per launch of the dominant kernel")
+    ap.add_argument("--traffic", default=os.path.join(ROOT, "profiles", "headline_step_hbm_traffic.txt"),
+                    help="rocprofv3 counter summary holding the measured HBM bytes per launch of the dominant kernel")
     return ap.parse_args()
 
 
@@ -81,6 +82,21 @@ def time_case(dev, case, steps, warmup):
     ms = t.ms(0, 1) / steps
     t.destroy()
     return ms
+
+
+def measured_traffic(path, kernel):
+    """HBM bytes per launch of `kernel` from the committed counter summary (FETCH_SIZE and WRITE_SIZE runs of
+    `bench.py --counters`, scaled by a copy kernel of known size); None when the summary is not there."""
+    if not path or not os.path.exists(path):
+        return None
+    with open(path) as f:
+        for line in f:
+            if kernel in line:
+                try:
+                    return int(line.split()[-1])
+                except ValueError:
+                    return None
+    return None
 
 
 def load_cpu():
@@ -153,10 +169,7 @@ def main():
     ms_per_step = wall * 1e3 / K
     value = step_bytes / (wall / K) / 1e9
 
-    traffic = None
-    if args.traffic and os.path.exists(args.traffic):
-        with open(args.traffic) as f:
-            traffic = json.load(f).get("bytes_per_launch")
+    traffic = measured_traffic(args.traffic, "ewVecKernel<float, nd4j_amd::Pairwise3F<0>")
     achieved = add.bytes / (per_kernel_ms[0] * 1e-3) / 1e9
     out = {
         "metric": "achieved HBM GB/s (algorithmic bytes) of the legacy op path: pairwise add + pairwise multiply + broadcast add row",

@@ -4,8 +4,8 @@
 A builder generates the synthetic inputs on the host (seeded numpy generators), keeps them resident on the
 device, prepares shapeInfo / TAD tables / extraPointers once (as nd4j's executioner caches them) and returns
 ``Case`` objects.  ``case.gpu()`` enqueues exactly one call of the library on the device stream;
-``case.cpu(lib)`` runs the same call on a CPU checker from tests/cpu_ref.py (used by bench.py's CPU baseline
-and by the tests only).  ``case.bytes`` is the algorithmic traffic of one call: every input element read once,
+``case.cpu(lib)`` runs the same call on a CPU checker from tests/cpu_ref.py and returns its output (used by
+bench.py's CPU baseline and by the tests only).  ``case.bytes`` is the algorithmic traffic of one call: every input element read once,
 every output element written once.
 """
 import numpy as np
@@ -134,7 +134,7 @@ def transform_tanh(dev, n=1 << 24, seed=42, copies=None):
         ex = dev.extra(xi, z_info=xi)
         return [Case("transform_tanh", "transform", n, 8 * n,
                      lambda: ops.execTransformFloat(ex, T_TANH, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, None),
-                     lambda lib: lib.transform(T_TANH, x, xi, zc, xi, None), True, Z.get)]
+                     lambda lib: (lib.transform(T_TANH, x, xi, zc, xi, None), zc)[1], True, Z.get)]
 
     return _replicated(dev, "transform tanh fp32 1-D 2^%d" % int(np.log2(n)), 8 * n, dict(x=x, xi=xi, z_cpu=zc),
                        device_set, copies)
@@ -167,11 +167,11 @@ def pairwise_broadcast(dev, rows=65536, cols=1024, seed=7, dtype=F32, copies=Non
             bc(ex_b, B_ADD, X.ptr, X.info_ptr, B.ptr, B.info_ptr, Z.ptr, Z.info_ptr, D.ptr, 1)
 
         return [Case("pairwise_add" + tag, "pairwise", n, 3 * sz * n, mk_pw(P_ADD),
-                     lambda lib: lib.pairwise(P_ADD, x, xi, y, xi, zc, xi, None), True, Z.get),
+                     lambda lib: (lib.pairwise(P_ADD, x, xi, y, xi, zc, xi, None), zc)[1], True, Z.get),
                 Case("pairwise_multiply" + tag, "pairwise", n, 3 * sz * n, mk_pw(P_MUL),
-                     lambda lib: lib.pairwise(P_MUL, x, xi, y, xi, zc, xi, None), True, Z.get),
+                     lambda lib: (lib.pairwise(P_MUL, x, xi, y, xi, zc, xi, None), zc)[1], True, Z.get),
                 Case("broadcast_add_row" + tag, "broadcast", n, 2 * sz * n + sz * cols, gpu_bc,
-                     lambda lib: lib.broadcast(B_ADD, x, xi, bias, bi, zc, xi, [1]), True, Z.get)]
+                     lambda lib: (lib.broadcast(B_ADD, x, xi, bias, bi, zc, xi, [1]), zc)[1], True, Z.get)]
 
     return _replicated(dev, "pairwise add+multiply, broadcast add row; %s [%d,%d] c-order" % (dtype.name, rows, cols),
                        3 * sz * n, dict(x=x, y=y, bias=bias, xi=xi, bi=bi, z_cpu=zc), device_set, copies)
@@ -205,6 +205,7 @@ def reductions(dev, rows=16384, cols=4096, seed=11, copies=None):
 
                 def cpu(lib, cpu_name=cpu_name, op=op, zc=zc, zi=zi, dim=dim):
                     getattr(lib, cpu_name)(op, x, xi, None, zc, zi, [dim])
+                    return zc
 
                 cases.append(Case("%s_dim%d" % (opname, dim), fam, n, 4 * n + 4 * out_len, gpu, cpu, dim == 1, Z.get))
         ex_s = dev.extra(xi)
@@ -253,6 +254,7 @@ def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
 
                 def cpu(lib, op=op, zc=zc, zi=zi, dim=dim):
                     lib.summarystats(op, 1, x, xi, zc, zi, [dim])
+                    return zc
 
                 # dim 0 TADs are the contiguous columns of the f-order matrix, dim 1 TADs have stride `rows`
                 cases.append(Case("%s_dim%d" % (opname, dim), "summarystats", n, 4 * n + 4 * out_len, gpu, cpu, dim == 0, Z.get))
@@ -266,19 +268,19 @@ def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
         steps = [
             ("softmax_1_max", "reduce", 4 * n + 4 * rows,
              lambda: ops.execReduceFloat(ex_r, R_MAX, X.ptr, X.info_ptr, None, M.ptr, M.info_ptr, D1.ptr, 1),
-             lambda lib: lib.reduce(R_MAX, x, xi, None, mc, ri, [1])),
+             lambda lib: (lib.reduce(R_MAX, x, xi, None, mc, ri, [1]), mc)[1]),
             ("softmax_2_subtract", "broadcast", 8 * n + 4 * rows,
              lambda: ops.execBroadcastFloat(ex_b, B_SUB, X.ptr, X.info_ptr, M.ptr, M.info_ptr, T.ptr, T.info_ptr, D0.ptr, 1),
-             lambda lib: lib.broadcast(B_SUB, x, xi, mc, ci, tc, xi, [0])),
+             lambda lib: (lib.broadcast(B_SUB, x, xi, mc, ci, tc, xi, [0]), tc)[1]),
             ("softmax_3_exp", "transform", 8 * n,
              lambda: ops.execTransformFloat(ex_t, T_EXP, T.ptr, T.info_ptr, T.ptr, T.info_ptr, None),
-             lambda lib: lib.transform(T_EXP, tc, xi, tc, xi, None)),
+             lambda lib: (lib.transform(T_EXP, tc, xi, tc, xi, None), tc)[1]),
             ("softmax_4_sum", "reduce", 4 * n + 4 * rows,
              lambda: ops.execReduceFloat(ex_r, R_SUM, T.ptr, T.info_ptr, None, S.ptr, S.info_ptr, D1.ptr, 1),
-             lambda lib: lib.reduce(R_SUM, tc, xi, None, sc, ri, [1])),
+             lambda lib: (lib.reduce(R_SUM, tc, xi, None, sc, ri, [1]), sc)[1]),
             ("softmax_5_divide", "broadcast", 8 * n + 4 * rows,
              lambda: ops.execBroadcastFloat(ex_b, B_DIV, T.ptr, T.info_ptr, S.ptr, S.info_ptr, T.ptr, T.info_ptr, D0.ptr, 1),
-             lambda lib: lib.broadcast(B_DIV, tc, xi, sc, ci, tc, xi, [0])),
+             lambda lib: (lib.broadcast(B_DIV, tc, xi, sc, ci, tc, xi, [0]), tc)[1]),
         ]
         for name, fam, nbytes, gpu, cpu in steps:
             cases.append(Case(name, fam, n, nbytes, gpu, cpu, False, T.get))
@@ -290,6 +292,7 @@ def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
         def chain_cpu(lib):
             for st in steps:
                 st[4](lib)
+            return tc
 
         cases.append(Case("softmax_chain", "chain", n, sum(st[2] for st in steps), chain_gpu, chain_cpu, False, T.get))
         return cases
@@ -325,19 +328,20 @@ def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data
         return [
             Case("uniform_fill", "random", n, 4 * n,
                  lambda: ops.execRandomFloat(ex, RND_UNIFORM, gen, Z.ptr, Z.info_ptr, a_uni.ptr),
-                 lambda lib: cpu_gen(lib).random_z(RND_UNIFORM, cpu_state["z"], zi, np.array([0, 1], F32)), True, Z.get),
+                 lambda lib: (cpu_gen(lib).random_z(RND_UNIFORM, cpu_state["z"], zi, np.array([0, 1], F32)), cpu_state["z"])[1], True, Z.get),
             Case("gaussian_fill", "random", n, 4 * n,
                  lambda: ops.execRandomFloat(ex, RND_GAUSSIAN, gen, Z.ptr, Z.info_ptr, Z.ptr, Z.info_ptr, Z.ptr, Z.info_ptr, a_gau.ptr),
-                 lambda lib: cpu_gen(lib).random_xyz(RND_GAUSSIAN, cpu_state["z"], zi, cpu_state["z"], zi, cpu_state["z"], zi,
-                                                     np.array([0, 1], F32)), True, Z.get),
+                 lambda lib: (cpu_gen(lib).random_xyz(RND_GAUSSIAN, cpu_state["z"], zi, cpu_state["z"], zi, cpu_state["z"], zi,
+                                                     np.array([0, 1], F32)), cpu_state["z"])[1], True, Z.get),
             Case("dropout_inplace", "random", m, 8 * m,
                  lambda: ops.execRandomFloat(ex, RND_DROPOUT, gen, Xd.ptr, Xd.info_ptr, Xd.ptr, Xd.info_ptr, a_drop.ptr),
-                 lambda lib: cpu_gen(lib).random_xz(RND_DROPOUT, cpu_state["x"], di, cpu_state["x"], di, np.array([0.5], F32)),
+                 lambda lib: (cpu_gen(lib).random_xz(RND_DROPOUT, cpu_state["x"], di, cpu_state["x"], di, np.array([0.5], F32)), cpu_state["x"])[1],
                  True, Xd.get)]
 
+    host_cpu_state = cpu_state
     w = _replicated(dev, "random uniform / gaussian fill 2^%d fp32, dropout p=0.5 in place [%d,%d]" % (int(np.log2(n)), side, side),
                     4 * n + 4 * m, dict(rng_buffer=host_buf, generator=gen, seed=seed, buffer_longs=buffer_longs,
-                                        dropout_x=xd, di=di, zi=zi), device_set, copies)
+                                        dropout_x=xd, di=di, zi=zi, cpu_state=host_cpu_state), device_set, copies)
     free0 = w.free
 
     def free():
