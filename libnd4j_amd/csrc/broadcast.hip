@@ -17,7 +17,10 @@ template <typename T> struct BroadcastBody {
                 const int colThreads = 1 << colShift, rowsPerBlock = kBlock >> colShift;
                 Long gy = (vecsPerTad + colThreads - 1) / colThreads;
                 if (gy > 65535) gy = 65535;
-                int gx = gridFor(pl.numTads, (Long)rowsPerBlock * kBcRows, kMaxGrid);
+                // four passes per block (the y vector is loaded once per block) while that leaves >= 4096 blocks
+                Long perBlock = (Long)rowsPerBlock * kBcRows;
+                if ((pl.numTads / (perBlock * 4)) * gy >= 4096) perBlock *= 4;
+                int gx = gridFor(pl.numTads, perBlock, kMaxGrid);
                 int aligned = (((uintptr_t)x | (uintptr_t)z) & 15) == 0 ? 1 : 0;
                 hipLaunchKernelGGL((bcRowKernel<T, F>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
                                    pl.zOffsets, pl.tadLength, pl.numTads, aligned, colShift);
