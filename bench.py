@@ -218,7 +218,8 @@ def main():
     # ---- every other family ---------------------------------------------------------------------------
     if args.families:
         fam = []
-        builders = [workloads.transform_tanh, lambda d: workloads.pairwise_broadcast(d, dtype="float16"),
+        builders = [workloads.transform_tanh, lambda d: workloads.pairwise_broadcast(d, copies=2),
+                    lambda d: workloads.pairwise_broadcast(d, dtype="float16"),
                     workloads.reductions, workloads.stats_softmax, workloads.random_fills]
         for build in builders:
             wl = build(dev)

@@ -85,8 +85,27 @@
     void execRandom##SUFFIX(Nd4jPointer *extraPointers, int opNum, Nd4jPointer state, T *x,                     \
                             Nd4jLong *xShapeBuffer, T *z, Nd4jLong *zShapeBuffer, T *extraArguments);
 
+// Scalar family, reference: blas/NativeOps.h:1046-1146 and 1160-1226 (Float / Half), 377-440 and 1183-1203
+// (Double): strided, shaped, indexed (launches nothing in the reference's CUDA back end:
+// blas/cuda/NativeOps.cu:2788-2816) and one-scalar-per-TAD overloads.  S is the by-value scalar type.
+#define ND4J_SCALAR_MEMBERS(SUFFIX, T, S)                                                                       \
+    void execScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong xStride, T *result,           \
+                            Nd4jLong resultStride, S scalar, T *extraParams, Nd4jLong n);                        \
+    void execScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *result,       \
+                            Nd4jLong *resultShapeInfo, S scalar, T *extraParams);                                \
+    void execScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *result,       \
+                            Nd4jLong *resultShapeInfo, S scalar, T *extraParams, Nd4jLong *xIndexes,             \
+                            Nd4jLong *resultIndexes);                                                            \
+    void execScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *z,            \
+                            Nd4jLong *zShapeInfo, T *scalars, T *extraParams, int *dimension,                    \
+                            int dimensionLength);
+
 class ND4J_EXPORT NativeOps {
 public:
+    ND4J_SCALAR_MEMBERS(Float, float, float)
+    ND4J_SCALAR_MEMBERS(Half, float16, float)
+    ND4J_SCALAR_MEMBERS(Double, double, double)
+
     ND4J_EXEC_MEMBERS(Float, float, float)
     ND4J_EXEC_MEMBERS(Half, float16, float)
     ND4J_EXEC_MEMBERS(Double, double, double)
@@ -143,3 +162,4 @@ public:
 };
 
 #undef ND4J_EXEC_MEMBERS
+#undef ND4J_SCALAR_MEMBERS

@@ -87,6 +87,26 @@ ND4J_C_EXEC(Half, float16, float)
 ND4J_C_EXEC(Double, double, double)
 #undef ND4J_C_EXEC
 
+/* Scalar family (blas/NativeOps.h:1046-1226, 377-440): z = op(x, scalar, extraParams).  Strided, shaped,
+ * indexed (a no-op, as in the reference's CUDA back end) and one-scalar-per-TAD variants; S is float for
+ * Float and Half, double for Double. */
+#define ND4J_C_SCALAR(SUFFIX, T, S)                                                                              \
+    void nd4j_execScalar##SUFFIX##Strided(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong xStride,         \
+                                          T *result, Nd4jLong resultStride, S scalar, T *extraParams,             \
+                                          Nd4jLong n);                                                            \
+    void nd4j_execScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *result,   \
+                                 Nd4jLong *resultShapeInfo, S scalar, T *extraParams);                            \
+    void nd4j_execScalar##SUFFIX##Indexed(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,     \
+                                          T *result, Nd4jLong *resultShapeInfo, S scalar, T *extraParams,         \
+                                          Nd4jLong *xIndexes, Nd4jLong *resultIndexes);                           \
+    void nd4j_execScalar##SUFFIX##AlongDimension(Nd4jPointer *extraPointers, int opNum, T *x,                    \
+                                                 Nd4jLong *xShapeInfo, T *z, Nd4jLong *zShapeInfo, T *scalars,    \
+                                                 T *extraParams, int *dimension, int dimensionLength);
+ND4J_C_SCALAR(Float, float, float)
+ND4J_C_SCALAR(Half, float16, float)
+ND4J_C_SCALAR(Double, double, double)
+#undef ND4J_C_SCALAR
+
 Nd4jPointer nd4j_initRandom(Nd4jPointer *extraPointers, long seed, long bufferSize, Nd4jPointer ptrToBuffer);
 void nd4j_refreshBuffer(Nd4jPointer *extraPointers, long seed, Nd4jPointer ptrRandom);
 void nd4j_reSeedBuffer(Nd4jPointer *extraPointers, long seed, Nd4jPointer ptrRandom);

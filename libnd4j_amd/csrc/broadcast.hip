@@ -22,16 +22,16 @@ template <typename T> struct BroadcastBody {
                 if ((pl.numTads / (perBlock * 4)) * gy >= 4096) perBlock *= 4;
                 int gx = gridFor(pl.numTads, perBlock, kMaxGrid);
                 int aligned = (((uintptr_t)x | (uintptr_t)z) & 15) == 0 ? 1 : 0;
-                hipLaunchKernelGGL((bcRowKernel<T, F>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
-                                   pl.zOffsets, pl.tadLength, pl.numTads, aligned, colShift);
+                hipLaunchKernelGGL((bcRowKernel<T, F, false>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
+                                   pl.zOffsets, pl.tadLength, pl.numTads, aligned, colShift, Params<T>{nullptr});
             } else if (pl.kind == BroadcastPlan::COL) {
                 int gx = (int)((pl.numTads + kBlock - 1) / kBlock);
                 Long gy = (Long)kGridCap / gx;
                 if (gy < 1) gy = 1;
                 if (gy > pl.tadLength) gy = pl.tadLength;
                 if (gy > 65535) gy = 65535;
-                hipLaunchKernelGGL((bcColKernel<T, F>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
-                                   pl.zOffsets, pl.tadLength, pl.numTads, pl.tadEws, pl.yEws, pl.zEws);
+                hipLaunchKernelGGL((bcColKernel<T, F, false>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
+                                   pl.zOffsets, pl.tadLength, pl.numTads, pl.tadEws, pl.yEws, pl.zEws, Params<T>{nullptr});
             } else {
                 int grid = gridFor(pl.numTads, 1, kGridCap);
                 hipLaunchKernelGGL((bcGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, pl.xm, y, pl.ym, z, pl.zm,

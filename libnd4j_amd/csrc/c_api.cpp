@@ -106,6 +106,27 @@ ND4J_C_EXEC(Half, float16, float)
 ND4J_C_EXEC(Double, double, double)
 #undef ND4J_C_EXEC
 
+#define ND4J_C_SCALAR(SUFFIX, T, S)                                                                                \
+    void nd4j_execScalar##SUFFIX##Strided(Nd4jPointer *e, int op, T *x, Nd4jLong xs, T *r, Nd4jLong rs, S sc, T *p, \
+                                          Nd4jLong n) {                                                             \
+        guardVoid([&] { gOps.execScalar##SUFFIX(e, op, x, xs, r, rs, sc, p, n); });                                 \
+    }                                                                                                              \
+    void nd4j_execScalar##SUFFIX(Nd4jPointer *e, int op, T *x, Nd4jLong *xs, T *r, Nd4jLong *rs, S sc, T *p) {      \
+        guardVoid([&] { gOps.execScalar##SUFFIX(e, op, x, xs, r, rs, sc, p); });                                    \
+    }                                                                                                              \
+    void nd4j_execScalar##SUFFIX##Indexed(Nd4jPointer *e, int op, T *x, Nd4jLong *xs, T *r, Nd4jLong *rs, S sc,     \
+                                          T *p, Nd4jLong *xi, Nd4jLong *ri) {                                       \
+        guardVoid([&] { gOps.execScalar##SUFFIX(e, op, x, xs, r, rs, sc, p, xi, ri); });                            \
+    }                                                                                                              \
+    void nd4j_execScalar##SUFFIX##AlongDimension(Nd4jPointer *e, int op, T *x, Nd4jLong *xs, T *z, Nd4jLong *zs,    \
+                                                 T *scalars, T *p, int *dim, int dl) {                              \
+        guardVoid([&] { gOps.execScalar##SUFFIX(e, op, x, xs, z, zs, scalars, p, dim, dl); });                      \
+    }
+ND4J_C_SCALAR(Float, float, float)
+ND4J_C_SCALAR(Half, float16, float)
+ND4J_C_SCALAR(Double, double, double)
+#undef ND4J_C_SCALAR
+
 Nd4jPointer nd4j_initRandom(Nd4jPointer *e, long seed, long size, Nd4jPointer buf) {
     return guardRet<Nd4jPointer>(nullptr, [&] { return gOps.initRandom(e, seed, size, buf); });
 }

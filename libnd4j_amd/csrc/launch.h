@@ -35,6 +35,18 @@ struct BroadcastPlan {
 template <typename T>
 bool launchBroadcast(hipStream_t stream, int opNum, const T *x, const T *y, T *z, const BroadcastPlan &plan);
 
+// ---- scalar ----------------------------------------------------------------------------------------
+template <typename T>
+bool launchScalarStrided(hipStream_t stream, int opNum, const T *x, Long xs, T *z, Long zs,
+                         typename Compute<T>::type scalar, const T *extra, Long n);
+template <typename T>
+bool launchScalarGeneral(hipStream_t stream, int opNum, const T *x, const DimMap &xm, T *z, const DimMap &zm,
+                         typename Compute<T>::type scalar, const T *extra, Long n);
+// one scalar per TAD: plan.kind ROW (tadEws == 1) or COL (tadEws > 1); yEws is unused
+template <typename T>
+bool launchScalarTad(hipStream_t stream, int opNum, const T *x, const T *scalars, T *z, const T *extra,
+                     const BroadcastPlan &plan);
+
 // ---- reductions ------------------------------------------------------------------------------------
 // How the elements of one TAD are addressed and how TADs relate to each other.
 struct TadPlan {

@@ -5,6 +5,7 @@
 //   broadcast  include/loops/cpu/broadcasting.cpp:42-156
 // extraPointers are decoded as the reference's CUDA back end does (blas/cuda/NativeOps.cu:1813-1823,
 // 3100-3131).
+#include <cstdio>
 #include <cstring>
 
 #include "../../include/NativeOps.h"
@@ -177,9 +178,99 @@ void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Lon
     checkLaunch("execBroadcast", s);
 }
 
+// ---- scalar family (include/loops/cpu/scalar.cpp) ---------------------------------------------------
+template <typename T, typename S>
+void scalarStrided(Nd4jPointer *extra, int opNum, T *x, Long xs, T *z, Long zs, S scalar, T *params, Long n) {
+    hipStream_t s = streamOf(extra);
+    if (!launchScalarStrided<T>(s, opNum, x, xs, z, zs, (typename Compute<T>::type)scalar, params, n)) {
+        reportUnknownOp("scalar", opNum);
+        return;
+    }
+    checkLaunch("execScalar(strided)", s);
+}
+
+template <typename T, typename S>
+void scalarShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, Long *zInfo, S scalar, T *params) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx, sz;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    const Long *hz = hostShapeInfo(extra, X_HOST_Z_SHAPE, zInfo, sz, s);
+    if (hx == nullptr || hz == nullptr) return;
+    Long n = siNumel(hx);
+    Long xe = siEws(hx), ze = siEws(hz);
+    const typename Compute<T>::type sv = (typename Compute<T>::type)scalar;
+    bool ok;
+    if (xe >= 1 && ze >= 1 && siOrder(hx) == siOrder(hz)) {
+        // scalar.cpp:129-132, 187-191
+        ok = launchScalarStrided<T>(s, opNum, x, xe, z, ze, sv, params, n);
+    } else {
+        // raw iteration over x's shape with both stride sets (scalar.cpp:135-181)
+        const Long *strides[3] = {siStride(hx), nullptr, siStride(hz)};
+        DimMap maps[3];
+        jointCanon(siRank(hx), siShape(hx), strides, maps);
+        ok = launchScalarGeneral<T>(s, opNum, x, maps[0], z, maps[2], sv, params, n);
+    }
+    if (!ok) { reportUnknownOp("scalar", opNum); return; }
+    checkLaunch("execScalar", s);
+}
+
+// one scalar per TAD along `dimension` (scalar.cpp:14-62)
+template <typename T>
+void scalarAlongDimension(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, Long *zInfo, T *scalars, T *params,
+                          int *dimension, int dimLen) {
+    (void)zInfo;
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    if (hx == nullptr) return;
+    ResolvedTad tx;
+    if (!resolveTad(extra, X_HOST_TAD_SHAPE, X_DEV_TAD_OFFSETS, hx, dimension, dimLen, tx, s)) return;
+    const Long *devZOff = reinterpret_cast<const Long *>(slotOf(extra, X_DEV_TAD_OFFSETS_Z));
+    BroadcastPlan pl;
+    pl.tadLength = tx.tadLength;
+    pl.numTads = tx.numTads;
+    pl.xOffsets = tx.devOffsets;
+    pl.zOffsets = devZOff != nullptr ? devZOff : tx.devOffsets;
+    pl.tadEws = siEws(tx.hostInfo);
+    pl.yEws = 0;
+    pl.zEws = pl.tadEws;  // the reference takes z's stride from the x TAD as well (scalar.cpp:22-23)
+    if (pl.tadEws < 1) {
+        // the only branch the reference has for such TADs (scalar.cpp:56-58)
+        std::printf("Super-bad loop visited. Shouldn't ever happen\n");
+        return;
+    }
+    pl.kind = pl.tadEws == 1 ? BroadcastPlan::ROW : BroadcastPlan::COL;
+    if (!launchScalarTad<T>(s, opNum, x, scalars, z, params, pl)) { reportUnknownOp("scalar", opNum); return; }
+    checkLaunch("execScalar(dimension)", s);
+}
+
 }  // namespace
 
 // ---- per-type members ---------------------------------------------------------------------------------
+#define ND4J_SCALAR_MEMBERS(SUFFIX, T, S)                                                                        \
+    void NativeOps::execScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong xStride, T *result, \
+                                       Nd4jLong resultStride, S scalar, T *extraParams, Nd4jLong n) {            \
+        scalarStrided<T, S>(extraPointers, opNum, x, xStride, result, resultStride, scalar, extraParams, n);     \
+    }                                                                                                            \
+    void NativeOps::execScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,        \
+                                       T *result, Nd4jLong *resultShapeInfo, S scalar, T *extraParams) {         \
+        scalarShaped<T, S>(extraPointers, opNum, x, xShapeInfo, result, resultShapeInfo, scalar, extraParams);   \
+    }                                                                                                            \
+    void NativeOps::execScalar##SUFFIX(Nd4jPointer *, int, T *, Nd4jLong *, T *, Nd4jLong *, S, T *, Nd4jLong *, \
+                                       Nd4jLong *) {                                                             \
+        /* indexed variant: launches nothing in the reference's CUDA back end (blas/cuda/NativeOps.cu:2788-2816) */ \
+    }                                                                                                            \
+    void NativeOps::execScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo, T *z,  \
+                                       Nd4jLong *zShapeInfo, T *scalars, T *extraParams, int *dimension,         \
+                                       int dimensionLength) {                                                    \
+        scalarAlongDimension<T>(extraPointers, opNum, x, xShapeInfo, z, zShapeInfo, scalars, extraParams,        \
+                                dimension, dimensionLength);                                                     \
+    }
+ND4J_SCALAR_MEMBERS(Float, float, float)
+ND4J_SCALAR_MEMBERS(Half, float16, float)
+ND4J_SCALAR_MEMBERS(Double, double, double)
+#undef ND4J_SCALAR_MEMBERS
+
 #define ND4J_ELEMENTWISE_MEMBERS(SUFFIX, T)                                                                      \
     void NativeOps::execTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong xStride,        \
                                           T *result, Nd4jLong resultStride, T *extraParams, Nd4jLong n) {        \

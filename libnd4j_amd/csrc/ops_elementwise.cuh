@@ -412,6 +412,37 @@ __host__ __device__ constexpr int pairwiseKind(int opNum) {
 }
 static constexpr int kPairwiseOpCount = 95;
 
+// SCALAR_OPS (include/loops/legacy_ops.h:165-189)
+__host__ __device__ constexpr int scalarKind(int opNum) {
+    switch (opNum) {
+        case 0: return B_Add;
+        case 1: return B_Subtract;
+        case 2: return B_Multiply;
+        case 3: return B_Divide;
+        case 4: return B_ReverseDivide;
+        case 5: return B_ReverseSubtract;
+        case 6: return B_Max;
+        case 7: return B_LessThan;
+        case 8: return B_GreaterThan;
+        case 9: return B_EqualTo;
+        case 10: return B_LessThanOrEqual;
+        case 11: return B_NotEqualTo;
+        case 12: return B_Min;
+        case 13: return B_Copy;
+        case 14: return B_Mod;
+        case 15: return B_ReverseMod;
+        case 16: return B_GreaterThanOrEqual;
+        case 17: return B_Remainder;
+        case 18: return B_FMod;
+        case 19: return B_TruncateDiv;
+        case 20: return B_FloorDiv;
+        case 21: return B_FloorMod;
+        case 22: return B_SquaredSubtract;
+        case 23: return B_SafeDivide;
+        default: return B_Invalid;
+    }
+}
+
 __host__ __device__ constexpr int broadcastKind(int opNum) {
     switch (opNum) {
         case 0: return B_Add;

@@ -44,7 +44,11 @@ template <> __device__ __forceinline__ float16 fromCompute<float16>(float v) {
 // so a null pointer is fine for ops that take no parameters.
 template <typename T> struct Params {
     const T *p;
+    // the scalar operand of the scalar family, handed over by value (unused elsewhere)
+    typename Compute<T>::type scalar = 0;
     __device__ __forceinline__ typename Compute<T>::type operator[](int i) const { return toCompute(p[i]); }
+    // the scalar as the storage type holds it (the reference converts it to T before the loop)
+    __device__ __forceinline__ typename Compute<T>::type scalarValue() const { return toCompute(fromCompute<T>(scalar)); }
 };
 
 }  // namespace nd4j_amd

@@ -41,6 +41,11 @@ _EXEC_SIGNATURES = {
     "nd4j_execRandom{S}": ([_P, c_int, _P, _P, _P, _P], False),
     "nd4j_execRandom{S}XYZ": ([_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P], False),
     "nd4j_execRandom{S}XZ": ([_P, c_int, _P, _P, _P, _P, _P, _P], False),
+    # _SCALAR stands for the by-value scalar: float for Float and Half, double for Double
+    "nd4j_execScalar{S}Strided": ([_P, c_int, _P, c_ll, _P, c_ll, "_SCALAR", _P, c_ll], False),
+    "nd4j_execScalar{S}": ([_P, c_int, _P, _P, _P, _P, "_SCALAR", _P], False),
+    "nd4j_execScalar{S}Indexed": ([_P, c_int, _P, _P, _P, _P, "_SCALAR", _P, _P, _P], False),
+    "nd4j_execScalar{S}AlongDimension": ([_P, c_int, _P, _P, _P, _P, _P, _P, _P, c_int], False),
 }
 
 _PLAIN_SIGNATURES = {
@@ -129,7 +134,7 @@ def load_library(path=None):
     for template, (args, scalar) in _EXEC_SIGNATURES.items():
         for suffix, ret in _SUFFIX_RET.items():
             fn = getattr(lib, template.format(S=suffix))
-            fn.argtypes = args
+            fn.argtypes = [ret if a == "_SCALAR" else a for a in args]
             fn.restype = ret if scalar else None
     _lib = lib
     return lib
@@ -202,6 +207,18 @@ class NativeOps(object):
         return self._call("nd4j_execSummaryStats%sFull" % S, extra, opNum, x, xShapeInfo, extraParams, result,
                           resultShapeInfo, int(bool(rest[0])))
 
+    def _scalar(self, S, extra, opNum, x, a, result, b, c, d, *rest):
+        # strided: (x, xStride, result, resultStride, scalar, extraParams, n); shaped: (x, xInfo, result, resultInfo,
+        # scalar, extraParams); indexed: shaped + two index buffers; along a dimension: (x, xInfo, z, zInfo, scalars,
+        # extraParams, dimension, dimensionLength)
+        if len(rest) == 1:
+            return self._call("nd4j_execScalar%sStrided" % S, extra, opNum, x, a, result, b, c, d, rest[0])
+        if len(rest) == 0:
+            return self._call("nd4j_execScalar%s" % S, extra, opNum, x, a, result, b, c, d)
+        if isinstance(rest[1], int) and not isinstance(c, float):
+            return self._call("nd4j_execScalar%sAlongDimension" % S, extra, opNum, x, a, result, b, c, d, rest[0], rest[1])
+        return self._call("nd4j_execScalar%sIndexed" % S, extra, opNum, x, a, result, b, c, d, rest[0], rest[1])
+
     def _random(self, S, extra, opNum, state, *rest):
         if len(rest) == 3:
             return self._call("nd4j_execRandom%s" % S, extra, opNum, state, *rest)
@@ -221,6 +238,7 @@ def _install_overloads():
         setattr(NativeOps, "execReduce" + S, mk("_reduce"))
         setattr(NativeOps, "execSummaryStats" + S, mk("_stats"))
         setattr(NativeOps, "execRandom" + S, mk("_random"))
+        setattr(NativeOps, "execScalar" + S, mk("_scalar"))
 
 
 _install_overloads()

@@ -17,6 +17,7 @@ F32 = np.float32
 # opNums (reference: include/loops/legacy_ops.h)
 T_EXP, T_TANH = 3, 15
 P_ADD, P_MUL = 0, 6
+S_MUL = 2  # scalar family
 B_ADD, B_SUB, B_DIV = 0, 1, 3
 R_MEAN, R_SUM, R_MAX = 0, 1, 3
 I_MAX = 0
@@ -149,7 +150,7 @@ def pairwise_broadcast(dev, rows=65536, cols=1024, seed=7, dtype=F32, copies=Non
     bias = _uniform(rs, cols, -1, 1, dtype)
     xi, bi = harness.shape_info([rows, cols]), _vec(cols)
     ops, suf, sz = dev.ops, _suffix(dtype), dtype.itemsize
-    pw, bc = getattr(ops, "execPairwiseTransform" + suf), getattr(ops, "execBroadcast" + suf)
+    pw, bc, scl = getattr(ops, "execPairwiseTransform" + suf), getattr(ops, "execBroadcast" + suf), getattr(ops, "execScalar" + suf)
     tad = dev.tad(xi, [1])
     zc = np.zeros(n, dtype)
     tag = "" if dtype == F32 else "_" + dtype.name
@@ -166,12 +167,16 @@ def pairwise_broadcast(dev, rows=65536, cols=1024, seed=7, dtype=F32, copies=Non
         def gpu_bc():
             bc(ex_b, B_ADD, X.ptr, X.info_ptr, B.ptr, B.info_ptr, Z.ptr, Z.info_ptr, D.ptr, 1)
 
-        return [Case("pairwise_add" + tag, "pairwise", n, 3 * sz * n, mk_pw(P_ADD),
+        ex_s = dev.extra(xi, z_info=xi)
+        extra_cases = [Case("scalar_multiply" + tag, "scalar", n, 2 * sz * n,
+                            lambda: scl(ex_s, S_MUL, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, 1.5, None),
+                            lambda lib: (lib.scalar(S_MUL, x, xi, zc, xi, 1.5, None), zc)[1], True, Z.get)]
+        return extra_cases[:0] + [Case("pairwise_add" + tag, "pairwise", n, 3 * sz * n, mk_pw(P_ADD),
                      lambda lib: (lib.pairwise(P_ADD, x, xi, y, xi, zc, xi, None), zc)[1], True, Z.get),
                 Case("pairwise_multiply" + tag, "pairwise", n, 3 * sz * n, mk_pw(P_MUL),
                      lambda lib: (lib.pairwise(P_MUL, x, xi, y, xi, zc, xi, None), zc)[1], True, Z.get),
                 Case("broadcast_add_row" + tag, "broadcast", n, 2 * sz * n + sz * cols, gpu_bc,
-                     lambda lib: (lib.broadcast(B_ADD, x, xi, bias, bi, zc, xi, [1]), zc)[1], True, Z.get)]
+                     lambda lib: (lib.broadcast(B_ADD, x, xi, bias, bi, zc, xi, [1]), zc)[1], True, Z.get)] + extra_cases
 
     return _replicated(dev, "pairwise add+multiply, broadcast add row; %s [%d,%d] c-order" % (dtype.name, rows, cols),
                        3 * sz * n, dict(x=x, y=y, bias=bias, xi=xi, bi=bi, z_cpu=zc), device_set, copies)

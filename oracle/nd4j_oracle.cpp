@@ -357,6 +357,14 @@ static Bin broadcastBin(int op) {
                                   AMax, SquaredSubtract, FloorMod, FloorDiv, ReverseMod, SafeDivide, Mod, TruncateDiv};
     return (op >= 0 && op < 24) ? table[op] : Invalid;
 }
+// SCALAR_OPS: include/loops/legacy_ops.h:165-189
+static Bin scalarBin(int op) {
+    static const Bin table[24] = {Add, Subtract, Multiply, Divide, ReverseDivide, ReverseSubtract, Max, LessThan,
+                                  GreaterThan, EqualTo, LessThanOrEqual, NotEqualTo, Min, Copy, Mod, ReverseMod,
+                                  GreaterThanOrEqual, Remainder, FMod, TruncateDiv, FloorDiv, FloorMod, SquaredSubtract,
+                                  SafeDivide};
+    return (op >= 0 && op < 24) ? table[op] : Invalid;
+}
 template <typename T, bool three> static inline T binaryOp(Bin b, T d1, T d2, T *p) {
     switch (b) {
         case Add: return d1 + d2;
@@ -509,6 +517,55 @@ template <typename T> static void transformShaped(int op, T *x, Long *xi, T *z, 
         for (int d = 0; d < rank; d++) { ox += c[d] * xst[d]; oz += c[d] * zst[d]; }
         transformOp<T>(op, x[ox], extra, z[oz]);
     });
+}
+
+// scalar: include/loops/cpu/scalar.cpp.  Strided 218-285 (one thread: num_threads is pinned to 1 there), shaped
+// 121-215 (EWS pair of equal order -> strided, otherwise raw iteration over x's shape with both stride sets),
+// per-TAD scalars 14-62 (z is walked with the x TAD's element-wise stride, lines 22-23; TADs without an
+// element-wise stride only print a message).
+// The scalar is invariant in these loops and the reference's release flags include -freciprocal-math, so the
+// compiled reference divides by it as a multiplication by 1 / scalar (checked on 200000 random operands: Divide,
+// SafeDivide and FloorDiv agree with x * (1 / s) everywhere, with x / s only on 60 %).  Written out here so that
+// the result does not depend on what the optimiser makes of this file.
+template <typename T> static inline T scalarBinary(Bin b, T d1, T s, T *extra) {
+    if (b == Divide) return d1 * ((T)1.0f / s);
+    if (b == SafeDivide) return s == (T)0.0f ? (T)0.0f : d1 * ((T)1.0f / s);
+    if (b == FloorDiv) return m_floor(d1 * ((T)1.0f / s));
+    return binaryOp<T, true>(b, d1, s, extra);
+}
+template <typename T> static void scalarStrided(Bin b, T *x, Long xs, T *z, Long zs, T scalar, T *extra, Long n) {
+    for (Long i = 0; i < n; i++) z[i * zs] = scalarBinary<T>(b, x[i * xs], scalar, extra);
+}
+template <typename T> static void scalarShaped(int op, T *x, Long *xi, T *z, Long *zi, T scalar, T *extra) {
+    Bin b = scalarBin(op);
+    if (b == Invalid) { printf("[ERROR] Unknown opNum=%d (oracle scalar)\n", op); return; }
+    Long n = siNumel(xi);
+    Long xe = siEws(xi), ze = siEws(zi);
+    if (xe >= 1 && ze >= 1 && siOrder(xi) == siOrder(zi)) { scalarStrided<T>(b, x, xe, z, ze, scalar, extra, n); return; }
+    int rank = siRank(xi);
+    const Long *xst = siStride(xi), *zst = siStride(zi);
+    rawIter(rank, siShape(xi), [&](const Long *c) {
+        Long ox = 0, oz = 0;
+        for (int d = 0; d < rank; d++) { ox += c[d] * xst[d]; oz += c[d] * zst[d]; }
+        z[oz] = scalarBinary<T>(b, x[ox], scalar, extra);
+    });
+}
+template <typename T>
+static void scalarTad(int op, T *x, Long *xi, T *z, Long *zi, T *scalars, T *extra, int *dim, int dimLen) {
+    (void)zi;
+    Bin b = scalarBin(op);
+    if (b == Invalid) { printf("[ERROR] Unknown opNum=%d (oracle scalar)\n", op); return; }
+    TadPack tp;
+    computeTad(xi, dim, dimLen, tp, true);
+    const Long tadEws = siEws(tp.shapeInfo.data());
+    const Long tadLength = siNumel(tp.shapeInfo.data());
+    if (tadEws < 1) { printf("Super-bad loop visited. Shouldn't ever happen\n"); return; }
+#pragma omp parallel for schedule(guided) if (tp.numTads / gTadThreshold > 1)
+    for (Long r = 0; r < tp.numTads; r++) {
+        T *ox = x + tp.offsets[r], *oz = z + tp.offsets[r];
+        const T scalar = scalars[r];
+        for (Long f = 0; f < tadLength; f++) oz[f * tadEws] = scalarBinary<T>(b, ox[f * tadEws], scalar, extra);
+    }
 }
 
 // pairwise: include/loops/pairwise_transform.h:154-424
@@ -1196,6 +1253,19 @@ static void randomExec(int op, Rng *g, int operands, T *x, Long *xi, T *y, Long 
 using namespace oracle;
 
 #define ND4J_CPU_FAMILY(SUF, T)                                                                                \
+    void nd4j_cpu_scalar_##SUF(int op, void *x, Long *xSI, void *z, Long *zSI, double scalar, void *extra) {   \
+        scalarShaped<T>(op, (T *)x, xSI, (T *)z, zSI, sizeof(T) < 8 ? (T)(float)scalar : (T)scalar, (T *)extra); \
+    }                                                                                                          \
+    void nd4j_cpu_scalar_strided_##SUF(int op, void *x, Long xs, void *z, Long zs, double scalar, void *extra, \
+                                       Long n) {                                                               \
+        Bin b = scalarBin(op);                                                                                 \
+        if (b == Invalid) { printf("[ERROR] Unknown opNum=%d (oracle scalar)\n", op); return; }                \
+        scalarStrided<T>(b, (T *)x, xs, (T *)z, zs, sizeof(T) < 8 ? (T)(float)scalar : (T)scalar, (T *)extra, n); \
+    }                                                                                                          \
+    void nd4j_cpu_scalar_tad_##SUF(int op, void *x, Long *xSI, void *z, Long *zSI, void *scalars, void *extra, \
+                                   int *dim, int dimLen) {                                                     \
+        scalarTad<T>(op, (T *)x, xSI, (T *)z, zSI, (T *)scalars, (T *)extra, dim, dimLen);                     \
+    }                                                                                                          \
     void nd4j_cpu_transform_##SUF(int op, void *x, Long *xSI, void *z, Long *zSI, void *extra) {               \
         transformShaped<T>(op, (T *)x, xSI, (T *)z, zSI, (T *)extra);                                          \
     }                                                                                                          \

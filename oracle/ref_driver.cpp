@@ -25,6 +25,7 @@
 #include <loops/indexreduce.h>
 #include <loops/summarystatsreduce.h>
 #include <loops/random.h>
+#include <loops/scalar.h>
 
 using functions::transform::Transform;
 using functions::pairwise_transforms::PairWiseTransform;
@@ -33,6 +34,7 @@ using functions::reduce::ReduceFunction;
 using functions::indexreduce::IndexReduce;
 using functions::summarystats::SummaryStatsReduce;
 using functions::random::RandomFunction;
+using functions::scalar::ScalarTransform;
 
 namespace {
 
@@ -54,7 +56,32 @@ T reduceScalarWithPrepass(int opNum, T *x, Nd4jLong *xSI, T *extra) {
 
 }  // namespace
 
+// per-TAD scalars: the caller of ScalarTransform::transform supplies the TAD tables (blas/cpu/NativeOps.cpp:2453-2481)
+template <typename T>
+void scalarAlongDimension(int opNum, T *x, Nd4jLong *xSI, T *z, Nd4jLong *zSI, T *scalars, T *extra, int *dim, int dimLen) {
+    shape::TAD tad;
+    tad.init(xSI, dim, dimLen);
+    tad.createTadOnlyShapeInfo();
+    tad.createOffsets();
+    ScalarTransform<T>::transform(opNum, x, xSI, extra, z, zSI, scalars, dim, dimLen, tad.tadOnlyShapeInfo, tad.tadOffsets,
+                                  nullptr, nullptr);
+}
+
 #define ND4J_CPU_FAMILY(SUF, T)                                                                              \
+    void nd4j_cpu_scalar_##SUF(int op, void *x, Nd4jLong *xSI, void *z, Nd4jLong *zSI, double scalar,        \
+                               void *extra) {                                                                \
+        ScalarTransform<T>::transform(op, (T *)x, xSI, (T *)z, zSI, sizeof(T) < 8 ? (T)(float)scalar : (T)scalar, \
+                                      (T *)extra);                                                           \
+    }                                                                                                        \
+    void nd4j_cpu_scalar_strided_##SUF(int op, void *x, Nd4jLong xs, void *z, Nd4jLong zs, double scalar,    \
+                                       void *extra, Nd4jLong n) {                                            \
+        ScalarTransform<T>::transform(op, (T *)x, xs, (T *)z, zs, sizeof(T) < 8 ? (T)(float)scalar : (T)scalar, \
+                                      (T *)extra, n);                                                        \
+    }                                                                                                        \
+    void nd4j_cpu_scalar_tad_##SUF(int op, void *x, Nd4jLong *xSI, void *z, Nd4jLong *zSI, void *scalars,    \
+                                   void *extra, int *dim, int dimLen) {                                      \
+        scalarAlongDimension<T>(op, (T *)x, xSI, (T *)z, zSI, (T *)scalars, (T *)extra, dim, dimLen);        \
+    }                                                                                                        \
     void nd4j_cpu_transform_##SUF(int op, void *x, Nd4jLong *xSI, void *z, Nd4jLong *zSI, void *extra) {     \
         Transform<T>::exec(op, (T *)x, xSI, (T *)z, zSI, (T *)extra, nullptr, nullptr);                     \
     }                                                                                                        \

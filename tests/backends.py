@@ -52,6 +52,21 @@ class CpuBackend(object):
         self.lib.pairwise(op, x, x_info, y, y_info, z, z_info, extra)
         return z
 
+    def scalar(self, op, x, x_info, z_info, scalar, extra=None):
+        z = np.zeros(_span(z_info), x.dtype)
+        self.lib.scalar(op, x, x_info, z, z_info, scalar, extra)
+        return z
+
+    def scalar_strided(self, op, x, xs, zs, scalar, extra, n):
+        z = np.zeros(max(1, (n - 1) * zs + 1), x.dtype)
+        self.lib.scalar_strided(op, x, xs, z, zs, scalar, extra, n)
+        return z
+
+    def scalar_tad(self, op, x, x_info, scalars, extra, dims):
+        z = np.zeros(_span(x_info), x.dtype)
+        self.lib.scalar_tad(op, x, x_info, z, x_info, scalars, extra, dims)
+        return z
+
     def pairwise_strided(self, op, x, xs, y, ys, zs, extra, n):
         z = np.zeros(max(1, (n - 1) * zs + 1), x.dtype)
         self.lib.pairwise_strided(op, x, xs, y, ys, z, zs, extra, n)
@@ -217,6 +232,39 @@ class GpuBackend(object):
                                                                       X.info_ptr, Y.ptr, Y.info_ptr, Z.ptr, Z.info_ptr, e)
         out = Z.get()
         self._finish(X, Y, Z, E)
+        return out
+
+    def scalar(self, op, x, x_info, z_info, scalar, extra=None):
+        X = self._op(x, x_info)
+        Z = self._op(np.zeros(_span(z_info), x.dtype), z_info)
+        E, e = self._up(extra, x.dtype)
+        getattr(self.ops, "execScalar" + self._suffix(x))(self.dev.extra(x_info, z_info=z_info), op, X.ptr, X.info_ptr, Z.ptr,
+                                                           Z.info_ptr, float(scalar), e)
+        out = Z.get()
+        self._finish(X, Z, E)
+        return out
+
+    def scalar_strided(self, op, x, xs, zs, scalar, extra, n):
+        zsize = max(1, (n - 1) * zs + 1)
+        X, xp = self._up(x)
+        Z, zp = self._up(np.zeros(zsize, x.dtype))
+        E, e = self._up(extra, x.dtype)
+        getattr(self.ops, "execScalar" + self._suffix(x))(self.dev.extra(), op, xp, int(xs), zp, int(zs), float(scalar), e, int(n))
+        out = Z.download(x.dtype, zsize)
+        self._finish(X, Z, E)
+        return out
+
+    def scalar_tad(self, op, x, x_info, scalars, extra, dims, pass_tads=True):
+        X = self._op(x, x_info)
+        Z = self._op(np.zeros(_span(x_info), x.dtype), x_info)
+        S, sp = self._up(scalars, x.dtype)
+        E, e = self._up(extra, x.dtype)
+        D, d = self._up(np.array(list(dims), np.int32))
+        tad = self.dev.tad(x_info, dims) if pass_tads else None
+        getattr(self.ops, "execScalar" + self._suffix(x))(self.dev.extra(x_info, z_info=x_info, tad=tad, tad_z=tad), op, X.ptr,
+                                                           X.info_ptr, Z.ptr, Z.info_ptr, sp, e, d, len(dims))
+        out = Z.get()
+        self._finish(X, Z, S, E, D)
         return out
 
     def pairwise_strided(self, op, x, xs, y, ys, zs, extra, n):

@@ -13,7 +13,7 @@ import os
 
 import numpy as np
 
-from golden_inputs import (BROADCAST_OPS, INDEX_OPS, PAIRWISE_OPS, REDUCE_OPS, TRANSFORM_OPS, from_hexbits, op_extra,
+from golden_inputs import (BROADCAST_OPS, INDEX_OPS, PAIRWISE_OPS, REDUCE_OPS, SCALAR_OPS, SCALAR_VALUES, TRANSFORM_OPS, from_hexbits, op_extra,
                            pairwise_inputs, reduce_input, shape_info_np, transform_input, ulp_distance)
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -184,6 +184,12 @@ def check_op_vectors(be, max_ulp=ELEMENTWISE_ULP, exact_composites=False):
         run(lambda: assert_ulp(be.broadcast(op, a, bxi, b[:8].copy(), shape_info_np([1, 8]), bxi, [1]), want1, max_ulp, "broadcast op %d dim 1" % op), "broadcast %d/1" % op)
         want0 = from_hexbits(vec["broadcast_f32_12x8"][str(op)]["dim0"], f32)
         run(lambda: assert_ulp(be.broadcast(op, a, bxi, b[8:20].copy(), shape_info_np([12, 1]), bxi, [0]), want0, max_ulp, "broadcast op %d dim 0" % op), "broadcast %d/0" % op)
+    for op in SCALAR_OPS:
+        w = vec["scalar_f32"][str(op)]
+        for k, value in enumerate(SCALAR_VALUES):
+            run(lambda: assert_ulp(be.scalar(op, a, ai, ai, value), from_hexbits(w["value%d" % k], f32), max_ulp, "scalar op %d value %g" % (op, value)), "scalar %d" % op)
+        run(lambda: assert_ulp(be.scalar_tad(op, a, bxi, b[:12].copy(), None, [1]), from_hexbits(w["tad_dim1"], f32), max_ulp, "scalar op %d per row" % op), "scalar %d/1" % op)
+        run(lambda: assert_ulp(be.scalar_tad(op, a, bxi, b[:8].copy(), None, [0]), from_hexbits(w["tad_dim0"], f32), max_ulp, "scalar op %d per column" % op), "scalar %d/0" % op)
     m = reduce_input()
     mi = shape_info_np([12, 10])
     scale = float(np.abs(m).sum())

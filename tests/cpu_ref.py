@@ -60,6 +60,9 @@ class CpuLib(object):
         sigs = {
             "transform": [I, V, V, V, V, V],
             "transform_strided": [I, V, LL, V, LL, V, LL],
+            "scalar": [I, V, V, V, V, ctypes.c_double, V],
+            "scalar_strided": [I, V, LL, V, LL, ctypes.c_double, V, LL],
+            "scalar_tad": [I, V, V, V, V, V, V, V, I],
             "pairwise": [I, V, V, V, V, V, V, V],
             "pairwise_strided": [I, V, LL, V, LL, V, LL, V, LL],
             "broadcast": [I, V, V, V, V, V, V, V, I],
@@ -92,6 +95,17 @@ class CpuLib(object):
 
     def transform_strided(self, op, x, xs, z, zs, extra, n):
         self._fn("transform_strided", x)(op, _p(x), xs, _p(z), zs, _p(extra), n)
+
+    def scalar(self, op, x, x_info, z, z_info, scalar, extra=None):
+        self._fn("scalar", x)(op, _p(x), _p(_info(x_info)), _p(z), _p(_info(z_info)), float(scalar), _p(extra) if extra is not None else None)
+
+    def scalar_strided(self, op, x, xs, z, zs, scalar, extra, n):
+        self._fn("scalar_strided", x)(op, _p(x), xs, _p(z), zs, float(scalar), _p(extra) if extra is not None else None, n)
+
+    def scalar_tad(self, op, x, x_info, z, z_info, scalars, extra, dims):
+        d = _ints(dims)
+        self._fn("scalar_tad", x)(op, _p(x), _p(_info(x_info)), _p(z), _p(_info(z_info)), _p(scalars),
+                                  _p(extra) if extra is not None else None, _p(d), len(dims))
 
     def pairwise(self, op, x, x_info, y, y_info, z, z_info, extra=None):
         self._fn("pairwise", x)(op, _p(x), _p(_info(x_info)), _p(y), _p(_info(y_info)), _p(z), _p(_info(z_info)),

@@ -17,8 +17,8 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(HERE))
 import cpu_ref  # noqa: E402
-from golden_inputs import (BROADCAST_OPS, INDEX_OPS, PAIRWISE_OPS, REDUCE_OPS, TRANSFORM_OPS, hexbits, op_extra,  # noqa: E402
-                           pairwise_inputs, reduce_input, shape_info_np, transform_input)
+from golden_inputs import (BROADCAST_OPS, INDEX_OPS, PAIRWISE_OPS, REDUCE_OPS, SCALAR_OPS, SCALAR_VALUES, TRANSFORM_OPS,  # noqa: E402
+                           hexbits, op_extra, pairwise_inputs, reduce_input, shape_info_np, transform_input)
 
 
 def main():
@@ -156,6 +156,23 @@ def main():
         ref.broadcast(op, a, bxi, col, shape_info_np([12, 1]), z0, bxi, [0])
         bc[str(op)] = {"dim1": hexbits(z), "dim0": hexbits(z0)}
     ops["broadcast_f32_12x8"] = bc
+    # scalar family: the first pairwise vector against a by-value scalar, and as a 12 x 8 matrix against one
+    # scalar per TAD (rows: the first 12 values of the second vector; columns: its first 8)
+    sc = {}
+    for op in SCALAR_OPS:
+        entry = {}
+        for k, value in enumerate(SCALAR_VALUES):
+            z = np.zeros_like(a)
+            ref.scalar(op, a, ai, z, ai, value, None)
+            entry["value%d" % k] = hexbits(z)
+        z = np.zeros_like(a)
+        ref.scalar_tad(op, a, bxi, z, bxi, b[:12].copy(), None, [1])
+        entry["tad_dim1"] = hexbits(z)
+        z = np.zeros_like(a)
+        ref.scalar_tad(op, a, bxi, z, bxi, b[:8].copy(), None, [0])
+        entry["tad_dim0"] = hexbits(z)
+        sc[str(op)] = entry
+    ops["scalar_f32"] = sc
     m = reduce_input()  # [12, 10]
     mi = shape_info_np([12, 10])
     rd = {}

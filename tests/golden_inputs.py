@@ -7,6 +7,8 @@ import numpy as np
 TRANSFORM_OPS = [o for o in range(0, 97) if o not in (36, 37, 38, 39, 40, 41, 43, 44, 48, 56, 57, 58, 60, 69, 70, 71)]
 PAIRWISE_OPS = list(range(0, 29)) + [45, 46, 56, 57, 58, 59, 60, 69, 92, 93, 94]
 BROADCAST_OPS = list(range(0, 24))
+SCALAR_OPS = list(range(0, 24))
+SCALAR_VALUES = [1.7, -2.25]
 REDUCE_OPS = [0, 1] + list(range(3, 27))
 INDEX_OPS = list(range(0, 6))
 RANDOM_PLAIN_OPS = [0, 1, 2, 3, 4, 7, 12, 13]

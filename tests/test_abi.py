@@ -14,10 +14,11 @@ def _declared_c_names():
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     text = text.replace("\\\n", " ")
     names = set(re.findall(r"\b(nd4j_(?:amd_)?[A-Za-z0-9]+)\s*\(", text))
-    macro = re.search(r"#define ND4J_C_EXEC\(SUFFIX, T, R\)(.*?)\n\s*\n", text, flags=re.S).group(1)
-    for templ in re.findall(r"\b(nd4j_[A-Za-z0-9#]+)\s*\(", macro):
-        for suffix in ("Float", "Half", "Double"):
-            names.add(templ.replace("##SUFFIX##", suffix).replace("##SUFFIX", suffix))
+    for macro_name in ("ND4J_C_EXEC", "ND4J_C_SCALAR"):
+        macro = re.search(r"#define %s\(SUFFIX, T, [RS]\)(.*?)\n\s*\n" % macro_name, text, flags=re.S).group(1)
+        for templ in re.findall(r"\b(nd4j_[A-Za-z0-9#]+)\s*\(", macro):
+            for suffix in ("Float", "Half", "Double"):
+                names.add(templ.replace("##SUFFIX##", suffix).replace("##SUFFIX", suffix))
     return {n for n in names if "#" not in n}
 
 
@@ -35,6 +36,7 @@ def test_cpp_class_members_are_exported():
     for member in ("execTransformFloat", "execTransformHalf", "execPairwiseTransformFloat", "execBroadcastFloat",
                    "execReduceFloat", "execReduceScalarFloat", "execIndexReduceFloat", "execIndexReduceScalarFloat",
                    "execSummaryStatsFloat", "execSummaryStatsScalarFloat", "execRandomFloat", "execRandomHalf",
+                   "execScalarFloat", "execScalarHalf", "execScalarDouble",
                    "initRandom", "refreshBuffer", "reSeedBuffer", "destroyRandom", "tadOnlyShapeInfo", "mallocDevice",
                    "createStream", "memcpyAsync", "streamSynchronize"):
         assert "NativeOps::%s(" % member in out, member

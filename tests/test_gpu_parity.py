@@ -239,6 +239,51 @@ def test_broadcast_on_views_all_ops(gpu, cpu):
             assert ulp_distance(g, c).max() <= 2, (shape, order, dims, op)
 
 
+def test_scalar_family(gpu, cpu):
+    from golden_inputs import SCALAR_OPS
+    rs = np.random.RandomState(32)
+    n = 20000
+    x = (rs.uniform(1.2, 50, n) * rs.choice([-1, 1], n)).astype(np.float32)
+    xi = shape_info_np([1, n])
+    for s in (1.7, -2.25):
+        multiples = (np.arange(1, n + 1).astype(np.float32) * np.float32(s)).astype(np.float32)
+        for op in SCALAR_OPS:
+            assert ulp_distance(gpu.scalar(op, x, xi, xi, s), cpu.scalar(op, x, xi, xi, s)).max() <= 2, (op, s)
+            assert ulp_distance(gpu.scalar(op, multiples, xi, xi, s), cpu.scalar(op, multiples, xi, xi, s)).max() <= 2, (op, s)
+    for op in (0, 3, 20, 23):
+        assert np.array_equal(gpu.scalar_strided(op, x, 3, 2, 1.7, None, n // 3), cpu.scalar_strided(op, x, 3, 2, 1.7, None, n // 3))
+        assert np.array_equal(gpu.scalar_strided(op, x, 1, 1, 1.7, None, n), cpu.scalar_strided(op, x, 1, 1, 1.7, None, n))
+    # views: dense f -> c, strided, permuted
+    for vx in VIEWS:
+        xv, xinfo = _mk(vx, rs)
+        for op in (0, 3, 4, 13):
+            assert np.array_equal(gpu.scalar(op, xv, xinfo, xinfo, 0.37), cpu.scalar(op, xv, xinfo, xinfo, 0.37)), (vx[0], op)
+    fi, ci = harness.shape_info([100, 200], "f"), harness.shape_info([100, 200], "c")
+    assert np.array_equal(gpu.scalar(1, x, fi, ci, 0.37), cpu.scalar(1, x, fi, ci, 0.37))
+    # one scalar per TAD: contiguous rows, strided columns, both orders, with and without the caller's TAD tables
+    for rows, cols in ((300, 150), (64, 1024), (5, 7)):
+        m = rs.uniform(1.2, 9, rows * cols).astype(np.float32)
+        for order in ("c", "f"):
+            mi = harness.shape_info([rows, cols], order)
+            for dims, count in (([1], rows), ([0], cols)):
+                sc = rs.uniform(1.2, 5, count).astype(np.float32)
+                for op in (0, 2, 3, 6, 14, 20, 23):
+                    want = cpu.scalar_tad(op, m, mi, sc, None, dims)
+                    assert np.array_equal(gpu.scalar_tad(op, m, mi, sc, None, dims), want), (rows, cols, order, dims, op)
+                assert np.array_equal(gpu.scalar_tad(0, m, mi, sc, None, dims, pass_tads=False), cpu.scalar_tad(0, m, mi, sc, None, dims))
+    # fp16: the scalar is rounded to fp16 before use; fp64
+    xh = rs.uniform(1, 4, 4096).astype(np.float16)
+    hi = shape_info_np([1, 4096])
+    g, c = gpu.scalar(2, xh, hi, hi, 1.2345678), cpu.scalar(2, xh, hi, hi, 1.2345678)
+    assert np.all(np.abs(g.astype(np.float64) - c.astype(np.float64)) <= 1e-2 * np.abs(c.astype(np.float64)))
+    assert np.array_equal(gpu.scalar(13, xh, hi, hi, 1.2345678), np.full(4096, np.float16(1.2345678)))
+    xd = rs.randn(1000)
+    di = shape_info_np([1, 1000])
+    assert np.allclose(gpu.scalar(3, xd, di, di, 1.7), cpu.scalar(3, xd, di, di, 1.7), rtol=1e-15, atol=0)
+    # unknown opNum: output untouched
+    assert np.all(gpu.scalar(99, x, xi, xi, 1.0) == 0)
+
+
 def test_nan_and_special_values(gpu, cpu):
     x = np.array([np.nan, 1.0, -np.inf, np.inf, 0.0, -0.0, 3.0, np.nan, 2.0, -1e38, 1e38, 5.0], np.float32)
     xi = shape_info_np([1, x.size])

@@ -102,6 +102,35 @@ def test_matches_compiled_reference_on_views(oracle, reference_lib):
         assert np.isclose(float(oracle.summarystats_scalar(1, 1, x, xi)), float(ref.summarystats_scalar(1, 1, x, xi)), rtol=1e-6)
 
 
+def test_scalar_family_matches_compiled_reference(oracle, reference_lib):
+    # by-value scalar on views, quotients that land on integers (where x / s and x * (1 / s) floor differently),
+    # strided calls and one scalar per TAD along either dimension
+    ref = backends.CpuBackend(reference_lib)
+    rs = np.random.RandomState(31)
+    n = 50000
+    x = (rs.uniform(1.2, 50, n) * rs.choice([-1, 1], n)).astype(np.float32)
+    xi = shape_info_np([1, n])
+    from golden_inputs import SCALAR_OPS
+    for s in (1.7, -2.25, 3.3):
+        multiples = (np.arange(1, n + 1).astype(np.float32) * np.float32(s)).astype(np.float32)
+        for op in SCALAR_OPS:
+            assert ulp_distance(oracle.scalar(op, x, xi, xi, s), ref.scalar(op, x, xi, xi, s)).max() == 0, (op, s)
+            assert ulp_distance(oracle.scalar(op, multiples, xi, xi, s), ref.scalar(op, multiples, xi, xi, s)).max() == 0, (op, s)
+    for op in (0, 3, 20, 23):
+        assert np.array_equal(oracle.scalar_strided(op, x, 3, 2, 1.7, None, n // 3), ref.scalar_strided(op, x, 3, 2, 1.7, None, n // 3))
+    m = x[:300 * 150].copy()
+    for order in ("c", "f"):
+        mi = shape_info_np([300, 150], order)
+        for dims, count in (([1], 300), ([0], 150)):
+            sc = rs.uniform(1.2, 5, count).astype(np.float32)
+            for op in (0, 2, 3, 6, 14, 20, 23):
+                assert np.array_equal(oracle.scalar_tad(op, m, mi, sc, None, dims), ref.scalar_tad(op, m, mi, sc, None, dims)), (order, dims, op)
+    fi = shape_info_np([200, 250], "f")
+    ci = shape_info_np([200, 250], "c")
+    for op in (1, 3, 5):
+        assert np.array_equal(oracle.scalar(op, x, fi, ci, 0.37), ref.scalar(op, x, fi, ci, 0.37)), op
+
+
 def test_broadcast_matches_compiled_reference(oracle, reference_lib):
     ref = backends.CpuBackend(reference_lib)
     rs = np.random.RandomState(12)
