@@ -1,7 +1,7 @@
 """Parity of the HIP path, driven through the C ABI of libnd4j_amd.so, against the CPU checkers.
 
 Sizes: the vector / fixture replays are tiny; the seeded comparisons use shapes the CPU checker finishes in
-seconds; BASELINE-size runs are in test_gpu_configs.py.  Tolerances are those of tests/checks.py.
+seconds; the benchmark-size runs are in test_gpu_configs.py.  Tolerances are those of tests/checks.py.
 """
 import itertools
 
