@@ -220,7 +220,7 @@ def main():
         fam = []
         builders = [workloads.transform_tanh, lambda d: workloads.pairwise_broadcast(d, copies=2),
                     lambda d: workloads.pairwise_broadcast(d, dtype="float16"),
-                    workloads.reductions, workloads.stats_softmax, workloads.random_fills]
+                    workloads.reductions, workloads.reduce3_pairs, workloads.stats_softmax, workloads.random_fills]
         for build in builders:
             wl = build(dev)
             for c in wl.cases:

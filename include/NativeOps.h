@@ -100,8 +100,30 @@
                             Nd4jLong *zShapeInfo, T *scalars, T *extraParams, int *dimension,                    \
                             int dimensionLength);
 
+// Reduce3 family (two inputs, one number per pair of runs), reference: blas/NativeOps.h:919-1044 (Float / Half),
+// 252-362 (Double and the all-pairs variant): whole arrays into result[0], whole arrays returned by value,
+// along `dimension`, and every TAD of x against every TAD of y.
+#define ND4J_REDUCE3_MEMBERS(SUFFIX, T, R)                                                                      \
+    void execReduce3##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,                 \
+                             T *extraParamsVals, T *y, Nd4jLong *yShapeInfo, T *result,                          \
+                             Nd4jLong *resultShapeInfo);                                                         \
+    R execReduce3Scalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,              \
+                                T *extraParamsVals, T *y, Nd4jLong *yShapeInfo);                                 \
+    void execReduce3##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,                 \
+                             T *extraParamsVals, T *y, Nd4jLong *yShapeInfo, T *result,                          \
+                             Nd4jLong *resultShapeInfoBuffer, int *dimension, int dimensionLength);              \
+    void execReduce3All##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xInfo,                   \
+                                T *extraParamsVals, T *y, Nd4jLong *yInfo, T *result,                            \
+                                Nd4jLong *resultShapeInfoBuffer, int *dimension, int dimensionLength,            \
+                                Nd4jLong *xTadShapeInfo, Nd4jLong *xOffsets, Nd4jLong *yTadShapeInfo,            \
+                                Nd4jLong *yOffsets);
+
 class ND4J_EXPORT NativeOps {
 public:
+    ND4J_REDUCE3_MEMBERS(Float, float, float)
+    ND4J_REDUCE3_MEMBERS(Half, float16, float)
+    ND4J_REDUCE3_MEMBERS(Double, double, double)
+
     ND4J_SCALAR_MEMBERS(Float, float, float)
     ND4J_SCALAR_MEMBERS(Half, float16, float)
     ND4J_SCALAR_MEMBERS(Double, double, double)
@@ -163,3 +185,4 @@ public:
 
 #undef ND4J_EXEC_MEMBERS
 #undef ND4J_SCALAR_MEMBERS
+#undef ND4J_REDUCE3_MEMBERS

@@ -107,6 +107,27 @@ ND4J_C_SCALAR(Half, float16, float)
 ND4J_C_SCALAR(Double, double, double)
 #undef ND4J_C_SCALAR
 
+/* Reduce3 family (blas/NativeOps.h:919-1044, 252-362): whole arrays into result[0] (Full), returned by value
+ * (Scalar), along `dimension`, and all pairs of TADs (All). */
+#define ND4J_C_REDUCE3(SUFFIX, T, R)                                                                             \
+    void nd4j_execReduce3##SUFFIX##Full(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,       \
+                                        T *extraParamsVals, T *y, Nd4jLong *yShapeInfo, T *result,                \
+                                        Nd4jLong *resultShapeInfo);                                               \
+    R nd4j_execReduce3Scalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,          \
+                                     T *extraParamsVals, T *y, Nd4jLong *yShapeInfo);                             \
+    void nd4j_execReduce3##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,             \
+                                  T *extraParamsVals, T *y, Nd4jLong *yShapeInfo, T *result,                      \
+                                  Nd4jLong *resultShapeInfoBuffer, int *dimension, int dimensionLength);          \
+    void nd4j_execReduce3All##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xInfo,               \
+                                     T *extraParamsVals, T *y, Nd4jLong *yInfo, T *result,                        \
+                                     Nd4jLong *resultShapeInfoBuffer, int *dimension, int dimensionLength,        \
+                                     Nd4jLong *xTadShapeInfo, Nd4jLong *xOffsets, Nd4jLong *yTadShapeInfo,        \
+                                     Nd4jLong *yOffsets);
+ND4J_C_REDUCE3(Float, float, float)
+ND4J_C_REDUCE3(Half, float16, float)
+ND4J_C_REDUCE3(Double, double, double)
+#undef ND4J_C_REDUCE3
+
 Nd4jPointer nd4j_initRandom(Nd4jPointer *extraPointers, long seed, long bufferSize, Nd4jPointer ptrToBuffer);
 void nd4j_refreshBuffer(Nd4jPointer *extraPointers, long seed, Nd4jPointer ptrRandom);
 void nd4j_reSeedBuffer(Nd4jPointer *extraPointers, long seed, Nd4jPointer ptrRandom);

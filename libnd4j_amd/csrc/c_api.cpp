@@ -127,6 +127,28 @@ ND4J_C_SCALAR(Half, float16, float)
 ND4J_C_SCALAR(Double, double, double)
 #undef ND4J_C_SCALAR
 
+#define ND4J_C_REDUCE3(SUFFIX, T, R)                                                                               \
+    void nd4j_execReduce3##SUFFIX##Full(Nd4jPointer *e, int op, T *x, Nd4jLong *xs, T *p, T *y, Nd4jLong *ys, T *r, \
+                                        Nd4jLong *rs) {                                                             \
+        guardVoid([&] { gOps.execReduce3##SUFFIX(e, op, x, xs, p, y, ys, r, rs); });                                \
+    }                                                                                                              \
+    R nd4j_execReduce3Scalar##SUFFIX(Nd4jPointer *e, int op, T *x, Nd4jLong *xs, T *p, T *y, Nd4jLong *ys) {        \
+        return guardRet<R>((R)0, [&] { return gOps.execReduce3Scalar##SUFFIX(e, op, x, xs, p, y, ys); });           \
+    }                                                                                                              \
+    void nd4j_execReduce3##SUFFIX(Nd4jPointer *e, int op, T *x, Nd4jLong *xs, T *p, T *y, Nd4jLong *ys, T *r,       \
+                                  Nd4jLong *rs, int *dim, int dl) {                                                 \
+        guardVoid([&] { gOps.execReduce3##SUFFIX(e, op, x, xs, p, y, ys, r, rs, dim, dl); });                       \
+    }                                                                                                              \
+    void nd4j_execReduce3All##SUFFIX(Nd4jPointer *e, int op, T *x, Nd4jLong *xs, T *p, T *y, Nd4jLong *ys, T *r,    \
+                                     Nd4jLong *rs, int *dim, int dl, Nd4jLong *xt, Nd4jLong *xo, Nd4jLong *yt,      \
+                                     Nd4jLong *yo) {                                                                \
+        guardVoid([&] { gOps.execReduce3All##SUFFIX(e, op, x, xs, p, y, ys, r, rs, dim, dl, xt, xo, yt, yo); });    \
+    }
+ND4J_C_REDUCE3(Float, float, float)
+ND4J_C_REDUCE3(Half, float16, float)
+ND4J_C_REDUCE3(Double, double, double)
+#undef ND4J_C_REDUCE3
+
 Nd4jPointer nd4j_initRandom(Nd4jPointer *e, long seed, long size, Nd4jPointer buf) {
     return guardRet<Nd4jPointer>(nullptr, [&] { return gOps.initRandom(e, seed, size, buf); });
 }

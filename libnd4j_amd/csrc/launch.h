@@ -97,6 +97,20 @@ template <typename T>
 bool launchSummaryStatsScalar(hipStream_t stream, int opNum, bool biasCorrected, const T *x, T *z,
                               const FlatPlan &plan, Workspace ws);
 
+// ---- reduce3 ---------------------------------------------------------------------------------------
+// numOut results; result r pairs the run of x at xOffsets[r / xDiv] with the run of y at yOffsets[r % yMod]
+// (a null table: offset 0); element f of a run sits at map(xm, f) / map(ym, f) behind the run's offset.
+struct Reduce3Launch {
+    Long runLength, numOut;
+    Long xDiv, yMod;
+    const Long *xOffsets;  // device
+    const Long *yOffsets;  // device
+    DimMap xm, ym;         // rank >= 1
+};
+template <typename T>
+bool launchReduce3(hipStream_t stream, int opNum, const T *x, const T *y, T *z, const T *extra, const Reduce3Launch &in,
+                   Workspace ws);
+
 // ---- random ----------------------------------------------------------------------------------------
 // Device image of the generator state that getElement() needs (reference: helper_generator.h:61-74,
 // 185-220).  Passed by value, so one op sees one consistent state.

@@ -5,6 +5,7 @@
 //   index-reduce   include/loops/cpu/indexreduce.cpp:36-129, 131-228
 //   summary stats  include/loops/cpu/summarystatsreduce.cpp:24-196
 // extraPointers decoding follows blas/cuda/NativeOps.cu:2098-2139 and 1600-1643.
+#include <cstdio>
 #include <cstring>
 
 #include "../../include/NativeOps.h"
@@ -279,6 +280,167 @@ void statsDims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, Long *zIn
 
 }  // namespace
 
+// ---- reduce3 (include/loops/reduce3.h) -------------------------------------------------------------------
+// Index -> offset map of one operand walked by its own linear index in C order ('c') or Fortran order.
+void orderedLinearMap(const Long *shape, const Long *stride, int rank, char order, DimMap &out) {
+    if (order != 'f') {
+        ownCanon(rank, shape, stride, out);
+    } else {
+        Long rs[kMaxRank], rt[kMaxRank];
+        for (int i = 0; i < rank; i++) { rs[i] = shape[rank - 1 - i]; rt[i] = stride[rank - 1 - i]; }
+        ownCanon(rank, rs, rt, out);
+    }
+    if (out.rank < 1) { out.rank = 1; out.shape[0] = 1; out.stride[0] = 1; }
+}
+
+// Whole arrays (reduce3.h:838-916): pairs are formed by linear index - memory-linear i * ews when both arrays
+// have an element-wise stride and the same order, C-order logical index otherwise.
+void reduce3WholePlan(const Long *hx, const Long *hy, Reduce3Launch &in) {
+    in.runLength = siNumel(hx);
+    in.numOut = 1;
+    in.xDiv = in.yMod = 1;
+    in.xOffsets = in.yOffsets = nullptr;
+    const Long xe = siEws(hx), ye = siEws(hy);
+    if (siOrder(hx) == siOrder(hy) && xe >= 1 && ye >= 1) {
+        in.xm.rank = in.ym.rank = 1;
+        in.xm.shape[0] = in.ym.shape[0] = (unsigned)(in.runLength > 0xffffffffLL ? 0xffffffffu : in.runLength);
+        in.xm.stride[0] = xe;
+        in.ym.stride[0] = ye;
+    } else {
+        orderedLinearMap(siShape(hx), siStride(hx), siRank(hx), 'c', in.xm);
+        orderedLinearMap(siShape(hy), siStride(hy), siRank(hy), 'c', in.ym);
+    }
+}
+
+template <typename T>
+bool reduce3WholeTo(Nd4jPointer *extra, hipStream_t s, int opNum, T *x, Long *xInfo, T *params, T *y, Long *yInfo, T *zDev) {
+    std::vector<Long> sx, sy;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    const Long *hy = hostShapeInfo(extra, X_HOST_Y_SHAPE, yInfo, sy, s);
+    if (hx == nullptr || hy == nullptr) return true;
+    Reduce3Launch in;
+    reduce3WholePlan(hx, hy, in);
+    Scratch sc = scratchFor(s);
+    if (!launchReduce3<T>(s, opNum, x, y, zDev, params, in, sc.rest)) { reportUnknownOp("reduce3", opNum); return false; }
+    return true;
+}
+
+template <typename T>
+typename ScalarOut<T>::R reduce3Scalar(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *y, Long *yInfo) {
+    hipStream_t s = streamOf(extra);
+    T *slot = reinterpret_cast<T *>(pinnedScalarFor(s));
+    if (!reduce3WholeTo<T>(extra, s, opNum, x, xInfo, params, y, yInfo, slot)) return 0;
+    return readScalar<T>(slot, s, "execReduce3Scalar");
+}
+
+template <typename T>
+void reduce3Full(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *y, Long *yInfo, T *z) {
+    hipStream_t s = streamOf(extra);
+    if (!reduce3WholeTo<T>(extra, s, opNum, x, xInfo, params, y, yInfo, z)) return;
+    checkLaunch("execReduce3", s);
+}
+
+// Along `dimension` (reduce3.h:998-1081 with a caller's TAD tables, 1083-1346 without): result r is the pair
+// (TAD r of x, TAD r of y) when the arrays are equally long, (TAD r of x, all of y) when y holds one TAD's
+// worth of elements.  Elements pair up by their linear index inside the TAD in the TAD's own order.
+template <typename T>
+void reduce3Dims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *y, Long *yInfo, T *z, Long *zInfo,
+                 int *dimension, int dimLen) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx, sy, sz;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    const Long *hy = hostShapeInfo(extra, X_HOST_Y_SHAPE, yInfo, sy, s);
+    const Long *hz = hostShapeInfo(extra, X_HOST_Z_SHAPE, zInfo, sz, s);
+    if (hx == nullptr || hy == nullptr || hz == nullptr) return;
+    if (siIsScalar(hz) || dimension == nullptr || dimLen >= siRank(hx)) {
+        reduce3Full<T>(extra, opNum, x, xInfo, params, y, yInfo, z);
+        return;
+    }
+    ResolvedTad tx;
+    if (!resolveTad(extra, X_HOST_TAD_SHAPE, X_DEV_TAD_OFFSETS, hx, dimension, dimLen, tx, s)) return;
+    Reduce3Launch in;
+    in.runLength = tx.tadLength;
+    in.numOut = tx.numTads;
+    in.xDiv = 1;
+    in.yMod = tx.numTads > 0 ? tx.numTads : 1;
+    in.xOffsets = tx.devOffsets;
+    const char order = siOrder(tx.hostInfo) == 'f' ? 'f' : 'c';
+    orderedLinearMap(siShape(tx.hostInfo), siStride(tx.hostInfo), siRank(tx.hostInfo), order, in.xm);
+    if (siNumel(hy) == siNumel(hx)) {
+        ResolvedTad ty;
+        if (!resolveTad(nullptr, 0, 0, hy, dimension, dimLen, ty, s)) return;
+        in.yOffsets = ty.devOffsets;
+        orderedLinearMap(siShape(ty.hostInfo), siStride(ty.hostInfo), siRank(ty.hostInfo), order, in.ym);
+    } else if (siNumel(hy) == tx.tadLength) {
+        in.yOffsets = nullptr;
+        orderedLinearMap(siShape(hy), siStride(hy), siRank(hy), order, in.ym);
+    } else {
+        std::printf("reduce3: y holds %lld elements, neither the %lld of x nor the %lld of one TAD\n", (long long)siNumel(hy),
+                    (long long)siNumel(hx), (long long)tx.tadLength);
+        return;
+    }
+    Scratch sc = scratchFor(s);
+    if (!launchReduce3<T>(s, opNum, x, y, z, params, in, sc.rest)) { reportUnknownOp("reduce3", opNum); return; }
+    checkLaunch("execReduce3", s);
+}
+
+// Every TAD of x against every TAD of y (reduce3.h:918-995): result[r * yTads + g].
+template <typename T>
+void reduce3All(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *y, Long *yInfo, T *z, int *dimension,
+                int dimLen) {
+    hipStream_t s = streamOf(extra);
+    std::vector<Long> sx, sy;
+    const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
+    const Long *hy = hostShapeInfo(extra, X_HOST_Y_SHAPE, yInfo, sy, s);
+    if (hx == nullptr || hy == nullptr) return;
+    ResolvedTad tx, ty;
+    if (!resolveTad(nullptr, 0, 0, hx, dimension, dimLen, tx, s)) return;
+    if (!resolveTad(nullptr, 0, 0, hy, dimension, dimLen, ty, s)) return;
+    if (tx.tadLength != ty.tadLength) {
+        std::printf("reduce3All: TAD lengths differ (%lld vs %lld)\n", (long long)tx.tadLength, (long long)ty.tadLength);
+        return;
+    }
+    Reduce3Launch in;
+    in.runLength = tx.tadLength;
+    in.numOut = tx.numTads * ty.numTads;
+    in.xDiv = ty.numTads > 0 ? ty.numTads : 1;
+    in.yMod = in.xDiv;
+    in.xOffsets = tx.devOffsets;
+    in.yOffsets = ty.devOffsets;
+    orderedLinearMap(siShape(tx.hostInfo), siStride(tx.hostInfo), siRank(tx.hostInfo), siOrder(tx.hostInfo) == 'f' ? 'f' : 'c', in.xm);
+    orderedLinearMap(siShape(ty.hostInfo), siStride(ty.hostInfo), siRank(ty.hostInfo), siOrder(ty.hostInfo) == 'f' ? 'f' : 'c', in.ym);
+    Scratch sc = scratchFor(s);
+    if (!launchReduce3<T>(s, opNum, x, y, z, params, in, sc.rest)) { reportUnknownOp("reduce3", opNum); return; }
+    checkLaunch("execReduce3All", s);
+}
+
+#define ND4J_REDUCE3_MEMBERS(SUFFIX, T, R)                                                                          \
+    void NativeOps::execReduce3##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,          \
+                                        T *extraParamsVals, T *y, Nd4jLong *yShapeInfo, T *result,                  \
+                                        Nd4jLong *resultShapeInfo) {                                                \
+        (void)resultShapeInfo;                                                                                      \
+        reduce3Full<T>(extraPointers, opNum, x, xShapeInfo, extraParamsVals, y, yShapeInfo, result);                \
+    }                                                                                                               \
+    R NativeOps::execReduce3Scalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,       \
+                                           T *extraParamsVals, T *y, Nd4jLong *yShapeInfo) {                        \
+        return reduce3Scalar<T>(extraPointers, opNum, x, xShapeInfo, extraParamsVals, y, yShapeInfo);               \
+    }                                                                                                               \
+    void NativeOps::execReduce3##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,          \
+                                        T *extraParamsVals, T *y, Nd4jLong *yShapeInfo, T *result,                  \
+                                        Nd4jLong *resultShapeInfoBuffer, int *dimension, int dimensionLength) {     \
+        reduce3Dims<T>(extraPointers, opNum, x, xShapeInfo, extraParamsVals, y, yShapeInfo, result,                 \
+                       resultShapeInfoBuffer, dimension, dimensionLength);                                          \
+    }                                                                                                               \
+    void NativeOps::execReduce3All##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xInfo,            \
+                                           T *extraParamsVals, T *y, Nd4jLong *yInfo, T *result,                    \
+                                           Nd4jLong *resultShapeInfoBuffer, int *dimension, int dimensionLength,    \
+                                           Nd4jLong *xTadShapeInfo, Nd4jLong *xOffsets, Nd4jLong *yTadShapeInfo,    \
+                                           Nd4jLong *yOffsets) {                                                    \
+        (void)resultShapeInfoBuffer; (void)xTadShapeInfo; (void)xOffsets; (void)yTadShapeInfo; (void)yOffsets;      \
+        reduce3All<T>(extraPointers, opNum, x, xInfo, extraParamsVals, y, yInfo, result, dimension,                 \
+                      dimensionLength);                                                                             \
+    }
+
 #define ND4J_REDUCE_MEMBERS(SUFFIX, T, R)                                                                            \
     R NativeOps::execReduceScalar##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,         \
                                           T *extraParams) {                                                          \
@@ -320,3 +482,6 @@ void statsDims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, Long *zIn
 ND4J_REDUCE_MEMBERS(Float, float, float)
 ND4J_REDUCE_MEMBERS(Half, float16, float)
 ND4J_REDUCE_MEMBERS(Double, double, double)
+ND4J_REDUCE3_MEMBERS(Float, float, float)
+ND4J_REDUCE3_MEMBERS(Half, float16, float)
+ND4J_REDUCE3_MEMBERS(Double, double, double)

@@ -1,0 +1,217 @@
+// Reduce3 family: one number per pair of equally long runs of x and y (distances, dot, cosine ...).
+// Reference: include/loops/reduce3.h:838-916 (whole arrays), 998-1081 and 1083-1346 (per TAD), 918-995 (all
+// pairs of TADs); functors include/ops/ops.h:2567-2990; opNum table include/loops/legacy_ops.h:183-191.
+//
+// Every functor is a sum of up to three per-pair terms - the reduction value and the two running values the
+// reference keeps in extraParams[0..1] - followed by a closed-form postProcess, so the accumulator is a triple
+// and partial triples merge by addition.
+//
+// One kernel serves all entry points: output r pairs the run of x that starts at xOffsets[r / xDiv] with the
+// run of y that starts at yOffsets[r % yMod] (null tables mean offset 0); element f of a run sits at
+// map(xm, f) / map(ym, f).  A whole-array call is a single output whose run is cut into slices that a second
+// kernel merges.
+#include "elementwise.cuh"
+#include "launch.h"
+#include "reduce_engine.cuh"
+
+namespace nd4j_amd {
+
+template <typename C> struct Acc3 { C r, e0, e1; };
+
+template <typename C, int OP> struct Reduce3Op {
+    static __device__ __forceinline__ void accumulate(Acc3<C> &a, C d1, C d2, C eps) {
+        switch (OP) {
+            case 0: a.r += m::abs_(d1 - d2); break;                                   // ManhattanDistance
+            case 1: { C d = d1 - d2; a.r += d * d; break; }                           // EuclideanDistance
+            case 2: a.e0 += d1 * d1; a.e1 += d2 * d2; a.r += d1 * d2; break;          // CosineSimilarity
+            case 3: a.r += d1 * d2; break;                                            // Dot
+            case 4: {                                                                 // EqualsWithEps
+                C diff = m::abs_(d1 - d2);
+                C v = (C)1;
+                if (diff <= eps) v = (C)0;
+                else if (diff <= m::max_(m::abs_(d1), m::abs_(d2)) * eps) v = (C)0;
+                a.r += v;
+                break;
+            }
+            case 5: a.e0 += m::abs_(d1) * m::abs_(d1); a.e1 += m::abs_(d2) * m::abs_(d2); a.r += d1 * d2; break;  // CosineDistance
+            case 6: a.e0 += m::min_(d1, d2); a.e1 += m::max_(d1, d2); break;          // JaccardDistance
+            default: a.r += (d1 == d2) ? (C)0 : (C)1; break;                          // SimpleHammingDistance
+        }
+    }
+    static __device__ __forceinline__ C finalize(const Acc3<C> &a, Long n) {
+        switch (OP) {
+            case 1: return m::sqrt_(a.r);
+            case 2: return a.r / (m::sqrt_(a.e0) * m::sqrt_(a.e1));
+            case 5: return (C)1 - (a.r / (m::sqrt_(a.e0) * m::sqrt_(a.e1)));
+            case 6: return (C)1 - (a.e0 / a.e1);
+            case 7: return a.r / (C)n;
+            default: return a.r;
+        }
+    }
+};
+
+template <typename C> __device__ __forceinline__ Acc3<C> add3(Acc3<C> a, Acc3<C> b) {
+    a.r += b.r; a.e0 += b.e0; a.e1 += b.e1;
+    return a;
+}
+// shape of the merge helpers in reduce_engine.cuh
+template <typename C> struct Acc3Merge {
+    typedef Acc3<C> Acc;
+    __device__ __forceinline__ Acc combine(Acc a, Acc b) const { return add3(a, b); }
+};
+
+struct Reduce3Plan {
+    Long runLength;        // pairs per output
+    Long numOut;
+    Long xDiv, yMod;       // output r -> x run r / xDiv, y run r % yMod
+    const Long *xOffsets;  // device; null: 0
+    const Long *yOffsets;  // device; null: 0
+    DimMap xm, ym;         // pair index inside a run -> element offset
+    bool contiguous;       // both maps are unit-stride
+};
+
+// GROUP lanes per output (16, 64 or the whole block).  `slices` > 1 (whole-array calls): blockIdx.x is the slice
+// of the single run and the block's triple goes to partials[blockIdx.x].
+template <typename T, int OP, int GROUP>
+__global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, T *z, const T *extra, Reduce3Plan pl,
+                                                        Acc3<typename Compute<T>::type> *partials, Long sliceLength) {
+    typedef typename Compute<T>::type C;
+    typedef Acc3<C> Acc;
+    constexpr int GROUPS = kBlock / GROUP;
+    constexpr int VEC = Pack<T>::N;
+    __shared__ Acc smem[kBlock / kWave];
+    const C eps = extra != nullptr ? toCompute(extra[0]) : (C)0;
+    const int g = threadIdx.x / GROUP, lane = threadIdx.x % GROUP;
+    const bool sliced = partials != nullptr;
+    const Long units = sliced ? (Long)gridDim.x : pl.numOut;
+    for (Long u0 = (Long)blockIdx.x * GROUPS; u0 < units; u0 += (Long)gridDim.x * GROUPS) {
+        const Long u = u0 + g;
+        const bool live = u < units;
+        Acc acc;
+        acc.r = acc.e0 = acc.e1 = (C)0;
+        if (live) {
+            const Long r = sliced ? 0 : u;
+            const Long f0 = sliced ? u * sliceLength : 0;
+            Long f1 = sliced ? f0 + sliceLength : pl.runLength;
+            if (f1 > pl.runLength) f1 = pl.runLength;
+            const T *xr = x + (pl.xOffsets != nullptr ? pl.xOffsets[r / pl.xDiv] : 0);
+            const T *yr = y + (pl.yOffsets != nullptr ? pl.yOffsets[r % pl.yMod] : 0);
+            const bool vec = pl.contiguous && ((reinterpret_cast<uintptr_t>(xr + f0) | reinterpret_cast<uintptr_t>(yr + f0)) & 15) == 0;
+            if (vec) {
+                const Long nvec = (f1 - f0) / VEC;
+                const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(xr + f0);
+                const Pack<T> *yv = reinterpret_cast<const Pack<T> *>(yr + f0);
+                Long v = lane;
+                for (; v + GROUP < nvec; v += 2 * GROUP) {
+                    Pack<T> a0 = loadPack(xv + v), b0 = loadPack(yv + v), a1 = loadPack(xv + v + GROUP), b1 = loadPack(yv + v + GROUP);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) Reduce3Op<C, OP>::accumulate(acc, toCompute(a0.v[e]), toCompute(b0.v[e]), eps);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) Reduce3Op<C, OP>::accumulate(acc, toCompute(a1.v[e]), toCompute(b1.v[e]), eps);
+                }
+                for (; v < nvec; v += GROUP) {
+                    Pack<T> a0 = loadPack(xv + v), b0 = loadPack(yv + v);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) Reduce3Op<C, OP>::accumulate(acc, toCompute(a0.v[e]), toCompute(b0.v[e]), eps);
+                }
+                for (Long f = f0 + nvec * VEC + lane; f < f1; f += GROUP)
+                    Reduce3Op<C, OP>::accumulate(acc, toCompute(xr[f]), toCompute(yr[f]), eps);
+            } else if (pl.contiguous) {
+                for (Long f = f0 + lane; f < f1; f += GROUP)
+                    Reduce3Op<C, OP>::accumulate(acc, toCompute(xr[f]), toCompute(yr[f]), eps);
+            } else {
+                for (Long f = f0 + lane; f < f1; f += GROUP)
+                    Reduce3Op<C, OP>::accumulate(acc, toCompute(xr[mapOffset64(pl.xm, (unsigned long long)f)]),
+                                                 toCompute(yr[mapOffset64(pl.ym, (unsigned long long)f)]), eps);
+            }
+        }
+        Acc3Merge<C> mg;
+        if (GROUP == kBlock) {
+            acc = blockMerge<Acc3Merge<C>>(mg, acc, smem);
+        } else {
+            if (live) acc = waveMerge<Acc3Merge<C>, GROUP>(mg, acc);
+        }
+        if (live && lane == 0) {
+            if (sliced) partials[u] = acc;
+            else z[u] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, pl.runLength));
+        }
+    }
+}
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(kBlock) reduce3Finish(T *z, const Acc3<typename Compute<T>::type> *partials, int count,
+                                                        Long runLength) {
+    typedef typename Compute<T>::type C;
+    typedef Acc3<C> Acc;
+    __shared__ Acc smem[kBlock / kWave];
+    Acc acc;
+    acc.r = acc.e0 = acc.e1 = (C)0;
+    for (int i = threadIdx.x; i < count; i += kBlock) acc = add3(acc, partials[i]);
+    Acc3Merge<C> mg;
+    acc = blockMerge<Acc3Merge<C>>(mg, acc, smem);
+    if (threadIdx.x == 0) z[0] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, runLength));
+}
+
+template <typename T> struct Reduce3Body {
+    template <int OP> struct Run {
+        static bool run(hipStream_t s, const T *x, const T *y, T *z, const T *extra, const Reduce3Plan &pl, Workspace ws) {
+            typedef Acc3<typename Compute<T>::type> Acc;
+            if (pl.numOut <= 0) return true;
+            if (pl.numOut == 1 && pl.runLength >= 4 * kBlock) {
+                Long perBlock = (Long)kBlock * 8 * Pack<T>::N;
+                Long slices = (pl.runLength + perBlock - 1) / perBlock;
+                if (slices > 2048) slices = 2048;
+                if ((size_t)slices * sizeof(Acc) > ws.bytes) slices = (Long)(ws.bytes / sizeof(Acc));
+                if (slices < 1) slices = 1;
+                // slices start on 16-byte boundaries whenever the run does
+                Long sliceLength = (pl.runLength + slices - 1) / slices;
+                sliceLength = (sliceLength + 63) / 64 * 64;
+                slices = (pl.runLength + sliceLength - 1) / sliceLength;
+                Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+                hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)slices), dim3(kBlock), 0, s, x, y, z, extra, pl,
+                                   partials, sliceLength);
+                hipLaunchKernelGGL((reduce3Finish<T, OP>), dim3(1), dim3(kBlock), 0, s, z, partials, (int)slices, pl.runLength);
+                return true;
+            }
+            Acc *none = nullptr;
+            if (pl.runLength >= 4096) {
+                int grid = gridFor(pl.numOut, 1, kGridCap);
+                hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0);
+            } else if (pl.runLength >= 128) {
+                int grid = gridFor(pl.numOut, kBlock / 64, kGridCap);
+                hipLaunchKernelGGL((reduce3Kernel<T, OP, 64>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0);
+            } else {
+                int grid = gridFor(pl.numOut, kBlock / 16, kGridCap);
+                hipLaunchKernelGGL((reduce3Kernel<T, OP, 16>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0);
+            }
+            return true;
+        }
+    };
+};
+
+template <typename T>
+bool launchReduce3(hipStream_t s, int opNum, const T *x, const T *y, T *z, const T *extra, const Reduce3Launch &in,
+                   Workspace ws) {
+    Reduce3Plan pl;
+    pl.runLength = in.runLength;
+    pl.numOut = in.numOut;
+    pl.xDiv = in.xDiv < 1 ? 1 : in.xDiv;
+    pl.yMod = in.yMod < 1 ? 1 : in.yMod;
+    pl.xOffsets = in.xOffsets;
+    pl.yOffsets = in.yOffsets;
+    pl.xm = in.xm;
+    pl.ym = in.ym;
+    pl.contiguous = in.xm.rank <= 1 && in.ym.rank <= 1 && (in.xm.rank == 0 || in.xm.stride[0] == 1) &&
+                    (in.ym.rank == 0 || in.ym.stride[0] == 1);
+    return dispatchSeq<Reduce3Body<T>::template Run>(opNum, std::make_integer_sequence<int, 8>{}, s, x, y, z, extra, pl, ws);
+}
+
+#define INST(T)                                                                                                  \
+    template bool launchReduce3<T>(hipStream_t, int, const T *, const T *, T *, const T *, const Reduce3Launch &, \
+                                   Workspace);
+INST(float)
+INST(float16)
+INST(double)
+#undef INST
+
+}  // namespace nd4j_amd

@@ -41,6 +41,10 @@ _EXEC_SIGNATURES = {
     "nd4j_execRandom{S}": ([_P, c_int, _P, _P, _P, _P], False),
     "nd4j_execRandom{S}XYZ": ([_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P], False),
     "nd4j_execRandom{S}XZ": ([_P, c_int, _P, _P, _P, _P, _P, _P], False),
+    "nd4j_execReduce3{S}Full": ([_P, c_int, _P, _P, _P, _P, _P, _P, _P], False),
+    "nd4j_execReduce3Scalar{S}": ([_P, c_int, _P, _P, _P, _P, _P], True),
+    "nd4j_execReduce3{S}": ([_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P, c_int], False),
+    "nd4j_execReduce3All{S}": ([_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P, c_int, _P, _P, _P, _P], False),
     # _SCALAR stands for the by-value scalar: float for Float and Half, double for Double
     "nd4j_execScalar{S}Strided": ([_P, c_int, _P, c_ll, _P, c_ll, "_SCALAR", _P, c_ll], False),
     "nd4j_execScalar{S}": ([_P, c_int, _P, _P, _P, _P, "_SCALAR", _P], False),
@@ -219,6 +223,11 @@ class NativeOps(object):
             return self._call("nd4j_execScalar%sAlongDimension" % S, extra, opNum, x, a, result, b, c, d, rest[0], rest[1])
         return self._call("nd4j_execScalar%sIndexed" % S, extra, opNum, x, a, result, b, c, d, rest[0], rest[1])
 
+    def _reduce3(self, S, extra, opNum, x, xInfo, params, y, yInfo, result, resultInfo, *rest):
+        if len(rest) == 2:
+            return self._call("nd4j_execReduce3%s" % S, extra, opNum, x, xInfo, params, y, yInfo, result, resultInfo, *rest)
+        return self._call("nd4j_execReduce3%sFull" % S, extra, opNum, x, xInfo, params, y, yInfo, result, resultInfo)
+
     def _random(self, S, extra, opNum, state, *rest):
         if len(rest) == 3:
             return self._call("nd4j_execRandom%s" % S, extra, opNum, state, *rest)
@@ -239,6 +248,7 @@ def _install_overloads():
         setattr(NativeOps, "execSummaryStats" + S, mk("_stats"))
         setattr(NativeOps, "execRandom" + S, mk("_random"))
         setattr(NativeOps, "execScalar" + S, mk("_scalar"))
+        setattr(NativeOps, "execReduce3" + S, mk("_reduce3"))
 
 
 _install_overloads()

@@ -232,6 +232,46 @@ def reductions(dev, rows=16384, cols=4096, seed=11, copies=None):
                        4 * n, dict(x=x, xi=xi), device_set, copies)
 
 
+# ---- reduce3 family on the configs[2] shape: dot over everything, Euclidean and cosine per row ----------
+def reduce3_pairs(dev, rows=16384, cols=4096, seed=12, copies=None):
+    n = rows * cols
+    rs = np.random.default_rng(seed)
+    x, y = _normal(rs, n, F32), _normal(rs, n, F32)
+    xi = harness.shape_info([rows, cols])
+    zi = _vec(rows)
+    ops = dev.ops
+    tad = dev.tad(xi, [1])
+    zc = np.zeros(rows, F32)
+
+    def device_set(w):
+        X, Y = w.operand(x, xi), w.operand(y, xi)
+        Z = w.operand(np.zeros(rows, F32), zi)
+        D = w.raw(np.array([1], np.int32))
+        ex = dev.extra(xi, xi, zi, tad=tad)
+        ex_s = dev.extra(xi, xi)
+        out = {}
+        cases = []
+        for op, opname in ((1, "euclidean"), (2, "cosine")):
+            def gpu(op=op):
+                ops.execReduce3Float(ex, op, X.ptr, X.info_ptr, None, Y.ptr, Y.info_ptr, Z.ptr, Z.info_ptr, D.ptr, 1)
+
+            def cpu(lib, op=op):
+                lib.reduce3(op, x, xi, y, xi, zc, zi, [1], None)
+                return zc
+
+            cases.append(Case("%s_dim1" % opname, "reduce3", n, 8 * n + 4 * rows, gpu, cpu, True, Z.get))
+
+        def gpu_dot():
+            out["dot"] = ops.execReduce3ScalarFloat(ex_s, 3, X.ptr, X.info_ptr, None, Y.ptr, Y.info_ptr)
+
+        cases.append(Case("dot_full", "reduce3", n, 8 * n + 4, gpu_dot, lambda lib: lib.reduce3_scalar(3, x, xi, y, xi, None), True,
+                          lambda: np.array([out["dot"]], F32)))
+        return cases
+
+    return _replicated(dev, "reduce3 euclidean/cosine per row + dot; fp32 [%d,%d] c-order" % (rows, cols), 8 * n,
+                       dict(x=x, y=y, xi=xi), device_set, copies)
+
+
 # ---- configs[3]: summary statistics and a softmax-style chain on an f-order matrix ---------------------
 def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
     n = rows * cols
@@ -359,4 +399,4 @@ def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data
     return w
 
 
-BUILDERS = [transform_tanh, pairwise_broadcast, reductions, stats_softmax, random_fills]
+BUILDERS = [transform_tanh, pairwise_broadcast, reductions, reduce3_pairs, stats_softmax, random_fills]

@@ -568,6 +568,120 @@ static void scalarTad(int op, T *x, Long *xi, T *z, Long *zi, T *scalars, T *ext
     }
 }
 
+// reduce3: include/loops/reduce3.h.  Functors ops.h:2567-2990: the reduction value plus the two running values
+// the reference keeps in extraParams[0..1]; EqualsWithEps reads its epsilon from extraParams[2], which
+// execScalar fills from the caller's extraParams[0] (reduce3.h:854-858).
+template <typename T> struct R3 { T r, e0, e1; };
+template <typename T> static inline void r3Op(int op, R3<T> &a, T d1, T d2, T eps) {
+    switch (op) {
+        case 0: a.r = a.r + m_abs(d1 - d2); break;
+        case 1: { T d = d1 - d2; a.r = d * d + a.r; break; }
+        case 2: a.e0 += d1 * d1; a.e1 += d2 * d2; a.r = a.r + d1 * d2; break;
+        case 3: a.r = d1 * d2 + a.r; break;
+        case 4: {
+            T diff = m_abs(d1 - d2);
+            T v = (T)1.0f;
+            if (diff <= eps) v = (T)0.0f;
+            else if (diff <= m_max(m_abs(d1), m_abs(d2)) * eps) v = (T)0.0f;
+            a.r = v + a.r;
+            break;
+        }
+        case 5: a.e0 += m_abs(d1) * m_abs(d1); a.e1 += m_abs(d2) * m_abs(d2); a.r = a.r + d1 * d2; break;
+        case 6: a.e0 += m_min(d1, d2); a.e1 += m_max(d1, d2); break;
+        default: a.r = a.r + ((d1 == d2) ? (T)0.0f : (T)1.0f); break;
+    }
+}
+template <typename T> static inline T r3Post(int op, const R3<T> &a, Long n) {
+    switch (op) {
+        case 1: return m_sqrt(a.r);
+        case 2: return a.r / (m_sqrt(a.e0) * m_sqrt(a.e1));
+        case 5: return (T)1.0f - (a.r / (m_sqrt(a.e0) * m_sqrt(a.e1)));
+        case 6: return (T)1.0f - (a.e0 / a.e1);
+        case 7: return (T)(a.r / (T)(float)n);
+        default: return a.r;
+    }
+}
+// whole arrays (reduce3.h:838-916): memory-linear pairing when both arrays have an element-wise stride and the
+// same order, C-order logical pairing otherwise; one sequential pass
+template <typename T> static T reduce3Scalar(int op, T *x, Long *xi, T *extra, T *y, Long *yi) {
+    if (op < 0 || op > 7) { printf("[ERROR] Unknown opNum=%d (oracle reduce3)\n", op); return (T)0.0f; }
+    const T eps = extra != nullptr ? extra[0] : (T)0.0f;
+    const Long n = siNumel(xi);
+    const Long xe = siEws(xi), ye = siEws(yi);
+    R3<T> a;
+    a.r = a.e0 = a.e1 = (T)0.0f;
+    if (siOrder(xi) == siOrder(yi) && xe >= 1 && ye >= 1) {
+        for (Long i = 0; i < n; i++) r3Op<T>(op, a, x[i * xe], y[i * ye], eps);
+    } else {
+        Long cx[kMaxRank], cy[kMaxRank];
+        for (Long i = 0; i < n; i++) {
+            ind2subC(siRank(xi), siShape(xi), (int)i, cx);
+            ind2subC(siRank(yi), siShape(yi), (int)i, cy);
+            r3Op<T>(op, a, x[getOffset(0, siShape(xi), siStride(xi), cx, siRank(xi))],
+                    y[getOffset(0, siShape(yi), siStride(yi), cy, siRank(yi))], eps);
+        }
+    }
+    return r3Post<T>(op, a, n);
+}
+// one run of `n` pairs: element f of each operand is found from its linear index in the given order
+template <typename T>
+static T reduce3Run(int op, T *x, const Long *xInfo, T *y, const Long *yInfo, char order, Long n, T eps) {
+    R3<T> a;
+    a.r = a.e0 = a.e1 = (T)0.0f;
+    Long cx[kMaxRank], cy[kMaxRank];
+    for (Long f = 0; f < n; f++) {
+        if (order == 'f') { ind2subF(siRank(xInfo), siShape(xInfo), (int)f, cx); ind2subF(siRank(yInfo), siShape(yInfo), (int)f, cy); }
+        else { ind2subC(siRank(xInfo), siShape(xInfo), (int)f, cx); ind2subC(siRank(yInfo), siShape(yInfo), (int)f, cy); }
+        r3Op<T>(op, a, x[getOffset(0, siShape(xInfo), siStride(xInfo), cx, siRank(xInfo))],
+                y[getOffset(0, siShape(yInfo), siStride(yInfo), cy, siRank(yInfo))], eps);
+    }
+    return r3Post<T>(op, a, n);
+}
+// along `dimension` (reduce3.h:998-1081, 1083-1346): TAD r of x against TAD r of y (equally long arrays) or against
+// all of y (y as long as one TAD); pairs by linear index inside the TAD, in the x TAD's order
+template <typename T>
+static void reduce3Dims(int op, T *x, Long *xi, T *extra, T *y, Long *yi, T *z, Long *zi, int *dim, int dimLen) {
+    if (op < 0 || op > 7) { printf("[ERROR] Unknown opNum=%d (oracle reduce3)\n", op); return; }
+    if (siIsScalar(zi)) { z[0] = reduce3Scalar<T>(op, x, xi, extra, y, yi); return; }
+    const T eps = extra != nullptr ? extra[0] : (T)0.0f;
+    TadPack tx;
+    computeTad(xi, dim, dimLen, tx, true);
+    const Long n = siNumel(tx.shapeInfo.data());
+    const char order = siOrder(tx.shapeInfo.data()) == 'f' ? 'f' : 'c';
+    if (siNumel(yi) == siNumel(xi)) {
+        TadPack ty;
+        computeTad(yi, dim, dimLen, ty, true);
+        for (Long r = 0; r < tx.numTads; r++)
+            z[r] = reduce3Run<T>(op, x + tx.offsets[r], tx.shapeInfo.data(), y + ty.offsets[r], ty.shapeInfo.data(), order, n, eps);
+    } else {
+        for (Long r = 0; r < tx.numTads; r++) z[r] = reduce3Run<T>(op, x + tx.offsets[r], tx.shapeInfo.data(), y, yi, order, n, eps);
+    }
+}
+// every TAD of x against every TAD of y (reduce3.h:918-995)
+template <typename T>
+static void reduce3All(int op, T *x, Long *xi, T *extra, T *y, Long *yi, T *z, int *dim, int dimLen) {
+    if (op < 0 || op > 7) { printf("[ERROR] Unknown opNum=%d (oracle reduce3)\n", op); return; }
+    const T eps = extra != nullptr ? extra[0] : (T)0.0f;
+    TadPack tx, ty;
+    computeTad(xi, dim, dimLen, tx, true);
+    computeTad(yi, dim, dimLen, ty, true);
+    const Long n = siNumel(tx.shapeInfo.data());
+    for (Long r = 0; r < tx.numTads; r++)
+        for (Long g = 0; g < ty.numTads; g++) {
+            R3<T> a;
+            a.r = a.e0 = a.e1 = (T)0.0f;
+            Long cx[kMaxRank], cy[kMaxRank];
+            const Long *xt = tx.shapeInfo.data(), *yt = ty.shapeInfo.data();
+            for (Long f = 0; f < n; f++) {
+                if (siOrder(yt) == 'c') ind2subC(siRank(yt), siShape(yt), (int)f, cy); else ind2subF(siRank(yt), siShape(yt), (int)f, cy);
+                if (siOrder(xt) == 'c') ind2subC(siRank(xt), siShape(xt), (int)f, cx); else ind2subF(siRank(xt), siShape(xt), (int)f, cx);
+                r3Op<T>(op, a, x[tx.offsets[r] + getOffset(0, siShape(xt), siStride(xt), cx, siRank(xt))],
+                        y[ty.offsets[g] + getOffset(0, siShape(yt), siStride(yt), cy, siRank(yt))], eps);
+            }
+            z[r * ty.numTads + g] = r3Post<T>(op, a, n);
+        }
+}
+
 // pairwise: include/loops/pairwise_transform.h:154-424
 template <typename T> static void pairwiseStrided(Bin b, T *x, Long xs, T *y, Long ys, T *z, Long zs, T *extra, Long n) {
     int threads = clampThreads(n, gElementThreshold);
@@ -1253,6 +1367,22 @@ static void randomExec(int op, Rng *g, int operands, T *x, Long *xi, T *y, Long 
 using namespace oracle;
 
 #define ND4J_CPU_FAMILY(SUF, T)                                                                                \
+    void nd4j_cpu_reduce3_scalar_##SUF(int op, void *x, Long *xSI, void *extra, void *y, Long *ySI, void *out) { \
+        *(T *)out = reduce3Scalar<T>(op, (T *)x, xSI, (T *)extra, (T *)y, ySI);                                \
+    }                                                                                                          \
+    void nd4j_cpu_reduce3_##SUF(int op, void *x, Long *xSI, void *extra, void *y, Long *ySI, void *z,          \
+                                Long *zSI, int *dim, int dimLen) {                                             \
+        reduce3Dims<T>(op, (T *)x, xSI, (T *)extra, (T *)y, ySI, (T *)z, zSI, dim, dimLen);                    \
+    }                                                                                                          \
+    void nd4j_cpu_reduce3_tad_##SUF(int op, void *x, Long *xSI, void *extra, void *y, Long *ySI, void *z,      \
+                                    Long *zSI, int *dim, int dimLen) {                                         \
+        reduce3Dims<T>(op, (T *)x, xSI, (T *)extra, (T *)y, ySI, (T *)z, zSI, dim, dimLen);                    \
+    }                                                                                                          \
+    void nd4j_cpu_reduce3_all_##SUF(int op, void *x, Long *xSI, void *extra, void *y, Long *ySI, void *z,      \
+                                    Long *zSI, int *dim, int dimLen) {                                         \
+        (void)zSI;                                                                                             \
+        reduce3All<T>(op, (T *)x, xSI, (T *)extra, (T *)y, ySI, (T *)z, dim, dimLen);                          \
+    }                                                                                                          \
     void nd4j_cpu_scalar_##SUF(int op, void *x, Long *xSI, void *z, Long *zSI, double scalar, void *extra) {   \
         scalarShaped<T>(op, (T *)x, xSI, (T *)z, zSI, sizeof(T) < 8 ? (T)(float)scalar : (T)scalar, (T *)extra); \
     }                                                                                                          \

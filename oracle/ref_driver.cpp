@@ -25,6 +25,7 @@
 #include <loops/indexreduce.h>
 #include <loops/summarystatsreduce.h>
 #include <loops/random.h>
+#include <loops/reduce3.h>
 #include <loops/scalar.h>
 
 using functions::transform::Transform;
@@ -35,6 +36,7 @@ using functions::indexreduce::IndexReduce;
 using functions::summarystats::SummaryStatsReduce;
 using functions::random::RandomFunction;
 using functions::scalar::ScalarTransform;
+using functions::reduce3::Reduce3;
 
 namespace {
 
@@ -67,7 +69,46 @@ void scalarAlongDimension(int opNum, T *x, Nd4jLong *xSI, T *z, Nd4jLong *zSI, T
                                   nullptr, nullptr);
 }
 
+// reduce3 with the caller's TAD tables ("going tad-way", blas/cpu/NativeOps.cpp:1100-1108) and all pairs of TADs
+// (1144-1161): the tables are built here with the reference's own shape::TAD
+template <typename T>
+void reduce3TadWay(int opNum, T *x, Nd4jLong *xSI, T *extra, T *y, Nd4jLong *ySI, T *z, Nd4jLong *zSI, int *dim, int dimLen) {
+    shape::TAD tad;
+    tad.init(xSI, dim, dimLen);
+    tad.createTadOnlyShapeInfo();
+    tad.createOffsets();
+    Reduce3<T>::exec(opNum, x, xSI, extra, y, ySI, z, zSI, dim, dimLen, tad.tadOnlyShapeInfo, tad.tadOffsets);
+}
+template <typename T>
+void reduce3AllPairs(int opNum, T *x, Nd4jLong *xSI, T *extra, T *y, Nd4jLong *ySI, T *z, Nd4jLong *zSI, int *dim, int dimLen) {
+    shape::TAD tx, ty;
+    tx.init(xSI, dim, dimLen);
+    tx.createTadOnlyShapeInfo();
+    tx.createOffsets();
+    ty.init(ySI, dim, dimLen);
+    ty.createTadOnlyShapeInfo();
+    ty.createOffsets();
+    Reduce3<T>::execAll(opNum, x, xSI, extra, y, ySI, z, zSI, dim, dimLen, tx.tadOnlyShapeInfo, tx.tadOffsets,
+                        ty.tadOnlyShapeInfo, ty.tadOffsets);
+}
+
 #define ND4J_CPU_FAMILY(SUF, T)                                                                              \
+    void nd4j_cpu_reduce3_scalar_##SUF(int op, void *x, Nd4jLong *xSI, void *extra, void *y, Nd4jLong *ySI,  \
+                                       void *out) {                                                          \
+        *(T *)out = Reduce3<T>::execScalar(op, (T *)x, xSI, (T *)extra, (T *)y, ySI);                       \
+    }                                                                                                        \
+    void nd4j_cpu_reduce3_##SUF(int op, void *x, Nd4jLong *xSI, void *extra, void *y, Nd4jLong *ySI,         \
+                                void *z, Nd4jLong *zSI, int *dim, int dimLen) {                              \
+        Reduce3<T>::exec(op, (T *)x, xSI, (T *)extra, (T *)y, ySI, (T *)z, zSI, dim, dimLen);               \
+    }                                                                                                        \
+    void nd4j_cpu_reduce3_tad_##SUF(int op, void *x, Nd4jLong *xSI, void *extra, void *y, Nd4jLong *ySI,     \
+                                    void *z, Nd4jLong *zSI, int *dim, int dimLen) {                          \
+        reduce3TadWay<T>(op, (T *)x, xSI, (T *)extra, (T *)y, ySI, (T *)z, zSI, dim, dimLen);               \
+    }                                                                                                        \
+    void nd4j_cpu_reduce3_all_##SUF(int op, void *x, Nd4jLong *xSI, void *extra, void *y, Nd4jLong *ySI,     \
+                                    void *z, Nd4jLong *zSI, int *dim, int dimLen) {                          \
+        reduce3AllPairs<T>(op, (T *)x, xSI, (T *)extra, (T *)y, ySI, (T *)z, zSI, dim, dimLen);             \
+    }                                                                                                        \
     void nd4j_cpu_scalar_##SUF(int op, void *x, Nd4jLong *xSI, void *z, Nd4jLong *zSI, double scalar,        \
                                void *extra) {                                                                \
         ScalarTransform<T>::transform(op, (T *)x, xSI, (T *)z, zSI, sizeof(T) < 8 ? (T)(float)scalar : (T)scalar, \

@@ -90,6 +90,22 @@ class CpuBackend(object):
         self.lib.indexreduce(op, x, x_info, extra, z, _vec_info(out_len), dims)
         return z
 
+    def reduce3_scalar(self, op, x, x_info, y, y_info, extra=None):
+        return self.lib.reduce3_scalar(op, x, x_info, y, y_info, extra)
+
+    def reduce3(self, op, x, x_info, y, y_info, extra, dims, out_len, tad_way=False):
+        """tad_way: the reference's variant that is handed the x TAD tables (its only defined one when y is a
+        single TAD); the other checkers treat both alike"""
+        z = np.zeros(out_len, x.dtype)
+        fn = self.lib.reduce3_tad if tad_way else self.lib.reduce3
+        fn(op, x, x_info, y, y_info, z, _vec_info(out_len), dims, extra)
+        return z
+
+    def reduce3_all(self, op, x, x_info, y, y_info, extra, dims, out_len):
+        z = np.zeros(out_len, x.dtype)
+        self.lib.reduce3_all(op, x, x_info, y, y_info, z, _vec_info(out_len), dims, extra)
+        return z
+
     def indexreduce_scalar(self, op, x, x_info, extra=None):
         return self.lib.indexreduce_scalar(op, x, x_info, extra)
 
@@ -308,6 +324,39 @@ class GpuBackend(object):
 
     def reduce(self, op, x, x_info, extra, dims, out_len, pass_tads=True):
         return self._reduce_like("execReduce", op, x, x_info, extra, dims, out_len, pass_tads=pass_tads)
+
+    def reduce3_scalar(self, op, x, x_info, y, y_info, extra=None):
+        X, Y = self._op(x, x_info), self._op(y, y_info)
+        E, e = self._up(extra, x.dtype)
+        r = getattr(self.ops, "execReduce3Scalar" + self._suffix(x))(self.dev.extra(x_info, y_info), op, X.ptr, X.info_ptr, e,
+                                                                    Y.ptr, Y.info_ptr)
+        self._finish(X, Y, E)
+        return x.dtype.type(r)
+
+    def reduce3(self, op, x, x_info, y, y_info, extra, dims, out_len, tad_way=False, pass_tads=True):
+        X, Y = self._op(x, x_info), self._op(y, y_info)
+        zi = _vec_info(out_len)
+        Z = self._op(np.zeros(out_len, x.dtype), zi)
+        E, e = self._up(extra, x.dtype)
+        D, d = self._up(np.array(list(dims), np.int32))
+        tad = self.dev.tad(x_info, dims) if (pass_tads and len(dims) < int(x_info[0])) else None
+        getattr(self.ops, "execReduce3" + self._suffix(x))(self.dev.extra(x_info, y_info, zi, tad=tad), op, X.ptr, X.info_ptr, e,
+                                                            Y.ptr, Y.info_ptr, Z.ptr, Z.info_ptr, d, len(dims))
+        out = Z.get()
+        self._finish(X, Y, Z, E, D)
+        return out
+
+    def reduce3_all(self, op, x, x_info, y, y_info, extra, dims, out_len):
+        X, Y = self._op(x, x_info), self._op(y, y_info)
+        zi = _vec_info(out_len)
+        Z = self._op(np.zeros(out_len, x.dtype), zi)
+        E, e = self._up(extra, x.dtype)
+        D, d = self._up(np.array(list(dims), np.int32))
+        getattr(self.ops, "execReduce3All" + self._suffix(x))(self.dev.extra(x_info, y_info, zi), op, X.ptr, X.info_ptr, e, Y.ptr,
+                                                               Y.info_ptr, Z.ptr, Z.info_ptr, d, len(dims), None, None, None, None)
+        out = Z.get()
+        self._finish(X, Y, Z, E, D)
+        return out
 
     def indexreduce(self, op, x, x_info, extra, dims, out_len, pass_tads=True):
         return self._reduce_like("execIndexReduce", op, x, x_info, extra, dims, out_len, pass_tads=pass_tads)

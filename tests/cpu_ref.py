@@ -60,6 +60,10 @@ class CpuLib(object):
         sigs = {
             "transform": [I, V, V, V, V, V],
             "transform_strided": [I, V, LL, V, LL, V, LL],
+            "reduce3_scalar": [I, V, V, V, V, V, V],
+            "reduce3": [I, V, V, V, V, V, V, V, V, I],
+            "reduce3_tad": [I, V, V, V, V, V, V, V, V, I],
+            "reduce3_all": [I, V, V, V, V, V, V, V, V, I],
             "scalar": [I, V, V, V, V, ctypes.c_double, V],
             "scalar_strided": [I, V, LL, V, LL, ctypes.c_double, V, LL],
             "scalar_tad": [I, V, V, V, V, V, V, V, I],
@@ -95,6 +99,25 @@ class CpuLib(object):
 
     def transform_strided(self, op, x, xs, z, zs, extra, n):
         self._fn("transform_strided", x)(op, _p(x), xs, _p(z), zs, _p(extra), n)
+
+    def reduce3_scalar(self, op, x, x_info, y, y_info, extra=None):
+        out = np.zeros(1, x.dtype)
+        self._fn("reduce3_scalar", x)(op, _p(x), _p(_info(x_info)), _p(extra), _p(y), _p(_info(y_info)), _p(out))
+        return out[0]
+
+    def _reduce3(self, which, op, x, x_info, y, y_info, z, z_info, dims, extra):
+        d = _ints(dims)
+        self._fn(which, x)(op, _p(x), _p(_info(x_info)), _p(extra), _p(y), _p(_info(y_info)), _p(z), _p(_info(z_info)),
+                           _p(d), len(dims))
+
+    def reduce3(self, op, x, x_info, y, y_info, z, z_info, dims, extra=None):
+        self._reduce3("reduce3", op, x, x_info, y, y_info, z, z_info, dims, extra)
+
+    def reduce3_tad(self, op, x, x_info, y, y_info, z, z_info, dims, extra=None):
+        self._reduce3("reduce3_tad", op, x, x_info, y, y_info, z, z_info, dims, extra)
+
+    def reduce3_all(self, op, x, x_info, y, y_info, z, z_info, dims, extra=None):
+        self._reduce3("reduce3_all", op, x, x_info, y, y_info, z, z_info, dims, extra)
 
     def scalar(self, op, x, x_info, z, z_info, scalar, extra=None):
         self._fn("scalar", x)(op, _p(x), _p(_info(x_info)), _p(z), _p(_info(z_info)), float(scalar), _p(extra) if extra is not None else None)

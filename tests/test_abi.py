@@ -14,7 +14,7 @@ def _declared_c_names():
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     text = text.replace("\\\n", " ")
     names = set(re.findall(r"\b(nd4j_(?:amd_)?[A-Za-z0-9]+)\s*\(", text))
-    for macro_name in ("ND4J_C_EXEC", "ND4J_C_SCALAR"):
+    for macro_name in ("ND4J_C_EXEC", "ND4J_C_SCALAR", "ND4J_C_REDUCE3"):
         macro = re.search(r"#define %s\(SUFFIX, T, [RS]\)(.*?)\n\s*\n" % macro_name, text, flags=re.S).group(1)
         for templ in re.findall(r"\b(nd4j_[A-Za-z0-9#]+)\s*\(", macro):
             for suffix in ("Float", "Half", "Double"):
@@ -36,7 +36,8 @@ def test_cpp_class_members_are_exported():
     for member in ("execTransformFloat", "execTransformHalf", "execPairwiseTransformFloat", "execBroadcastFloat",
                    "execReduceFloat", "execReduceScalarFloat", "execIndexReduceFloat", "execIndexReduceScalarFloat",
                    "execSummaryStatsFloat", "execSummaryStatsScalarFloat", "execRandomFloat", "execRandomHalf",
-                   "execScalarFloat", "execScalarHalf", "execScalarDouble",
+                   "execScalarFloat", "execScalarHalf", "execScalarDouble", "execReduce3Float", "execReduce3ScalarFloat",
+                   "execReduce3AllFloat", "execReduce3Half", "execReduce3Double",
                    "initRandom", "refreshBuffer", "reSeedBuffer", "destroyRandom", "tadOnlyShapeInfo", "mallocDevice",
                    "createStream", "memcpyAsync", "streamSynchronize"):
         assert "NativeOps::%s(" % member in out, member

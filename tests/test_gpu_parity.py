@@ -284,6 +284,80 @@ def test_scalar_family(gpu, cpu):
     assert np.all(gpu.scalar(99, x, xi, xi, 1.0) == 0)
 
 
+def test_reduce3_family(gpu, cpu):
+    rs = np.random.RandomState(34)
+    eps = np.array([0.05], np.float32)
+
+    def close(a, b, what):
+        # relative 1e-5 on the sums; cosine / Jaccard distances are 1 - ratio, so the 1e-5 of the ratio (of order one)
+        # is an absolute error on them
+        assert np.allclose(np.asarray(a, np.float64), np.asarray(b, np.float64), rtol=1e-5, atol=2e-5), what
+
+    # whole arrays: contiguous (vector kernel, sliced), odd lengths, f-order, strided views, mixed orders
+    for shape, order in (([1, 777], "c"), ([1, 300001], "c"), ([33, 65], "c"), ([33, 65], "f"), ([5, 6, 7], "c"), ([3, 2, 4, 5], "f")):
+        xi = harness.shape_info(shape, order)
+        n = int(np.prod(shape))
+        x = rs.uniform(0.1, 2, n).astype(np.float32)
+        y = (x + rs.uniform(-0.1, 0.1, n)).astype(np.float32)
+        y[::7] = x[::7]
+        for op in range(8):
+            e = eps if op == 4 else None
+            close(gpu.reduce3_scalar(op, x, xi, y, xi, e), cpu.reduce3_scalar(op, x, xi, y, xi, e), (shape, order, op))
+        other = harness.shape_info(shape, "f" if order == "c" else "c")
+        for op in (0, 2, 3):
+            close(gpu.reduce3_scalar(op, x, xi, y, other), cpu.reduce3_scalar(op, x, xi, y, other), (shape, "mixed", op))
+    vx = VIEWS[4]  # strided
+    xs, xsi = _mk(vx, rs)
+    ys = (xs + 0.25).astype(np.float32)
+    for op in (0, 1, 3, 7):
+        close(gpu.reduce3_scalar(op, xs, xsi, ys, xsi), cpu.reduce3_scalar(op, xs, xsi, ys, xsi), ("strided", op))
+    # along dimensions: TAD against TAD, TAD against one vector (with and without the caller's TAD tables)
+    for shape, order, dims in (([33, 65], "c", [1]), ([33, 65], "c", [0]), ([6, 5, 7], "c", [2]), ([6, 5, 7], "c", [1, 2]),
+                               ([6, 5, 7], "c", [0]), ([40, 5000], "c", [1]), ([300, 130], "f", [0])):
+        xi = harness.shape_info(shape, order)
+        n = int(np.prod(shape))
+        x = rs.uniform(0.1, 2, n).astype(np.float32)
+        y = (x + rs.uniform(-0.1, 0.1, n)).astype(np.float32)
+        out_len = n // int(np.prod([shape[d] for d in dims]))
+        tad_len = n // out_len
+        for op in (0, 1, 2, 3, 5, 6, 7):
+            # without element-wise strides on the arrays and their TADs the reference keeps one set of running norms
+            # for all TADs (reduce3.h:1322-1341) and its cosine / Jaccard results drift: no checker for those
+            if not ((len(dims) > 1 or order == "f") and op in (2, 5, 6)):
+                close(gpu.reduce3(op, x, xi, y, xi, None, dims, out_len), cpu.reduce3(op, x, xi, y, xi, None, dims, out_len), (shape, dims, op))
+            yv = y[:tad_len].copy()
+            yi = shape_info_np([1, tad_len])
+            want = cpu.reduce3(op, x, xi, yv, yi, None, dims, out_len, tad_way=True)
+            close(gpu.reduce3(op, x, xi, yv, yi, None, dims, out_len), want, (shape, dims, op, "vector y"))
+            close(gpu.reduce3(op, x, xi, yv, yi, None, dims, out_len, pass_tads=False), want, (shape, dims, op, "no tables"))
+    # all pairs of TADs
+    xi, yi = shape_info_np([7, 190]), shape_info_np([4, 190])
+    x, y = rs.uniform(0.1, 2, 7 * 190).astype(np.float32), rs.uniform(0.1, 2, 4 * 190).astype(np.float32)
+    for op in (0, 1, 2, 3, 5, 6, 7):
+        close(gpu.reduce3_all(op, x, xi, y, yi, None, [1], 28), cpu.reduce3_all(op, x, xi, y, yi, None, [1], 28), ("all", op))
+    # float64 ground truth at a size the sliced kernel splits
+    n = 1 << 20
+    x = rs.randn(n).astype(np.float32)
+    y = rs.randn(n).astype(np.float32)
+    vi = shape_info_np([1, n])
+    x64, y64 = x.astype(np.float64), y.astype(np.float64)
+    scale = np.abs(x64 * y64).sum() / np.sqrt(n)
+    assert abs(float(gpu.reduce3_scalar(3, x, vi, y, vi)) - np.dot(x64, y64)) <= 1e-5 * max(abs(np.dot(x64, y64)), scale)
+    assert abs(float(gpu.reduce3_scalar(1, x, vi, y, vi)) - np.linalg.norm(x64 - y64)) <= 1e-5 * np.linalg.norm(x64 - y64)
+    cos = np.dot(x64, y64) / (np.linalg.norm(x64) * np.linalg.norm(y64))
+    assert abs(float(gpu.reduce3_scalar(2, x, vi, y, vi)) - cos) <= 1e-5
+    # fp16 and fp64
+    xh, yh = rs.uniform(0.5, 1.5, 4096).astype(np.float16), rs.uniform(0.5, 1.5, 4096).astype(np.float16)
+    hi = shape_info_np([1, 4096])
+    dot = np.dot(xh.astype(np.float64), yh.astype(np.float64))
+    assert abs(float(gpu.reduce3_scalar(3, xh, hi, yh, hi)) - dot) <= 1e-2 * dot
+    xd, yd = rs.randn(5000), rs.randn(5000)
+    di = shape_info_np([1, 5000])
+    assert abs(float(gpu.reduce3_scalar(0, xd, di, yd, di)) - np.abs(xd - yd).sum()) <= 1e-12 * np.abs(xd - yd).sum()
+    # unknown opNum
+    assert float(gpu.reduce3_scalar(42, x, vi, y, vi)) == 0.0
+
+
 def test_nan_and_special_values(gpu, cpu):
     x = np.array([np.nan, 1.0, -np.inf, np.inf, 0.0, -0.0, 3.0, np.nan, 2.0, -1e38, 1e38, 5.0], np.float32)
     xi = shape_info_np([1, x.size])

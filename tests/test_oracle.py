@@ -131,6 +131,73 @@ def test_scalar_family_matches_compiled_reference(oracle, reference_lib):
         assert np.array_equal(oracle.scalar(op, x, fi, ci, 0.37), ref.scalar(op, x, fi, ci, 0.37)), op
 
 
+REDUCE3_OPS = list(range(8))
+
+
+def test_reduce3_matches_compiled_reference(oracle, reference_lib):
+    """Whole arrays (every view), along a dimension for equally long same-order operands, against a single-TAD y
+    through the reference's TAD-table variant, and all pairs.  Inputs on which the reference itself is undefined
+    are left out: cosine / Jaccard over TADs without an element-wise stride in the no-table variant (one set of
+    running norms shared by all TADs), EqualsWithEps along a dimension (reads extraParams[2] of a null or zero-length array),
+    operands of different order along a dimension (its raw-iteration branch indexes the result by
+    offset / resultLength) and the no-table variant with a shorter y (walks the TAD strides as a shape)."""
+    ref = backends.CpuBackend(reference_lib)
+    rs = np.random.RandomState(33)
+
+    def close(a, b):
+        # the reference's sums are re-associated by its release flags (vectorised partial sums), so the two
+        # sequentially written loops agree to rounding, not bit for bit; all terms here are positive
+        return np.allclose(np.asarray(a, np.float64), np.asarray(b, np.float64), rtol=1e-5, atol=1e-6)
+
+    eps = np.array([0.05], np.float32)
+    for shape, order in (([1, 777], "c"), ([33, 65], "c"), ([33, 65], "f"), ([5, 6, 7], "c"), ([3, 2, 4, 5], "f")):
+        xi = shape_info_np(shape, order)
+        n = int(np.prod(shape))
+        x = rs.uniform(0.1, 2, n).astype(np.float32)
+        y = (x + rs.uniform(-0.1, 0.1, n)).astype(np.float32)
+        y[::7] = x[::7]
+        for op in REDUCE3_OPS:
+            e = eps if op == 4 else None
+            assert close(oracle.reduce3_scalar(op, x, xi, y, xi, e), ref.reduce3_scalar(op, x, xi, y, xi, e)), (shape, order, op)
+        # mixed orders pair by logical index
+        other = shape_info_np(shape, "f" if order == "c" else "c")
+        for op in (0, 2, 3):
+            assert close(oracle.reduce3_scalar(op, x, xi, y, other), ref.reduce3_scalar(op, x, xi, y, other)), (shape, op)
+    for shape, order, dims in (([33, 65], "c", [1]), ([33, 65], "c", [0]), ([6, 5, 7], "c", [2]), ([6, 5, 7], "c", [1, 2]),
+                               ([6, 5, 7], "c", [0])):
+        xi = shape_info_np(shape, order)
+        n = int(np.prod(shape))
+        x = rs.uniform(0.1, 2, n).astype(np.float32)
+        y = (x + rs.uniform(-0.1, 0.1, n)).astype(np.float32)
+        out_len = n // int(np.prod([shape[d] for d in dims]))
+        tad_len = n // out_len
+        for op in (0, 1, 2, 3, 5, 6, 7):
+            if len(dims) > 1 and op in (2, 5, 6):
+                # TADs without an element-wise stride: the reference's branch for them (reduce3.h:1322-1341) keeps
+                # one set of running norms for all TADs, so its cosine / Jaccard results drift from TAD to TAD
+                continue
+            assert close(oracle.reduce3(op, x, xi, y, xi, None, dims, out_len), ref.reduce3(op, x, xi, y, xi, None, dims, out_len)), (shape, dims, op)
+            yv = y[:tad_len].copy()
+            yi = shape_info_np([1, tad_len])
+            assert close(oracle.reduce3(op, x, xi, yv, yi, None, dims, out_len, tad_way=True),
+                         ref.reduce3(op, x, xi, yv, yi, None, dims, out_len, tad_way=True)), (shape, dims, op)
+    xi, yi = shape_info_np([7, 19]), shape_info_np([4, 19])
+    x, y = rs.uniform(0.1, 2, 7 * 19).astype(np.float32), rs.uniform(0.1, 2, 4 * 19).astype(np.float32)
+    for op in (0, 1, 2, 3, 5, 6, 7):
+        assert close(oracle.reduce3_all(op, x, xi, y, yi, None, [1], 28), ref.reduce3_all(op, x, xi, y, yi, None, [1], 28)), op
+    # closed forms on the same data
+    x64, y64 = x.astype(np.float64)[:76], y.astype(np.float64)
+    vi = shape_info_np([1, 76])
+    xs = x[:76].copy()
+    assert abs(oracle.reduce3_scalar(3, xs, vi, y, vi) - np.dot(x64, y64)) <= 1e-5 * abs(np.dot(x64, y64))
+    assert abs(oracle.reduce3_scalar(1, xs, vi, y, vi) - np.linalg.norm(x64 - y64)) <= 1e-5 * np.linalg.norm(x64 - y64)
+    cos = np.dot(x64, y64) / (np.linalg.norm(x64) * np.linalg.norm(y64))
+    assert abs(oracle.reduce3_scalar(2, xs, vi, y, vi) - cos) <= 1e-5
+    assert abs(oracle.reduce3_scalar(5, xs, vi, y, vi) - (1 - cos)) <= 1e-5
+    assert abs(oracle.reduce3_scalar(6, xs, vi, y, vi) - (1 - np.minimum(x64, y64).sum() / np.maximum(x64, y64).sum())) <= 1e-5
+    assert abs(oracle.reduce3_scalar(0, xs, vi, y, vi) - np.abs(x64 - y64).sum()) <= 1e-5 * np.abs(x64 - y64).sum()
+
+
 def test_broadcast_matches_compiled_reference(oracle, reference_lib):
     ref = backends.CpuBackend(reference_lib)
     rs = np.random.RandomState(12)
