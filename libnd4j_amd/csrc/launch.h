@@ -111,6 +111,19 @@ template <typename T>
 bool launchReduce3(hipStream_t stream, int opNum, const T *x, const T *y, T *z, const T *extra, const Reduce3Launch &in,
                    Workspace ws);
 
+// ---- special transforms ----------------------------------------------------------------------------
+// numRows rows of `length` elements: row r starts at r * xRow (z: r * zRow), its elements are xEl (zEl) apart
+struct SoftmaxPlan {
+    Long numRows, length;
+    Long xRow, xEl, zRow, zEl;
+};
+// opNum 38 SoftMax, 39 SoftMaxDerivative, 40 LogSoftMax
+template <typename T> bool launchSoftmax(hipStream_t stream, int opNum, const T *x, T *z, const SoftmaxPlan &plan);
+// z = one-hot of the position stored (as a T) in index[0] / index[tad]; `zp` / `zt` walk z the way the index
+// reduction walked x
+template <typename T> void launchIsMaxFill(hipStream_t stream, T *z, const T *index, const FlatPlan &zp);
+template <typename T> void launchIsMaxTadFill(hipStream_t stream, T *z, const T *index, const TadPlan &zt);
+
 // ---- random ----------------------------------------------------------------------------------------
 // Device image of the generator state that getElement() needs (reference: helper_generator.h:61-74,
 // 185-220).  Passed by value, so one op sees one consistent state.

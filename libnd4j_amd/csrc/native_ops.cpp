@@ -47,6 +47,11 @@ void transformShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, Lon
     const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
     const Long *hz = hostShapeInfo(extra, X_HOST_Z_SHAPE, zInfo, sz, s);
     if (hx == nullptr || hz == nullptr) return;
+    if (opNum >= 38 && opNum <= 41) {
+        // whole-array special ops: SoftMax, SoftMaxDerivative, LogSoftMax, IsMax
+        if (!specialTransform<T>(extra, opNum, x, hx, z, hz, params, s)) reportUnknownOp("transform", opNum);
+        return;
+    }
     Long n = siNumel(hx);
     Long xe = siEws(hx), ze = siEws(hz);
     bool ok;

@@ -414,6 +414,99 @@ void reduce3All(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *
     checkLaunch("execReduce3All", s);
 }
 
+// ---- special transforms (include/ops/special_ops.h:1422-2260) -------------------------------------------
+namespace nd4j_amd {
+
+template <typename T>
+bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z, const Long *hz, T *params, hipStream_t s) {
+    if (opNum < 38 || opNum > 41) return false;
+    const int rank = siRank(hx);
+    const Long n = siNumel(hx);
+    if (n <= 0) return true;
+    if (opNum != 41) {
+        // SoftMax family: over each row of a matrix, over a vector as a whole; other ranks are left alone, as in
+        // the reference (special_ops.h:1483, 1533)
+        SoftmaxPlan pl;
+        const bool vector = rank <= 1 || (rank == 2 && (siShape(hx)[0] == 1 || siShape(hx)[1] == 1));
+        if (vector) {
+            pl.numRows = 1;
+            pl.length = n;
+            pl.xRow = pl.zRow = 0;
+            // the stride of the dimension that is walked (the EWS field says the same for a vector)
+            const int xd = (rank == 2 && siShape(hx)[0] != 1) ? 0 : rank - 1;
+            const int zd = (siRank(hz) == 2 && siShape(hz)[0] != 1) ? 0 : siRank(hz) - 1;
+            pl.xEl = rank >= 1 ? siStride(hx)[xd] : 1;
+            pl.zEl = siRank(hz) >= 1 ? siStride(hz)[zd] : 1;
+        } else if (rank == 2 && siRank(hz) == 2) {
+            pl.numRows = siShape(hx)[0];
+            pl.length = siShape(hx)[1];
+            pl.xRow = siStride(hx)[0];
+            pl.xEl = siStride(hx)[1];
+            pl.zRow = siStride(hz)[0];
+            pl.zEl = siStride(hz)[1];
+        } else {
+            return true;
+        }
+        if (!launchSoftmax<T>(s, opNum, x, z, pl)) return false;
+        checkLaunch("execTransform(softmax)", s);
+        return true;
+    }
+    // IsMax.  Without extraParams (or with the "all dimensions" marker): one-hot of the first maximum of the whole
+    // array.  With dimensions - extraPointers[15] / [18] hold the device dimension array and its length
+    // (blas/cuda/NativeOps.cu:3280-3284): one-hot per TAD.
+    int dimLen = 0;
+    const int *devDims = nullptr;
+    if (params != nullptr && extra != nullptr) {
+        devDims = reinterpret_cast<const int *>(slotOf(extra, 15));
+        dimLen = (int)reinterpret_cast<intptr_t>(slotOf(extra, 18));
+        if (devDims == nullptr || dimLen <= 0 || dimLen >= rank) dimLen = 0;
+    }
+    if (dimLen == 0) {
+        Scratch sc = scratchFor(s);
+        T *slot = reinterpret_cast<T *>(sc.scalars);
+        FlatPlan xp = flatIndexed(hx);
+        if (!launchIndexReduceScalar<T>(s, 0, x, nullptr, slot, xp, sc.rest)) return false;
+        FlatPlan zp = flatIndexed(hz);
+        launchIsMaxFill<T>(s, z, slot, zp);
+        checkLaunch("execTransform(IsMax)", s);
+        return true;
+    }
+    ResolvedTad tx, tz;
+    if (!resolveTad(extra, X_HOST_TAD_SHAPE, X_DEV_TAD_OFFSETS, hx, devDims, dimLen, tx, s)) return true;
+    if (!resolveTad(nullptr, 0, 0, hz, devDims, dimLen, tz, s)) return true;
+    Scratch sc = scratchFor(s, kScalarArea + (size_t)tx.numTads * sizeof(T) + (size_t)(4u << 20));
+    T *index = reinterpret_cast<T *>(sc.rest.ptr);
+    Workspace rest = sc.rest;
+    size_t used = ((size_t)tx.numTads * sizeof(T) + 255) / 256 * 256;
+    rest.ptr = reinterpret_cast<char *>(rest.ptr) + used;
+    rest.bytes -= used;
+    TadPlan xp = tadPlanFrom(tx);
+    if (tx.numTads == 1) {
+        FlatPlan fp = flatIndexed(hx);
+        if (!launchIndexReduceScalar<T>(s, 0, x, nullptr, index, fp, rest)) return false;
+    } else if (!launchIndexReduceTad<T>(s, 0, x, nullptr, index, xp, rest)) {
+        return false;
+    }
+    TadPlan zp = tadPlanFrom(tz);
+    if (tx.numTads == 1) {
+        FlatPlan fz = flatIndexed(hz);
+        launchIsMaxFill<T>(s, z, index, fz);
+    } else {
+        launchIsMaxTadFill<T>(s, z, index, zp);
+    }
+    checkLaunch("execTransform(IsMax)", s);
+    return true;
+}
+
+#define INST(T) \
+    template bool specialTransform<T>(Nd4jPointer *, int, T *, const Long *, T *, const Long *, T *, hipStream_t);
+INST(float)
+INST(float16)
+INST(double)
+#undef INST
+
+}  // namespace nd4j_amd
+
 #define ND4J_REDUCE3_MEMBERS(SUFFIX, T, R)                                                                          \
     void NativeOps::execReduce3##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,          \
                                         T *extraParamsVals, T *y, Nd4jLong *yShapeInfo, T *result,                  \

@@ -86,4 +86,10 @@ struct ResolvedTad {
 bool resolveTad(Nd4jPointer *extra, int hostSlot, int offsetSlot, const Long *hostXInfo, const int *dimension,
                 int dimLen, ResolvedTad &out, hipStream_t s);
 
+// Whole-array special transforms reached through execTransform (opNums 38-41): SoftMax, SoftMaxDerivative,
+// LogSoftMax, IsMax.  Returns false when opNum is not one of them.
+template <typename T>
+bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hostXInfo, T *z, const Long *hostZInfo, T *params,
+                      hipStream_t s);
+
 }  // namespace nd4j_amd

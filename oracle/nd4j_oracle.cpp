@@ -504,7 +504,98 @@ template <typename T> static void transformStrided(int op, T *x, Long xs, T *z, 
         for (Long i = start; i < end; i++) transformOp<T>(op, x[i * xs], extra, z[i * zs]);
     }
 }
+// Whole-array special transforms (include/ops/special_ops.h): SoftMax 38 (1483-1568), SoftMaxDerivative 39
+// (1806-1937), LogSoftMax 40 (1635-1726) over each row of a matrix or over a vector; IsMax 41 (1951-2260): one-hot of
+// the first maximum of the whole array, or of every TAD along the dimensions listed in extraParams
+// ([0] = count, [1..] = dimensions).  Restated as what the routines compute when called in place (x == z), which is
+// how the reference's vector branches of 39 / 40 and the matrix branch of 39 read their input.
+template <typename T> static void specialTransform(int op, T *x, Long *xi, T *z, Long *zi, T *extra) {
+    const int rank = siRank(xi);
+    const Long n = siNumel(xi);
+    if (n <= 0) return;
+    if (op != 41) {
+        const bool vector = rank <= 1 || (rank == 2 && (siShape(xi)[0] == 1 || siShape(xi)[1] == 1));
+        Long rows, len, xRow, xEl, zRow, zEl;
+        if (vector) {
+            const int xd = (rank == 2 && siShape(xi)[0] != 1) ? 0 : rank - 1;
+            const int zd = (siRank(zi) == 2 && siShape(zi)[0] != 1) ? 0 : siRank(zi) - 1;
+            rows = 1; len = n; xRow = zRow = 0;
+            xEl = siStride(xi)[xd];
+            zEl = siStride(zi)[zd];
+        } else if (rank == 2) {
+            rows = siShape(xi)[0]; len = siShape(xi)[1];
+            xRow = siStride(xi)[0]; xEl = siStride(xi)[1];
+            zRow = siStride(zi)[0]; zEl = siStride(zi)[1];
+        } else {
+            return;
+        }
+        for (Long r = 0; r < rows; r++) {
+            T *xr = x + r * xRow, *zr = z + r * zRow;
+            T mx = xr[0];
+            for (Long c = 1; c < len; c++) mx = m_max(mx, xr[c * xEl]);
+            T sum = (T)0.0f;
+            for (Long c = 0; c < len; c++) { T e = m_exp(xr[c * xEl] - mx); zr[c * zEl] = e; sum += e; }
+            for (Long c = 0; c < len; c++) {
+                T v = zr[c * zEl] / sum;
+                if (op == 39) v = v * ((T)1.0f - v);
+                else if (op == 40) v = m_log(v);
+                zr[c * zEl] = v;
+            }
+        }
+        return;
+    }
+    int dimLen = extra == nullptr ? 0 : toInt(extra[0]);
+    if (dimLen == 1 && toInt(extra[1]) == 0x7fffffff) dimLen = 0;
+    if (dimLen <= 0 || dimLen >= rank) {
+        // first maximum in the element order of the index reductions: memory-linear with an element-wise stride,
+        // C-order coordinates otherwise
+        const Long xe = siEws(xi), ze = siEws(zi);
+        Long best = 0;
+        T bestV = x[0];
+        Long cx[kMaxRank];
+        for (Long i = 0; i < n; i++) {
+            Long ox;
+            if (xe >= 1) ox = i * xe;
+            else { ind2subC(rank, siShape(xi), (int)i, cx); ox = getOffset(0, siShape(xi), siStride(xi), cx, rank); }
+            if (x[ox] > bestV) { bestV = x[ox]; best = i; }
+        }
+        for (Long i = 0; i < n; i++) {
+            Long oz;
+            if (ze >= 1) oz = i * ze;
+            else { ind2subC(siRank(zi), siShape(zi), (int)i, cx); oz = getOffset(0, siShape(zi), siStride(zi), cx, siRank(zi)); }
+            z[oz] = i == best ? (T)1.0f : (T)0.0f;
+        }
+        return;
+    }
+    int dims[kMaxRank];
+    for (int i = 0; i < dimLen; i++) dims[i] = toInt(extra[i + 1]);
+    TadPack tx, tz;
+    computeTad(xi, dims, dimLen, tx, true);
+    computeTad(zi, dims, dimLen, tz, true);
+    const Long *xt = tx.shapeInfo.data(), *zt = tz.shapeInfo.data();
+    const Long len = siNumel(xt);
+    Long c[kMaxRank];
+    for (Long r = 0; r < tx.numTads; r++) {
+        Long best = 0;
+        T bestV = (T)0.0f;
+        for (Long f = 0; f < len; f++) {
+            Long ox;
+            if (siEws(xt) >= 1) ox = f * siEws(xt);
+            else { ind2subC(siRank(xt), siShape(xt), (int)f, c); ox = getOffset(0, siShape(xt), siStride(xt), c, siRank(xt)); }
+            T v = x[tx.offsets[r] + ox];
+            if (f == 0 || v > bestV) { bestV = v; best = f; }
+        }
+        for (Long f = 0; f < len; f++) {
+            Long oz;
+            if (siEws(zt) >= 1) oz = f * siEws(zt);
+            else { ind2subC(siRank(zt), siShape(zt), (int)f, c); oz = getOffset(0, siShape(zt), siStride(zt), c, siRank(zt)); }
+            z[tz.offsets[r] + oz] = f == best ? (T)1.0f : (T)0.0f;
+        }
+    }
+}
+
 template <typename T> static void transformShaped(int op, T *x, Long *xi, T *z, Long *zi, T *extra) {
+    if (op >= 38 && op <= 41) { specialTransform<T>(op, x, xi, z, zi, extra); return; }
     Long n = siNumel(xi);
     Long xe = siEws(xi), ze = siEws(zi);
     if (xe >= 1 && ze >= 1 && siOrder(xi) == siOrder(zi)) { transformStrided<T>(op, x, xe, z, ze, extra, n); return; }

@@ -215,10 +215,18 @@ class GpuBackend(object):
         X = self._op(x, x_info)
         Z = self._op(np.zeros(_span(z_info), x.dtype) if z is None else z, z_info)
         E, e = self._up(extra, x.dtype)
-        getattr(self.ops, "execTransform" + self._suffix(x))(self.dev.extra(x_info, z_info=z_info), op, X.ptr, X.info_ptr,
-                                                              Z.ptr, Z.info_ptr, e)
+        ptrs = self.dev.extra(x_info, z_info=z_info)
+        D = None
+        if op == 41 and extra is not None:
+            # IsMax along dimensions: the CUDA convention carries them in extraPointers[15] (device int array) and
+            # [18] (their count); extraParams only has to be non-null
+            dims = [int(v) for v in np.asarray(extra)[1:1 + int(np.asarray(extra)[0])]]
+            D, d = self._up(np.array(dims, np.int32))
+            ptrs[15] = d
+            ptrs[18] = len(dims)
+        getattr(self.ops, "execTransform" + self._suffix(x))(ptrs, op, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, e)
         out = Z.get()
-        self._finish(X, Z, E)
+        self._finish(X, Z, E, D)
         return out
 
     def transform_inplace(self, op, x, x_info, extra=None):

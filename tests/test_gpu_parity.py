@@ -358,6 +358,76 @@ def test_reduce3_family(gpu, cpu):
     assert float(gpu.reduce3_scalar(42, x, vi, y, vi)) == 0.0
 
 
+def test_special_transforms(gpu, cpu):
+    rs = np.random.RandomState(36)
+
+    def close(a, b, what):
+        a64, b64 = np.asarray(a, np.float64), np.asarray(b, np.float64)
+        assert np.all(np.abs(a64 - b64) <= 1e-5 * np.abs(b64) + 1e-7), what
+
+    # softmax family: short / wave / block rows, vectors, f-order (rows adjacent in memory), f -> c
+    for shape, order in (([37, 129], "c"), ([300, 17], "c"), ([9, 5000], "c"), ([1, 500], "c"), ([700, 1], "c"), ([1, 70001], "c"),
+                         ([257, 96], "f"), ([64, 300], "f"), ([8, 8], "c")):
+        n = int(np.prod(shape))
+        xi = harness.shape_info(shape, order)
+        x = rs.uniform(-6, 6, n).astype(np.float32)
+        logical = x.astype(np.float64).reshape(shape, order="F" if order == "f" else "C")
+        rows = logical if min(shape) > 1 else logical.reshape(1, -1)
+        truth = np.exp(rows - rows.max(axis=1, keepdims=True))
+        truth /= truth.sum(axis=1, keepdims=True)
+        for op, f in ((38, lambda v: v), (39, lambda v: v * (1 - v)), (40, np.log)):
+            got = gpu.transform(op, x, xi, xi).astype(np.float64).reshape(shape, order="F" if order == "f" else "C")
+            got = got if min(shape) > 1 else got.reshape(1, -1)
+            assert np.all(np.abs(got - f(truth)) <= 2e-5 * np.abs(f(truth)) + 1e-7), (shape, order, op)
+        if order == "c":
+            close(gpu.transform(38, x, xi, xi), cpu.transform(38, x, xi, xi), (shape, "vs cpu"))
+            if shape[1] != 1:
+                close(gpu.transform_inplace(40, x, xi), cpu.transform_inplace(40, x, xi), (shape, "log in place"))
+    fi, ci = harness.shape_info([40, 50], "f"), harness.shape_info([40, 50], "c")
+    x = rs.uniform(-3, 3, 2000).astype(np.float32)
+    got = gpu.transform(38, x, fi, ci).reshape(40, 50).astype(np.float64)
+    rows = x.astype(np.float64).reshape(40, 50, order="F")
+    truth = np.exp(rows - rows.max(axis=1, keepdims=True))
+    truth /= truth.sum(axis=1, keepdims=True)
+    assert np.all(np.abs(got - truth) <= 2e-5 * truth)
+    # half and double
+    xh = rs.uniform(-2, 2, 64 * 96).astype(np.float16)
+    hi = shape_info_np([64, 96])
+    g = gpu.transform(38, xh, hi, hi).astype(np.float64).reshape(64, 96)
+    rows = xh.astype(np.float64).reshape(64, 96)
+    truth = np.exp(rows - rows.max(axis=1, keepdims=True))
+    truth /= truth.sum(axis=1, keepdims=True)
+    assert np.all(np.abs(g - truth) <= 1e-2 * truth + 1e-4)
+    xd = rs.randn(30 * 40)
+    di = shape_info_np([30, 40])
+    rows = xd.reshape(30, 40)
+    truth = np.exp(rows - rows.max(axis=1, keepdims=True))
+    truth /= truth.sum(axis=1, keepdims=True)
+    assert np.allclose(gpu.transform(38, xd, di, di).reshape(30, 40), truth, rtol=1e-13)
+    # IsMax: whole array (also a large one, f-order and 3-D), and along a dimension
+    for shape, order in (([1, 300], "c"), ([12, 40], "c"), ([5, 6, 7], "c"), ([12, 40], "f"), ([1, 200003], "c")):
+        n = int(np.prod(shape))
+        xi = harness.shape_info(shape, order)
+        x = rs.permutation(n).astype(np.float32)
+        got = gpu.transform(41, x, xi, xi)
+        assert np.array_equal(got, cpu.transform(41, x, xi, xi)), (shape, order)
+        assert got.sum() == 1 and got[np.argmax(x)] == 1
+    tie = np.array([1, 7, 7, 3, 7, 0], np.float32)
+    assert np.array_equal(gpu.transform(41, tie, shape_info_np([1, 6]), shape_info_np([1, 6])), [0, 1, 0, 0, 0, 0])
+    for shape, order in (([12, 40], "c"), ([12, 40], "f"), ([300, 700], "c")):
+        xi = harness.shape_info(shape, order)
+        n = shape[0] * shape[1]
+        x = rs.permutation(n).astype(np.float32)
+        m = x.reshape(shape, order="F" if order == "f" else "C")
+        for dim in (0, 1):
+            e = np.array([1, dim], np.float32)
+            got = gpu.transform(41, x, xi, xi, e)
+            want = (m == m.max(axis=dim, keepdims=True)).astype(np.float32)
+            assert np.array_equal(got.reshape(shape, order="F" if order == "f" else "C"), want), (shape, order, dim)
+            if order == "c":
+                assert np.array_equal(got, cpu.transform(41, x, xi, xi, e)), (shape, dim)
+
+
 def test_nan_and_special_values(gpu, cpu):
     x = np.array([np.nan, 1.0, -np.inf, np.inf, 0.0, -0.0, 3.0, np.nan, 2.0, -1e38, 1e38, 5.0], np.float32)
     xi = shape_info_np([1, x.size])
@@ -374,7 +444,7 @@ def test_unknown_op_leaves_output_untouched(gpu, capfd):
     xi = shape_info_np([1, 64])
     got = gpu.transform(500, x, xi, xi, z=np.full(64, 9.0, np.float32))
     assert np.all(got == 9.0)
-    got = gpu.transform(38, x, xi, xi, z=np.full(64, 9.0, np.float32))  # SoftMax: whole-array op, not on this path
+    got = gpu.transform(36, x, xi, xi, z=np.full(64, 9.0, np.float32))  # Col2Im: a whole-array op that is not on this path
     assert np.all(got == 9.0)
     assert float(gpu.reduce_scalar(2, x, xi)) == 0.0  # opNum 2 is a gap in the reduce table
 

@@ -198,6 +198,52 @@ def test_reduce3_matches_compiled_reference(oracle, reference_lib):
     assert abs(oracle.reduce3_scalar(0, xs, vi, y, vi) - np.abs(x64 - y64).sum()) <= 1e-5 * np.abs(x64 - y64).sum()
 
 
+def test_special_transforms_match_compiled_reference(oracle, reference_lib):
+    """SoftMax out of place; SoftMaxDerivative and LogSoftMax in place (the only way the reference's own routines
+    read the right operand, see oracle/nd4j_oracle.cpp); IsMax over everything and along a dimension."""
+    ref = backends.CpuBackend(reference_lib)
+    rs = np.random.RandomState(35)
+
+    def close(a, b, what):
+        a64, b64 = np.asarray(a, np.float64), np.asarray(b, np.float64)
+        assert np.all(np.abs(a64 - b64) <= 1e-5 * np.abs(b64) + 1e-7), what
+
+    for shape in ([37, 129], [1, 500], [300, 1], [8, 8]):
+        n = int(np.prod(shape))
+        xi = shape_info_np(shape)
+        x = rs.uniform(-6, 6, n).astype(np.float32)
+        close(oracle.transform(38, x, xi, xi), ref.transform(38, x, xi, xi), ("softmax", shape))
+        for op in (39, 40):
+            if shape[1] == 1:
+                # the reference tests these two ops with isMatrix(shapeInfo, 2), which reads the rank field as a
+                # dimension and so takes a column vector for a matrix of one-element rows (special_ops.h:1642, 1813)
+                continue
+            close(oracle.transform_inplace(op, x, xi), ref.transform_inplace(op, x, xi), (op, shape))
+        # rows sum to one
+        sm = oracle.transform(38, x, xi, xi).astype(np.float64)
+        rows = sm.reshape(shape) if min(shape) > 1 else sm.reshape(1, -1)
+        assert np.all(np.abs(rows.sum(axis=1) - 1) <= 1e-5)
+        truth = np.exp(x.astype(np.float64).reshape(rows.shape) - x.astype(np.float64).reshape(rows.shape).max(axis=1, keepdims=True))
+        truth /= truth.sum(axis=1, keepdims=True)
+        assert np.all(np.abs(rows - truth) <= 1e-5 * truth + 1e-9)
+    for shape in ([1, 300], [12, 40], [5, 6, 7]):
+        n = int(np.prod(shape))
+        xi = shape_info_np(shape)
+        x = rs.permutation(n).astype(np.float32)
+        got = oracle.transform(41, x, xi, xi)
+        assert np.array_equal(got, ref.transform(41, x, xi, xi)), shape
+        assert got.sum() == 1 and got[np.argmax(x)] == 1
+    xi = shape_info_np([12, 40])
+    x = rs.permutation(480).astype(np.float32)
+    for dim in (0, 1):
+        e = np.array([1, dim], np.float32)
+        got = oracle.transform(41, x, xi, xi, e)
+        assert np.array_equal(got, ref.transform(41, x, xi, xi, e)), dim
+        m = x.reshape(12, 40)
+        want = (m == m.max(axis=dim, keepdims=True)).astype(np.float32)
+        assert np.array_equal(got.reshape(12, 40), want)
+
+
 def test_broadcast_matches_compiled_reference(oracle, reference_lib):
     ref = backends.CpuBackend(reference_lib)
     rs = np.random.RandomState(12)
