@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--families", action="store_true", help="also time every op family of the other configurations")
+    ap.add_argument("--only", default="", help="with --families: comma-separated workload builders to run "
+                                               "(transform,pairwise,half,reductions,reduce3,stats,random)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU sample of the headline step")
     ap.add_argument("--counters", action="store_true",
@@ -218,10 +220,14 @@ def main():
     # ---- every other family ---------------------------------------------------------------------------
     if args.families:
         fam = []
-        builders = [workloads.transform_tanh, lambda d: workloads.pairwise_broadcast(d, copies=2),
-                    lambda d: workloads.pairwise_broadcast(d, dtype="float16"),
-                    workloads.reductions, workloads.reduce3_pairs, workloads.stats_softmax, workloads.random_fills]
-        for build in builders:
+        builders = [("transform", workloads.transform_tanh), ("pairwise", lambda d: workloads.pairwise_broadcast(d, copies=2)),
+                    ("half", lambda d: workloads.pairwise_broadcast(d, dtype="float16")),
+                    ("reductions", workloads.reductions), ("reduce3", workloads.reduce3_pairs),
+                    ("stats", workloads.stats_softmax), ("random", workloads.random_fills)]
+        only = [o for o in args.only.split(",") if o]
+        for key, build in builders:
+            if only and key not in only:
+                continue
             wl = build(dev)
             for c in wl.cases:
                 ms = time_case(dev, c, max(3, min(K, 20)), 2)

@@ -43,12 +43,14 @@ template <typename T> __device__ __forceinline__ void storePack(Pack<T> *p, cons
 // Functor adapters: apply(a, b, params)
 template <int OP> struct TransformF {
     static constexpr int nin = 1;
+    static constexpr bool tables = !transformIsPlain(OP);
     template <typename C, typename P> static __device__ __forceinline__ C apply(C a, C, P p) {
         return TransformOp<OP>::template op<C, P>(a, p);
     }
 };
 template <int KIND> struct Pairwise3F {
     static constexpr int nin = 2;
+    static constexpr bool tables = !binaryIsPlain(KIND);
     template <typename C, typename P> static __device__ __forceinline__ C apply(C a, C b, P p) {
         return BinaryOp<KIND>::template op3<C, P>(a, b, p);
     }
@@ -66,6 +68,7 @@ template <int KIND, typename C, typename P> __device__ __forceinline__ C scalarO
 // one scalar for the whole array, carried by value in Params
 template <int KIND> struct Scalar3F {
     static constexpr int nin = 1;
+    static constexpr bool tables = !binaryIsPlain(KIND);
     template <typename C, typename P> static __device__ __forceinline__ C apply(C a, C, P p) {
         return scalarOp<KIND, C, P>(a, p.scalarValue(), p);
     }
@@ -73,12 +76,14 @@ template <int KIND> struct Scalar3F {
 // one scalar per TAD, passed as the second operand
 template <int KIND> struct ScalarTad3F {
     static constexpr int nin = 2;
+    static constexpr bool tables = !binaryIsPlain(KIND);
     template <typename C, typename P> static __device__ __forceinline__ C apply(C a, C b, P p) {
         return scalarOp<KIND, C, P>(a, b, p);
     }
 };
 template <int KIND> struct Broadcast2F {
     static constexpr int nin = 2;
+    static constexpr bool tables = !binaryIsPlain(KIND);
     template <typename C, typename P> static __device__ __forceinline__ C apply(C a, C b, P) {
         return BinaryOp<KIND>::template op2<C>(a, b);
     }
@@ -103,16 +108,43 @@ __global__ void __launch_bounds__(kBlock) ewVecKernel(const T *x, const T *y, T 
 
     // one vector per thread and pass: many short blocks sustain a higher HBM rate on this chip than fewer
     // blocks with several vectors in flight per thread
-    for (Long j = (Long)blockIdx.x * kBlock + threadIdx.x; j < nvec; j += (Long)gridDim.x * kBlock) {
-        Pack<T> a = loadPack(xv + j), b;
-        if (F::nin == 2 && !yScalar) b = loadPack(yv + j);
-        Pack<T> r;
-#pragma unroll
-        for (int e = 0; e < VEC; e++) {
-            C bv = (F::nin == 2) ? (yScalar ? ys : toCompute(b.v[e])) : (C)0;
-            r.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), bv, p));
+    if (F::tables) {
+        // the first vectors are requested before the lookup tables are staged, so the two waits overlap
+        Long j = (Long)blockIdx.x * kBlock + threadIdx.x;
+        bool have = j < nvec;
+        Pack<T> a, b;
+        if (have) {
+            a = loadPack(xv + j);
+            if (F::nin == 2 && !yScalar) b = loadPack(yv + j);
         }
-        storePack(zv + j, r);
+        lm::loadTables();
+        while (have) {
+            Pack<T> r;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                C bv = (F::nin == 2) ? (yScalar ? ys : toCompute(b.v[e])) : (C)0;
+                r.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), bv, p));
+            }
+            storePack(zv + j, r);
+            j += (Long)gridDim.x * kBlock;
+            have = j < nvec;
+            if (have) {
+                a = loadPack(xv + j);
+                if (F::nin == 2 && !yScalar) b = loadPack(yv + j);
+            }
+        }
+    } else {
+        for (Long j = (Long)blockIdx.x * kBlock + threadIdx.x; j < nvec; j += (Long)gridDim.x * kBlock) {
+            Pack<T> a = loadPack(xv + j), b;
+            if (F::nin == 2 && !yScalar) b = loadPack(yv + j);
+            Pack<T> r;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                C bv = (F::nin == 2) ? (yScalar ? ys : toCompute(b.v[e])) : (C)0;
+                r.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), bv, p));
+            }
+            storePack(zv + j, r);
+        }
     }
     // head and tail elements
     const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
@@ -153,6 +185,7 @@ template <typename T, typename F>
 __global__ void __launch_bounds__(kBlock) ewGeneralKernel(const T *x, DimMap xm, const T *y, DimMap ym, T *z,
                                                           DimMap zm, Params<T> p, Long n) {
     typedef typename Compute<T>::type C;
+    if (F::tables) lm::loadTables();
     const Long stride = (Long)gridDim.x * kBlock;
     if (n <= 0xffffffffLL) {
         for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
@@ -187,6 +220,7 @@ __global__ void __launch_bounds__(kBlock) bcRowKernel(const T *x, const T *y, T 
                                                       const Long *zOffsets, Long tadLength, Long numTads,
                                                       int basesAligned, int colShift, Params<T> p) {
     typedef typename Compute<T>::type C;
+    if (F::tables) lm::loadTables();
     constexpr int VEC = Pack<T>::N;
     const int colThreads = 1 << colShift;
     const int rowsPerBlock = kBlock >> colShift;
@@ -254,6 +288,7 @@ __global__ void __launch_bounds__(kBlock) bcColKernel(const T *x, const T *y, T 
                                                       const Long *zOffsets, Long tadLength, Long numTads,
                                                       Long tadEws, Long yEws, Long zEws, Params<T> p) {
     typedef typename Compute<T>::type C;
+    if (F::tables) lm::loadTables();
     const Long t = (Long)blockIdx.x * kBlock + threadIdx.x;
     if (t >= numTads) return;
     const T *xr = x + xOffsets[t];
@@ -271,6 +306,7 @@ __global__ void __launch_bounds__(kBlock) bcGeneralKernel(const T *x, DimMap xm,
                                                           DimMap zm, const Long *xOffsets, const Long *zOffsets,
                                                           Long tadLength, Long numTads) {
     typedef typename Compute<T>::type C;
+    if (F::tables) lm::loadTables();
     Params<T> p{nullptr};
     for (Long r = blockIdx.x; r < numTads; r += gridDim.x) {
         const Long xo = xOffsets[r];

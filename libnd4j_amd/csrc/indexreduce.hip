@@ -20,6 +20,7 @@ template <typename TT, int OP> struct IndexPol {
     typedef TT T;
     typedef typename Compute<TT>::type C;
     typedef IndexAcc<C> Acc;
+    static constexpr bool tables = false;  // no exp / log / pow in these accumulators
     Params<TT> p;
 
     __device__ __forceinline__ void setTad(Long, const TT *) {}

@@ -35,6 +35,17 @@ __device__ static const unsigned long long kExp2Tab[32] = {
     0x3fef5818dcfba487ULL, 0x3fef7c97337b9b5fULL, 0x3fefa4afa2a490daULL, 0x3fefd0765b6e4540ULL,
 };
 
+// While a kernel runs, the three lookup tables below (exp2, log, and pow's log2; 256 bytes each) are read from LDS:
+// a per-lane table read from global memory goes through the vector cache next to the kernel's own streaming
+// loads and costs a fused softmax row a third of its time, an LDS read does not.  Every kernel that may evaluate
+// expf_, logf_ or powf_ calls loadTables() first, with all threads of the block, before any thread leaves.
+struct Tables {
+    unsigned long long exp2[32];
+    double log[16][2];
+    double powLog2[16][2];
+};
+static __shared__ Tables sTab;
+
 __device__ __forceinline__ float expf_(float x) {
     const double invLn2N = 0x1.71547652b82fep+0 * 32;
     const double c0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, c1 = 0x1.ebfce50fac4f3p-3 / 32 / 32,
@@ -52,7 +63,7 @@ __device__ __forceinline__ float expf_(float x) {
     unsigned long long ki = asU64(kd);
     kd -= shift;
     double r = z - kd;
-    unsigned long long t = kExp2Tab[ki % 32];
+    unsigned long long t = sTab.exp2[ki % 32];
     t += ki << (52 - 5);
     double s = asF64(t);
     z = c0 * r + c1;
@@ -90,7 +101,7 @@ __device__ __forceinline__ float logf_(float x) {
     int i = (tmp >> (23 - 4)) % 16;
     int k = (int)tmp >> 23;
     unsigned iz = ix - (tmp & (0x1ffu << 23));
-    double invc = kLogTab[i][0], logc = kLogTab[i][1];
+    double invc = sTab.log[i][0], logc = sTab.log[i][1];
     double z = (double)asF32(iz);
     double r = z * invc - 1;
     double y0 = logc + (double)k * ln2;
@@ -286,6 +297,15 @@ __device__ static const double kPowLog2Tab[16][2] = {
     {0x1.886e6037841edp-1, 0x1.88e9c2c1b9ff8p-2},  {0x1.767dcf5534862p-1, 0x1.ce0a44eb17bccp-2},
 };
 
+__device__ __forceinline__ void loadTables() {
+    for (int t = threadIdx.x; t < 96; t += blockDim.x) {
+        if (t < 32) sTab.exp2[t] = kExp2Tab[t];
+        else if (t < 64) (&sTab.log[0][0])[t - 32] = (&kLogTab[0][0])[t - 32];
+        else (&sTab.powLog2[0][0])[t - 64] = (&kPowLog2Tab[0][0])[t - 64];
+    }
+    __syncthreads();
+}
+
 __device__ __forceinline__ bool zeroInfNan(unsigned i) { return 2 * i - 1 >= 2u * 0x7f800000u - 1; }
 
 // 0: y is not an integer, 1: odd integer, 2: even integer
@@ -339,8 +359,8 @@ __device__ __forceinline__ float powf_(float x, float y) {
     const unsigned top = tmp & 0xff800000u;
     const int k = (int)top >> 23;
     const double z = (double)asF32(ix - top);
-    const double r = z * kPowLog2Tab[i][0] - 1;
-    const double y0 = kPowLog2Tab[i][1] + (double)k;
+    const double r = z * sTab.powLog2[i][0] - 1;
+    const double y0 = sTab.powLog2[i][1] + (double)k;
     const double r2 = r * r;
     double yy = 0x1.27616c9496e0bp-2 * r + -0x1.71969a075c67ap-2;
     const double p = 0x1.ec70a6ca7baddp-2 * r + -0x1.7154748bef6c8p-1;
@@ -358,7 +378,7 @@ __device__ __forceinline__ float powf_(float x, float y) {
     const unsigned long long ki = asU64(kd);
     kd -= shift;
     const double rr = ylogx - kd;
-    unsigned long long t = kExp2Tab[ki % 32];
+    unsigned long long t = sTab.exp2[ki % 32];
     t += (ki + signBias) << (52 - 5);
     const double s = asF64(t);
     const double zz = 0x1.c6af84b912394p-5 * rr + 0x1.ebfce50fac4f3p-3;

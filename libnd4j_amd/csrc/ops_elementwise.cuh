@@ -241,6 +241,20 @@ ND4J_TRANSFORM(96, RELU6, {
 
 static constexpr int kTransformOpCount = 97;
 
+// Transforms that evaluate none of exp / log / pow in float, directly or through sigmoid and the like: their
+// kernels skip loading the lookup tables of those routines.  Anything not listed loads them.
+__host__ __device__ constexpr bool transformIsPlain(int op) {
+    switch (op) {
+        case 0: case 1: case 2: case 4: case 6: case 8: case 11: case 12: case 14: case 15: case 19: case 20: case 23: case 24:
+        case 25: case 26: case 27: case 61: case 62:
+        case 31: case 32: case 33: case 34: case 35: case 42: case 49: case 50: case 51: case 52: case 76: case 79:
+        case 80: case 81: case 87: case 94: case 96:
+            return true;
+        default:
+            return false;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Two-operand functors.  `op3` is the (x, y, params) overload that pairwise calls
 // (pairwise_transform.h:154-424); `op2` is the (x, y) overload that broadcast calls
@@ -255,6 +269,11 @@ enum BinaryKind {
 };
 
 template <int KIND> struct BinaryOp;
+
+// Two-operand functors without exp / log / pow (see transformIsPlain)
+__host__ __device__ constexpr bool binaryIsPlain(int kind) {
+    return kind <= B_AMax || kind == B_FloorDiv || kind == B_SafeDivide || kind == B_Axpy;
+}
 
 #define ND4J_BINARY(KIND, BODY3, BODY2)                                                                   \
     template <> struct BinaryOp<KIND> {                                                                   \

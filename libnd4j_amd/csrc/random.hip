@@ -231,6 +231,7 @@ template <typename TT, int OP>
 __global__ void __launch_bounds__(kBlock) randomPlainKernel(RandomCtx<TT> c, const TT *x, const TT *y, TT *z, int nOperands,
                                                             int strided, Long xEws, Long yEws, Long zEws, DimMap xm,
                                                             DimMap ym, DimMap zm) {
+    lm::loadTables();
     typedef typename Compute<TT>::type C;
     const Long chunk = (Long)kBlock * kRngIter;
     RngWalk w;
@@ -258,6 +259,7 @@ __global__ void __launch_bounds__(kBlock) randomPlainKernel(RandomCtx<TT> c, con
 // (LogNormal, 900-969).
 template <typename TT, bool EXP>
 __global__ void __launch_bounds__(kBlock) gaussianKernel(RandomCtx<TT> c, const TT *y, TT *z, int yIsZ, Long yEws, Long zEws) {
+    lm::loadTables();
     typedef typename Compute<TT>::type C;
     const C twoPi = (C)(2.0 * 3.14159265358979323846);
     const C mean = c.args[0];
@@ -292,6 +294,7 @@ __global__ void __launch_bounds__(kBlock) gaussianKernel(RandomCtx<TT> c, const 
 template <typename TT>
 __global__ void __launch_bounds__(kBlock) truncatedNormalKernel(RandomCtx<TT> c, const TT *y, TT *z, int yIsZ, Long yEws,
                                                                 Long zEws) {
+    lm::loadTables();
     typedef typename Compute<TT>::type C;
     const C twoPi = (C)(2.0 * 3.14159265358979323846);
     const C mean = c.args[0];
@@ -324,6 +327,7 @@ __global__ void __launch_bounds__(kBlock) truncatedNormalKernel(RandomCtx<TT> c,
 // Binomial (405-520): trials draws at index (e+1)*t; probabilities args[1] or y[t-1] (EX: y[e], 531-650).
 template <typename TT, bool EX>
 __global__ void __launch_bounds__(kBlock) binomialKernel(RandomCtx<TT> c, const TT *y, TT *z, int yIsZ, Long yEws, Long zEws) {
+    lm::loadTables();
     typedef typename Compute<TT>::type C;
     const int trials = m::toIntX86(c.args[0]);
     const Long stride = (Long)gridDim.x * kBlock;
@@ -344,6 +348,7 @@ template <typename TT>
 __global__ void __launch_bounds__(kBlock) choiceKernel(RandomCtx<TT> c, const TT *x, const TT *y, TT *z, int strided,
                                                        Long xEws, Long yEws, Long zEws, DimMap xm, DimMap ym, DimMap zm,
                                                        Long yLength) {
+    lm::loadTables();
     typedef typename Compute<TT>::type C;
     const Long stride = (Long)gridDim.x * kBlock;
     for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < c.length; i += stride) {

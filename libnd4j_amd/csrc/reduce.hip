@@ -78,6 +78,9 @@ template <typename TT, int OP> struct ReducePol {
     typedef TT T;
     typedef typename Compute<TT>::type C;
     typedef C Acc;
+    // ops whose functor or post-processing evaluates exp / log / pow (variance and standard deviation square their
+    // bias term with pow); 20-23 have no functor
+    static constexpr bool tables = OP == 9 || OP == 10 || (OP >= 16 && OP <= 24);
     Params<TT> p;
     const TT *shiftSource;  // LogSumExp: per-TAD (TAD calls) or single (scalar calls) maximum; else null
     int shiftPerTad;

@@ -107,6 +107,7 @@ __device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc
 template <class Pol, int GROUP>
 __global__ void __launch_bounds__(kBlock) tadRowKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
                                                        const Long *offsets, Long tadLength, Long numTads) {
+    if (Pol::tables) lm::loadTables();
     typedef typename Pol::Acc Acc;
     constexpr int GROUPS = kBlock / GROUP;
     __shared__ Acc smem[kBlock / kWave];
@@ -136,6 +137,7 @@ template <class Pol>
 __global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
                                                        typename Pol::Acc *partials, const Long *offsets, Long tadLength,
                                                        Long numTads, Long tadEws, Long rowsPerSplit) {
+    if (Pol::tables) lm::loadTables();
     typedef typename Pol::Acc Acc;
     const Long t = (Long)blockIdx.x * kBlock + threadIdx.x;
     if (t >= numTads) return;
@@ -168,6 +170,7 @@ template <class Pol>
 __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
                                                           typename Pol::Acc *partials, const Long *offsets, Long tadLength,
                                                           Long numTads, Long tadEws, Long rowsPerSplit) {
+    if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
     constexpr int VEC = Pack<T>::N;
@@ -244,6 +247,7 @@ template <class Pol>
 __global__ void __launch_bounds__(kBlock) tadColFinish(Pol pol, typename Pol::T *z,
                                                        const typename Pol::Acc *__restrict__ partials, Long tadLength,
                                                        Long numTads, int splits) {
+    if (Pol::tables) lm::loadTables();
     typedef typename Pol::Acc Acc;
     constexpr int GROUPS = kBlock / kWave;
     __shared__ Acc smem[kBlock];
@@ -268,6 +272,7 @@ __global__ void __launch_bounds__(kBlock) tadColFinish(Pol pol, typename Pol::T 
 template <class Pol>
 __global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
                                                            const Long *offsets, DimMap tm, Long tadLength, Long numTads) {
+    if (Pol::tables) lm::loadTables();
     typedef typename Pol::Acc Acc;
     __shared__ Acc smem[kBlock / kWave];
     for (Long r = blockIdx.x; r < numTads; r += gridDim.x) {
@@ -285,6 +290,7 @@ __global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typena
 template <class Pol>
 __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol::T *x, typename Pol::Acc *partials,
                                                      Long n, int strided, Long ews, DimMap xm) {
+    if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
     __shared__ Acc smem[kBlock / kWave];
@@ -336,6 +342,7 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
 template <class Pol>
 __global__ void __launch_bounds__(kBlock) flatFinish(Pol pol, const typename Pol::T *x, typename Pol::T *z,
                                                      const typename Pol::Acc *partials, int count, Long n) {
+    if (Pol::tables) lm::loadTables();
     typedef typename Pol::Acc Acc;
     __shared__ Acc smem[kBlock / kWave];
     pol.setTad(0, nullptr);

@@ -33,8 +33,11 @@ template <typename C> __device__ __forceinline__ C laneBroadcast(C v, int srcLan
 }
 
 // MODE 0: softmax, 1: softmax * (1 - softmax), 2: log(softmax)
-template <int MODE, typename C> __device__ __forceinline__ C softmaxFinish(C e, C sum) {
-    C v = e / sum;
+// `inv` is 1 / sum, taken once per row: multiplying by it is within 1 ULP of dividing every element by the sum (what
+// the reference's loops say; its build allows the compiler the same substitution), far inside the tolerance that the
+// re-associated row sum already needs
+template <int MODE, typename C> __device__ __forceinline__ C softmaxFinish(C e, C inv) {
+    C v = e * inv;
     if (MODE == 1) return v * ((C)1 - v);
     if (MODE == 2) return m::log_(v);
     return v;
@@ -44,6 +47,7 @@ template <int MODE, typename C> __device__ __forceinline__ C softmaxFinish(C e, 
 template <typename T, int MODE, int GROUP>
 __global__ void __launch_bounds__(kBlock) softmaxRowKernel(const T *x, T *z, Long numRows, Long length, Long xRow, Long xEl,
                                                            Long zRow, Long zEl) {
+    lm::loadTables();
     typedef typename Compute<T>::type C;
     constexpr int GROUPS = kBlock / GROUP;
     __shared__ C smem[kBlock / kWave];
@@ -85,6 +89,7 @@ __global__ void __launch_bounds__(kBlock) softmaxRowKernel(const T *x, T *z, Lon
             sum = waveMerge<SumMerge<C>, GROUP>(mg, sum);
             sum = laneBroadcast(sum, 0, GROUP);
         }
+        sum = (C)1 / sum;
         if (live)
             for (Long c = lane; c < length; c += GROUP)
                 zr[c * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(xr[c * xEl]) - mx), sum));
@@ -97,6 +102,7 @@ __global__ void __launch_bounds__(kBlock) softmaxRowKernel(const T *x, T *z, Lon
 template <typename T, int MODE>
 __global__ void __launch_bounds__(kBlock) softmaxColKernel(const T *x, T *z, Long numRows, Long length, Long xRow, Long xEl,
                                                            Long zRow, Long zEl) {
+    lm::loadTables();
     typedef typename Compute<T>::type C;
     constexpr int WAVES = kBlock / kWave;
     __shared__ C smem[WAVES][kWave];
@@ -135,6 +141,7 @@ __global__ void __launch_bounds__(kBlock) softmaxColKernel(const T *x, T *z, Lon
     sum = (C)0;
 #pragma unroll
     for (int w = 0; w < WAVES; w++) sum += smem[w][lane];
+    sum = (C)1 / sum;
     if (live) {
         Long c = wave;
         for (; c + 3 * WAVES < length; c += 4 * WAVES) {
@@ -149,8 +156,211 @@ __global__ void __launch_bounds__(kBlock) softmaxColKernel(const T *x, T *z, Lon
     }
 }
 
+template <typename C> __device__ __forceinline__ C laneXor(C v, int mask) {
+    static_assert(sizeof(C) % 4 == 0, "compute type is a multiple of 4 bytes");
+    constexpr int W = sizeof(C) / 4;
+    struct Words { int w[W]; };
+    Words in = __builtin_bit_cast(Words, v), out;
+#pragma unroll
+    for (int i = 0; i < W; i++) out.w[i] = __shfl_xor(in.w[i], mask);
+    return __builtin_bit_cast(C, out);
+}
+
+// Every lane of a GROUP-lane team (a part of a wave, a wave, or the whole block) gets the merged value.
+template <class Merge, int GROUP, typename C> __device__ __forceinline__ C teamAll(C v, C *smem) {
+    Merge mg;
+    constexpr int W = GROUP < kWave ? GROUP : kWave;
+#pragma unroll
+    for (int d = W / 2; d >= 1; d >>= 1) v = mg.combine(v, laneXor(v, d));
+    if (GROUP > kWave) {
+        const int wave = threadIdx.x / kWave;
+        __syncthreads();  // smem may still be read from the previous merge
+        if (threadIdx.x % kWave == 0) smem[wave] = v;
+        __syncthreads();
+        v = smem[0];
+#pragma unroll
+        for (int w = 1; w < GROUP / kWave; w++) v = mg.combine(v, smem[w]);
+    }
+    return v;
+}
+
+// Contiguous rows short enough to stay in registers: GROUP lanes own a row and keep PACKS 16-byte vectors of it
+// each (vector j of a lane is vector lane + j * GROUP of the row), so x is read once and z written once.  exp(x - max)
+// replaces x in the registers (rounded to T, which only matters for half).
+template <typename T, int MODE, int GROUP, int PACKS>
+__global__ void __launch_bounds__(kBlock) softmaxRowRegKernel(const T *x, T *z, Long numRows, Long npack, Long xRow, Long zRow) {
+    lm::loadTables();
+    typedef typename Compute<T>::type C;
+    constexpr int N = Pack<T>::N;
+    constexpr int GROUPS = kBlock / GROUP;
+    __shared__ C smem[kBlock / kWave];
+    const int g = threadIdx.x / GROUP, lane = threadIdx.x % GROUP;
+    // GROUP == kBlock: every thread of the block runs the same trip count, so teamAll may synchronise
+    for (Long r0 = (Long)blockIdx.x * GROUPS; r0 < numRows; r0 += (Long)gridDim.x * GROUPS) {
+        const Long r = r0 + g;
+        const bool live = r < numRows;
+        const Pack<T> *xr = reinterpret_cast<const Pack<T> *>(x + (live ? r * xRow : 0));
+        Pack<T> *zr = reinterpret_cast<Pack<T> *>(z + (live ? r * zRow : 0));
+        Pack<T> cache[PACKS];
+#pragma unroll
+        for (int j = 0; j < PACKS; j++)
+            if (live && lane + j * GROUP < npack) cache[j] = loadPack(xr + lane + j * GROUP);
+        C mx = (C)-3.4028235e38;
+#pragma unroll
+        for (int j = 0; j < PACKS; j++)
+            if (live && lane + j * GROUP < npack) {
+#pragma unroll
+                for (int e = 0; e < N; e++) mx = m::max_(mx, toCompute(cache[j].v[e]));
+            }
+        mx = teamAll<MaxMerge<C>, GROUP>(mx, smem);
+        C sum = (C)0;
+#pragma unroll
+        for (int j = 0; j < PACKS; j++)
+            if (live && lane + j * GROUP < npack) {
+#pragma unroll
+                for (int e = 0; e < N; e++) {
+                    const C ex = m::exp_(toCompute(cache[j].v[e]) - mx);
+                    sum += ex;
+                    cache[j].v[e] = fromCompute<T>(ex);
+                }
+            }
+        sum = teamAll<SumMerge<C>, GROUP>(sum, smem);
+        sum = (C)1 / sum;
+#pragma unroll
+        for (int j = 0; j < PACKS; j++)
+            if (live && lane + j * GROUP < npack) {
+                Pack<T> o;
+#pragma unroll
+                for (int e = 0; e < N; e++) o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(toCompute(cache[j].v[e]), sum));
+                storePack(zr + lane + j * GROUP, o);
+            }
+    }
+}
+
+// Rows adjacent in memory (an f-order matrix) and at most kColCols * PACKS columns: a 1024-thread block owns
+// 8 * Pack::N neighbouring rows - eight row lanes, each loading Pack::N rows of one column as one 16-byte vector,
+// times 128 column groups - and keeps all of it in registers (PACKS vectors a thread).  Row maxima and sums are
+// merged over the column groups with three butterfly steps inside a wave and through LDS across the 16 waves.
+static constexpr int kColBlock = 1024, kColRowLanes = 8, kColCols = kColBlock / kColRowLanes;
+template <typename T, int MODE, int PACKS>
+__global__ void __launch_bounds__(kColBlock) softmaxColRegKernel(const T *x, T *z, Long numRows, Long length, Long xEl, Long zEl) {
+    lm::loadTables();
+    typedef typename Compute<T>::type C;
+    constexpr int N = Pack<T>::N;
+    constexpr int WAVES = kColBlock / kWave;
+    __shared__ C smax[WAVES][kColRowLanes][N], ssum[WAVES][kColRowLanes][N];
+    const int rl = threadIdx.x % kColRowLanes, cg = threadIdx.x / kColRowLanes;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const Long row0 = ((Long)blockIdx.x * kColRowLanes + rl) * N;  // numRows is a multiple of N: a vector is all live or all dead
+    const bool live = row0 < numRows;
+    Pack<T> cache[PACKS];
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (live && cg + j * kColCols < length) cache[j] = loadPack(reinterpret_cast<const Pack<T> *>(x + row0 + (Long)(cg + j * kColCols) * xEl));
+    C mx[N], sum[N];
+#pragma unroll
+    for (int e = 0; e < N; e++) mx[e] = (C)-3.4028235e38;
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (live && cg + j * kColCols < length) {
+#pragma unroll
+            for (int e = 0; e < N; e++) mx[e] = m::max_(mx[e], toCompute(cache[j].v[e]));
+        }
+#pragma unroll
+    for (int d = kColRowLanes; d < kWave; d <<= 1) {
+#pragma unroll
+        for (int e = 0; e < N; e++) mx[e] = m::max_(mx[e], laneXor(mx[e], d));
+    }
+    if (lane < kColRowLanes) {
+#pragma unroll
+        for (int e = 0; e < N; e++) smax[wave][lane][e] = mx[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < WAVES; w++) {
+#pragma unroll
+        for (int e = 0; e < N; e++) mx[e] = m::max_(mx[e], smax[w][rl][e]);
+    }
+#pragma unroll
+    for (int e = 0; e < N; e++) sum[e] = (C)0;
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (live && cg + j * kColCols < length) {
+#pragma unroll
+            for (int e = 0; e < N; e++) {
+                const C ex = m::exp_(toCompute(cache[j].v[e]) - mx[e]);
+                sum[e] += ex;
+                cache[j].v[e] = fromCompute<T>(ex);
+            }
+        }
+#pragma unroll
+    for (int d = kColRowLanes; d < kWave; d <<= 1) {
+#pragma unroll
+        for (int e = 0; e < N; e++) sum[e] += laneXor(sum[e], d);
+    }
+    if (lane < kColRowLanes) {
+#pragma unroll
+        for (int e = 0; e < N; e++) ssum[wave][lane][e] = sum[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < N; e++) sum[e] = ssum[0][rl][e];
+#pragma unroll
+    for (int w = 1; w < WAVES; w++) {
+#pragma unroll
+        for (int e = 0; e < N; e++) sum[e] += ssum[w][rl][e];
+    }
+#pragma unroll
+    for (int e = 0; e < N; e++) sum[e] = (C)1 / sum[e];
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (live && cg + j * kColCols < length) {
+            Pack<T> o;
+#pragma unroll
+            for (int e = 0; e < N; e++) o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(toCompute(cache[j].v[e]), sum[e]));
+            storePack(reinterpret_cast<Pack<T> *>(z + row0 + (Long)(cg + j * kColCols) * zEl), o);
+        }
+}
+
+template <typename T> static bool aligned16(const T *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <typename T, int MODE, int GROUP, int PACKS> void runRowReg(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
+    int grid = gridFor(pl.numRows, kBlock / GROUP, kMaxGrid);
+    hipLaunchKernelGGL((softmaxRowRegKernel<T, MODE, GROUP, PACKS>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows,
+                       pl.length / Pack<T>::N, pl.xRow, pl.zRow);
+}
+template <typename T, int MODE, int PACKS> void runColReg(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
+    const Long rowsPerBlock = (Long)kColRowLanes * Pack<T>::N;
+    int grid = (int)((pl.numRows + rowsPerBlock - 1) / rowsPerBlock);
+    hipLaunchKernelGGL((softmaxColRegKernel<T, MODE, PACKS>), dim3(grid), dim3(kColBlock), 0, s, x, z, pl.numRows, pl.length, pl.xEl,
+                       pl.zEl);
+}
+
 template <typename T, int MODE> void runSoftmax(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
     if (pl.numRows <= 0 || pl.length <= 0) return;
+    constexpr int N = Pack<T>::N;
+    // vectors a thread of the neighbouring-rows kernel may hold: a half vector unpacks to eight float maxima and
+    // sums, which leaves room for fewer of them
+    constexpr int kColPacks = sizeof(T) == 2 ? 8 : 16;
+    const bool base16 = aligned16(x) && aligned16(z);
+    // rows in registers: contiguous rows whose vectors are aligned in every row
+    if (base16 && pl.xEl == 1 && pl.zEl == 1 && pl.length % N == 0 && pl.length >= 16 * N &&
+        (pl.numRows == 1 || (pl.xRow % N == 0 && pl.zRow % N == 0))) {
+        const Long npack = pl.length / N;
+        if (npack <= 16 * 2) { runRowReg<T, MODE, 16, 2>(s, x, z, pl); return; }
+        if (npack <= 64 * 2) { runRowReg<T, MODE, 64, 2>(s, x, z, pl); return; }
+        if (npack <= 64 * 8) { runRowReg<T, MODE, 64, 8>(s, x, z, pl); return; }
+        if (npack <= 256 * 4) { runRowReg<T, MODE, kBlock, 4>(s, x, z, pl); return; }
+        if (npack <= 256 * 16) { runRowReg<T, MODE, kBlock, 16>(s, x, z, pl); return; }
+    }
+    // neighbouring rows in registers: an f-order matrix whose column stride keeps the row vectors aligned
+    if (base16 && pl.xRow == 1 && pl.zRow == 1 && pl.numRows % N == 0 && pl.xEl % N == 0 && pl.zEl % N == 0 &&
+        pl.numRows >= kWave && pl.length <= (Long)kColCols * kColPacks && (Long)((pl.numRows + 8 * N - 1) / (8 * N)) <= kMaxGrid) {
+        if (pl.length <= (Long)kColCols * 2) runColReg<T, MODE, 2>(s, x, z, pl);
+        else if (pl.length <= (Long)kColCols * kColPacks / 2) runColReg<T, MODE, kColPacks / 2>(s, x, z, pl);
+        else runColReg<T, MODE, kColPacks>(s, x, z, pl);
+        return;
+    }
     if (pl.xRow == 1 && pl.zRow == 1 && pl.numRows >= kWave) {
         int grid = (int)((pl.numRows + kWave - 1) / kWave);
         hipLaunchKernelGGL((softmaxColKernel<T, MODE>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows, pl.length, pl.xRow, pl.xEl,
@@ -204,6 +414,47 @@ __global__ void __launch_bounds__(kBlock) isMaxTadFillKernel(T *z, const T *inde
     }
 }
 
+// TADs with contiguous elements: GROUP lanes write one TAD, with 16-byte stores where the TAD allows them
+template <typename T, int GROUP>
+__global__ void __launch_bounds__(kBlock) isMaxRowFillKernel(T *z, const T *index, const Long *offsets, Long tadLength, Long numTads) {
+    typedef typename Compute<T>::type C;
+    constexpr int N = Pack<T>::N;
+    constexpr int GROUPS = kBlock / GROUP;
+    const int g = threadIdx.x / GROUP, lane = threadIdx.x % GROUP;
+    const T one = fromCompute<T>((C)1), zero = fromCompute<T>((C)0);
+    for (Long r = (Long)blockIdx.x * GROUPS + g; r < numTads; r += (Long)gridDim.x * GROUPS) {
+        T *zr = z + offsets[r];
+        const Long hit = (Long)toCompute(index[r]);
+        if ((reinterpret_cast<uintptr_t>(zr) & 15) == 0 && tadLength % N == 0) {
+            Pack<T> *zv = reinterpret_cast<Pack<T> *>(zr);
+            for (Long p = lane; p < tadLength / N; p += GROUP) {
+                Pack<T> o;
+#pragma unroll
+                for (int e = 0; e < N; e++) o.v[e] = (p * N + e == hit) ? one : zero;
+                storePack(zv + p, o);
+            }
+        } else {
+            for (Long f = lane; f < tadLength; f += GROUP) zr[f] = (f == hit) ? one : zero;
+        }
+    }
+}
+// TADs whose elements are tadEws apart: thread <-> TAD (neighbouring TADs are neighbours in memory for the usual
+// layouts), blockIdx.y splits the TAD's elements
+template <typename T>
+__global__ void __launch_bounds__(kBlock) isMaxColFillKernel(T *z, const T *index, const Long *offsets, Long tadLength, Long numTads,
+                                                             Long tadEws, Long perSplit) {
+    typedef typename Compute<T>::type C;
+    const Long t = (Long)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= numTads) return;
+    const T one = fromCompute<T>((C)1), zero = fromCompute<T>((C)0);
+    T *zt = z + offsets[t];
+    const Long hit = (Long)toCompute(index[t]);
+    const Long f0 = (Long)blockIdx.y * perSplit;
+    Long f1 = f0 + perSplit;
+    if (f1 > tadLength) f1 = tadLength;
+    for (Long f = f0; f < f1; f++) zt[f * tadEws] = (f == hit) ? one : zero;
+}
+
 template <typename T> void launchIsMaxFill(hipStream_t s, T *z, const T *index, const FlatPlan &zp) {
     if (zp.n <= 0) return;
     int grid = gridFor(zp.n, kBlock * 4, kGridCap);
@@ -211,6 +462,32 @@ template <typename T> void launchIsMaxFill(hipStream_t s, T *z, const T *index, 
 }
 template <typename T> void launchIsMaxTadFill(hipStream_t s, T *z, const T *index, const TadPlan &zt) {
     if (zt.numTads <= 0 || zt.tadLength <= 0) return;
+    if (zt.kind == TadPlan::ROW) {
+        if (zt.tadLength >= 2048) {
+            hipLaunchKernelGGL((isMaxRowFillKernel<T, kBlock>), dim3(gridFor(zt.numTads, 1, kMaxGrid)), dim3(kBlock), 0, s, z, index,
+                               zt.offsets, zt.tadLength, zt.numTads);
+        } else if (zt.tadLength >= 256) {
+            hipLaunchKernelGGL((isMaxRowFillKernel<T, 64>), dim3(gridFor(zt.numTads, kBlock / 64, kMaxGrid)), dim3(kBlock), 0, s, z,
+                               index, zt.offsets, zt.tadLength, zt.numTads);
+        } else {
+            hipLaunchKernelGGL((isMaxRowFillKernel<T, 16>), dim3(gridFor(zt.numTads, kBlock / 16, kMaxGrid)), dim3(kBlock), 0, s, z,
+                               index, zt.offsets, zt.tadLength, zt.numTads);
+        }
+        return;
+    }
+    if (zt.kind == TadPlan::COL && zt.numTads >= kBlock) {
+        const Long gx = (zt.numTads + kBlock - 1) / kBlock;
+        Long splits = (4096 + gx - 1) / gx;  // enough blocks to fill the chip
+        if (splits > zt.tadLength) splits = zt.tadLength;
+        if (splits > 65535) splits = 65535;
+        const Long per = (zt.tadLength + splits - 1) / splits;
+        splits = (zt.tadLength + per - 1) / per;
+        if (gx <= kMaxGrid) {
+            hipLaunchKernelGGL((isMaxColFillKernel<T>), dim3((unsigned)gx, (unsigned)splits), dim3(kBlock), 0, s, z, index, zt.offsets,
+                               zt.tadLength, zt.numTads, zt.tadEws, per);
+            return;
+        }
+    }
     int grid = gridFor(zt.numTads * zt.tadLength, kBlock * 4, kGridCap);
     hipLaunchKernelGGL((isMaxTadFillKernel<T>), dim3(grid), dim3(kBlock), 0, s, z, index, zt.offsets, zt.tadLength, zt.numTads,
                        zt.kind == TadPlan::GENERAL ? 0 : 1, zt.tadEws, zt.tm);

@@ -40,6 +40,7 @@ template <typename TT, int OP> struct StatsPol {
     typedef TT T;
     typedef typename Compute<TT>::type C;
     typedef StatsAcc Acc;
+    static constexpr bool tables = false;  // no exp / log / pow in these accumulators
     int biasCorrected;
     int phantomZero;  // the reference's single-dimension non-EWS branch starts from a zero sample
 

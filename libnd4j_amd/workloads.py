@@ -16,6 +16,7 @@ F32 = np.float32
 
 # opNums (reference: include/loops/legacy_ops.h)
 T_EXP, T_TANH = 3, 15
+T_SOFTMAX, T_LOGSOFTMAX, T_ISMAX = 38, 40, 41
 P_ADD, P_MUL = 0, 6
 S_MUL = 2  # scalar family
 B_ADD, B_SUB, B_DIV = 0, 1, 3
@@ -281,6 +282,7 @@ def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
     tad1, tad0 = dev.tad(xi, [1]), dev.tad(xi, [0])
     ri = _vec(rows)
     ci = harness.shape_info([rows, 1])
+    xci = harness.shape_info([rows, cols], "c")
     mc, sc, tc = np.zeros(rows, F32), np.zeros(rows, F32), np.zeros(n, F32)
     host_out = {(dim, out_len): np.zeros(out_len, F32) for dim, out_len in ((1, rows), (0, cols))}
 
@@ -340,6 +342,32 @@ def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
             return tc
 
         cases.append(Case("softmax_chain", "chain", n, sum(st[2] for st in steps), chain_gpu, chain_cpu, False, T.get))
+
+        # the same softmax as ONE call (transform opNum 38), on the f-order matrix and on the same memory read as a
+        # c-order [rows, cols] matrix (rows contiguous); IsMax over the whole array and along dimension 1
+        XCI = w.raw(np.ascontiguousarray(xci, dtype=np.int64))
+        ex_c = dev.extra(xci, z_info=xci)
+        cases.append(Case("softmax_fused_forder", "special", n, 8 * n,
+                          lambda: ops.execTransformFloat(ex_t, T_SOFTMAX, X.ptr, X.info_ptr, T.ptr, T.info_ptr, None),
+                          lambda lib: (lib.transform(T_SOFTMAX, x, xi, tc, xi, None), tc)[1], False, T.get))
+        cases.append(Case("softmax_fused_corder", "special", n, 8 * n,
+                          lambda: ops.execTransformFloat(ex_c, T_SOFTMAX, X.ptr, XCI.ptr, T.ptr, XCI.ptr, None),
+                          lambda lib: (lib.transform(T_SOFTMAX, x, xci, tc, xci, None), tc)[1], True, T.get))
+        cases.append(Case("logsoftmax_fused_corder", "special", n, 8 * n,
+                          lambda: ops.execTransformFloat(ex_c, T_LOGSOFTMAX, X.ptr, XCI.ptr, T.ptr, XCI.ptr, None),
+                          lambda lib: (lib.transform(T_LOGSOFTMAX, x, xci, tc, xci, None), tc)[1], True, T.get))
+        cases.append(Case("ismax_whole", "special", n, 8 * n,
+                          lambda: ops.execTransformFloat(ex_c, T_ISMAX, X.ptr, XCI.ptr, T.ptr, XCI.ptr, None),
+                          lambda lib: (lib.transform(T_ISMAX, x, xci, tc, xci, None), tc)[1], True, T.get))
+        DM = w.raw(np.array([1], np.int32))
+        EP = w.raw(np.array([1, 1], F32))
+        ex_m = dev.extra(xci, z_info=xci)
+        ex_m[15] = DM.ptr
+        ex_m[18] = 1
+        ismax_params = np.array([1, 1], F32)
+        cases.append(Case("ismax_dim1", "special", n, 8 * n,
+                          lambda: ops.execTransformFloat(ex_m, T_ISMAX, X.ptr, XCI.ptr, T.ptr, XCI.ptr, EP.ptr),
+                          lambda lib: (lib.transform(T_ISMAX, x, xci, tc, xci, ismax_params), tc)[1], True, T.get))
         return cases
 
     return _replicated(dev, "summary stats var/std + softmax-style chain; fp32 [%d,%d] f-order" % (rows, cols), 8 * n,
