@@ -355,7 +355,8 @@ inline void launchStrided(hipStream_t s, const T *x, Long xs, const T *y, Long y
         if (head >= 0) {
             if (head > n) head = (int)n;
             Long nvec = (n - head) / Pack<T>::N;
-            int grid = gridFor(nvec > 0 ? nvec : 1, (Long)kBlock, kMaxGrid);
+            // kernels that stage the lookup tables run several passes per block, so the staging is paid less often
+            int grid = gridFor(nvec > 0 ? nvec : 1, (Long)kBlock, F::tables ? kGridCap : kMaxGrid);
             hipLaunchKernelGGL((ewVecKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, two ? y : x, z, p, n, head,
                                (two && ys == 0) ? 1 : 0);
             return;
