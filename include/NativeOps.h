@@ -103,6 +103,28 @@
 // Reduce3 family (two inputs, one number per pair of runs), reference: blas/NativeOps.h:919-1044 (Float / Half),
 // 252-362 (Double and the all-pairs variant): whole arrays into result[0], whole arrays returned by value,
 // along `dimension`, and every TAD of x against every TAD of y.
+// Data-movement specials, reference: blas/NativeOps.h:1457-1499 (flatten), 1510-1555 (concat), 1904-1967
+// (pullRows), 2076-2130 (shuffle), 2876-2899 (tear).  Pointer conventions of the CUDA back end: concat takes
+// data[0] / inputShapeInfo[0] = device tables of device pointers, the result's host shapeInfo in extraPointers[0]
+// and (optionally) a host table of the inputs' host shapeInfos in extraPointers[9]; tadPointers / offsetPointers
+// are accepted and not needed.  flatten takes the input's host shapeInfo in extraPointers[7].  For pullRows, tear
+// and shuffle every argument, the tables of pointers included, is a device pointer.  shuffle swaps TAD r with TAD
+// shuffleMap[r] (entries < 0 are skipped; the pairs of one map must be disjoint) in each of the N arrays.
+#define ND4J_SPECIAL_MEMBERS(SUFFIX, T)                                                                          \
+    void flatten##SUFFIX(Nd4jPointer *extraPointers, int offset, char order, T *result, Nd4jLong *resultShapeInfo, \
+                         T *input, Nd4jLong *inputShapeInfo);                                                    \
+    void concat##SUFFIX(Nd4jPointer *extraPointers, int dimension, int numArrays, Nd4jPointer *data,             \
+                        Nd4jPointer *inputShapeInfo, T *result, Nd4jLong *resultShapeInfo,                       \
+                        Nd4jPointer *tadPointers, Nd4jPointer *offsetPointers);                                  \
+    void pullRows##SUFFIX(Nd4jPointer *extraPointers, T *x, Nd4jLong *xShapeInfo, T *z, Nd4jLong *zShapeInfo,    \
+                          Nd4jLong n, Nd4jLong *indexes, Nd4jLong *tadShapeInfo, Nd4jLong *tadOffsets,           \
+                          Nd4jLong *zTadShapeInfo, Nd4jLong *zTadOffsets);                                       \
+    void tear##SUFFIX(Nd4jPointer *extraPointers, T *x, Nd4jLong *xShapeInfo, Nd4jPointer *targets,              \
+                      Nd4jLong *zShapeInfo, Nd4jLong *tadShapeInfo, Nd4jLong *tadOffsets);                       \
+    void shuffle##SUFFIX(Nd4jPointer *extras, Nd4jPointer *dx, Nd4jPointer *xShapeInfo, Nd4jPointer *dz,         \
+                         Nd4jPointer *zShapeInfo, int N, int *shuffleMap, Nd4jPointer *tadShapeInfo,             \
+                         Nd4jPointer *tadOffsets);
+
 #define ND4J_REDUCE3_MEMBERS(SUFFIX, T, R)                                                                      \
     void execReduce3##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *x, Nd4jLong *xShapeInfo,                 \
                              T *extraParamsVals, T *y, Nd4jLong *yShapeInfo, T *result,                          \
@@ -127,6 +149,13 @@ public:
     ND4J_SCALAR_MEMBERS(Float, float, float)
     ND4J_SCALAR_MEMBERS(Half, float16, float)
     ND4J_SCALAR_MEMBERS(Double, double, double)
+
+    ND4J_SPECIAL_MEMBERS(Float, float)
+    ND4J_SPECIAL_MEMBERS(Half, float16)
+    ND4J_SPECIAL_MEMBERS(Double, double)
+    // z[i] = (dst)(float)x[i] between device buffers; srcType / dstType 3 half, 6 float, 7 double
+    // (reference: blas/NativeOps.h:2144, include/loops/type_conversions.h:11-18)
+    void convertTypes(Nd4jPointer *extras, int srcType, Nd4jPointer x, Nd4jLong N, int dstType, Nd4jPointer z);
 
     ND4J_EXEC_MEMBERS(Float, float, float)
     ND4J_EXEC_MEMBERS(Half, float16, float)
@@ -186,3 +215,4 @@ public:
 #undef ND4J_EXEC_MEMBERS
 #undef ND4J_SCALAR_MEMBERS
 #undef ND4J_REDUCE3_MEMBERS
+#undef ND4J_SPECIAL_MEMBERS

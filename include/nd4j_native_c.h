@@ -128,6 +128,28 @@ ND4J_C_REDUCE3(Half, float16, float)
 ND4J_C_REDUCE3(Double, double, double)
 #undef ND4J_C_REDUCE3
 
+/* Data-movement specials (blas/NativeOps.h:1457-1499 flatten, 1510-1555 concat, 1904-1967 pullRows, 2076-2130
+ * shuffle, 2876-2899 tear, 2144 convertTypes); pointer conventions as documented in include/NativeOps.h. */
+#define ND4J_C_SPECIAL(SUFFIX, T)                                                                                \
+    void nd4j_flatten##SUFFIX(Nd4jPointer *extraPointers, int offset, char order, T *result,                     \
+                              Nd4jLong *resultShapeInfo, T *input, Nd4jLong *inputShapeInfo);                    \
+    void nd4j_concat##SUFFIX(Nd4jPointer *extraPointers, int dimension, int numArrays, Nd4jPointer *data,        \
+                             Nd4jPointer *inputShapeInfo, T *result, Nd4jLong *resultShapeInfo,                  \
+                             Nd4jPointer *tadPointers, Nd4jPointer *offsetPointers);                             \
+    void nd4j_pullRows##SUFFIX(Nd4jPointer *extraPointers, T *x, Nd4jLong *xShapeInfo, T *z,                     \
+                               Nd4jLong *zShapeInfo, Nd4jLong n, Nd4jLong *indexes, Nd4jLong *tadShapeInfo,      \
+                               Nd4jLong *tadOffsets, Nd4jLong *zTadShapeInfo, Nd4jLong *zTadOffsets);            \
+    void nd4j_tear##SUFFIX(Nd4jPointer *extraPointers, T *x, Nd4jLong *xShapeInfo, Nd4jPointer *targets,         \
+                           Nd4jLong *zShapeInfo, Nd4jLong *tadShapeInfo, Nd4jLong *tadOffsets);                  \
+    void nd4j_shuffle##SUFFIX(Nd4jPointer *extras, Nd4jPointer *dx, Nd4jPointer *xShapeInfo, Nd4jPointer *dz,    \
+                              Nd4jPointer *zShapeInfo, int N, int *shuffleMap, Nd4jPointer *tadShapeInfo,        \
+                              Nd4jPointer *tadOffsets);
+ND4J_C_SPECIAL(Float, float)
+ND4J_C_SPECIAL(Half, float16)
+ND4J_C_SPECIAL(Double, double)
+#undef ND4J_C_SPECIAL
+void nd4j_convertTypes(Nd4jPointer *extras, int srcType, Nd4jPointer x, Nd4jLong N, int dstType, Nd4jPointer z);
+
 Nd4jPointer nd4j_initRandom(Nd4jPointer *extraPointers, long seed, long bufferSize, Nd4jPointer ptrToBuffer);
 void nd4j_refreshBuffer(Nd4jPointer *extraPointers, long seed, Nd4jPointer ptrRandom);
 void nd4j_reSeedBuffer(Nd4jPointer *extraPointers, long seed, Nd4jPointer ptrRandom);

@@ -149,6 +149,34 @@ ND4J_C_REDUCE3(Half, float16, float)
 ND4J_C_REDUCE3(Double, double, double)
 #undef ND4J_C_REDUCE3
 
+#define ND4J_C_SPECIAL(SUFFIX, T)                                                                                  \
+    void nd4j_flatten##SUFFIX(Nd4jPointer *e, int offset, char order, T *r, Nd4jLong *rs, T *in, Nd4jLong *is) {   \
+        guardVoid([&] { gOps.flatten##SUFFIX(e, offset, order, r, rs, in, is); });                                 \
+    }                                                                                                              \
+    void nd4j_concat##SUFFIX(Nd4jPointer *e, int dim, int n, Nd4jPointer *data, Nd4jPointer *infos, T *r,          \
+                             Nd4jLong *rs, Nd4jPointer *tads, Nd4jPointer *offs) {                                 \
+        guardVoid([&] { gOps.concat##SUFFIX(e, dim, n, data, infos, r, rs, tads, offs); });                        \
+    }                                                                                                              \
+    void nd4j_pullRows##SUFFIX(Nd4jPointer *e, T *x, Nd4jLong *xs, T *z, Nd4jLong *zs, Nd4jLong n, Nd4jLong *idx,  \
+                               Nd4jLong *ti, Nd4jLong *to, Nd4jLong *zti, Nd4jLong *zto) {                         \
+        guardVoid([&] { gOps.pullRows##SUFFIX(e, x, xs, z, zs, n, idx, ti, to, zti, zto); });                      \
+    }                                                                                                              \
+    void nd4j_tear##SUFFIX(Nd4jPointer *e, T *x, Nd4jLong *xs, Nd4jPointer *targets, Nd4jLong *zs, Nd4jLong *ti,   \
+                           Nd4jLong *to) {                                                                         \
+        guardVoid([&] { gOps.tear##SUFFIX(e, x, xs, targets, zs, ti, to); });                                      \
+    }                                                                                                              \
+    void nd4j_shuffle##SUFFIX(Nd4jPointer *e, Nd4jPointer *dx, Nd4jPointer *xs, Nd4jPointer *dz, Nd4jPointer *zs,  \
+                              int N, int *map, Nd4jPointer *ti, Nd4jPointer *to) {                                 \
+        guardVoid([&] { gOps.shuffle##SUFFIX(e, dx, xs, dz, zs, N, map, ti, to); });                               \
+    }
+ND4J_C_SPECIAL(Float, float)
+ND4J_C_SPECIAL(Half, float16)
+ND4J_C_SPECIAL(Double, double)
+#undef ND4J_C_SPECIAL
+void nd4j_convertTypes(Nd4jPointer *e, int st, Nd4jPointer x, Nd4jLong n, int dt, Nd4jPointer z) {
+    guardVoid([&] { gOps.convertTypes(e, st, x, n, dt, z); });
+}
+
 Nd4jPointer nd4j_initRandom(Nd4jPointer *e, long seed, long size, Nd4jPointer buf) {
     return guardRet<Nd4jPointer>(nullptr, [&] { return gOps.initRandom(e, seed, size, buf); });
 }

@@ -1,0 +1,333 @@
+// Data-movement specials: concat, pullRows, tear, shuffle and the float-type conversions.  (flatten needs no
+// kernel of its own: the host turns it into an Identity transform between two index maps.)
+// Reference: include/loops/special_kernels.h:140-360 (concat), 579-625 (pullRows), 824-874 (tear), 890-967
+// (shuffle), include/loops/type_conversions.h:38-49 (convert); CPU counterparts include/ops/impl/specials.cpp:17-200
+// and blas/cpu/NativeOps.cpp:2045-2160, 2266-2325.
+//
+// As in the reference's CUDA back end every pointer these calls receive - data, shapeInfo, TAD tables, and the
+// tables of such pointers - is a device pointer, so the kernels decode shapeInfo themselves.  All of them are pure
+// copies: 16-byte streaming accesses wherever source and destination runs are contiguous and equally aligned.
+#include "elementwise.cuh"
+#include "launch.h"
+#include "reduce_engine.cuh"
+
+namespace nd4j_amd {
+
+// ---- shapeInfo on the device: [rank, shape.., stride.., offset, ews, order] --------------------------------
+__device__ __forceinline__ int dRank(const Long *si) { return (int)si[0]; }
+__device__ __forceinline__ const Long *dShape(const Long *si) { return si + 1; }
+__device__ __forceinline__ const Long *dStride(const Long *si) { return si + 1 + si[0]; }
+__device__ __forceinline__ Long dEws(const Long *si) { return si[2 * si[0] + 2]; }
+__device__ __forceinline__ char dOrder(const Long *si) { return (char)si[2 * si[0] + 3]; }
+__device__ __forceinline__ Long dLength(const Long *si) {
+    Long n = 1;
+    for (int i = 0; i < (int)si[0]; i++) n *= si[1 + i];
+    return n;
+}
+// element offset of linear index i decomposed over the shape in C order / in F order (shape::ind2subC / ind2sub
+// followed by shape::getOffset)
+__device__ __forceinline__ Long dOffsetC(const Long *si, Long i) {
+    const int rank = dRank(si);
+    const Long *shape = dShape(si), *stride = dStride(si);
+    Long off = 0;
+    for (int d = rank - 1; d >= 0; d--) {
+        const Long q = i / shape[d];
+        off += (i - q * shape[d]) * stride[d];
+        i = q;
+    }
+    return off;
+}
+__device__ __forceinline__ Long dOffsetF(const Long *si, Long i) {
+    const int rank = dRank(si);
+    const Long *shape = dShape(si), *stride = dStride(si);
+    Long off = 0;
+    for (int d = 0; d < rank; d++) {
+        const Long q = i / shape[d];
+        off += (i - q * shape[d]) * stride[d];
+        i = q;
+    }
+    return off;
+}
+
+template <typename T> __device__ __forceinline__ bool sameAlignment(const T *a, const T *b) {
+    const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+    return (pa & 15) == (pb & 15) && (pa & (sizeof(T) - 1)) == 0;
+}
+
+// `lanes` cooperating lanes copy len elements from src to dst.  se / de: element-wise strides (>= 1) or, when
+// either is < 1, offsets come from the coordinate decomposition of the two shapeInfos (FORDER: ind2sub, else ind2subC).
+template <typename T, bool FORDER>
+__device__ __forceinline__ void copyRun(const T *src, Long se, const Long *sInfo, T *dst, Long de, const Long *dInfo, Long len,
+                                        int lane, int lanes) {
+    if (se == 1 && de == 1) {
+        constexpr int N = Pack<T>::N;
+        if (sameAlignment(src, dst)) {
+            Long head = (Long)(((16 - (reinterpret_cast<uintptr_t>(src) & 15)) & 15) / sizeof(T));
+            if (head > len) head = len;
+            for (Long i = lane; i < head; i += lanes) dst[i] = src[i];
+            const Long nvec = (len - head) / N;
+            const Pack<T> *sv = reinterpret_cast<const Pack<T> *>(src + head);
+            Pack<T> *dv = reinterpret_cast<Pack<T> *>(dst + head);
+            Long v = lane;
+            for (; v + 3 * (Long)lanes < nvec; v += 4 * (Long)lanes) {
+                Pack<T> p0 = loadPack(sv + v), p1 = loadPack(sv + v + lanes), p2 = loadPack(sv + v + 2 * lanes),
+                        p3 = loadPack(sv + v + 3 * lanes);
+                storePack(dv + v, p0);
+                storePack(dv + v + lanes, p1);
+                storePack(dv + v + 2 * lanes, p2);
+                storePack(dv + v + 3 * lanes, p3);
+            }
+            for (; v < nvec; v += lanes) storePack(dv + v, loadPack(sv + v));
+            for (Long i = head + nvec * N + lane; i < len; i += lanes) dst[i] = src[i];
+        } else {
+            for (Long i = lane; i < len; i += lanes) dst[i] = src[i];
+        }
+    } else if (se >= 1 && de >= 1) {
+        for (Long i = lane; i < len; i += lanes) dst[i * de] = src[i * se];
+    } else {
+        for (Long i = lane; i < len; i += lanes)
+            dst[FORDER ? dOffsetF(dInfo, i) : dOffsetC(dInfo, i)] = src[FORDER ? dOffsetF(sInfo, i) : dOffsetC(sInfo, i)];
+    }
+}
+
+// A block works on one long TAD or on four short ones (a wave each)
+__device__ __forceinline__ int lanesPerTad(Long tadLength) { return tadLength >= 1024 ? kBlock : kWave; }
+
+// ---- pullRows: z TAD idx <- x TAD indexes[idx] ---------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(kBlock) pullRowsKernel(const T *x, T *z, Long n, const Long *indexes, const Long *tadInfo,
+                                                         const Long *tadOffsets, const Long *zTadInfo, const Long *zTadOffsets) {
+    const Long tadLength = dLength(tadInfo);
+    const Long xe = dEws(tadInfo), ze = dEws(zTadInfo);
+    const int lanes = lanesPerTad(tadLength), groups = kBlock / lanes;
+    const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
+    for (Long idx = (Long)blockIdx.x * groups + g; idx < n; idx += (Long)gridDim.x * groups)
+        copyRun<T, false>(x + tadOffsets[indexes[idx]], xe, tadInfo, z + zTadOffsets[idx], ze, zTadInfo, tadLength, lane, lanes);
+}
+
+// ---- tear: target[r] <- x TAD r (the stride-less branch decomposes in F order, as both reference back ends do) ----
+template <typename T>
+__global__ void __launch_bounds__(kBlock) tearKernel(const T *x, const Long *xInfo, T *const *targets, const Long *zInfo,
+                                                     const Long *tadInfo, const Long *tadOffsets) {
+    const Long tadLength = dLength(tadInfo);
+    const Long numTads = dLength(xInfo) / tadLength;
+    const Long xe = dEws(tadInfo), ze = dEws(zInfo);
+    const int lanes = lanesPerTad(tadLength), groups = kBlock / lanes;
+    const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
+    for (Long r = (Long)blockIdx.x * groups + g; r < numTads; r += (Long)gridDim.x * groups)
+        copyRun<T, true>(x + tadOffsets[r], xe, tadInfo, targets[r], ze, zInfo, tadLength, lane, lanes);
+}
+
+// ---- shuffle: TAD r and TAD map[r] of every array trade places (map[r] < 0: leave r alone) -----------------------
+// The pairs of one map are disjoint (each TAD appears in at most one pair), which is what makes the reference's
+// sequential loop and a parallel one agree.  Values are read from x and written to z; the callers pass z == x.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) shuffleKernel(T *const *xs, const Long *const *xInfos, T *const *zs, int N,
+                                                        const int *map, const Long *const *tadInfos,
+                                                        const Long *const *tadOffsets) {
+    constexpr int VEC = Pack<T>::N;
+    for (int f = blockIdx.y; f < N; f += gridDim.y) {
+        const T *x = xs[f];
+        T *z = zs[f];
+        const Long *ti = tadInfos[f], *off = tadOffsets[f];
+        const Long tadLength = dLength(ti);
+        const Long numTads = dLength(xInfos[f]) / tadLength;
+        const Long ews = dEws(ti);
+        const int lanes = lanesPerTad(tadLength), groups = kBlock / lanes;
+        const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
+        for (Long r = (Long)blockIdx.x * groups + g; r < numTads; r += (Long)gridDim.x * groups) {
+            const int m = map[r];
+            if (m < 0) continue;
+            const Long oa = off[r], ob = off[m];
+            if (ews == 1 && tadLength % VEC == 0 && (reinterpret_cast<uintptr_t>(x + oa) & 15) == 0 &&
+                (reinterpret_cast<uintptr_t>(x + ob) & 15) == 0 && (reinterpret_cast<uintptr_t>(z + oa) & 15) == 0 &&
+                (reinterpret_cast<uintptr_t>(z + ob) & 15) == 0) {
+                const Pack<T> *xa = reinterpret_cast<const Pack<T> *>(x + oa), *xb = reinterpret_cast<const Pack<T> *>(x + ob);
+                Pack<T> *za = reinterpret_cast<Pack<T> *>(z + oa), *zb = reinterpret_cast<Pack<T> *>(z + ob);
+                for (Long v = lane; v < tadLength / VEC; v += lanes) {
+                    const Pack<T> a = loadPack(xa + v), b = loadPack(xb + v);
+                    storePack(za + v, b);
+                    storePack(zb + v, a);
+                }
+            } else if (ews >= 1) {
+                for (Long i = lane; i < tadLength; i += lanes) {
+                    const T a = x[oa + i * ews], b = x[ob + i * ews];
+                    z[oa + i * ews] = b;
+                    z[ob + i * ews] = a;
+                }
+            } else {
+                for (Long i = lane; i < tadLength; i += lanes) {
+                    const Long o = dOffsetC(ti, i);
+                    const T a = x[oa + o], b = x[ob + o];
+                    z[oa + o] = b;
+                    z[ob + o] = a;
+                }
+            }
+        }
+    }
+}
+
+// ---- concat ----------------------------------------------------------------------------------------------------
+// cum[r] = sum of shape[dim] of the inputs before r, cum[n] = the total; one block.
+__global__ void __launch_bounds__(kBlock) concatPrefixKernel(const Long *const *infos, int n, int dim, Long *cum) {
+    __shared__ Long part[kBlock];
+    const int chunk = (n + kBlock - 1) / kBlock;
+    const int lo = threadIdx.x * chunk, hi = lo + chunk < n ? lo + chunk : n;
+    Long sum = 0;
+    for (int f = lo; f < hi; f++) sum += dShape(infos[f])[dim];
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        Long run = 0;
+        for (int t = 0; t < kBlock; t++) {
+            const Long p = part[t];
+            part[t] = run;
+            run += p;
+        }
+        cum[n] = run;
+    }
+    __syncthreads();
+    Long run = part[threadIdx.x];
+    for (int f = lo; f < hi; f++) {
+        cum[f] = run;
+        run += dShape(infos[f])[dim];
+    }
+}
+
+// Input r (blockIdx.y) is copied into the slab [cum[r], cum[r+1]) of dimension `dim` of z.  Elements are walked in
+// the input's logical C order; contiguous C-order inputs into a contiguous C-order result move whole runs.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) concatKernel(const T *const *data, const Long *const *infos, T *z, ConcatView v,
+                                                       const Long *cum, int n) {
+    constexpr int VEC = Pack<T>::N;
+    for (int r = blockIdx.y; r < n; r += gridDim.y) {
+        const Long *si = infos[r];
+        const T *x = data[r];
+        const int rank = dRank(si);
+        const Long len = dLength(si);
+        const Long start = cum[r];
+        if (rank == v.rank && v.zContig && dOrder(si) == 'c' && dEws(si) == 1) {
+            const Long run = dShape(si)[v.dim] * v.inner;  // contiguous on both sides
+            const Long zRun = v.dimTotal * v.inner;        // distance between consecutive runs in z
+            T *zb = z + start * v.inner;
+            if (run % VEC == 0 && zRun % VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                (reinterpret_cast<uintptr_t>(zb) & 15) == 0) {
+                const Long runV = run / VEC, zRunV = zRun / VEC, nv = len / VEC;
+                const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x);
+                Pack<T> *zv = reinterpret_cast<Pack<T> *>(zb);
+                for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < nv; i += (Long)gridDim.x * kBlock) {
+                    const Long o = i / runV;
+                    storePack(zv + o * zRunV + (i - o * runV), loadPack(xv + i));
+                }
+            } else {
+                for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < len; i += (Long)gridDim.x * kBlock) {
+                    const Long o = i / run;
+                    zb[o * zRun + (i - o * run)] = x[i];
+                }
+            }
+        } else if (rank == v.rank) {
+            const Long *shape = dShape(si), *stride = dStride(si);
+            for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < len; i += (Long)gridDim.x * kBlock) {
+                Long rem = i, xo = 0, zo = 0;
+                for (int d = rank - 1; d >= 0; d--) {
+                    const Long q = rem / shape[d], c = rem - q * shape[d];
+                    xo += c * stride[d];
+                    zo += (c + (d == v.dim ? start : 0)) * v.zStride[d];
+                    rem = q;
+                }
+                z[zo] = x[xo];
+            }
+        }
+    }
+}
+
+template <typename T>
+void launchPullRows(hipStream_t s, const T *x, T *z, Long n, const Long *indexes, const Long *tadInfo, const Long *tadOffsets,
+                    const Long *zTadInfo, const Long *zTadOffsets) {
+    if (n <= 0) return;
+    hipLaunchKernelGGL((pullRowsKernel<T>), dim3(gridFor(n, 1, kGridCap * 4)), dim3(kBlock), 0, s, x, z, n, indexes, tadInfo,
+                       tadOffsets, zTadInfo, zTadOffsets);
+}
+template <typename T>
+void launchTear(hipStream_t s, const T *x, const Long *xInfo, T *const *targets, const Long *zInfo, const Long *tadInfo,
+                const Long *tadOffsets, Long numTadsHint) {
+    hipLaunchKernelGGL((tearKernel<T>), dim3(gridFor(numTadsHint > 0 ? numTadsHint : kGridCap, 1, kGridCap * 4)), dim3(kBlock), 0, s,
+                       x, xInfo, targets, zInfo, tadInfo, tadOffsets);
+}
+template <typename T>
+void launchShuffle(hipStream_t s, T *const *xs, const Long *const *xInfos, T *const *zs, int N, const int *map,
+                   const Long *const *tadInfos, const Long *const *tadOffsets, Long numTadsHint) {
+    if (N <= 0) return;
+    const int gy = N < 64 ? N : 64;
+    hipLaunchKernelGGL((shuffleKernel<T>), dim3(gridFor(numTadsHint > 0 ? numTadsHint : 4096, 1, kGridCap), gy), dim3(kBlock), 0, s,
+                       xs, xInfos, zs, N, map, tadInfos, tadOffsets);
+}
+template <typename T>
+void launchConcat(hipStream_t s, const T *const *data, const Long *const *infos, T *z, const ConcatView &v, int n, Long maxLength,
+                  Long *cum) {
+    if (n <= 0) return;
+    hipLaunchKernelGGL(concatPrefixKernel, dim3(1), dim3(kBlock), 0, s, infos, n, v.dim, cum);
+    const int gy = n < 65535 ? n : 65535;
+    int budget = (kGridCap * 4) / gy;
+    if (budget < 1) budget = 1;
+    const int gx = gridFor(maxLength > 0 ? maxLength : 1, (Long)kBlock * Pack<T>::N, budget);
+    hipLaunchKernelGGL((concatKernel<T>), dim3(gx, gy), dim3(kBlock), 0, s, data, infos, z, v, cum, n);
+}
+
+// ---- conversions between half, float and double: z[i] = (D)(float)x[i] (type_conversions.h:38-49) -----------------
+template <typename S, typename D> __device__ __forceinline__ D convertOne(S v) {
+    const float f = (float)toCompute(v);
+    return fromCompute<D>((typename Compute<D>::type)f);
+}
+template <typename S, typename D>
+__global__ void __launch_bounds__(kBlock) convertKernel(const S *x, D *z, Long n, int vectors) {
+    constexpr int E = 8;  // elements per thread and pass: 16 bytes of half, 32 of float, 64 of double
+    const Long chunks = vectors ? n / E : 0;
+    for (Long c = (Long)blockIdx.x * kBlock + threadIdx.x; c < chunks; c += (Long)gridDim.x * kBlock) {
+        alignas(16) S in[E];
+        alignas(16) D out[E];
+        constexpr int NS = E * sizeof(S) / 16, ND = E * sizeof(D) / 16;
+        const U32x4 *src = reinterpret_cast<const U32x4 *>(x + c * E);
+#pragma unroll
+        for (int k = 0; k < NS; k++) reinterpret_cast<U32x4 *>(in)[k] = __builtin_nontemporal_load(src + k);
+#pragma unroll
+        for (int e = 0; e < E; e++) out[e] = convertOne<S, D>(in[e]);
+        U32x4 *dst = reinterpret_cast<U32x4 *>(z + c * E);
+#pragma unroll
+        for (int k = 0; k < ND; k++) __builtin_nontemporal_store(reinterpret_cast<const U32x4 *>(out)[k], dst + k);
+    }
+    for (Long i = chunks * E + (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock)
+        z[i] = convertOne<S, D>(x[i]);
+}
+template <typename S, typename D> void runConvert(hipStream_t s, const void *x, void *z, Long n) {
+    if (n <= 0) return;
+    const int vectors = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(z)) & 15) == 0 ? 1 : 0;
+    hipLaunchKernelGGL((convertKernel<S, D>), dim3(gridFor(n, (Long)kBlock * 8, kMaxGrid)), dim3(kBlock), 0, s,
+                       reinterpret_cast<const S *>(x), reinterpret_cast<D *>(z), n, vectors);
+}
+// type codes of type_conversions.h:11-18: 3 half, 6 float, 7 double
+bool launchConvert(hipStream_t s, int srcType, const void *x, Long n, int dstType, void *z) {
+    if (srcType == 3 && dstType == 6) runConvert<float16, float>(s, x, z, n);
+    else if (srcType == 3 && dstType == 7) runConvert<float16, double>(s, x, z, n);
+    else if (srcType == 6 && dstType == 3) runConvert<float, float16>(s, x, z, n);
+    else if (srcType == 6 && dstType == 7) runConvert<float, double>(s, x, z, n);
+    else if (srcType == 7 && dstType == 3) runConvert<double, float16>(s, x, z, n);
+    else if (srcType == 7 && dstType == 6) runConvert<double, float>(s, x, z, n);
+    else return false;
+    return true;
+}
+
+#define INST(T)                                                                                                              \
+    template void launchPullRows<T>(hipStream_t, const T *, T *, Long, const Long *, const Long *, const Long *, const Long *, \
+                                    const Long *);                                                                           \
+    template void launchTear<T>(hipStream_t, const T *, const Long *, T *const *, const Long *, const Long *, const Long *,  \
+                                Long);                                                                                       \
+    template void launchShuffle<T>(hipStream_t, T *const *, const Long *const *, T *const *, int, const int *,               \
+                                   const Long *const *, const Long *const *, Long);                                          \
+    template void launchConcat<T>(hipStream_t, const T *const *, const Long *const *, T *, const ConcatView &, int, Long, Long *);
+INST(float)
+INST(float16)
+INST(double)
+#undef INST
+
+}  // namespace nd4j_amd

@@ -124,6 +124,31 @@ template <typename T> bool launchSoftmax(hipStream_t stream, int opNum, const T 
 template <typename T> void launchIsMaxFill(hipStream_t stream, T *z, const T *index, const FlatPlan &zp);
 template <typename T> void launchIsMaxTadFill(hipStream_t stream, T *z, const T *index, const TadPlan &zt);
 
+// ---- data movement ---------------------------------------------------------------------------------
+// The result of a concat as the kernel needs it: strides per dimension, the concatenated dimension, and for a
+// contiguous C-order result the run geometry (inner = product of the dimensions after `dim`).
+struct ConcatView {
+    int rank, dim, zContig;
+    Long zStride[kMaxDims];
+    Long inner, dimTotal;
+};
+// Every pointer below is a device pointer (tables of pointers included), as in the reference's CUDA back end.
+template <typename T>
+void launchPullRows(hipStream_t stream, const T *x, T *z, Long n, const Long *indexes, const Long *tadInfo,
+                    const Long *tadOffsets, const Long *zTadInfo, const Long *zTadOffsets);
+template <typename T>
+void launchTear(hipStream_t stream, const T *x, const Long *xInfo, T *const *targets, const Long *zInfo, const Long *tadInfo,
+                const Long *tadOffsets, Long numTadsHint);
+template <typename T>
+void launchShuffle(hipStream_t stream, T *const *xs, const Long *const *xInfos, T *const *zs, int N, const int *map,
+                   const Long *const *tadInfos, const Long *const *tadOffsets, Long numTadsHint);
+// `cum` is device scratch of numArrays + 1 Longs; maxLength the element count of the largest input
+template <typename T>
+void launchConcat(hipStream_t stream, const T *const *data, const Long *const *infos, T *z, const ConcatView &view,
+                  int numArrays, Long maxLength, Long *cum);
+// srcType / dstType: 3 half, 6 float, 7 double (type_conversions.h:11-18); false for any other pair
+bool launchConvert(hipStream_t stream, int srcType, const void *x, Long n, int dstType, void *z);
+
 // ---- random ----------------------------------------------------------------------------------------
 // Device image of the generator state that getElement() needs (reference: helper_generator.h:61-74,
 // 185-220).  Passed by value, so one op sees one consistent state.

@@ -50,6 +50,12 @@ _EXEC_SIGNATURES = {
     "nd4j_execScalar{S}": ([_P, c_int, _P, _P, _P, _P, "_SCALAR", _P], False),
     "nd4j_execScalar{S}Indexed": ([_P, c_int, _P, _P, _P, _P, "_SCALAR", _P, _P, _P], False),
     "nd4j_execScalar{S}AlongDimension": ([_P, c_int, _P, _P, _P, _P, _P, _P, _P, c_int], False),
+    # data-movement specials
+    "nd4j_flatten{S}": ([_P, c_int, ctypes.c_char, _P, _P, _P, _P], False),
+    "nd4j_concat{S}": ([_P, c_int, c_int, _P, _P, _P, _P, _P, _P], False),
+    "nd4j_pullRows{S}": ([_P, _P, _P, _P, _P, c_ll, _P, _P, _P, _P, _P], False),
+    "nd4j_tear{S}": ([_P, _P, _P, _P, _P, _P, _P], False),
+    "nd4j_shuffle{S}": ([_P, _P, _P, _P, _P, c_int, _P, _P, _P], False),
 }
 
 _PLAIN_SIGNATURES = {
@@ -59,6 +65,7 @@ _PLAIN_SIGNATURES = {
     "nd4j_reSeedBuffer": ([_P, ctypes.c_long, _P], None),
     "nd4j_destroyRandom": ([_P], None),
     "nd4j_tadOnlyShapeInfo": ([_P, _P, c_int, _P, _P], None),
+    "nd4j_convertTypes": ([_P, c_int, _P, c_ll, c_int, _P], None),
     "nd4j_initializeDevicesAndFunctions": ([], None),
     "nd4j_mallocHost": ([c_ll, c_int], _P),
     "nd4j_mallocDevice": ([c_ll, _P, c_int], _P),

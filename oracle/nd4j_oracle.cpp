@@ -1453,6 +1453,129 @@ static void randomExec(int op, Rng *g, int operands, T *x, Long *xi, T *y, Long 
     g->rewind(length);
 }
 
+
+// ---- data-movement specials ---------------------------------------------------------------------------------
+// flatten: blas/cpu/NativeOps.cpp:1529-1664.  The input's elements in `order`, written from result + offset on;
+// only the same-order branch with element-wise strides honours the result's stride (1566-1579), the others write
+// densely (1586-1598, 1608-1660).
+template <typename T>
+void flatten(int offset, char order, T *result, const Long *zi, const T *input, const Long *xi) {
+    result += offset;
+    const Long len = siNumel(xi);
+    const int rank = siRank(xi);
+    const Long xe = siEws(xi), ze = siEws(zi);
+    if (siOrder(xi) == order && xe >= 1 && ze >= 1) {
+        for (Long i = 0; i < len; i++) result[i * ze] = input[i * xe];
+        return;
+    }
+    Long c[kMaxRank];
+    for (Long i = 0; i < len; i++) {
+        if (order == 'f') ind2subF(rank, siShape(xi), (int)i, c);
+        else ind2subC(rank, siShape(xi), (int)i, c);
+        result[i] = input[getOffset(0, siShape(xi), siStride(xi), c, rank)];
+    }
+}
+
+// concat: include/ops/impl/specials.cpp:17-200 - the inputs one after the other along `dimension` of the result.
+// Restated by coordinates (what every branch there computes for inputs that agree in the other dimensions);
+// all-scalar inputs fill result[i] = data[i][0] (47-52).
+template <typename T>
+void concat(int dimension, int numArrays, T **data, Long **infos, T *result, const Long *zi) {
+    bool allScalar = true;
+    for (int r = 0; r < numArrays; r++) allScalar = allScalar && siNumel(infos[r]) == 1;
+    if (allScalar) {
+        for (int r = 0; r < numArrays; r++) result[r * (siEws(zi) >= 1 ? siEws(zi) : 1)] = data[r][0];
+        return;
+    }
+    const int rank = siRank(zi);
+    Long start = 0;
+    Long c[kMaxRank];
+    for (int r = 0; r < numArrays; r++) {
+        const Long *xi = infos[r];
+        const Long len = siNumel(xi);
+        for (Long i = 0; i < len; i++) {
+            ind2subC(rank, siShape(xi), (int)i, c);
+            const Long xo = getOffset(0, siShape(xi), siStride(xi), c, rank);
+            c[dimension] += start;
+            result[getOffset(0, siShape(zi), siStride(zi), c, rank)] = data[r][xo];
+        }
+        start += siShape(xi)[dimension];
+    }
+}
+
+// pullRows: blas/cpu/NativeOps.cpp:2044-2104
+template <typename T>
+void pullRows(const T *x, T *z, Long n, const Long *indexes, const Long *ti, const Long *tadOffsets, const Long *zti,
+              const Long *zTadOffsets) {
+    const Long xe = siEws(ti), ze = siEws(zti), tadLength = siNumel(ti);
+    Long cx[kMaxRank], cz[kMaxRank];
+    for (Long idx = 0; idx < n; idx++) {
+        const T *rx = x + tadOffsets[indexes[idx]];
+        T *rz = z + zTadOffsets[idx];
+        if (xe >= 1 && ze >= 1) {
+            for (Long i = 0; i < tadLength; i++) rz[i * ze] = rx[i * xe];
+        } else {
+            for (Long i = 0; i < tadLength; i++) {
+                ind2subC(siRank(ti), siShape(ti), (int)i, cx);
+                ind2subC(siRank(zti), siShape(zti), (int)i, cz);
+                rz[getOffset(0, siShape(zti), siStride(zti), cz, siRank(zti))] =
+                    rx[getOffset(0, siShape(ti), siStride(ti), cx, siRank(ti))];
+            }
+        }
+    }
+}
+
+// tear: blas/cpu/NativeOps.cpp:2118-2160 (the stride-less branch decomposes with ind2sub, i.e. in F order)
+template <typename T>
+void tear(const T *x, const Long *xi, T **targets, const Long *zi, const Long *ti, const Long *tadOffsets) {
+    const Long tadLength = siNumel(ti), te = siEws(ti), ze = siEws(zi);
+    const Long numTads = siNumel(xi) / tadLength;
+    Long cx[kMaxRank], cz[kMaxRank];
+    for (Long r = 0; r < numTads; r++) {
+        T *z = targets[r];
+        const T *src = x + tadOffsets[r];
+        if (ze > 0 && te > 0) {
+            for (Long j = 0; j < tadLength; j++) z[j * ze] = src[j * te];
+        } else {
+            for (Long j = 0; j < tadLength; j++) {
+                ind2subF(siRank(ti), siShape(ti), (int)j, cx);
+                ind2subF(siRank(zi), siShape(zi), (int)j, cz);
+                z[getOffset(0, siShape(zi), siStride(zi), cz, siRank(zi))] = src[getOffset(0, siShape(ti), siStride(ti), cx, siRank(ti))];
+            }
+        }
+    }
+}
+
+// shuffle: blas/cpu/NativeOps.cpp:2265-2325 - in place on x, TAD r swapped with TAD map[r], r ascending
+template <typename T>
+void shuffle(T **xs, Long **xInfos, int N, const int *map, Long **tadInfos, Long **tadOffsets) {
+    Long c[kMaxRank];
+    for (int f = 0; f < N; f++) {
+        T *x = xs[f];
+        const Long *ti = tadInfos[f], *off = tadOffsets[f];
+        const Long tadLength = siNumel(ti), ews = siEws(ti);
+        const Long numTads = siNumel(xInfos[f]) / tadLength;
+        for (Long r = 0; r < numTads; r++) {
+            if (map[r] < 0) continue;
+            const Long oa = off[r], ob = off[map[r]];
+            for (Long i = 0; i < tadLength; i++) {
+                Long o;
+                if (ews == 1) o = i;
+                else { ind2subC(siRank(ti), siShape(ti), (int)i, c); o = getOffset(0, siShape(ti), siStride(ti), c, siRank(ti)); }
+                T t = x[oa + o];
+                x[oa + o] = x[ob + o];
+                x[ob + o] = t;
+            }
+        }
+    }
+}
+
+// conversions: include/loops/type_conversions.h:592-611 - z[i] = (D)((float)x[i])
+template <typename S, typename D> void convert(const void *x, Long n, void *z) {
+    const S *in = (const S *)x;
+    D *out = (D *)z;
+    for (Long i = 0; i < n; i++) out[i] = (D)((float)in[i]);
+}
 }  // namespace oracle
 
 using namespace oracle;
@@ -1552,6 +1675,40 @@ const char *nd4j_cpu_kind() { return "port"; }
 ND4J_CPU_FAMILY(f32, float)
 ND4J_CPU_FAMILY(f16, half)
 ND4J_CPU_FAMILY(f64, double)
+
+#define ND4J_CPU_SPECIALS(SUF, T)                                                                                  \
+    void nd4j_cpu_flatten_##SUF(int offset, int order, void *z, Long *zSI, void *x, Long *xSI) {                   \
+        flatten<T>(offset, (char)order, (T *)z, zSI, (T *)x, xSI);                                                 \
+    }                                                                                                              \
+    void nd4j_cpu_concat_##SUF(int dim, int n, void **data, Long **infos, void *z, Long *zSI) {                    \
+        concat<T>(dim, n, (T **)data, infos, (T *)z, zSI);                                                         \
+    }                                                                                                              \
+    void nd4j_cpu_pullrows_##SUF(void *x, Long *xSI, void *z, Long *zSI, long long n, Long *idx, Long *tadSI,      \
+                                 Long *tadOff, Long *zTadSI, Long *zTadOff) {                                      \
+        (void)xSI; (void)zSI;                                                                                      \
+        pullRows<T>((T *)x, (T *)z, n, idx, tadSI, tadOff, zTadSI, zTadOff);                                       \
+    }                                                                                                              \
+    void nd4j_cpu_tear_##SUF(void *x, Long *xSI, void **targets, Long *zSI, Long *tadSI, Long *tadOff) {           \
+        tear<T>((T *)x, xSI, (T **)targets, zSI, tadSI, tadOff);                                                   \
+    }                                                                                                              \
+    void nd4j_cpu_shuffle_##SUF(void **x, Long **xSI, int N, int *map, Long **tadSI, Long **tadOff) {              \
+        shuffle<T>((T **)x, xSI, N, map, tadSI, tadOff);                                                           \
+    }
+ND4J_CPU_SPECIALS(f32, float)
+ND4J_CPU_SPECIALS(f16, half)
+ND4J_CPU_SPECIALS(f64, double)
+
+// type codes of type_conversions.h:11-18 (3 half, 6 float, 7 double); returns 0 for any other pair
+int nd4j_cpu_convert(int srcType, void *x, long long n, int dstType, void *z) {
+    if (srcType == 3 && dstType == 6) convert<half, float>(x, n, z);
+    else if (srcType == 3 && dstType == 7) convert<half, double>(x, n, z);
+    else if (srcType == 6 && dstType == 3) convert<float, half>(x, n, z);
+    else if (srcType == 6 && dstType == 7) convert<float, double>(x, n, z);
+    else if (srcType == 7 && dstType == 3) convert<double, half>(x, n, z);
+    else if (srcType == 7 && dstType == 6) convert<double, float>(x, n, z);
+    else return 0;
+    return 1;
+}
 
 // blas/cpu/NativeOps.cpp:2877-2906
 void *nd4j_cpu_rng_init(long long seed, long long size, uint64_t *buffer) {

@@ -38,6 +38,27 @@ using functions::random::RandomFunction;
 using functions::scalar::ScalarTransform;
 using functions::reduce3::Reduce3;
 
+// Data-movement specials.  flatten / pullRows / tear / shuffle are function templates defined and explicitly
+// instantiated in blas/cpu/NativeOps.cpp (1529-1664, 2044-2160, 2265-2325, instantiations 3574-3588); that file is
+// compiled where it lies with hidden visibility and per-function sections, and the link drops everything these
+// wrappers do not reach.  concat is nd4j::SpecialMethods<T>::concatCpuGeneric of include/ops/impl/specials.cpp,
+// the conversions go through NativeOps::convertTypes itself (include/loops/type_conversions.h:696-850, a
+// host loop in both of the reference's back ends).
+#include <ops/specials.h>
+template <typename T>
+void flattenGeneric(Nd4jPointer *extraPointers, int offset, char order, T *result, Nd4jLong *resultShapeInfo, T *input,
+                    Nd4jLong *inputShapeInfo);
+template <typename T>
+void pullRowsGeneric(T *x, Nd4jLong *xShapeInfo, T *z, Nd4jLong *zShapeInfo, const int n, Nd4jLong *indexes,
+                     Nd4jLong *tadShapeInfo, Nd4jLong *tadOffsets, Nd4jLong *zTadShapeInfo, Nd4jLong *zTadOffsets);
+template <typename T>
+void tearGeneric(T *x, Nd4jLong *xShapeInfo, Nd4jPointer *targets, Nd4jLong *zShapeInfo, Nd4jLong *tadShapeInfo,
+                 Nd4jLong *tadOffsets);
+template <typename T>
+void shuffleGeneric(T **dX, Nd4jLong **xShapeInfo, T **dZ, Nd4jLong **zShapeInfo, int N, int *shuffleMap,
+                    Nd4jLong **tadOnlyShapeInfo, Nd4jLong **tadOffsets);
+#include <NativeOps.h>
+
 namespace {
 
 template <typename T>
@@ -178,9 +199,40 @@ void reduce3AllPairs(int opNum, T *x, Nd4jLong *xSI, T *extra, T *y, Nd4jLong *y
         RandomFunction<T>::execTransform(op, state, (T *)x, xSI, (T *)y, ySI, (T *)z, zSI, (T *)args);      \
     }
 
+#define ND4J_CPU_SPECIALS(SUF, T)                                                                                  \
+    void nd4j_cpu_flatten_##SUF(int offset, int order, void *z, Nd4jLong *zSI, void *x, Nd4jLong *xSI) {           \
+        flattenGeneric<T>(nullptr, offset, (char)order, (T *)z, zSI, (T *)x, xSI);                                 \
+    }                                                                                                              \
+    void nd4j_cpu_concat_##SUF(int dim, int n, void **data, Nd4jLong **infos, void *z, Nd4jLong *zSI) {            \
+        nd4j::SpecialMethods<T>::concatCpuGeneric(dim, n, data, (Nd4jPointer *)infos, (T *)z, zSI);                \
+    }                                                                                                              \
+    void nd4j_cpu_pullrows_##SUF(void *x, Nd4jLong *xSI, void *z, Nd4jLong *zSI, long long n, Nd4jLong *idx,       \
+                                 Nd4jLong *tadSI, Nd4jLong *tadOff, Nd4jLong *zTadSI, Nd4jLong *zTadOff) {         \
+        pullRowsGeneric<T>((T *)x, xSI, (T *)z, zSI, (int)n, idx, tadSI, tadOff, zTadSI, zTadOff);                 \
+    }                                                                                                              \
+    void nd4j_cpu_tear_##SUF(void *x, Nd4jLong *xSI, void **targets, Nd4jLong *zSI, Nd4jLong *tadSI,               \
+                             Nd4jLong *tadOff) {                                                                   \
+        tearGeneric<T>((T *)x, xSI, targets, zSI, tadSI, tadOff);                                                  \
+    }                                                                                                              \
+    void nd4j_cpu_shuffle_##SUF(void **x, Nd4jLong **xSI, int N, int *map, Nd4jLong **tadSI, Nd4jLong **tadOff) {  \
+        shuffleGeneric<T>((T **)x, xSI, (T **)x, xSI, N, map, tadSI, tadOff);                                      \
+    }
+
 extern "C" {
 
 const char *nd4j_cpu_kind() { return "reference"; }
+
+ND4J_CPU_SPECIALS(f32, float)
+ND4J_CPU_SPECIALS(f16, float16)
+ND4J_CPU_SPECIALS(f64, double)
+
+int nd4j_cpu_convert(int srcType, void *x, long long n, int dstType, void *z) {
+    const bool known = (srcType == 3 || srcType == 6 || srcType == 7) && (dstType == 3 || dstType == 6 || dstType == 7);
+    if (!known || srcType == dstType) return 0;
+    NativeOps ops;
+    ops.convertTypes(nullptr, srcType, x, n, dstType, z);
+    return 1;
+}
 
 ND4J_CPU_FAMILY(f32, float)
 ND4J_CPU_FAMILY(f16, float16)

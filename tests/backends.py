@@ -7,6 +7,8 @@ pointed at a CPU checker (oracle restatement or compiled reference) or at the HI
 
 Array arguments are flat numpy buffers (the memory of the view); *_info are shapeInfo arrays.
 """
+import ctypes
+
 import numpy as np
 
 from golden_inputs import shape_info_np
@@ -117,6 +119,37 @@ class CpuBackend(object):
     def summarystats_scalar(self, op, bias, x, x_info):
         return self.lib.summarystats_scalar(op, bias, x, x_info)
 
+    # ---- data movement ---------------------------------------------------------------------------
+    def flatten(self, offset, order, x, x_info, z_len, z_info=None):
+        z = np.zeros(z_len, x.dtype)
+        self.lib.flatten(offset, order, z, _vec_info(z_len) if z_info is None else z_info, x, x_info)
+        return z
+
+    def concat(self, dim, arrays, infos, z_info):
+        z = np.zeros(_span(z_info), arrays[0].dtype)
+        self.lib.concat(dim, arrays, infos, z, z_info)
+        return z
+
+    def pullrows(self, x, x_info, z_info, indexes, tad, z_tad):
+        z = np.zeros(_span(z_info), x.dtype)
+        self.lib.pullrows(x, x_info, z, z_info, indexes, tad, z_tad)
+        return z
+
+    def tear(self, x, x_info, z_info, tad):
+        targets = [np.zeros(_span(z_info), x.dtype) for _ in range(len(tad[1]))]
+        self.lib.tear(x, x_info, targets, z_info, tad)
+        return targets
+
+    def shuffle(self, arrays, infos, shuffle_map, tads):
+        out = [a.copy() for a in arrays]
+        self.lib.shuffle(out, infos, shuffle_map, tads)
+        return out
+
+    def convert(self, src_type, x, dst_type):
+        z = np.zeros(x.size, TYPE_OF_CODE[dst_type])
+        assert self.lib.convert(src_type, x, dst_type, z) == 1
+        return z
+
     def tad(self, x_info, dims):
         return self.lib.tad(x_info, dims)
 
@@ -180,6 +213,9 @@ class _CpuRng(object):
         self.g.destroy()
 
 
+TYPE_OF_CODE = {3: np.float16, 6: np.float32, 7: np.float64}
+
+
 class GpuBackend(object):
     name = "gpu"
     kind = "hip"
@@ -209,6 +245,86 @@ class GpuBackend(object):
             if o is not None:
                 o.free()
         self.dev.release()
+
+    # ---- data movement ---------------------------------------------------------------------------
+    def _ptr_table(self, device_arrays):
+        return self.dev.upload(np.array([d.ptr for d in device_arrays], dtype=np.uint64))
+
+    def flatten(self, offset, order, x, x_info, z_len, z_info=None):
+        z_info = _vec_info(z_len) if z_info is None else z_info
+        X = self._op(x, x_info)
+        Z = self._op(np.zeros(z_len, x.dtype), z_info)
+        ptrs = self.dev.extra(y_info=x_info)  # the input's host shapeInfo travels in slot 7
+        getattr(self.ops, "flatten" + self._suffix(x))(ptrs, offset, order.encode(), Z.ptr, Z.info_ptr, X.ptr, X.info_ptr)
+        out = Z.get()
+        self._finish(X, Z)
+        return out
+
+    def concat(self, dim, arrays, infos, z_info, host_shapes=True):
+        ops = [self._op(a, i) for a, i in zip(arrays, infos)]
+        Z = self._op(np.zeros(_span(z_info), arrays[0].dtype), z_info)
+        data_tab = self._ptr_table([o.buf for o in ops])
+        info_tab = self._ptr_table([o.dinfo for o in ops])
+        ptrs = self.dev.extra(z_info)  # the result's host shapeInfo travels in slot 0
+        host_infos = [np.ascontiguousarray(i, dtype=np.int64) for i in infos]
+        host_tab = (ctypes.c_void_p * len(infos))(*[h.ctypes.data for h in host_infos])
+        if host_shapes:
+            ptrs[9] = ctypes.cast(host_tab, ctypes.c_void_p)
+        data = (ctypes.c_void_p * 1)(data_tab.ptr)
+        shapes = (ctypes.c_void_p * 1)(info_tab.ptr)
+        getattr(self.ops, "concat" + self._suffix(arrays[0]))(ptrs, dim, len(arrays), data, shapes, Z.ptr, Z.info_ptr, None, None)
+        out = Z.get()
+        self._finish(Z, data_tab, info_tab, *ops)
+        return out
+
+    def pullrows(self, x, x_info, z_info, indexes, tad, z_tad):
+        X = self._op(x, x_info)
+        Z = self._op(np.zeros(_span(z_info), x.dtype), z_info)
+        I, i = self._up(indexes, np.int64)
+        parts = [self._up(v, np.int64) for v in (tad[0], tad[1], z_tad[0], z_tad[1])]
+        getattr(self.ops, "pullRows" + self._suffix(x))(self.dev.extra(x_info), X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, len(indexes), i,
+                                                        *[p[1] for p in parts])
+        out = Z.get()
+        self._finish(X, Z, I, *[p[0] for p in parts])
+        return out
+
+    def tear(self, x, x_info, z_info, tad):
+        X = self._op(x, x_info)
+        n = len(tad[1])
+        span = _span(z_info)
+        targets = [self.dev.upload(np.zeros(span, x.dtype)) for _ in range(n)]
+        tab = self._ptr_table(targets)
+        ZI, zi = self._up(z_info, np.int64)
+        TI, ti = self._up(tad[0], np.int64)
+        TO, to = self._up(tad[1], np.int64)
+        getattr(self.ops, "tear" + self._suffix(x))(self.dev.extra(x_info), X.ptr, X.info_ptr, tab.ptr, zi, ti, to)
+        self.dev.sync()
+        out = [t.download(x.dtype, span) for t in targets]
+        self._finish(X, tab, ZI, TI, TO, *targets)
+        return out
+
+    def shuffle(self, arrays, infos, shuffle_map, tads):
+        ops = [self._op(a, i) for a, i in zip(arrays, infos)]
+        tis = [self.dev.upload(np.ascontiguousarray(t[0], dtype=np.int64)) for t in tads]
+        tos = [self.dev.upload(np.ascontiguousarray(t[1], dtype=np.int64)) for t in tads]
+        x_tab = self._ptr_table([o.buf for o in ops])
+        i_tab = self._ptr_table([o.dinfo for o in ops])
+        ti_tab, to_tab = self._ptr_table(tis), self._ptr_table(tos)
+        M, m = self._up(shuffle_map, np.int32)
+        getattr(self.ops, "shuffle" + self._suffix(arrays[0]))(self.dev.extra(), x_tab.ptr, i_tab.ptr, x_tab.ptr, i_tab.ptr,
+                                                               len(arrays), m, ti_tab.ptr, to_tab.ptr)
+        out = [o.get() for o in ops]
+        self._finish(x_tab, i_tab, ti_tab, to_tab, M, *(ops + tis + tos))
+        return out
+
+    def convert(self, src_type, x, dst_type):
+        X, xp = self._up(x)
+        dt = np.dtype(TYPE_OF_CODE[dst_type])
+        Z = self.dev.upload(np.zeros(x.size, dt))
+        self.ops.convertTypes(self.dev.extra(), src_type, xp, x.size, dst_type, Z.ptr)
+        out = Z.download(dt, x.size)
+        self._finish(X, Z)
+        return out
 
     # ---- elementwise ---------------------------------------------------------------------------
     def transform(self, op, x, x_info, z_info, extra=None, z=None):

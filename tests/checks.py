@@ -382,3 +382,141 @@ def check_rng_closed_forms(be):
         assert np.array_equal(u, (np.array(want, np.uint64).astype(np.float32) * np.float32(2.0 ** -64)))
         assert g.state()[1] == 0 and g.state()[3] == 2  # offset wrapped exactly once: generation 1 -> 2
         g.destroy()
+
+
+# ---- data-movement specials: flatten, concat, pullRows, tear, shuffle, convertTypes ----------------------------
+def _view(shape, order="c", strides=None):
+    """(flat buffer of distinct values, shapeInfo, logical array) of a dense array or a strided view."""
+    from libnd4j_amd.harness import element_offsets, shape_info, span_of
+    info = shape_info(shape, order, strides)
+    buf = np.arange(1, span_of(info) + 1, dtype=np.float64)
+    logical = buf[element_offsets(info)].reshape(shape)
+    return buf, info, logical
+
+
+def _logical(buf, info):
+    from libnd4j_amd.harness import element_offsets, info_shape
+    return np.asarray(buf)[element_offsets(info)].reshape(info_shape(info))
+
+
+def _cast(a, dt):
+    """Values as the data type under test; for half they are folded into the range it holds exactly."""
+    a = np.asarray(a)
+    if np.dtype(dt) == np.float16:
+        a = np.mod(a, 2039.0)
+    return a.astype(dt)
+
+
+def check_data_movement(be, dtypes=(np.float32, np.float64, np.float16), big=False):
+    """Every result is compared bit for bit with what numpy says the operation means."""
+    from libnd4j_amd.harness import shape_info, span_of
+    rs = np.random.RandomState(77)
+    for dt in dtypes:
+        # flatten: the input read in the requested order, written from `offset` on
+        cases = [([3, 4], "c", None), ([3, 4], "f", None), ([2, 3, 4], "c", None), ([2, 3, 4], "f", None),
+                 ([5, 7], "c", [14, 1]), ([5, 7], "c", [1, 5]), ([4, 3, 5], "c", [40, 10, 2]), ([1, 9], "c", None)]
+        if big:
+            cases += [([700, 300], "c", None), ([700, 300], "f", None), ([64, 33, 17], "f", None)]
+        for shape, order, strides in cases:
+            buf, info, logical = _view(shape, order, strides)
+            x = _cast(buf, dt)
+            n = logical.size
+            for want_order in "cf":
+                got = be.flatten(3, want_order, x, info, n + 5)
+                want = np.zeros(n + 5, dt)
+                want[3:3 + n] = _cast(logical.ravel(order=want_order.upper()), dt)
+                assert np.array_equal(got, want), ("flatten", shape, order, strides, want_order, np.dtype(dt).name)
+
+        # concat along every dimension, equal and unequal extents, c- and f-order inputs and results
+        ccases = [(0, [[2, 5], [3, 5], [1, 5]], "c", "c"), (1, [[4, 2], [4, 3]], "c", "c"), (1, [[4, 2], [4, 3]], "f", "c"),
+                  (0, [[2, 3, 4], [5, 3, 4]], "c", "c"), (1, [[2, 3, 4], [2, 1, 4]], "c", "f"), (2, [[2, 3, 4], [2, 3, 2]], "f", "f"),
+                  (1, [[1, 6], [1, 4], [1, 8]], "c", "c"), (0, [[1, 8]] * 9, "c", "c"), (1, [[1, 1]] * 5, "c", "c")]
+        if big:
+            ccases += [(0, [[200, 96]] * 12, "c", "c"), (1, [[300, 64], [300, 32], [300, 128]], "c", "c"),
+                       (0, [[1, 4096]] * 300, "c", "c")]
+        for dim, shapes, in_order, out_order in ccases:
+            arrays, infos, logicals = [], [], []
+            base = 0
+            for shp in shapes:
+                buf, info, logical = _view(shp, in_order)
+                arrays.append(_cast(buf + base, dt))
+                infos.append(info)
+                logicals.append(_cast(logical + base, dt))
+                base += buf.size
+            want = np.concatenate(logicals, axis=dim)
+            z_info = shape_info(list(want.shape), out_order)
+            got = be.concat(dim, arrays, infos, z_info)
+            assert np.array_equal(_logical(got, z_info), want), ("concat", dim, shapes, in_order, out_order, np.dtype(dt).name)
+
+        # pullRows: z row i <- x row indexes[i]; rows of a c-order matrix (contiguous) and of an f-order one (strided),
+        # and "rows" that are 2-D slices of a rank-3 array
+        pcases = [([9, 6], "c", [1], "c"), ([9, 6], "f", [1], "c"), ([9, 6], "c", [1], "f"), ([7, 3, 4], "c", [1, 2], "c"),
+                  ([7, 3, 4], "f", [1, 2], "f")]
+        if big:
+            pcases += [([500, 1024], "c", [1], "c"), ([300, 2052], "c", [1], "c"), ([400, 130], "f", [1], "c")]
+        for shape, order, dims, z_order in pcases:
+            buf, info, logical = _view(shape, order)
+            x = _cast(buf, dt)
+            idx = rs.randint(0, shape[0], size=shape[0] + 3)
+            z_shape = [len(idx)] + shape[1:]
+            z_info = shape_info(z_shape, z_order)
+            tad, z_tad = be.tad(info, dims), be.tad(z_info, dims)
+            got = be.pullrows(x, info, z_info, idx, tad, z_tad)
+            assert np.array_equal(_logical(got, z_info), _cast(logical[idx], dt)), ("pullRows", shape, order, dims, z_order)
+
+        # tear: target r <- TAD r
+        tcases = [([5, 8], "c", [1], [1, 8], "c"), ([5, 8], "f", [1], [1, 8], "c"), ([4, 3, 6], "c", [1, 2], [3, 6], "c"),
+                  ([4, 3, 6], "c", [1, 2], [3, 6], "f"), ([4, 3, 6], "f", [1, 2], [3, 6], "f")]
+        if big:
+            tcases += [([40, 2048], "c", [1], [1, 2048], "c"), ([33, 20, 30], "c", [1, 2], [20, 30], "c")]
+        for shape, order, dims, t_shape, t_order in tcases:
+            buf, info, logical = _view(shape, order)
+            x = _cast(buf, dt)
+            z_info = shape_info(t_shape, t_order)
+            tad = be.tad(info, dims)
+            got = be.tear(x, info, z_info, tad)
+            assert len(got) == shape[0]
+            for r in range(shape[0]):
+                assert np.array_equal(_logical(got[r], z_info), _cast(logical[r].reshape(t_shape), dt)), ("tear", shape, order, r)
+
+        # shuffle: disjoint pairs of rows trade places in every array of the set
+        scases = [[([8, 5], "c"), ([8, 3], "c")], [([8, 5], "f"), ([8, 2, 3], "c")]]
+        if big:
+            scases += [[([256, 1024], "c"), ([256, 10], "c"), ([256, 7], "f")]]
+        for group in scases:
+            rows = group[0][0][0]
+            perm = rs.permutation(rows)
+            smap = -np.ones(rows, np.int32)
+            for a, b in zip(perm[0::2], perm[1::2]):
+                smap[a] = b  # one entry per pair, the partner stays -1
+            arrays, infos, tads, wants = [], [], [], []
+            for shape, order in group:
+                buf, info, logical = _view(shape, order)
+                arrays.append(_cast(buf, dt))
+                infos.append(info)
+                tads.append(be.tad(info, list(range(1, len(shape)))))
+                want = logical.copy()
+                for a in range(rows):
+                    if smap[a] >= 0:
+                        want[[a, smap[a]]] = want[[smap[a], a]]
+                wants.append(_cast(want, dt))
+            got = be.shuffle(arrays, infos, smap, tads)
+            for g, info, want in zip(got, infos, wants):
+                assert np.array_equal(_logical(g, info), want), ("shuffle", group)
+
+    # conversions: z = (dst)(float)x
+    codes = {np.dtype(np.float16): 3, np.dtype(np.float32): 6, np.dtype(np.float64): 7}
+    vals = np.concatenate([rs.randn(1001) * 100, [0.0, -0.0, 1e-8, 65504.0, 70000.0, -1e10, 1e-40, np.inf, -np.inf, 3.14159265358979],
+                           rs.randn(40) * 1e-6])
+    if big:
+        vals = np.concatenate([vals, rs.randn(200003)])
+    for src in codes:
+        for dst in codes:
+            if src == dst:
+                continue
+            with np.errstate(over="ignore"):
+                x = vals.astype(src)
+                want = x.astype(np.float32).astype(dst)
+            got = be.convert(codes[src], x, codes[dst])
+            assert np.array_equal(got.view(np.dtype("u%d" % np.dtype(dst).itemsize)),
+                                  want.view(np.dtype("u%d" % np.dtype(dst).itemsize))), ("convert", src, dst)

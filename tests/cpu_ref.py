@@ -79,7 +79,14 @@ class CpuLib(object):
             "random_z": [I, V, V, V, V],
             "random_xz": [I, V, V, V, V, V, V],
             "random_xyz": [I, V, V, V, V, V, V, V, V],
+            "flatten": [I, I, V, V, V, V],
+            "concat": [I, I, V, V, V, V],
+            "pullrows": [V, V, V, V, LL, V, V, V, V, V],
+            "tear": [V, V, V, V, V, V],
+            "shuffle": [V, V, I, V, V, V],
         }
+        L.nd4j_cpu_convert.restype = I
+        L.nd4j_cpu_convert.argtypes = [I, V, LL, I, V]
         for fam, sig in sigs.items():
             for suf in SUF.values():
                 fn = getattr(L, "nd4j_cpu_%s_%s" % (fam, suf))
@@ -92,6 +99,39 @@ class CpuLib(object):
 
     def _fn(self, fam, arr):
         return getattr(self.lib, "nd4j_cpu_%s_%s" % (fam, SUF[np.dtype(arr.dtype)]))
+
+    # -- data movement ---------------------------------------------------------------------------------
+    @staticmethod
+    def _table(arrays):
+        return (ctypes.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+
+    def flatten(self, offset, order, z, z_info, x, x_info):
+        self._fn("flatten", x)(offset, ord(order), _p(z), _p(_info(z_info)), _p(x), _p(_info(x_info)))
+
+    def concat(self, dim, arrays, infos, z, z_info):
+        infos = [_info(i) for i in infos]
+        self._fn("concat", z)(dim, len(arrays), self._table(arrays), self._table(infos), _p(z), _p(_info(z_info)))
+
+    def pullrows(self, x, x_info, z, z_info, indexes, tad, z_tad):
+        idx = np.ascontiguousarray(indexes, dtype=np.int64)
+        ti, to, zi, zo = [_info(v) for v in (tad[0], tad[1], z_tad[0], z_tad[1])]
+        self._fn("pullrows", x)(_p(x), _p(_info(x_info)), _p(z), _p(_info(z_info)), len(idx), _p(idx), _p(ti), _p(to), _p(zi),
+                                _p(zo))
+
+    def tear(self, x, x_info, targets, z_info, tad):
+        ti, to = _info(tad[0]), _info(tad[1])
+        self._fn("tear", x)(_p(x), _p(_info(x_info)), self._table(targets), _p(_info(z_info)), _p(ti), _p(to))
+
+    def shuffle(self, arrays, infos, shuffle_map, tads):
+        infos = [_info(i) for i in infos]
+        tis = [_info(t[0]) for t in tads]
+        tos = [_info(t[1]) for t in tads]
+        m = _ints(shuffle_map)
+        self._fn("shuffle", arrays[0])(self._table(arrays), self._table(infos), len(arrays), _p(m), self._table(tis),
+                                       self._table(tos))
+
+    def convert(self, src_type, x, dst_type, z):
+        return self.lib.nd4j_cpu_convert(src_type, _p(x), x.size, dst_type, _p(z))
 
     # -- families -----------------------------------------------------------------------------------
     def transform(self, op, x, x_info, z, z_info, extra=None):

@@ -14,8 +14,8 @@ def _declared_c_names():
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     text = text.replace("\\\n", " ")
     names = set(re.findall(r"\b(nd4j_(?:amd_)?[A-Za-z0-9]+)\s*\(", text))
-    for macro_name in ("ND4J_C_EXEC", "ND4J_C_SCALAR", "ND4J_C_REDUCE3"):
-        macro = re.search(r"#define %s\(SUFFIX, T, [RS]\)(.*?)\n\s*\n" % macro_name, text, flags=re.S).group(1)
+    for macro_name in ("ND4J_C_EXEC", "ND4J_C_SCALAR", "ND4J_C_REDUCE3", "ND4J_C_SPECIAL"):
+        macro = re.search(r"#define %s\(SUFFIX, T(?:, [RS])?\)(.*?)\n\s*\n" % macro_name, text, flags=re.S).group(1)
         for templ in re.findall(r"\b(nd4j_[A-Za-z0-9#]+)\s*\(", macro):
             for suffix in ("Float", "Half", "Double"):
                 names.add(templ.replace("##SUFFIX##", suffix).replace("##SUFFIX", suffix))
@@ -37,7 +37,8 @@ def test_cpp_class_members_are_exported():
                    "execReduceFloat", "execReduceScalarFloat", "execIndexReduceFloat", "execIndexReduceScalarFloat",
                    "execSummaryStatsFloat", "execSummaryStatsScalarFloat", "execRandomFloat", "execRandomHalf",
                    "execScalarFloat", "execScalarHalf", "execScalarDouble", "execReduce3Float", "execReduce3ScalarFloat",
-                   "execReduce3AllFloat", "execReduce3Half", "execReduce3Double",
+                   "execReduce3AllFloat", "execReduce3Half", "execReduce3Double", "flattenFloat", "concatFloat", "concatHalf",
+                   "pullRowsFloat", "pullRowsDouble", "tearFloat", "shuffleFloat", "shuffleHalf", "convertTypes",
                    "initRandom", "refreshBuffer", "reSeedBuffer", "destroyRandom", "tadOnlyShapeInfo", "mallocDevice",
                    "createStream", "memcpyAsync", "streamSynchronize"):
         assert "NativeOps::%s(" % member in out, member

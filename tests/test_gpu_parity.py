@@ -428,6 +428,18 @@ def test_special_transforms(gpu, cpu):
                 assert np.array_equal(got, cpu.transform(41, x, xi, xi, e)), (shape, dim)
 
 
+def test_data_movement(gpu):
+    """flatten / concat / pullRows / tear / shuffle / convertTypes through the C ABI, bit for bit against numpy (the
+    same check the CPU restatement and the compiled reference pass)."""
+    checks.check_data_movement(gpu, big=True)
+    # concat without the host table of input shapes (extraPointers[9] absent): same result
+    from libnd4j_amd.harness import shape_info
+    arrays = [np.arange(12, dtype=np.float32), np.arange(100, 118, dtype=np.float32)]
+    infos = [shape_info([2, 6]), shape_info([3, 6])]
+    got = gpu.concat(0, arrays, infos, shape_info([5, 6]), host_shapes=False)
+    assert np.array_equal(got, np.concatenate(arrays))
+
+
 def test_nan_and_special_values(gpu, cpu):
     x = np.array([np.nan, 1.0, -np.inf, np.inf, 0.0, -0.0, 3.0, np.nan, 2.0, -1e38, 1e38, 5.0], np.float32)
     xi = shape_info_np([1, x.size])

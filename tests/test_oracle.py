@@ -290,3 +290,10 @@ def test_rng_matches_compiled_reference(oracle, reference_lib):
         assert np.array_equal(za, zb)
         a.destroy()
         b.destroy()
+
+
+def test_data_movement_matches_numpy_and_compiled_reference(oracle_lib, reference_lib):
+    """flatten / concat / pullRows / tear / shuffle / convertTypes: the restatement and the compiled reference
+    (blas/cpu/NativeOps.cpp templates, specials.cpp, convertTypes) against what numpy says each call means."""
+    checks.check_data_movement(backends.CpuBackend(oracle_lib), big=True)
+    checks.check_data_movement(backends.CpuBackend(reference_lib), big=True)
