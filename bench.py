@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--families", action="store_true", help="also time every op family of the other configurations")
     ap.add_argument("--only", default="", help="with --families: comma-separated workload builders to run "
-                                               "(transform,pairwise,half,reductions,reduce3,stats,random)")
+                                               "(transform,pairwise,half,reductions,reduce3,stats,random,movement)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU sample of the headline step")
     ap.add_argument("--counters", action="store_true",
@@ -223,7 +223,8 @@ def main():
         builders = [("transform", workloads.transform_tanh), ("pairwise", lambda d: workloads.pairwise_broadcast(d, copies=2)),
                     ("half", lambda d: workloads.pairwise_broadcast(d, dtype="float16")),
                     ("reductions", workloads.reductions), ("reduce3", workloads.reduce3_pairs),
-                    ("stats", workloads.stats_softmax), ("random", workloads.random_fills)]
+                    ("stats", workloads.stats_softmax), ("random", workloads.random_fills),
+                    ("movement", workloads.data_movement)]
         only = [o for o in args.only.split(",") if o]
         for key, build in builders:
             if only and key not in only:
@@ -234,7 +235,7 @@ def main():
                 row = {"config": wl.name, "case": c.name, "family": c.family, "contiguous": c.contiguous,
                        "ms": round(ms, 4), "GB/s": round(c.bytes / ms / 1e6, 1),
                        "frac": round(c.bytes / ms / 1e6 / HBM_PEAK_GBS, 4), "elements_per_sec": round(c.elements / ms * 1e3, 1)}
-                if cpu_lib is not None and not (c.name.endswith("float16")):
+                if cpu_lib is not None and c.cpu is not None and not (c.name.endswith("float16")):
                     med, runs = cpu_time(c.cpu, cpu_lib, 1.0, min_runs=2, max_runs=10)
                     row["cpu_ms"] = round(med * 1e3, 3)
                     row["cpu_GB/s"] = round(c.bytes / med / 1e9, 2)

@@ -374,6 +374,109 @@ def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
                        dict(x=x, xi=xi, softmax_cpu=tc), device_set, copies)
 
 
+# ---- data-movement specials: gathers, concatenations, reorders, conversions ---------------------------------
+def data_movement(dev, rows=65536, cols=1024, seed=31, copies=None):
+    import ctypes
+    n = rows * cols
+    rs = np.random.default_rng(seed)
+    x = _normal(rs, n, F32)
+    xi = harness.shape_info([rows, cols])
+    xfi = harness.shape_info([rows, cols], "f")
+    flat = _vec(n)
+    ops = dev.ops
+    tad_rows = dev.tad(xi, [1])
+    perm = rs.permutation(rows).astype(np.int64)
+    smap = -np.ones(rows, np.int32)
+    smap[perm[0::2]] = perm[1::2]
+    parts0, parts1 = 8, 4
+    r0, c1 = rows // parts0, cols // parts1
+    i0, i1 = harness.shape_info([r0, cols]), harness.shape_info([rows, c1])
+    x2 = x.reshape(rows, cols)
+    in0 = [np.ascontiguousarray(x2[k * r0:(k + 1) * r0]).ravel() for k in range(parts0)]
+    in1 = [np.ascontiguousarray(x2[:, k * c1:(k + 1) * c1]).ravel() for k in range(parts1)]
+    t_rows, t_len = 1024, n // 1024
+    ti_x = harness.shape_info([t_rows, t_len])
+    tad_tear = dev.tad(ti_x, [1])
+    ti_z = harness.shape_info([1, t_len])
+    zc = np.zeros(n, F32)
+    hc = np.zeros(n, np.float16)
+    xh = x.astype(np.float16)
+
+    def table(device_arrays):
+        return np.array([d.ptr for d in device_arrays], dtype=np.uint64)
+
+    def device_set(w):
+        X, Z = w.operand(x, xi), w.operand(np.zeros(n, F32), xi)
+        XF = w.raw(np.ascontiguousarray(xfi, dtype=np.int64))
+        FL = w.raw(np.ascontiguousarray(flat, dtype=np.int64))
+        cases = []
+        # pullRows: every row of x lands at a random row of z
+        IDX = w.raw(perm)
+        TI, TO = w.raw(tad_rows[0]), w.raw(tad_rows[1])
+        ex = dev.extra(xi)
+        cases.append(Case("pullrows_permute", "pullrows", n, 8 * n + 8 * rows,
+                          lambda: ops.pullRowsFloat(ex, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, rows, IDX.ptr, TI.ptr, TO.ptr, TI.ptr,
+                                                    TO.ptr),
+                          lambda lib: (lib.pullrows(x, xi, zc, xi, perm, tad_rows, tad_rows), zc)[1], True, Z.get))
+        # concat along dimension 0 (whole-array runs) and along dimension 1 (1 KiB runs)
+        for name, dim, parts, pinfo in (("concat_dim0", 0, in0, i0), ("concat_dim1", 1, in1, i1)):
+            P = [w.operand(p, pinfo) for p in parts]
+            DT, ST = w.raw(table([o.buf for o in P])), w.raw(table([o.dinfo for o in P]))
+            exc = dev.extra(xi)
+            host_infos = [np.ascontiguousarray(pinfo, dtype=np.int64) for _ in parts]
+            host_tab = (ctypes.c_void_p * len(parts))(*[h.ctypes.data for h in host_infos])
+            exc[9] = ctypes.cast(host_tab, ctypes.c_void_p)
+            exc._keep_concat = (host_infos, host_tab)
+            data, shapes = (ctypes.c_void_p * 1)(DT.ptr), (ctypes.c_void_p * 1)(ST.ptr)
+
+            def gpu(dim=dim, k=len(parts), exc=exc, data=data, shapes=shapes):
+                ops.concatFloat(exc, dim, k, data, shapes, Z.ptr, Z.info_ptr, None, None)
+
+            def cpu(lib, dim=dim, parts=parts, pinfo=pinfo):
+                lib.concat(dim, parts, [pinfo] * len(parts), zc, xi)
+                return zc
+
+            cases.append(Case(name, "concat", n, 8 * n, gpu, cpu, True, Z.get))
+        # flatten: a dense copy, and an f-order matrix read out in C order (a transpose)
+        exf = dev.extra(y_info=xi)
+        cases.append(Case("flatten_same_order", "flatten", n, 8 * n,
+                          lambda: ops.flattenFloat(exf, 0, b"c", Z.ptr, FL.ptr, X.ptr, X.info_ptr),
+                          lambda lib: (lib.flatten(0, "c", zc, flat, x, xi), zc)[1], True, Z.get))
+        exff = dev.extra(y_info=xfi)
+        cases.append(Case("flatten_f_to_c", "flatten", n, 8 * n,
+                          lambda: ops.flattenFloat(exff, 0, b"c", Z.ptr, FL.ptr, X.ptr, XF.ptr),
+                          lambda lib: (lib.flatten(0, "c", zc, flat, x, xfi), zc)[1], False, Z.get))
+        # tear: 1024 rows of 256 KiB into 1024 separate buffers
+        TG = [dev.empty(4 * t_len) for _ in range(t_rows)]
+        w._operands.extend(TG)
+        TT = w.raw(table(TG))
+        TXI, TZI = w.raw(np.ascontiguousarray(ti_x, dtype=np.int64)), w.raw(np.ascontiguousarray(ti_z, dtype=np.int64))
+        TTI, TTO = w.raw(tad_tear[0]), w.raw(tad_tear[1])
+        cases.append(Case("tear_rows", "tear", n, 8 * n,
+                          lambda: ops.tearFloat(ex, X.ptr, TXI.ptr, TT.ptr, TZI.ptr, TTI.ptr, TTO.ptr),
+                          None, True, lambda: TG[5].download(F32, t_len)))
+        # shuffle: every row trades places with a partner, in place
+        S = w.operand(x, xi)
+        SX, SI = w.raw(table([S.buf])), w.raw(table([S.dinfo]))
+        STI, STO = w.raw(table([TI])), w.raw(table([TO]))
+        M = w.raw(smap)
+        cases.append(Case("shuffle_rows", "shuffle", n, 8 * n,
+                          lambda: ops.shuffleFloat(ex, SX.ptr, SI.ptr, SX.ptr, SI.ptr, 1, M.ptr, STI.ptr, STO.ptr),
+                          None, True, S.get))
+        # conversions
+        H = w.raw(xh)
+        cases.append(Case("convert_float_to_half", "convert", n, 6 * n,
+                          lambda: ops.convertTypes(ex, 6, X.ptr, n, 3, H.ptr),
+                          lambda lib: (lib.convert(6, x, 3, hc), hc)[1], True, lambda: H.download(np.float16, n)))
+        cases.append(Case("convert_half_to_float", "convert", n, 6 * n,
+                          lambda: ops.convertTypes(ex, 3, H.ptr, n, 6, Z.ptr),
+                          lambda lib: (lib.convert(3, xh, 6, zc), zc)[1], True, Z.get))
+        return cases
+
+    return _replicated(dev, "data movement: pullRows, concat, flatten, tear, shuffle, convert; fp32 [%d,%d]" % (rows, cols), 8 * n,
+                       dict(x=x, xi=xi, perm=perm, smap=smap), device_set, copies)
+
+
 # ---- configs[4]: random fills and dropout ---------------------------------------------------------------
 def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data_seed=5, copies=None):
     ops = dev.ops
