@@ -90,8 +90,12 @@ __device__ __forceinline__ void copyRun(const T *src, Long se, const Long *sInfo
     }
 }
 
-// A block works on one long TAD or on four short ones (a wave each)
-__device__ __forceinline__ int lanesPerTad(Long tadLength) { return tadLength >= 1024 ? kBlock : kWave; }
+// A block works on one long TAD, on four shorter ones (a wave each) or on sixteen short ones, sized so that a lane
+// keeps about four 16-byte vectors in flight
+template <typename T> __device__ __forceinline__ int lanesPerTad(Long tadLength) {
+    const Long vectors = tadLength / Pack<T>::N;
+    return vectors >= 1024 ? kBlock : (vectors >= 256 ? kWave : 16);
+}
 
 // ---- pullRows: z TAD idx <- x TAD indexes[idx] ---------------------------------------------------------------
 template <typename T>
@@ -99,7 +103,7 @@ __global__ void __launch_bounds__(kBlock) pullRowsKernel(const T *x, T *z, Long 
                                                          const Long *tadOffsets, const Long *zTadInfo, const Long *zTadOffsets) {
     const Long tadLength = dLength(tadInfo);
     const Long xe = dEws(tadInfo), ze = dEws(zTadInfo);
-    const int lanes = lanesPerTad(tadLength), groups = kBlock / lanes;
+    const int lanes = lanesPerTad<T>(tadLength), groups = kBlock / lanes;
     const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
     for (Long idx = (Long)blockIdx.x * groups + g; idx < n; idx += (Long)gridDim.x * groups)
         copyRun<T, false>(x + tadOffsets[indexes[idx]], xe, tadInfo, z + zTadOffsets[idx], ze, zTadInfo, tadLength, lane, lanes);
@@ -112,7 +116,7 @@ __global__ void __launch_bounds__(kBlock) tearKernel(const T *x, const Long *xIn
     const Long tadLength = dLength(tadInfo);
     const Long numTads = dLength(xInfo) / tadLength;
     const Long xe = dEws(tadInfo), ze = dEws(zInfo);
-    const int lanes = lanesPerTad(tadLength), groups = kBlock / lanes;
+    const int lanes = lanesPerTad<T>(tadLength), groups = kBlock / lanes;
     const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
     for (Long r = (Long)blockIdx.x * groups + g; r < numTads; r += (Long)gridDim.x * groups)
         copyRun<T, true>(x + tadOffsets[r], xe, tadInfo, targets[r], ze, zInfo, tadLength, lane, lanes);
@@ -133,7 +137,7 @@ __global__ void __launch_bounds__(kBlock) shuffleKernel(T *const *xs, const Long
         const Long tadLength = dLength(ti);
         const Long numTads = dLength(xInfos[f]) / tadLength;
         const Long ews = dEws(ti);
-        const int lanes = lanesPerTad(tadLength), groups = kBlock / lanes;
+        const int lanes = lanesPerTad<T>(tadLength), groups = kBlock / lanes;
         const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
         for (Long r = (Long)blockIdx.x * groups + g; r < numTads; r += (Long)gridDim.x * groups) {
             const int m = map[r];
@@ -199,7 +203,6 @@ __global__ void __launch_bounds__(kBlock) concatPrefixKernel(const Long *const *
 template <typename T>
 __global__ void __launch_bounds__(kBlock) concatKernel(const T *const *data, const Long *const *infos, T *z, ConcatView v,
                                                        const Long *cum, int n) {
-    constexpr int VEC = Pack<T>::N;
     for (int r = blockIdx.y; r < n; r += gridDim.y) {
         const Long *si = infos[r];
         const T *x = data[r];
@@ -209,21 +212,18 @@ __global__ void __launch_bounds__(kBlock) concatKernel(const T *const *data, con
         if (rank == v.rank && v.zContig && dOrder(si) == 'c' && dEws(si) == 1) {
             const Long run = dShape(si)[v.dim] * v.inner;  // contiguous on both sides
             const Long zRun = v.dimTotal * v.inner;        // distance between consecutive runs in z
+            const Long outer = run > 0 ? len / run : 0;
             T *zb = z + start * v.inner;
-            if (run % VEC == 0 && zRun % VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-                (reinterpret_cast<uintptr_t>(zb) & 15) == 0) {
-                const Long runV = run / VEC, zRunV = zRun / VEC, nv = len / VEC;
-                const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x);
-                Pack<T> *zv = reinterpret_cast<Pack<T> *>(zb);
-                for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < nv; i += (Long)gridDim.x * kBlock) {
-                    const Long o = i / runV;
-                    storePack(zv + o * zRunV + (i - o * runV), loadPack(xv + i));
-                }
+            if (outer * 4 <= (Long)gridDim.x) {
+                // few long runs: all threads of this input share each run
+                for (Long o = 0; o < outer; o++)
+                    copyRun<T, false>(x + o * run, 1, nullptr, zb + o * zRun, 1, nullptr, run, (int)(blockIdx.x * kBlock + threadIdx.x),
+                                      (int)(gridDim.x * kBlock));
             } else {
-                for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < len; i += (Long)gridDim.x * kBlock) {
-                    const Long o = i / run;
-                    zb[o * zRun + (i - o * run)] = x[i];
-                }
+                const int lanes = lanesPerTad<T>(run), groups = kBlock / lanes;
+                const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
+                for (Long o = (Long)blockIdx.x * groups + g; o < outer; o += (Long)gridDim.x * groups)
+                    copyRun<T, false>(x + o * run, 1, nullptr, zb + o * zRun, 1, nullptr, run, lane, lanes);
             }
         } else if (rank == v.rank) {
             const Long *shape = dShape(si), *stride = dStride(si);
@@ -239,6 +239,83 @@ __global__ void __launch_bounds__(kBlock) concatKernel(const T *const *data, con
             }
         }
     }
+}
+
+// ---- strided copy whose destination stride is the EWS field of a device shapeInfo ---------------------------------
+// (flatten with equal orders: the result's shapeInfo is only known on the device, and reading one field of it here
+// spares the host a stream synchronisation)
+template <typename T>
+__global__ void __launch_bounds__(kBlock) copyToEwsKernel(const T *x, Long xe, T *z, const Long *zInfo, Long n) {
+    Long ze = dEws(zInfo);
+    if (ze < 1) ze = 1;
+    copyRun<T, false>(x, xe, nullptr, z, ze, nullptr, n, (int)(blockIdx.x * kBlock + threadIdx.x), (int)(gridDim.x * kBlock));
+}
+template <typename T> void launchCopyToEws(hipStream_t s, const T *x, Long xe, T *z, const Long *zInfo, Long n) {
+    if (n <= 0) return;
+    hipLaunchKernelGGL((copyToEwsKernel<T>), dim3(gridFor(n, (Long)kBlock * Pack<T>::N * 4, kGridCap * 2)), dim3(kBlock), 0, s, x, xe,
+                       z, zInfo, n);
+}
+
+// ---- transposing copy: z[r * zRowStride + c] = x[r + c * xColStride] --------------------------------------------
+// x is contiguous along r, z along c (an f-order matrix read out in C order, or the other way round).  A block moves
+// a 64 x 64 tile through LDS: it is read with the lanes running along r and written with the lanes running along c,
+// so both sides see full-width accesses; ACC elements per access (a 16-byte vector, or 1 when shapes or alignment
+// do not allow vectors).  The tile rows are padded by one element, which spreads both access patterns over the banks.
+static constexpr int kTile = 64;
+template <typename T, int ACC>
+__global__ void __launch_bounds__(kBlock) transposeCopyKernel(const T *x, T *z, Long rows, Long cols, Long xColStride,
+                                                              Long zRowStride) {
+    __shared__ T tile[kTile][kTile + 1];  // tile[c][r]
+    constexpr int LANES = kTile / ACC;    // threads along the contiguous direction
+    constexpr int STEP = kBlock / LANES;  // lines of the other direction per pass
+    const int fast = (threadIdx.x % LANES) * ACC, slow = threadIdx.x / LANES;
+    const Long r0 = (Long)blockIdx.x * kTile;
+    const Long colTiles = (cols + kTile - 1) / kTile;
+    for (Long ct = blockIdx.y; ct < colTiles; ct += gridDim.y) {
+        const Long c0 = ct * kTile;
+#pragma unroll
+        for (int lc = slow; lc < kTile; lc += STEP) {
+            const Long r = r0 + fast, c = c0 + lc;
+            if (r < rows && c < cols) {
+                const T *src = x + r + c * xColStride;
+                if (ACC > 1) {
+                    const Pack<T> p = loadPack(reinterpret_cast<const Pack<T> *>(src));
+#pragma unroll
+                    for (int k = 0; k < ACC; k++) tile[lc][fast + k] = p.v[k % Pack<T>::N];
+                } else {
+                    tile[lc][fast] = src[0];
+                }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int lr = slow; lr < kTile; lr += STEP) {
+            const Long r = r0 + lr, c = c0 + fast;
+            if (r < rows && c < cols) {
+                T *dst = z + r * zRowStride + c;
+                if (ACC > 1) {
+                    Pack<T> p;
+#pragma unroll
+                    for (int k = 0; k < ACC; k++) p.v[k % Pack<T>::N] = tile[fast + k][lr];
+                    storePack(reinterpret_cast<Pack<T> *>(dst), p);
+                } else {
+                    dst[0] = tile[fast][lr];
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+template <typename T>
+void launchTransposeCopy(hipStream_t s, const T *x, T *z, Long rows, Long cols, Long xColStride, Long zRowStride) {
+    if (rows <= 0 || cols <= 0) return;
+    constexpr int N = Pack<T>::N;
+    const Long rowTiles = (rows + kTile - 1) / kTile, colTiles = (cols + kTile - 1) / kTile;
+    const dim3 grid((unsigned)rowTiles, (unsigned)(colTiles < 65535 ? colTiles : 65535));
+    const bool vec = rows % N == 0 && cols % N == 0 && xColStride % N == 0 && zRowStride % N == 0 &&
+                     (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(z) & 15) == 0;
+    if (vec) hipLaunchKernelGGL((transposeCopyKernel<T, N>), grid, dim3(kBlock), 0, s, x, z, rows, cols, xColStride, zRowStride);
+    else hipLaunchKernelGGL((transposeCopyKernel<T, 1>), grid, dim3(kBlock), 0, s, x, z, rows, cols, xColStride, zRowStride);
 }
 
 template <typename T>
@@ -270,7 +347,7 @@ void launchConcat(hipStream_t s, const T *const *data, const Long *const *infos,
     const int gy = n < 65535 ? n : 65535;
     int budget = (kGridCap * 4) / gy;
     if (budget < 1) budget = 1;
-    const int gx = gridFor(maxLength > 0 ? maxLength : 1, (Long)kBlock * Pack<T>::N, budget);
+    const int gx = gridFor(maxLength > 0 ? maxLength : 1, (Long)kBlock * Pack<T>::N * 4, budget);  // four vectors a thread
     hipLaunchKernelGGL((concatKernel<T>), dim3(gx, gy), dim3(kBlock), 0, s, data, infos, z, v, cum, n);
 }
 
@@ -324,7 +401,9 @@ bool launchConvert(hipStream_t s, int srcType, const void *x, Long n, int dstTyp
                                 Long);                                                                                       \
     template void launchShuffle<T>(hipStream_t, T *const *, const Long *const *, T *const *, int, const int *,               \
                                    const Long *const *, const Long *const *, Long);                                          \
-    template void launchConcat<T>(hipStream_t, const T *const *, const Long *const *, T *, const ConcatView &, int, Long, Long *);
+    template void launchConcat<T>(hipStream_t, const T *const *, const Long *const *, T *, const ConcatView &, int, Long, Long *); \
+    template void launchTransposeCopy<T>(hipStream_t, const T *, T *, Long, Long, Long, Long);                            \
+    template void launchCopyToEws<T>(hipStream_t, const T *, Long, T *, const Long *, Long);
 INST(float)
 INST(float16)
 INST(double)

@@ -146,6 +146,11 @@ void launchShuffle(hipStream_t stream, T *const *xs, const Long *const *xInfos, 
 template <typename T>
 void launchConcat(hipStream_t stream, const T *const *data, const Long *const *infos, T *z, const ConcatView &view,
                   int numArrays, Long maxLength, Long *cum);
+// z[i * ews(zInfo)] = x[i * xe]; zInfo is a device shapeInfo, read by the kernel
+template <typename T> void launchCopyToEws(hipStream_t stream, const T *x, Long xe, T *z, const Long *zInfo, Long n);
+// z[r * zRowStride + c] = x[r + c * xColStride] for r < rows, c < cols, through LDS tiles
+template <typename T>
+void launchTransposeCopy(hipStream_t stream, const T *x, T *z, Long rows, Long cols, Long xColStride, Long zRowStride);
 // srcType / dstType: 3 half, 6 float, 7 double (type_conversions.h:11-18); false for any other pair
 bool launchConvert(hipStream_t stream, int srcType, const void *x, Long n, int dstType, void *z);
 

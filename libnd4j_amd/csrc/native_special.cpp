@@ -21,18 +21,25 @@ constexpr int kIdentity = 27;  // TRANSFORM_OPS Identity: z = x
 template <typename T>
 void flattenImpl(Nd4jPointer *extra, int offset, char order, T *result, Long *resultInfo, T *input, Long *inputInfo) {
     hipStream_t s = streamOf(extra);
-    std::vector<Long> sx, sz;
+    std::vector<Long> sx;
     const Long *hx = hostShapeInfo(extra, X_HOST_Y_SHAPE, inputInfo, sx, s);
-    const Long *hz = hostShapeInfo(nullptr, 0, resultInfo, sz, s);  // no slot carries the result's host copy
-    if (hx == nullptr || hz == nullptr) return;
+    if (hx == nullptr) return;
     const Long n = siNumel(hx);
     if (n <= 0) return;
-    const Long xe = siEws(hx), ze = siEws(hz);
+    const Long xe = siEws(hx);
     T *z = result + offset;
     bool ok;
-    if (siOrder(hx) == order && xe >= 1 && ze >= 1) {
-        // same order on both sides: the input's memory order is the requested order
-        ok = launchTransformStrided<T>(s, kIdentity, input, xe, z, ze, nullptr, n);
+    if (siOrder(hx) == order && xe >= 1) {
+        // same order on both sides: the input's memory order is the requested order.  Only this branch honours the
+        // result's element-wise stride; no slot carries a host copy of the result's shapeInfo, so unless the argument
+        // itself is host memory the kernel reads the field
+        if (resultInfo == nullptr || !isDeviceMemory(resultInfo)) {
+            const Long ze = (resultInfo != nullptr && siEws(resultInfo) >= 1) ? siEws(resultInfo) : 1;
+            ok = launchTransformStrided<T>(s, kIdentity, input, xe, z, ze, nullptr, n);
+        } else {
+            launchCopyToEws<T>(s, input, xe, z, resultInfo, n);
+            ok = true;
+        }
     } else {
         // walk the input in the requested order (F order = C order over the reversed dimensions), write densely
         const int rank = siRank(hx);
@@ -44,6 +51,12 @@ void flattenImpl(Nd4jPointer *extra, int offset, char order, T *result, Long *re
         }
         DimMap xm, zm;
         ownCanon(rank, shp, str, xm);
+        if (xm.rank == 2 && xm.stride[0] == 1 && xm.stride[1] >= (Long)xm.shape[0]) {
+            // the input runs along the slower dimension of the requested order: a matrix transpose
+            launchTransposeCopy<T>(s, input, z, xm.shape[0], xm.shape[1], xm.stride[1], xm.shape[1]);
+            checkLaunch("flatten", s);
+            return;
+        }
         zm.rank = 1;
         zm.shape[0] = (unsigned)(n > 0xffffffffLL ? 0xffffffffu : n);
         zm.stride[0] = 1;
