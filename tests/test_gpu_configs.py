@@ -126,6 +126,53 @@ def test_config3_summary_stats_and_softmax_chain(gpu, lib):
         truth = np.exp(m - m.max(axis=1, keepdims=True))
         truth /= truth.sum(axis=1, keepdims=True)
         assert np.all(np.abs(sm - truth) <= 2e-5 * truth + 1e-30)
+        # the same softmax as one call, on the f-order matrix and on the same memory read as a c-order matrix
+        fused = _run(w.case("softmax_fused_forder")).astype(np.float64).reshape(cols, rows).T
+        assert np.all(np.abs(fused - truth) <= 2e-5 * truth + 1e-30)
+        assert np.all(np.abs(fused.sum(axis=1) - 1.0) <= 1e-5)
+        mc = x.astype(np.float64).reshape(rows, cols)
+        truth_c = np.exp(mc - mc.max(axis=1, keepdims=True))
+        truth_c /= truth_c.sum(axis=1, keepdims=True)
+        fused = _run(w.case("softmax_fused_corder")).astype(np.float64).reshape(rows, cols)
+        assert np.all(np.abs(fused - truth_c) <= 2e-5 * truth_c + 1e-30)
+        want = w.case("softmax_fused_corder").cpu(lib).astype(np.float64).reshape(rows, cols)
+        assert np.all(np.abs(fused - want) <= 2e-5 * np.maximum(want, 1e-30))
+        logsm = _run(w.case("logsoftmax_fused_corder")).astype(np.float64).reshape(rows, cols)
+        assert np.all(np.abs(logsm - np.log(truth_c)) <= 2e-5 * np.abs(np.log(truth_c)) + 1e-6)
+        # IsMax: one-hot of the first maximum, whole array and per row; bit-exact
+        xf = x.reshape(rows, cols)
+        # (the winning index travels as a value of the data type, in the reference too - execIndexReduceScalarFloat
+        # returns a float - so beyond 2^24 elements the one lands on the index rounded to float)
+        got = _run(w.case("ismax_whole"))
+        assert got.sum() == 1 and got[int(np.float32(np.argmax(x)))] == 1
+        got = _run(w.case("ismax_dim1")).reshape(rows, cols)
+        assert np.all(got.sum(axis=1) == 1)
+        assert np.array_equal(np.argmax(got, axis=1), np.argmax(xf, axis=1))
+    finally:
+        w.free()
+
+
+def test_data_movement_at_benchmark_size(gpu, lib):
+    w = workloads.data_movement(gpu.dev, copies=1)
+    try:
+        rows, cols = 65536, 1024
+        x, perm, smap = w.host["x"], w.host["perm"], w.host["smap"]
+        m = x.reshape(rows, cols)
+        assert np.array_equal(_run(w.case("pullrows_permute")).reshape(rows, cols), m[perm])
+        assert np.array_equal(_run(w.case("concat_dim0")), x)      # row blocks of x put back together
+        assert np.array_equal(_run(w.case("concat_dim1")), x)      # column blocks of x put back together
+        assert np.array_equal(_run(w.case("concat_dim1")), w.case("concat_dim1").cpu(lib))
+        assert np.array_equal(_run(w.case("flatten_same_order")), x)
+        # the buffer read as an f-order [rows, cols] matrix, flattened in C order
+        assert np.array_equal(_run(w.case("flatten_f_to_c")), x.reshape(cols, rows).T.ravel())
+        assert np.array_equal(_run(w.case("tear_rows")), x.reshape(1024, -1)[5])
+        want = m.copy()
+        a = np.nonzero(smap >= 0)[0]
+        want[a], want[smap[a]] = m[smap[a]], m[a]
+        assert np.array_equal(_run(w.case("shuffle_rows")).reshape(rows, cols), want)
+        half = _run(w.case("convert_float_to_half"))
+        assert np.array_equal(half.view(np.uint16), x.astype(np.float16).view(np.uint16))
+        assert np.array_equal(_run(w.case("convert_half_to_float")), x.astype(np.float16).astype(np.float32))
     finally:
         w.free()
 
