@@ -473,7 +473,13 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
     }
     ResolvedTad tx, tz;
     if (!resolveTad(extra, X_HOST_TAD_SHAPE, X_DEV_TAD_OFFSETS, hx, devDims, dimLen, tx, s)) return true;
-    if (!resolveTad(nullptr, 0, 0, hz, devDims, dimLen, tz, s)) return true;
+    // a result laid out like the input shares its TAD tables (the reference's fill kernel always assumes so,
+    // blas/cuda/NativeOps.cu:3277-3290); any other layout gets tables of its own
+    bool sameLayout = siRank(hz) == rank && siOrder(hz) == siOrder(hx);
+    for (int d = 0; sameLayout && d < rank; d++)
+        sameLayout = siShape(hz)[d] == siShape(hx)[d] && siStride(hz)[d] == siStride(hx)[d];
+    if (sameLayout) tz = tx;
+    else if (!resolveTad(nullptr, 0, 0, hz, devDims, dimLen, tz, s)) return true;
     Scratch sc = scratchFor(s, kScalarArea + (size_t)tx.numTads * sizeof(T) + (size_t)(4u << 20));
     T *index = reinterpret_cast<T *>(sc.rest.ptr);
     Workspace rest = sc.rest;

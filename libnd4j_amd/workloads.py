@@ -361,7 +361,7 @@ def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
                           lambda lib: (lib.transform(T_ISMAX, x, xci, tc, xci, None), tc)[1], True, T.get))
         DM = w.raw(np.array([1], np.int32))
         EP = w.raw(np.array([1, 1], F32))
-        ex_m = dev.extra(xci, z_info=xci)
+        ex_m = dev.extra(xci, z_info=xci, tad=dev.tad(xci, [1]))  # TAD tables in slots 9-11, as nd4j passes them
         ex_m[15] = DM.ptr
         ex_m[18] = 1
         ismax_params = np.array([1, 1], F32)
