@@ -198,23 +198,30 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
         if ((reinterpret_cast<uintptr_t>(x + off[0]) & 15) != 0 || (tadEws % VEC) != 0) vec = false;
         if (vec) {
             const T *base = x + off[0];
-            Long j = j0 + wave;
-            for (; j + 3 * WAVES < j1; j += 4 * WAVES) {
-                Pack<T> pk[4];
+            // Row ranges start a power-of-two number of bytes apart, so blocks that all began at the top of their range
+            // would keep hitting the same few memory channels: each range is walked from a different row, wrapping round.
+            const Long span = j1 - j0;
+            const Long turn = span >= 8 * WAVES ? (((Long)blockIdx.y * 3) % (span / (4 * WAVES))) * (4 * WAVES) : 0;
+            for (int part = 0; part < 2; part++) {
+                const Long a = part == 0 ? j0 + turn : j0, b = part == 0 ? j1 : j0 + turn;
+                Long j = a + wave;
+                for (; j + 3 * WAVES < b; j += 4 * WAVES) {
+                    Pack<T> pk[4];
 #pragma unroll
-                for (int u = 0; u < 4; u++) pk[u] = loadPack(reinterpret_cast<const Pack<T> *>(base + (j + u * WAVES) * tadEws));
+                    for (int u = 0; u < 4; u++) pk[u] = loadPack(reinterpret_cast<const Pack<T> *>(base + (j + u * WAVES) * tadEws));
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
+                    for (int u = 0; u < 4; u++) {
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) pe[e].accumulate(acc[e], toCompute(pk[u].v[e]), j + u * WAVES);
+                        for (int e = 0; e < VEC; e++) pe[e].accumulate(acc[e], toCompute(pk[u].v[e]), j + u * WAVES);
+                    }
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) pe[e].checkpoint(acc[e]);
                 }
+                for (; j < b; j += WAVES) {
+                    Pack<T> pk = loadPack(reinterpret_cast<const Pack<T> *>(base + j * tadEws));
 #pragma unroll
-                for (int e = 0; e < VEC; e++) pe[e].checkpoint(acc[e]);
-            }
-            for (; j < j1; j += WAVES) {
-                Pack<T> pk = loadPack(reinterpret_cast<const Pack<T> *>(base + j * tadEws));
-#pragma unroll
-                for (int e = 0; e < VEC; e++) { pe[e].accumulate(acc[e], toCompute(pk.v[e]), j); pe[e].checkpoint(acc[e]); }
+                    for (int e = 0; e < VEC; e++) { pe[e].accumulate(acc[e], toCompute(pk.v[e]), j); pe[e].checkpoint(acc[e]); }
+                }
             }
         } else {
 #pragma unroll
