@@ -356,6 +356,30 @@ void reduce3Dims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T 
         reduce3Full<T>(extra, opNum, x, xInfo, params, y, yInfo, z);
         return;
     }
+    if (siNumel(hx) < siNumel(hy)) {
+        // x is the single run, y has the TADs (reduce3.h:1186-1215 picks the longer operand to iterate over)
+        ResolvedTad ty;
+        if (!resolveTad(nullptr, 0, 0, hy, dimension, dimLen, ty, s)) return;
+        if (siNumel(hx) != ty.tadLength) {
+            std::printf("reduce3: x holds %lld elements, neither the %lld of y nor the %lld of one TAD\n", (long long)siNumel(hx),
+                        (long long)siNumel(hy), (long long)ty.tadLength);
+            return;
+        }
+        Reduce3Launch in;
+        in.runLength = ty.tadLength;
+        in.numOut = ty.numTads;
+        in.xDiv = 1;
+        in.yMod = ty.numTads > 0 ? ty.numTads : 1;
+        in.xOffsets = nullptr;
+        in.yOffsets = ty.devOffsets;
+        const char order = siOrder(ty.hostInfo) == 'f' ? 'f' : 'c';
+        orderedLinearMap(siShape(hx), siStride(hx), siRank(hx), order, in.xm);
+        orderedLinearMap(siShape(ty.hostInfo), siStride(ty.hostInfo), siRank(ty.hostInfo), order, in.ym);
+        Scratch sc = scratchFor(s);
+        if (!launchReduce3<T>(s, opNum, x, y, z, params, in, sc.rest)) { reportUnknownOp("reduce3", opNum); return; }
+        checkLaunch("execReduce3", s);
+        return;
+    }
     ResolvedTad tx;
     if (!resolveTad(extra, X_HOST_TAD_SHAPE, X_DEV_TAD_OFFSETS, hx, dimension, dimLen, tx, s)) return;
     Reduce3Launch in;

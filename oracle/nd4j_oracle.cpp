@@ -735,6 +735,15 @@ static void reduce3Dims(int op, T *x, Long *xi, T *extra, T *y, Long *yi, T *z, 
     if (op < 0 || op > 7) { printf("[ERROR] Unknown opNum=%d (oracle reduce3)\n", op); return; }
     if (siIsScalar(zi)) { z[0] = reduce3Scalar<T>(op, x, xi, extra, y, yi); return; }
     const T eps = extra != nullptr ? extra[0] : (T)0.0f;
+    if (siNumel(xi) < siNumel(yi)) {
+        // x is the single run, y has the TADs (reduce3.h:1186-1215 iterates over the longer operand)
+        TadPack ty;
+        computeTad(yi, dim, dimLen, ty, true);
+        const Long n = siNumel(ty.shapeInfo.data());
+        const char order = siOrder(ty.shapeInfo.data()) == 'f' ? 'f' : 'c';
+        for (Long r = 0; r < ty.numTads; r++) z[r] = reduce3Run<T>(op, x, xi, y + ty.offsets[r], ty.shapeInfo.data(), order, n, eps);
+        return;
+    }
     TadPack tx;
     computeTad(xi, dim, dimLen, tx, true);
     const Long n = siNumel(tx.shapeInfo.data());

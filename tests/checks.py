@@ -98,6 +98,17 @@ def check_reference_fixtures(be):
         xi = np.array(c["x_info"], np.int64)
         x = np.linspace(c["linspace"][0], c["linspace"][1], 25).astype(f32)
         assert float(be.indexreduce_scalar(c["opNum"], x, xi)) == c["expected"], c["source"]
+    for c in fx["reduce3"]:
+        x, y = np.array(c["x"], f32), np.array(c["y"], f32)
+        xi = shape_info_np(c["shape"])
+        yi = shape_info_np(c.get("y_shape", c["shape"]))
+        if c["kind"] == "scalar":
+            got = np.array([be.reduce3_scalar(c["opNum"], x, xi, y, yi)], f32)
+        elif c["kind"] == "all":
+            got = be.reduce3_all(c["opNum"], x, xi, y, yi, None, c["dims"], len(c["expected"]))
+        else:
+            got = be.reduce3(c["opNum"], x, xi, y, yi, np.zeros(1, f32), c["dims"], len(c["expected"]))
+        assert np.allclose(got, c["expected"], atol=c["tol"] + 1e-6 * (c["tol"] > 0), rtol=0), "%s: %r" % (c["source"], got)
     for c in fx["summary_stats"]:
         got = be.summarystats(c["opNum"], c["bias"], np.array(c["x"], f32), shape_info_np(c["shape"]), c["dims"],
                               len(c["expected"]))
