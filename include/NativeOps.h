@@ -22,6 +22,16 @@
 
 #include "nd4j_types.h"
 
+#include <string>
+
+// Return types of three graph members that are only declared here (see "Members outside the path" below)
+namespace nd4j {
+class ShapeList;
+namespace graph {
+template <typename T> class VariablesSet;
+}
+}  // namespace nd4j
+
 #ifndef ND4J_EXPORT
 #define ND4J_EXPORT __attribute__((visibility("default")))
 #endif
@@ -149,6 +159,22 @@ public:
     ND4J_SCALAR_MEMBERS(Float, float, float)
     ND4J_SCALAR_MEMBERS(Half, float16, float)
     ND4J_SCALAR_MEMBERS(Double, double, double)
+    // the reference's indexed Double variant carries an extra element count (blas/NativeOps.h:419-430)
+    void execScalarDouble(Nd4jPointer *extraPointers, int opNum, double *x, Nd4jLong *xShapeInfo, double *result,
+                          Nd4jLong *resultShapeInfo, double scalar, double *extraParams, Nd4jLong n, Nd4jLong *xIndexes,
+                          Nd4jLong *resultIndexes);
+
+    // n buffers of `length` elements summed (accumulate) or averaged (average) into dz; with `propagate` the average
+    // is written back to every input as well.  dx is a device table of device pointers, dz may be null for average.
+    // Reference: blas/NativeOps.h:1980-2040, kernels include/loops/special_kernels.h:700-822.  On one GPU all n
+    // buffers are local; the reference's use of the same call across peer devices is not part of this build.
+#define ND4J_AVERAGE_MEMBERS(SUFFIX, T)                                                              \
+    void average##SUFFIX(Nd4jPointer *extras, Nd4jPointer *dx, T *dz, int n, Nd4jLong length, bool propagate); \
+    void accumulate##SUFFIX(Nd4jPointer *extras, Nd4jPointer *dx, T *dz, int n, Nd4jLong length);
+    ND4J_AVERAGE_MEMBERS(Float, float)
+    ND4J_AVERAGE_MEMBERS(Half, float16)
+    ND4J_AVERAGE_MEMBERS(Double, double)
+#undef ND4J_AVERAGE_MEMBERS
 
     ND4J_SPECIAL_MEMBERS(Float, float)
     ND4J_SPECIAL_MEMBERS(Half, float16)
@@ -210,6 +236,103 @@ public:
     void setGridLimit(int gridSize);
     void setElementThreshold(int num);
     void setTADThreshold(int num);
+
+    // ---- Members outside the path ------------------------------------------------------------------
+    // Everything else the reference's class declares (blas/NativeOps.h: 1557-1605 specialConcat, 1609 initializeFunctions,
+    // 2047-2060 P2P switches, 2172-2330 aggregates, 2564-2760 meta-ops, 2815-2870 numpy helpers, 2902-2935 gradient
+    // compression, 2940-2960 sort, 2963-3026 mmap, graphs, custom ops and their helpers), with the same signatures,
+    // so that a binding generated from the reference header links against this library.  They do
+    // no work here: each prints one line naming itself and returns 0 / null / false (isP2PAvailable,
+    // isExperimentalEnabled: false; pointerForAddress, lengthForShapeBufferPointer and the delete*Array helpers do
+    // what their names say).  Implemented in libnd4j_amd/csrc/native_stubs.cpp.
+#define ND4J_OFFPATH_MEMBERS(SUFFIX, T)                                                                            \
+    void specialConcat##SUFFIX(Nd4jPointer *extraPointers, int dimension, int numArrays, Nd4jPointer *data,       \
+                               Nd4jPointer *inputShapeInfo, T *result, Nd4jLong *resultShapeInfo,                 \
+                               Nd4jPointer *tadPointers, Nd4jPointer *offsetPointers);                            \
+    void execAggregate##SUFFIX(Nd4jPointer *extraPointers, int opNum, T **arguments, int numArguments,            \
+                               Nd4jLong **shapeArguments, int numShapeArguments, int *indexArguments,             \
+                               int numIndexArguments, int **intArrays, int numIntArrays, T *realArguments,        \
+                               int numRealArguments);                                                             \
+    void execAggregateBatch##SUFFIX(Nd4jPointer *extraPointers, int numAggregates, int opNum, int maxArgs,        \
+                                    int maxShapes, int maxIntArrays, int maxIntArraySize, int maxIdx, int maxReals, \
+                                    void *ptrToArguments);                                                        \
+    void execMetaPredicateStrided##SUFFIX(Nd4jPointer *extras, const int opTypeA, const int opNumA,               \
+                                          const int opTypeB, const int opNumB, Nd4jLong N, T *dx, Nd4jLong xStride, \
+                                          T *dy, Nd4jLong yStride, T *dz, Nd4jLong zStride, T *extraA, T *extraB, \
+                                          S scalarA, S scalarB);                                                  \
+    void execMetaPredicateShape##SUFFIX(Nd4jPointer *extras, const int opTypeA, const int opNumA, const int opTypeB, \
+                                        const int opNumB, Nd4jLong N, T *dx, Nd4jLong *xShapeInfo, T *dy,         \
+                                        Nd4jLong *yShapeInfo, T *dz, Nd4jLong *zShapeInfo, T *extraA, T *extraB,  \
+                                        S scalarA, S scalarB);                                                    \
+    Nd4jLong encodeBitmap##SUFFIX(Nd4jPointer *extraPointers, T *dx, Nd4jLong N, int *dz, float threshold);       \
+    void decodeBitmap##SUFFIX(Nd4jPointer *extraPointers, void *dx, Nd4jLong N, T *dz);                           \
+    void encodeThresholdP1##SUFFIX(Nd4jPointer *extraPointers, T *dx, Nd4jLong N, int *dz, float threshold);      \
+    void encodeThresholdP3##SUFFIX(Nd4jPointer *extraPointers, T *dx, int *offsets, Nd4jLong N, int *dz);         \
+    void decodeThreshold##SUFFIX(Nd4jPointer *extraPointers, void *dx, Nd4jLong N, T *dz);                        \
+    void sort##SUFFIX(Nd4jPointer *extraPointers, T *x, Nd4jLong *xShapeInfo, bool descending);                   \
+    void sortTad##SUFFIX(Nd4jPointer *extraPointers, T *x, Nd4jLong *xShapeInfo, int *dimension,                  \
+                         int dimensionLength, Nd4jLong *tadShapeInfo, Nd4jLong *tadOffsets, bool descending);     \
+    void sortCooIndices##SUFFIX(Nd4jPointer *extraPointers, Nd4jLong *indices, T *values, Nd4jLong length, int rank); \
+    Nd4jPointer executeFlatGraph##SUFFIX(Nd4jPointer *extraPointers, Nd4jPointer flatBufferPointer);              \
+    int execCustomOp##SUFFIX(Nd4jPointer *extraPointers, Nd4jLong hash, Nd4jPointer *inputBuffers,                \
+                             Nd4jPointer *inputShapes, int numInputs, Nd4jPointer *outputBuffers,                 \
+                             Nd4jPointer *outputShapes, int numOutputs, T *tArgs, int numTArgs, Nd4jLong *iArgs,  \
+                             int numIArgs, bool isInplace);                                                       \
+    nd4j::ShapeList *calculateOutputShapes##SUFFIX(Nd4jPointer *extraPointers, Nd4jLong hash,                     \
+                                                   Nd4jPointer *inputShapes, int numInputShapes, T *tArgs,        \
+                                                   int numTArgs, Nd4jLong *iArgs, int numIArgs);                  \
+    nd4j::ShapeList *calculateOutputShapes##SUFFIX(Nd4jPointer *extraPointers, Nd4jLong hash,                     \
+                                                   Nd4jPointer *inputBuffers, Nd4jPointer *inputShapes,           \
+                                                   int numInputShapes, T *tArgs, int numTArgs, Nd4jLong *iArgs,   \
+                                                   int numIArgs);                                                 \
+    int registerGraph##SUFFIX(Nd4jPointer *extraPointers, Nd4jLong graphId, Nd4jPointer flatBufferPointer);       \
+    nd4j::graph::VariablesSet<T> *executeStoredGraph##SUFFIX(Nd4jPointer *extraPointers, Nd4jLong graphId,        \
+                                                             Nd4jPointer *inputBuffers, Nd4jPointer *inputShapes, \
+                                                             int *inputIndices, int numInputs);                   \
+    void deleteVariablesSet##SUFFIX(Nd4jPointer pointer);                                                         \
+    Nd4jPointer getGraphState##SUFFIX(Nd4jLong id);                                                               \
+    void deleteGraphState##SUFFIX(Nd4jPointer state);                                                             \
+    Nd4jStatus execCustomOpWithScope##SUFFIX(Nd4jPointer *extraPointers, Nd4jPointer state, Nd4jLong opHash,      \
+                                             Nd4jLong *scopes, int numScopes, Nd4jPointer *inputBuffers,          \
+                                             Nd4jPointer *inputShapes, int numInputs, Nd4jPointer *outputBuffers, \
+                                             Nd4jPointer *outputShapes, int numOutputs);
+#define S float
+    ND4J_OFFPATH_MEMBERS(Float, float)
+    ND4J_OFFPATH_MEMBERS(Half, float16)
+#undef S
+#define S double
+    ND4J_OFFPATH_MEMBERS(Double, double)
+#undef S
+#undef ND4J_OFFPATH_MEMBERS
+    void execMetaPredicateReduceFloat(Nd4jPointer *extras, const int opTypeA, const int opNumA, const int opTypeB,
+                                      const int opNumB, float *dx, Nd4jLong *xShapeInfo, float *dy, Nd4jLong *yShapeInfo,
+                                      float *dz, Nd4jLong *zShapeInfo, int *dimension, int dimensionLength,
+                                      Nd4jLong *tadShapeInfo, Nd4jLong *tadOffsets, float *extraA, float *extraB,
+                                      float scalarA, float scalarB, bool scalarReturned);
+    void encodeThresholdP2Int(Nd4jPointer *extraPointers, int *dx, Nd4jLong N, int *dz);
+    Nd4jPointer executeProtoGraphFloat(Nd4jPointer *extraPointers, Nd4jPointer protoBufferPointer);
+    Nd4jPointer executeProtoGraphFloat(Nd4jPointer *extraPointers, const char *fileName);
+    void initializeFunctions(Nd4jPointer *functions);
+    void enableP2P(bool enable);
+    void checkP2P();
+    bool isP2PAvailable();
+    bool isExperimentalEnabled();
+    Nd4jPointer shapeBufferForNumpy(Nd4jPointer npyArray);
+    Nd4jPointer dataPointForNumpy(Nd4jPointer npArray);
+    Nd4jPointer numpyFromFile(std::string path);
+    void releaseNumpy(Nd4jPointer npyArray);
+    int lengthForShapeBufferPointer(Nd4jPointer buffer);
+    int elementSizeForNpyArray(Nd4jPointer npyArray);
+    Nd4jPointer pointerForAddress(Nd4jLong address);
+    Nd4jLong *mmapFile(Nd4jPointer *extraPointers, const char *fileName, Nd4jLong length);
+    void munmapFile(Nd4jPointer *extraPointers, Nd4jLong *ptrMap, Nd4jLong length);
+    const char *getAllCustomOps();
+    const char *getAllOperations();
+    void deleteShapeList(Nd4jPointer shapeList);
+    int unregisterGraph(Nd4jPointer *extraPointers, Nd4jLong graphId);
+    void deleteIntArray(Nd4jPointer pointer);
+    void deleteLongArray(Nd4jPointer pointer);
+    void deletePointerArray(Nd4jPointer pointer);
 };
 
 #undef ND4J_EXEC_MEMBERS

@@ -129,7 +129,7 @@ ND4J_C_REDUCE3(Double, double, double)
 #undef ND4J_C_REDUCE3
 
 /* Data-movement specials (blas/NativeOps.h:1457-1499 flatten, 1510-1555 concat, 1904-1967 pullRows, 2076-2130
- * shuffle, 2876-2899 tear, 2144 convertTypes); pointer conventions as documented in include/NativeOps.h. */
+ * shuffle, 2876-2899 tear, 2144 convertTypes, 1980-2040 average / accumulate of n local buffers); pointer conventions as documented in include/NativeOps.h. */
 #define ND4J_C_SPECIAL(SUFFIX, T)                                                                                \
     void nd4j_flatten##SUFFIX(Nd4jPointer *extraPointers, int offset, char order, T *result,                     \
                               Nd4jLong *resultShapeInfo, T *input, Nd4jLong *inputShapeInfo);                    \
@@ -143,7 +143,9 @@ ND4J_C_REDUCE3(Double, double, double)
                            Nd4jLong *zShapeInfo, Nd4jLong *tadShapeInfo, Nd4jLong *tadOffsets);                  \
     void nd4j_shuffle##SUFFIX(Nd4jPointer *extras, Nd4jPointer *dx, Nd4jPointer *xShapeInfo, Nd4jPointer *dz,    \
                               Nd4jPointer *zShapeInfo, int N, int *shuffleMap, Nd4jPointer *tadShapeInfo,        \
-                              Nd4jPointer *tadOffsets);
+                              Nd4jPointer *tadOffsets);                                                          \
+    void nd4j_average##SUFFIX(Nd4jPointer *extras, Nd4jPointer *dx, T *dz, int n, Nd4jLong length, int propagate); \
+    void nd4j_accumulate##SUFFIX(Nd4jPointer *extras, Nd4jPointer *dx, T *dz, int n, Nd4jLong length);
 ND4J_C_SPECIAL(Float, float)
 ND4J_C_SPECIAL(Half, float16)
 ND4J_C_SPECIAL(Double, double)

@@ -7,6 +7,7 @@
 
 typedef void *Nd4jPointer;
 typedef long long Nd4jLong;
+typedef int Nd4jStatus; /* include/pointercast.h:12 */
 
 #ifdef __cplusplus
 struct float16 {

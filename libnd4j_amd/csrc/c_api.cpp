@@ -168,6 +168,12 @@ ND4J_C_REDUCE3(Double, double, double)
     void nd4j_shuffle##SUFFIX(Nd4jPointer *e, Nd4jPointer *dx, Nd4jPointer *xs, Nd4jPointer *dz, Nd4jPointer *zs,  \
                               int N, int *map, Nd4jPointer *ti, Nd4jPointer *to) {                                 \
         guardVoid([&] { gOps.shuffle##SUFFIX(e, dx, xs, dz, zs, N, map, ti, to); });                               \
+    }                                                                                                              \
+    void nd4j_average##SUFFIX(Nd4jPointer *e, Nd4jPointer *dx, T *dz, int n, Nd4jLong length, int propagate) {     \
+        guardVoid([&] { gOps.average##SUFFIX(e, dx, dz, n, length, propagate != 0); });                            \
+    }                                                                                                              \
+    void nd4j_accumulate##SUFFIX(Nd4jPointer *e, Nd4jPointer *dx, T *dz, int n, Nd4jLong length) {                 \
+        guardVoid([&] { gOps.accumulate##SUFFIX(e, dx, dz, n, length); });                                         \
     }
 ND4J_C_SPECIAL(Float, float)
 ND4J_C_SPECIAL(Half, float16)

@@ -351,6 +351,48 @@ void launchConcat(hipStream_t s, const T *const *data, const Long *const *infos,
     hipLaunchKernelGGL((concatKernel<T>), dim3(gx, gy), dim3(kBlock), 0, s, data, infos, z, v, cum, n);
 }
 
+// ---- accumulate / average: z[i] = sum_k x[k][i] (/ n), optionally written back to every x[k] ------------------------
+// (special_kernels.h:700-822).  x is a device table of n device pointers.  The sum runs in the compute type, in table
+// order; one thread owns a 16-byte vector of the result.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) averageKernel(T *const *xs, T *z, int n, Long length, int average, int propagate) {
+    typedef typename Compute<T>::type C;
+    constexpr int VEC = Pack<T>::N;
+    // the vector part needs every buffer on a 16-byte boundary (whole device allocations are; views may not be)
+    bool aligned = z == nullptr || (reinterpret_cast<uintptr_t>(z) & 15) == 0;
+    for (int k = 0; k < n; k++) aligned = aligned && (reinterpret_cast<uintptr_t>(xs[k]) & 15) == 0;
+    const Long nvec = aligned ? length / VEC : 0;
+    for (Long v = (Long)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += (Long)gridDim.x * kBlock) {
+        C acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] = (C)0;
+        for (int k = 0; k < n; k++) {
+            const Pack<T> p = loadPack(reinterpret_cast<const Pack<T> *>(xs[k]) + v);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) acc[e] += toCompute(p.v[e]);
+        }
+        Pack<T> o;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) o.v[e] = fromCompute<T>(average ? acc[e] / (C)n : acc[e]);
+        if (z != nullptr) storePack(reinterpret_cast<Pack<T> *>(z) + v, o);
+        if (propagate)
+            for (int k = 0; k < n; k++) storePack(reinterpret_cast<Pack<T> *>(xs[k]) + v, o);
+    }
+    for (Long i = nvec * VEC + (Long)blockIdx.x * kBlock + threadIdx.x; i < length; i += (Long)gridDim.x * kBlock) {
+        C acc = (C)0;
+        for (int k = 0; k < n; k++) acc += toCompute(xs[k][i]);
+        const T o = fromCompute<T>(average ? acc / (C)n : acc);
+        if (z != nullptr) z[i] = o;
+        if (propagate)
+            for (int k = 0; k < n; k++) xs[k][i] = o;
+    }
+}
+template <typename T> void launchAverage(hipStream_t s, T *const *xs, T *z, int n, Long length, bool average, bool propagate) {
+    if (n <= 0 || length <= 0) return;
+    const int grid = gridFor(length, (Long)kBlock * Pack<T>::N, kGridCap * 4);
+    hipLaunchKernelGGL((averageKernel<T>), dim3(grid), dim3(kBlock), 0, s, xs, z, n, length, average ? 1 : 0, propagate ? 1 : 0);
+}
+
 // ---- conversions between half, float and double: z[i] = (D)(float)x[i] (type_conversions.h:38-49) -----------------
 template <typename S, typename D> __device__ __forceinline__ D convertOne(S v) {
     const float f = (float)toCompute(v);
@@ -403,7 +445,8 @@ bool launchConvert(hipStream_t s, int srcType, const void *x, Long n, int dstTyp
                                    const Long *const *, const Long *const *, Long);                                          \
     template void launchConcat<T>(hipStream_t, const T *const *, const Long *const *, T *, const ConcatView &, int, Long, Long *); \
     template void launchTransposeCopy<T>(hipStream_t, const T *, T *, Long, Long, Long, Long);                            \
-    template void launchCopyToEws<T>(hipStream_t, const T *, Long, T *, const Long *, Long);
+    template void launchCopyToEws<T>(hipStream_t, const T *, Long, T *, const Long *, Long);                              \
+    template void launchAverage<T>(hipStream_t, T *const *, T *, int, Long, bool, bool);
 INST(float)
 INST(float16)
 INST(double)

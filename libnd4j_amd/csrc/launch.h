@@ -151,6 +151,8 @@ template <typename T> void launchCopyToEws(hipStream_t stream, const T *x, Long 
 // z[r * zRowStride + c] = x[r + c * xColStride] for r < rows, c < cols, through LDS tiles
 template <typename T>
 void launchTransposeCopy(hipStream_t stream, const T *x, T *z, Long rows, Long cols, Long xColStride, Long zRowStride);
+// z[i] = sum over the n buffers in the device table xs (average: / n); propagate: also written back to each of them
+template <typename T> void launchAverage(hipStream_t stream, T *const *xs, T *z, int n, Long length, bool average, bool propagate);
 // srcType / dstType: 3 half, 6 float, 7 double (type_conversions.h:11-18); false for any other pair
 bool launchConvert(hipStream_t stream, int srcType, const void *x, Long n, int dstType, void *z);
 

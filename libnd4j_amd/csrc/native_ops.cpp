@@ -275,6 +275,10 @@ ND4J_SCALAR_MEMBERS(Float, float, float)
 ND4J_SCALAR_MEMBERS(Half, float16, float)
 ND4J_SCALAR_MEMBERS(Double, double, double)
 #undef ND4J_SCALAR_MEMBERS
+// the reference's indexed Double variant carries an extra element count (blas/NativeOps.h:419-430); like the others
+// it launches nothing
+void NativeOps::execScalarDouble(Nd4jPointer *, int, double *, Nd4jLong *, double *, Nd4jLong *, double, double *, Nd4jLong,
+                                 Nd4jLong *, Nd4jLong *) {}
 
 #define ND4J_ELEMENTWISE_MEMBERS(SUFFIX, T)                                                                      \
     void NativeOps::execTransform##SUFFIX(Nd4jPointer *extraPointers, int opNum, T *dx, Nd4jLong xStride,        \

@@ -155,6 +155,21 @@ void shuffleImpl(Nd4jPointer *extra, Nd4jPointer *dx, Nd4jPointer *xInfo, Nd4jPo
         shuffleImpl<T>(extras, dx, xShapeInfo, dz, N, shuffleMap, tadShapeInfo, tadOffsets);                             \
     }
 
+#define ND4J_AVERAGE_MEMBERS(SUFFIX, T)                                                                                  \
+    void NativeOps::average##SUFFIX(Nd4jPointer *extras, Nd4jPointer *dx, T *dz, int n, Nd4jLong length, bool propagate) { \
+        hipStream_t s = streamOf(extras);                                                                                \
+        launchAverage<T>(s, reinterpret_cast<T *const *>(dx), dz, n, length, true, propagate);                           \
+        checkLaunch("average", s);                                                                                       \
+    }                                                                                                                    \
+    void NativeOps::accumulate##SUFFIX(Nd4jPointer *extras, Nd4jPointer *dx, T *dz, int n, Nd4jLong length) {            \
+        hipStream_t s = streamOf(extras);                                                                                \
+        launchAverage<T>(s, reinterpret_cast<T *const *>(dx), dz, n, length, false, false);                              \
+        checkLaunch("accumulate", s);                                                                                    \
+    }
+ND4J_AVERAGE_MEMBERS(Float, float)
+ND4J_AVERAGE_MEMBERS(Half, float16)
+ND4J_AVERAGE_MEMBERS(Double, double)
+
 ND4J_SPECIAL_MEMBERS(Float, float)
 ND4J_SPECIAL_MEMBERS(Half, float16)
 ND4J_SPECIAL_MEMBERS(Double, double)

@@ -56,6 +56,8 @@ _EXEC_SIGNATURES = {
     "nd4j_pullRows{S}": ([_P, _P, _P, _P, _P, c_ll, _P, _P, _P, _P, _P], False),
     "nd4j_tear{S}": ([_P, _P, _P, _P, _P, _P, _P], False),
     "nd4j_shuffle{S}": ([_P, _P, _P, _P, _P, c_int, _P, _P, _P], False),
+    "nd4j_average{S}": ([_P, _P, _P, c_int, c_ll, c_int], False),
+    "nd4j_accumulate{S}": ([_P, _P, _P, c_int, c_ll], False),
 }
 
 _PLAIN_SIGNATURES = {

@@ -1579,6 +1579,25 @@ void shuffle(T **xs, Long **xInfos, int N, const int *map, Long **tadInfos, Long
     }
 }
 
+// accumulate / average of n buffers as the reference's device kernels do it (include/loops/special_kernels.h:710-742,
+// 757-809): a running sum in the data type starting from zero, in table order; average divides the sum by n, writes
+// it to z when z is there, and with `propagate` back to every input.  (The CPU loops of include/ops/impl/specials.cpp:
+// 344-440 differ by rounding only: they add x[k] / n term by term, and accumulate adds into what z already holds.)
+// (compiled without the reciprocal / reassociation licences the rest of this file inherits from the reference's CPU
+// flags: the device kernel divides and adds in IEEE arithmetic)
+template <typename T>
+__attribute__((optimize("no-reciprocal-math", "no-associative-math", "no-unsafe-math-optimizations"))) void accumulateBuffers(
+    T **x, T *z, int n, Long length, bool average, bool propagate) {
+    for (Long i = 0; i < length; i++) {
+        T acc = (T)0.0f;
+        for (int k = 0; k < n; k++) acc += x[k][i];
+        if (average) acc = acc / (T)n;
+        if (z != nullptr) z[i] = acc;
+        if (propagate)
+            for (int k = 0; k < n; k++) x[k][i] = acc;
+    }
+}
+
 // conversions: include/loops/type_conversions.h:592-611 - z[i] = (D)((float)x[i])
 template <typename S, typename D> void convert(const void *x, Long n, void *z) {
     const S *in = (const S *)x;
@@ -1702,6 +1721,12 @@ ND4J_CPU_FAMILY(f64, double)
     }                                                                                                              \
     void nd4j_cpu_shuffle_##SUF(void **x, Long **xSI, int N, int *map, Long **tadSI, Long **tadOff) {              \
         shuffle<T>((T **)x, xSI, N, map, tadSI, tadOff);                                                           \
+    }                                                                                                              \
+    void nd4j_cpu_average_##SUF(void **x, void *z, int n, long long length, int propagate) {                       \
+        accumulateBuffers<T>((T **)x, (T *)z, n, length, true, propagate != 0);                                    \
+    }                                                                                                              \
+    void nd4j_cpu_accumulate_##SUF(void **x, void *z, int n, long long length) {                                   \
+        accumulateBuffers<T>((T **)x, (T *)z, n, length, false, false);                                            \
     }
 ND4J_CPU_SPECIALS(f32, float)
 ND4J_CPU_SPECIALS(f16, half)

@@ -216,6 +216,15 @@ void reduce3AllPairs(int opNum, T *x, Nd4jLong *xSI, T *extra, T *y, Nd4jLong *y
     }                                                                                                              \
     void nd4j_cpu_shuffle_##SUF(void **x, Nd4jLong **xSI, int N, int *map, Nd4jLong **tadSI, Nd4jLong **tadOff) {  \
         shuffleGeneric<T>((T **)x, xSI, (T **)x, xSI, N, map, tadSI, tadOff);                                      \
+    }                                                                                                              \
+    /* the CPU loops of specials.cpp: average adds x[k] / n term by term; accumulate adds into z, which is zeroed  \
+       here first so that the result is the plain sum the device kernel of the same name produces */               \
+    void nd4j_cpu_average_##SUF(void **x, void *z, int n, long long length, int propagate) {                       \
+        nd4j::SpecialMethods<T>::averageGeneric((T **)x, (T *)z, n, length, propagate != 0);                       \
+    }                                                                                                              \
+    void nd4j_cpu_accumulate_##SUF(void **x, void *z, int n, long long length) {                                   \
+        std::memset(z, 0, (size_t)length * sizeof(T));                                                             \
+        nd4j::SpecialMethods<T>::accumulateGeneric((T **)x, (T *)z, n, length);                                    \
     }
 
 extern "C" {

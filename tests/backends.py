@@ -145,6 +145,18 @@ class CpuBackend(object):
         self.lib.shuffle(out, infos, shuffle_map, tads)
         return out
 
+    def average(self, arrays, propagate=False, with_z=True):
+        """returns (z or None, the inputs afterwards)"""
+        xs = [a.copy() for a in arrays]
+        z = np.zeros(xs[0].size, xs[0].dtype) if with_z else None
+        self.lib.average(xs, z, propagate)
+        return z, xs
+
+    def accumulate(self, arrays):
+        z = np.zeros(arrays[0].size, arrays[0].dtype)
+        self.lib.accumulate([a.copy() for a in arrays], z)
+        return z
+
     def convert(self, src_type, x, dst_type):
         z = np.zeros(x.size, TYPE_OF_CODE[dst_type])
         assert self.lib.convert(src_type, x, dst_type, z) == 1
@@ -316,6 +328,29 @@ class GpuBackend(object):
         out = [o.get() for o in ops]
         self._finish(x_tab, i_tab, ti_tab, to_tab, M, *(ops + tis + tos))
         return out
+
+    def average(self, arrays, propagate=False, with_z=True):
+        xs = [self.dev.upload(np.ascontiguousarray(a)) for a in arrays]
+        tab = self._ptr_table(xs)
+        n, dt = arrays[0].size, arrays[0].dtype
+        Z = self.dev.upload(np.zeros(n, dt)) if with_z else None
+        getattr(self.ops, "average" + self._suffix(arrays[0]))(self.dev.extra(), tab.ptr, Z.ptr if with_z else None, len(arrays), n,
+                                                               int(propagate))
+        self.dev.sync()
+        z = Z.download(dt, n) if with_z else None
+        out = [x.download(dt, n) for x in xs]
+        self._finish(tab, Z, *xs)
+        return z, out
+
+    def accumulate(self, arrays):
+        xs = [self.dev.upload(np.ascontiguousarray(a)) for a in arrays]
+        tab = self._ptr_table(xs)
+        n, dt = arrays[0].size, arrays[0].dtype
+        Z = self.dev.upload(np.full(n, 7, dt))  # stale contents must not leak into the sum
+        getattr(self.ops, "accumulate" + self._suffix(arrays[0]))(self.dev.extra(), tab.ptr, Z.ptr, len(arrays), n)
+        z = Z.download(dt, n)
+        self._finish(tab, Z, *xs)
+        return z
 
     def convert(self, src_type, x, dst_type):
         X, xp = self._up(x)

@@ -418,7 +418,7 @@ def _cast(a, dt):
     return a.astype(dt)
 
 
-def check_data_movement(be, dtypes=(np.float32, np.float64, np.float16), big=False):
+def check_data_movement(be, dtypes=(np.float32, np.float64, np.float16), big=False, exact_sums=True):
     """Every result is compared bit for bit with what numpy says the operation means."""
     from libnd4j_amd.harness import shape_info, span_of
     rs = np.random.RandomState(77)
@@ -514,6 +514,41 @@ def check_data_movement(be, dtypes=(np.float32, np.float64, np.float16), big=Fal
             got = be.shuffle(arrays, infos, smap, tads)
             for g, info, want in zip(got, infos, wants):
                 assert np.array_equal(_logical(g, info), want), ("shuffle", group)
+
+    # accumulate / average of n buffers: a running sum from zero in table order (one IEEE addition per term, which numpy
+    # reproduces exactly for float and double), divided by n for the average; `exact_sums` is off for a checker that
+    # orders or scales the terms differently (the reference's CPU loops) and for half, which the path sums in float
+    for dt in dtypes:
+        for n_arrays, length in ((3, 37), (8, 1024), (5, 4099)) + (((16, 300001),) if big else ()):
+            arrays = [(rs.randn(length) * 3).astype(dt) for _ in range(n_arrays)]
+            acc = np.zeros(length, np.float32 if dt == np.float16 else dt)
+            for a in arrays:
+                acc = acc + a.astype(acc.dtype)
+            exact = exact_sums and dt != np.float16
+            tol = 1e-2 if dt == np.float16 else (1e-5 if dt == np.float32 else 1e-12)
+            # a running sum in half (the reference's kernels) loses up to 2^-11 of the partial sum per term
+            scale = np.sum([np.abs(a.astype(np.float64)) for a in arrays], axis=0) + 1
+
+            def same(got, want, what, div=1):
+                if exact:
+                    assert np.array_equal(got, want.astype(dt)), what
+                else:
+                    g, w = got.astype(np.float64), want.astype(np.float64)
+                    assert np.all(np.abs(g - w) <= tol * scale / div), what
+
+            same(be.accumulate(arrays), acc, ("accumulate", np.dtype(dt).name, n_arrays, length))
+            mean = acc / acc.dtype.type(n_arrays)
+            z, after = be.average(arrays, propagate=False)
+            same(z, mean, ("average", np.dtype(dt).name, n_arrays, length), n_arrays)
+            if exact_sums:  # the reference's CPU loop copies the average into every input whatever `propagate` says
+                assert all(np.array_equal(a, b) for a, b in zip(after, arrays)), "average without propagate changed an input"
+            z, after = be.average(arrays, propagate=True)
+            same(z, mean, "average + propagate", n_arrays)
+            assert all(np.array_equal(a, z) for a in after), "propagate"
+            z, after = be.average(arrays, propagate=True, with_z=False)
+            assert z is None
+            for a in after:
+                same(a, mean, "average into the inputs only", n_arrays)
 
     # conversions: z = (dst)(float)x
     codes = {np.dtype(np.float16): 3, np.dtype(np.float32): 6, np.dtype(np.float64): 7}

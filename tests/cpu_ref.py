@@ -84,6 +84,8 @@ class CpuLib(object):
             "pullrows": [V, V, V, V, LL, V, V, V, V, V],
             "tear": [V, V, V, V, V, V],
             "shuffle": [V, V, I, V, V, V],
+            "average": [V, V, I, LL, I],
+            "accumulate": [V, V, I, LL],
         }
         L.nd4j_cpu_convert.restype = I
         L.nd4j_cpu_convert.argtypes = [I, V, LL, I, V]
@@ -129,6 +131,12 @@ class CpuLib(object):
         m = _ints(shuffle_map)
         self._fn("shuffle", arrays[0])(self._table(arrays), self._table(infos), len(arrays), _p(m), self._table(tis),
                                        self._table(tos))
+
+    def average(self, arrays, z, propagate):
+        self._fn("average", arrays[0])(self._table(arrays), _p(z), len(arrays), arrays[0].size, int(propagate))
+
+    def accumulate(self, arrays, z):
+        self._fn("accumulate", arrays[0])(self._table(arrays), _p(z), len(arrays), arrays[0].size)
 
     def convert(self, src_type, x, dst_type, z):
         return self.lib.nd4j_cpu_convert(src_type, _p(x), x.size, dst_type, _p(z))

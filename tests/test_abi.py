@@ -59,3 +59,21 @@ def test_missing_library_fails_loudly(tmp_path):
     import pytest
     with pytest.raises(ImportError):
         native.load_library(str(tmp_path / "nope.so"))
+
+
+def test_every_member_of_the_reference_class_is_exported():
+    """The reference's CPU back end, compiled where it lies for the checker (oracle/_ref/NativeOps.o), defines every
+    member of class NativeOps; each of those mangled names must be a defined export of this library, so that a
+    binding generated from the reference's header links against it."""
+    import pytest
+    ref_obj = os.path.join(ROOT, "oracle", "_ref", "NativeOps.o")
+    if not os.path.exists(ref_obj):
+        pytest.skip("oracle/_ref/NativeOps.o not built (needs the reference tree)")
+
+    def members(path, dynamic):
+        out = subprocess.check_output(["nm", "--defined-only"] + (["-D"] if dynamic else []) + [path]).decode()
+        return {line.split()[-1] for line in out.splitlines() if " T _ZN9NativeOps" in line}
+
+    want, have = members(ref_obj, False), members(native.LIBRARY_PATH, True)
+    assert len(want) > 200
+    assert not (want - have), sorted(want - have)[:5]

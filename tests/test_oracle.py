@@ -296,4 +296,4 @@ def test_data_movement_matches_numpy_and_compiled_reference(oracle_lib, referenc
     """flatten / concat / pullRows / tear / shuffle / convertTypes: the restatement and the compiled reference
     (blas/cpu/NativeOps.cpp templates, specials.cpp, convertTypes) against what numpy says each call means."""
     checks.check_data_movement(backends.CpuBackend(oracle_lib), big=True)
-    checks.check_data_movement(backends.CpuBackend(reference_lib), big=True)
+    checks.check_data_movement(backends.CpuBackend(reference_lib), big=True, exact_sums=False)
