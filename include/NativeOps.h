@@ -1,11 +1,11 @@
 // class NativeOps - the drop-in surface of the legacy op-execution path.
 //
 // Same class name, member names, argument order and POD argument types as the reference's
-// blas/NativeOps.h, restricted to the members on the hot path (transform, pairwise, broadcast, reduce,
-// index-reduce, summary-stats, random) and the lifecycle members a host needs around them.  A JavaCPP
-// binding generated against the reference header resolves these members to the same Itanium-mangled
-// symbols in libnd4j_amd.so.  Members of the reference class that are outside this path are not
-// declared here.
+// blas/NativeOps.h.  The members on the hot path (transform, pairwise, broadcast, scalar, reduce, reduce3,
+// index-reduce, summary-stats, random, the data-movement specials) and the lifecycle members a host needs
+// around them do their work; every other member of the reference's class is declared at the end and
+// defined as a stub.  A JavaCPP binding generated against the reference header resolves all of them to the
+// same Itanium-mangled symbols in libnd4j_amd.so.
 //
 // Calling convention = the reference's CUDA backend (blas/cuda/NativeOps.cu):
 //   * data pointers, shapeInfo arguments, `dimension` and `extraParams` are DEVICE pointers;
