@@ -9,7 +9,12 @@ template <typename T> struct BroadcastBody {
         static bool run(hipStream_t s, const T *x, const T *y, T *z, const BroadcastPlan &pl) {
             typedef Broadcast2F<KIND> F;
             if (pl.numTads <= 0 || pl.tadLength <= 0) return true;
-            if (pl.kind == BroadcastPlan::ROW) {
+            if (pl.kind == BroadcastPlan::ROW && pl.consecutive && pl.tadLength % Pack<T>::N == 0 &&
+                pl.tadLength / Pack<T>::N < 0xffffffffLL && (((uintptr_t)x | (uintptr_t)y | (uintptr_t)z) & 15) == 0) {
+                const Long nvec = pl.numTads * (pl.tadLength / Pack<T>::N);
+                hipLaunchKernelGGL((bcFlatKernel<T, F>), dim3(gridFor(nvec, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0,
+                                   s, x, y, z, nvec, (unsigned)(pl.tadLength / Pack<T>::N), Params<T>{nullptr});
+            } else if (pl.kind == BroadcastPlan::ROW) {
                 constexpr int VEC = Pack<T>::N;
                 Long vecsPerTad = (pl.tadLength + VEC - 1) / VEC;
                 int colShift = 0;

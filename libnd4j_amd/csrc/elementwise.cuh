@@ -281,6 +281,30 @@ __global__ void __launch_bounds__(kBlock) bcRowKernel(const T *x, const T *y, T 
     }
 }
 
+// Broadcast over contiguous TADs that follow one another without gaps in x and in z (the rows of a dense c-order
+// matrix): the array is walked as one long vector, one 16-byte vector per thread as in ewVecKernel, and the only
+// trace of the TADs is the position inside the row, which selects the vector of y (read through the caches).  No
+// offset tables are read.  Needs tadLength % VEC == 0 and 16-byte aligned x, y, z.
+template <typename T, typename F>
+__global__ void __launch_bounds__(kBlock) bcFlatKernel(const T *x, const T *y, T *z, Long nvec, unsigned vecsPerTad,
+                                                       Params<T> p) {
+    typedef typename Compute<T>::type C;
+    if (F::tables) lm::loadTables();
+    constexpr int VEC = Pack<T>::N;
+    const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x);
+    const Pack<T> *yv = reinterpret_cast<const Pack<T> *>(y);
+    Pack<T> *zv = reinterpret_cast<Pack<T> *>(z);
+    for (Long j = (Long)blockIdx.x * kBlock + threadIdx.x; j < nvec; j += (Long)gridDim.x * kBlock) {
+        const Pack<T> a = loadPack(xv + j);
+        const unsigned col = (j >> 32) == 0 ? (unsigned)j % vecsPerTad : (unsigned)((unsigned long long)j % vecsPerTad);
+        const Pack<T> b = yv[col];
+        Pack<T> r;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) r.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), toCompute(b.v[e]), p));
+        storePack(zv + j, r);
+    }
+}
+
 // Broadcast over strided TADs: thread <-> TAD, loop over the TAD's elements.  When neighbouring TADs
 // are neighbours in memory (a column of a c-order matrix) each wave reads and writes full lines.
 template <typename T, typename F, bool BYTAD>

@@ -31,6 +31,7 @@ struct BroadcastPlan {
     DimMap xm, ym, zm;           // GENERAL: element index inside the TAD -> offset
     const Long *xOffsets;        // device, numTads entries
     const Long *zOffsets;        // device, numTads entries
+    bool consecutive = false;    // ROW only: TAD r starts at r * tadLength in x and in z (rows of a dense c-order array)
 };
 template <typename T>
 bool launchBroadcast(hipStream_t stream, int opNum, const T *x, const T *y, T *z, const BroadcastPlan &plan);

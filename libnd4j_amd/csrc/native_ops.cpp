@@ -22,6 +22,18 @@ inline bool sameShape(const Long *a, const Long *b) {
     return true;
 }
 
+// true when the strides are those of a gap-free array in the given order (unit dimensions may carry any stride)
+inline bool isDense(const Long *info, char order) {
+    const int rank = siRank(info);
+    Long expect = 1;
+    for (int k = 0; k < rank; k++) {
+        const int d = order == 'c' ? rank - 1 - k : k;
+        if (siShape(info)[d] != 1 && siStride(info)[d] != expect) return false;
+        expect *= siShape(info)[d];
+    }
+    return true;
+}
+
 // Index -> offset map of one operand walked by its own linear index, in C order or Fortran order.
 void linearMap(const Long *shape, const Long *stride, int rank, char order, DimMap &out) {
     if (order == 'c') {
@@ -171,6 +183,12 @@ void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Lon
     pl.zEws = siEws(zTadInfo);
     if (pl.tadEws > 0 && pl.yEws > 0 && pl.zEws > 0 && dimLen == 1) {
         pl.kind = (pl.tadEws == 1 && pl.yEws == 1 && pl.zEws == 1) ? BroadcastPlan::ROW : BroadcastPlan::COL;
+        // contiguous TADs of a dense array are its trailing (c order) or leading (f order) block, so they follow one
+        // another without gaps;
+        // when the result has the same dense layout the kernel needs no offset tables
+        if (pl.kind == BroadcastPlan::ROW && zTadInfo == tx.hostInfo && sameShape(hx, hz) && siNumel(hy) == tx.tadLength &&
+            ((isDense(hx, 'c') && isDense(hz, 'c')) || (isDense(hx, 'f') && isDense(hz, 'f'))))
+            pl.consecutive = true;
     } else {
         pl.kind = BroadcastPlan::GENERAL;
         char xo = siOrder(tx.hostInfo) == 'c' ? 'c' : 'f';
