@@ -13,6 +13,12 @@
 // inputs.  The RandomBuffer stream beyond the plain xoroshiro128+ fill has no golden vector in the
 // reference's tests; it is pinned by vectors produced with the compiled reference
 // (tests/golden/rng_stream.json, generator script beside it).
+// The families added around the op loops are pinned the same way: scalar and reduce3 by vectors of and comparison
+// with the compiled reference (reduce3 also by the reference's own known answers); the SoftMax family and IsMax by
+// the compiled reference where its code is well defined and by float64 ground truth; flatten, concat, pullRows,
+// tear, shuffle and the type conversions bit for bit by numpy and by the compiled reference; accumulate / average
+// by the exact IEEE sequence in numpy (float, double) and by the reference's CPU loops within rounding.  No function
+// of this file is "parity unpinned".
 //
 // shapeInfo / TAD decoding is shared with the product's host code (libnd4j_amd/csrc/shape_host.h, plain
 // host C++ with no device dependency); that logic is pinned on its own against the reference's TadTests /
