@@ -172,13 +172,23 @@ __global__ void __launch_bounds__(kBlock) shuffleKernel(T *const *xs, const Long
 }
 
 // ---- concat ----------------------------------------------------------------------------------------------------
-// cum[r] = sum of shape[dim] of the inputs before r, cum[n] = the total; one block.
-__global__ void __launch_bounds__(kBlock) concatPrefixKernel(const Long *const *infos, int n, int dim, Long *cum) {
+// What the copy kernel needs to know about one input, prepared by a one-block kernel so that the copy blocks start
+// with a single small load instead of a chain of dependent ones through the tables of pointers and shapeInfos.
+struct ConcatDesc {
+    const void *data;
+    Long length;  // elements of the input
+    Long start;   // sum of shape[dim] of the inputs before it
+    Long run;     // shape[dim] * inner: elements that stay together in the result
+    Long fast;    // 1: C-contiguous input of the result's rank going into a C-contiguous result
+};
+
+__global__ void __launch_bounds__(kBlock) concatPrepareKernel(const void *const *data, const Long *const *infos, int n,
+                                                              ConcatView v, ConcatDesc *desc) {
     __shared__ Long part[kBlock];
     const int chunk = (n + kBlock - 1) / kBlock;
     const int lo = threadIdx.x * chunk, hi = lo + chunk < n ? lo + chunk : n;
     Long sum = 0;
-    for (int f = lo; f < hi; f++) sum += dShape(infos[f])[dim];
+    for (int f = lo; f < hi; f++) sum += dShape(infos[f])[v.dim];
     part[threadIdx.x] = sum;
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -188,51 +198,61 @@ __global__ void __launch_bounds__(kBlock) concatPrefixKernel(const Long *const *
             part[t] = run;
             run += p;
         }
-        cum[n] = run;
     }
     __syncthreads();
     Long run = part[threadIdx.x];
     for (int f = lo; f < hi; f++) {
-        cum[f] = run;
-        run += dShape(infos[f])[dim];
+        const Long *si = infos[f];
+        ConcatDesc d;
+        d.data = data[f];
+        d.length = dLength(si);
+        d.start = run;
+        d.run = dShape(si)[v.dim] * v.inner;
+        d.fast = (dRank(si) == v.rank && v.zContig && dOrder(si) == 'c' && dEws(si) == 1) ? 1 : 0;
+        desc[f] = d;
+        run += dShape(si)[v.dim];
     }
 }
 
-// Input r (blockIdx.y) is copied into the slab [cum[r], cum[r+1]) of dimension `dim` of z.  Elements are walked in
-// the input's logical C order; contiguous C-order inputs into a contiguous C-order result move whole runs.
+// Input r (blockIdx.y) is copied into the slab [start, start + shape[dim]) of dimension `dim` of z.  C-contiguous
+// inputs into a C-contiguous result move as 16-byte vectors, one per thread: vector j of the input belongs to run
+// j / runV and lands zRunV vectors further on for every run.  Other layouts are walked in the input's logical C order.
 template <typename T>
-__global__ void __launch_bounds__(kBlock) concatKernel(const T *const *data, const Long *const *infos, T *z, ConcatView v,
-                                                       const Long *cum, int n) {
+__global__ void __launch_bounds__(kBlock) concatKernel(const Long *const *infos, T *z, ConcatView v, const ConcatDesc *desc, int n) {
+    constexpr int VEC = Pack<T>::N;
     for (int r = blockIdx.y; r < n; r += gridDim.y) {
-        const Long *si = infos[r];
-        const T *x = data[r];
-        const int rank = dRank(si);
-        const Long len = dLength(si);
-        const Long start = cum[r];
-        if (rank == v.rank && v.zContig && dOrder(si) == 'c' && dEws(si) == 1) {
-            const Long run = dShape(si)[v.dim] * v.inner;  // contiguous on both sides
-            const Long zRun = v.dimTotal * v.inner;        // distance between consecutive runs in z
-            const Long outer = run > 0 ? len / run : 0;
-            T *zb = z + start * v.inner;
-            if (outer * 4 <= (Long)gridDim.x) {
-                // few long runs: all threads of this input share each run
-                for (Long o = 0; o < outer; o++)
-                    copyRun<T, false>(x + o * run, 1, nullptr, zb + o * zRun, 1, nullptr, run, (int)(blockIdx.x * kBlock + threadIdx.x),
-                                      (int)(gridDim.x * kBlock));
+        const ConcatDesc d = desc[r];
+        const T *x = reinterpret_cast<const T *>(d.data);
+        if (d.fast) {
+            const Long zRun = v.dimTotal * v.inner;  // distance between consecutive runs in z
+            T *zb = z + d.start * v.inner;
+            if (d.run % VEC == 0 && zRun % VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                (reinterpret_cast<uintptr_t>(zb) & 15) == 0) {
+                const Long runV = d.run / VEC, zRunV = zRun / VEC, nv = d.length / VEC;
+                const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x);
+                Pack<T> *zv = reinterpret_cast<Pack<T> *>(zb);
+                const bool small = (nv >> 32) == 0;
+                for (Long j = (Long)blockIdx.x * kBlock + threadIdx.x; j < nv; j += (Long)gridDim.x * kBlock) {
+                    const Long o = runV >= nv ? 0 : (small ? (Long)((unsigned)j / (unsigned)runV) : j / runV);
+                    storePack(zv + o * zRunV + (j - o * runV), loadPack(xv + j));
+                }
             } else {
-                const int lanes = lanesPerTad<T>(run), groups = kBlock / lanes;
-                const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
-                for (Long o = (Long)blockIdx.x * groups + g; o < outer; o += (Long)gridDim.x * groups)
-                    copyRun<T, false>(x + o * run, 1, nullptr, zb + o * zRun, 1, nullptr, run, lane, lanes);
+                for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < d.length; i += (Long)gridDim.x * kBlock) {
+                    const Long o = i / d.run;
+                    zb[o * zRun + (i - o * d.run)] = x[i];
+                }
             }
-        } else if (rank == v.rank) {
+        } else {
+            const Long *si = infos[r];
+            const int rank = dRank(si);
+            if (rank != v.rank) continue;
             const Long *shape = dShape(si), *stride = dStride(si);
-            for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < len; i += (Long)gridDim.x * kBlock) {
+            for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < d.length; i += (Long)gridDim.x * kBlock) {
                 Long rem = i, xo = 0, zo = 0;
-                for (int d = rank - 1; d >= 0; d--) {
-                    const Long q = rem / shape[d], c = rem - q * shape[d];
-                    xo += c * stride[d];
-                    zo += (c + (d == v.dim ? start : 0)) * v.zStride[d];
+                for (int dd = rank - 1; dd >= 0; dd--) {
+                    const Long q = rem / shape[dd], c = rem - q * shape[dd];
+                    xo += c * stride[dd];
+                    zo += (c + (dd == v.dim ? d.start : 0)) * v.zStride[dd];
                     rem = q;
                 }
                 z[zo] = x[xo];
@@ -248,12 +268,13 @@ template <typename T>
 __global__ void __launch_bounds__(kBlock) copyToEwsKernel(const T *x, Long xe, T *z, const Long *zInfo, Long n) {
     Long ze = dEws(zInfo);
     if (ze < 1) ze = 1;
+    // the grid holds one thread per 16-byte vector: a plain streaming copy is fastest as very many short blocks
     copyRun<T, false>(x, xe, nullptr, z, ze, nullptr, n, (int)(blockIdx.x * kBlock + threadIdx.x), (int)(gridDim.x * kBlock));
 }
 template <typename T> void launchCopyToEws(hipStream_t s, const T *x, Long xe, T *z, const Long *zInfo, Long n) {
     if (n <= 0) return;
-    hipLaunchKernelGGL((copyToEwsKernel<T>), dim3(gridFor(n, (Long)kBlock * Pack<T>::N * 4, kGridCap * 2)), dim3(kBlock), 0, s, x, xe,
-                       z, zInfo, n);
+    hipLaunchKernelGGL((copyToEwsKernel<T>), dim3(gridFor(n, (Long)kBlock * Pack<T>::N, 1 << 22)), dim3(kBlock), 0, s, x, xe, z,
+                       zInfo, n);
 }
 
 // ---- transposing copy: z[r * zRowStride + c] = x[r + c * xColStride] --------------------------------------------
@@ -341,15 +362,18 @@ void launchShuffle(hipStream_t s, T *const *xs, const Long *const *xInfos, T *co
 }
 template <typename T>
 void launchConcat(hipStream_t s, const T *const *data, const Long *const *infos, T *z, const ConcatView &v, int n, Long maxLength,
-                  Long *cum) {
+                  void *scratch) {
     if (n <= 0) return;
-    hipLaunchKernelGGL(concatPrefixKernel, dim3(1), dim3(kBlock), 0, s, infos, n, v.dim, cum);
+    ConcatDesc *desc = reinterpret_cast<ConcatDesc *>(scratch);
+    hipLaunchKernelGGL(concatPrepareKernel, dim3(1), dim3(kBlock), 0, s, reinterpret_cast<const void *const *>(data), infos, n, v, desc);
     const int gy = n < 65535 ? n : 65535;
-    int budget = (kGridCap * 4) / gy;
+    // one 16-byte vector per thread while that keeps the grid below 2^22 blocks
+    int budget = (1 << 22) / gy;
     if (budget < 1) budget = 1;
-    const int gx = gridFor(maxLength > 0 ? maxLength : 1, (Long)kBlock * Pack<T>::N * 4, budget);  // four vectors a thread
-    hipLaunchKernelGGL((concatKernel<T>), dim3(gx, gy), dim3(kBlock), 0, s, data, infos, z, v, cum, n);
+    const int gx = gridFor(maxLength > 0 ? maxLength : 1, (Long)kBlock * Pack<T>::N, budget);
+    hipLaunchKernelGGL((concatKernel<T>), dim3(gx, gy), dim3(kBlock), 0, s, infos, z, v, desc, n);
 }
+size_t concatScratchBytes(int numArrays) { return (size_t)(numArrays > 0 ? numArrays : 1) * sizeof(ConcatDesc); }
 
 // ---- accumulate / average: z[i] = sum_k x[k][i] (/ n), optionally written back to every x[k] ------------------------
 // (special_kernels.h:700-822).  x is a device table of n device pointers.  The sum runs in the compute type, in table
@@ -443,7 +467,7 @@ bool launchConvert(hipStream_t s, int srcType, const void *x, Long n, int dstTyp
                                 Long);                                                                                       \
     template void launchShuffle<T>(hipStream_t, T *const *, const Long *const *, T *const *, int, const int *,               \
                                    const Long *const *, const Long *const *, Long);                                          \
-    template void launchConcat<T>(hipStream_t, const T *const *, const Long *const *, T *, const ConcatView &, int, Long, Long *); \
+    template void launchConcat<T>(hipStream_t, const T *const *, const Long *const *, T *, const ConcatView &, int, Long, void *); \
     template void launchTransposeCopy<T>(hipStream_t, const T *, T *, Long, Long, Long, Long);                            \
     template void launchCopyToEws<T>(hipStream_t, const T *, Long, T *, const Long *, Long);                              \
     template void launchAverage<T>(hipStream_t, T *const *, T *, int, Long, bool, bool);

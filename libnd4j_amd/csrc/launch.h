@@ -143,10 +143,11 @@ void launchTear(hipStream_t stream, const T *x, const Long *xInfo, T *const *tar
 template <typename T>
 void launchShuffle(hipStream_t stream, T *const *xs, const Long *const *xInfos, T *const *zs, int N, const int *map,
                    const Long *const *tadInfos, const Long *const *tadOffsets, Long numTadsHint);
-// `cum` is device scratch of numArrays + 1 Longs; maxLength the element count of the largest input
+// `scratch` is device memory of concatScratchBytes(numArrays) bytes; maxLength the element count of the largest input
+size_t concatScratchBytes(int numArrays);
 template <typename T>
 void launchConcat(hipStream_t stream, const T *const *data, const Long *const *infos, T *z, const ConcatView &view,
-                  int numArrays, Long maxLength, Long *cum);
+                  int numArrays, Long maxLength, void *scratch);
 // z[i * ews(zInfo)] = x[i * xe]; zInfo is a device shapeInfo, read by the kernel
 template <typename T> void launchCopyToEws(hipStream_t stream, const T *x, Long xe, T *z, const Long *zInfo, Long n);
 // z[r * zRowStride + c] = x[r + c * xColStride] for r < rows, c < cols, through LDS tiles

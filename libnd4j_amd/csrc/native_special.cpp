@@ -94,9 +94,9 @@ void concatImpl(Nd4jPointer *extra, int dimension, int numArrays, Nd4jPointer *d
         for (int i = 0; i < numArrays; i++)
             if (hostShapes[i] != nullptr && siNumel(hostShapes[i]) > maxLength) maxLength = siNumel(hostShapes[i]);
     }
-    Workspace ws = workspaceFor(s, (size_t)(numArrays + 1) * sizeof(Long));
+    Workspace ws = workspaceFor(s, concatScratchBytes(numArrays));
     launchConcat<T>(s, reinterpret_cast<const T *const *>(data[0]), reinterpret_cast<const Long *const *>(inputShapeInfo[0]), result,
-                    v, numArrays, maxLength, reinterpret_cast<Long *>(ws.ptr));
+                    v, numArrays, maxLength, ws.ptr);
     checkLaunch("concat", s);
 }
 
