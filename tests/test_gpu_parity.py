@@ -366,8 +366,12 @@ def test_special_transforms(gpu, cpu):
         assert np.all(np.abs(a64 - b64) <= 1e-5 * np.abs(b64) + 1e-7), what
 
     # softmax family: short / wave / block rows, vectors, f-order (rows adjacent in memory), f -> c
+    # (row lengths chosen to reach every register-resident variant: 16 / 64 / 256 lanes per row with 2..16 vectors each,
+    # and the f-order kernel with 2, 8 and 16 vectors per thread, next to the shapes that fall back to three passes)
     for shape, order in (([37, 129], "c"), ([300, 17], "c"), ([9, 5000], "c"), ([1, 500], "c"), ([700, 1], "c"), ([1, 70001], "c"),
-                         ([257, 96], "f"), ([64, 300], "f"), ([8, 8], "c")):
+                         ([7, 100], "c"), ([6, 200], "c"), ([4, 600], "c"), ([5, 3000], "c"), ([3, 16384], "c"), ([2, 16388], "c"),
+                         ([257, 96], "f"), ([64, 300], "f"), ([128, 200], "f"), ([96, 1500], "f"), ([64, 2048], "f"),
+                         ([64, 2052], "f"), ([8, 8], "c")):
         n = int(np.prod(shape))
         xi = harness.shape_info(shape, order)
         x = rs.uniform(-6, 6, n).astype(np.float32)
@@ -390,20 +394,24 @@ def test_special_transforms(gpu, cpu):
     truth = np.exp(rows - rows.max(axis=1, keepdims=True))
     truth /= truth.sum(axis=1, keepdims=True)
     assert np.all(np.abs(got - truth) <= 2e-5 * truth)
-    # half and double
-    xh = rs.uniform(-2, 2, 64 * 96).astype(np.float16)
-    hi = shape_info_np([64, 96])
-    g = gpu.transform(38, xh, hi, hi).astype(np.float64).reshape(64, 96)
-    rows = xh.astype(np.float64).reshape(64, 96)
-    truth = np.exp(rows - rows.max(axis=1, keepdims=True))
-    truth /= truth.sum(axis=1, keepdims=True)
-    assert np.all(np.abs(g - truth) <= 1e-2 * truth + 1e-4)
-    xd = rs.randn(30 * 40)
-    di = shape_info_np([30, 40])
-    rows = xd.reshape(30, 40)
-    truth = np.exp(rows - rows.max(axis=1, keepdims=True))
-    truth /= truth.sum(axis=1, keepdims=True)
-    assert np.allclose(gpu.transform(38, xd, di, di).reshape(30, 40), truth, rtol=1e-13)
+    # half and double, row-major and column-major, short and long rows
+    for shape, order in (([64, 96], "c"), ([5, 4000], "c"), ([3, 30000], "c"), ([128, 600], "f"), ([64, 1100], "f")):
+        n = shape[0] * shape[1]
+        od = "F" if order == "f" else "C"
+        info = harness.shape_info(shape, order)
+        xh = rs.uniform(-2, 2, n).astype(np.float16)
+        g = gpu.transform(38, xh, info, info).astype(np.float64).reshape(shape, order=od)
+        rows = xh.astype(np.float64).reshape(shape, order=od)
+        truth = np.exp(rows - rows.max(axis=1, keepdims=True))
+        truth /= truth.sum(axis=1, keepdims=True)
+        assert np.all(np.abs(g - truth) <= 1e-2 * truth + 1e-4), ("half", shape, order)
+        xd = rs.randn(n)
+        rows = xd.reshape(shape, order=od)
+        truth = np.exp(rows - rows.max(axis=1, keepdims=True))
+        truth /= truth.sum(axis=1, keepdims=True)
+        for op, f in ((38, lambda v: v), (39, lambda v: v * (1 - v)), (40, np.log)):
+            got = gpu.transform(op, xd, info, info).reshape(shape, order=od)
+            assert np.allclose(got, f(truth), rtol=1e-12, atol=1e-300), ("double", shape, order, op)
     # IsMax: whole array (also a large one, f-order and 3-D), and along a dimension
     for shape, order in (([1, 300], "c"), ([12, 40], "c"), ([5, 6, 7], "c"), ([12, 40], "f"), ([1, 200003], "c")):
         n = int(np.prod(shape))
