@@ -436,6 +436,34 @@ def test_special_transforms(gpu, cpu):
                 assert np.array_equal(got, cpu.transform(41, x, xi, xi, e)), (shape, dim)
 
 
+def test_broadcast_over_gap_free_tads(gpu):
+    """Rows of a dense c-order array and columns of a dense f-order one go through the kernel that walks the array as
+    one vector; every result is a single IEEE operation, so numpy gives the expected bits.  Shapes whose TAD length is
+    not a multiple of the vector width, and a result laid out differently, take the other broadcast kernels."""
+    rs = np.random.RandomState(5)
+    for dt in (np.float32, np.float16, np.float64):
+        for shape, order, dim in (([33, 64], "c", 1), ([64, 33], "f", 0), ([5, 7, 24], "c", 2), ([40, 3, 2], "f", 0), ([33, 62], "c", 1),
+                                  ([1000, 1024], "c", 1), ([2048, 300], "f", 0)):
+            od = "F" if order == "f" else "C"
+            n = int(np.prod(shape))
+            info = harness.shape_info(shape, order)
+            x = rs.randn(n).astype(dt)
+            y = rs.randn(shape[dim]).astype(dt)
+            logical = x.reshape(shape, order=od)
+            bshape = [1] * len(shape)
+            bshape[dim] = shape[dim]
+            for op, f in ((0, np.add), (2, np.multiply), (1, np.subtract)):
+                got = gpu.broadcast(op, x, info, y, shape_info_np([1, shape[dim]]), info, [dim]).reshape(shape, order=od)
+                want = f(logical, y.reshape(bshape)).astype(dt)
+                assert np.array_equal(got, want), (np.dtype(dt).name, shape, order, op)
+    # c-order input into an f-order result: not gap-free on the result side
+    xi, zi = harness.shape_info([16, 32], "c"), harness.shape_info([16, 32], "f")
+    x = rs.randn(512).astype(np.float32)
+    y = rs.randn(32).astype(np.float32)
+    got = gpu.broadcast(0, x, xi, y, shape_info_np([1, 32]), zi, [1]).reshape(16, 32, order="F")
+    assert np.array_equal(got, x.reshape(16, 32) + y[None, :])
+
+
 def test_data_movement(gpu):
     """flatten / concat / pullRows / tear / shuffle / convertTypes through the C ABI, bit for bit against numpy (the
     same check the CPU restatement and the compiled reference pass)."""
