@@ -391,8 +391,14 @@ void reduce3Dims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T 
     const char order = siOrder(tx.hostInfo) == 'f' ? 'f' : 'c';
     orderedLinearMap(siShape(tx.hostInfo), siStride(tx.hostInfo), siRank(tx.hostInfo), order, in.xm);
     if (siNumel(hy) == siNumel(hx)) {
+        // a y laid out like x shares its TAD tables; any other layout gets tables of its own (which needs the
+        // dimensions on the host, a small synchronous copy)
         ResolvedTad ty;
-        if (!resolveTad(nullptr, 0, 0, hy, dimension, dimLen, ty, s)) return;
+        bool sameLayout = siRank(hy) == siRank(hx) && siOrder(hy) == siOrder(hx);
+        for (int d = 0; sameLayout && d < siRank(hx); d++)
+            sameLayout = siShape(hy)[d] == siShape(hx)[d] && siStride(hy)[d] == siStride(hx)[d];
+        if (sameLayout) ty = tx;
+        else if (!resolveTad(nullptr, 0, 0, hy, dimension, dimLen, ty, s)) return;
         in.yOffsets = ty.devOffsets;
         orderedLinearMap(siShape(ty.hostInfo), siStride(ty.hostInfo), siRank(ty.hostInfo), order, in.ym);
     } else if (siNumel(hy) == tx.tadLength) {

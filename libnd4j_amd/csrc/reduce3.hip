@@ -94,20 +94,29 @@ __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, 
             const Long f0 = sliced ? u * sliceLength : 0;
             Long f1 = sliced ? f0 + sliceLength : pl.runLength;
             if (f1 > pl.runLength) f1 = pl.runLength;
-            const T *xr = x + (pl.xOffsets != nullptr ? pl.xOffsets[r / pl.xDiv] : 0);
-            const T *yr = y + (pl.yOffsets != nullptr ? pl.yOffsets[r % pl.yMod] : 0);
+            // (the usual pairing - run r of x with run r of y - needs neither the division nor the remainder)
+            const Long xi = pl.xDiv == 1 ? r : r / pl.xDiv, yi = r < pl.yMod ? r : r % pl.yMod;
+            const T *xr = x + (pl.xOffsets != nullptr ? pl.xOffsets[xi] : 0);
+            const T *yr = y + (pl.yOffsets != nullptr ? pl.yOffsets[yi] : 0);
             const bool vec = pl.contiguous && ((reinterpret_cast<uintptr_t>(xr + f0) | reinterpret_cast<uintptr_t>(yr + f0)) & 15) == 0;
             if (vec) {
                 const Long nvec = (f1 - f0) / VEC;
                 const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(xr + f0);
                 const Pack<T> *yv = reinterpret_cast<const Pack<T> *>(yr + f0);
                 Long v = lane;
-                for (; v + GROUP < nvec; v += 2 * GROUP) {
-                    Pack<T> a0 = loadPack(xv + v), b0 = loadPack(yv + v), a1 = loadPack(xv + v + GROUP), b1 = loadPack(yv + v + GROUP);
+                // four vectors of each operand requested before the first is used
+                for (; v + 3 * GROUP < nvec; v += 4 * GROUP) {
+                    Pack<T> a[4], b[4];
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) Reduce3Op<C, OP>::accumulate(acc, toCompute(a0.v[e]), toCompute(b0.v[e]), eps);
+                    for (int k = 0; k < 4; k++) {
+                        a[k] = loadPack(xv + v + k * GROUP);
+                        b[k] = loadPack(yv + v + k * GROUP);
+                    }
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) Reduce3Op<C, OP>::accumulate(acc, toCompute(a1.v[e]), toCompute(b1.v[e]), eps);
+                    for (int k = 0; k < 4; k++) {
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) Reduce3Op<C, OP>::accumulate(acc, toCompute(a[k].v[e]), toCompute(b[k].v[e]), eps);
+                    }
                 }
                 for (; v < nvec; v += GROUP) {
                     Pack<T> a0 = loadPack(xv + v), b0 = loadPack(yv + v);
