@@ -231,8 +231,11 @@ def main():
                 continue
             wl = build(dev)
             for c in wl.cases:
+                fetched = dev.ops.amd_hostFetchCount()
                 ms = time_case(dev, c, max(3, min(K, 20)), 2)
+                fetched = dev.ops.amd_hostFetchCount() - fetched
                 row = {"config": wl.name, "case": c.name, "family": c.family, "contiguous": c.contiguous,
+                       "host_fetches": int(fetched),  # shapeInfo / dimension read-backs (each one a stream synchronisation)
                        "ms": round(ms, 4), "GB/s": round(c.bytes / ms / 1e6, 1),
                        "frac": round(c.bytes / ms / 1e6 / HBM_PEAK_GBS, 4), "elements_per_sec": round(c.elements / ms * 1e3, 1)}
                 if cpu_lib is not None and c.cpu is not None and not (c.name.endswith("float16")):
@@ -240,9 +243,10 @@ def main():
                     row["cpu_ms"] = round(med * 1e3, 3)
                     row["cpu_GB/s"] = round(c.bytes / med / 1e9, 2)
                 fam.append(row)
-                print("%-22s %-12s %9.4f ms %8.1f GB/s %5.1f%%%s" % (
+                print("%-22s %-12s %9.4f ms %8.1f GB/s %5.1f%%%s%s" % (
                     c.name, c.family, ms, row["GB/s"], 100 * row["frac"],
-                    "   cpu %9.2f ms" % row["cpu_ms"] if "cpu_ms" in row else ""), file=sys.stderr, flush=True)
+                    "   cpu %9.2f ms" % row["cpu_ms"] if "cpu_ms" in row else "",
+                    "   (%d read-backs from the device)" % fetched if fetched else ""), file=sys.stderr, flush=True)
             wl.free()
         out["families"] = fam
     print(json.dumps(out), flush=True)

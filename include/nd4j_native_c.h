@@ -210,6 +210,10 @@ Nd4jPointer nd4j_amd_timerCreate(void);
 int nd4j_amd_timerRecord(Nd4jPointer timer, Nd4jPointer stream);
 float nd4j_amd_timerElapsedMs(Nd4jPointer start, Nd4jPointer stop);
 int nd4j_amd_timerDestroy(Nd4jPointer timer);
+/* number of times, since the library was loaded, that a call had to read a shapeInfo or a dimension array back from
+ * the device because the host copy / TAD tables of the CUDA convention were not passed: each one synchronises the
+ * stream, so a caller that wants asynchronous array-result calls keeps this from growing */
+Nd4jLong nd4j_amd_hostFetchCount(void);
 /* plain device-to-device copy kernel of `bytes` bytes (16-byte vectors): the yardstick against which
  * hardware traffic counters are scaled */
 void nd4j_amd_copyKernel(Nd4jPointer *extraPointers, void *dst, const void *src, Nd4jLong bytes);

@@ -270,6 +270,7 @@ float nd4j_amd_timerElapsedMs(Nd4jPointer start, Nd4jPointer stop) {
     return ms;
 }
 int nd4j_amd_timerDestroy(Nd4jPointer timer) { return hipEventDestroy(reinterpret_cast<hipEvent_t>(timer)) == hipSuccess ? 1 : 0; }
+Nd4jLong nd4j_amd_hostFetchCount(void) { return (Nd4jLong)nd4j_amd::hostFetchCount(); }
 void nd4j_amd_copyKernel(Nd4jPointer *extraPointers, void *dst, const void *src, Nd4jLong bytes) {
     guardVoid([&] {
         hipStream_t s = nd4j_amd::streamOf(extraPointers);

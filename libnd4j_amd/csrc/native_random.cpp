@@ -27,10 +27,17 @@ void randomExec(Nd4jPointer *extra, int opNum, Nd4jPointer state, T *x, Long *xI
     RandomBuffer *rb = reinterpret_cast<RandomBuffer *>(state);
     if (rb == nullptr) return;
     std::vector<Long> sx, sy, sz;
-    // on this entry point extraPointers[0] is not a shapeInfo slot, so shapes come from the arguments
-    const Long *hz = hostShapeInfo(nullptr, 0, zInfo, sz, s);
-    const Long *hx = operands >= 2 ? hostShapeInfo(nullptr, 0, xInfo, sx, s) : nullptr;
-    const Long *hy = operands >= 3 ? hostShapeInfo(nullptr, 0, yInfo, sy, s) : nullptr;
+    // The reference's device code decodes the shapeInfos itself and keeps the generator's position on the device, so
+    // its host side needs none of them; here the host advances the generator and sizes the launch.  nd4j passes the
+    // host copy of z's shapeInfo in extraPointers[0] on these calls: it is used when it is there and looks like one.
+    // Operands that share one shapeInfo buffer (x == z in place, x = y = z for the distributions) are read once.
+    const Long *hz = nullptr;
+    if (const Long *h0 = reinterpret_cast<const Long *>(slotOf(extra, X_HOST_X_SHAPE))) {
+        if (!isDeviceMemory(h0) && h0[0] >= 1 && h0[0] <= kMaxRank && (siOrder(h0) == 'c' || siOrder(h0) == 'f')) hz = h0;
+    }
+    if (hz == nullptr) hz = hostShapeInfo(nullptr, 0, zInfo, sz, s);
+    const Long *hx = operands >= 2 ? (xInfo == zInfo ? hz : hostShapeInfo(nullptr, 0, xInfo, sx, s)) : nullptr;
+    const Long *hy = operands >= 3 ? (yInfo == zInfo ? hz : (yInfo == xInfo ? hx : hostShapeInfo(nullptr, 0, yInfo, sy, s))) : nullptr;
     if (hz == nullptr || (operands >= 2 && hx == nullptr) || (operands >= 3 && hy == nullptr)) return;
 
     RandomPlan pl;

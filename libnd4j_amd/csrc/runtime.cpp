@@ -28,10 +28,15 @@ static void throwHip(const char *what, hipError_t e) {
     throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
 }
 
+// Calls that had to read a shapeInfo or a dimension array back from the device (each one a stream synchronisation)
+static std::atomic<long long> gHostFetches{0};
+long long hostFetchCount() { return gHostFetches.load(); }
+
 const Long *hostShapeInfo(Nd4jPointer *extra, int slot, const Long *arg, std::vector<Long> &storage, hipStream_t s) {
     if (void *h = slotOf(extra, slot)) return reinterpret_cast<const Long *>(h);
     if (arg == nullptr) return nullptr;
     if (!isDeviceMemory(arg)) return arg;
+    gHostFetches++;
     Long rank = 0;
     hipError_t e = hipMemcpyAsync(&rank, arg, sizeof(Long), hipMemcpyDeviceToHost, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
@@ -52,6 +57,7 @@ bool hostInts(const int *arg, int count, std::vector<int> &out, hipStream_t s) {
         for (int i = 0; i < count; i++) out[i] = arg[i];
         return true;
     }
+    gHostFetches++;
     hipError_t e = hipMemcpyAsync(out.data(), arg, count * sizeof(int), hipMemcpyDeviceToHost, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     if (e != hipSuccess) throwHip("fetching dimension", e);

@@ -56,6 +56,10 @@ bool isDeviceMemory(const void *p);
 // last case synchronises the stream).  Null when there is nothing to read.
 const Long *hostShapeInfo(Nd4jPointer *extra, int slot, const Long *arg, std::vector<Long> &storage, hipStream_t s);
 
+// How often hostShapeInfo / hostInts had to fetch from the device since the library was loaded: a caller that
+// passes the host copies and TAD tables of the CUDA convention keeps this at zero on the array-result calls.
+long long hostFetchCount();
+
 // Host copy of a small int array argument (`dimension`), which is a device pointer on this convention.
 bool hostInts(const int *arg, int count, std::vector<int> &out, hipStream_t s);
 

@@ -499,7 +499,9 @@ def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data
     def device_set(w):
         Z = w.operand(np.zeros(n, F32), zi)
         a_uni, a_gau, a_drop = w.raw(np.array([0, 1], F32)), w.raw(np.array([0, 1], F32)), w.raw(np.array([0.5], F32))
-        ex = dev.extra()
+        # the host copy of the result's shapeInfo in slot 0, as nd4j passes it on these calls: without it the library
+        # reads the shapeInfo back from the device, which synchronises the stream
+        ex, ex_d = dev.extra(zi), dev.extra(di)
         Xd = w.operand(xd, di)
         return [
             Case("uniform_fill", "random", n, 4 * n,
@@ -510,7 +512,7 @@ def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data
                  lambda lib: (cpu_gen(lib).random_xyz(RND_GAUSSIAN, cpu_state["z"], zi, cpu_state["z"], zi, cpu_state["z"], zi,
                                                      np.array([0, 1], F32)), cpu_state["z"])[1], True, Z.get),
             Case("dropout_inplace", "random", m, 8 * m,
-                 lambda: ops.execRandomFloat(ex, RND_DROPOUT, gen, Xd.ptr, Xd.info_ptr, Xd.ptr, Xd.info_ptr, a_drop.ptr),
+                 lambda: ops.execRandomFloat(ex_d, RND_DROPOUT, gen, Xd.ptr, Xd.info_ptr, Xd.ptr, Xd.info_ptr, a_drop.ptr),
                  lambda lib: (cpu_gen(lib).random_xz(RND_DROPOUT, cpu_state["x"], di, cpu_state["x"], di, np.array([0.5], F32)), cpu_state["x"])[1],
                  True, Xd.get)]
 
