@@ -207,3 +207,28 @@ def test_config4_random(gpu, lib):
         assert abs(float(kept.mean()) - 0.5) < 1e-3
     finally:
         w.free()
+
+
+def test_array_result_calls_need_no_read_back_from_the_device(gpu):
+    """Every benchmark case passes what the CUDA convention provides (host copies of the shapeInfos, TAD tables); with
+    that, no call may have to read a shapeInfo or a dimension array back from the device, because each read-back
+    synchronises the stream.  Small shapes: the host paths are the same as at full size."""
+    ops = gpu.dev.ops
+    builders = (lambda d: workloads.transform_tanh(d, n=1 << 12, copies=1),
+                lambda d: workloads.pairwise_broadcast(d, rows=64, cols=128, copies=1),
+                lambda d: workloads.pairwise_broadcast(d, rows=64, cols=128, dtype="float16", copies=1),
+                lambda d: workloads.reductions(d, rows=64, cols=128, copies=1),
+                lambda d: workloads.reduce3_pairs(d, rows=64, cols=128, copies=1),
+                lambda d: workloads.stats_softmax(d, rows=128, cols=64, copies=1),
+                lambda d: workloads.data_movement(d, rows=2048, cols=64, copies=1),
+                lambda d: workloads.random_fills(d, n=1 << 12, side=64, buffer_longs=1 << 10, copies=1))
+    for build in builders:
+        w = build(gpu.dev)
+        try:
+            for c in w.cases:
+                before = ops.amd_hostFetchCount()
+                c.gpu(0)
+                gpu.dev.sync()
+                assert ops.amd_hostFetchCount() == before, (w.name, c.name)
+        finally:
+            w.free()
