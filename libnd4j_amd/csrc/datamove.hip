@@ -148,7 +148,16 @@ __global__ void __launch_bounds__(kBlock) shuffleKernel(T *const *xs, const Long
                 (reinterpret_cast<uintptr_t>(z + ob) & 15) == 0) {
                 const Pack<T> *xa = reinterpret_cast<const Pack<T> *>(x + oa), *xb = reinterpret_cast<const Pack<T> *>(x + ob);
                 Pack<T> *za = reinterpret_cast<Pack<T> *>(z + oa), *zb = reinterpret_cast<Pack<T> *>(z + ob);
-                for (Long v = lane; v < tadLength / VEC; v += lanes) {
+                const Long nv = tadLength / VEC;
+                Long v = lane;
+                for (; v + lanes < nv; v += 2 * (Long)lanes) {  // four loads in flight
+                    const Pack<T> a0 = loadPack(xa + v), b0 = loadPack(xb + v), a1 = loadPack(xa + v + lanes), b1 = loadPack(xb + v + lanes);
+                    storePack(za + v, b0);
+                    storePack(zb + v, a0);
+                    storePack(za + v + lanes, b1);
+                    storePack(zb + v + lanes, a1);
+                }
+                for (; v < nv; v += lanes) {
                     const Pack<T> a = loadPack(xa + v), b = loadPack(xb + v);
                     storePack(za + v, b);
                     storePack(zb + v, a);
