@@ -118,6 +118,17 @@ __global__ void __launch_bounds__(kBlock) tearKernel(const T *x, const Long *xIn
     const Long xe = dEws(tadInfo), ze = dEws(zInfo);
     const int lanes = lanesPerTad<T>(tadLength), groups = kBlock / lanes;
     const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
+    if (lanes == kBlock && xe == 1 && ze == 1) {
+        // long contiguous TADs are cut into pieces of four vectors per lane, so that a few long TADs still fill the chip
+        const Long piece = (Long)kBlock * 4 * Pack<T>::N;
+        const Long pieces = (tadLength + piece - 1) / piece;
+        for (Long u = blockIdx.x; u < numTads * pieces; u += gridDim.x) {
+            const Long r = u / pieces, f0 = (u - r * pieces) * piece;
+            const Long len = tadLength - f0 < piece ? tadLength - f0 : piece;
+            copyRun<T, true>(x + tadOffsets[r] + f0, 1, tadInfo, reinterpret_cast<T *>(targets[r]) + f0, 1, zInfo, len, lane, lanes);
+        }
+        return;
+    }
     for (Long r = (Long)blockIdx.x * groups + g; r < numTads; r += (Long)gridDim.x * groups)
         copyRun<T, true>(x + tadOffsets[r], xe, tadInfo, targets[r], ze, zInfo, tadLength, lane, lanes);
 }

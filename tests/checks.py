@@ -479,7 +479,8 @@ def check_data_movement(be, dtypes=(np.float32, np.float64, np.float16), big=Fal
         tcases = [([5, 8], "c", [1], [1, 8], "c"), ([5, 8], "f", [1], [1, 8], "c"), ([4, 3, 6], "c", [1, 2], [3, 6], "c"),
                   ([4, 3, 6], "c", [1, 2], [3, 6], "f"), ([4, 3, 6], "f", [1, 2], [3, 6], "f")]
         if big:
-            tcases += [([40, 2048], "c", [1], [1, 2048], "c"), ([33, 20, 30], "c", [1, 2], [20, 30], "c")]
+            tcases += [([40, 2048], "c", [1], [1, 2048], "c"), ([33, 20, 30], "c", [1, 2], [20, 30], "c"),
+                       ([6, 9000], "c", [1], [1, 9000], "c"), ([5, 9001], "c", [1], [1, 9001], "c")]  # long TADs go in pieces
         for shape, order, dims, t_shape, t_order in tcases:
             buf, info, logical = _view(shape, order)
             x = _cast(buf, dt)
