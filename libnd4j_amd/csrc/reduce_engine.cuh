@@ -67,11 +67,11 @@ __device__ __forceinline__ typename Pol::Acc blockMerge(const Pol &pol, typename
     return a;
 }
 
-// Folds n contiguous elements starting at `p` (element positions base.. in the run) using `lanes`
+// Folds n contiguous elements starting at `p` (they are elements base, base + 1, .. of their run) using `lanes`
 // cooperating lanes, this lane being `lane`.
 template <class Pol>
 __device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc &acc, const typename Pol::T *p, Long n,
-                                               int lane, int lanes) {
+                                               int lane, int lanes, Long base = 0) {
     typedef typename Pol::T T;
     constexpr int VEC = Pack<T>::N;
     const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
@@ -79,7 +79,7 @@ __device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc
     if ((addr & (sizeof(T) - 1)) == 0) head = (Long)(((16 - (addr & 15)) & 15) / sizeof(T));
     else head = n;  // cannot be vectorised
     if (head > n) head = n;
-    for (Long i = lane; i < head; i += lanes) { pol.accumulate(acc, toCompute(p[i]), i); pol.checkpoint(acc); }
+    for (Long i = lane; i < head; i += lanes) { pol.accumulate(acc, toCompute(p[i]), base + i); pol.checkpoint(acc); }
     const Long nvec = (n - head) / VEC;
     const Pack<T> *pv = reinterpret_cast<const Pack<T> *>(p + head);
     Long v = lane;
@@ -91,17 +91,17 @@ __device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc
 #pragma unroll
         for (int u = 0; u < 4; u++) {
 #pragma unroll
-            for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[u].v[e]), head + (v + u * (Long)lanes) * VEC + e);
+            for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[u].v[e]), base + head + (v + u * (Long)lanes) * VEC + e);
             pol.checkpoint(acc);
         }
     }
     for (; v < nvec; v += lanes) {
         Pack<T> pk = loadPack(pv + v);
 #pragma unroll
-        for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk.v[e]), head + v * VEC + e);
+        for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk.v[e]), base + head + v * VEC + e);
         pol.checkpoint(acc);
     }
-    for (Long i = head + nvec * VEC + lane; i < n; i += lanes) { pol.accumulate(acc, toCompute(p[i]), i); pol.checkpoint(acc); }
+    for (Long i = head + nvec * VEC + lane; i < n; i += lanes) { pol.accumulate(acc, toCompute(p[i]), base + i); pol.checkpoint(acc); }
 }
 
 template <class Pol, int GROUP>
@@ -248,6 +248,27 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
     }
 }
 
+// A few very long contiguous TADs: blockIdx.x is the TAD, blockIdx.y one slice of it; the slices' accumulators go to
+// partials[slice * numTads + tad] and are merged by tadColFinish.  (One block per TAD would leave most of the chip idle.)
+template <class Pol>
+__global__ void __launch_bounds__(kBlock) tadRowSliceKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
+                                                            typename Pol::Acc *partials, const Long *offsets, Long tadLength,
+                                                            Long numTads, Long sliceLength) {
+    if (Pol::tables) lm::loadTables();
+    typedef typename Pol::Acc Acc;
+    __shared__ Acc smem[kBlock / kWave];
+    const Long r = blockIdx.x;
+    const Long f0 = (Long)blockIdx.y * sliceLength;
+    Long f1 = f0 + sliceLength;
+    if (f1 > tadLength) f1 = tadLength;
+    pol.setTad(r, z);
+    const typename Pol::T *tx = x + offsets[r];
+    Acc acc = pol.init(tx);
+    if (f0 < f1) foldContiguous<Pol>(pol, acc, tx + f0, f1 - f0, (int)threadIdx.x, kBlock, f0);
+    acc = blockMerge<Pol>(pol, acc, smem);
+    if (threadIdx.x == 0) partials[(Long)blockIdx.y * numTads + r] = acc;
+}
+
 // Merges the `splits` partial accumulators of each TAD: 64 TADs per block, the four waves of the block take
 // every fourth split (independent loads, several in flight), then merge through LDS.
 template <class Pol>
@@ -365,6 +386,25 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
                          Workspace ws) {
     typedef typename Pol::Acc Acc;
     if (pl.numTads <= 0) return;
+    if (pl.kind == TadPlan::ROW && pl.tadLength >= 16384 && pl.numTads <= 1024) {
+        // few long TADs: slices of at least 4096 elements, about 2048 blocks in all
+        Long slices = 2048 / pl.numTads;
+        const Long maxSlices = pl.tadLength / 4096;
+        if (slices > maxSlices) slices = maxSlices;
+        if (slices > 65535) slices = 65535;
+        while (slices > 1 && (size_t)slices * (size_t)pl.numTads * sizeof(Acc) > ws.bytes) slices /= 2;
+        if (slices >= 2) {
+            Long sliceLength = (pl.tadLength + slices - 1) / slices;
+            sliceLength = (sliceLength + 63) / 64 * 64;  // slices start on 16-byte boundaries whenever the TAD does
+            slices = (pl.tadLength + sliceLength - 1) / sliceLength;
+            Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+            hipLaunchKernelGGL((tadRowSliceKernel<Pol>), dim3((unsigned)pl.numTads, (unsigned)slices), dim3(kBlock), 0, s, pol, x, z,
+                               partials, pl.offsets, pl.tadLength, pl.numTads, sliceLength);
+            hipLaunchKernelGGL((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kWave - 1) / kWave)), dim3(kBlock), 0, s, pol, z,
+                               partials, pl.tadLength, pl.numTads, (int)slices);
+            return;
+        }
+    }
     if (pl.kind == TadPlan::ROW && pl.tadLength >= 32) {
         if (pl.tadLength >= 8192) {
             int grid = gridFor(pl.numTads, 1, kGridCap);

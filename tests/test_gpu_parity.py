@@ -436,6 +436,34 @@ def test_special_transforms(gpu, cpu):
                 assert np.array_equal(got, cpu.transform(41, x, xi, xi, e)), (shape, dim)
 
 
+def test_reductions_over_few_very_long_rows(gpu, cpu):
+    """A handful of contiguous TADs of several hundred thousand elements are reduced in slices (one block per TAD would
+    idle most of the chip): same results as the CPU checker and as float64 arithmetic."""
+    rs = np.random.RandomState(21)
+    for rows, cols in ((3, 200000), (1, 70001 * 3), (7, 65536)):
+        if rows == 1:
+            continue  # a single TAD is a full-array reduction, covered elsewhere
+        info = shape_info_np([rows, cols])
+        x = rs.randn(rows * cols).astype(np.float32)
+        m = x.astype(np.float64).reshape(rows, cols)
+        scale = np.abs(m).sum(axis=1) / np.sqrt(cols)
+        got = gpu.reduce(1, x, info, None, [1], rows).astype(np.float64)
+        assert np.all(np.abs(got - m.sum(axis=1)) <= 1e-5 * np.maximum(np.abs(m.sum(axis=1)), scale)), (rows, cols, "sum")
+        assert np.array_equal(gpu.reduce(3, x, info, None, [1], rows), m.max(axis=1).astype(np.float32)), (rows, cols, "max")
+        got = gpu.reduce(0, x, info, None, [1], rows).astype(np.float64)
+        assert np.all(np.abs(got - m.mean(axis=1)) <= 1e-5 * np.maximum(np.abs(m.mean(axis=1)), scale / cols)), (rows, cols, "mean")
+        assert np.array_equal(gpu.indexreduce(0, x, info, None, [1], rows), np.argmax(m, axis=1).astype(np.float32)), (rows, cols)
+        assert np.array_equal(gpu.indexreduce(0, x, info, None, [1], rows), cpu.indexreduce(0, x, info, None, [1], rows))
+        var = m.var(axis=1, ddof=1)
+        got = gpu.summarystats(0, 1, x, info, [1], rows).astype(np.float64)
+        assert np.all(np.abs(got - var) <= 1e-5 * var), (rows, cols, "variance")
+        xd = rs.randn(rows * cols)
+        assert np.allclose(gpu.reduce(1, xd, info, None, [1], rows), xd.reshape(rows, cols).sum(axis=1), rtol=1e-10, atol=1e-9)
+        xh = (rs.randn(rows * cols) * 0.1).astype(np.float16)
+        got = gpu.reduce(3, xh, info, None, [1], rows)
+        assert np.array_equal(got, xh.reshape(rows, cols).max(axis=1))
+
+
 def test_broadcast_over_gap_free_tads(gpu):
     """Rows of a dense c-order array and columns of a dense f-order one go through the kernel that walks the array as
     one vector; every result is a single IEEE operation, so numpy gives the expected bits.  Shapes whose TAD length is
