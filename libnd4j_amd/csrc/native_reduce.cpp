@@ -458,6 +458,7 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
         // the reference (special_ops.h:1483, 1533)
         SoftmaxPlan pl;
         const bool vector = rank <= 1 || (rank == 2 && (siShape(hx)[0] == 1 || siShape(hx)[1] == 1));
+        int walked = 1;  // the dimension of x that a row runs along
         if (vector) {
             pl.numRows = 1;
             pl.length = n;
@@ -465,6 +466,7 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
             // the stride of the dimension that is walked (the EWS field says the same for a vector)
             const int xd = (rank == 2 && siShape(hx)[0] != 1) ? 0 : rank - 1;
             const int zd = (siRank(hz) == 2 && siShape(hz)[0] != 1) ? 0 : siRank(hz) - 1;
+            walked = xd;
             pl.xEl = rank >= 1 ? siStride(hx)[xd] : 1;
             pl.zEl = siRank(hz) >= 1 ? siStride(hz)[zd] : 1;
         } else if (rank == 2 && siRank(hz) == 2) {
@@ -475,6 +477,28 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
             pl.zRow = siStride(hz)[0];
             pl.zEl = siStride(hz)[1];
         } else {
+            return true;
+        }
+        // Long rows that are few: a block (or a wave) per row would leave most of the chip idle and read the row three
+        // times.  The row maxima and the row sums of exp(x - max) come from the reduction kernels instead, which cut
+        // long rows into slices, and one elementwise pass finishes.  (Not for half: a row sum may exceed its range.)
+        const bool rowMajor = pl.xEl == 1 && pl.zEl == 1, colMajor = pl.xRow == 1 && pl.zRow == 1 && pl.numRows >= 256;
+        if (sizeof(T) >= 4 && rank >= 1 && pl.length >= 4096 && pl.numRows <= 4096 && (rowMajor || colMajor) &&
+            !softmaxFitsRegisters<T>(x, z, pl)) {
+            ResolvedTad tx;
+            if (!resolveTad(nullptr, 0, 0, hx, &walked, 1, tx, s)) return true;
+            const size_t perRow = ((size_t)pl.numRows * sizeof(T) + 255) / 256 * 256;
+            Scratch sc = scratchFor(s, 2 * perRow + kWorkspaceBytes);
+            T *maxima = reinterpret_cast<T *>(sc.rest.ptr);
+            T *sums = reinterpret_cast<T *>(reinterpret_cast<char *>(sc.rest.ptr) + perRow);
+            Workspace rest;
+            rest.ptr = reinterpret_cast<char *>(sc.rest.ptr) + 2 * perRow;
+            rest.bytes = sc.rest.bytes - 2 * perRow;
+            const TadPlan tp = tadPlanFrom(tx);
+            if (!launchReduceTad<T>(s, 3, x, nullptr, maxima, tp, rest)) return false;
+            if (!launchSoftmaxSums<T>(s, x, maxima, sums, tp, rest)) return false;
+            if (!launchSoftmaxFinish<T>(s, opNum, x, z, maxima, sums, pl)) return false;
+            checkLaunch("execTransform(softmax)", s);
             return true;
         }
         if (!launchSoftmax<T>(s, opNum, x, z, pl)) return false;

@@ -382,6 +382,112 @@ template <typename T, int MODE> void runSoftmax(hipStream_t s, const T *x, T *z,
     }
 }
 
+// true when runSoftmax would take one of the kernels that keep their rows in registers
+template <typename T> bool softmaxFitsRegisters(const T *x, const T *z, const SoftmaxPlan &pl) {
+    constexpr int N = Pack<T>::N;
+    constexpr int kColPacks = sizeof(T) == 2 ? 8 : 16;
+    if (!(aligned16(x) && aligned16(z))) return false;
+    if (pl.xEl == 1 && pl.zEl == 1 && pl.length % N == 0 && pl.length >= 16 * N &&
+        (pl.numRows == 1 || (pl.xRow % N == 0 && pl.zRow % N == 0)) && pl.length / N <= 256 * 16)
+        return true;
+    return pl.xRow == 1 && pl.zRow == 1 && pl.numRows % N == 0 && pl.xEl % N == 0 && pl.zEl % N == 0 && pl.numRows >= kWave &&
+           pl.length <= (Long)kColCols * kColPacks;
+}
+
+// Last step of the softmax family when the row maxima and the row sums of exp(x - max) came from the reduction
+// kernels (rows too long for registers): p = exp(x - max[r]) / sum[r], as the register-resident kernels compute it.
+// Threads run along the direction in which x is contiguous (alongRows: down the rows of an f-order matrix),
+// blockIdx.y walks the other one.
+template <typename T, int MODE>
+__global__ void __launch_bounds__(kBlock) softmaxFinishKernel(const T *x, T *z, const T *maxima, const T *sums, Long numRows,
+                                                              Long length, Long xRow, Long xEl, Long zRow, Long zEl, int alongRows) {
+    typedef typename Compute<T>::type C;
+    lm::loadTables();
+    const Long fastLen = alongRows ? numRows : length, slowLen = alongRows ? length : numRows;
+    for (Long sl = blockIdx.y; sl < slowLen; sl += gridDim.y) {
+        for (Long f = (Long)blockIdx.x * kBlock + threadIdx.x; f < fastLen; f += (Long)gridDim.x * kBlock) {
+            const Long r = alongRows ? f : sl, c = alongRows ? sl : f;
+            const C e = m::exp_(toCompute(x[r * xRow + c * xEl]) - toCompute(maxima[r]));
+            z[r * zRow + c * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(e, (C)1 / toCompute(sums[r])));
+        }
+    }
+}
+// The same with 16-byte accesses.  ALONG 0: rows are contiguous, blockIdx.y is the row and its maximum and sum are
+// uniform over the block.  ALONG 1: rows are adjacent in memory (f-order), blockIdx.y is the column and each lane
+// holds one vector of neighbouring rows with their maxima and sums.
+template <typename T, int MODE, int ALONG>
+__global__ void __launch_bounds__(kBlock) softmaxFinishVecKernel(const T *x, T *z, const T *maxima, const T *sums, Long fastVecs,
+                                                                 Long slowLen, Long xSlow, Long zSlow) {
+    typedef typename Compute<T>::type C;
+    constexpr int N = Pack<T>::N;
+    lm::loadTables();
+    for (Long sl = blockIdx.y; sl < slowLen; sl += gridDim.y) {
+        const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x + sl * xSlow);
+        Pack<T> *zv = reinterpret_cast<Pack<T> *>(z + sl * zSlow);
+        C mx = 0, inv = 0;
+        if (ALONG == 0) {
+            mx = toCompute(maxima[sl]);
+            inv = (C)1 / toCompute(sums[sl]);
+        }
+        for (Long v = (Long)blockIdx.x * kBlock + threadIdx.x; v < fastVecs; v += (Long)gridDim.x * kBlock) {
+            Pack<T> a = loadPack(xv + v), o, pm, ps;
+            if (ALONG == 1) {
+                pm = reinterpret_cast<const Pack<T> *>(maxima)[v];
+                ps = reinterpret_cast<const Pack<T> *>(sums)[v];
+            }
+#pragma unroll
+            for (int e = 0; e < N; e++) {
+                const C m1 = ALONG == 1 ? toCompute(pm.v[e]) : mx;
+                const C i1 = ALONG == 1 ? (C)1 / toCompute(ps.v[e]) : inv;
+                o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(a.v[e]) - m1), i1));
+            }
+            storePack(zv + v, o);
+        }
+    }
+}
+
+template <typename T>
+bool launchSoftmaxFinish(hipStream_t s, int opNum, const T *x, T *z, const T *maxima, const T *sums, const SoftmaxPlan &pl) {
+    if (pl.numRows <= 0 || pl.length <= 0) return true;
+    const int alongRows = (pl.xRow == 1 && pl.xEl != 1) ? 1 : 0;
+    const Long fastLen = alongRows ? pl.numRows : pl.length, slowLen = alongRows ? pl.length : pl.numRows;
+    constexpr int N = Pack<T>::N;
+    const Long xSlow = alongRows ? pl.xEl : pl.xRow, zSlow = alongRows ? pl.zEl : pl.zRow;
+    const bool contiguous = alongRows ? (pl.xRow == 1 && pl.zRow == 1) : (pl.xEl == 1 && pl.zEl == 1);
+    if (contiguous && fastLen % N == 0 && (slowLen == 1 || (xSlow % N == 0 && zSlow % N == 0)) && aligned16(x) && aligned16(z) &&
+        aligned16(maxima) && aligned16(sums)) {
+        const Long vecs = fastLen / N;
+        const dim3 vgrid((unsigned)gridFor(vecs, kBlock, 65535), (unsigned)(slowLen < 65535 ? slowLen : 65535));
+#define ND4J_FINISH_VEC(MODE)                                                                                              \
+    do {                                                                                                                   \
+        if (alongRows)                                                                                                     \
+            hipLaunchKernelGGL((softmaxFinishVecKernel<T, MODE, 1>), vgrid, dim3(kBlock), 0, s, x, z, maxima, sums, vecs,   \
+                               slowLen, xSlow, zSlow);                                                                     \
+        else                                                                                                               \
+            hipLaunchKernelGGL((softmaxFinishVecKernel<T, MODE, 0>), vgrid, dim3(kBlock), 0, s, x, z, maxima, sums, vecs,   \
+                               slowLen, xSlow, zSlow);                                                                     \
+    } while (0)
+        switch (opNum) {
+            case 38: ND4J_FINISH_VEC(0); return true;
+            case 39: ND4J_FINISH_VEC(1); return true;
+            case 40: ND4J_FINISH_VEC(2); return true;
+            default: return false;
+        }
+#undef ND4J_FINISH_VEC
+    }
+    const dim3 grid((unsigned)gridFor(fastLen, kBlock, 4096), (unsigned)(slowLen < 65535 ? slowLen : 65535));
+#define ND4J_FINISH(MODE)                                                                                                 \
+    hipLaunchKernelGGL((softmaxFinishKernel<T, MODE>), grid, dim3(kBlock), 0, s, x, z, maxima, sums, pl.numRows, pl.length, \
+                       pl.xRow, pl.xEl, pl.zRow, pl.zEl, alongRows)
+    switch (opNum) {
+        case 38: ND4J_FINISH(0); return true;
+        case 39: ND4J_FINISH(1); return true;
+        case 40: ND4J_FINISH(2); return true;
+        default: return false;
+    }
+#undef ND4J_FINISH
+}
+
 template <typename T> bool launchSoftmax(hipStream_t s, int opNum, const T *x, T *z, const SoftmaxPlan &pl) {
     switch (opNum) {
         case 38: runSoftmax<T, 0>(s, x, z, pl); return true;
@@ -495,6 +601,8 @@ template <typename T> void launchIsMaxTadFill(hipStream_t s, T *z, const T *inde
 
 #define INST(T)                                                                                           \
     template bool launchSoftmax<T>(hipStream_t, int, const T *, T *, const SoftmaxPlan &);                \
+    template bool softmaxFitsRegisters<T>(const T *, const T *, const SoftmaxPlan &);                     \
+    template bool launchSoftmaxFinish<T>(hipStream_t, int, const T *, T *, const T *, const T *, const SoftmaxPlan &); \
     template void launchIsMaxFill<T>(hipStream_t, T *, const T *, const FlatPlan &);                      \
     template void launchIsMaxTadFill<T>(hipStream_t, T *, const T *, const TadPlan &);
 INST(float)

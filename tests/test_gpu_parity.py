@@ -371,7 +371,10 @@ def test_special_transforms(gpu, cpu):
     for shape, order in (([37, 129], "c"), ([300, 17], "c"), ([9, 5000], "c"), ([1, 500], "c"), ([700, 1], "c"), ([1, 70001], "c"),
                          ([7, 100], "c"), ([6, 200], "c"), ([4, 600], "c"), ([5, 3000], "c"), ([3, 16384], "c"), ([2, 16388], "c"),
                          ([257, 96], "f"), ([64, 300], "f"), ([128, 200], "f"), ([96, 1500], "f"), ([64, 2048], "f"),
-                         ([64, 2052], "f"), ([8, 8], "c")):
+                         ([64, 2052], "f"), ([8, 8], "c"),
+                         # rows too long for registers: maxima and sums from the reduction kernels (sliced from 16384 on)
+                         ([32, 50257], "c"), ([4, 100000], "c"), ([3, 20000], "c"), ([6, 9001], "c"), ([100000, 1], "c"),
+                         ([256, 4100], "f"), ([300, 2500], "f")):
         n = int(np.prod(shape))
         xi = harness.shape_info(shape, order)
         x = rs.uniform(-6, 6, n).astype(np.float32)
@@ -395,7 +398,8 @@ def test_special_transforms(gpu, cpu):
     truth /= truth.sum(axis=1, keepdims=True)
     assert np.all(np.abs(got - truth) <= 2e-5 * truth)
     # half and double, row-major and column-major, short and long rows
-    for shape, order in (([64, 96], "c"), ([5, 4000], "c"), ([3, 30000], "c"), ([128, 600], "f"), ([64, 1100], "f")):
+    for shape, order in (([64, 96], "c"), ([5, 4000], "c"), ([3, 30000], "c"), ([128, 600], "f"), ([64, 1100], "f"),
+                         ([2, 70000], "c"), ([300, 4500], "f")):
         n = shape[0] * shape[1]
         od = "F" if order == "f" else "C"
         info = harness.shape_info(shape, order)
