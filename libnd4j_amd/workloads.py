@@ -356,6 +356,13 @@ def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
         cases.append(Case("logsoftmax_fused_corder", "special", n, 8 * n,
                           lambda: ops.execTransformFloat(ex_c, T_LOGSOFTMAX, X.ptr, XCI.ptr, T.ptr, XCI.ptr, None),
                           lambda lib: (lib.transform(T_LOGSOFTMAX, x, xci, tc, xci, None), tc)[1], True, T.get))
+        # few long rows (the same memory as [rows / 64, cols * 64]): row maxima and sums come from the sliced reductions
+        xli = harness.shape_info([rows // 64, cols * 64], "c")
+        XLI = w.raw(np.ascontiguousarray(xli, dtype=np.int64))
+        ex_l = dev.extra(xli, z_info=xli)
+        cases.append(Case("softmax_fused_long_rows", "special", n, 8 * n,
+                          lambda: ops.execTransformFloat(ex_l, T_SOFTMAX, X.ptr, XLI.ptr, T.ptr, XLI.ptr, None),
+                          lambda lib: (lib.transform(T_SOFTMAX, x, xli, tc, xli, None), tc)[1], True, T.get))
         cases.append(Case("ismax_whole", "special", n, 8 * n,
                           lambda: ops.execTransformFloat(ex_c, T_ISMAX, X.ptr, XCI.ptr, T.ptr, XCI.ptr, None),
                           lambda lib: (lib.transform(T_ISMAX, x, xci, tc, xci, None), tc)[1], True, T.get))

@@ -139,6 +139,13 @@ def test_config3_summary_stats_and_softmax_chain(gpu, lib):
         assert np.all(np.abs(fused - want) <= 2e-5 * np.maximum(want, 1e-30))
         logsm = _run(w.case("logsoftmax_fused_corder")).astype(np.float64).reshape(rows, cols)
         assert np.all(np.abs(logsm - np.log(truth_c)) <= 2e-5 * np.abs(np.log(truth_c)) + 1e-6)
+        # few long rows: the same memory read as [rows / 64, cols * 64]
+        ml = x.astype(np.float64).reshape(rows // 64, cols * 64)
+        truth_l = np.exp(ml - ml.max(axis=1, keepdims=True))
+        truth_l /= truth_l.sum(axis=1, keepdims=True)
+        fused = _run(w.case("softmax_fused_long_rows")).astype(np.float64).reshape(rows // 64, cols * 64)
+        assert np.all(np.abs(fused - truth_l) <= 2e-5 * truth_l + 1e-30)
+        assert np.all(np.abs(fused.sum(axis=1) - 1.0) <= 1e-5)
         # IsMax: one-hot of the first maximum, whole array and per row; bit-exact
         xf = x.reshape(rows, cols)
         # (the winning index travels as a value of the data type, in the reference too - execIndexReduceScalarFloat
