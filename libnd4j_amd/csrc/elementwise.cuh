@@ -181,6 +181,11 @@ __device__ __forceinline__ Long mapOffset64(const DimMap &m, unsigned long long 
     return off + (Long)idx * m.stride[0];
 }
 
+// for walks over whole arrays, which may hold more than 2^32 elements: 32-bit divisions while the index allows them
+__device__ __forceinline__ Long mapOffsetAny(const DimMap &m, Long idx) {
+    return idx <= 0xffffffffLL ? mapOffset32(m, (unsigned)idx) : mapOffset64(m, (unsigned long long)idx);
+}
+
 template <typename T, typename F>
 __global__ void __launch_bounds__(kBlock) ewGeneralKernel(const T *x, DimMap xm, const T *y, DimMap ym, T *z,
                                                           DimMap zm, Params<T> p, Long n) {

@@ -243,9 +243,9 @@ __global__ void __launch_bounds__(kBlock) randomPlainKernel(RandomCtx<TT> c, con
             if (strided) {
                 ox = i * xEws; oy = i * yEws; oz = i * zEws;
             } else {
-                ox = nOperands >= 2 ? mapOffset32(xm, (unsigned)i) : 0;
-                oy = nOperands >= 3 ? mapOffset32(ym, (unsigned)i) : 0;
-                oz = mapOffset32(zm, (unsigned)i);
+                ox = nOperands >= 2 ? mapOffsetAny(xm, i) : 0;
+                oy = nOperands >= 3 ? mapOffsetAny(ym, i) : 0;
+                oz = mapOffsetAny(zm, i);
             }
             C xv = nOperands >= 2 ? toCompute(x[ox]) : (C)0;
             C yv = nOperands >= 3 ? toCompute(y[oy]) : (C)0;
@@ -354,13 +354,13 @@ __global__ void __launch_bounds__(kBlock) choiceKernel(RandomCtx<TT> c, const TT
     for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < c.length; i += stride) {
         C prob = c.unit(i);
         C cum = (C)0;
-        Long oz = strided ? i * zEws : mapOffset32(zm, (unsigned)i);
+        Long oz = strided ? i * zEws : mapOffsetAny(zm, i);
         for (Long f = 0; f < yLength; f++) {
             // in the coordinate branch the reference indexes the probabilities with the OUTPUT index i
-            Long oy = strided ? f * yEws : mapOffset32(ym, (unsigned)i);
+            Long oy = strided ? f * yEws : mapOffsetAny(ym, i);
             cum = toCompute(fromCompute<TT>(cum + toCompute(y[oy])));
             if (prob <= cum || f == yLength - 1) {
-                Long ox = strided ? f * xEws : mapOffset32(xm, (unsigned)f);
+                Long ox = strided ? f * xEws : mapOffsetAny(xm, f);
                 z[oz] = x[ox];
                 break;
             }

@@ -358,7 +358,7 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
             { pol.accumulate(acc, toCompute(x[i * ews]), i); pol.checkpoint(acc); }
     } else {
         for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock)
-            { pol.accumulate(acc, toCompute(x[mapOffset32(xm, (unsigned)i)]), i); pol.checkpoint(acc); }
+            { pol.accumulate(acc, toCompute(x[mapOffsetAny(xm, i)]), i); pol.checkpoint(acc); }
     }
     acc = blockMerge<Pol>(pol, acc, smem);
     if (threadIdx.x == 0) partials[blockIdx.x] = acc;

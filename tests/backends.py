@@ -524,18 +524,19 @@ class GpuBackend(object):
         return self._reduce_like("execSummaryStats", op, x, x_info, None, dims, out_len, trailing=(int(bool(bias)),),
                                  pass_tads=pass_tads)
 
-    def _scalar(self, member, op, x, x_info, extra, trailing=()):
+    def _scalar(self, member, op, x, x_info, extra, trailing=(), raw=False):
         X = self._op(x, x_info)
         E, e = self._up(extra, x.dtype)
         r = getattr(self.ops, member + self._suffix(x))(self.dev.extra(x_info), op, X.ptr, X.info_ptr, e, *trailing)
         self._finish(X, E)
-        return x.dtype.type(r)
+        return float(r) if raw else x.dtype.type(r)
 
     def reduce_scalar(self, op, x, x_info, extra=None):
         return self._scalar("execReduceScalar", op, x, x_info, extra)
 
-    def indexreduce_scalar(self, op, x, x_info, extra=None):
-        return self._scalar("execIndexReduceScalar", op, x, x_info, extra)
+    def indexreduce_scalar(self, op, x, x_info, extra=None, raw=False):
+        """raw: the value as the entry point returns it (a float also for half data) rather than cast to x's type"""
+        return self._scalar("execIndexReduceScalar", op, x, x_info, extra, raw=raw)
 
     def summarystats_scalar(self, op, bias, x, x_info):
         return self._scalar("execSummaryStatsScalar", op, x, x_info, None, trailing=(int(bool(bias)),))

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 from golden_inputs import ulp_distance
-from libnd4j_amd import workloads
+from libnd4j_amd import harness, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -239,3 +239,64 @@ def test_array_result_calls_need_no_read_back_from_the_device(gpu):
                 assert ops.amd_hostFetchCount() == before, (w.name, c.name)
         finally:
             w.free()
+
+
+def test_arrays_of_more_than_2_to_the_31_elements(gpu):
+    """Lengths are Nd4jLong in the reference's entry points (blas/NativeOps.h): element indexes, vector counts and
+    reduction positions must not pass through 32 bits anywhere.  Half arrays keep the transfers to a few GB; the data are a
+    short pattern repeated, so that the expected results are known without a second pass of numpy arithmetic."""
+    n = (1 << 31) + 65539  # odd: the 16-byte vector path ends in a scalar tail
+    L = 4099
+    rs = np.random.RandomState(77)
+    px = rs.randint(-200, 200, L).astype(np.float16)
+    py = rs.randint(-200, 200, L).astype(np.float16)
+    reps = n // L + 1
+    x, y = np.tile(px, reps)[:n], np.tile(py, reps)[:n]
+    info = harness.shape_info([1, n])
+
+    def matches(out, pattern):
+        k = n // L
+        body = out[:k * L].view(np.uint16).reshape(k, L)
+        return bool(np.all(body == pattern.view(np.uint16))) and np.array_equal(out[k * L:].view(np.uint16),
+                                                                                 pattern[:n - k * L].view(np.uint16))
+
+    print("pairwise add over %d halves" % n, flush=True)
+    assert matches(gpu.pairwise(0, x, info, y, info, info), px + py)
+    del y
+    print("scalar multiply", flush=True)
+    assert matches(gpu.scalar(2, x, info, info, 0.5), (px.astype(np.float32) * np.float32(0.5)).astype(np.float16))
+    print("mean, max, argmax", flush=True)
+    tail = px[:n - (n // L) * L].astype(np.float64)
+    total = px.astype(np.float64).sum() * (n // L) + tail.sum()
+    # Mean divides by the length cast to int (include/ops/ops.h:2147), which wraps beyond 2^31 - 1: the reference's own
+    # result for this length, and so this library's
+    mean = total / (n - (1 << 32))
+    assert abs(gpu.reduce_scalar(0, x, info) - mean) <= 1e-2 * abs(mean) + 1e-3
+    where = (1 << 31) + 1000
+    x[where] = 300
+    assert gpu.reduce_scalar(3, x, info) == 300.0
+    # the position passes through the data type on its way back (the CUDA back end stores it in a half buffer before
+    # widening it, blas/cuda/NativeOps.cu execIndexReduceScalarHalf): beyond 65504 that is infinity
+    assert gpu.indexreduce_scalar(0, x, info, raw=True) == float("inf")
+    x[where] = px[where % L]
+    # in fp32 the position survives, rounded to the 24 bits of a float
+    print("argmax over %d floats" % n, flush=True)
+    xf = x.astype(np.float32)
+    xf[where] = 300
+    assert gpu.indexreduce_scalar(0, xf, info, raw=True) == float(np.float32(where))
+    del xf
+    # a view that is not element-wise strided and spans more than 2^32 positions of a c-order walk
+    print("transform over a padded [65537, 65536] view", flush=True)
+    rows, cols, pitch = 65537, 65536, 65544
+    del x
+    xv = np.tile(px, (rows * pitch) // L + 1)[:rows * pitch]
+    vinfo = harness.shape_info([rows, cols], strides=[pitch, 1], ews=0)
+    out = gpu.transform(0, xv, vinfo, vinfo)  # Abs
+    got = out[:(rows - 1) * pitch + cols]
+    want = np.abs(xv[:got.size]).view(np.uint16).reshape(-1)
+    grid_got = np.lib.stride_tricks.as_strided(got.view(np.uint16), (rows, cols), (pitch * 2, 2))
+    grid_want = np.lib.stride_tricks.as_strided(want, (rows, cols), (pitch * 2, 2))
+    assert np.array_equal(grid_got, grid_want)
+    # the padding between the rows is not touched
+    pad = np.lib.stride_tricks.as_strided(got.view(np.uint16)[cols:], (rows - 1, pitch - cols), (pitch * 2, 2))
+    assert not pad.any()
