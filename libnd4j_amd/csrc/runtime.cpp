@@ -94,8 +94,26 @@ struct CachedTad {
     TadPack pack;
     Long *devOffsets = nullptr;
     Long tadLength = 0;
+    ~CachedTad() { if (devOffsets != nullptr) (void)hipFree(devOffsets); }
 };
-std::map<std::vector<Long>, CachedTad *> gTadCache;
+std::map<std::vector<Long>, std::shared_ptr<CachedTad> > gTadCache;
+size_t gTadCacheBytes = 0;
+// Beyond this the cache is emptied (after the devices have drained: queued kernels may still read the tables).
+// Callers that pass their own TAD tables, as nd4j does, never fill it.
+const size_t kTadCacheLimitBytes = (size_t)1 << 30;
+const size_t kTadCacheLimitEntries = 16384;
+
+void dropTadCacheLocked() {
+    int current = 0, count = 0;
+    (void)hipGetDevice(&current);
+    (void)hipGetDeviceCount(&count);
+    for (int d = 0; d < count; d++) {
+        if (hipSetDevice(d) == hipSuccess) (void)hipDeviceSynchronize();
+    }
+    (void)hipSetDevice(current);
+    gTadCache.clear();  // a call that still holds an entry keeps it (and its device table) until it returns
+    gTadCacheBytes = 0;
+}
 }  // namespace
 
 Workspace workspaceFor(hipStream_t s, size_t minBytes) {
@@ -155,25 +173,31 @@ bool resolveTad(Nd4jPointer *extra, int hostSlot, int offsetSlot, const Long *ho
     std::vector<Long> key(hostXInfo, hostXInfo + siLength(rank));
     key.push_back(-777);
     for (int d : dims) key.push_back(d);
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    key.push_back(dev);  // the offsets live in this device's memory
 
     std::lock_guard<std::mutex> lock(gMutex);
     auto it = gTadCache.find(key);
-    CachedTad *c = nullptr;
+    std::shared_ptr<CachedTad> c;
     if (it != gTadCache.end()) {
         c = it->second;
     } else {
-        c = new CachedTad();
+        if (gTadCache.size() >= kTadCacheLimitEntries || gTadCacheBytes >= kTadCacheLimitBytes) dropTadCacheLocked();
+        c = std::make_shared<CachedTad>();
         computeTad(hostXInfo, dims.data(), dimLen, c->pack, true);
         c->tadLength = tadLengthOf(hostXInfo, dims.data(), dimLen);
         size_t bytes = c->pack.offsets.size() * sizeof(Long);
         hipError_t e = hipMalloc(reinterpret_cast<void **>(&c->devOffsets), bytes ? bytes : sizeof(Long));
-        if (e != hipSuccess) { delete c; throwHip("TAD offsets allocation", e); }
+        if (e != hipSuccess) { c->devOffsets = nullptr; throwHip("TAD offsets allocation", e); }
         if (bytes) {
             e = hipMemcpy(c->devOffsets, c->pack.offsets.data(), bytes, hipMemcpyHostToDevice);
-            if (e != hipSuccess) { (void)hipFree(c->devOffsets); delete c; throwHip("TAD offsets upload", e); }
+            if (e != hipSuccess) throwHip("TAD offsets upload", e);
         }
         gTadCache[key] = c;
+        gTadCacheBytes += bytes + c->pack.shapeInfo.size() * sizeof(Long) + key.size() * sizeof(Long);
     }
+    out.keep = c;
     out.hostInfo = c->pack.shapeInfo.data();
     out.devOffsets = c->devOffsets;
     out.numTads = c->pack.numTads;

@@ -6,6 +6,7 @@
 
 #include <atomic>
 #include <cstdio>
+#include <memory>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -83,6 +84,7 @@ struct ResolvedTad {
     const Long *devOffsets = nullptr;
     Long numTads = 0;
     Long tadLength = 0;
+    std::shared_ptr<const void> keep;  // keeps a cached table's host side alive while this call uses it
 };
 // Uses extraPointers[hostSlot]/[offsetSlot] when both are present; otherwise computes the TAD from the
 // host xShapeInfo and `dimension` (fetched from the device if needed), uploads the offsets once and caches
