@@ -479,12 +479,15 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
         } else {
             return true;
         }
-        // Long rows that are few: a block (or a wave) per row would leave most of the chip idle and read the row three
-        // times.  The row maxima and the row sums of exp(x - max) come from the reduction kernels instead, which cut
-        // long rows into slices, and one elementwise pass finishes.  (Not for half: a row sum may exceed its range.)
-        const bool rowMajor = pl.xEl == 1 && pl.zEl == 1, colMajor = pl.xRow == 1 && pl.zRow == 1 && pl.numRows >= 256;
-        if (sizeof(T) >= 4 && rank >= 1 && pl.length >= 4096 && pl.numRows <= 4096 && (rowMajor || colMajor) &&
-            !softmaxFitsRegisters<T>(x, z, pl)) {
+        // Rows that do not fit the register-resident kernels.  A block (or a wave) per row would read the row three
+        // times, and would leave most of the chip idle when the rows are few.  The row maxima and the row sums of
+        // exp(x - max) come from one pass of the reduction kernels instead, which cut long rows into slices, and one
+        // elementwise pass finishes: 12 bytes per element.  Measured against the per-row kernels this wins for rows of
+        // 16384 elements or more, for shorter rows when they are few, and always for f-order matrices.  (Not for half:
+        // a row sum may exceed its range.)
+        const bool rowMajor = pl.xEl == 1 && pl.zEl == 1 && (pl.length >= 16384 || (pl.length >= 4096 && pl.numRows <= 512));
+        const bool colMajor = pl.xRow == 1 && pl.zRow == 1 && pl.numRows >= 256 && pl.length >= 256;
+        if (sizeof(T) >= 4 && rank >= 1 && (rowMajor || colMajor) && !softmaxFitsRegisters<T>(x, z, pl)) {
             ResolvedTad tx;
             if (!resolveTad(nullptr, 0, 0, hx, &walked, 1, tx, s)) return true;
             const size_t perRow = ((size_t)pl.numRows * sizeof(T) + 255) / 256 * 256;
@@ -495,8 +498,7 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
             rest.ptr = reinterpret_cast<char *>(sc.rest.ptr) + 2 * perRow;
             rest.bytes = sc.rest.bytes - 2 * perRow;
             const TadPlan tp = tadPlanFrom(tx);
-            if (!launchReduceTad<T>(s, 3, x, nullptr, maxima, tp, rest)) return false;
-            if (!launchSoftmaxSums<T>(s, x, maxima, sums, tp, rest)) return false;
+            if (!launchSoftmaxStats<T>(s, x, maxima, sums, tp, rest)) return false;
             if (!launchSoftmaxFinish<T>(s, opNum, x, z, maxima, sums, pl)) return false;
             checkLaunch("execTransform(softmax)", s);
             return true;

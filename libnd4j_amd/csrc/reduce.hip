@@ -69,14 +69,10 @@ ND4J_REDUCE(23, NormFrobenius, START_ZERO, {
 ND4J_REDUCE(24, NormP, START_ZERO, return m::pow_(m::abs_(d1), (C)p[0]);, ND4J_SUM_UPD, return m::pow_(r, (C)1 / (C)p[0]);)
 ND4J_REDUCE(25, SquaredNorm, START_ZERO, return d1 * d1;, ND4J_SUM_UPD, return r;)
 ND4J_REDUCE(26, CountZero, START_ZERO, return d1 == (C)0 ? (C)1 : (C)0;, ND4J_SUM_UPD, return r;)
-// Not an op number of the reference (the public dispatch stops below it): the row sums of exp(x - max) that the
-// softmax family needs for rows too long to keep in registers
-ND4J_REDUCE(27, SumExpShifted, START_ZERO, return m::exp_(d1 - shift);, ND4J_SUM_UPD, return r;)
 #undef ND4J_REDUCE
 #undef ND4J_SUM_UPD
 
 static constexpr int kReduceOpCount = 27;
-static constexpr int kSumExpShifted = 27;
 
 template <typename TT, int OP> struct ReducePol {
     typedef TT T;
@@ -84,14 +80,14 @@ template <typename TT, int OP> struct ReducePol {
     typedef C Acc;
     // ops whose functor or post-processing evaluates exp / log / pow (variance and standard deviation square their
     // bias term with pow); 20-23 have no functor
-    static constexpr bool tables = OP == 9 || OP == 10 || (OP >= 16 && OP <= 24) || OP == 27;
+    static constexpr bool tables = OP == 9 || OP == 10 || (OP >= 16 && OP <= 24);
     Params<TT> p;
     const TT *shiftSource;  // LogSumExp: per-TAD (TAD calls) or single (scalar calls) maximum; else null
     int shiftPerTad;
     C shift;
 
     __device__ __forceinline__ void setTad(Long r, const TT *) {
-        if (OP == 19 || OP == 27) shift = toCompute(shiftSource[shiftPerTad ? r : 0]);
+        if (OP == 19) shift = toCompute(shiftSource[shiftPerTad ? r : 0]);
     }
     __device__ __forceinline__ Acc init(const TT *first) const {
         if (ReduceOp<OP>::start == START_FIRST) return toCompute(first[0]);
@@ -153,21 +149,59 @@ bool launchReduceScalar(hipStream_t s, int opNum, const T *x, const T *extra, T 
                                                         extra, z, plan, ws);
 }
 
+// Row maximum and row sum of exp(x - maximum) in ONE pass, for the softmax family over rows too long for registers:
+// the running sum is rescaled whenever the running maximum rises, so each element costs one exp.  Not an op of the
+// reference (its loops take the maximum first, special_ops.h:1488-1518); the sums differ from a two-pass sum by the
+// roundings of the few rescalings.  The maximum is the stored result, the sum goes to a second per-row array.
+template <typename TT> struct SoftmaxStatsPol {
+    typedef TT T;
+    typedef typename Compute<TT>::type C;
+    struct Acc { C m, s; };
+    static constexpr bool tables = true;
+    TT *sums;
+    Long row;
+
+    __device__ __forceinline__ void setTad(Long r, const TT *) { row = r; }
+    __device__ __forceinline__ Acc init(const TT *first) const {
+        Acc a;
+        a.m = toCompute(first[0]);
+        a.s = (C)0;
+        return a;
+    }
+    __device__ __forceinline__ void accumulate(Acc &a, C v, Long) const {
+        const C d = v - a.m;
+        const C e = m::exp_(-m::abs_(d));
+        const bool rises = d > (C)0;
+        a.s = rises ? a.s * e + (C)1 : a.s + e;
+        a.m = rises ? v : a.m;
+    }
+    __device__ __forceinline__ void checkpoint(Acc &) const {}
+    __device__ __forceinline__ Acc combine(Acc a, Acc b) const {
+        Acc r;
+        r.m = m::max_(a.m, b.m);
+        // an accumulator that has seen nothing yet holds s == 0 and the row's first element as m
+        r.s = a.s * m::exp_(a.m - r.m) + b.s * m::exp_(b.m - r.m);
+        return r;
+    }
+    __device__ __forceinline__ TT finalize(Acc a, Long) const {
+        sums[row] = fromCompute<TT>(a.s);
+        return fromCompute<TT>(a.m);
+    }
+};
+
 template <typename T>
-bool launchSoftmaxSums(hipStream_t s, const T *x, const T *maxima, T *sums, const TadPlan &plan, Workspace ws) {
-    ReducePol<T, kSumExpShifted> pol;
-    pol.p.p = nullptr;
-    pol.shiftSource = maxima;
-    pol.shiftPerTad = 1;
-    pol.shift = 0;
-    runTadReduce(s, pol, x, sums, plan, ws);
+bool launchSoftmaxStats(hipStream_t s, const T *x, T *maxima, T *sums, const TadPlan &plan, Workspace ws) {
+    SoftmaxStatsPol<T> pol;
+    pol.sums = sums;
+    pol.row = 0;
+    runTadReduce(s, pol, x, maxima, plan, ws);
     return true;
 }
 
 #define INST(T)                                                                                                    \
     template bool launchReduceTad<T>(hipStream_t, int, const T *, const T *, T *, const TadPlan &, Workspace);     \
     template bool launchReduceScalar<T>(hipStream_t, int, const T *, const T *, T *, const FlatPlan &, Workspace); \
-    template bool launchSoftmaxSums<T>(hipStream_t, const T *, const T *, T *, const TadPlan &, Workspace);
+    template bool launchSoftmaxStats<T>(hipStream_t, const T *, T *, T *, const TadPlan &, Workspace);
 INST(float)
 INST(float16)
 INST(double)

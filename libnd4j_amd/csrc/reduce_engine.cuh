@@ -269,6 +269,23 @@ __global__ void __launch_bounds__(kBlock) tadRowSliceKernel(Pol pol, const typen
     if (threadIdx.x == 0) partials[(Long)blockIdx.y * numTads + r] = acc;
 }
 
+// Merges the slices of tadRowSliceKernel: one block per TAD, its threads take every kBlock-th slice and merge through
+// the wave butterflies and LDS (there are few TADs and up to thousands of slices).
+template <class Pol>
+__global__ void __launch_bounds__(kBlock) tadSliceFinish(Pol pol, const typename Pol::T *x, typename Pol::T *z,
+                                                         const typename Pol::Acc *__restrict__ partials, const Long *offsets,
+                                                         Long tadLength, Long numTads, int slices) {
+    if (Pol::tables) lm::loadTables();
+    typedef typename Pol::Acc Acc;
+    __shared__ Acc smem[kBlock / kWave];
+    const Long r = blockIdx.x;
+    pol.setTad(r, z);
+    Acc acc = pol.init(x + offsets[r]);  // what a lane that saw nothing holds, as in the slices themselves
+    for (int sl = threadIdx.x; sl < slices; sl += kBlock) acc = pol.combine(acc, partials[(Long)sl * numTads + r]);
+    acc = blockMerge<Pol>(pol, acc, smem);
+    if (threadIdx.x == 0) z[r] = pol.finalize(acc, tadLength);
+}
+
 // Merges the `splits` partial accumulators of each TAD: 64 TADs per block, the four waves of the block take
 // every fourth split (independent loads, several in flight), then merge through LDS.
 template <class Pol>
@@ -400,8 +417,8 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
             Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
             hipLaunchKernelGGL((tadRowSliceKernel<Pol>), dim3((unsigned)pl.numTads, (unsigned)slices), dim3(kBlock), 0, s, pol, x, z,
                                partials, pl.offsets, pl.tadLength, pl.numTads, sliceLength);
-            hipLaunchKernelGGL((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kWave - 1) / kWave)), dim3(kBlock), 0, s, pol, z,
-                               partials, pl.tadLength, pl.numTads, (int)slices);
+            hipLaunchKernelGGL((tadSliceFinish<Pol>), dim3((unsigned)pl.numTads), dim3(kBlock), 0, s, pol, x, z, partials,
+                               pl.offsets, pl.tadLength, pl.numTads, (int)slices);
             return;
         }
     }

@@ -412,37 +412,57 @@ __global__ void __launch_bounds__(kBlock) softmaxFinishKernel(const T *x, T *z, 
         }
     }
 }
-// The same with 16-byte accesses.  ALONG 0: rows are contiguous, blockIdx.y is the row and its maximum and sum are
-// uniform over the block.  ALONG 1: rows are adjacent in memory (f-order), blockIdx.y is the column and each lane
-// holds one vector of neighbouring rows with their maxima and sums.
+// The same with 16-byte accesses over the matrix as one list of vectors.  ALONG 0: rows are contiguous, a vector lies
+// within one row.  ALONG 1: rows are adjacent in memory (f-order), a vector holds neighbouring rows of one column, with
+// their maxima and sums as vectors too.  A capped grid walks the list (the lookup tables are staged once per block), and
+// each thread asks for its next vector before it works on the current one; the first is requested before the tables.
+template <typename T, int MODE, int ALONG> struct SoftmaxFinishItem {
+    typedef typename Compute<T>::type C;
+    Pack<T> a, pm, ps;
+    C mx, sum;
+    Long sl, v;
+    __device__ __forceinline__ void load(Long id, bool small, const T *x, const T *maxima, const T *sums, Long fastVecs, Long xSlow) {
+        sl = small ? (Long)((unsigned)id / (unsigned)fastVecs) : id / fastVecs;
+        v = id - sl * fastVecs;
+        a = loadPack(reinterpret_cast<const Pack<T> *>(x + sl * xSlow) + v);
+        if (ALONG == 1) {
+            pm = reinterpret_cast<const Pack<T> *>(maxima)[v];
+            ps = reinterpret_cast<const Pack<T> *>(sums)[v];
+        } else {
+            mx = toCompute(maxima[sl]);
+            sum = toCompute(sums[sl]);
+        }
+    }
+    __device__ __forceinline__ void finish(T *z, Long zSlow) const {
+        constexpr int N = Pack<T>::N;
+        Pack<T> o;
+        const C inv = ALONG == 1 ? (C)0 : (C)1 / sum;
+#pragma unroll
+        for (int e = 0; e < N; e++) {
+            const C m1 = ALONG == 1 ? toCompute(pm.v[e]) : mx;
+            const C i1 = ALONG == 1 ? (C)1 / toCompute(ps.v[e]) : inv;
+            o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(a.v[e]) - m1), i1));
+        }
+        storePack(reinterpret_cast<Pack<T> *>(z + sl * zSlow) + v, o);
+    }
+};
 template <typename T, int MODE, int ALONG>
 __global__ void __launch_bounds__(kBlock) softmaxFinishVecKernel(const T *x, T *z, const T *maxima, const T *sums, Long fastVecs,
                                                                  Long slowLen, Long xSlow, Long zSlow) {
-    typedef typename Compute<T>::type C;
-    constexpr int N = Pack<T>::N;
+    const Long total = fastVecs * slowLen, stride = (Long)gridDim.x * kBlock;
+    const bool small = total <= 0xffffffffLL;
+    Long id = (Long)blockIdx.x * kBlock + threadIdx.x;
+    SoftmaxFinishItem<T, MODE, ALONG> cur, next;
+    bool have = id < total;
+    if (have) cur.load(id, small, x, maxima, sums, fastVecs, xSlow);
     lm::loadTables();
-    for (Long sl = blockIdx.y; sl < slowLen; sl += gridDim.y) {
-        const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x + sl * xSlow);
-        Pack<T> *zv = reinterpret_cast<Pack<T> *>(z + sl * zSlow);
-        C mx = 0, inv = 0;
-        if (ALONG == 0) {
-            mx = toCompute(maxima[sl]);
-            inv = (C)1 / toCompute(sums[sl]);
-        }
-        for (Long v = (Long)blockIdx.x * kBlock + threadIdx.x; v < fastVecs; v += (Long)gridDim.x * kBlock) {
-            Pack<T> a = loadPack(xv + v), o, pm, ps;
-            if (ALONG == 1) {
-                pm = reinterpret_cast<const Pack<T> *>(maxima)[v];
-                ps = reinterpret_cast<const Pack<T> *>(sums)[v];
-            }
-#pragma unroll
-            for (int e = 0; e < N; e++) {
-                const C m1 = ALONG == 1 ? toCompute(pm.v[e]) : mx;
-                const C i1 = ALONG == 1 ? (C)1 / toCompute(ps.v[e]) : inv;
-                o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(a.v[e]) - m1), i1));
-            }
-            storePack(zv + v, o);
-        }
+    while (have) {
+        id += stride;
+        const bool more = id < total;
+        if (more) next.load(id, small, x, maxima, sums, fastVecs, xSlow);
+        cur.finish(z, zSlow);
+        cur = next;
+        have = more;
     }
 }
 
@@ -457,7 +477,7 @@ bool launchSoftmaxFinish(hipStream_t s, int opNum, const T *x, T *z, const T *ma
     if (contiguous && fastLen % N == 0 && (slowLen == 1 || (xSlow % N == 0 && zSlow % N == 0)) && aligned16(x) && aligned16(z) &&
         aligned16(maxima) && aligned16(sums)) {
         const Long vecs = fastLen / N;
-        const dim3 vgrid((unsigned)gridFor(vecs, kBlock, 65535), (unsigned)(slowLen < 65535 ? slowLen : 65535));
+        const dim3 vgrid((unsigned)gridFor(vecs * slowLen, kBlock, kGridCap));
 #define ND4J_FINISH_VEC(MODE)                                                                                              \
     do {                                                                                                                   \
         if (alongRows)                                                                                                     \

@@ -374,7 +374,7 @@ def test_special_transforms(gpu, cpu):
                          ([64, 2052], "f"), ([8, 8], "c"),
                          # rows too long for registers: maxima and sums from the reduction kernels (sliced from 16384 on)
                          ([32, 50257], "c"), ([4, 100000], "c"), ([3, 20000], "c"), ([6, 9001], "c"), ([100000, 1], "c"),
-                         ([256, 4100], "f"), ([300, 2500], "f")):
+                         ([256, 4100], "f"), ([300, 2500], "f"), ([600, 16500], "c"), ([520, 4100], "c")):
         n = int(np.prod(shape))
         xi = harness.shape_info(shape, order)
         x = rs.uniform(-6, 6, n).astype(np.float32)
