@@ -519,6 +519,42 @@ def test_nan_and_special_values(gpu, cpu):
     assert float(gpu.indexreduce_scalar(1, x, xi)) == float(cpu.indexreduce_scalar(1, x, xi))
 
 
+def test_empty_and_single_element_inputs(gpu, cpu):
+    """Lengths 0 and 1, the smallest TADs and the smallest number of TADs: what the reference's loops do when a caller
+    hands them nothing or next to nothing (strided overloads with n == 0 write nothing)."""
+    x = np.array([3.5, -2.0, 7.0, 1.0], np.float32)
+    for n, want in ((0, [0, 0, 0, 0]), (1, [3.5, 0, 0, 0])):
+        assert np.array_equal(gpu.transform_strided(0, x, 1, 1, None, n, zsize=4), want), n
+    assert gpu.pairwise_strided(0, x, 1, x, 1, 1, None, 0)[0] == 0.0 and gpu.pairwise_strided(0, x, 1, x, 1, 1, None, 1)[0] == 7.0
+    assert gpu.scalar_strided(0, x, 1, 1, 2.0, None, 0)[0] == 0.0 and gpu.scalar_strided(0, x, 1, 1, 2.0, None, 1)[0] == 5.5
+    one = shape_info_np([1, 1])
+    v = np.array([-4.25], np.float32)
+    assert gpu.transform(0, v, one, one)[0] == 4.25
+    assert gpu.pairwise(6, v, one, v, one, one)[0] == np.float32(-4.25) * np.float32(-4.25)
+    assert float(gpu.reduce_scalar(1, v, one)) == float(cpu.reduce_scalar(1, v, one)) == -4.25
+    assert float(gpu.reduce_scalar(3, v, one)) == -4.25
+    assert float(gpu.indexreduce_scalar(0, v, one)) == float(cpu.indexreduce_scalar(0, v, one)) == 0.0
+    for bias in (False, True):
+        assert float(gpu.summarystats_scalar(0, bias, v, one)) == float(cpu.summarystats_scalar(0, bias, v, one)) == 0.0
+    # TADs of length 1 (reducing a column vector along its unit dimension) and a single TAD spanning the array
+    col, row = shape_info_np([5, 1]), shape_info_np([1, 5])
+    w = np.array([2.0, -1.0, 9.0, 9.0, 0.5], np.float32)
+    for op in (0, 1, 3):
+        assert np.array_equal(gpu.reduce(op, w, col, None, [1], 5), cpu.reduce(op, w, col, None, [1], 5)), op
+        assert np.array_equal(gpu.reduce(op, w, row, None, [1], 1), cpu.reduce(op, w, row, None, [1], 1)), op
+    assert np.array_equal(gpu.indexreduce(0, w, col, None, [1], 5), np.zeros(5, np.float32))
+    assert np.array_equal(gpu.indexreduce(0, w, row, None, [1], 1), [2.0])
+    assert np.array_equal(gpu.summarystats(0, True, w, col, [1], 5), cpu.summarystats(0, True, w, col, [1], 5))
+    # softmax of a single element and of a single row; IsMax of a single element
+    assert gpu.transform(38, v, one, one)[0] == 1.0
+    assert gpu.transform(41, v, one, one)[0] == 1.0
+    sm = gpu.transform(38, w, row, row).astype(np.float64)
+    assert abs(sm.sum() - 1.0) <= 1e-6 and sm[2] == sm[3] == sm.max()
+    # broadcast of a one-element vector along a unit dimension
+    assert np.array_equal(gpu.broadcast(0, w, col, np.array([10.0], np.float32), shape_info_np([1, 1]), col, [1]),
+                          cpu.broadcast(0, w, col, np.array([10.0], np.float32), shape_info_np([1, 1]), col, [1]))
+
+
 def test_unknown_op_leaves_output_untouched(gpu, capfd):
     x = np.ones(64, np.float32)
     xi = shape_info_np([1, 64])
