@@ -660,3 +660,47 @@ def test_random_on_strided_output(gpu, cpu):
     assert a.state() == b.state()
     a.destroy()
     b.destroy()
+
+
+def test_concurrent_callers_on_their_own_streams():
+    """The reference's entry points are re-entrant: nd4j calls them from many threads, each with its own stream and
+    scratch (blas/cuda/NativeOps.cu:1609-1624).  Four threads with a stream each hammer the calls that touch the
+    library's shared state - the TAD cache (no caller tables), the per-stream workspace (which has to grow for the
+    long rows) and the pinned scalar slot - and every result is checked."""
+    import threading
+
+    errors = []
+
+    def worker(seed):
+        try:
+            be = backends.GpuBackend()
+            rs = np.random.RandomState(seed)
+            rows, cols = 48 + seed, 96
+            info = shape_info_np([rows, cols])
+            long_info = shape_info_np([3, 40000])
+            for it in range(12):
+                x = rs.randn(rows * cols).astype(np.float32)
+                m = x.reshape(rows, cols).astype(np.float64)
+                got = be.reduce(1, x, info, None, [1], rows, pass_tads=False)
+                assert np.allclose(got, m.sum(axis=1), rtol=1e-5, atol=1e-5), "sum dim1"
+                got = be.reduce(3, x, info, None, [0], cols, pass_tads=False)
+                assert np.array_equal(got, x.reshape(rows, cols).max(axis=0)), "max dim0"
+                assert abs(float(be.reduce_scalar(1, x, info)) - m.sum()) <= 1e-4 * np.abs(m).sum(), "sum"
+                assert float(be.indexreduce_scalar(0, x, info)) == float(np.argmax(x)), "argmax"
+                y = rs.randn(3 * 40000).astype(np.float32)
+                sm = be.transform(38, y, long_info, long_info).astype(np.float64).reshape(3, 40000)
+                rows64 = y.astype(np.float64).reshape(3, 40000)
+                truth = np.exp(rows64 - rows64.max(axis=1, keepdims=True))
+                truth /= truth.sum(axis=1, keepdims=True)
+                assert np.all(np.abs(sm - truth) <= 2e-5 * truth + 1e-30), "softmax"
+                assert np.array_equal(be.pairwise(0, x, info, x, info, info), x + x), "add"
+        except BaseException as e:  # noqa: B036 - reported by the main thread
+            errors.append((seed, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(s,)) for s in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads), "a caller did not finish"
+    assert errors == []
