@@ -7,6 +7,8 @@
 // As in the reference's CUDA back end every pointer these calls receive - data, shapeInfo, TAD tables, and the
 // tables of such pointers - is a device pointer, so the kernels decode shapeInfo themselves.  All of them are pure
 // copies: 16-byte streaming accesses wherever source and destination runs are contiguous and equally aligned.
+#include <type_traits>
+
 #include "elementwise.cuh"
 #include "launch.h"
 #include "reduce_engine.cuh"
@@ -445,22 +447,51 @@ template <typename S, typename D> __device__ __forceinline__ D convertOne(S v) {
     const float f = (float)toCompute(v);
     return fromCompute<D>((typename Compute<D>::type)f);
 }
+// Narrowing (or equal width): a thread converts 8 elements per pass, reading two or four 16-byte vectors and writing
+// one or two.  Widening: every store instruction should cover one contiguous stretch per wave (stores of 16 bytes
+// that alternate between the lanes' halves of 32-byte pieces were a third slower), so a thread converts the
+// 16 / sizeof(D) elements of ONE output vector per step and takes four steps a block-width apart.
 template <typename S, typename D>
 __global__ void __launch_bounds__(kBlock) convertKernel(const S *x, D *z, Long n, int vectors) {
-    constexpr int E = 8;  // elements per thread and pass: 16 bytes of half, 32 of float, 64 of double
+    constexpr bool widening = sizeof(D) > sizeof(S);
+    constexpr int E = widening ? 16 / (int)sizeof(D) : 8;
     const Long chunks = vectors ? n / E : 0;
-    for (Long c = (Long)blockIdx.x * kBlock + threadIdx.x; c < chunks; c += (Long)gridDim.x * kBlock) {
-        alignas(16) S in[E];
-        alignas(16) D out[E];
-        constexpr int NS = E * sizeof(S) / 16, ND = E * sizeof(D) / 16;
-        const U32x4 *src = reinterpret_cast<const U32x4 *>(x + c * E);
+    if (widening) {
+        constexpr int STEPS = 4;
+        typedef typename std::conditional<E * sizeof(S) == 8, unsigned long long, unsigned>::type Word;  // E source elements
+        for (Long c0 = (Long)blockIdx.x * (kBlock * STEPS) + threadIdx.x; c0 < chunks; c0 += (Long)gridDim.x * (kBlock * STEPS)) {
+            Word w[STEPS];
 #pragma unroll
-        for (int k = 0; k < NS; k++) reinterpret_cast<U32x4 *>(in)[k] = __builtin_nontemporal_load(src + k);
+            for (int k = 0; k < STEPS; k++) {
+                const Long c = c0 + (Long)k * kBlock;
+                if (c < chunks) w[k] = __builtin_nontemporal_load(reinterpret_cast<const Word *>(x) + c);
+            }
 #pragma unroll
-        for (int e = 0; e < E; e++) out[e] = convertOne<S, D>(in[e]);
-        U32x4 *dst = reinterpret_cast<U32x4 *>(z + c * E);
+            for (int k = 0; k < STEPS; k++) {
+                const Long c = c0 + (Long)k * kBlock;
+                if (c >= chunks) break;
+                alignas(8) S in[E];
+                alignas(16) D out[E];
+                *reinterpret_cast<Word *>(in) = w[k];
 #pragma unroll
-        for (int k = 0; k < ND; k++) __builtin_nontemporal_store(reinterpret_cast<const U32x4 *>(out)[k], dst + k);
+                for (int e = 0; e < E; e++) out[e] = convertOne<S, D>(in[e]);
+                __builtin_nontemporal_store(*reinterpret_cast<const U32x4 *>(out), reinterpret_cast<U32x4 *>(z) + c);
+            }
+        }
+    } else {
+        for (Long c = (Long)blockIdx.x * kBlock + threadIdx.x; c < chunks; c += (Long)gridDim.x * kBlock) {
+            alignas(16) S in[E];
+            alignas(16) D out[E];
+            constexpr int NS = E * sizeof(S) / 16, ND = E * sizeof(D) / 16;
+            const U32x4 *src = reinterpret_cast<const U32x4 *>(x + c * E);
+#pragma unroll
+            for (int k = 0; k < NS; k++) reinterpret_cast<U32x4 *>(in)[k] = __builtin_nontemporal_load(src + k);
+#pragma unroll
+            for (int e = 0; e < E; e++) out[e] = convertOne<S, D>(in[e]);
+            U32x4 *dst = reinterpret_cast<U32x4 *>(z + c * E);
+#pragma unroll
+            for (int k = 0; k < ND; k++) __builtin_nontemporal_store(reinterpret_cast<const U32x4 *>(out)[k], dst + k);
+        }
     }
     for (Long i = chunks * E + (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock)
         z[i] = convertOne<S, D>(x[i]);
@@ -468,7 +499,9 @@ __global__ void __launch_bounds__(kBlock) convertKernel(const S *x, D *z, Long n
 template <typename S, typename D> void runConvert(hipStream_t s, const void *x, void *z, Long n) {
     if (n <= 0) return;
     const int vectors = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(z)) & 15) == 0 ? 1 : 0;
-    hipLaunchKernelGGL((convertKernel<S, D>), dim3(gridFor(n, (Long)kBlock * 8, kMaxGrid)), dim3(kBlock), 0, s,
+    // elements per block and pass: 8 per thread when narrowing, four output vectors per thread when widening
+    const Long perBlock = sizeof(D) > sizeof(S) ? (Long)kBlock * 4 * (16 / (Long)sizeof(D)) : (Long)kBlock * 8;
+    hipLaunchKernelGGL((convertKernel<S, D>), dim3(gridFor(n, perBlock, kMaxGrid)), dim3(kBlock), 0, s,
                        reinterpret_cast<const S *>(x), reinterpret_cast<D *>(z), n, vectors);
 }
 // type codes of type_conversions.h:11-18: 3 half, 6 float, 7 double

@@ -266,6 +266,7 @@ __global__ void __launch_bounds__(kBlock) gaussianKernel(RandomCtx<TT> c, const 
     const C stddev = c.args[1];
     const Long pairs = (c.length + 1) / 2;
     const Long chunk = (Long)kBlock * kRngIter;
+    const bool pairStores = zEws == 1 && (reinterpret_cast<uintptr_t>(z) & (2 * sizeof(TT) - 1)) == 0;
     RngWalk w;
     for (Long base = (Long)blockIdx.x * chunk; base < pairs; base += (Long)gridDim.x * chunk)
     for (int it = 0; it < kRngIter; it++) {
@@ -280,11 +281,21 @@ __global__ void __launch_bounds__(kBlock) gaussianKernel(RandomCtx<TT> c, const 
         C z1 = r * m::sin_(ang);
         C m0 = yIsZ ? mean : toCompute(y[e * yEws]);
         C v0 = z0 * stddev + m0;
-        z[e * zEws] = fromCompute<TT>(EXP ? m::exp_(v0) : v0);
+        const TT r0 = fromCompute<TT>(EXP ? m::exp_(v0) : v0);
         if (e + 1 < c.length) {
             C m1 = yIsZ ? mean : toCompute(y[(e + 1) * yEws]);
             C v1 = z1 * stddev + m1;
-            z[(e + 1) * zEws] = fromCompute<TT>(EXP ? m::exp_(v1) : v1);
+            const TT r1 = fromCompute<TT>(EXP ? m::exp_(v1) : v1);
+            if (pairStores) {
+                // one store per pair: a wave's store then covers one contiguous stretch instead of every other element
+                struct alignas(2 * sizeof(TT)) Two { TT a, b; } two = {r0, r1};
+                *reinterpret_cast<Two *>(z + e) = two;
+            } else {
+                z[e * zEws] = r0;
+                z[(e + 1) * zEws] = r1;
+            }
+        } else {
+            z[e * zEws] = r0;
         }
     }
 }
