@@ -79,20 +79,25 @@ __device__ __forceinline__ u64 magicFor(u64 y) {
 }
 
 // RandomBuffer::safeShift (helper_generator.h:238-242): x > MAX / y ? x / y + 11 : x * y + 11.
-// For y < 2^32, "x > floor((2^64 - 1) / y)" is "x * y does not fit 64 bits", read off the 96-bit product, and
-// with m = floor((2^64 - 1) / y) the quotient is mulhi(x, m) or one more (x / y - x m / 2^64 lies in [0, 1)).
+// For y < 2^32 the caller passes m = floor((2^64 - 1) / y), which is the threshold of the comparison itself, and the
+// quotient is mulhi(x, m) or one more (x / y - x m / 2^64 lies in [0, 1)); the remainder that decides is below 2 y, so
+// for y < 2^31 its low 32 bits are enough.
 __device__ __forceinline__ u64 safeShiftDev(u64 x, u64 y, u64 m) {
     if (y == 0) return 11;
     if ((y >> 32) == 0) {
         const unsigned ys = (unsigned)y;
-        const u64 lo = (u64)(unsigned)x * ys;
-        const u64 hi = (x >> 32) * ys + (lo >> 32);
-        if ((hi >> 32) != 0) {
+        if (x > m) {
             u64 q = __umul64hi(x, m);
-            if (x - q * (u64)ys >= (u64)ys) q++;
+            if ((ys >> 31) == 0) {
+                const unsigned rem = (unsigned)x - (unsigned)q * ys;
+                if (rem >= ys) q++;
+            } else if (x - q * (u64)ys >= (u64)ys) {
+                q++;
+            }
             return q + 11;
         }
-        return ((hi << 32) | (lo & 0xffffffffULL)) + 11;
+        // x * y fits 64 bits
+        return (((x >> 32) * ys) << 32) + (u64)(unsigned)x * ys + 11;
     }
     if (x > 0xffffffffffffffffULL / y) return x / y + 11;
     return x * y + 11;
@@ -235,7 +240,13 @@ __global__ void __launch_bounds__(kBlock) randomPlainKernel(RandomCtx<TT> c, con
     typedef typename Compute<TT>::type C;
     const Long chunk = (Long)kBlock * kRngIter;
     RngWalk w;
-    for (Long base = (Long)blockIdx.x * chunk; base < c.length; base += (Long)gridDim.x * chunk) {
+    // a block takes consecutive chunks: its positions then stay within one or two generations of the buffer, and the
+    // multiplier of the generation divisor (RngWalk::m) is rarely recomputed
+    const Long nChunks = (c.length + chunk - 1) / chunk, perBlock = (nChunks + gridDim.x - 1) / gridDim.x;
+    Long lastChunk = ((Long)blockIdx.x + 1) * perBlock;
+    if (lastChunk > nChunks) lastChunk = nChunks;
+    for (Long ci = (Long)blockIdx.x * perBlock; ci < lastChunk; ci++) {
+        const Long base = ci * chunk;
         for (int k = 0; k < kRngIter; k++) {
             const Long i = base + (Long)k * kBlock + threadIdx.x;
             if (i >= c.length) break;
@@ -268,7 +279,11 @@ __global__ void __launch_bounds__(kBlock) gaussianKernel(RandomCtx<TT> c, const 
     const Long chunk = (Long)kBlock * kRngIter;
     const bool pairStores = zEws == 1 && (reinterpret_cast<uintptr_t>(z) & (2 * sizeof(TT) - 1)) == 0;
     RngWalk w;
-    for (Long base = (Long)blockIdx.x * chunk; base < pairs; base += (Long)gridDim.x * chunk)
+    // consecutive chunks per block, as in randomPlainKernel
+    const Long nChunks = (pairs + chunk - 1) / chunk, perBlock = (nChunks + gridDim.x - 1) / gridDim.x;
+    Long lastChunk = ((Long)blockIdx.x + 1) * perBlock;
+    if (lastChunk > nChunks) lastChunk = nChunks;
+    for (Long base = (Long)blockIdx.x * perBlock * chunk; base < lastChunk * chunk; base += chunk)
     for (int it = 0; it < kRngIter; it++) {
         const Long k = base + (Long)it * kBlock + threadIdx.x;
         if (k >= pairs) break;
