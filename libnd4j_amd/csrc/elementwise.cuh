@@ -299,9 +299,12 @@ __global__ void __launch_bounds__(kBlock) bcFlatKernel(const T *x, const T *y, T
     const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x);
     const Pack<T> *yv = reinterpret_cast<const Pack<T> *>(y);
     Pack<T> *zv = reinterpret_cast<Pack<T> *>(z);
+    const bool pow2 = (vecsPerTad & (vecsPerTad - 1)) == 0;
     for (Long j = (Long)blockIdx.x * kBlock + threadIdx.x; j < nvec; j += (Long)gridDim.x * kBlock) {
         const Pack<T> a = loadPack(xv + j);
-        const unsigned col = (j >> 32) == 0 ? (unsigned)j % vecsPerTad : (unsigned)((unsigned long long)j % vecsPerTad);
+        unsigned col;
+        if (pow2) col = (unsigned)j & (vecsPerTad - 1);  // the usual case: no division
+        else col = (j >> 32) == 0 ? (unsigned)j % vecsPerTad : (unsigned)((unsigned long long)j % vecsPerTad);
         const Pack<T> b = yv[col];
         Pack<T> r;
 #pragma unroll
