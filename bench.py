@@ -110,7 +110,7 @@ def load_cpu():
     return lib, ("reference" if lib.kind == "reference" else "port")
 
 
-def cpu_time(fn, lib, budget_s, min_runs=3, max_runs=200):
+def cpu_time(fn, lib, budget_s, min_runs=3, max_runs=5000):
     fn(lib)  # warm-up (page faults of the output buffer, OpenMP pool start)
     times = []
     start = time.perf_counter()
