@@ -240,9 +240,13 @@ __global__ void __launch_bounds__(kBlock) concatPrepareKernel(const void *const 
 // inputs into a C-contiguous result move as 16-byte vectors, one per thread: vector j of the input belongs to run
 // j / runV and lands zRunV vectors further on for every run.  Other layouts are walked in the input's logical C order.
 template <typename T>
-__global__ void __launch_bounds__(kBlock) concatKernel(const Long *const *infos, T *z, ConcatView v, const ConcatDesc *desc, int n) {
+__global__ void __launch_bounds__(kBlock) concatKernel(const Long *const *infos, T *z, ConcatView v, const ConcatDesc *desc, int n,
+                                                       int inputFastest) {
     constexpr int VEC = Pack<T>::N;
-    for (int r = blockIdx.y; r < n; r += gridDim.y) {
+    // inputFastest: neighbouring blocks take the same stretch of different inputs, whose short runs are neighbours in z
+    const Long bx = inputFastest ? blockIdx.y : blockIdx.x, gdx = inputFastest ? gridDim.y : gridDim.x;
+    const int by = inputFastest ? blockIdx.x : blockIdx.y, gdy = inputFastest ? gridDim.x : gridDim.y;
+    for (int r = by; r < n; r += gdy) {
         const ConcatDesc d = desc[r];
         const T *x = reinterpret_cast<const T *>(d.data);
         if (d.fast) {
@@ -254,12 +258,23 @@ __global__ void __launch_bounds__(kBlock) concatKernel(const Long *const *infos,
                 const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x);
                 Pack<T> *zv = reinterpret_cast<Pack<T> *>(zb);
                 const bool small = (nv >> 32) == 0;
-                for (Long j = (Long)blockIdx.x * kBlock + threadIdx.x; j < nv; j += (Long)gridDim.x * kBlock) {
-                    const Long o = runV >= nv ? 0 : (small ? (Long)((unsigned)j / (unsigned)runV) : j / runV);
-                    storePack(zv + o * zRunV + (j - o * runV), loadPack(xv + j));
+                // a block moves four vectors per thread, all four loads in flight before the first store
+                constexpr int STEPS = 4;
+                for (Long j0 = bx * (kBlock * STEPS) + threadIdx.x; j0 < nv; j0 += gdx * (kBlock * STEPS)) {
+                    Pack<T> a[STEPS];
+#pragma unroll
+                    for (int k = 0; k < STEPS; k++)
+                        if (j0 + k * kBlock < nv) a[k] = loadPack(xv + j0 + k * kBlock);
+#pragma unroll
+                    for (int k = 0; k < STEPS; k++) {
+                        const Long j = j0 + k * kBlock;
+                        if (j >= nv) break;
+                        const Long o = runV >= nv ? 0 : (small ? (Long)((unsigned)j / (unsigned)runV) : j / runV);
+                        storePack(zv + o * zRunV + (j - o * runV), a[k]);
+                    }
                 }
             } else {
-                for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < d.length; i += (Long)gridDim.x * kBlock) {
+                for (Long i = bx * kBlock + threadIdx.x; i < d.length; i += gdx * kBlock) {
                     const Long o = i / d.run;
                     zb[o * zRun + (i - o * d.run)] = x[i];
                 }
@@ -269,7 +284,7 @@ __global__ void __launch_bounds__(kBlock) concatKernel(const Long *const *infos,
             const int rank = dRank(si);
             if (rank != v.rank) continue;
             const Long *shape = dShape(si), *stride = dStride(si);
-            for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < d.length; i += (Long)gridDim.x * kBlock) {
+            for (Long i = bx * kBlock + threadIdx.x; i < d.length; i += gdx * kBlock) {
                 Long rem = i, xo = 0, zo = 0;
                 for (int dd = rank - 1; dd >= 0; dd--) {
                     const Long q = rem / shape[dd], c = rem - q * shape[dd];
@@ -392,11 +407,15 @@ void launchConcat(hipStream_t s, const T *const *data, const Long *const *infos,
     ConcatDesc *desc = reinterpret_cast<ConcatDesc *>(scratch);
     hipLaunchKernelGGL(concatPrepareKernel, dim3(1), dim3(kBlock), 0, s, reinterpret_cast<const void *const *>(data), infos, n, v, desc);
     const int gy = n < 65535 ? n : 65535;
-    // one 16-byte vector per thread while that keeps the grid below 2^22 blocks
+    // four 16-byte vectors per thread while that keeps the grid below 2^22 blocks
     int budget = (1 << 22) / gy;
     if (budget < 1) budget = 1;
-    const int gx = gridFor(maxLength > 0 ? maxLength : 1, (Long)kBlock * Pack<T>::N, budget);
-    hipLaunchKernelGGL((concatKernel<T>), dim3(gx, gy), dim3(kBlock), 0, s, infos, z, v, desc, n);
+    const int gx = gridFor(maxLength > 0 ? maxLength : 1, (Long)kBlock * 4 * Pack<T>::N, budget);
+    // Short runs (the inputs' slabs alternate in z every few KB): blocks that run together should fill neighbouring
+    // runs, so the input index varies fastest.  Long runs: one input after the other.
+    const bool inputFastest = v.dim > 0 && n > 1 && gx <= 65535;
+    if (inputFastest) hipLaunchKernelGGL((concatKernel<T>), dim3(gy, gx), dim3(kBlock), 0, s, infos, z, v, desc, n, 1);
+    else hipLaunchKernelGGL((concatKernel<T>), dim3(gx, gy), dim3(kBlock), 0, s, infos, z, v, desc, n, 0);
 }
 size_t concatScratchBytes(int numArrays) { return (size_t)(numArrays > 0 ? numArrays : 1) * sizeof(ConcatDesc); }
 
