@@ -163,6 +163,19 @@ __global__ void __launch_bounds__(kBlock) shuffleKernel(T *const *xs, const Long
                 Pack<T> *za = reinterpret_cast<Pack<T> *>(z + oa), *zb = reinterpret_cast<Pack<T> *>(z + ob);
                 const Long nv = tadLength / VEC;
                 Long v = lane;
+                for (; v + 3 * (Long)lanes < nv; v += 4 * (Long)lanes) {  // eight loads in flight: a 4 KiB float row per wave in one go
+                    Pack<T> a[4], b[4];
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        a[k] = loadPack(xa + v + k * lanes);
+                        b[k] = loadPack(xb + v + k * lanes);
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        storePack(za + v + k * lanes, b[k]);
+                        storePack(zb + v + k * lanes, a[k]);
+                    }
+                }
                 for (; v + lanes < nv; v += 2 * (Long)lanes) {  // four loads in flight
                     const Pack<T> a0 = loadPack(xa + v), b0 = loadPack(xb + v), a1 = loadPack(xa + v + lanes), b1 = loadPack(xb + v + lanes);
                     storePack(za + v, b0);
