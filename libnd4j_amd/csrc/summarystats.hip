@@ -16,7 +16,7 @@ struct StatsAcc {
     double cn, cs1, cs2, cp; // current run: count, shifted sums, shift
 };
 
-static constexpr double kStatsRun = 32.0;
+static constexpr double kStatsRun = 128.0;
 
 __device__ __forceinline__ void statsMerge(double &n, double &mean, double &m2, double nb, double meanb, double m2b) {
     if (nb == 0.0) return;
