@@ -336,26 +336,40 @@ template <typename T, int MODE, int PACKS> void runColReg(hipStream_t s, const T
                        pl.zEl);
 }
 
-template <typename T, int MODE> void runSoftmax(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
-    if (pl.numRows <= 0 || pl.length <= 0) return;
+// Which kind of kernel a softmax call gets: rows in registers, neighbouring rows in registers, or three passes.
+enum SoftmaxRoute { SM_ROW_REGISTERS, SM_COL_REGISTERS, SM_PASSES };
+template <typename T> SoftmaxRoute softmaxRoute(const T *x, const T *z, const SoftmaxPlan &pl) {
     constexpr int N = Pack<T>::N;
     // vectors a thread of the neighbouring-rows kernel may hold: a half vector unpacks to eight float maxima and
     // sums, which leaves room for fewer of them
     constexpr int kColPacks = sizeof(T) == 2 ? 8 : 16;
-    const bool base16 = aligned16(x) && aligned16(z);
-    // rows in registers: contiguous rows whose vectors are aligned in every row
-    if (base16 && pl.xEl == 1 && pl.zEl == 1 && pl.length % N == 0 && pl.length >= 16 * N &&
-        (pl.numRows == 1 || (pl.xRow % N == 0 && pl.zRow % N == 0))) {
+    if (!(aligned16(x) && aligned16(z))) return SM_PASSES;
+    // contiguous rows whose vectors are aligned in every row, up to 16 vectors for each of 256 lanes
+    if (pl.xEl == 1 && pl.zEl == 1 && pl.length % N == 0 && pl.length >= 16 * N &&
+        (pl.numRows == 1 || (pl.xRow % N == 0 && pl.zRow % N == 0)) && pl.length / N <= 256 * 16)
+        return SM_ROW_REGISTERS;
+    // an f-order matrix whose column stride keeps the row vectors aligned
+    if (pl.xRow == 1 && pl.zRow == 1 && pl.numRows % N == 0 && pl.xEl % N == 0 && pl.zEl % N == 0 && pl.numRows >= kWave &&
+        pl.length <= (Long)kColCols * kColPacks && (Long)((pl.numRows + 8 * N - 1) / (8 * N)) <= kMaxGrid)
+        return SM_COL_REGISTERS;
+    return SM_PASSES;
+}
+
+template <typename T, int MODE> void runSoftmax(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
+    if (pl.numRows <= 0 || pl.length <= 0) return;
+    constexpr int N = Pack<T>::N;
+    constexpr int kColPacks = sizeof(T) == 2 ? 8 : 16;
+    const SoftmaxRoute route = softmaxRoute<T>(x, z, pl);
+    if (route == SM_ROW_REGISTERS) {
         const Long npack = pl.length / N;
-        if (npack <= 16 * 2) { runRowReg<T, MODE, 16, 2>(s, x, z, pl); return; }
-        if (npack <= 64 * 2) { runRowReg<T, MODE, 64, 2>(s, x, z, pl); return; }
-        if (npack <= 64 * 8) { runRowReg<T, MODE, 64, 8>(s, x, z, pl); return; }
-        if (npack <= 256 * 4) { runRowReg<T, MODE, kBlock, 4>(s, x, z, pl); return; }
-        if (npack <= 256 * 16) { runRowReg<T, MODE, kBlock, 16>(s, x, z, pl); return; }
+        if (npack <= 16 * 2) runRowReg<T, MODE, 16, 2>(s, x, z, pl);
+        else if (npack <= 64 * 2) runRowReg<T, MODE, 64, 2>(s, x, z, pl);
+        else if (npack <= 64 * 8) runRowReg<T, MODE, 64, 8>(s, x, z, pl);
+        else if (npack <= 256 * 4) runRowReg<T, MODE, kBlock, 4>(s, x, z, pl);
+        else runRowReg<T, MODE, kBlock, 16>(s, x, z, pl);
+        return;
     }
-    // neighbouring rows in registers: an f-order matrix whose column stride keeps the row vectors aligned
-    if (base16 && pl.xRow == 1 && pl.zRow == 1 && pl.numRows % N == 0 && pl.xEl % N == 0 && pl.zEl % N == 0 &&
-        pl.numRows >= kWave && pl.length <= (Long)kColCols * kColPacks && (Long)((pl.numRows + 8 * N - 1) / (8 * N)) <= kMaxGrid) {
+    if (route == SM_COL_REGISTERS) {
         if (pl.length <= (Long)kColCols * 2) runColReg<T, MODE, 2>(s, x, z, pl);
         else if (pl.length <= (Long)kColCols * kColPacks / 2) runColReg<T, MODE, kColPacks / 2>(s, x, z, pl);
         else runColReg<T, MODE, kColPacks>(s, x, z, pl);
@@ -384,14 +398,7 @@ template <typename T, int MODE> void runSoftmax(hipStream_t s, const T *x, T *z,
 
 // true when runSoftmax would take one of the kernels that keep their rows in registers
 template <typename T> bool softmaxFitsRegisters(const T *x, const T *z, const SoftmaxPlan &pl) {
-    constexpr int N = Pack<T>::N;
-    constexpr int kColPacks = sizeof(T) == 2 ? 8 : 16;
-    if (!(aligned16(x) && aligned16(z))) return false;
-    if (pl.xEl == 1 && pl.zEl == 1 && pl.length % N == 0 && pl.length >= 16 * N &&
-        (pl.numRows == 1 || (pl.xRow % N == 0 && pl.zRow % N == 0)) && pl.length / N <= 256 * 16)
-        return true;
-    return pl.xRow == 1 && pl.zRow == 1 && pl.numRows % N == 0 && pl.xEl % N == 0 && pl.zEl % N == 0 && pl.numRows >= kWave &&
-           pl.length <= (Long)kColCols * kColPacks;
+    return softmaxRoute<T>(x, z, pl) != SM_PASSES;
 }
 
 // Last step of the softmax family when the row maxima and the row sums of exp(x - max) came from the reduction
