@@ -176,11 +176,13 @@ template <typename T> struct Reduce3Body {
                 Long sliceLength = (pl.runLength + slices - 1) / slices;
                 sliceLength = (sliceLength + 63) / 64 * 64;
                 slices = (pl.runLength + sliceLength - 1) / sliceLength;
-                Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
-                hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)slices), dim3(kBlock), 0, s, x, y, z, extra, pl,
-                                   partials, sliceLength);
-                hipLaunchKernelGGL((reduce3Finish<T, OP>), dim3(1), dim3(kBlock), 0, s, z, partials, (int)slices, pl.runLength);
-                return true;
+                if (slices >= 2) {  // a single slice needs no second launch: the per-result kernels below do it in one
+                    Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+                    hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)slices), dim3(kBlock), 0, s, x, y, z, extra, pl,
+                                       partials, sliceLength);
+                    hipLaunchKernelGGL((reduce3Finish<T, OP>), dim3(1), dim3(kBlock), 0, s, z, partials, (int)slices, pl.runLength);
+                    return true;
+                }
             }
             Acc *none = nullptr;
             if (pl.runLength >= 4096) {

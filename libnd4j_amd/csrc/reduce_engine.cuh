@@ -332,9 +332,10 @@ __global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typena
 }
 
 // Stage 1 of the full-array reduction: block b folds the chunks b, b+grid, ... of kBlock*kUnroll vectors.
+// A one-block launch (small arrays) is handed the result pointer and finishes by itself.
 template <class Pol>
 __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol::T *x, typename Pol::Acc *partials,
-                                                     Long n, int strided, Long ews, DimMap xm) {
+                                                     Long n, int strided, Long ews, DimMap xm, typename Pol::T *zDirect) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
@@ -378,7 +379,10 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
             { pol.accumulate(acc, toCompute(x[mapOffsetAny(xm, i)]), i); pol.checkpoint(acc); }
     }
     acc = blockMerge<Pol>(pol, acc, smem);
-    if (threadIdx.x == 0) partials[blockIdx.x] = acc;
+    if (threadIdx.x == 0) {
+        if (zDirect != nullptr) zDirect[0] = pol.finalize(acc, n);
+        else partials[blockIdx.x] = acc;
+    }
 }
 
 // Stage 2: one block merges the per-block partials.  (Doing this in the first launch, by the block that
@@ -499,8 +503,8 @@ inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, type
     if (grid < 1) grid = 1;
     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
     hipLaunchKernelGGL((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
-                       pl.ews, pl.xm);
-    hipLaunchKernelGGL((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n);
+                       pl.ews, pl.xm, grid == 1 ? z : nullptr);
+    if (grid > 1) hipLaunchKernelGGL((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n);
 }
 
 }  // namespace nd4j_amd
