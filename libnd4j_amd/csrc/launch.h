@@ -65,6 +65,11 @@ struct TadPlan {
 struct Workspace {
     void *ptr;
     size_t bytes;
+    // Optional completion signal of a scalar-result launch: the thread that stores the result then stores `ticket`
+    // into `*signal` (host memory the device can write), behind a system-scope fence, so that the host may wait for
+    // the value itself instead of for the stream.  Null for array results.
+    unsigned *signal = nullptr;
+    unsigned ticket = 0;
 };
 
 // Full-array view for scalar reductions: either 1-D strided (ews >= 1) or a C-order coordinate map.

@@ -32,6 +32,12 @@ Scratch scratchFor(hipStream_t s, size_t wantRest = 0) {
     return sc;
 }
 
+Workspace withSignal(Workspace w, const ScalarSignal &sig) {
+    w.signal = sig.flag;
+    w.ticket = sig.ticket;
+    return w;
+}
+
 void cLinearMap(const Long *info, DimMap &out) { ownCanon(siRank(info), siShape(info), siStride(info), out); }
 
 // Order-independent full-array walk: 1-D strided when the EWS field says so, otherwise the view with its
@@ -97,24 +103,26 @@ template <> struct ScalarOut<float> { typedef float R; static R get(float v) { r
 template <> struct ScalarOut<double> { typedef double R; static R get(double v) { return v; } };
 template <> struct ScalarOut<float16> { typedef float R; static R get(float16 v) { return halfBitsToFloatHost(v.x); } };
 
-template <typename T> typename ScalarOut<T>::R readScalar(const void *pinnedSlot, hipStream_t s, const char *what) {
-    syncAndCheck(what, s);
+template <typename T>
+typename ScalarOut<T>::R readScalar(const void *pinnedSlot, hipStream_t s, const char *what, const ScalarSignal &sig) {
+    waitForScalar(sig, s, what);
     T v;
     std::memcpy(&v, pinnedSlot, sizeof(T));
     return ScalarOut<T>::get(v);
 }
 
 // ---- reduce -----------------------------------------------------------------------------------------
-template <typename T> bool reduceScalarTo(hipStream_t s, int opNum, const T *x, const Long *hx, const T *extra, T *zDev) {
+template <typename T>
+bool reduceScalarTo(hipStream_t s, int opNum, const T *x, const Long *hx, const T *extra, T *zDev, const ScalarSignal &sig = ScalarSignal()) {
     Scratch sc = scratchFor(s);
     FlatPlan pl = flatAnyOrder(hx);
     if (opNum == 19) {
         // LogSumExp: maximum first, then exp(x - max) summed (NativeOpExcutioner.cpp:138-141)
         T *maxSlot = reinterpret_cast<T *>(reinterpret_cast<char *>(sc.scalars) + 64);
         if (!launchReduceScalar<T>(s, 3, x, extra, maxSlot, pl, sc.rest)) return false;
-        return launchReduceScalar<T>(s, 19, x, maxSlot, zDev, pl, sc.rest);
+        return launchReduceScalar<T>(s, 19, x, maxSlot, zDev, pl, withSignal(sc.rest, sig));
     }
-    return launchReduceScalar<T>(s, opNum, x, extra, zDev, pl, sc.rest);
+    return launchReduceScalar<T>(s, opNum, x, extra, zDev, pl, withSignal(sc.rest, sig));
 }
 
 template <typename T> typename ScalarOut<T>::R reduceScalar(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params) {
@@ -124,8 +132,9 @@ template <typename T> typename ScalarOut<T>::R reduceScalar(Nd4jPointer *extra, 
     if (hx == nullptr) return 0;
     Scratch sc = scratchFor(s);
     T *slot = reinterpret_cast<T *>(pinnedScalarFor(s));
-    if (!reduceScalarTo<T>(s, opNum, x, hx, params, slot)) { reportUnknownOp("reduce", opNum); return 0; }
-    return readScalar<T>(slot, s, "execReduceScalar");
+    const ScalarSignal sig = nextScalarSignal(s);
+    if (!reduceScalarTo<T>(s, opNum, x, hx, params, slot, sig)) { reportUnknownOp("reduce", opNum); return 0; }
+    return readScalar<T>(slot, s, "execReduceScalar", sig);
 }
 
 template <typename T> void reduceFull(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *z) {
@@ -166,10 +175,11 @@ void reduceDims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *
 }
 
 // ---- index reduce -----------------------------------------------------------------------------------
-template <typename T> bool indexScalarTo(hipStream_t s, int opNum, const T *x, const Long *hx, const T *extra, T *zDev) {
+template <typename T>
+bool indexScalarTo(hipStream_t s, int opNum, const T *x, const Long *hx, const T *extra, T *zDev, const ScalarSignal &sig = ScalarSignal()) {
     Scratch sc = scratchFor(s);
     FlatPlan pl = flatIndexed(hx);
-    return launchIndexReduceScalar<T>(s, opNum, x, extra, zDev, pl, sc.rest);
+    return launchIndexReduceScalar<T>(s, opNum, x, extra, zDev, pl, withSignal(sc.rest, sig));
 }
 
 template <typename T> typename ScalarOut<T>::R indexReduceScalar(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params) {
@@ -179,8 +189,9 @@ template <typename T> typename ScalarOut<T>::R indexReduceScalar(Nd4jPointer *ex
     if (hx == nullptr) return 0;
     Scratch sc = scratchFor(s);
     T *slot = reinterpret_cast<T *>(pinnedScalarFor(s));
-    if (!indexScalarTo<T>(s, opNum, x, hx, params, slot)) { reportUnknownOp("indexreduce", opNum); return 0; }
-    return readScalar<T>(slot, s, "execIndexReduceScalar");
+    const ScalarSignal sig = nextScalarSignal(s);
+    if (!indexScalarTo<T>(s, opNum, x, hx, params, slot, sig)) { reportUnknownOp("indexreduce", opNum); return 0; }
+    return readScalar<T>(slot, s, "execIndexReduceScalar", sig);
 }
 
 template <typename T>
@@ -210,12 +221,13 @@ void indexReduceDims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params
 }
 
 // ---- summary stats ----------------------------------------------------------------------------------
-template <typename T> bool statsScalarTo(hipStream_t s, int opNum, bool bias, const T *x, const Long *hx, T *zDev) {
+template <typename T>
+bool statsScalarTo(hipStream_t s, int opNum, bool bias, const T *x, const Long *hx, T *zDev, const ScalarSignal &sig = ScalarSignal()) {
     Scratch sc = scratchFor(s);
     FlatPlan pl = flatAnyOrder(hx);
     // the reference walks EWS == 1 arrays linearly and everything else by C-order coordinates
     // (cpu/summarystatsreduce.cpp:31-62); the moments do not depend on the visiting order
-    return launchSummaryStatsScalar<T>(s, opNum, bias, x, zDev, pl, sc.rest);
+    return launchSummaryStatsScalar<T>(s, opNum, bias, x, zDev, pl, withSignal(sc.rest, sig));
 }
 
 template <typename T>
@@ -226,8 +238,9 @@ typename ScalarOut<T>::R statsScalar(Nd4jPointer *extra, int opNum, T *x, Long *
     if (hx == nullptr) return 0;
     Scratch sc = scratchFor(s);
     T *slot = reinterpret_cast<T *>(pinnedScalarFor(s));
-    if (!statsScalarTo<T>(s, opNum, bias, x, hx, slot)) { reportUnknownOp("summarystats", opNum); return 0; }
-    return readScalar<T>(slot, s, "execSummaryStatsScalar");
+    const ScalarSignal sig = nextScalarSignal(s);
+    if (!statsScalarTo<T>(s, opNum, bias, x, hx, slot, sig)) { reportUnknownOp("summarystats", opNum); return 0; }
+    return readScalar<T>(slot, s, "execSummaryStatsScalar", sig);
 }
 
 template <typename T> void statsFull(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, bool bias) {
@@ -313,7 +326,8 @@ void reduce3WholePlan(const Long *hx, const Long *hy, Reduce3Launch &in) {
 }
 
 template <typename T>
-bool reduce3WholeTo(Nd4jPointer *extra, hipStream_t s, int opNum, T *x, Long *xInfo, T *params, T *y, Long *yInfo, T *zDev) {
+bool reduce3WholeTo(Nd4jPointer *extra, hipStream_t s, int opNum, T *x, Long *xInfo, T *params, T *y, Long *yInfo, T *zDev,
+                    const ScalarSignal &sig = ScalarSignal()) {
     std::vector<Long> sx, sy;
     const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
     const Long *hy = hostShapeInfo(extra, X_HOST_Y_SHAPE, yInfo, sy, s);
@@ -321,7 +335,7 @@ bool reduce3WholeTo(Nd4jPointer *extra, hipStream_t s, int opNum, T *x, Long *xI
     Reduce3Launch in;
     reduce3WholePlan(hx, hy, in);
     Scratch sc = scratchFor(s);
-    if (!launchReduce3<T>(s, opNum, x, y, zDev, params, in, sc.rest)) { reportUnknownOp("reduce3", opNum); return false; }
+    if (!launchReduce3<T>(s, opNum, x, y, zDev, params, in, withSignal(sc.rest, sig))) { reportUnknownOp("reduce3", opNum); return false; }
     return true;
 }
 
@@ -329,8 +343,9 @@ template <typename T>
 typename ScalarOut<T>::R reduce3Scalar(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *y, Long *yInfo) {
     hipStream_t s = streamOf(extra);
     T *slot = reinterpret_cast<T *>(pinnedScalarFor(s));
-    if (!reduce3WholeTo<T>(extra, s, opNum, x, xInfo, params, y, yInfo, slot)) return 0;
-    return readScalar<T>(slot, s, "execReduce3Scalar");
+    const ScalarSignal sig = nextScalarSignal(s);
+    if (!reduce3WholeTo<T>(extra, s, opNum, x, xInfo, params, y, yInfo, slot, sig)) return 0;
+    return readScalar<T>(slot, s, "execReduce3Scalar", sig);
 }
 
 template <typename T>

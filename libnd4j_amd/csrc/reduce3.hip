@@ -74,7 +74,8 @@ struct Reduce3Plan {
 // of the single run and the block's triple goes to partials[blockIdx.x].
 template <typename T, int OP, int GROUP>
 __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, T *z, const T *extra, Reduce3Plan pl,
-                                                        Acc3<typename Compute<T>::type> *partials, Long sliceLength) {
+                                                        Acc3<typename Compute<T>::type> *partials, Long sliceLength,
+                                                        unsigned *signal, unsigned ticket) {
     typedef typename Compute<T>::type C;
     typedef Acc3<C> Acc;
     constexpr int GROUPS = kBlock / GROUP;
@@ -141,15 +142,19 @@ __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, 
             if (live) acc = waveMerge<Acc3Merge<C>, GROUP>(mg, acc);
         }
         if (live && lane == 0) {
-            if (sliced) partials[u] = acc;
-            else z[u] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, pl.runLength));
+            if (sliced) {
+                partials[u] = acc;
+            } else {
+                z[u] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, pl.runLength));
+                signalResult(signal, ticket);  // set only for a launch with a single result
+            }
         }
     }
 }
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlock) reduce3Finish(T *z, const Acc3<typename Compute<T>::type> *partials, int count,
-                                                        Long runLength) {
+                                                        Long runLength, unsigned *signal, unsigned ticket) {
     typedef typename Compute<T>::type C;
     typedef Acc3<C> Acc;
     __shared__ Acc smem[kBlock / kWave];
@@ -158,7 +163,10 @@ __global__ void __launch_bounds__(kBlock) reduce3Finish(T *z, const Acc3<typenam
     for (int i = threadIdx.x; i < count; i += kBlock) acc = add3(acc, partials[i]);
     Acc3Merge<C> mg;
     acc = blockMerge<Acc3Merge<C>>(mg, acc, smem);
-    if (threadIdx.x == 0) z[0] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, runLength));
+    if (threadIdx.x == 0) {
+        z[0] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, runLength));
+        signalResult(signal, ticket);
+    }
 }
 
 template <typename T> struct Reduce3Body {
@@ -179,21 +187,24 @@ template <typename T> struct Reduce3Body {
                 if (slices >= 2) {  // a single slice needs no second launch: the per-result kernels below do it in one
                     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
                     hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)slices), dim3(kBlock), 0, s, x, y, z, extra, pl,
-                                       partials, sliceLength);
-                    hipLaunchKernelGGL((reduce3Finish<T, OP>), dim3(1), dim3(kBlock), 0, s, z, partials, (int)slices, pl.runLength);
+                                       partials, sliceLength, (unsigned *)nullptr, 0u);
+                    hipLaunchKernelGGL((reduce3Finish<T, OP>), dim3(1), dim3(kBlock), 0, s, z, partials, (int)slices, pl.runLength,
+                                       ws.signal, ws.ticket);
                     return true;
                 }
             }
             Acc *none = nullptr;
+            unsigned *signal = pl.numOut == 1 ? ws.signal : nullptr;
+            const unsigned ticket = ws.ticket;
             if (pl.runLength >= 4096) {
                 int grid = gridFor(pl.numOut, 1, kGridCap);
-                hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0);
+                hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, signal, ticket);
             } else if (pl.runLength >= 128) {
                 int grid = gridFor(pl.numOut, kBlock / 64, kGridCap);
-                hipLaunchKernelGGL((reduce3Kernel<T, OP, 64>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0);
+                hipLaunchKernelGGL((reduce3Kernel<T, OP, 64>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, signal, ticket);
             } else {
                 int grid = gridFor(pl.numOut, kBlock / 16, kGridCap);
-                hipLaunchKernelGGL((reduce3Kernel<T, OP, 16>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0);
+                hipLaunchKernelGGL((reduce3Kernel<T, OP, 16>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, signal, ticket);
             }
             return true;
         }

@@ -331,11 +331,19 @@ __global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typena
     }
 }
 
+// After a scalar result has been stored by this thread: make it visible to the host, then raise the caller's ticket.
+__device__ __forceinline__ void signalResult(unsigned *signal, unsigned ticket) {
+    if (signal == nullptr) return;
+    __threadfence_system();
+    __hip_atomic_store(signal, ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // Stage 1 of the full-array reduction: block b folds the chunks b, b+grid, ... of kBlock*kUnroll vectors.
 // A one-block launch (small arrays) is handed the result pointer and finishes by itself.
 template <class Pol>
 __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol::T *x, typename Pol::Acc *partials,
-                                                     Long n, int strided, Long ews, DimMap xm, typename Pol::T *zDirect) {
+                                                     Long n, int strided, Long ews, DimMap xm, typename Pol::T *zDirect,
+                                                     unsigned *signal, unsigned ticket) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
@@ -380,8 +388,12 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
     }
     acc = blockMerge<Pol>(pol, acc, smem);
     if (threadIdx.x == 0) {
-        if (zDirect != nullptr) zDirect[0] = pol.finalize(acc, n);
-        else partials[blockIdx.x] = acc;
+        if (zDirect != nullptr) {
+            zDirect[0] = pol.finalize(acc, n);
+            signalResult(signal, ticket);
+        } else {
+            partials[blockIdx.x] = acc;
+        }
     }
 }
 
@@ -390,7 +402,8 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
 // the streaming kernel more than twice its run time, a second launch costs a few microseconds.)
 template <class Pol>
 __global__ void __launch_bounds__(kBlock) flatFinish(Pol pol, const typename Pol::T *x, typename Pol::T *z,
-                                                     const typename Pol::Acc *partials, int count, Long n) {
+                                                     const typename Pol::Acc *partials, int count, Long n, unsigned *signal,
+                                                     unsigned ticket) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::Acc Acc;
     __shared__ Acc smem[kBlock / kWave];
@@ -398,7 +411,10 @@ __global__ void __launch_bounds__(kBlock) flatFinish(Pol pol, const typename Pol
     Acc acc = pol.init(x);
     for (int i = threadIdx.x; i < count; i += kBlock) acc = pol.combine(acc, partials[i]);
     acc = blockMerge<Pol>(pol, acc, smem);
-    if (threadIdx.x == 0) z[0] = pol.finalize(acc, n);
+    if (threadIdx.x == 0) {
+        z[0] = pol.finalize(acc, n);
+        signalResult(signal, ticket);
+    }
 }
 
 // ---- host launch logic shared by the three families ---------------------------------------------------
@@ -503,8 +519,9 @@ inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, type
     if (grid < 1) grid = 1;
     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
     hipLaunchKernelGGL((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
-                       pl.ews, pl.xm, grid == 1 ? z : nullptr);
-    if (grid > 1) hipLaunchKernelGGL((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n);
+                       pl.ews, pl.xm, grid == 1 ? z : nullptr, ws.signal, ws.ticket);
+    if (grid > 1)
+        hipLaunchKernelGGL((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n, ws.signal, ws.ticket);
 }
 
 }  // namespace nd4j_amd

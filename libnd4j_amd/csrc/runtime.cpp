@@ -1,5 +1,6 @@
 #include "runtime.h"
 
+#include <chrono>
 #include <cstring>
 
 #include <map>
@@ -138,18 +139,70 @@ Workspace workspaceFor(hipStream_t s, size_t minBytes) {
     return w;
 }
 
-void *pinnedScalarFor(hipStream_t s) {
-    static std::map<std::pair<int, hipStream_t>, void *> slots;
+namespace {
+struct PinnedSlot {
+    void *block = nullptr;  // 256 bytes: value at 0, flag word at 128
+    unsigned ticket = 0;
+};
+PinnedSlot &pinnedSlotLocked(hipStream_t s) {
+    static std::map<std::pair<int, hipStream_t>, PinnedSlot> slots;
     int dev = 0;
     (void)hipGetDevice(&dev);
-    std::lock_guard<std::mutex> lock(gMutex);
-    void *&p = slots[std::make_pair(dev, s)];
-    if (p == nullptr) {
-        hipError_t e = hipHostMalloc(&p, 256, hipHostMallocDefault);
-        if (e != hipSuccess) { p = nullptr; throwHip("pinned scalar slot", e); }
-        std::memset(p, 0, 256);
+    PinnedSlot &p = slots[std::make_pair(dev, s)];
+    if (p.block == nullptr) {
+        // coherent: the device's stores reach host memory while the kernel runs, not only when it has ended
+        hipError_t e = hipHostMalloc(&p.block, 256, hipHostMallocCoherent);
+        if (e != hipSuccess) { p.block = nullptr; throwHip("pinned scalar slot", e); }
+        std::memset(p.block, 0, 256);
     }
     return p;
+}
+}  // namespace
+
+void *pinnedScalarFor(hipStream_t s) {
+    std::lock_guard<std::mutex> lock(gMutex);
+    return pinnedSlotLocked(s).block;
+}
+
+ScalarSignal nextScalarSignal(hipStream_t s) {
+    std::lock_guard<std::mutex> lock(gMutex);
+    PinnedSlot &p = pinnedSlotLocked(s);
+    ScalarSignal sig;
+    sig.flag = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(p.block) + 128);
+    sig.ticket = ++p.ticket;
+    if (sig.ticket == 0) sig.ticket = ++p.ticket;  // zero is what a fresh slot holds
+    return sig;
+}
+
+void waitForScalar(const ScalarSignal &sig, hipStream_t s, const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) throwHip(what, e);
+    if (sig.flag == nullptr || environment().debug.load()) {
+        e = hipStreamSynchronize(s);
+        if (e != hipSuccess) throwHip(what, e);
+        return;
+    }
+    const volatile unsigned *flag = sig.flag;
+    // Spin on the flag alone at first (asking the runtime about the stream costs microseconds and delays the answer);
+    // a launch that failed or wrote nothing never raises the flag, so from 50 us on the stream is asked as well.
+    const auto start = std::chrono::steady_clock::now();
+    auto nextQuery = start + std::chrono::microseconds(50);
+    for (unsigned spins = 1; *flag != sig.ticket; spins++) {
+        if ((spins & 0xff) != 0) continue;
+        const auto now = std::chrono::steady_clock::now();
+        if (now < nextQuery) continue;
+        if (now - start > std::chrono::microseconds(300)) {
+            // a long kernel: wait the runtime's way (which may yield the core) rather than spin on
+            e = hipStreamSynchronize(s);
+            if (e != hipSuccess) throwHip(what, e);
+            break;
+        }
+        e = hipStreamQuery(s);
+        if (e == hipSuccess) break;
+        if (e != hipErrorNotReady) throwHip(what, e);
+        nextQuery = now + std::chrono::microseconds(20);
+    }
+    std::atomic_thread_fence(std::memory_order_acquire);
 }
 
 bool resolveTad(Nd4jPointer *extra, int hostSlot, int offsetSlot, const Long *hostXInfo, const int *dimension,

@@ -77,6 +77,17 @@ Workspace workspaceFor(hipStream_t s, size_t minBytes);
 // 256 bytes of pinned, device-visible host memory per (device, stream): the kernels of the scalar-returning
 // entry points write their result there, so the host reads it after the stream synchronisation without a copy.
 void *pinnedScalarFor(hipStream_t s);
+// The completion signal that goes with that slot: a flag word in the same pinned block and the next ticket of this
+// (device, stream).  waitForScalar returns once the flag shows the ticket (the kernel stores it after the value,
+// behind a system-scope fence) or the stream has drained, whichever the host sees first, and throws on a HIP error:
+// the host gets the value a few microseconds before the stream's own completion would reach it.  In debug mode it
+// synchronises the stream instead.
+struct ScalarSignal {
+    unsigned *flag = nullptr;
+    unsigned ticket = 0;
+};
+ScalarSignal nextScalarSignal(hipStream_t s);
+void waitForScalar(const ScalarSignal &sig, hipStream_t s, const char *what);
 
 // TAD tables resolved for a call: host shapeInfo of one TAD + device offsets.
 struct ResolvedTad {
