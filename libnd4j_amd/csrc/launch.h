@@ -112,6 +112,7 @@ struct Reduce3Launch {
     const Long *xOffsets;  // device
     const Long *yOffsets;  // device
     DimMap xm, ym;         // rank >= 1
+    bool allPairs = false; // every run of x against every run of y (xDiv == yMod == runs of y): may be tiled
 };
 template <typename T>
 bool launchReduce3(hipStream_t stream, int opNum, const T *x, const T *y, T *z, const T *extra, const Reduce3Launch &in,

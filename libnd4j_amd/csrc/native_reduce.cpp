@@ -439,8 +439,11 @@ void reduce3All(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *
     const Long *hy = hostShapeInfo(extra, X_HOST_Y_SHAPE, yInfo, sy, s);
     if (hx == nullptr || hy == nullptr) return;
     ResolvedTad tx, ty;
-    if (!resolveTad(nullptr, 0, 0, hx, dimension, dimLen, tx, s)) return;
-    if (!resolveTad(nullptr, 0, 0, hy, dimension, dimLen, ty, s)) return;
+    // the dimensions are a device array: one read-back serves both operands
+    std::vector<int> dims;
+    if (!hostInts(dimension, dimLen, dims, s)) return;
+    if (!resolveTad(nullptr, 0, 0, hx, dims.data(), dimLen, tx, s)) return;
+    if (!resolveTad(nullptr, 0, 0, hy, dims.data(), dimLen, ty, s)) return;
     if (tx.tadLength != ty.tadLength) {
         std::printf("reduce3All: TAD lengths differ (%lld vs %lld)\n", (long long)tx.tadLength, (long long)ty.tadLength);
         return;
@@ -452,6 +455,7 @@ void reduce3All(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *
     in.yMod = in.xDiv;
     in.xOffsets = tx.devOffsets;
     in.yOffsets = ty.devOffsets;
+    in.allPairs = true;
     orderedLinearMap(siShape(tx.hostInfo), siStride(tx.hostInfo), siRank(tx.hostInfo), siOrder(tx.hostInfo) == 'f' ? 'f' : 'c', in.xm);
     orderedLinearMap(siShape(ty.hostInfo), siStride(ty.hostInfo), siRank(ty.hostInfo), siOrder(ty.hostInfo) == 'f' ? 'f' : 'c', in.ym);
     Scratch sc = scratchFor(s);

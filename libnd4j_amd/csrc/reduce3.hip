@@ -68,6 +68,7 @@ struct Reduce3Plan {
     const Long *yOffsets;  // device; null: 0
     DimMap xm, ym;         // pair index inside a run -> element offset
     bool contiguous;       // both maps are unit-stride
+    bool allPairs;         // every run of x against every run of y: xDiv == yMod == number of runs of y
 };
 
 // GROUP lanes per output (16, 64 or the whole block).  `slices` > 1 (whole-array calls): blockIdx.x is the slice
@@ -169,11 +170,143 @@ __global__ void __launch_bounds__(kBlock) reduce3Finish(T *z, const Acc3<typenam
     }
 }
 
+// Every run of x against every run of y (execReduce3All), contiguous runs: a block computes a 64 x 64 tile of
+// results.  The naive pairing reads both runs from the caches for every result (nx * ny * 2 * length elements: it
+// ran at the L2's 9-15 TB/s and no faster); here a block stages 32 elements of its 64 + 64 runs in LDS per step and
+// every staged element serves 64 results, a thread keeping a 4 x 4 patch of accumulator triples in registers.
+// Each result still sums its pairs in run order, one after the other, as the reference's loop does.
+static constexpr int kTileK = 32;    // elements of each run staged per step
+static constexpr int kTilePad = 4;   // keeps the LDS rows 16-byte aligned and spreads them over the banks
+
+// PER elements of one run, staged by one thread per step
+template <typename T, int PER> struct TileStage {
+    typedef typename Compute<T>::type C;
+    C v[PER];
+    // elements k .. k + PER - 1 of the run at `run` (null: a row beyond the last run), those beyond `length` as zero
+    __device__ __forceinline__ void load(const T *run, Long k, Long length) {
+        constexpr int N = Pack<T>::N, NP = PER / N > 0 ? PER / N : 1;
+        if (run == nullptr || k >= length) {
+#pragma unroll
+            for (int e = 0; e < PER; e++) v[e] = (C)0;
+            return;
+        }
+        if (PER % N == 0 && k + PER <= length && (reinterpret_cast<uintptr_t>(run + k) & 15) == 0) {
+            const Pack<T> *pv = reinterpret_cast<const Pack<T> *>(run + k);
+#pragma unroll
+            for (int q = 0; q < NP; q++) {
+                const Pack<T> pk = pv[q];
+#pragma unroll
+                for (int e = 0; e < N; e++) v[q * N + e] = toCompute(pk.v[e]);
+            }
+            return;
+        }
+#pragma unroll
+        for (int e = 0; e < PER; e++) v[e] = k + e < length ? toCompute(run[k + e]) : (C)0;
+    }
+};
+
+// TR runs of x and of y per block (64, or 32 when 64 would leave most of the chip without a tile); a thread owns a
+// TR/16 x TR/16 patch of results.
+template <typename T, int OP, int TR>
+__global__ void __launch_bounds__(kBlock) reduce3AllTileKernel(const T *x, const T *y, T *z, const T *extra, const Long *xOffsets,
+                                                               const Long *yOffsets, Long nx, Long ny, Long length) {
+    typedef typename Compute<T>::type C;
+    typedef Acc3<C> Acc;
+    constexpr int ROW = kTileK + kTilePad;
+    constexpr int P = TR / 16;                   // patch edge
+    constexpr int PER = TR * kTileK / kBlock;    // staged elements per thread, run and step
+    constexpr int LANES_K = kTileK / PER;        // threads along a staged row
+    __shared__ __attribute__((aligned(16))) C xs[TR][ROW];
+    __shared__ __attribute__((aligned(16))) C ys[TR][ROW];
+    const C eps = extra != nullptr ? toCompute(extra[0]) : (C)0;
+    const Long tilesY = (ny + TR - 1) / TR;
+    const Long tileX = blockIdx.x / tilesY, tileY = blockIdx.x - tileX * tilesY;
+    const Long row0 = tileX * TR, col0 = tileY * TR;
+    // staging role: one run of x and one of y, PER elements of each per step
+    const int sRun = threadIdx.x / LANES_K, sK = (threadIdx.x % LANES_K) * PER;
+    const T *xRun = row0 + sRun < nx ? x + xOffsets[row0 + sRun] : nullptr;
+    const T *yRun = col0 + sRun < ny ? y + yOffsets[col0 + sRun] : nullptr;
+    // computing role: results (row0 + P ti + a, col0 + P tj + b)
+    const int ti = threadIdx.x / 16, tj = threadIdx.x % 16;
+    Acc acc[P][P];
+#pragma unroll
+    for (int a = 0; a < P; a++)
+#pragma unroll
+        for (int b = 0; b < P; b++) acc[a][b].r = acc[a][b].e0 = acc[a][b].e1 = (C)0;
+
+    TileStage<T, PER> sx, sy;
+    sx.load(xRun, sK, length);
+    sy.load(yRun, sK, length);
+    for (Long k0 = 0; k0 < length; k0 += kTileK) {
+#pragma unroll
+        for (int e = 0; e < PER; e++) {
+            xs[sRun][sK + e] = sx.v[e];
+            ys[sRun][sK + e] = sy.v[e];
+        }
+        __syncthreads();
+        if (k0 + kTileK < length) {  // the next step's elements travel while this step is computed
+            sx.load(xRun, k0 + kTileK + sK, length);
+            sy.load(yRun, k0 + kTileK + sK, length);
+        }
+        const int kmax = length - k0 < kTileK ? (int)(length - k0) : kTileK;
+        int kk = 0;
+        for (; kk + 4 <= kmax; kk += 4) {
+            C xa[P][4], yb[P][4];
+#pragma unroll
+            for (int a = 0; a < P; a++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    xa[a][q] = xs[P * ti + a][kk + q];
+                    yb[a][q] = ys[P * tj + a][kk + q];
+                }
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+#pragma unroll
+                for (int a = 0; a < P; a++)
+#pragma unroll
+                    for (int b = 0; b < P; b++) Reduce3Op<C, OP>::accumulate(acc[a][b], xa[a][q], yb[b][q], eps);
+        }
+        for (; kk < kmax; kk++) {
+#pragma unroll
+            for (int a = 0; a < P; a++)
+#pragma unroll
+                for (int b = 0; b < P; b++) Reduce3Op<C, OP>::accumulate(acc[a][b], xs[P * ti + a][kk], ys[P * tj + b][kk], eps);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int a = 0; a < P; a++) {
+        const Long r = row0 + P * ti + a;
+        if (r >= nx) continue;
+#pragma unroll
+        for (int b = 0; b < P; b++) {
+            const Long g = col0 + P * tj + b;
+            if (g < ny) z[r * ny + g] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc[a][b], length));
+        }
+    }
+}
+
 template <typename T> struct Reduce3Body {
     template <int OP> struct Run {
         static bool run(hipStream_t s, const T *x, const T *y, T *z, const T *extra, const Reduce3Plan &pl, Workspace ws) {
             typedef Acc3<typename Compute<T>::type> Acc;
             if (pl.numOut <= 0) return true;
+            // all pairs of contiguous runs, enough of them to fill tiles
+            if (pl.allPairs && pl.contiguous && pl.xOffsets != nullptr && pl.yOffsets != nullptr && pl.yMod >= 16 &&
+                pl.numOut / pl.yMod >= 16 && pl.runLength >= 8) {
+                const Long nx = pl.numOut / pl.yMod, ny = pl.yMod;
+                const Long tiles64 = ((nx + 63) / 64) * ((ny + 63) / 64), tiles32 = ((nx + 31) / 32) * ((ny + 31) / 32);
+                if (tiles64 >= 512 && tiles64 <= kMaxGrid) {
+                    hipLaunchKernelGGL((reduce3AllTileKernel<T, OP, 64>), dim3((unsigned)tiles64), dim3(kBlock), 0, s, x, y, z, extra,
+                                       pl.xOffsets, pl.yOffsets, nx, ny, pl.runLength);
+                    return true;
+                }
+                if (tiles32 <= kMaxGrid) {
+                    hipLaunchKernelGGL((reduce3AllTileKernel<T, OP, 32>), dim3((unsigned)tiles32), dim3(kBlock), 0, s, x, y, z, extra,
+                                       pl.xOffsets, pl.yOffsets, nx, ny, pl.runLength);
+                    return true;
+                }
+            }
             if (pl.numOut == 1 && pl.runLength >= 4 * kBlock) {
                 Long perBlock = (Long)kBlock * 8 * Pack<T>::N;
                 Long slices = (pl.runLength + perBlock - 1) / perBlock;
@@ -223,6 +356,7 @@ bool launchReduce3(hipStream_t s, int opNum, const T *x, const T *y, T *z, const
     pl.yOffsets = in.yOffsets;
     pl.xm = in.xm;
     pl.ym = in.ym;
+    pl.allPairs = in.allPairs;
     pl.contiguous = in.xm.rank <= 1 && in.ym.rank <= 1 && (in.xm.rank == 0 || in.xm.stride[0] == 1) &&
                     (in.ym.rank == 0 || in.ym.stride[0] == 1);
     return dispatchSeq<Reduce3Body<T>::template Run>(opNum, std::make_integer_sequence<int, 8>{}, s, x, y, z, extra, pl, ws);

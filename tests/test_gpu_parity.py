@@ -335,6 +335,36 @@ def test_reduce3_family(gpu, cpu):
     x, y = rs.uniform(0.1, 2, 7 * 190).astype(np.float32), rs.uniform(0.1, 2, 4 * 190).astype(np.float32)
     for op in (0, 1, 2, 3, 5, 6, 7):
         close(gpu.reduce3_all(op, x, xi, y, yi, None, [1], 28), cpu.reduce3_all(op, x, xi, y, yi, None, [1], 28), ("all", op))
+    # enough pairs for the tiled kernel: ragged tile edges, a run length that ends inside a staged step, misaligned runs
+    # (the last shape has enough 64 x 64 tiles for the larger tile; the others run 32 x 32 ones)
+    for (nx, ny, length) in ((70, 33, 100), (64, 128, 256), (17, 16, 9), (130, 65, 1027), (1450, 1420, 43)):
+        xi, yi = shape_info_np([nx, length]), shape_info_np([ny, length])
+        x, y = rs.uniform(0.1, 2, nx * length).astype(np.float32), rs.uniform(0.1, 2, ny * length).astype(np.float32)
+        x64, y64 = x.astype(np.float64).reshape(nx, length), y.astype(np.float64).reshape(ny, length)
+        for op in (0, 1, 2, 3, 5, 6, 7):
+            got = gpu.reduce3_all(op, x, xi, y, yi, None, [1], nx * ny)
+            close(got, cpu.reduce3_all(op, x, xi, y, yi, None, [1], nx * ny), ("tiled all", nx, ny, length, op))
+        dots = x64 @ y64.T
+        assert np.allclose(gpu.reduce3_all(3, x, xi, y, yi, None, [1], nx * ny).reshape(nx, ny), dots, rtol=1e-5)
+        if nx * ny > 100000:
+            xd, yd = rs.randn(nx * length), rs.randn(ny * length)
+            assert np.allclose(gpu.reduce3_all(1, xd, xi, yd, yi, None, [1], nx * ny).reshape(nx, ny),
+                               np.sqrt(((xd.reshape(nx, 1, length) - yd.reshape(1, ny, length)) ** 2).sum(axis=2)), rtol=1e-12)
+            continue
+        # EqualsWithEps counts the pairs that differ: elements staged beyond the end of a run must not be counted
+        y2 = x[:ny * length].copy() if nx >= ny else np.resize(x, ny * length)
+        y2[::7] += 1.0
+        xa, yb = x.reshape(nx, 1, length), y2.reshape(1, ny, length)
+        diff, eps = np.abs(xa - yb), np.float32(1e-5)  # the op's rule (ops.h EqualsWithEps), in float as the op applies it
+        want = ((diff > eps) & (diff > np.maximum(np.abs(xa), np.abs(yb)) * eps)).sum(axis=2)
+        got = gpu.reduce3_all(4, x, xi, y2, yi, np.array([1e-5, 0, 0], np.float32), [1], nx * ny).reshape(nx, ny)
+        assert np.array_equal(got, want.astype(np.float32)), ("equals", nx, ny, length)
+        xd, yd = rs.randn(nx * length), rs.randn(ny * length)
+        assert np.allclose(gpu.reduce3_all(3, xd, xi, yd, yi, None, [1], nx * ny).reshape(nx, ny),
+                           xd.reshape(nx, length) @ yd.reshape(ny, length).T, rtol=1e-12, atol=1e-12)
+        xh, yh = x.astype(np.float16), y.astype(np.float16)
+        hd = xh.astype(np.float64).reshape(nx, length) @ yh.astype(np.float64).reshape(ny, length).T
+        assert np.allclose(gpu.reduce3_all(3, xh, xi, yh, yi, None, [1], nx * ny).astype(np.float64).reshape(nx, ny), hd, rtol=1e-2)
     # float64 ground truth at a size the sliced kernel splits
     n = 1 << 20
     x = rs.randn(n).astype(np.float32)
