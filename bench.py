@@ -242,11 +242,14 @@ def main():
                     med, runs = cpu_time(c.cpu, cpu_lib, 1.0, min_runs=2, max_runs=10)
                     row["cpu_ms"] = round(med * 1e3, 3)
                     row["cpu_GB/s"] = round(c.bytes / med / 1e9, 2)
+                if c.note:
+                    row["note"] = c.note
                 fam.append(row)
                 print("%-22s %-12s %9.4f ms %8.1f GB/s %5.1f%%%s%s" % (
                     c.name, c.family, ms, row["GB/s"], 100 * row["frac"],
                     "   cpu %9.2f ms" % row["cpu_ms"] if "cpu_ms" in row else "",
-                    "   (%d read-backs from the device)" % fetched if fetched else ""), file=sys.stderr, flush=True)
+                    "   (%d read-backs from the device)" % fetched if fetched else "") + ("   [%s]" % c.note if c.note else ""),
+                    file=sys.stderr, flush=True)
             wl.free()
         out["families"] = fam
     print(json.dumps(out), flush=True)

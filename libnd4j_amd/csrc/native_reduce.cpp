@@ -432,18 +432,36 @@ void reduce3Dims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T 
 // Every TAD of x against every TAD of y (reduce3.h:918-995): result[r * yTads + g].
 template <typename T>
 void reduce3All(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *y, Long *yInfo, T *z, int *dimension,
-                int dimLen) {
+                int dimLen, const Long *xOffsetsDev, const Long *yOffsetsDev) {
     hipStream_t s = streamOf(extra);
     std::vector<Long> sx, sy;
     const Long *hx = hostShapeInfo(extra, X_HOST_X_SHAPE, xInfo, sx, s);
     const Long *hy = hostShapeInfo(extra, X_HOST_Y_SHAPE, yInfo, sy, s);
     if (hx == nullptr || hy == nullptr) return;
     ResolvedTad tx, ty;
-    // the dimensions are a device array: one read-back serves both operands
-    std::vector<int> dims;
-    if (!hostInts(dimension, dimLen, dims, s)) return;
-    if (!resolveTad(nullptr, 0, 0, hx, dims.data(), dimLen, tx, s)) return;
-    if (!resolveTad(nullptr, 0, 0, hy, dims.data(), dimLen, ty, s)) return;
+    // What nd4j passes (blas/cuda/NativeOps.cu, execReduce3AllFloat): the device offset tables of both operands as
+    // arguments and the host shapeInfo of x's TAD in extraPointers[9].  That describes y's TADs too when y is laid
+    // out like x in every dimension but the first (the usual case: two batches of equally shaped rows); then nothing
+    // has to be read back.  Otherwise the dimensions are fetched once and serve both operands.
+    const Long *hostTad = reinterpret_cast<const Long *>(slotOf(extra, X_HOST_TAD_SHAPE));
+    bool sameTads = hostTad != nullptr && xOffsetsDev != nullptr && yOffsetsDev != nullptr && siRank(hx) == siRank(hy) &&
+                    siOrder(hx) == siOrder(hy) && siNumel(hostTad) > 0 && siNumel(hx) % siNumel(hostTad) == 0 &&
+                    siNumel(hy) % siNumel(hostTad) == 0;
+    for (int d = 0; sameTads && d < siRank(hx); d++)
+        sameTads = siStride(hx)[d] == siStride(hy)[d] && (d == 0 || siShape(hx)[d] == siShape(hy)[d]);
+    if (sameTads) {
+        tx.hostInfo = ty.hostInfo = hostTad;
+        tx.tadLength = ty.tadLength = siNumel(hostTad);
+        tx.devOffsets = xOffsetsDev;
+        ty.devOffsets = yOffsetsDev;
+        tx.numTads = siNumel(hx) / tx.tadLength;
+        ty.numTads = siNumel(hy) / ty.tadLength;
+    } else {
+        std::vector<int> dims;
+        if (!hostInts(dimension, dimLen, dims, s)) return;
+        if (!resolveTad(nullptr, 0, 0, hx, dims.data(), dimLen, tx, s)) return;
+        if (!resolveTad(nullptr, 0, 0, hy, dims.data(), dimLen, ty, s)) return;
+    }
     if (tx.tadLength != ty.tadLength) {
         std::printf("reduce3All: TAD lengths differ (%lld vs %lld)\n", (long long)tx.tadLength, (long long)ty.tadLength);
         return;
@@ -610,9 +628,9 @@ INST(double)
                                            Nd4jLong *resultShapeInfoBuffer, int *dimension, int dimensionLength,    \
                                            Nd4jLong *xTadShapeInfo, Nd4jLong *xOffsets, Nd4jLong *yTadShapeInfo,    \
                                            Nd4jLong *yOffsets) {                                                    \
-        (void)resultShapeInfoBuffer; (void)xTadShapeInfo; (void)xOffsets; (void)yTadShapeInfo; (void)yOffsets;      \
+        (void)resultShapeInfoBuffer; (void)xTadShapeInfo; (void)yTadShapeInfo;                                      \
         reduce3All<T>(extraPointers, opNum, x, xInfo, extraParamsVals, y, yInfo, result, dimension,                 \
-                      dimensionLength);                                                                             \
+                      dimensionLength, xOffsets, yOffsets);                                                         \
     }
 
 #define ND4J_REDUCE_MEMBERS(SUFFIX, T, R)                                                                            \

@@ -43,6 +43,7 @@ class Case(object):
         self._result = [result]
         self.cpu = cpu
         self.contiguous = contiguous
+        self.note = None  # printed beside the case by the benchmark
 
     @property
     def sets(self):
@@ -267,6 +268,21 @@ def reduce3_pairs(dev, rows=16384, cols=4096, seed=12, copies=None):
 
         cases.append(Case("dot_full", "reduce3", n, 8 * n + 4, gpu_dot, lambda lib: lib.reduce3_scalar(3, x, xi, y, xi, None), True,
                           lambda: np.array([out["dot"]], F32)))
+        # every row of a [2048,1024] corner of x against every row of the same corner of y: 2048 x 2048 dot products.
+        # Not a streaming case: each operand is read from HBM once and reused from LDS (its "bytes" are the 16 MiB of
+        # operands and the 16 MiB of results), so what bounds it is the vector ALUs; `elements` counts the pairs.
+        ar, al = 2048, 1024
+        ai, azi = harness.shape_info([ar, al]), harness.shape_info([ar, ar])
+        ZA = w.operand(np.zeros(ar * ar, F32), azi)
+        ex_a = dev.extra(ai, ai, azi, tad=dev.tad(ai, [1]))  # host TAD shapeInfo in slot 9, device tables in 10 / 11
+        AI = w.raw(np.ascontiguousarray(ai, dtype=np.int64))
+        za = np.zeros(ar * ar, F32)
+        case = Case("dot_all_pairs", "reduce3", ar * ar * al, 8 * ar * al + 4 * ar * ar,
+                    lambda: ops.execReduce3AllFloat(ex_a, 3, X.ptr, AI.ptr, None, Y.ptr, AI.ptr, ZA.ptr, ZA.info_ptr, D.ptr, 1, ex_a[10],
+                                                    ex_a[11], ex_a[10], ex_a[11]),
+                    lambda lib: (lib.reduce3_all(3, x[:ar * al], ai, y[:ar * al], ai, za, azi, [1], None), za)[1], True, ZA.get)
+        case.note = "compute-bound: %.0f G pairs, fp32 FMA on the vector ALUs" % (ar * ar * al / 1e9)
+        cases.append(case)
         return cases
 
     return _replicated(dev, "reduce3 euclidean/cosine per row + dot; fp32 [%d,%d] c-order" % (rows, cols), 8 * n,

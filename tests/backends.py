@@ -505,14 +505,23 @@ class GpuBackend(object):
         self._finish(X, Y, Z, E, D)
         return out
 
-    def reduce3_all(self, op, x, x_info, y, y_info, extra, dims, out_len):
+    def reduce3_all(self, op, x, x_info, y, y_info, extra, dims, out_len, pass_tads=False):
+        """pass_tads: hand over what nd4j does - x's host TAD shapeInfo in extraPointers[9] and the device TAD tables of
+        both operands as arguments - instead of leaving the library to build them from the (device) dimensions"""
         X, Y = self._op(x, x_info), self._op(y, y_info)
         zi = _vec_info(out_len)
         Z = self._op(np.zeros(out_len, x.dtype), zi)
         E, e = self._up(extra, x.dtype)
         D, d = self._up(np.array(list(dims), np.int32))
-        getattr(self.ops, "execReduce3All" + self._suffix(x))(self.dev.extra(x_info, y_info, zi), op, X.ptr, X.info_ptr, e, Y.ptr,
-                                                               Y.info_ptr, Z.ptr, Z.info_ptr, d, len(dims), None, None, None, None)
+        tables = [None] * 4
+        if pass_tads:
+            ptrs = self.dev.extra(x_info, y_info, zi, tad=self.dev.tad(x_info, dims), tad_z=self.dev.tad(y_info, dims))
+            tables = [ptrs[10], ptrs[11], ptrs[12], ptrs[13]]
+            ptrs[12] = ptrs[13] = None  # the y tables travel as arguments, not in the slots of a result's TADs
+        else:
+            ptrs = self.dev.extra(x_info, y_info, zi)
+        getattr(self.ops, "execReduce3All" + self._suffix(x))(ptrs, op, X.ptr, X.info_ptr, e, Y.ptr, Y.info_ptr, Z.ptr, Z.info_ptr, d,
+                                                               len(dims), *tables)
         out = Z.get()
         self._finish(X, Y, Z, E, D)
         return out

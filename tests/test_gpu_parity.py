@@ -346,6 +346,10 @@ def test_reduce3_family(gpu, cpu):
             close(got, cpu.reduce3_all(op, x, xi, y, yi, None, [1], nx * ny), ("tiled all", nx, ny, length, op))
         dots = x64 @ y64.T
         assert np.allclose(gpu.reduce3_all(3, x, xi, y, yi, None, [1], nx * ny).reshape(nx, ny), dots, rtol=1e-5)
+        # with the caller's TAD tables (nothing is read back from the device then)
+        before = gpu.ops.amd_hostFetchCount()
+        assert np.allclose(gpu.reduce3_all(3, x, xi, y, yi, None, [1], nx * ny, pass_tads=True).reshape(nx, ny), dots, rtol=1e-5)
+        assert gpu.ops.amd_hostFetchCount() == before
         if nx * ny > 100000:
             xd, yd = rs.randn(nx * length), rs.randn(ny * length)
             assert np.allclose(gpu.reduce3_all(1, xd, xi, yd, yi, None, [1], nx * ny).reshape(nx, ny),
