@@ -363,7 +363,7 @@ inline int gridFor(Long work, Long perBlock, int cap) {
 }
 
 static constexpr int kGridCap = 256 * 32;  // 32 blocks of 256 threads per CU
-static constexpr int kMaxGrid = 1 << 30;    // blockIdx.x limit kept well below 2^31
+static constexpr int kMaxGrid = (1 << 24) - 1;  // blocks of 256 threads: a launch may not exceed 2^32 threads in all
 
 // Returns the number of leading scalar elements that brings every pointer to a 16-byte boundary, or -1
 // when the pointers do not share one misalignment.

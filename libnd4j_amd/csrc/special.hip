@@ -350,7 +350,7 @@ template <typename T> SoftmaxRoute softmaxRoute(const T *x, const T *z, const So
         return SM_ROW_REGISTERS;
     // an f-order matrix whose column stride keeps the row vectors aligned
     if (pl.xRow == 1 && pl.zRow == 1 && pl.numRows % N == 0 && pl.xEl % N == 0 && pl.zEl % N == 0 && pl.numRows >= kWave &&
-        pl.length <= (Long)kColCols * kColPacks && (Long)((pl.numRows + 8 * N - 1) / (8 * N)) <= kMaxGrid)
+        pl.length <= (Long)kColCols * kColPacks && (Long)((pl.numRows + 8 * N - 1) / (8 * N)) <= kMaxGrid / 4)  // blocks of 1024 threads
         return SM_COL_REGISTERS;
     return SM_PASSES;
 }
