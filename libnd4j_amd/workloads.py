@@ -268,10 +268,11 @@ def reduce3_pairs(dev, rows=16384, cols=4096, seed=12, copies=None):
 
         cases.append(Case("dot_full", "reduce3", n, 8 * n + 4, gpu_dot, lambda lib: lib.reduce3_scalar(3, x, xi, y, xi, None), True,
                           lambda: np.array([out["dot"]], F32)))
-        # every row of a [2048,1024] corner of x against every row of the same corner of y: 2048 x 2048 dot products.
+        # every row of a [2048,1024] piece of x (its first 2 Mi elements) against every row of the same piece of y: 2048 x 2048
+        # dot products.
         # Not a streaming case: each operand is read from HBM once and reused from LDS (its "bytes" are the 16 MiB of
         # operands and the 16 MiB of results), so what bounds it is the vector ALUs; `elements` counts the pairs.
-        ar, al = 2048, 1024
+        ar, al = min(2048, rows), min(1024, cols)
         ai, azi = harness.shape_info([ar, al]), harness.shape_info([ar, ar])
         ZA = w.operand(np.zeros(ar * ar, F32), azi)
         ex_a = dev.extra(ai, ai, azi, tad=dev.tad(ai, [1]))  # host TAD shapeInfo in slot 9, device tables in 10 / 11
