@@ -107,6 +107,17 @@ __global__ void __launch_bounds__(kBlock) pullRowsKernel(const T *x, T *z, Long 
     const Long xe = dEws(tadInfo), ze = dEws(zTadInfo);
     const int lanes = lanesPerTad<T>(tadLength), groups = kBlock / lanes;
     const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
+    if (lanes == kBlock && xe == 1 && ze == 1) {
+        // long contiguous TADs are cut into pieces of four vectors per lane, so that a few long rows still fill the chip
+        const Long piece = (Long)kBlock * 4 * Pack<T>::N;
+        const Long pieces = (tadLength + piece - 1) / piece;
+        for (Long u = blockIdx.x; u < n * pieces; u += gridDim.x) {
+            const Long idx = u / pieces, f0 = (u - idx * pieces) * piece;
+            const Long len = tadLength - f0 < piece ? tadLength - f0 : piece;
+            copyRun<T, false>(x + tadOffsets[indexes[idx]] + f0, 1, tadInfo, z + zTadOffsets[idx] + f0, 1, zTadInfo, len, lane, lanes);
+        }
+        return;
+    }
     for (Long idx = (Long)blockIdx.x * groups + g; idx < n; idx += (Long)gridDim.x * groups)
         copyRun<T, false>(x + tadOffsets[indexes[idx]], xe, tadInfo, z + zTadOffsets[idx], ze, zTadInfo, tadLength, lane, lanes);
 }
@@ -400,8 +411,9 @@ template <typename T>
 void launchPullRows(hipStream_t s, const T *x, T *z, Long n, const Long *indexes, const Long *tadInfo, const Long *tadOffsets,
                     const Long *zTadInfo, const Long *zTadOffsets) {
     if (n <= 0) return;
-    hipLaunchKernelGGL((pullRowsKernel<T>), dim3(gridFor(n, 1, kGridCap * 4)), dim3(kBlock), 0, s, x, z, n, indexes, tadInfo,
-                       tadOffsets, zTadInfo, zTadOffsets);
+    // (a launch with few rows gets the full grid: the kernel cuts long rows into pieces, and idle blocks leave at once)
+    hipLaunchKernelGGL((pullRowsKernel<T>), dim3(n >= kGridCap ? gridFor(n, 1, kGridCap * 4) : kGridCap), dim3(kBlock), 0, s, x, z, n,
+                       indexes, tadInfo, tadOffsets, zTadInfo, zTadOffsets);
 }
 template <typename T>
 void launchTear(hipStream_t s, const T *x, const Long *xInfo, T *const *targets, const Long *zInfo, const Long *tadInfo,

@@ -464,7 +464,8 @@ def check_data_movement(be, dtypes=(np.float32, np.float64, np.float16), big=Fal
         pcases = [([9, 6], "c", [1], "c"), ([9, 6], "f", [1], "c"), ([9, 6], "c", [1], "f"), ([7, 3, 4], "c", [1, 2], "c"),
                   ([7, 3, 4], "f", [1, 2], "f")]
         if big:
-            pcases += [([500, 1024], "c", [1], "c"), ([300, 2052], "c", [1], "c"), ([400, 130], "f", [1], "c")]
+            pcases += [([500, 1024], "c", [1], "c"), ([300, 2052], "c", [1], "c"), ([400, 130], "f", [1], "c"),
+                       ([6, 9000], "c", [1], "c"), ([5, 9001], "c", [1], "c")]  # long rows go in pieces
         for shape, order, dims, z_order in pcases:
             buf, info, logical = _view(shape, order)
             x = _cast(buf, dt)
