@@ -377,7 +377,37 @@ inline void computeTad(const Long *xsi, const int *dim, int dimLen, TadPack &out
     out.offsets.clear();
     if (wantOffsets) {
         out.offsets.resize((size_t)numTads);
-        for (Long i = 0; i < numTads; i++) out.offsets[(size_t)i] = tadOffsetOf(xsi, dim, dimLen, whole, i);
+        // The coordinates tadOffsetOf derives from the index by division are those of an odometer over the dimensions
+        // outside the TAD (last one fastest), as long as their product stays within the reference's 32-bit arithmetic:
+        // then the offsets are stepped instead of divided out (a million TADs in a few milliseconds instead of fifty).
+        int left[kMaxRank];
+        int nl = 0;
+        Long product = 1;
+        const Long *shp = siShape(xsi), *str = siStride(xsi);
+        for (int i = 0; i < rank; i++) {
+            bool inDim = false;
+            for (int j = 0; j < dimLen; j++) if (dim[j] == i) { inDim = true; break; }
+            if (!inDim) { left[nl++] = i; product *= shp[i]; }
+        }
+        if (whole) {
+            for (Long i = 0; i < numTads; i++) out.offsets[(size_t)i] = i;
+        } else if (nl > 0 && product == numTads && product <= 0x7fffffffLL) {
+            Long coord[kMaxRank] = {0};
+            Long off = 0;
+            for (Long i = 0; i < numTads; i++) {
+                out.offsets[(size_t)i] = off;
+                for (int k = nl - 1; k >= 0; k--) {
+                    const Long extent = shp[left[k]], stride = extent != 1 ? str[left[k]] : 0;
+                    coord[k]++;
+                    off += stride;
+                    if (coord[k] < extent) break;
+                    off -= coord[k] * stride;
+                    coord[k] = 0;
+                }
+            }
+        } else {
+            for (Long i = 0; i < numTads; i++) out.offsets[(size_t)i] = tadOffsetOf(xsi, dim, dimLen, whole, i);
+        }
     }
 }
 
