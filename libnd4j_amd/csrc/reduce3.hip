@@ -75,7 +75,7 @@ struct Reduce3Plan {
 // of the single run and the block's triple goes to partials[blockIdx.x].
 template <typename T, int OP, int GROUP>
 __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, T *z, const T *extra, Reduce3Plan pl,
-                                                        Acc3<typename Compute<T>::type> *partials, Long sliceLength,
+                                                        Acc3<typename Compute<T>::type> *partials, Long sliceLength, Long slices,
                                                         unsigned *signal, unsigned ticket) {
     typedef typename Compute<T>::type C;
     typedef Acc3<C> Acc;
@@ -85,15 +85,15 @@ __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, 
     const C eps = extra != nullptr ? toCompute(extra[0]) : (C)0;
     const int g = threadIdx.x / GROUP, lane = threadIdx.x % GROUP;
     const bool sliced = partials != nullptr;
-    const Long units = sliced ? (Long)gridDim.x : pl.numOut;
+    const Long units = sliced ? pl.numOut * slices : pl.numOut;
     for (Long u0 = (Long)blockIdx.x * GROUPS; u0 < units; u0 += (Long)gridDim.x * GROUPS) {
         const Long u = u0 + g;
         const bool live = u < units;
         Acc acc;
         acc.r = acc.e0 = acc.e1 = (C)0;
         if (live) {
-            const Long r = sliced ? 0 : u;
-            const Long f0 = sliced ? u * sliceLength : 0;
+            const Long r = sliced ? u / slices : u;
+            const Long f0 = sliced ? (u - r * slices) * sliceLength : 0;
             Long f1 = sliced ? f0 + sliceLength : pl.runLength;
             if (f1 > pl.runLength) f1 = pl.runLength;
             // (the usual pairing - run r of x with run r of y - needs neither the division nor the remainder)
@@ -159,14 +159,16 @@ __global__ void __launch_bounds__(kBlock) reduce3Finish(T *z, const Acc3<typenam
     typedef typename Compute<T>::type C;
     typedef Acc3<C> Acc;
     __shared__ Acc smem[kBlock / kWave];
+    // blockIdx.x is the result; its `count` slices lie next to each other
+    partials += (Long)blockIdx.x * count;
     Acc acc;
     acc.r = acc.e0 = acc.e1 = (C)0;
     for (int i = threadIdx.x; i < count; i += kBlock) acc = add3(acc, partials[i]);
     Acc3Merge<C> mg;
     acc = blockMerge<Acc3Merge<C>>(mg, acc, smem);
     if (threadIdx.x == 0) {
-        z[0] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, runLength));
-        signalResult(signal, ticket);
+        z[blockIdx.x] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, runLength));
+        signalResult(signal, ticket);  // set only for a launch with a single result
     }
 }
 
@@ -307,11 +309,13 @@ template <typename T> struct Reduce3Body {
                     return true;
                 }
             }
-            if (pl.numOut == 1 && pl.runLength >= 4 * kBlock) {
+            // one long run, or a few: cut into slices that a second kernel merges (a block per run would leave most of
+            // the chip idle)
+            if ((pl.numOut == 1 && pl.runLength >= 4 * kBlock) || (pl.numOut <= 1024 && pl.runLength >= 16384)) {
                 Long perBlock = (Long)kBlock * 8 * Pack<T>::N;
                 Long slices = (pl.runLength + perBlock - 1) / perBlock;
-                if (slices > 2048) slices = 2048;
-                if ((size_t)slices * sizeof(Acc) > ws.bytes) slices = (Long)(ws.bytes / sizeof(Acc));
+                if (slices > 2048 / pl.numOut) slices = 2048 / pl.numOut;
+                if ((size_t)(slices * pl.numOut) * sizeof(Acc) > ws.bytes) slices = (Long)(ws.bytes / sizeof(Acc)) / pl.numOut;
                 if (slices < 1) slices = 1;
                 // slices start on 16-byte boundaries whenever the run does
                 Long sliceLength = (pl.runLength + slices - 1) / slices;
@@ -319,10 +323,10 @@ template <typename T> struct Reduce3Body {
                 slices = (pl.runLength + sliceLength - 1) / sliceLength;
                 if (slices >= 2) {  // a single slice needs no second launch: the per-result kernels below do it in one
                     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
-                    hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)slices), dim3(kBlock), 0, s, x, y, z, extra, pl,
-                                       partials, sliceLength, (unsigned *)nullptr, 0u);
-                    hipLaunchKernelGGL((reduce3Finish<T, OP>), dim3(1), dim3(kBlock), 0, s, z, partials, (int)slices, pl.runLength,
-                                       ws.signal, ws.ticket);
+                    hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)(slices * pl.numOut)), dim3(kBlock), 0, s, x, y, z,
+                                       extra, pl, partials, sliceLength, slices, (unsigned *)nullptr, 0u);
+                    hipLaunchKernelGGL((reduce3Finish<T, OP>), dim3((unsigned)pl.numOut), dim3(kBlock), 0, s, z, partials, (int)slices,
+                                       pl.runLength, pl.numOut == 1 ? ws.signal : nullptr, ws.ticket);
                     return true;
                 }
             }
@@ -331,13 +335,13 @@ template <typename T> struct Reduce3Body {
             const unsigned ticket = ws.ticket;
             if (pl.runLength >= 4096) {
                 int grid = gridFor(pl.numOut, 1, kGridCap);
-                hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, signal, ticket);
+                hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
             } else if (pl.runLength >= 128) {
                 int grid = gridFor(pl.numOut, kBlock / 64, kGridCap);
-                hipLaunchKernelGGL((reduce3Kernel<T, OP, 64>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, signal, ticket);
+                hipLaunchKernelGGL((reduce3Kernel<T, OP, 64>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
             } else {
                 int grid = gridFor(pl.numOut, kBlock / 16, kGridCap);
-                hipLaunchKernelGGL((reduce3Kernel<T, OP, 16>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, signal, ticket);
+                hipLaunchKernelGGL((reduce3Kernel<T, OP, 16>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
             }
             return true;
         }

@@ -313,7 +313,8 @@ def test_reduce3_family(gpu, cpu):
         close(gpu.reduce3_scalar(op, xs, xsi, ys, xsi), cpu.reduce3_scalar(op, xs, xsi, ys, xsi), ("strided", op))
     # along dimensions: TAD against TAD, TAD against one vector (with and without the caller's TAD tables)
     for shape, order, dims in (([33, 65], "c", [1]), ([33, 65], "c", [0]), ([6, 5, 7], "c", [2]), ([6, 5, 7], "c", [1, 2]),
-                               ([6, 5, 7], "c", [0]), ([40, 5000], "c", [1]), ([300, 130], "f", [0])):
+                               ([6, 5, 7], "c", [0]), ([40, 5000], "c", [1]), ([300, 130], "f", [0]),
+                               ([5, 40003], "c", [1]), ([3, 70000], "c", [1])):  # few long runs: sliced over the chip
         xi = harness.shape_info(shape, order)
         n = int(np.prod(shape))
         x = rs.uniform(0.1, 2, n).astype(np.float32)
@@ -335,6 +336,11 @@ def test_reduce3_family(gpu, cpu):
     x, y = rs.uniform(0.1, 2, 7 * 190).astype(np.float32), rs.uniform(0.1, 2, 4 * 190).astype(np.float32)
     for op in (0, 1, 2, 3, 5, 6, 7):
         close(gpu.reduce3_all(op, x, xi, y, yi, None, [1], 28), cpu.reduce3_all(op, x, xi, y, yi, None, [1], 28), ("all", op))
+    # a few long runs, every pair of them: sliced, not tiled
+    xi, yi = shape_info_np([3, 50001]), shape_info_np([2, 50001])
+    x, y = rs.uniform(0.1, 2, 3 * 50001).astype(np.float32), rs.uniform(0.1, 2, 2 * 50001).astype(np.float32)
+    for op in (0, 1, 2, 3, 5, 6, 7):
+        close(gpu.reduce3_all(op, x, xi, y, yi, None, [1], 6), cpu.reduce3_all(op, x, xi, y, yi, None, [1], 6), ("long all", op))
     # enough pairs for the tiled kernel: ragged tile edges, a run length that ends inside a staged step, misaligned runs
     # (the last shape has enough 64 x 64 tiles for the larger tile; the others run 32 x 32 ones)
     for (nx, ny, length) in ((70, 33, 100), (64, 128, 256), (17, 16, 9), (130, 65, 1027), (1450, 1420, 43)):
