@@ -555,6 +555,28 @@ __global__ void __launch_bounds__(kBlock) isMaxRowFillKernel(T *z, const T *inde
     constexpr int GROUPS = kBlock / GROUP;
     const int g = threadIdx.x / GROUP, lane = threadIdx.x % GROUP;
     const T one = fromCompute<T>((C)1), zero = fromCompute<T>((C)0);
+    if (GROUP == kBlock) {
+        // long TADs are written in pieces of four vectors per lane, so that a few of them still fill the chip
+        const Long piece = (Long)kBlock * 4 * N, pieces = (tadLength + piece - 1) / piece;
+        for (Long u = blockIdx.x; u < numTads * pieces; u += gridDim.x) {
+            const Long r = u / pieces, f0 = (u - r * pieces) * piece;
+            const Long f1 = f0 + piece < tadLength ? f0 + piece : tadLength;
+            T *zr = z + offsets[r];
+            const Long hit = (Long)toCompute(index[r]);
+            if ((reinterpret_cast<uintptr_t>(zr) & 15) == 0 && tadLength % N == 0) {
+                Pack<T> *zv = reinterpret_cast<Pack<T> *>(zr);
+                for (Long p = f0 / N + lane; p < f1 / N; p += GROUP) {
+                    Pack<T> o;
+#pragma unroll
+                    for (int e = 0; e < N; e++) o.v[e] = (p * N + e == hit) ? one : zero;
+                    storePack(zv + p, o);
+                }
+            } else {
+                for (Long f = f0 + lane; f < f1; f += GROUP) zr[f] = (f == hit) ? one : zero;
+            }
+        }
+        return;
+    }
     for (Long r = (Long)blockIdx.x * GROUPS + g; r < numTads; r += (Long)gridDim.x * GROUPS) {
         T *zr = z + offsets[r];
         const Long hit = (Long)toCompute(index[r]);
@@ -597,8 +619,9 @@ template <typename T> void launchIsMaxTadFill(hipStream_t s, T *z, const T *inde
     if (zt.numTads <= 0 || zt.tadLength <= 0) return;
     if (zt.kind == TadPlan::ROW) {
         if (zt.tadLength >= 2048) {
-            hipLaunchKernelGGL((isMaxRowFillKernel<T, kBlock>), dim3(gridFor(zt.numTads, 1, kMaxGrid)), dim3(kBlock), 0, s, z, index,
-                               zt.offsets, zt.tadLength, zt.numTads);
+            const Long pieces = (zt.tadLength + (Long)kBlock * 4 * Pack<T>::N - 1) / ((Long)kBlock * 4 * Pack<T>::N);
+            hipLaunchKernelGGL((isMaxRowFillKernel<T, kBlock>), dim3(gridFor(zt.numTads * pieces, 1, kMaxGrid)), dim3(kBlock), 0, s, z,
+                               index, zt.offsets, zt.tadLength, zt.numTads);
         } else if (zt.tadLength >= 256) {
             hipLaunchKernelGGL((isMaxRowFillKernel<T, 64>), dim3(gridFor(zt.numTads, kBlock / 64, kMaxGrid)), dim3(kBlock), 0, s, z,
                                index, zt.offsets, zt.tadLength, zt.numTads);

@@ -466,7 +466,7 @@ def test_special_transforms(gpu, cpu):
         assert got.sum() == 1 and got[np.argmax(x)] == 1
     tie = np.array([1, 7, 7, 3, 7, 0], np.float32)
     assert np.array_equal(gpu.transform(41, tie, shape_info_np([1, 6]), shape_info_np([1, 6])), [0, 1, 0, 0, 0, 0])
-    for shape, order in (([12, 40], "c"), ([12, 40], "f"), ([300, 700], "c")):
+    for shape, order in (([12, 40], "c"), ([12, 40], "f"), ([300, 700], "c"), ([3, 9000], "c"), ([2, 9001], "c")):  # long rows: pieces
         xi = harness.shape_info(shape, order)
         n = shape[0] * shape[1]
         x = rs.permutation(n).astype(np.float32)
