@@ -242,6 +242,8 @@ def main():
                     med, runs = cpu_time(c.cpu, cpu_lib, 1.0, min_runs=2, max_runs=10)
                     row["cpu_ms"] = round(med * 1e3, 3)
                     row["cpu_GB/s"] = round(c.bytes / med / 1e9, 2)
+                    time.sleep(0.05)  # the OpenMP workers spin for a while after a parallel region: let them go to sleep
+                                      # before the next case's host thread needs a core to itself
                 if c.note:
                     row["note"] = c.note
                 fam.append(row)
