@@ -188,6 +188,9 @@ void waitForScalar(const ScalarSignal &sig, hipStream_t s, const char *what) {
     const auto start = std::chrono::steady_clock::now();
     auto nextQuery = start + std::chrono::microseconds(50);
     for (unsigned spins = 1; *flag != sig.ticket; spins++) {
+#if defined(__x86_64__)
+        __builtin_ia32_pause();  // leaves the core's shared resources to a sibling thread while this one spins
+#endif
         if ((spins & 0xff) != 0) continue;
         const auto now = std::chrono::steady_clock::now();
         if (now < nextQuery) continue;
