@@ -568,3 +568,106 @@ def check_data_movement(be, dtypes=(np.float32, np.float64, np.float16), big=Fal
             got = be.convert(codes[src], x, codes[dst])
             assert np.array_equal(got.view(np.dtype("u%d" % np.dtype(dst).itemsize)),
                                   want.view(np.dtype("u%d" % np.dtype(dst).itemsize))), ("convert", src, dst)
+
+
+# ---- random views: every family on generated shapes, strides and dimensions, one implementation against another ------
+def random_view(rs, shape=None):
+    """A shapeInfo for `shape` (or for a random shape of rank 1-4): dense c, dense f, permuted dense strides, or permuted
+    strides with padding between the dimensions.  A given shape is kept as it is.  Unit dimensions only appear in the
+    dense kinds: the EWS field of a vector-shaped view is the stride of its last dimension whatever that dimension's
+    extent (shape.h:1467), so an [n,1] view with arbitrary strides would describe memory its buffer does not have."""
+    from libnd4j_amd import harness
+    fixed = shape is not None
+    if shape is None:
+        rank = rs.randint(1, 5)
+        shape = [int(rs.choice([1, 2, 3, 4, 5, 7, 8, 16, 33, 64, 100])) for _ in range(rank)]
+        if rank == 1:
+            shape = [1] + shape
+    shape = [int(v) for v in shape]
+    rank = len(shape)
+    kind = rs.randint(0, 4)
+    if fixed and any(v == 1 for v in shape):
+        kind = rs.randint(0, 2)
+    if kind < 2:
+        return harness.shape_info(shape, "c" if kind == 0 else "f")
+    shape = [max(2, v) for v in shape]
+    strides = [0] * rank
+    run = 1 if kind == 2 else int(rs.choice([1, 2, 3]))
+    for d in rs.permutation(rank):
+        strides[d] = run
+        run *= shape[d] + (int(rs.randint(0, 3)) if kind == 3 else 0)
+    info = harness.shape_info(shape, "c" if rs.rand() < 0.5 else "f", strides=strides)
+    offsets = harness.element_offsets(info)
+    assert 0 <= offsets.min() and offsets.max() < harness.span_of(info)
+    return info
+
+
+def check_random_views(be, ref, seed, cases):
+    """`be` against `ref` (two backends of tests/backends.py) on `cases` generated calls.  Elementwise results within
+    ELEMENTWISE_ULP (pairwise and scalar arithmetic exactly), nothing written outside the result's view; reductions
+    within REDUCE_RTOL of the result plus the rounding of the summed magnitudes; index reductions (on distinct values)
+    exactly."""
+    from libnd4j_amd import harness
+    rs = np.random.RandomState(seed)
+    done = {}
+
+    def kw(**k):  # the GPU backend can be told to withhold the caller's TAD tables; the CPU ones have no such switch
+        return k if getattr(be, "kind", "") == "hip" else {}
+
+    for _ in range(cases):
+        xi = random_view(rs)
+        shape = [int(v) for v in harness.info_shape(xi)]
+        n, rank = int(np.prod(shape)), len(shape)
+        x = rs.uniform(-3, 3, harness.span_of(xi)).astype(np.float32)
+        what = int(rs.randint(0, 7))
+        if what == 0:
+            zi, op = random_view(rs, shape), int(rs.choice([0, 3, 15, 6, 10, 23, 42]))
+            g, c = be.transform(op, x, xi, zi), ref.transform(op, x, xi, zi)
+            sel = harness.element_offsets(zi)
+            assert ulp_distance(g[sel], c[sel]).max() <= ELEMENTWISE_ULP, ("transform", op, list(xi), list(zi))
+            assert np.all(np.delete(g, sel) == 0), ("transform wrote outside its view", list(zi))
+        elif what == 1:
+            yi, zi, op = random_view(rs, shape), random_view(rs, shape), int(rs.choice([0, 1, 2, 6, 13]))
+            y = rs.uniform(-3, 3, harness.span_of(yi)).astype(np.float32)
+            g, c = be.pairwise(op, x, xi, y, yi, zi), ref.pairwise(op, x, xi, y, yi, zi)
+            sel = harness.element_offsets(zi)
+            assert np.array_equal(g[sel], c[sel]), ("pairwise", op, list(xi), list(yi), list(zi))
+            assert np.all(np.delete(g, sel) == 0), ("pairwise wrote outside its view", list(zi))
+        elif what in (2, 3, 4):
+            k = int(rs.randint(1, rank + 1)) if rank > 1 else 1
+            dims = sorted(int(d) for d in rs.choice(rank, size=min(k, rank), replace=False))
+            out_len = n // int(np.prod([shape[d] for d in dims]))
+            if what == 2:
+                op = int(rs.choice([0, 1, 3, 4, 5]))
+                g = be.reduce(op, x, xi, None, dims, out_len, **kw(pass_tads=bool(rs.randint(0, 2))))
+                c = ref.reduce(op, x, xi, None, dims, out_len)
+                scale = np.abs(x).sum() / max(1, out_len)
+                assert np.all(np.abs(g.astype(np.float64) - c) <= 2 * REDUCE_RTOL * np.abs(c) + 2e-6 * scale), ("reduce", op, dims, list(xi))
+            elif what == 3:
+                xu = rs.permutation(harness.span_of(xi)).astype(np.float32)  # distinct values: no ties to resolve
+                op = int(rs.choice([0, 1]))
+                assert np.array_equal(be.indexreduce(op, xu, xi, None, dims, out_len), ref.indexreduce(op, xu, xi, None, dims, out_len)), (
+                    "indexreduce", op, dims, list(xi))
+            else:
+                if len(dims) != 1 and out_len > 1:
+                    continue  # the reference's summary statistics take one dimension (or all of them)
+                g, c = be.summarystats(0, True, x, xi, dims, out_len), ref.summarystats(0, True, x, xi, dims, out_len)
+                assert np.allclose(g, c, rtol=2 * REDUCE_RTOL, atol=1e-6), ("summarystats", dims, list(xi))
+        elif what == 5:
+            if rank < 2:
+                continue
+            d = int(rs.randint(0, rank))
+            yi = harness.shape_info([1, shape[d]])
+            y = rs.uniform(-3, 3, shape[d]).astype(np.float32)
+            op = int(rs.choice([0, 1, 2, 3]))
+            g = be.broadcast(op, x, xi, y, yi, xi, [d], **kw(pass_tads=bool(rs.randint(0, 2))))
+            c = ref.broadcast(op, x, xi, y, yi, xi, [d])
+            sel = harness.element_offsets(xi)
+            assert ulp_distance(g[sel], c[sel]).max() <= 1, ("broadcast", op, d, list(xi))
+        else:
+            zi, op = random_view(rs, shape), int(rs.choice([0, 1, 2]))
+            g, c = be.scalar(op, x, xi, zi, 1.5), ref.scalar(op, x, xi, zi, 1.5)
+            sel = harness.element_offsets(zi)
+            assert np.array_equal(g[sel], c[sel]), ("scalar", op, list(xi), list(zi))
+        done[what] = done.get(what, 0) + 1
+    return done

@@ -744,3 +744,10 @@ def test_concurrent_callers_on_their_own_streams():
         t.join(timeout=100)
     assert not any(t.is_alive() for t in threads), "a caller did not finish"
     assert errors == []
+
+
+def test_random_views_against_the_cpu_checker(gpu, cpu):
+    """Generated shapes, strides and dimensions through every loop family (tests/checks.py: check_random_views), with and
+    without the caller's TAD tables.  Fixed seed: the same few thousand calls every run."""
+    done = checks.check_random_views(gpu, cpu, seed=7, cases=4000)
+    assert len(done) == 7 and min(done.values()) > 200
