@@ -220,6 +220,19 @@ static __device__ __noinline__ float expm1fSlow_(float x) {
     return y;
 }
 
+// a / b for operands that need neither scaling nor special cases (normal, far from overflow and underflow): reciprocal
+// estimate, quotient, two residual corrections - six instructions where the general correctly rounded division takes
+// eleven.  expm1f_ and tanhf_ divide such operands only; with this division they return, for every one of the 2^32 float
+// arguments, the bits they return with the general one (compared exhaustively on the device).
+__device__ __forceinline__ float divShort_(float a, float b) {
+    const float y = __builtin_amdgcn_rcpf(b);
+    float q = a * y;
+    float r = __builtin_fmaf(-b, q, a);
+    q = __builtin_fmaf(r, y, q);
+    r = __builtin_fmaf(-b, q, a);
+    return __builtin_fmaf(r, y, q);
+}
+
 // The same arithmetic with the case distinctions turned into selects: every lane of a wave runs one
 // instruction stream whatever case its argument falls in.  fdlibm's cases differ only in k (0, +-1 near
 // +-ln2, round(x / ln2) otherwise - with t = k the reduction x - t ln2_hi, t ln2_lo is the same expression in
@@ -242,7 +255,7 @@ __device__ __forceinline__ float expm1f_(float x0) {
     const float hfx = 0.5f * x, hxs = x * hfx;
     const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
     t = 3.0f - r1 * hfx;
-    const float e = hxs * ((r1 - t) / (6.0f - x * t));
+    const float e = hxs * divShort_(r1 - t, 6.0f - x * t);
     const float res0 = x - (x * e - hxs);  // k == 0
     float e2 = (x * (e - c) - c);
     e2 -= hxs;
@@ -276,7 +289,7 @@ __device__ __forceinline__ float tanhf_(float x) {
     float arg = (big ? two : -two) * __builtin_fabsf(x);
     if (sat) arg = one;  // result unused; keeps expm1f_ on its main path
     const float t = expm1f_(arg);
-    const float q = (big ? two : -t) / (t + two);
+    const float q = divShort_(big ? two : -t, t + two);
     float z = big ? one - q : q;
     z = sat ? one - tiny : z;
     float r = jx >= 0 ? z : -z;
