@@ -128,13 +128,14 @@ struct SoftmaxPlan {
 template <typename T> bool launchSoftmax(hipStream_t stream, int opNum, const T *x, T *z, const SoftmaxPlan &plan);
 // For rows that do not fit the register-resident kernels of launchSoftmax (softmaxFitsRegisters false) and are few:
 // launchSoftmaxStats (one pass of the reduction kernels, which cut long rows into slices) leaves the row maxima and the
-// row sums of exp(x - max) in two per-row arrays, and launchSoftmaxFinish writes exp(x - max) / sum (38), its
+// row sums of exp(x - max) (these in the compute type) in two per-row arrays, and launchSoftmaxFinish writes exp(x - max) / sum (38), its
 // derivative p (1 - p) (39) or its logarithm (40)
 template <typename T> bool softmaxFitsRegisters(const T *x, const T *z, const SoftmaxPlan &plan);
 template <typename T>
-bool launchSoftmaxStats(hipStream_t stream, const T *x, T *maxima, T *sums, const TadPlan &plan, Workspace ws);
+bool launchSoftmaxStats(hipStream_t stream, const T *x, T *maxima, typename Compute<T>::type *sums, const TadPlan &plan, Workspace ws);
 template <typename T>
-bool launchSoftmaxFinish(hipStream_t stream, int opNum, const T *x, T *z, const T *maxima, const T *sums, const SoftmaxPlan &plan);
+bool launchSoftmaxFinish(hipStream_t stream, int opNum, const T *x, T *z, const T *maxima, const typename Compute<T>::type *sums,
+                         const SoftmaxPlan &plan);
 // z = one-hot of the position stored (as a T) in index[0] / index[tad]; `zp` / `zt` walk z the way the index
 // reduction walked x
 template <typename T> void launchIsMaxFill(hipStream_t stream, T *z, const T *index, const FlatPlan &zp);

@@ -520,17 +520,17 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
         // times, and would leave most of the chip idle when the rows are few.  The row maxima and the row sums of
         // exp(x - max) come from one pass of the reduction kernels instead, which cut long rows into slices, and one
         // elementwise pass finishes: 12 bytes per element.  Measured against the per-row kernels this wins for rows of
-        // 16384 elements or more, for shorter rows when they are few, and always for f-order matrices.  (Not for half:
-        // a row sum may exceed its range.)
+        // 16384 elements or more, for shorter rows when they are few, and always for f-order matrices.
         const bool rowMajor = pl.xEl == 1 && pl.zEl == 1 && (pl.length >= 16384 || (pl.length >= 4096 && pl.numRows <= 512));
         const bool colMajor = pl.xRow == 1 && pl.zRow == 1 && pl.numRows >= 256 && pl.length >= 256;
-        if (sizeof(T) >= 4 && rank >= 1 && (rowMajor || colMajor) && !softmaxFitsRegisters<T>(x, z, pl)) {
+        if (rank >= 1 && (rowMajor || colMajor) && !softmaxFitsRegisters<T>(x, z, pl)) {
             ResolvedTad tx;
             if (!resolveTad(nullptr, 0, 0, hx, &walked, 1, tx, s)) return true;
-            const size_t perRow = ((size_t)pl.numRows * sizeof(T) + 255) / 256 * 256;
+            typedef typename Compute<T>::type C;  // the row sums stay in the compute type: those of half rows may exceed half
+            const size_t perRow = ((size_t)pl.numRows * sizeof(C) + 255) / 256 * 256;
             Scratch sc = scratchFor(s, 2 * perRow + kWorkspaceBytes);
             T *maxima = reinterpret_cast<T *>(sc.rest.ptr);
-            T *sums = reinterpret_cast<T *>(reinterpret_cast<char *>(sc.rest.ptr) + perRow);
+            C *sums = reinterpret_cast<C *>(reinterpret_cast<char *>(sc.rest.ptr) + perRow);
             Workspace rest;
             rest.ptr = reinterpret_cast<char *>(sc.rest.ptr) + 2 * perRow;
             rest.bytes = sc.rest.bytes - 2 * perRow;

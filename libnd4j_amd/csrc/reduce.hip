@@ -158,7 +158,7 @@ template <typename TT> struct SoftmaxStatsPol {
     typedef typename Compute<TT>::type C;
     struct Acc { C m, s; };
     static constexpr bool tables = true;
-    TT *sums;
+    C *sums;  // in the compute type: a row sum of a half array may exceed the range of half
     Long row;
 
     __device__ __forceinline__ void setTad(Long r, const TT *) { row = r; }
@@ -184,13 +184,13 @@ template <typename TT> struct SoftmaxStatsPol {
         return r;
     }
     __device__ __forceinline__ TT finalize(Acc a, Long) const {
-        sums[row] = fromCompute<TT>(a.s);
+        sums[row] = a.s;
         return fromCompute<TT>(a.m);
     }
 };
 
 template <typename T>
-bool launchSoftmaxStats(hipStream_t s, const T *x, T *maxima, T *sums, const TadPlan &plan, Workspace ws) {
+bool launchSoftmaxStats(hipStream_t s, const T *x, T *maxima, typename Compute<T>::type *sums, const TadPlan &plan, Workspace ws) {
     SoftmaxStatsPol<T> pol;
     pol.sums = sums;
     pol.row = 0;
@@ -201,7 +201,7 @@ bool launchSoftmaxStats(hipStream_t s, const T *x, T *maxima, T *sums, const Tad
 #define INST(T)                                                                                                    \
     template bool launchReduceTad<T>(hipStream_t, int, const T *, const T *, T *, const TadPlan &, Workspace);     \
     template bool launchReduceScalar<T>(hipStream_t, int, const T *, const T *, T *, const FlatPlan &, Workspace); \
-    template bool launchSoftmaxStats<T>(hipStream_t, const T *, T *, T *, const TadPlan &, Workspace);
+    template bool launchSoftmaxStats<T>(hipStream_t, const T *, T *, Compute<T>::type *, const TadPlan &, Workspace);
 INST(float)
 INST(float16)
 INST(double)

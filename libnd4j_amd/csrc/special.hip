@@ -406,7 +406,8 @@ template <typename T> bool softmaxFitsRegisters(const T *x, const T *z, const So
 // Threads run along the direction in which x is contiguous (alongRows: down the rows of an f-order matrix),
 // blockIdx.y walks the other one.
 template <typename T, int MODE>
-__global__ void __launch_bounds__(kBlock) softmaxFinishKernel(const T *x, T *z, const T *maxima, const T *sums, Long numRows,
+__global__ void __launch_bounds__(kBlock) softmaxFinishKernel(const T *x, T *z, const T *maxima,
+                                                              const typename Compute<T>::type *sums, Long numRows,
                                                               Long length, Long xRow, Long xEl, Long zRow, Long zEl, int alongRows) {
     typedef typename Compute<T>::type C;
     lm::loadTables();
@@ -415,7 +416,7 @@ __global__ void __launch_bounds__(kBlock) softmaxFinishKernel(const T *x, T *z, 
         for (Long f = (Long)blockIdx.x * kBlock + threadIdx.x; f < fastLen; f += (Long)gridDim.x * kBlock) {
             const Long r = alongRows ? f : sl, c = alongRows ? sl : f;
             const C e = m::exp_(toCompute(x[r * xRow + c * xEl]) - toCompute(maxima[r]));
-            z[r * zRow + c * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(e, (C)1 / toCompute(sums[r])));
+            z[r * zRow + c * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(e, (C)1 / sums[r]));
         }
     }
 }
@@ -425,19 +426,21 @@ __global__ void __launch_bounds__(kBlock) softmaxFinishKernel(const T *x, T *z, 
 // each thread asks for its next vector before it works on the current one; the first is requested before the tables.
 template <typename T, int MODE, int ALONG> struct SoftmaxFinishItem {
     typedef typename Compute<T>::type C;
-    Pack<T> a, pm, ps;
+    Pack<T> a, pm;
+    C ps[Pack<T>::N];
     C mx, sum;
     Long sl, v;
-    __device__ __forceinline__ void load(Long id, bool small, const T *x, const T *maxima, const T *sums, Long fastVecs, Long xSlow) {
+    __device__ __forceinline__ void load(Long id, bool small, const T *x, const T *maxima, const C *sums, Long fastVecs, Long xSlow) {
         sl = small ? (Long)((unsigned)id / (unsigned)fastVecs) : id / fastVecs;
         v = id - sl * fastVecs;
         a = loadPack(reinterpret_cast<const Pack<T> *>(x + sl * xSlow) + v);
         if (ALONG == 1) {
             pm = reinterpret_cast<const Pack<T> *>(maxima)[v];
-            ps = reinterpret_cast<const Pack<T> *>(sums)[v];
+#pragma unroll
+            for (int e = 0; e < Pack<T>::N; e++) ps[e] = sums[v * Pack<T>::N + e];
         } else {
             mx = toCompute(maxima[sl]);
-            sum = toCompute(sums[sl]);
+            sum = sums[sl];
         }
     }
     __device__ __forceinline__ void finish(T *z, Long zSlow) const {
@@ -447,14 +450,15 @@ template <typename T, int MODE, int ALONG> struct SoftmaxFinishItem {
 #pragma unroll
         for (int e = 0; e < N; e++) {
             const C m1 = ALONG == 1 ? toCompute(pm.v[e]) : mx;
-            const C i1 = ALONG == 1 ? (C)1 / toCompute(ps.v[e]) : inv;
+            const C i1 = ALONG == 1 ? (C)1 / ps[e] : inv;
             o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(a.v[e]) - m1), i1));
         }
         storePack(reinterpret_cast<Pack<T> *>(z + sl * zSlow) + v, o);
     }
 };
 template <typename T, int MODE, int ALONG>
-__global__ void __launch_bounds__(kBlock) softmaxFinishVecKernel(const T *x, T *z, const T *maxima, const T *sums, Long fastVecs,
+__global__ void __launch_bounds__(kBlock) softmaxFinishVecKernel(const T *x, T *z, const T *maxima,
+                                                                 const typename Compute<T>::type *sums, Long fastVecs,
                                                                  Long slowLen, Long xSlow, Long zSlow) {
     const Long total = fastVecs * slowLen, stride = (Long)gridDim.x * kBlock;
     const bool small = total <= 0xffffffffLL;
@@ -474,7 +478,8 @@ __global__ void __launch_bounds__(kBlock) softmaxFinishVecKernel(const T *x, T *
 }
 
 template <typename T>
-bool launchSoftmaxFinish(hipStream_t s, int opNum, const T *x, T *z, const T *maxima, const T *sums, const SoftmaxPlan &pl) {
+bool launchSoftmaxFinish(hipStream_t s, int opNum, const T *x, T *z, const T *maxima, const typename Compute<T>::type *sums,
+                         const SoftmaxPlan &pl) {
     if (pl.numRows <= 0 || pl.length <= 0) return true;
     const int alongRows = (pl.xRow == 1 && pl.xEl != 1) ? 1 : 0;
     const Long fastLen = alongRows ? pl.numRows : pl.length, slowLen = alongRows ? pl.length : pl.numRows;
@@ -652,7 +657,7 @@ template <typename T> void launchIsMaxTadFill(hipStream_t s, T *z, const T *inde
 #define INST(T)                                                                                           \
     template bool launchSoftmax<T>(hipStream_t, int, const T *, T *, const SoftmaxPlan &);                \
     template bool softmaxFitsRegisters<T>(const T *, const T *, const SoftmaxPlan &);                     \
-    template bool launchSoftmaxFinish<T>(hipStream_t, int, const T *, T *, const T *, const T *, const SoftmaxPlan &); \
+    template bool launchSoftmaxFinish<T>(hipStream_t, int, const T *, T *, const T *, const Compute<T>::type *, const SoftmaxPlan &); \
     template void launchIsMaxFill<T>(hipStream_t, T *, const T *, const FlatPlan &);                      \
     template void launchIsMaxTadFill<T>(hipStream_t, T *, const T *, const TadPlan &);
 INST(float)
