@@ -477,6 +477,43 @@ __global__ void __launch_bounds__(kBlock) softmaxFinishVecKernel(const T *x, T *
     }
 }
 
+// Contiguous rows whose starts are not all 16-byte aligned (an odd row length, e.g. a 50257-word vocabulary): each row
+// is finished with 16-byte accesses between its own aligned head and tail, which works whenever x and z are misaligned
+// alike in every row (same row stride, bases equally aligned).  blockIdx.y walks the rows, blockIdx.x the row's vectors.
+template <typename T, int MODE>
+__global__ void __launch_bounds__(kBlock) softmaxFinishRowsKernel(const T *x, T *z, const T *maxima,
+                                                                  const typename Compute<T>::type *sums, Long numRows, Long length,
+                                                                  Long xRow, Long zRow) {
+    typedef typename Compute<T>::type C;
+    constexpr int N = Pack<T>::N;
+    lm::loadTables();
+    for (Long r = blockIdx.y; r < numRows; r += gridDim.y) {
+        const T *xr = x + r * xRow;
+        T *zr = z + r * zRow;
+        const C mx = toCompute(maxima[r]), inv = (C)1 / sums[r];
+        Long head = (Long)(((16 - (reinterpret_cast<uintptr_t>(xr) & 15)) & 15) / sizeof(T));
+        if (head > length) head = length;
+        const Long nvec = (length - head) / N;
+        const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(xr + head);
+        Pack<T> *zv = reinterpret_cast<Pack<T> *>(zr + head);
+        for (Long v = (Long)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += (Long)gridDim.x * kBlock) {
+            const Pack<T> a = loadPack(xv + v);
+            Pack<T> o;
+#pragma unroll
+            for (int e = 0; e < N; e++) o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(a.v[e]) - mx), inv));
+            storePack(zv + v, o);
+        }
+        if (blockIdx.x == 0) {
+            // the elements before the first and after the last whole vector: fewer than 2 N of them
+            const Long tail0 = head + nvec * N;
+            for (Long f = threadIdx.x; f < head + (length - tail0); f += kBlock) {
+                const Long c = f < head ? f : tail0 + (f - head);
+                zr[c] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(xr[c]) - mx), inv));
+            }
+        }
+    }
+}
+
 template <typename T>
 bool launchSoftmaxFinish(hipStream_t s, int opNum, const T *x, T *z, const T *maxima, const typename Compute<T>::type *sums,
                          const SoftmaxPlan &pl) {
@@ -506,6 +543,25 @@ bool launchSoftmaxFinish(hipStream_t s, int opNum, const T *x, T *z, const T *ma
             default: return false;
         }
 #undef ND4J_FINISH_VEC
+    }
+    if (!alongRows && pl.xEl == 1 && pl.zEl == 1 && pl.length >= 8 * N &&
+        (reinterpret_cast<uintptr_t>(x) & 15) == (reinterpret_cast<uintptr_t>(z) & 15) &&
+        (reinterpret_cast<uintptr_t>(x) & (sizeof(T) - 1)) == 0 && (pl.numRows == 1 || pl.xRow == pl.zRow)) {
+        const Long gy = pl.numRows < 65535 ? pl.numRows : 65535;
+        Long gx = (pl.length / N + kBlock - 1) / kBlock;
+        const Long budget = kGridCap * 2 / gy > 0 ? kGridCap * 2 / gy : 1;  // about 16384 blocks in all
+        if (gx > budget) gx = budget;
+        const dim3 rgrid((unsigned)gx, (unsigned)gy);
+#define ND4J_FINISH_ROWS(MODE)                                                                                                \
+    hipLaunchKernelGGL((softmaxFinishRowsKernel<T, MODE>), rgrid, dim3(kBlock), 0, s, x, z, maxima, sums, pl.numRows, pl.length, \
+                       pl.xRow, pl.zRow)
+        switch (opNum) {
+            case 38: ND4J_FINISH_ROWS(0); return true;
+            case 39: ND4J_FINISH_ROWS(1); return true;
+            case 40: ND4J_FINISH_ROWS(2); return true;
+            default: return false;
+        }
+#undef ND4J_FINISH_ROWS
     }
     const dim3 grid((unsigned)gridFor(fastLen, kBlock, 4096), (unsigned)(slowLen < 65535 ? slowLen : 65535));
 #define ND4J_FINISH(MODE)                                                                                                 \
