@@ -41,15 +41,24 @@ template <typename A> __device__ __forceinline__ A shflDownAny(A v, int delta) {
     return __builtin_bit_cast(A, out);
 }
 
+// A policy may merge the lanes of a wave its own way (a member template waveMergeOwn<WIDTH>(acc), announced by a
+// member constant ownWaveMerge): the summary statistics shuffle three of their seven doubles when they can.
+template <class Pol, typename = void> struct HasOwnWaveMerge { static constexpr bool value = false; };
+template <class Pol> struct HasOwnWaveMerge<Pol, decltype((void)Pol::ownWaveMerge)> { static constexpr bool value = Pol::ownWaveMerge; };
+
 // Merge over the lanes of one wave; lane 0 (of each WIDTH-lane segment) ends up with the result.
 template <class Pol, int WIDTH = kWave>
 __device__ __forceinline__ typename Pol::Acc waveMerge(const Pol &pol, typename Pol::Acc a) {
+    if constexpr (HasOwnWaveMerge<Pol>::value) {
+        return pol.template waveMergeOwn<WIDTH>(a);
+    } else {
 #pragma unroll
-    for (int d = WIDTH / 2; d >= 1; d >>= 1) {
-        typename Pol::Acc o = shflDownAny(a, d);
-        a = pol.combine(a, o);
+        for (int d = WIDTH / 2; d >= 1; d >>= 1) {
+            typename Pol::Acc o = shflDownAny(a, d);
+            a = pol.combine(a, o);
+        }
+        return a;
     }
-    return a;
 }
 
 // Merge over a whole 256-thread block; thread 0 gets the result.  `smem` holds kBlock/kWave accumulators.

@@ -45,15 +45,19 @@ template <typename TT, int OP> struct StatsPol {
     int phantomZero;  // the reference's single-dimension non-EWS branch starts from a zero sample
 
     __device__ __forceinline__ void setTad(Long, const TT *) {}
-    __device__ __forceinline__ Acc init(const TT *) const {
+    // Every lane's first run is shifted by the same value, the first sample of the TAD (of the array): lanes that have
+    // not closed a run yet then merge by adding their three sums (combine), which is what the merge tree of a short
+    // TAD consists of.  A run opened after a merge is shifted by its own first sample, as before.
+    __device__ __forceinline__ Acc init(const TT *first) const {
         Acc a;
         a.n = a.mean = a.m2 = 0.0;
-        a.cn = a.cs1 = a.cs2 = a.cp = 0.0;
+        a.cn = a.cs1 = a.cs2 = 0.0;
+        a.cp = (double)toCompute(first[0]);
         return a;
     }
     __device__ __forceinline__ void accumulate(Acc &a, C v, Long) const {
         double d = (double)v;
-        if (a.cn == 0.0) a.cp = d;
+        if (a.cn == 0.0 && a.n != 0.0) a.cp = d;
         double e = d - a.cp;
         a.cs1 += e;
         a.cs2 += e * e;
@@ -65,9 +69,34 @@ template <typename TT, int OP> struct StatsPol {
         if (a.cn >= kStatsRun) statsFlush(a);
     }
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const {
+        if (a.n == 0.0 && b.n == 0.0 && a.cp == b.cp) {  // two open first runs around the common shift: no divisions
+            a.cn += b.cn;
+            a.cs1 += b.cs1;
+            a.cs2 += b.cs2;
+            return a;
+        }
         statsFlush(a);
         statsFlush(b);
         statsMerge(a.n, a.mean, a.m2, b.n, b.mean, b.m2);
+        return a;
+    }
+    // While no lane of the wave has closed a run, every lane holds three sums around the TAD's common shift: those are
+    // all that has to travel (6 words per step instead of 14), and they merge by addition.
+    static constexpr bool ownWaveMerge = true;
+    template <int WIDTH> __device__ __forceinline__ Acc waveMergeOwn(Acc a) const {
+        if (__all(a.n == 0.0)) {
+#pragma unroll
+            for (int d = WIDTH / 2; d >= 1; d >>= 1) {
+                // (lanes of one segment work on one TAD and share its shift; what arrives from beyond the segment's end
+                // lands in lanes whose result is not used)
+                a.cn += shflDownAny(a.cn, d);
+                a.cs1 += shflDownAny(a.cs1, d);
+                a.cs2 += shflDownAny(a.cs2, d);
+            }
+            return a;
+        }
+#pragma unroll
+        for (int d = WIDTH / 2; d >= 1; d >>= 1) a = combine(a, shflDownAny(a, d));
         return a;
     }
     __device__ __forceinline__ TT finalize(Acc a, Long) const {
