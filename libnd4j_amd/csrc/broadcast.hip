@@ -14,6 +14,12 @@ template <typename T> struct BroadcastBody {
                 const Long nvec = pl.numTads * (pl.tadLength / Pack<T>::N);
                 hipLaunchKernelGGL((bcFlatKernel<T, F>), dim3(gridFor(nvec, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0,
                                    s, x, y, z, nvec, (unsigned)(pl.tadLength / Pack<T>::N), Params<T>{nullptr});
+            } else if (pl.kind == BroadcastPlan::ROW && pl.consecutive && pl.tadLength >= Pack<T>::N && pl.tadLength < 0xffffffffLL &&
+                       (((uintptr_t)x | (uintptr_t)z) & 15) == 0) {
+                // gap-free rows whose length is not a multiple of the vector width
+                const Long n = pl.numTads * pl.tadLength;
+                hipLaunchKernelGGL((bcFlatAnyKernel<T, F>), dim3(gridFor(n / Pack<T>::N + 1, kBlock, F::tables ? kGridCap : kMaxGrid)),
+                                   dim3(kBlock), 0, s, x, y, z, n, pl.tadLength, Params<T>{nullptr});
             } else if (pl.kind == BroadcastPlan::ROW) {
                 constexpr int VEC = Pack<T>::N;
                 Long vecsPerTad = (pl.tadLength + VEC - 1) / VEC;

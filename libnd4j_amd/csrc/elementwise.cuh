@@ -313,6 +313,38 @@ __global__ void __launch_bounds__(kBlock) bcFlatKernel(const T *x, const T *y, T
     }
 }
 
+// The same walk when the TAD length is not a multiple of the vector width (rows of odd length: only every fourth row
+// of a float matrix then starts on a 16-byte boundary): x and z are still one aligned vector after the other, and a
+// vector's elements take their y one by one, from the position inside the row where the vector begins, wrapping into
+// the next row.  The last n % VEC elements are done singly.
+template <typename T, typename F>
+__global__ void __launch_bounds__(kBlock) bcFlatAnyKernel(const T *x, const T *y, T *z, Long n, Long tadLength, Params<T> p) {
+    typedef typename Compute<T>::type C;
+    if (F::tables) lm::loadTables();
+    constexpr int VEC = Pack<T>::N;
+    const Long nvec = n / VEC;
+    const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x);
+    Pack<T> *zv = reinterpret_cast<Pack<T> *>(z);
+    const bool small = n <= 0xffffffffLL;
+    for (Long j = (Long)blockIdx.x * kBlock + threadIdx.x; j < nvec; j += (Long)gridDim.x * kBlock) {
+        const Pack<T> a = loadPack(xv + j);
+        const Long i0 = j * VEC;
+        Long f = small ? (Long)((unsigned)i0 % (unsigned)tadLength) : i0 % tadLength;
+        Pack<T> r;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            r.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), toCompute(y[f]), p));
+            f = f + 1 == tadLength ? 0 : f + 1;
+        }
+        storePack(zv + j, r);
+    }
+    const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
+    if (gtid < n - nvec * VEC) {
+        const Long i = nvec * VEC + gtid;
+        z[i] = fromCompute<T>(F::template apply<C>(toCompute(x[i]), toCompute(y[i % tadLength]), p));
+    }
+}
+
 // Broadcast over strided TADs: thread <-> TAD, loop over the TAD's elements.  When neighbouring TADs
 // are neighbours in memory (a column of a c-order matrix) each wave reads and writes full lines.
 template <typename T, typename F, bool BYTAD>

@@ -515,7 +515,9 @@ def test_broadcast_over_gap_free_tads(gpu):
     rs = np.random.RandomState(5)
     for dt in (np.float32, np.float16, np.float64):
         for shape, order, dim in (([33, 64], "c", 1), ([64, 33], "f", 0), ([5, 7, 24], "c", 2), ([40, 3, 2], "f", 0), ([33, 62], "c", 1),
-                                  ([1000, 1024], "c", 1), ([2048, 300], "f", 0)):
+                                  ([1000, 1024], "c", 1), ([2048, 300], "f", 0),
+                                  # odd row lengths, and an element count that leaves single elements after the last vector
+                                  ([700, 1023], "c", 1), ([513, 1025], "c", 1), ([7, 9], "c", 1), ([1021, 67], "f", 0), ([3, 5, 11], "c", 2)):
             od = "F" if order == "f" else "C"
             n = int(np.prod(shape))
             info = harness.shape_info(shape, order)
