@@ -153,19 +153,20 @@ __global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename P
     pol.setTad(t, z);
     const typename Pol::T *base = x + offsets[t];
     Acc acc = pol.init(base);
-    const Long j0 = (Long)blockIdx.y * rowsPerSplit;
-    Long j1 = j0 + rowsPerSplit;
-    if (j1 > tadLength) j1 = tadLength;
-    Long j = j0;
-    for (; j + 8 <= j1; j += 8) {
+    // Split y takes the rows y, y + splits, y + 2 splits, ...: the blocks that run at the same time then read
+    // neighbouring rows - one compact stretch of memory - instead of stretches a whole row range apart.
+    (void)rowsPerSplit;
+    const Long S = gridDim.y;
+    Long j = blockIdx.y;
+    for (; j + 7 * S < tadLength; j += 8 * S) {
         typename Pol::T v[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = base[(j + u) * tadEws];
+        for (int u = 0; u < 8; u++) v[u] = base[(j + u * S) * tadEws];
 #pragma unroll
-        for (int u = 0; u < 8; u++) pol.accumulate(acc, toCompute(v[u]), j + u);
+        for (int u = 0; u < 8; u++) pol.accumulate(acc, toCompute(v[u]), j + u * S);
         pol.checkpoint(acc);
     }
-    for (; j < j1; j++) { pol.accumulate(acc, toCompute(base[j * tadEws]), j); pol.checkpoint(acc); }
+    for (; j < tadLength; j += S) { pol.accumulate(acc, toCompute(base[j * tadEws]), j); pol.checkpoint(acc); }
     if (gridDim.y == 1) z[t] = pol.finalize(acc, tadLength);
     else partials[(Long)blockIdx.y * numTads + t] = acc;
 }
@@ -467,7 +468,11 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         }
         return;
     }
-    if (pl.kind == TadPlan::COL && pl.numTads >= 2 * kWave * Pack<typename Pol::T>::N) {
+    // (the vector loads need every row of the TADs' common pitch to start on a 16-byte boundary: a pitch that is not a
+    // multiple of the vector width goes to the lane-per-TAD kernel below, whose neighbouring lanes read neighbouring
+    // elements)
+    if (pl.kind == TadPlan::COL && pl.numTads >= 2 * kWave * Pack<typename Pol::T>::N &&
+        pl.tadEws % Pack<typename Pol::T>::N == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
         // lane per Pack::N adjacent TADs, 64 lanes per block column, rows split over the block's waves and blockIdx.y
         constexpr int VEC = Pack<typename Pol::T>::N;
         int gx = (int)((pl.numTads + (Long)kWave * VEC - 1) / ((Long)kWave * VEC));
