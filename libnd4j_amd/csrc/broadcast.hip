@@ -35,6 +35,12 @@ template <typename T> struct BroadcastBody {
                 int aligned = (((uintptr_t)x | (uintptr_t)z) & 15) == 0 ? 1 : 0;
                 hipLaunchKernelGGL((bcRowKernel<T, F, false>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
                                    pl.zOffsets, pl.tadLength, pl.numTads, aligned, colShift, Params<T>{nullptr});
+            } else if (pl.kind == BroadcastPlan::COL && pl.denseAlike && pl.tadEws >= 1 && pl.tadEws < 0xffffffffLL &&
+                       pl.tadLength < 0xffffffffLL && (((uintptr_t)x | (uintptr_t)z) & 15) == 0) {
+                // any single dimension of a dense array: runs of tadEws consecutive elements share one y
+                const Long n = pl.numTads * pl.tadLength;
+                hipLaunchKernelGGL((bcFlatInnerKernel<T, F>), dim3(gridFor(n / Pack<T>::N + 1, kBlock, F::tables ? kGridCap : kMaxGrid)),
+                                   dim3(kBlock), 0, s, x, y, z, n, pl.tadEws, pl.tadLength, Params<T>{nullptr});
             } else if (pl.kind == BroadcastPlan::COL) {
                 int gx = (int)((pl.numTads + kBlock - 1) / kBlock);
                 Long gy = (Long)kGridCap / gx;

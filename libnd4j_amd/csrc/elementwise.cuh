@@ -345,6 +345,51 @@ __global__ void __launch_bounds__(kBlock) bcFlatAnyKernel(const T *x, const T *y
     }
 }
 
+// Broadcast along one dimension of a dense array, whatever its position (a column vector added to the rows of a c-order
+// matrix, a per-channel bias in the middle of a rank-3 array): in memory order, `inner` consecutive elements share one
+// y (inner is the dimension's stride) and the y index then steps through the dimension's `extent` values.  x and z are
+// walked as aligned vectors; a vector finds its run by two divisions and steps on from there.
+template <typename T, typename F>
+__global__ void __launch_bounds__(kBlock) bcFlatInnerKernel(const T *x, const T *y, T *z, Long n, Long inner, Long extent, Params<T> p) {
+    typedef typename Compute<T>::type C;
+    if (F::tables) lm::loadTables();
+    constexpr int VEC = Pack<T>::N;
+    const Long nvec = n / VEC;
+    const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x);
+    Pack<T> *zv = reinterpret_cast<Pack<T> *>(z);
+    const bool small = n <= 0xffffffffLL;
+    for (Long j = (Long)blockIdx.x * kBlock + threadIdx.x; j < nvec; j += (Long)gridDim.x * kBlock) {
+        const Pack<T> a = loadPack(xv + j);
+        const Long i0 = j * VEC;
+        Long q, yi;
+        if (small) {
+            q = (Long)((unsigned)i0 / (unsigned)inner);
+            yi = (Long)((unsigned)q % (unsigned)extent);
+        } else {
+            q = i0 / inner;
+            yi = q % extent;
+        }
+        Long rem = i0 - q * inner;
+        C yv = toCompute(y[yi]);
+        Pack<T> r;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            r.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), yv, p));
+            if (++rem == inner) {
+                rem = 0;
+                yi = yi + 1 == extent ? 0 : yi + 1;
+                yv = toCompute(y[yi]);
+            }
+        }
+        storePack(zv + j, r);
+    }
+    const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
+    if (gtid < n - nvec * VEC) {
+        const Long i = nvec * VEC + gtid;
+        z[i] = fromCompute<T>(F::template apply<C>(toCompute(x[i]), toCompute(y[(i / inner) % extent]), p));
+    }
+}
+
 // Broadcast over strided TADs: thread <-> TAD, loop over the TAD's elements.  When neighbouring TADs
 // are neighbours in memory (a column of a c-order matrix) each wave reads and writes full lines.
 template <typename T, typename F, bool BYTAD>

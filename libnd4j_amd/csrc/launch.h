@@ -32,6 +32,8 @@ struct BroadcastPlan {
     const Long *xOffsets;        // device, numTads entries
     const Long *zOffsets;        // device, numTads entries
     bool consecutive = false;    // ROW only: TAD r starts at r * tadLength in x and in z (rows of a dense c-order array)
+    bool denseAlike = false;     // ROW / COL: x and z are dense arrays of one layout, y is contiguous: memory position i of
+                                 // either takes y[(i / tadEws) % tadLength]
 };
 template <typename T>
 bool launchBroadcast(hipStream_t stream, int opNum, const T *x, const T *y, T *z, const BroadcastPlan &plan);

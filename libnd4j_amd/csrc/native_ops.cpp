@@ -186,9 +186,12 @@ void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Lon
         // contiguous TADs of a dense array are its trailing (c order) or leading (f order) block, so they follow one
         // another without gaps;
         // when the result has the same dense layout the kernel needs no offset tables
-        if (pl.kind == BroadcastPlan::ROW && zTadInfo == tx.hostInfo && sameShape(hx, hz) && siNumel(hy) == tx.tadLength &&
-            ((isDense(hx, 'c') && isDense(hz, 'c')) || (isDense(hx, 'f') && isDense(hz, 'f'))))
-            pl.consecutive = true;
+        if (zTadInfo == tx.hostInfo && sameShape(hx, hz) && siNumel(hy) == tx.tadLength &&
+            ((isDense(hx, 'c') && isDense(hz, 'c')) || (isDense(hx, 'f') && isDense(hz, 'f')))) {
+            pl.consecutive = pl.kind == BroadcastPlan::ROW;
+            // a single dimension of a dense array: its stride is the number of consecutive elements that share one y
+            pl.denseAlike = pl.yEws == 1 && pl.zEws == pl.tadEws;
+        }
     } else {
         pl.kind = BroadcastPlan::GENERAL;
         char xo = siOrder(tx.hostInfo) == 'c' ? 'c' : 'f';

@@ -517,7 +517,10 @@ def test_broadcast_over_gap_free_tads(gpu):
         for shape, order, dim in (([33, 64], "c", 1), ([64, 33], "f", 0), ([5, 7, 24], "c", 2), ([40, 3, 2], "f", 0), ([33, 62], "c", 1),
                                   ([1000, 1024], "c", 1), ([2048, 300], "f", 0),
                                   # odd row lengths, and an element count that leaves single elements after the last vector
-                                  ([700, 1023], "c", 1), ([513, 1025], "c", 1), ([7, 9], "c", 1), ([1021, 67], "f", 0), ([3, 5, 11], "c", 2)):
+                                  ([700, 1023], "c", 1), ([513, 1025], "c", 1), ([7, 9], "c", 1), ([1021, 67], "f", 0), ([3, 5, 11], "c", 2),
+                                  # any other single dimension of a dense array: runs of `stride` elements share one y
+                                  ([33, 64], "c", 0), ([64, 33], "f", 1), ([5, 7, 24], "c", 1), ([5, 7, 24], "c", 0), ([40, 3, 2], "f", 1),
+                                  ([700, 1023], "c", 0), ([9, 5, 11], "f", 1), ([9, 5, 11], "f", 2), ([2, 3, 5, 7], "c", 2), ([1000, 7], "c", 0)):
             od = "F" if order == "f" else "C"
             n = int(np.prod(shape))
             info = harness.shape_info(shape, order)
