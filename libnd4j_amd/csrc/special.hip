@@ -185,10 +185,14 @@ template <class Merge, int GROUP, typename C> __device__ __forceinline__ C teamA
 }
 
 // Contiguous rows short enough to stay in registers: GROUP lanes own a row and keep PACKS 16-byte vectors of it
-// each (vector j of a lane is vector lane + j * GROUP of the row), so x is read once and z written once.  exp(x - max)
-// replaces x in the registers (rounded to T, which only matters for half).
-template <typename T, int MODE, int GROUP, int PACKS>
-__global__ void __launch_bounds__(kBlock) softmaxRowRegKernel(const T *x, T *z, Long numRows, Long npack, Long xRow, Long zRow) {
+// each (vector j of a lane is vector lane + j * GROUP of the row's aligned part), so x is read once and z written once.
+// exp(x - max) replaces x in the registers (rounded to T, which only matters for half).
+// A row need not start on a 16-byte boundary, nor hold a whole number of vectors: the elements before its first and
+// after its last aligned vector (fewer than 2 N, the "edge") are kept one per lane by the team's first lanes.  x and z
+// must be misaligned alike in every row (the host checks it).
+// (EDGES false: the host has seen that every row starts aligned and holds whole vectors, and the edge code folds away.)
+template <typename T, int MODE, int GROUP, int PACKS, bool EDGES>
+__global__ void __launch_bounds__(kBlock) softmaxRowRegKernel(const T *x, T *z, Long numRows, Long length, Long xRow, Long zRow) {
     lm::loadTables();
     typedef typename Compute<T>::type C;
     constexpr int N = Pack<T>::N;
@@ -199,13 +203,23 @@ __global__ void __launch_bounds__(kBlock) softmaxRowRegKernel(const T *x, T *z, 
     for (Long r0 = (Long)blockIdx.x * GROUPS; r0 < numRows; r0 += (Long)gridDim.x * GROUPS) {
         const Long r = r0 + g;
         const bool live = r < numRows;
-        const Pack<T> *xr = reinterpret_cast<const Pack<T> *>(x + (live ? r * xRow : 0));
-        Pack<T> *zr = reinterpret_cast<Pack<T> *>(z + (live ? r * zRow : 0));
+        const T *xrow = x + (live ? r * xRow : 0);
+        T *zrow = z + (live ? r * zRow : 0);
+        Long head = EDGES ? (Long)(((16 - (reinterpret_cast<uintptr_t>(xrow) & 15)) & 15) / sizeof(T)) : 0;
+        if (head > length) head = length;
+        const Long npack = (length - head) / N;
+        const Long tail0 = head + npack * N;           // first element after the last whole vector
+        const int edges = (int)(head + (length - tail0));  // < 2 N <= 16 <= GROUP
+        const Long edgeAt = lane < head ? lane : tail0 + (lane - head);
+        const bool hasEdge = EDGES && live && lane < edges;
+        const Pack<T> *xr = reinterpret_cast<const Pack<T> *>(xrow + head);
+        Pack<T> *zr = reinterpret_cast<Pack<T> *>(zrow + head);
         Pack<T> cache[PACKS];
 #pragma unroll
         for (int j = 0; j < PACKS; j++)
             if (live && lane + j * GROUP < npack) cache[j] = loadPack(xr + lane + j * GROUP);
-        C mx = (C)-3.4028235e38;
+        C edge = hasEdge ? toCompute(xrow[edgeAt]) : (C)0;
+        C mx = hasEdge ? edge : (C)-3.4028235e38;
 #pragma unroll
         for (int j = 0; j < PACKS; j++)
             if (live && lane + j * GROUP < npack) {
@@ -214,6 +228,10 @@ __global__ void __launch_bounds__(kBlock) softmaxRowRegKernel(const T *x, T *z, 
             }
         mx = teamAll<MaxMerge<C>, GROUP>(mx, smem);
         C sum = (C)0;
+        if (hasEdge) {
+            edge = toCompute(fromCompute<T>(m::exp_(edge - mx)));  // rounded to T like the cached ones
+            sum = edge;
+        }
 #pragma unroll
         for (int j = 0; j < PACKS; j++)
             if (live && lane + j * GROUP < npack) {
@@ -234,6 +252,7 @@ __global__ void __launch_bounds__(kBlock) softmaxRowRegKernel(const T *x, T *z, 
                 for (int e = 0; e < N; e++) o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(toCompute(cache[j].v[e]), sum));
                 storePack(zr + lane + j * GROUP, o);
             }
+        if (hasEdge) zrow[edgeAt] = fromCompute<T>(softmaxFinish<MODE, C>(edge, sum));
     }
 }
 
@@ -326,8 +345,14 @@ template <typename T> static bool aligned16(const T *p) { return (reinterpret_ca
 
 template <typename T, int MODE, int GROUP, int PACKS> void runRowReg(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
     int grid = gridFor(pl.numRows, kBlock / GROUP, kMaxGrid);
-    hipLaunchKernelGGL((softmaxRowRegKernel<T, MODE, GROUP, PACKS>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows,
-                       pl.length / Pack<T>::N, pl.xRow, pl.zRow);
+    constexpr int N = Pack<T>::N;
+    const bool whole = aligned16(x) && aligned16(z) && pl.length % N == 0 && (pl.numRows == 1 || (pl.xRow % N == 0 && pl.zRow % N == 0));
+    if (whole)
+        hipLaunchKernelGGL((softmaxRowRegKernel<T, MODE, GROUP, PACKS, false>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows,
+                           pl.length, pl.xRow, pl.zRow);
+    else
+        hipLaunchKernelGGL((softmaxRowRegKernel<T, MODE, GROUP, PACKS, true>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows,
+                           pl.length, pl.xRow, pl.zRow);
 }
 template <typename T, int MODE, int PACKS> void runColReg(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
     const Long rowsPerBlock = (Long)kColRowLanes * Pack<T>::N;
@@ -343,11 +368,13 @@ template <typename T> SoftmaxRoute softmaxRoute(const T *x, const T *z, const So
     // vectors a thread of the neighbouring-rows kernel may hold: a half vector unpacks to eight float maxima and
     // sums, which leaves room for fewer of them
     constexpr int kColPacks = sizeof(T) == 2 ? 8 : 16;
-    if (!(aligned16(x) && aligned16(z))) return SM_PASSES;
-    // contiguous rows whose vectors are aligned in every row, up to 16 vectors for each of 256 lanes
-    if (pl.xEl == 1 && pl.zEl == 1 && pl.length % N == 0 && pl.length >= 16 * N &&
-        (pl.numRows == 1 || (pl.xRow % N == 0 && pl.zRow % N == 0)) && pl.length / N <= 256 * 16)
+    // contiguous rows of up to 16 vectors for each of 256 lanes; x and z misaligned alike in every row (equal distance
+    // of the bases and of the row pitches from a 16-byte boundary), so that one row's aligned vectors are the other's
+    const uintptr_t xa = reinterpret_cast<uintptr_t>(x), za = reinterpret_cast<uintptr_t>(z);
+    if (pl.xEl == 1 && pl.zEl == 1 && pl.length >= 16 * N && xa % sizeof(T) == 0 && (xa & 15) == (za & 15) &&
+        (pl.numRows == 1 || ((pl.xRow - pl.zRow) * (Long)sizeof(T)) % 16 == 0) && (pl.length + N - 1) / N + 1 <= 256 * 16)
         return SM_ROW_REGISTERS;
+    if (!(aligned16(x) && aligned16(z))) return SM_PASSES;
     // an f-order matrix whose column stride keeps the row vectors aligned
     if (pl.xRow == 1 && pl.zRow == 1 && pl.numRows % N == 0 && pl.xEl % N == 0 && pl.zEl % N == 0 && pl.numRows >= kWave &&
         pl.length <= (Long)kColCols * kColPacks && (Long)((pl.numRows + 8 * N - 1) / (8 * N)) <= kMaxGrid / 4)  // blocks of 1024 threads
@@ -361,7 +388,7 @@ template <typename T, int MODE> void runSoftmax(hipStream_t s, const T *x, T *z,
     constexpr int kColPacks = sizeof(T) == 2 ? 8 : 16;
     const SoftmaxRoute route = softmaxRoute<T>(x, z, pl);
     if (route == SM_ROW_REGISTERS) {
-        const Long npack = pl.length / N;
+        const Long npack = (pl.length + N - 1) / N;  // at most this many aligned vectors in a row
         if (npack <= 16 * 2) runRowReg<T, MODE, 16, 2>(s, x, z, pl);
         else if (npack <= 64 * 2) runRowReg<T, MODE, 64, 2>(s, x, z, pl);
         else if (npack <= 64 * 8) runRowReg<T, MODE, 64, 8>(s, x, z, pl);
