@@ -88,29 +88,42 @@ __device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc
     if ((addr & (sizeof(T) - 1)) == 0) head = (Long)(((16 - (addr & 15)) & 15) / sizeof(T));
     else head = n;  // cannot be vectorised
     if (head > n) head = n;
-    for (Long i = lane; i < head; i += lanes) { pol.accumulate(acc, toCompute(p[i]), base + i); pol.checkpoint(acc); }
     const Long nvec = (n - head) / VEC;
+    // The elements before the first and after the last aligned vector (fewer than 2 VEC when the run can be vectorised at
+    // all): one per lane, requested before the vectors so that a run costs one round trip to memory, not three.
+    const Long tail0 = head + nvec * VEC, edges = head + (n - tail0);
+    const bool oneEach = edges <= lanes;
+    const bool hasEdge = oneEach && lane < edges;
+    const Long edgeAt = lane < head ? lane : tail0 + (lane - head);
+    T edge;
+    if (hasEdge) edge = p[edgeAt];
+    if (!oneEach) {
+        for (Long i = lane; i < head; i += lanes) { pol.accumulate(acc, toCompute(p[i]), base + i); pol.checkpoint(acc); }
+    }
     const Pack<T> *pv = reinterpret_cast<const Pack<T> *>(p + head);
     Long v = lane;
-    // four independent 16-byte loads in flight per lane, then the arithmetic
-    for (; v + 3 * (Long)lanes < nvec; v += 4 * (Long)lanes) {
+    // Four independent 16-byte loads in flight per lane, then the arithmetic.  Each of the four is guarded on its own: a
+    // lane whose last batch is short still runs it with the rest of its wave (an all-or-nothing batch sent such lanes
+    // through a second, vector-by-vector loop that the whole wave had to sit through; a separate unguarded copy of the
+    // batch for the full ones measured slower again, for the code it adds).
+    for (; v < nvec; v += 4 * (Long)lanes) {
         Pack<T> pk[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++) pk[u] = loadPack(pv + v + u * (Long)lanes);
+        for (int u = 0; u < 4; u++)
+            if (v + u * (Long)lanes < nvec) pk[u] = loadPack(pv + v + u * (Long)lanes);
 #pragma unroll
         for (int u = 0; u < 4; u++) {
+            if (v + u * (Long)lanes < nvec) {
 #pragma unroll
-            for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[u].v[e]), base + head + (v + u * (Long)lanes) * VEC + e);
-            pol.checkpoint(acc);
+                for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[u].v[e]), base + head + (v + u * (Long)lanes) * VEC + e);
+                pol.checkpoint(acc);
+            }
         }
     }
-    for (; v < nvec; v += lanes) {
-        Pack<T> pk = loadPack(pv + v);
-#pragma unroll
-        for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk.v[e]), base + head + v * VEC + e);
-        pol.checkpoint(acc);
+    if (hasEdge) { pol.accumulate(acc, toCompute(edge), base + edgeAt); pol.checkpoint(acc); }
+    if (!oneEach) {
+        for (Long i = tail0 + lane; i < n; i += lanes) { pol.accumulate(acc, toCompute(p[i]), base + i); pol.checkpoint(acc); }
     }
-    for (Long i = head + nvec * VEC + lane; i < n; i += lanes) { pol.accumulate(acc, toCompute(p[i]), base + i); pol.checkpoint(acc); }
 }
 
 template <class Pol, int GROUP>
