@@ -34,6 +34,8 @@ struct BroadcastPlan {
     bool consecutive = false;    // ROW only: TAD r starts at r * tadLength in x and in z (rows of a dense c-order array)
     bool denseAlike = false;     // ROW / COL: x and z are dense arrays of one layout, y is contiguous: memory position i of
                                  // either takes y[(i / tadEws) % tadLength]
+    Long flatInner = 0, flatExtent = 0;  // per-TAD scalars over dense x and z of one layout: memory position i takes
+                                         // scalars[(i / flatInner) % flatExtent]; 0 = not applicable
 };
 template <typename T>
 bool launchBroadcast(hipStream_t stream, int opNum, const T *x, const T *y, T *z, const BroadcastPlan &plan);

@@ -266,6 +266,18 @@ void scalarAlongDimension(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z
         return;
     }
     pl.kind = pl.tadEws == 1 ? BroadcastPlan::ROW : BroadcastPlan::COL;
+    // Dense x, z laid out like it, and TADs whose numbering follows memory order: the arrays can be walked as plain
+    // vectors, the TAD index falling out of the position (rows of a c-order array: i / tadLength; its columns, or whatever
+    // lies along its leading dimension: i % numTads).  For f-order arrays that holds in two dimensions only (the
+    // reference numbers TADs in C order over the remaining dimensions).
+    const Long *hz = reinterpret_cast<const Long *>(slotOf(extra, X_HOST_Z_SHAPE));
+    const bool zLikeX = devZOff == nullptr || (hz != nullptr && siRank(hz) == siRank(hx) &&
+                                               std::memcmp(hx, hz, sizeof(Long) * siLength(siRank(hx))) == 0);
+    const bool numbered = isDense(hx, 'c') || (siRank(hx) <= 2 && isDense(hx, 'f'));
+    if (zLikeX && numbered && tx.numTads * tx.tadLength == siNumel(hx)) {
+        if (pl.kind == BroadcastPlan::ROW) { pl.flatInner = pl.tadLength; pl.flatExtent = pl.numTads; }
+        else if (pl.tadEws == pl.numTads) { pl.flatInner = 1; pl.flatExtent = pl.numTads; }
+    }
     if (!launchScalarTad<T>(s, opNum, x, scalars, z, params, pl)) { reportUnknownOp("scalar", opNum); return; }
     checkLaunch("execScalar(dimension)", s);
 }

@@ -30,6 +30,13 @@ template <typename T> struct ScalarTadBody {
             typedef ScalarTad3F<KIND> F;
             if (pl.numTads <= 0 || pl.tadLength <= 0) return true;
             Params<T> p{extra};
+            if (pl.flatInner > 0 && pl.flatInner < 0xffffffffLL && pl.flatExtent < 0xffffffffLL &&
+                (((uintptr_t)x | (uintptr_t)z) & 15) == 0) {
+                const Long n = pl.numTads * pl.tadLength;
+                hipLaunchKernelGGL((bcFlatInnerKernel<T, F>), dim3(gridFor(n / Pack<T>::N + 1, kBlock, F::tables ? kGridCap : kMaxGrid)),
+                                   dim3(kBlock), 0, s, x, scalars, z, n, pl.flatInner, pl.flatExtent, p);
+                return true;
+            }
             if (pl.kind == BroadcastPlan::ROW) {
                 constexpr int VEC = Pack<T>::N;
                 Long vecsPerTad = (pl.tadLength + VEC - 1) / VEC;

@@ -261,7 +261,7 @@ def test_scalar_family(gpu, cpu):
     fi, ci = harness.shape_info([100, 200], "f"), harness.shape_info([100, 200], "c")
     assert np.array_equal(gpu.scalar(1, x, fi, ci, 0.37), cpu.scalar(1, x, fi, ci, 0.37))
     # one scalar per TAD: contiguous rows, strided columns, both orders, with and without the caller's TAD tables
-    for rows, cols in ((300, 150), (64, 1024), (5, 7)):
+    for rows, cols in ((300, 150), (64, 1024), (5, 7), (257, 1023), (1021, 33)):  # also odd lengths and counts
         m = rs.uniform(1.2, 9, rows * cols).astype(np.float32)
         for order in ("c", "f"):
             mi = harness.shape_info([rows, cols], order)
@@ -271,6 +271,14 @@ def test_scalar_family(gpu, cpu):
                     want = cpu.scalar_tad(op, m, mi, sc, None, dims)
                     assert np.array_equal(gpu.scalar_tad(op, m, mi, sc, None, dims), want), (rows, cols, order, dims, op)
                 assert np.array_equal(gpu.scalar_tad(0, m, mi, sc, None, dims, pass_tads=False), cpu.scalar_tad(0, m, mi, sc, None, dims))
+    # rank 3: TADs over the trailing, the leading and the middle dimension, both orders (the TAD numbering follows memory
+    # order only for some of them; the others take the kernels that read the offset tables)
+    for order in ("c", "f"):
+        mi = harness.shape_info([6, 5, 28], order)
+        m = rs.uniform(1.2, 9, 6 * 5 * 28).astype(np.float32)
+        for dims in ([2], [0], [1]):
+            sc = rs.uniform(1.2, 5, 840 // [6, 5, 28][dims[0]]).astype(np.float32)
+            assert np.array_equal(gpu.scalar_tad(0, m, mi, sc, None, dims), cpu.scalar_tad(0, m, mi, sc, None, dims)), (order, dims)
     # fp16: the scalar is rounded to fp16 before use; fp64
     xh = rs.uniform(1, 4, 4096).astype(np.float16)
     hi = shape_info_np([1, 4096])
