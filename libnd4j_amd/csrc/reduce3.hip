@@ -100,11 +100,18 @@ __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, 
             const Long xi = pl.xDiv == 1 ? r : r / pl.xDiv, yi = r < pl.yMod ? r : r % pl.yMod;
             const T *xr = x + (pl.xOffsets != nullptr ? pl.xOffsets[xi] : 0);
             const T *yr = y + (pl.yOffsets != nullptr ? pl.yOffsets[yi] : 0);
-            const bool vec = pl.contiguous && ((reinterpret_cast<uintptr_t>(xr + f0) | reinterpret_cast<uintptr_t>(yr + f0)) & 15) == 0;
+            // vectors wherever the two runs are misaligned alike (rows of odd length: every row starts elsewhere, but at
+            // the same place in x and in y): the elements before the first and after the last aligned vector go singly
+            const uintptr_t xa = reinterpret_cast<uintptr_t>(xr + f0), ya = reinterpret_cast<uintptr_t>(yr + f0);
+            const bool vec = pl.contiguous && ((xa ^ ya) & 15) == 0 && xa % sizeof(T) == 0;
             if (vec) {
-                const Long nvec = (f1 - f0) / VEC;
-                const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(xr + f0);
-                const Pack<T> *yv = reinterpret_cast<const Pack<T> *>(yr + f0);
+                Long head = (Long)(((16 - (xa & 15)) & 15) / sizeof(T));
+                if (head > f1 - f0) head = f1 - f0;
+                const Long nvec = (f1 - f0 - head) / VEC;
+                const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(xr + f0 + head);
+                const Pack<T> *yv = reinterpret_cast<const Pack<T> *>(yr + f0 + head);
+                for (Long f = f0 + lane; f < f0 + head; f += GROUP)
+                    Reduce3Op<C, OP>::accumulate(acc, toCompute(xr[f]), toCompute(yr[f]), eps);
                 Long v = lane;
                 // four vectors of each operand requested before the first is used
                 for (; v + 3 * GROUP < nvec; v += 4 * GROUP) {
@@ -125,7 +132,7 @@ __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, 
 #pragma unroll
                     for (int e = 0; e < VEC; e++) Reduce3Op<C, OP>::accumulate(acc, toCompute(a0.v[e]), toCompute(b0.v[e]), eps);
                 }
-                for (Long f = f0 + nvec * VEC + lane; f < f1; f += GROUP)
+                for (Long f = f0 + head + nvec * VEC + lane; f < f1; f += GROUP)
                     Reduce3Op<C, OP>::accumulate(acc, toCompute(xr[f]), toCompute(yr[f]), eps);
             } else if (pl.contiguous) {
                 for (Long f = f0 + lane; f < f1; f += GROUP)
