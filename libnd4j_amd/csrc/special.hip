@@ -372,7 +372,7 @@ template <typename T> SoftmaxRoute softmaxRoute(const T *x, const T *z, const So
     // of the bases and of the row pitches from a 16-byte boundary), so that one row's aligned vectors are the other's
     const uintptr_t xa = reinterpret_cast<uintptr_t>(x), za = reinterpret_cast<uintptr_t>(z);
     if (pl.xEl == 1 && pl.zEl == 1 && pl.length >= 16 * N && xa % sizeof(T) == 0 && (xa & 15) == (za & 15) &&
-        (pl.numRows == 1 || ((pl.xRow - pl.zRow) * (Long)sizeof(T)) % 16 == 0) && (pl.length + N - 1) / N + 1 <= 256 * 16)
+        (pl.numRows == 1 || ((pl.xRow - pl.zRow) * (Long)sizeof(T)) % 16 == 0) && pl.length / N <= 256 * 16)
         return SM_ROW_REGISTERS;
     if (!(aligned16(x) && aligned16(z))) return SM_PASSES;
     // an f-order matrix whose column stride keeps the row vectors aligned
@@ -388,11 +388,12 @@ template <typename T, int MODE> void runSoftmax(hipStream_t s, const T *x, T *z,
     constexpr int kColPacks = sizeof(T) == 2 ? 8 : 16;
     const SoftmaxRoute route = softmaxRoute<T>(x, z, pl);
     if (route == SM_ROW_REGISTERS) {
-        const Long npack = (pl.length + N - 1) / N;  // at most this many aligned vectors in a row
+        const Long npack = pl.length / N;  // at most this many aligned vectors in a row (fewer when it starts off a boundary)
         if (npack <= 16 * 2) runRowReg<T, MODE, 16, 2>(s, x, z, pl);
         else if (npack <= 64 * 2) runRowReg<T, MODE, 64, 2>(s, x, z, pl);
         else if (npack <= 64 * 8) runRowReg<T, MODE, 64, 8>(s, x, z, pl);
         else if (npack <= 256 * 4) runRowReg<T, MODE, kBlock, 4>(s, x, z, pl);
+        else if (npack <= 256 * 8) runRowReg<T, MODE, kBlock, 8>(s, x, z, pl);
         else runRowReg<T, MODE, kBlock, 16>(s, x, z, pl);
         return;
     }
