@@ -479,6 +479,103 @@ inline void launchStrided(hipStream_t s, const T *x, Long xs, const T *y, Long y
     hipLaunchKernelGGL((ewGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, xm, two ? y : x, ym, z, zm, p, n);
 }
 
+// Dense matrices in mixed orders (z = op(x, y) with x or y laid out the other way round than z: a + b.transpose()): in
+// z's frame z[r * cols + c]; an operand of z's order is read where z is written, a transposed one, t[r + c * rows], goes
+// through an LDS tile - read with the lanes along r, where it is contiguous, used with the lanes along c.  Tiles and
+// block order as in the transposing copy (32 x 64, neighbouring blocks on neighbouring column tiles); ACC elements per
+// access (a 16-byte vector, or 1 when shapes or alignment do not allow vectors).
+template <typename T, typename F, int ACC, bool XT, bool YT>
+__global__ void __launch_bounds__(kBlock) ewMixedOrderKernel(const T *x, const T *y, T *z, Long rows, Long cols, Params<T> p) {
+    typedef typename Compute<T>::type C;
+    constexpr int TR = 32, TC = 64;
+    constexpr bool two = F::nin == 2;
+    __shared__ T tileX[XT ? TC : 1][TR + 1];
+    __shared__ T tileY[(two && YT) ? TC : 1][TR + 1];
+    if (F::tables) lm::loadTables();
+    constexpr int LANES_R = TR / ACC, STEP_R = kBlock / LANES_R;
+    constexpr int LANES_C = TC / ACC, STEP_C = kBlock / LANES_C;
+    const int rFast = (threadIdx.x % LANES_R) * ACC, rSlow = threadIdx.x / LANES_R;
+    const int cFast = (threadIdx.x % LANES_C) * ACC, cSlow = threadIdx.x / LANES_C;
+    const Long colTiles = (cols + TC - 1) / TC, rowTiles = (rows + TR - 1) / TR;
+    for (Long tile_ = blockIdx.x; tile_ < colTiles * rowTiles; tile_ += gridDim.x) {
+        const Long rt = tile_ / colTiles, ct = tile_ - rt * colTiles;
+        const Long r0 = rt * TR, c0 = ct * TC;
+        if (XT || (two && YT)) {
+#pragma unroll
+            for (int lc = rSlow; lc < TC; lc += STEP_R) {
+                const Long r = r0 + rFast, c = c0 + lc;
+                if (r < rows && c < cols) {
+                    if (XT) {
+                        if (ACC > 1) {
+                            const Pack<T> v = loadPack(reinterpret_cast<const Pack<T> *>(x + r + c * rows));
+#pragma unroll
+                            for (int k = 0; k < ACC; k++) tileX[lc][rFast + k] = v.v[k % Pack<T>::N];
+                        } else {
+                            tileX[lc][rFast] = x[r + c * rows];
+                        }
+                    }
+                    if (two && YT) {
+                        if (ACC > 1) {
+                            const Pack<T> v = loadPack(reinterpret_cast<const Pack<T> *>(y + r + c * rows));
+#pragma unroll
+                            for (int k = 0; k < ACC; k++) tileY[lc][rFast + k] = v.v[k % Pack<T>::N];
+                        } else {
+                            tileY[lc][rFast] = y[r + c * rows];
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int lr = cSlow; lr < TR; lr += STEP_C) {
+            const Long r = r0 + lr, c = c0 + cFast;
+            if (r < rows && c < cols) {
+                const Long at = r * cols + c;
+                if (ACC > 1) {
+                    Pack<T> xa, ya, o;
+                    if (!XT) xa = loadPack(reinterpret_cast<const Pack<T> *>(x + at));
+                    if (two && !YT) ya = loadPack(reinterpret_cast<const Pack<T> *>(y + at));
+#pragma unroll
+                    for (int k = 0; k < ACC; k++) {
+                        const C a = toCompute(XT ? tileX[cFast + k][lr] : xa.v[k % Pack<T>::N]);
+                        const C b = two ? toCompute(YT ? tileY[cFast + k][lr] : ya.v[k % Pack<T>::N]) : (C)0;
+                        o.v[k % Pack<T>::N] = fromCompute<T>(F::template apply<C>(a, b, p));
+                    }
+                    storePack(reinterpret_cast<Pack<T> *>(z + at), o);
+                } else {
+                    const C a = toCompute(XT ? tileX[cFast][lr] : x[at]);
+                    const C b = two ? toCompute(YT ? tileY[cFast][lr] : y[at]) : (C)0;
+                    z[at] = fromCompute<T>(F::template apply<C>(a, b, p));
+                }
+            }
+        }
+        if (XT || (two && YT)) __syncthreads();
+    }
+}
+
+// 0: contiguous along dimension 1 (c-like), 1: along dimension 0 (f-like), -1: neither, for a rank-2 map
+inline int denseClass2D(const DimMap &m) {
+    if (m.rank != 2) return -1;
+    if (m.stride[1] == 1 && m.stride[0] == (Long)m.shape[1]) return 0;
+    if (m.stride[0] == 1 && m.stride[1] == (Long)m.shape[0]) return 1;
+    return -1;
+}
+
+template <typename T, typename F, int ACC>
+inline void launchMixedOrder(hipStream_t s, const T *x, const T *y, T *z, Long rows, Long cols, bool xt, bool yt, Params<T> p) {
+    const Long tiles = ((rows + 31) / 32) * ((cols + 63) / 64);
+    const dim3 grid((unsigned)(tiles < kMaxGrid ? tiles : kMaxGrid));
+    if constexpr (F::nin == 2) {
+        if (xt && yt) hipLaunchKernelGGL((ewMixedOrderKernel<T, F, ACC, true, true>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
+        else if (xt) hipLaunchKernelGGL((ewMixedOrderKernel<T, F, ACC, true, false>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
+        else hipLaunchKernelGGL((ewMixedOrderKernel<T, F, ACC, false, true>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
+    } else {
+        (void)yt;  // one input: it is the transposed one
+        hipLaunchKernelGGL((ewMixedOrderKernel<T, F, ACC, true, false>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
+    }
+}
+
 template <typename T, typename F>
 inline void launchGeneral(hipStream_t s, const T *x, const DimMap &xm, const T *y, const DimMap &ym, T *z,
                           const DimMap &zm, const T *extra, Long n, typename Compute<T>::type scalar = 0) {
@@ -486,6 +583,22 @@ inline void launchGeneral(hipStream_t s, const T *x, const DimMap &xm, const T *
     const bool two = F::nin == 2;
     if (xm.rank == 1 && zm.rank == 1 && (!two || ym.rank == 1)) {
         launchStrided<T, F>(s, x, xm.stride[0], y, two ? ym.stride[0] : 0, z, zm.stride[0], extra, n, scalar);
+        return;
+    }
+    // dense matrices of one shape whose orders differ
+    const int zc = denseClass2D(zm), xc = denseClass2D(xm), yc = two ? denseClass2D(ym) : zc;
+    if (zc >= 0 && xc >= 0 && yc >= 0 && xm.shape[0] == zm.shape[0] && xm.shape[1] == zm.shape[1] &&
+        (!two || (ym.shape[0] == zm.shape[0] && ym.shape[1] == zm.shape[1])) && (xc != zc || yc != zc) &&
+        (Long)zm.shape[0] * zm.shape[1] == n) {
+        // z's frame: c runs along z's contiguous dimension
+        const Long cols = zm.shape[zc == 0 ? 1 : 0], rows = zm.shape[zc == 0 ? 0 : 1];
+        Params<T> p{extra};
+        p.scalar = scalar;
+        constexpr int N = Pack<T>::N;
+        const bool vec = rows % N == 0 && cols % N == 0 &&
+                         ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(z) | (two ? reinterpret_cast<uintptr_t>(y) : 0)) & 15) == 0;
+        if (vec) launchMixedOrder<T, F, N>(s, x, two ? y : x, z, rows, cols, xc != zc, two && yc != zc, p);
+        else launchMixedOrder<T, F, 1>(s, x, two ? y : x, z, rows, cols, xc != zc, two && yc != zc, p);
         return;
     }
     Params<T> p{extra};

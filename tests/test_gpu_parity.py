@@ -764,3 +764,30 @@ def test_random_views_against_the_cpu_checker(gpu, cpu):
     without the caller's TAD tables.  Fixed seed: the same few thousand calls every run."""
     done = checks.check_random_views(gpu, cpu, seed=7, cases=4000)
     assert len(done) == 7 and min(done.values()) > 200
+
+
+def test_dense_matrices_in_mixed_orders(gpu):
+    """z = op(x, y) over dense matrices whose orders differ (a + b.transpose()): every combination of c and f for x, y
+    and z, shapes that allow 16-byte accesses and shapes that do not, all three data types.  Add and Abs are single IEEE
+    operations, so numpy gives the expected bits."""
+    rs = np.random.RandomState(77)
+    for dt in (np.float32, np.float16, np.float64):
+        for shape in ([128, 256], [96, 40], [33, 65], [64, 7]):
+            n = shape[0] * shape[1]
+            a, b = rs.randn(*shape).astype(dt), rs.randn(*shape).astype(dt)
+            for ox, oy, oz in itertools.product("cf", repeat=3):
+                if ox == oy == oz:
+                    continue
+                xi, yi, zi = (harness.shape_info(shape, o) for o in (ox, oy, oz))
+                x = np.ascontiguousarray(a if ox == "c" else a.T).ravel()
+                y = np.ascontiguousarray(b if oy == "c" else b.T).ravel()
+                got = gpu.pairwise(0, x, xi, y, yi, zi).reshape(shape, order="F" if oz == "f" else "C")
+                assert np.array_equal(got, a + b), (np.dtype(dt).name, shape, ox, oy, oz)
+            for ox, oz in (("c", "f"), ("f", "c")):
+                xi, zi = harness.shape_info(shape, ox), harness.shape_info(shape, oz)
+                x = np.ascontiguousarray(a if ox == "c" else a.T).ravel()
+                got = gpu.transform(0, x, xi, zi).reshape(shape, order="F" if oz == "f" else "C")
+                assert np.array_equal(got, np.abs(a)), (np.dtype(dt).name, shape, ox, oz)
+                got = gpu.scalar(0, x, xi, zi, 2.0).reshape(shape, order="F" if oz == "f" else "C")
+                assert np.array_equal(got, (a.astype(np.float32) + np.float32(2.0)).astype(dt) if dt == np.float16 else a + dt(2.0)), (
+                    "scalar", np.dtype(dt).name, shape, ox, oz)
