@@ -191,15 +191,16 @@ template <class Merge, int GROUP, typename C> __device__ __forceinline__ C teamA
 // after its last aligned vector (fewer than 2 N, the "edge") are kept one per lane by the team's first lanes.  x and z
 // must be misaligned alike in every row (the host checks it).
 // (EDGES false: the host has seen that every row starts aligned and holds whole vectors, and the edge code folds away.)
-template <typename T, int MODE, int GROUP, int PACKS, bool EDGES>
-__global__ void __launch_bounds__(kBlock) softmaxRowRegKernel(const T *x, T *z, Long numRows, Long length, Long xRow, Long zRow) {
+// (BLOCK: threads of a block, a multiple of GROUP; the 1024-thread blocks serve the longest rows, one team a block.)
+template <typename T, int MODE, int GROUP, int PACKS, bool EDGES, int BLOCK = kBlock>
+__global__ void __launch_bounds__(BLOCK) softmaxRowRegKernel(const T *x, T *z, Long numRows, Long length, Long xRow, Long zRow) {
     lm::loadTables();
     typedef typename Compute<T>::type C;
     constexpr int N = Pack<T>::N;
-    constexpr int GROUPS = kBlock / GROUP;
-    __shared__ C smem[kBlock / kWave];
+    constexpr int GROUPS = BLOCK / GROUP;
+    __shared__ C smem[BLOCK / kWave];
     const int g = threadIdx.x / GROUP, lane = threadIdx.x % GROUP;
-    // GROUP == kBlock: every thread of the block runs the same trip count, so teamAll may synchronise
+    // GROUP == BLOCK: every thread of the block runs the same trip count, so teamAll may synchronise
     for (Long r0 = (Long)blockIdx.x * GROUPS; r0 < numRows; r0 += (Long)gridDim.x * GROUPS) {
         const Long r = r0 + g;
         const bool live = r < numRows;
@@ -343,15 +344,15 @@ __global__ void __launch_bounds__(kColBlock) softmaxColRegKernel(const T *x, T *
 
 template <typename T> static bool aligned16(const T *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-template <typename T, int MODE, int GROUP, int PACKS> void runRowReg(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
-    int grid = gridFor(pl.numRows, kBlock / GROUP, kMaxGrid);
+template <typename T, int MODE, int GROUP, int PACKS, int BLOCK = kBlock> void runRowReg(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
+    int grid = gridFor(pl.numRows, BLOCK / GROUP, kMaxGrid / (BLOCK / kBlock));
     constexpr int N = Pack<T>::N;
     const bool whole = aligned16(x) && aligned16(z) && pl.length % N == 0 && (pl.numRows == 1 || (pl.xRow % N == 0 && pl.zRow % N == 0));
     if (whole)
-        hipLaunchKernelGGL((softmaxRowRegKernel<T, MODE, GROUP, PACKS, false>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows,
+        hipLaunchKernelGGL((softmaxRowRegKernel<T, MODE, GROUP, PACKS, false, BLOCK>), dim3(grid), dim3(BLOCK), 0, s, x, z, pl.numRows,
                            pl.length, pl.xRow, pl.zRow);
     else
-        hipLaunchKernelGGL((softmaxRowRegKernel<T, MODE, GROUP, PACKS, true>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows,
+        hipLaunchKernelGGL((softmaxRowRegKernel<T, MODE, GROUP, PACKS, true, BLOCK>), dim3(grid), dim3(BLOCK), 0, s, x, z, pl.numRows,
                            pl.length, pl.xRow, pl.zRow);
 }
 template <typename T, int MODE, int PACKS> void runColReg(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
@@ -361,6 +362,16 @@ template <typename T, int MODE, int PACKS> void runColReg(hipStream_t s, const T
                        pl.zEl);
 }
 
+// The widest team of the rows-in-registers kernel, and the vectors each of its lanes keeps: a 1024-thread block leaves
+// a lane 128 registers, which hold 16 vectors of floats or 8 of doubles.  Halves (widened to float while they are
+// worked on) would spill there, so their longest rows stay with 256 lanes of 16 vectors.
+// One such block works on a row alone, so the wide team is for matrices with enough rows to occupy a good part of
+// the chip; fewer, longer rows are spread over many blocks by the kernels that pass over the data more than once.
+static constexpr int kRowRegLanes = 1024, kWideRowsFrom = 128;
+template <typename T> struct WideRow {
+    static constexpr int PACKS = sizeof(T) == 4 ? 16 : sizeof(T) == 8 ? 8 : 0;
+    static constexpr Long kMostPacks = PACKS ? (Long)kRowRegLanes * PACKS : 256 * 16;  // vectors of the longest row kept in registers
+};
 // Which kind of kernel a softmax call gets: rows in registers, neighbouring rows in registers, or three passes.
 enum SoftmaxRoute { SM_ROW_REGISTERS, SM_COL_REGISTERS, SM_PASSES };
 template <typename T> SoftmaxRoute softmaxRoute(const T *x, const T *z, const SoftmaxPlan &pl) {
@@ -368,11 +379,11 @@ template <typename T> SoftmaxRoute softmaxRoute(const T *x, const T *z, const So
     // vectors a thread of the neighbouring-rows kernel may hold: a half vector unpacks to eight float maxima and
     // sums, which leaves room for fewer of them
     constexpr int kColPacks = sizeof(T) == 2 ? 8 : 16;
-    // contiguous rows of up to 16 vectors for each of 256 lanes; x and z misaligned alike in every row (equal distance
+    // contiguous rows of up to WideRow::kMostPacks vectors; x and z misaligned alike in every row (equal distance
     // of the bases and of the row pitches from a 16-byte boundary), so that one row's aligned vectors are the other's
     const uintptr_t xa = reinterpret_cast<uintptr_t>(x), za = reinterpret_cast<uintptr_t>(z);
     if (pl.xEl == 1 && pl.zEl == 1 && pl.length >= 16 * N && xa % sizeof(T) == 0 && (xa & 15) == (za & 15) &&
-        (pl.numRows == 1 || ((pl.xRow - pl.zRow) * (Long)sizeof(T)) % 16 == 0) && pl.length / N <= 256 * 16)
+        (pl.numRows == 1 || ((pl.xRow - pl.zRow) * (Long)sizeof(T)) % 16 == 0) && pl.length / N <= (pl.numRows >= kWideRowsFrom ? WideRow<T>::kMostPacks : 256 * 16))
         return SM_ROW_REGISTERS;
     if (!(aligned16(x) && aligned16(z))) return SM_PASSES;
     // an f-order matrix whose column stride keeps the row vectors aligned
@@ -394,7 +405,8 @@ template <typename T, int MODE> void runSoftmax(hipStream_t s, const T *x, T *z,
         else if (npack <= 64 * 8) runRowReg<T, MODE, 64, 8>(s, x, z, pl);
         else if (npack <= 256 * 4) runRowReg<T, MODE, kBlock, 4>(s, x, z, pl);
         else if (npack <= 256 * 8) runRowReg<T, MODE, kBlock, 8>(s, x, z, pl);
-        else runRowReg<T, MODE, kBlock, 16>(s, x, z, pl);
+        else if (npack <= 256 * 16) runRowReg<T, MODE, kBlock, 16>(s, x, z, pl);
+        else if constexpr (WideRow<T>::PACKS > 0) runRowReg<T, MODE, kRowRegLanes, WideRow<T>::PACKS, kRowRegLanes>(s, x, z, pl);
         return;
     }
     if (route == SM_COL_REGISTERS) {

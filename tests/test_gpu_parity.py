@@ -422,7 +422,11 @@ def test_special_transforms(gpu, cpu):
                          ([64, 2052], "f"), ([8, 8], "c"),
                          # rows too long for registers: maxima and sums from the reduction kernels (sliced from 16384 on)
                          ([32, 50257], "c"), ([4, 100000], "c"), ([3, 20000], "c"), ([6, 9001], "c"), ([100000, 1], "c"),
-                         ([256, 4100], "f"), ([300, 2500], "f"), ([600, 16500], "c"), ([520, 4100], "c")):
+                         ([256, 4100], "f"), ([300, 2500], "f"), ([600, 16500], "c"), ([520, 4100], "c"),
+                         # many rows of 16385..65536 floats: one 1024-thread block keeps a row in registers
+                         # (from 128 rows on; fewer rows, or longer ones, go through the reduction kernels)
+                         ([128, 20000], "c"), ([130, 65536], "c"), ([129, 50001], "c"), ([128, 65537], "c"), ([128, 65540], "c"),
+                         ([127, 40000], "c")):
         n = int(np.prod(shape))
         xi = harness.shape_info(shape, order)
         x = rs.uniform(-6, 6, n).astype(np.float32)
@@ -447,7 +451,8 @@ def test_special_transforms(gpu, cpu):
     assert np.all(np.abs(got - truth) <= 2e-5 * truth)
     # half and double, row-major and column-major, short and long rows
     for shape, order in (([64, 96], "c"), ([5, 4000], "c"), ([3, 30000], "c"), ([128, 600], "f"), ([64, 1100], "f"),
-                         ([2, 70000], "c"), ([300, 4500], "f"), ([3, 100000], "c")):  # a half row sum beyond 65504 stays finite
+                         ([2, 70000], "c"), ([300, 4500], "f"), ([3, 100000], "c"),  # a half row sum beyond 65504 stays finite
+                         ([128, 12000], "c"), ([130, 16383], "c")):  # doubles: rows of 8193..16384 in 1024-thread blocks
         n = shape[0] * shape[1]
         od = "F" if order == "f" else "C"
         info = harness.shape_info(shape, order)
