@@ -218,6 +218,19 @@ Nd4jLong nd4j_amd_hostFetchCount(void);
  * hardware traffic counters are scaled */
 void nd4j_amd_copyKernel(Nd4jPointer *extraPointers, void *dst, const void *src, Nd4jLong bytes);
 
+/* ---- for callers that cannot allocate: no counterpart in the reference ------------------------------- */
+/* execReduceFloat over the whole array (no dimensions): result[0], a device pointer, receives what
+ * nd4j_execReduceFloatFull leaves there, bit for bit.  For callers that may not call hipMalloc while they run
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid allocation): this entry point
+ * allocates and frees nothing, reads nothing back and does not synchronise.  Its partial accumulators live in
+ * a 64 KiB device array inside the library, one copy per GPU, kept until the process ends and shared by every
+ * call on that GPU: calls that overlap on one GPU (two streams, two threads) race on it, so issue them one
+ * after the other.  The host copy of xShapeInfo must be in extraPointers[0] (or xShapeInfo itself a host
+ * pointer); extraPointers[1] is the stream.  Arrays of more than 2^36 elements, empty arrays, a missing host
+ * shapeInfo and unknown opNums are rejected: nd4j_lastError() says why and result is left untouched. */
+void nd4j_amd_execReduceFloatNoAlloc(Nd4jPointer *extraPointers, int opNum, float *x, Nd4jLong *xShapeInfo,
+                                     float *extraParams, float *result);
+
 #if defined(__GNUC__)
 #pragma GCC visibility pop
 #endif

@@ -270,6 +270,10 @@ float nd4j_amd_timerElapsedMs(Nd4jPointer start, Nd4jPointer stop) {
     return ms;
 }
 int nd4j_amd_timerDestroy(Nd4jPointer timer) { return hipEventDestroy(reinterpret_cast<hipEvent_t>(timer)) == hipSuccess ? 1 : 0; }
+void nd4j_amd_execReduceFloatNoAlloc(Nd4jPointer *extraPointers, int opNum, float *x, Nd4jLong *xShapeInfo, float *extraParams,
+                                     float *result) {
+    guardVoid([&] { nd4j_amd::reduceFloatNoAlloc(extraPointers, opNum, x, xShapeInfo, extraParams, result); });
+}
 Nd4jLong nd4j_amd_hostFetchCount(void) { return (Nd4jLong)nd4j_amd::hostFetchCount(); }
 void nd4j_amd_copyKernel(Nd4jPointer *extraPointers, void *dst, const void *src, Nd4jLong bytes) {
     guardVoid([&] {

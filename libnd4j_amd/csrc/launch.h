@@ -93,6 +93,12 @@ template <typename T>
 bool launchReduceScalar(hipStream_t stream, int opNum, const T *x, const T *extra, T *z, const FlatPlan &plan,
                         Workspace ws);
 
+// The whole-array reduction with its partial accumulators in a file-scope device array instead of a workspace: no
+// device memory is allocated or freed.  Calls that overlap on one GPU share (and race on) that array.
+// prepareNoAllocScratch looks the array's address up for the current device (the launch does so on its first call too).
+void prepareNoAllocScratch();
+bool launchReduceScalarNoAlloc(hipStream_t stream, int opNum, const float *x, const float *extra, float *z, const FlatPlan &plan);
+
 template <typename T>
 bool launchIndexReduceTad(hipStream_t stream, int opNum, const T *x, const T *extra, T *z, const TadPlan &plan,
                           Workspace ws);

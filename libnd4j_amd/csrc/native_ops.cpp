@@ -366,7 +366,12 @@ static int deviceIdOf(Nd4jPointer p) { return (int)(intptr_t)p; }
 
 void NativeOps::initializeDevicesAndFunctions() {
     int n = 0;
-    if (hipGetDeviceCount(&n) != hipSuccess) (void)hipGetLastError();
+    if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return; }
+    // the address of the no-allocation entry point's scratch array on the current device (other devices: looked up
+    // by the first call that runs on them)
+    if (n > 0) {
+        try { prepareNoAllocScratch(); } catch (const std::exception &) { (void)hipGetLastError(); }
+    }
 }
 
 Nd4jPointer NativeOps::mallocHost(Nd4jLong memorySize, int) {

@@ -7,6 +7,8 @@
 // extraPointers decoding follows blas/cuda/NativeOps.cu:2098-2139 and 1600-1643.
 #include <cstdio>
 #include <cstring>
+#include <stdexcept>
+#include <string>
 
 #include "../../include/NativeOps.h"
 #include "runtime.h"
@@ -604,6 +606,36 @@ INST(float16)
 INST(double)
 #undef INST
 
+}  // namespace nd4j_amd
+
+// ---- whole-array reduction that allocates nothing ---------------------------------------------------------
+// No counterpart in the reference.  Same result as execReduceFloat without dimensions (result[0] on the device), for
+// callers that may not allocate: the partial accumulators live in a file-scope device array (reduce.hip), the host
+// shapeInfo must be at hand (extraPointers[0], or a host pointer as xShapeInfo), nothing is read back and nothing is
+// synchronised.  Calls that overlap on one GPU race on the shared array.
+namespace nd4j_amd {
+static const Long kNoAllocMaxElements = (Long)1 << 36;  // 256 GiB of floats: beyond what one GPU's memory holds
+
+void reduceFloatNoAlloc(Nd4jPointer *extra, int opNum, float *x, Long *xInfo, float *params, float *z) {
+    hipStream_t s = streamOf(extra);
+    const Long *hx = reinterpret_cast<const Long *>(slotOf(extra, X_HOST_X_SHAPE));
+    if (hx == nullptr && xInfo != nullptr && !isDeviceMemory(xInfo)) hx = xInfo;
+    if (hx == nullptr)
+        throw std::invalid_argument("execReduceFloatNoAlloc: needs the host copy of xShapeInfo in extraPointers[0] "
+                                    "(a device shapeInfo would have to be read back)");
+    if (x == nullptr || z == nullptr) throw std::invalid_argument("execReduceFloatNoAlloc: null data pointer");
+    const Long rank = hx[0];
+    if (rank < 0 || rank > kMaxRank) throw std::invalid_argument("execReduceFloatNoAlloc: shapeInfo rank out of range");
+    const Long n = siNumel(hx);
+    if (n < 1) throw std::invalid_argument("execReduceFloatNoAlloc: empty array");
+    if (n > kNoAllocMaxElements)
+        throw std::invalid_argument("execReduceFloatNoAlloc: " + std::to_string(n) + " elements; at most 2^36 are accepted");
+    FlatPlan pl = flatAnyOrder(hx);
+    if (!launchReduceScalarNoAlloc(s, opNum, x, params, z, pl))
+        throw std::invalid_argument("execReduceFloatNoAlloc: unknown opNum " + std::to_string(opNum));
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) throw std::runtime_error(std::string("execReduceFloatNoAlloc: ") + hipGetErrorString(e));
+}
 }  // namespace nd4j_amd
 
 #define ND4J_REDUCE3_MEMBERS(SUFFIX, T, R)                                                                          \

@@ -3,10 +3,22 @@
 // functors: include/ops/ops.h:1534-2560 and include/ops/special_accumulation_ops.h:16-45; opNum table:
 // include/loops/legacy_ops.h:195-221.  Partial accumulators are merged with `update`, never `merge`,
 // exactly as both reference back ends do (cpu/reduce.cpp:258-260).
+#include <mutex>
+#include <stdexcept>
+#include <string>
+
 #include "launch.h"
 #include "reduce_engine.cuh"
 
 namespace nd4j_amd {
+
+// Scratch of the whole-array reduction that allocates nothing (launchReduceScalarNoAlloc below): the first 256 bytes
+// hold the maximum that LogSumExp's first pass leaves for its second, the rest the per-block partial accumulators.
+// Every GPU the library runs on holds its own copy of this array until the process ends.  Host code never uses the
+// array's name as an address: it asks for the array's address on the current device once, and passes that on.
+static constexpr size_t kNoAllocScratchBytes = 64 * 1024;
+static constexpr size_t kNoAllocPartialsOffset = 256;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 
 enum StartKind { START_ZERO, START_ONE, START_FIRST };
 
@@ -196,6 +208,46 @@ bool launchSoftmaxStats(hipStream_t s, const T *x, T *maxima, typename Compute<T
     pol.row = 0;
     runTadReduce(s, pol, x, maxima, plan, ws);
     return true;
+}
+
+// ---- the whole-array reduction over the static scratch ---------------------------------------------------
+namespace {
+constexpr int kScratchDevices = 64;
+std::mutex gScratchMutex;
+void *gScratchAddress[kScratchDevices] = {};
+
+// Address of `scratch` on the current device, looked up once per device.
+void *scratchOnCurrentDevice() {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) throw std::runtime_error(std::string("hipGetDevice: ") + hipGetErrorString(e));
+    if (dev < 0 || dev >= kScratchDevices) throw std::runtime_error("device index beyond the no-allocation scratch table");
+    std::lock_guard<std::mutex> lock(gScratchMutex);
+    if (gScratchAddress[dev] == nullptr) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            throw std::runtime_error(std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(e));
+        gScratchAddress[dev] = ptr;
+    }
+    return gScratchAddress[dev];
+}
+}  // namespace
+
+void prepareNoAllocScratch() { (void)scratchOnCurrentDevice(); }
+
+bool launchReduceScalarNoAlloc(hipStream_t s, int opNum, const float *x, const float *extra, float *z, const FlatPlan &plan) {
+    char *base = reinterpret_cast<char *>(scratchOnCurrentDevice());
+    Workspace ws;
+    ws.ptr = base + kNoAllocPartialsOffset;
+    ws.bytes = kNoAllocScratchBytes - kNoAllocPartialsOffset;
+    if (opNum == 19) {
+        // LogSumExp: the maximum first, then exp(x - maximum) summed (blas/cpu/NativeOpExcutioner.cpp:138-141)
+        float *maxSlot = reinterpret_cast<float *>(base);
+        if (!launchReduceScalar<float>(s, 3, x, extra, maxSlot, plan, ws)) return false;
+        return launchReduceScalar<float>(s, 19, x, maxSlot, z, plan, ws);
+    }
+    return launchReduceScalar<float>(s, opNum, x, extra, z, plan, ws);
 }
 
 #define INST(T)                                                                                                    \

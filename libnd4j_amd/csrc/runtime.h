@@ -109,4 +109,8 @@ template <typename T>
 bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hostXInfo, T *z, const Long *hostZInfo, T *params,
                       hipStream_t s);
 
+// Whole-array reduce of a float array into z[0] (device) without allocating: see native_reduce.cpp.  Throws
+// std::invalid_argument for what it does not accept (no host shapeInfo, more than 2^36 elements, unknown opNum).
+void reduceFloatNoAlloc(Nd4jPointer *extra, int opNum, float *x, Long *xInfo, float *params, float *z);
+
 }  // namespace nd4j_amd
