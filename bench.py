@@ -36,7 +36,11 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--families", action="store_true", help="also time every op family of the other configurations")
+    ap.add_argument("--families", action="store_true", help="(default) also time every op family of the other configurations")
+    ap.add_argument("--no-families", action="store_true", help="headline step only")
+    ap.add_argument("--families-cpu-seconds", type=float, default=25.0,
+                    help="total budget of the CPU passes beside the family rows; cases left over when it is spent get no "
+                         "CPU column")
     ap.add_argument("--only", default="", help="with --families: comma-separated workload builders to run "
                                                "(transform,pairwise,half,reductions,reduce3,stats,random,movement)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -218,8 +222,9 @@ def main():
     w.free()
 
     # ---- every other family ---------------------------------------------------------------------------
-    if args.families:
+    if not args.no_families:
         fam = []
+        cpu_left = args.families_cpu_seconds
         builders = [("transform", workloads.transform_tanh), ("pairwise", lambda d: workloads.pairwise_broadcast(d, copies=2)),
                     ("half", lambda d: workloads.pairwise_broadcast(d, dtype="float16")),
                     ("reductions", workloads.reductions), ("reduce3", workloads.reduce3_pairs),
@@ -234,12 +239,22 @@ def main():
                 fetched = dev.ops.amd_hostFetchCount()
                 ms = time_case(dev, c, max(3, min(K, 20)), 2)
                 fetched = dev.ops.amd_hostFetchCount() - fetched
-                row = {"config": wl.name, "case": c.name, "family": c.family, "contiguous": c.contiguous,
-                       "host_fetches": int(fetched),  # shapeInfo / dimension read-backs (each one a stream synchronisation)
-                       "ms": round(ms, 4), "GB/s": round(c.bytes / ms / 1e6, 1),
-                       "frac": round(c.bytes / ms / 1e6 / HBM_PEAK_GBS, 4), "elements_per_sec": round(c.elements / ms * 1e3, 1)}
-                if cpu_lib is not None and c.cpu is not None and not (c.name.endswith("float16")):
-                    med, runs = cpu_time(c.cpu, cpu_lib, 1.0, min_runs=2, max_runs=10)
+                row = {"case": c.name, "family": c.family, "ms": round(ms, 4), "GB/s": round(c.bytes / ms / 1e6, 1),
+                       "frac": round(c.bytes / ms / 1e6 / HBM_PEAK_GBS, 4), "elements_per_sec": float("%.4g" % (c.elements / ms * 1e3))}
+                if fetched:  # shapeInfo / dimension read-backs (each one a stream synchronisation)
+                    row["host_fetches"] = int(fetched)
+                row["bound"] = getattr(c, "bound", "hbm")
+                # one warm-up and up to three timed passes of the compiled reference, while the budget lasts; a case whose
+                # single pass is known to take seconds (note "cpu once") is run once, cold
+                if cpu_lib is not None and c.cpu is not None and not (c.name.endswith("float16")) and cpu_left > 0:
+                    t_cpu = time.perf_counter()
+                    if getattr(c, "cpu_once", False):
+                        t0 = time.perf_counter()
+                        c.cpu(cpu_lib)
+                        med = time.perf_counter() - t0
+                    else:
+                        med, runs = cpu_time(c.cpu, cpu_lib, 0.3, min_runs=1, max_runs=3)
+                    cpu_left -= time.perf_counter() - t_cpu
                     row["cpu_ms"] = round(med * 1e3, 3)
                     row["cpu_GB/s"] = round(c.bytes / med / 1e9, 2)
                     time.sleep(0.05)  # the OpenMP workers spin for a while after a parallel region: let them go to sleep

@@ -44,6 +44,8 @@ class Case(object):
         self.cpu = cpu
         self.contiguous = contiguous
         self.note = None  # printed beside the case by the benchmark
+        self.bound = "hbm"  # what limits the case: "hbm", or "valu" when instruction issue does
+        self.cpu_once = False  # the benchmark times a single cold CPU pass of this case
 
     @property
     def sets(self):
@@ -283,6 +285,8 @@ def reduce3_pairs(dev, rows=16384, cols=4096, seed=12, copies=None):
                                                     ex_a[11], ex_a[10], ex_a[11]),
                     lambda lib: (lib.reduce3_all(3, x[:ar * al], ai, y[:ar * al], ai, za, azi, [1], None), za)[1], True, ZA.get)
         case.note = "compute-bound: %.0f G pairs, fp32 FMA on the vector ALUs" % (ar * ar * al / 1e9)
+        case.bound = "valu"
+        case.cpu_once = True  # one pass of the reference takes seconds
         cases.append(case)
         return cases
 
