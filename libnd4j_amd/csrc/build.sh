@@ -15,7 +15,7 @@ OUT=../libnd4j_amd.so
 OBJ=build
 mkdir -p $OBJ
 HIPFLAGS="--offload-arch=gfx950 -O3 -std=c++17 -fPIC -ffp-contract=off -fhip-fp32-correctly-rounded-divide-sqrt -fvisibility=hidden -Xclang -target-feature -Xclang -packed-fp32-ops -Wno-unused-command-line-argument"
-SRCS="transform.hip pairwise.hip broadcast.hip scalar.hip reduce.hip reduce3.hip special.hip datamove.hip indexreduce.hip summarystats.hip random.hip native_ops.cpp native_reduce.cpp native_random.cpp native_special.cpp native_stubs.cpp runtime.cpp c_api.cpp"
+SRCS="transform.hip pairwise.hip broadcast.hip scalar.hip reduce.hip reduce3.hip special.hip wholearray.hip datamove.hip indexreduce.hip summarystats.hip random.hip native_ops.cpp native_reduce.cpp native_random.cpp native_special.cpp native_whole.cpp native_stubs.cpp runtime.cpp c_api.cpp"
 cat > $OBJ/Makefile <<MK
 OBJS := \$(addsuffix .o,\$(basename $SRCS))
 all: ../$OUT

@@ -151,6 +151,36 @@ bool launchSoftmaxFinish(hipStream_t stream, int opNum, const T *x, T *z, const 
 template <typename T> void launchIsMaxFill(hipStream_t stream, T *z, const T *index, const FlatPlan &zp);
 template <typename T> void launchIsMaxTadFill(hipStream_t stream, T *z, const T *index, const TadPlan &zt);
 
+// ---- whole-array transforms (Col2Im 36, Im2col 37, Histogram 48, Reverse 70, Pooling2D 71) ---------------------
+struct ReversePlan {
+    Long n = 0;
+    bool contiguous = false;  // x and z dense in one order (or x == z with unit stride): vector kernels
+    bool swap = false;        // in place with an element-wise stride: exchange e and n - 1 - e for e < n / 2
+    Long count = 0;           // mapped kernels: elements e < count are moved (n, or n / 2 in place)
+    DimMap xm, zm;            // element e of x -> offset, element of z -> offset (each in its own order)
+};
+template <typename T> void launchReverse(hipStream_t stream, const T *x, T *z, const ReversePlan &plan);
+// counts: capacity 32-bit counters of scratch; capacity = length of z (the bins that can be written)
+template <typename T>
+void launchHistogram(hipStream_t stream, const T *x, Long n, T *z, int capacity, const T *extra, unsigned *counts);
+// An image [bS, iC, iH, iW] with strides imS, and either its column form [bS, iC, kH, kW, oH, oW] with strides colS
+// (Im2col, Col2Im) or its pooled form [bS, iC, oH, oW] with strides colS[0..3] (Pooling2D).  Element counts stay below 2^31.
+struct ConvGeometry {
+    int bS, iC, iH, iW, kH, kW, oH, oW;
+    Long imS[4], colS[6];
+    FastDiv dOW, dOH, dKW, dKH, dIC, dIW, dIH;
+};
+template <typename T> void launchIm2col(hipStream_t stream, const T *x, T *z, const T *extra, const ConvGeometry &g);
+// clearFirst > 0: that many leading elements of z's buffer are cleared first and the sums are added onto what z holds
+template <typename T> void launchCol2im(hipStream_t stream, const T *x, T *z, const T *extra, const ConvGeometry &g, Long clearFirst);
+template <typename T> void launchPooling2d(hipStream_t stream, const T *x, T *z, const T *extra, const ConvGeometry &g);
+
+// DropOut 43 / DropOutInverted 44 as transforms: element i of x (through xm) survives when a hash of (seed + i) falls
+// below extra[0]
+template <typename T>
+void launchDropoutTransform(hipStream_t stream, bool inverted, const T *x, const DimMap &xm, T *z, const DimMap &zm,
+                            const T *extra, Long n, unsigned long long seed);
+
 // ---- data movement ---------------------------------------------------------------------------------
 // The result of a concat as the kernel needs it: strides per dimension, the concatenated dimension, and for a
 // contiguous C-order result the run geometry (inner = product of the dimensions after `dim`).

@@ -5,8 +5,10 @@
 //   broadcast  include/loops/cpu/broadcasting.cpp:42-156
 // extraPointers are decoded as the reference's CUDA back end does (blas/cuda/NativeOps.cu:1813-1823,
 // 3100-3131).
+#include <atomic>
 #include <cstdio>
 #include <cstring>
+#include <stdexcept>
 
 #include "../../include/NativeOps.h"
 #include "runtime.h"
@@ -45,9 +47,35 @@ void linearMap(const Long *shape, const Long *stride, int rank, char order, DimM
     ownCanon(rank, rs, rt, out);
 }
 
+// DropOut 43 / DropOutInverted 44 (include/ops/ops.h:3520-3562) draw from an unseeded generator in the reference; here
+// every call takes the next value of a process-wide counter as its seed.
+constexpr int kDropOut = 43, kDropOutInverted = 44;
+unsigned long long nextDropoutSeed() {
+    static std::atomic<unsigned long long> calls{0};
+    return (calls.fetch_add(1) + 1) * 0x2545f4914f6cdd1dull;
+}
+template <typename T>
+void dropoutTransform(hipStream_t s, int opNum, T *x, const DimMap &xm, T *z, const DimMap &zm, T *params, Long n) {
+    if (params == nullptr) throw std::invalid_argument("DropOut: extraParams [probability] required");
+    launchDropoutTransform<T>(s, opNum == kDropOutInverted, x, xm, z, zm, params, n, nextDropoutSeed());
+    checkLaunch("execTransform(dropout)", s);
+}
+void stridedMap(Long n, Long stride, DimMap &m) {
+    m.rank = 1;
+    m.shape[0] = (unsigned)(n > 0xffffffffLL ? 0xffffffffu : n);
+    m.stride[0] = stride;
+}
+
 template <typename T>
 void transformStrided(Nd4jPointer *extra, int opNum, T *x, Long xs, T *z, Long zs, T *params, Long n) {
     hipStream_t s = streamOf(extra);
+    if (opNum == kDropOut || opNum == kDropOutInverted) {
+        DimMap xm, zm;
+        stridedMap(n, xs, xm);
+        stridedMap(n, zs, zm);
+        dropoutTransform<T>(s, opNum, x, xm, z, zm, params, n);
+        return;
+    }
     if (!launchTransformStrided<T>(s, opNum, x, xs, z, zs, params, n)) { reportUnknownOp("transform", opNum); return; }
     checkLaunch("execTransform(strided)", s);
 }
@@ -64,16 +92,29 @@ void transformShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, Lon
         if (!specialTransform<T>(extra, opNum, x, hx, z, hz, params, s)) reportUnknownOp("transform", opNum);
         return;
     }
+    if (wholeArrayTransform<T>(opNum, x, hx, z, hz, params, s)) {
+        // Col2Im, Im2col, Histogram, Reverse, Pooling2D
+        checkLaunch("execTransform(whole array)", s);
+        return;
+    }
     Long n = siNumel(hx);
     Long xe = siEws(hx), ze = siEws(hz);
     bool ok;
     if (xe >= 1 && ze >= 1 && siOrder(hx) == siOrder(hz)) {
+        if (opNum == kDropOut || opNum == kDropOutInverted) {
+            transformStrided<T>(extra, opNum, x, xe, z, ze, params, n);
+            return;
+        }
         ok = launchTransformStrided<T>(s, opNum, x, xe, z, ze, params, n);
     } else {
         // same logical coordinates on both sides (raw iteration over x's shape)
         const Long *strides[3] = {siStride(hx), nullptr, siStride(hz)};
         DimMap maps[3];
         jointCanon(siRank(hx), siShape(hx), strides, maps);
+        if (opNum == kDropOut || opNum == kDropOutInverted) {
+            dropoutTransform<T>(s, opNum, x, maps[0], z, maps[2], params, n);
+            return;
+        }
         ok = launchTransformGeneral<T>(s, opNum, x, maps[0], z, maps[2], params, n);
     }
     if (!ok) { reportUnknownOp("transform", opNum); return; }

@@ -3,6 +3,7 @@
 // selection and the rewind after every op), include/ops/special_random_ops.h (special ops, which only the
 // (x, y, z) overload runs: cpu/random.cpp:15-18).
 #include <cstring>
+#include <stdexcept>
 
 #include "../../include/NativeOps.h"
 #include "rng.h"
@@ -54,6 +55,13 @@ void randomExec(Nd4jPointer *extra, int opNum, Nd4jPointer state, T *x, Long *xI
             // Gaussian / Binomial / TruncatedNormal / LogNormal address y and z through their EWS only
             printf("[ERROR] random op %d needs element-wise strides on y and z\n", opNum);
             return;
+        }
+        if (opNum == 5 && operands == 3 && pl.n > pl.yLength) {
+            // Without element-wise strides the reference's Choice indexes the probabilities with the RESULT's index
+            // (special_random_ops.h:214): defined (and followed here) while there are no more results than
+            // probabilities, a read beyond the probabilities otherwise - which a device must not replay
+            throw std::invalid_argument("Choice without element-wise strides needs length(z) <= length(y): the reference "
+                                        "reads outside the probabilities there");
         }
         fLinearMap(hz, pl.zm);
         if (hx) fLinearMap(hx, pl.xm);

@@ -136,6 +136,18 @@ ND4J_TRANSFORM(33, RELU, {
 })
 ND4J_TRANSFORM(34, Step, return d1 > p[0] ? (C)1 : (C)0;)
 ND4J_TRANSFORM(35, OneMinus, return (C)1 - d1;)
+// The whole-array ops have a per-element op() as well, which is what the strided entry point runs for them
+// (special_ops.h:361, 665, 885, 1131, 1416: identity; 1567, 1724, 1938, 2446: softplus); the shapeInfo entry point
+// routes these opNums to their own routines before it gets here.
+ND4J_TRANSFORM(36, Col2Im, return d1;)
+ND4J_TRANSFORM(37, Im2col, return d1;)
+ND4J_TRANSFORM(38, SoftMax, return m::log_((C)1 + m::exp_(d1));)
+ND4J_TRANSFORM(39, SoftMaxDerivative, return m::log_((C)1 + m::exp_(d1));)
+ND4J_TRANSFORM(40, LogSoftMax, return m::log_((C)1 + m::exp_(d1));)
+ND4J_TRANSFORM(41, IsMax, return m::log_((C)1 + m::exp_(d1));)
+ND4J_TRANSFORM(48, Histogram, return d1;)
+ND4J_TRANSFORM(70, Reverse, return d1;)
+ND4J_TRANSFORM(71, Pooling2D, return d1;)
 ND4J_TRANSFORM(42, SpecialDerivative, return d1 * ((C)1 - d1);)
 ND4J_TRANSFORM(45, CompareAndSet, {
     bool known;

@@ -109,6 +109,12 @@ template <typename T>
 bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hostXInfo, T *z, const Long *hostZInfo, T *params,
                       hipStream_t s);
 
+// The other whole-array transforms reached through execTransform's shapeInfo form: Col2Im 36, Im2col 37, Histogram 48,
+// Reverse 70, Pooling2D 71 (native_whole.cpp).  Returns false when opNum is not one of them; throws
+// std::invalid_argument for arguments the op cannot take (wrong ranks, missing extraParams, 2^31 elements or more).
+template <typename T>
+bool wholeArrayTransform(int opNum, T *x, const Long *hostXInfo, T *z, const Long *hostZInfo, T *params, hipStream_t s);
+
 // Whole-array reduce of a float array into z[0] (device) without allocating: see native_reduce.cpp.  Throws
 // std::invalid_argument for what it does not accept (no host shapeInfo, more than 2^36 elements, unknown opNum).
 void reduceFloatNoAlloc(Nd4jPointer *extra, int opNum, float *x, Long *xInfo, float *params, float *z);

@@ -27,6 +27,37 @@ struct DimMap {
     Long stride[kMaxDims];
 };
 
+// n / d and n % d for 0 <= n < 2^31 and 1 <= d < 2^31 through one high multiplication: with s = ceil(log2 d) and
+// m = ceil(2^(31 + s) / d) (which fits 32 bits), floor(n * m / 2^(31 + s)) == floor(n / d) because the excess
+// n * (m * d - 2^(31 + s)) / (d * 2^(31 + s)) stays below 1 / d.
+struct FastDiv {
+    unsigned d = 1, m = 0, shift = 0;
+    FastDiv() {}
+    explicit FastDiv(unsigned divisor) : d(divisor < 1 ? 1 : divisor) {
+        unsigned s = 0;
+        while (((unsigned long long)1 << s) < d) s++;
+        if (s == 0) { m = 0; shift = 0; return; }  // d == 1
+        m = (unsigned)((((unsigned long long)1 << (31 + s)) + d - 1) / d);
+        shift = s - 1;
+    }
+#if defined(__HIPCC__)
+    __host__ __device__
+#endif
+    inline unsigned div(unsigned n) const {
+        const unsigned q = (unsigned)(((unsigned long long)n * m) >> 32) >> shift;
+        return d == 1 ? n : q;
+    }
+    // returns n / d and leaves n % d in rem
+#if defined(__HIPCC__)
+    __host__ __device__
+#endif
+    inline unsigned divmod(unsigned n, unsigned &rem) const {
+        const unsigned q = div(n);
+        rem = n - q * d;
+        return q;
+    }
+};
+
 // C-order merge of one operand (drop unit dims, fuse dims d,d+1 when stride[d] == shape[d+1]*stride[d+1]).
 inline void ownCanon(int rank, const Long *shape, const Long *stride, DimMap &out) {
     Long shp[kMaxDims], str[kMaxDims];

@@ -1,0 +1,427 @@
+// Whole-array transforms that travel through execTransform* with a routine of their own instead of a per-element
+// functor: Col2Im 36, Im2col 37, Histogram 48, Reverse 70, Pooling2D 71.
+// Reference: include/ops/special_ops.h - Pooling2D::execSpecial 227-359, Im2col::execSpecial 530-663,
+// Histogram::execSpecial 811-882, Col2Im::execSpecial 997-1129, Reverse::execSpecial 1317-1414.
+//
+// Shapes and strides come from the host copies of the shapeInfos (the launchers' arguments); extraParams is a device
+// pointer in the caller's storage type and is read by the kernels.  All five are data movement with little arithmetic:
+// one thread per result element, neighbouring threads on neighbouring result elements, index decomposition through
+// host-prepared multipliers instead of divisions.
+#include "elementwise.cuh"
+#include "launch.h"
+
+namespace nd4j_amd {
+
+namespace {
+
+constexpr int kMaxGrid = 1 << 20;
+
+inline int gridFor(Long items, int perBlock = kBlock) {
+    Long blocks = (items + perBlock - 1) / perBlock;
+    if (blocks < 1) blocks = 1;
+    return (int)(blocks > kMaxGrid ? kMaxGrid : blocks);
+}
+
+template <typename T> __device__ __forceinline__ int paramInt(const T *extra, int i) { return (int)toCompute(extra[i]); }
+
+// what storing into T and reading back leaves of a value of the compute type (half rounds; float and double keep it):
+// the reference's loops accumulate in T
+template <typename T> __device__ __forceinline__ typename Compute<T>::type stored(typename Compute<T>::type v) {
+    return toCompute(fromCompute<T>(v));
+}
+
+__device__ __forceinline__ bool inRange(int a, int b) { return (unsigned)a < (unsigned)b; }
+
+// 16 bytes at an address that is only aligned to the element size: the hardware serves misaligned global accesses
+typedef U32x4 U32x4A2 __attribute__((aligned(2)));
+typedef U32x4 U32x4A4 __attribute__((aligned(4)));
+typedef U32x4 U32x4A8 __attribute__((aligned(8)));
+template <typename T> __device__ __forceinline__ Pack<T> loadPackAnywhere(const T *p) {
+    U32x4 v;
+    if (sizeof(T) == 2) v = *reinterpret_cast<const U32x4A2 *>(p);
+    else if (sizeof(T) == 4) v = *reinterpret_cast<const U32x4A4 *>(p);
+    else v = *reinterpret_cast<const U32x4A8 *>(p);
+    return __builtin_bit_cast(Pack<T>, v);
+}
+template <typename T> __device__ __forceinline__ void storePackAnywhere(T *p, const Pack<T> &a) {
+    const U32x4 v = __builtin_bit_cast(U32x4, a);
+    if (sizeof(T) == 2) *reinterpret_cast<U32x4A2 *>(p) = v;
+    else if (sizeof(T) == 4) *reinterpret_cast<U32x4A4 *>(p) = v;
+    else *reinterpret_cast<U32x4A8 *>(p) = v;
+}
+
+}  // namespace
+
+// ---- Reverse ---------------------------------------------------------------------------------------------------
+// Contiguous, out of place: a thread stores one aligned 16-byte vector of z and loads the mirrored stretch of x, which
+// is aligned only when the length and the two pointers happen to agree (the hardware serves misaligned global loads).
+template <typename T>
+__global__ void __launch_bounds__(kBlock) reverseVecKernel(const T *x, T *z, Long n, int head) {
+    constexpr int N = Pack<T>::N;
+    // z[0 .. head) one by one, so that the vectors of z start on a 16-byte boundary
+    const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
+    const Long lead = head < n ? head : n;
+    if (gtid < lead) z[gtid] = x[n - 1 - gtid];
+    const Long nvec = (n - lead) / N;
+    for (Long v = gtid; v < nvec; v += (Long)gridDim.x * kBlock) {
+        const Long j = lead + v * N;  // z[j .. j + N) <- x[n - N - j .. n - j) back to front
+        const Pack<T> a = loadPackAnywhere(x + (n - N - j));
+        Pack<T> r;
+#pragma unroll
+        for (int k = 0; k < N; k++) r.v[k] = a.v[N - 1 - k];
+        storePack(reinterpret_cast<Pack<T> *>(z + j), r);
+    }
+    const Long tail = lead + nvec * N;
+    if (gtid < n - tail) z[tail + gtid] = x[n - 1 - tail - gtid];
+}
+
+// Contiguous, in place: element e swaps with element n - 1 - e for e < n / 2.  A thread takes an aligned vector of
+// the front half and the mirrored (possibly misaligned) one of the back half; the pairs left over go one by one.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) reverseSwapVecKernel(T *x, Long n, int head) {
+    constexpr int N = Pack<T>::N;
+    const Long pairs = n / 2;
+    const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
+    if (gtid < head && gtid < pairs) {
+        const T t = x[gtid];
+        x[gtid] = x[n - 1 - gtid];
+        x[n - 1 - gtid] = t;
+    }
+    const Long nvec = pairs > head ? (pairs - head) / N : 0;
+    for (Long v = gtid; v < nvec; v += (Long)gridDim.x * kBlock) {
+        const Long j = head + v * N;
+        Pack<T> *front = reinterpret_cast<Pack<T> *>(x + j);
+        T *back = x + (n - N - j);
+        const Pack<T> a = *front, b = loadPackAnywhere(back);
+        Pack<T> ra, rb;
+#pragma unroll
+        for (int k = 0; k < N; k++) { ra.v[k] = b.v[N - 1 - k]; rb.v[k] = a.v[N - 1 - k]; }
+        *front = ra;
+        storePackAnywhere(back, rb);
+    }
+    const Long tail = head + nvec * N;
+    if (pairs > tail && gtid < pairs - tail) {
+        const Long e = tail + gtid;
+        const T t = x[e];
+        x[e] = x[n - 1 - e];
+        x[n - 1 - e] = t;
+    }
+}
+
+// Strided or mapped: z[zmap(n - 1 - e)] = x[xmap(e)] for e < count; SWAP exchanges the two elements of x instead.
+template <typename T, bool SWAP>
+__global__ void __launch_bounds__(kBlock) reverseMapKernel(const T *x, DimMap xm, T *z, DimMap zm, Long n, Long count) {
+    for (Long e = (Long)blockIdx.x * kBlock + threadIdx.x; e < count; e += (Long)gridDim.x * kBlock) {
+        const Long ox = mapOffsetAny(xm, e), oz = mapOffsetAny(zm, n - 1 - e);
+        if (SWAP) {
+            const T a = z[ox], b = z[oz];
+            z[ox] = b;
+            z[oz] = a;
+        } else {
+            z[oz] = x[ox];
+        }
+    }
+}
+
+template <typename T> void launchReverse(hipStream_t s, const T *x, T *z, const ReversePlan &p) {
+    if (p.n <= 0) return;
+    constexpr int N = Pack<T>::N;
+    if (p.contiguous) {
+        const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(z) & 15)) & 15) / sizeof(T));
+        if (p.swap) {
+            hipLaunchKernelGGL(reverseSwapVecKernel<T>, dim3(gridFor(p.n / 2 / N + 1)), dim3(kBlock), 0, s, z, p.n, head);
+        } else {
+            hipLaunchKernelGGL(reverseVecKernel<T>, dim3(gridFor(p.n / N + 1)), dim3(kBlock), 0, s, x, z, p.n, head);
+        }
+        return;
+    }
+    if (p.swap) {
+        hipLaunchKernelGGL((reverseMapKernel<T, true>), dim3(gridFor(p.count)), dim3(kBlock), 0, s, x, p.xm, z, p.zm, p.n, p.count);
+    } else {
+        hipLaunchKernelGGL((reverseMapKernel<T, false>), dim3(gridFor(p.count)), dim3(kBlock), 0, s, x, p.xm, z, p.zm, p.n, p.count);
+    }
+}
+
+// ---- Histogram -------------------------------------------------------------------------------------------------
+// extra = [numBins, min, max].  The reference's compiled loop multiplies (x - min) by 1 / binSize (its release flags
+// turn the loop-invariant division into a reciprocal) and truncates the way x86 does; half rounds the difference and
+// the product to half, while the reciprocal stays in float (float16's operators compute in float and round the result).
+template <typename T> struct HistogramBins {
+    typedef typename Compute<T>::type C;
+    int numBins;
+    C lo, perBin;
+    __device__ __forceinline__ HistogramBins(const T *extra, int capacity) {
+        numBins = paramInt(extra, 0);
+        lo = toCompute(extra[1]);
+        const C hi = toCompute(extra[2]);
+        const C binSize = stored<T>(stored<T>(hi - lo) / stored<T>((C)numBins));
+        perBin = (C)1 / binSize;
+        if (numBins > capacity) numBins = capacity;
+    }
+    __device__ __forceinline__ int operator()(T v) const {
+        int idx = m::toIntX86(stored<T>(stored<T>(toCompute(v) - lo) * perBin));
+        if (idx < 0) idx = 0;
+        else if (idx >= numBins) idx = numBins - 1;
+        return idx;
+    }
+};
+
+__global__ void __launch_bounds__(kBlock) clearCountsKernel(unsigned *counts, int n) {
+    for (int i = blockIdx.x * kBlock + threadIdx.x; i < n; i += gridDim.x * kBlock) counts[i] = 0u;
+}
+
+// Counts per block in LDS (when the bins fit), flushed with one atomic per non-empty bin; otherwise atomics on the
+// global counters directly.
+constexpr int kLdsBins = 8192;
+template <typename T, bool LDS>
+__global__ void __launch_bounds__(kBlock) histogramCountKernel(const T *x, Long n, const T *extra, unsigned *counts, int capacity) {
+    __shared__ unsigned local[LDS ? kLdsBins : 1];
+    const HistogramBins<T> bins(extra, capacity);
+    if (bins.numBins <= 0) return;
+    if (LDS) {
+        for (int b = threadIdx.x; b < bins.numBins; b += kBlock) local[b] = 0u;
+        __syncthreads();
+    }
+    constexpr int N = Pack<T>::N;
+    const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(x) & 15)) & 15) / sizeof(T));
+    const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
+    auto count = [&](T v) {
+        const int idx = bins(v);
+        if (LDS) atomicAdd(&local[idx], 1u);
+        else atomicAdd(&counts[idx], 1u);
+    };
+    const Long lead = head < n ? head : n;
+    if (gtid < lead) count(x[gtid]);
+    const Long nvec = (n - lead) / N;
+    const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x + lead);
+    for (Long v = gtid; v < nvec; v += (Long)gridDim.x * kBlock) {
+        const Pack<T> a = loadPack(xv + v);
+#pragma unroll
+        for (int k = 0; k < N; k++) count(a.v[k]);
+    }
+    const Long tail = lead + nvec * N;
+    if (gtid < n - tail) count(x[tail + gtid]);
+    if (LDS) {
+        __syncthreads();
+        for (int b = threadIdx.x; b < bins.numBins; b += kBlock) {
+            const unsigned c = local[b];
+            if (c != 0u) atomicAdd(&counts[b], c);
+        }
+    }
+}
+
+// z[b] += count[b], as the reference adds its counts onto what the result holds
+template <typename T>
+__global__ void __launch_bounds__(kBlock) histogramAddKernel(T *z, const T *extra, const unsigned *counts, int capacity) {
+    int numBins = paramInt(extra, 0);
+    if (numBins > capacity) numBins = capacity;
+    for (int b = blockIdx.x * kBlock + threadIdx.x; b < numBins; b += gridDim.x * kBlock) {
+        typedef typename Compute<T>::type C;
+        z[b] = fromCompute<T>(toCompute(z[b]) + (C)(int)counts[b]);
+    }
+}
+
+template <typename T>
+void launchHistogram(hipStream_t s, const T *x, Long n, T *z, int capacity, const T *extra, unsigned *counts) {
+    if (capacity <= 0) return;
+    hipLaunchKernelGGL(clearCountsKernel, dim3(gridFor(capacity)), dim3(kBlock), 0, s, counts, capacity);
+    if (n > 0) {
+        // enough blocks to fill the chip, few enough that the flushes of the per-block counts stay cheap
+        const int grid = gridFor(n / Pack<T>::N + 1) > 2048 ? 2048 : gridFor(n / Pack<T>::N + 1);
+        if (capacity <= kLdsBins)
+            hipLaunchKernelGGL((histogramCountKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
+        else
+            hipLaunchKernelGGL((histogramCountKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
+    }
+    hipLaunchKernelGGL(histogramAddKernel<T>, dim3(gridFor(capacity)), dim3(kBlock), 0, s, z, extra, counts, capacity);
+}
+
+// ---- Im2col ----------------------------------------------------------------------------------------------------
+// z[b, c, kr, kc, orow, ocol] = x[b, c, kr * dH + orow * sH - pH, kc * dW + ocol * sW - pW], zero outside the image.
+// extra = [kH, kW, sH, sW, pH, pW, dH, dW]; the kernel extents are taken from z's shape.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) im2colKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned total) {
+    const int sH = paramInt(extra, 2), sW = paramInt(extra, 3), pH = paramInt(extra, 4), pW = paramInt(extra, 5);
+    const int dH = paramInt(extra, 6), dW = paramInt(extra, 7);
+    for (unsigned i = blockIdx.x * kBlock + threadIdx.x; i < total; i += gridDim.x * kBlock) {
+        unsigned t = i, ocol, orow, kc, kr, c;
+        t = g.dOW.divmod(t, ocol);
+        t = g.dOH.divmod(t, orow);
+        t = g.dKW.divmod(t, kc);
+        t = g.dKH.divmod(t, kr);
+        const unsigned b = g.dIC.divmod(t, c);
+        const int r = (int)kr * dH + (int)orow * sH - pH, q = (int)kc * dW + (int)ocol * sW - pW;
+        T v = fromCompute<T>(0);
+        if (inRange(r, g.iH) && inRange(q, g.iW)) v = x[b * g.imS[0] + c * g.imS[1] + r * g.imS[2] + q * g.imS[3]];
+        z[b * g.colS[0] + c * g.colS[1] + kr * g.colS[2] + kc * g.colS[3] + orow * g.colS[4] + ocol * g.colS[5]] = v;
+    }
+}
+
+template <typename T> void launchIm2col(hipStream_t s, const T *x, T *z, const T *extra, const ConvGeometry &g) {
+    const Long total = (Long)g.bS * g.iC * g.kH * g.kW * g.oH * g.oW;
+    if (total <= 0) return;
+    hipLaunchKernelGGL(im2colKernel<T>, dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
+}
+
+// ---- Col2Im ----------------------------------------------------------------------------------------------------
+// z[b, c, h, w] = sum of the column entries that im2col would have read from (h, w), added one after the other in the
+// order (kr, kc) the reference's scatter loop reaches them (for one (kr, kc) at most one output position maps to a
+// pixel).  extra = [sH, sW, pH, pW, iH, iW, dH, dW].  ACCUMULATE: start from what z holds instead of from zero.
+template <typename T, bool ACCUMULATE>
+__global__ void __launch_bounds__(kBlock) col2imKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned total) {
+    typedef typename Compute<T>::type C;
+    const int sH = paramInt(extra, 0), sW = paramInt(extra, 1), pH = paramInt(extra, 2), pW = paramInt(extra, 3);
+    const int iH = paramInt(extra, 4), iW = paramInt(extra, 5), dH = paramInt(extra, 6), dW = paramInt(extra, 7);
+    for (unsigned i = blockIdx.x * kBlock + threadIdx.x; i < total; i += gridDim.x * kBlock) {
+        unsigned t = i, w, h, c;
+        t = g.dIW.divmod(t, w);
+        t = g.dIH.divmod(t, h);
+        const unsigned b = g.dIC.divmod(t, c);
+        T *out = z + (b * g.imS[0] + c * g.imS[1] + h * g.imS[2] + w * g.imS[3]);
+        C acc = ACCUMULATE ? toCompute(*out) : (C)0;
+        if ((int)h < iH && (int)w < iW) {
+            const T *col = x + (b * g.colS[0] + c * g.colS[1]);
+            for (int kr = 0; kr < g.kH; kr++) {
+                const int hh = (int)h + pH - kr * dH;
+                if (hh < 0) break;
+                const int orow = hh / sH;
+                if (orow * sH != hh || orow >= g.oH) continue;
+                for (int kc = 0; kc < g.kW; kc++) {
+                    const int ww = (int)w + pW - kc * dW;
+                    if (ww < 0) break;
+                    const int ocol = ww / sW;
+                    if (ocol * sW != ww || ocol >= g.oW) continue;
+                    acc = stored<T>(acc + toCompute(col[kr * g.colS[2] + kc * g.colS[3] + orow * g.colS[4] + ocol * g.colS[5]]));
+                }
+            }
+        }
+        *out = fromCompute<T>(acc);
+    }
+}
+
+__global__ void __launch_bounds__(kBlock) clearBytesKernel(U32x4 *p, Long vectors, unsigned char *tail, int tailBytes) {
+    const U32x4 zero = {0u, 0u, 0u, 0u};
+    const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
+    for (Long v = gtid; v < vectors; v += (Long)gridDim.x * kBlock) p[v] = zero;
+    if (gtid < tailBytes) tail[gtid] = 0;
+}
+
+template <typename T> void launchCol2im(hipStream_t s, const T *x, T *z, const T *extra, const ConvGeometry &g, Long clearFirst) {
+    const Long total = (Long)g.bS * g.iC * g.iH * g.iW;
+    if (total <= 0) return;
+    if (clearFirst > 0) {
+        // the reference clears the first length(z) elements of z's buffer whatever z's strides are, and adds onto the rest
+        unsigned char *base = reinterpret_cast<unsigned char *>(z);
+        Long bytes = clearFirst * (Long)sizeof(T);
+        Long lead = (Long)((16 - (reinterpret_cast<uintptr_t>(base) & 15)) & 15);
+        if (lead > bytes) lead = bytes;
+        if (lead > 0) hipLaunchKernelGGL(clearBytesKernel, dim3(1), dim3(kBlock), 0, s, nullptr, 0, base, (int)lead);
+        const Long vectors = (bytes - lead) / 16;
+        const int tailBytes = (int)(bytes - lead - vectors * 16);
+        hipLaunchKernelGGL(clearBytesKernel, dim3(gridFor(vectors + 1)), dim3(kBlock), 0, s, reinterpret_cast<U32x4 *>(base + lead), vectors,
+                           base + lead + vectors * 16, tailBytes);
+        hipLaunchKernelGGL((col2imKernel<T, true>), dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
+    } else {
+        hipLaunchKernelGGL((col2imKernel<T, false>), dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
+    }
+}
+
+// ---- Pooling2D -------------------------------------------------------------------------------------------------
+// extra = [kH, kW, sH, sW, pH, pW, dH, dW, -, mode, p]: mode 0 maximum (from -1e37, the reference's MAX_FLOAT), 1 average
+// (p == 0: over the cells inside the image, p == 1: over kH * kW), 2 p-norm.  One thread per result element; the window
+// is clipped to the image in steps of the dilation, as the reference clips it.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) pooling2dKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned total) {
+    typedef typename Compute<T>::type C;
+    lm::loadTables();  // the p-norm's powf
+    const int kH = paramInt(extra, 0), kW = paramInt(extra, 1), sH = paramInt(extra, 2), sW = paramInt(extra, 3);
+    const int pH = paramInt(extra, 4), pW = paramInt(extra, 5), dH = paramInt(extra, 6), dW = paramInt(extra, 7);
+    const int mode = paramInt(extra, 9);
+    const C p0 = toCompute(extra[10]);
+    const int kHEff = kH + (kH - 1) * (dH - 1), kWEff = kW + (kW - 1) * (dW - 1);
+    for (unsigned i = blockIdx.x * kBlock + threadIdx.x; i < total; i += gridDim.x * kBlock) {
+        unsigned t = i, xx, yy, c;
+        t = g.dOW.divmod(t, xx);
+        t = g.dOH.divmod(t, yy);
+        const unsigned b = g.dIC.divmod(t, c);
+        int hs = (int)yy * sH - pH, ws = (int)xx * sW - pW, he = hs + kHEff, we = ws + kWEff;
+        if (hs < 0) hs += ((-hs + dH - 1) / dH) * dH;
+        if (ws < 0) ws += ((-ws + dW - 1) / dW) * dW;
+        if (he > g.iH) he -= ((he - g.iH + dH - 1) / dH) * dH;
+        if (we > g.iW) we -= ((we - g.iW + dW - 1) / dW) * dW;
+        const T *in = x + (b * g.imS[0] + c * g.imS[1]);
+        C acc = mode == 0 ? (C)-1e37 : (C)0;
+        for (int ky = hs; ky < he; ky += dH)
+            for (int kx = ws; kx < we; kx += dW) {
+                const C v = toCompute(in[ky * g.imS[2] + kx * g.imS[3]]);
+                if (mode == 0) { if (v > acc) acc = v; }
+                else if (mode == 1) acc = stored<T>(acc + v);
+                else if (mode == 2) acc = stored<T>(acc + stored<T>(m::pow_(m::abs_(v), p0)));
+            }
+        if (mode == 1) {
+            // ceil((he - hs) / dH) * ceil((we - ws) / dW), also where clipping has turned a window inside out
+            const int rowsIn = he >= hs ? (he - hs + dH - 1) / dH : -((hs - he) / dH);
+            const int colsIn = we >= ws ? (we - ws + dW - 1) / dW : -((ws - we) / dW);
+            int div = 0;
+            if ((int)p0 == 0) div = rowsIn * colsIn;
+            else if ((int)p0 == 1) div = kH * kW;
+            acc = acc / (C)div;
+        } else if (mode == 2) {
+            acc = m::pow_(acc, stored<T>((C)1 / p0));
+        }
+        z[b * g.colS[0] + c * g.colS[1] + yy * g.colS[2] + xx * g.colS[3]] = fromCompute<T>(acc);
+    }
+}
+
+template <typename T> void launchPooling2d(hipStream_t s, const T *x, T *z, const T *extra, const ConvGeometry &g) {
+    const Long total = (Long)g.bS * g.iC * g.oH * g.oW;
+    if (total <= 0) return;
+    hipLaunchKernelGGL(pooling2dKernel<T>, dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
+}
+
+// ---- DropOut 43 / DropOutInverted 44 as transforms ---------------------------------------------------------------
+// z = rnd >= p ? 0 : x (inverted: x / p) with rnd uniform in [0, 1).  The reference draws rnd from the C library's
+// unseeded rand() on the CPU and from the clock on CUDA (include/ops/ops.h:3520-3562), so no two of its runs agree;
+// here rnd is a hash of the element's index and a per-call seed.
+__device__ __forceinline__ float unitHash(unsigned long long v) {
+    v += 0x9e3779b97f4a7c15ull;
+    v = (v ^ (v >> 30)) * 0xbf58476d1ce4e5b9ull;
+    v = (v ^ (v >> 27)) * 0x94d049bb133111ebull;
+    v ^= v >> 31;
+    return (float)(v >> 40) * (1.0f / 16777216.0f);
+}
+template <typename T, bool INVERTED>
+__global__ void __launch_bounds__(kBlock) dropoutTransformKernel(const T *x, DimMap xm, T *z, DimMap zm, const T *extra, Long n,
+                                                                 unsigned long long seed) {
+    typedef typename Compute<T>::type C;
+    const C prob = toCompute(extra[0]);
+    for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock) {
+        const C v = toCompute(x[mapOffsetAny(xm, i)]);
+        const C rnd = (C)unitHash(seed + (unsigned long long)i);
+        z[mapOffsetAny(zm, i)] = fromCompute<T>(rnd >= prob ? (C)0 : (INVERTED ? v / prob : v));
+    }
+}
+template <typename T>
+void launchDropoutTransform(hipStream_t s, bool inverted, const T *x, const DimMap &xm, T *z, const DimMap &zm, const T *extra,
+                            Long n, unsigned long long seed) {
+    if (n <= 0) return;
+    if (inverted)
+        hipLaunchKernelGGL((dropoutTransformKernel<T, true>), dim3(gridFor(n)), dim3(kBlock), 0, s, x, xm, z, zm, extra, n, seed);
+    else
+        hipLaunchKernelGGL((dropoutTransformKernel<T, false>), dim3(gridFor(n)), dim3(kBlock), 0, s, x, xm, z, zm, extra, n, seed);
+}
+
+#define INST(T)                                                                                                   \
+    template void launchDropoutTransform<T>(hipStream_t, bool, const T *, const DimMap &, T *, const DimMap &, const T *, Long, \
+                                            unsigned long long);                                                  \
+    template void launchReverse<T>(hipStream_t, const T *, T *, const ReversePlan &);                             \
+    template void launchHistogram<T>(hipStream_t, const T *, Long, T *, int, const T *, unsigned *);              \
+    template void launchIm2col<T>(hipStream_t, const T *, T *, const T *, const ConvGeometry &);                  \
+    template void launchCol2im<T>(hipStream_t, const T *, T *, const T *, const ConvGeometry &, Long);            \
+    template void launchPooling2d<T>(hipStream_t, const T *, T *, const T *, const ConvGeometry &);
+INST(float)
+INST(float16)
+INST(double)
+#undef INST
+
+}  // namespace nd4j_amd

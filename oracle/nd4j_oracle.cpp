@@ -258,6 +258,10 @@ template <typename T> static inline bool transformOp(int op, T d1, T *p, T &out)
         case 33: out = d1 < p[0] ? p[0] : d1; break;
         case 34: out = d1 > p[0] ? (T)1.0f : (T)0.0f; break;
         case 35: out = (T)1.0f - d1; break;
+        // the whole-array ops' own op(): what the strided entry point runs for them (special_ops.h:361, 665, 885,
+        // 1131, 1416: identity; 1567, 1724, 1938, 2446: softplus)
+        case 36: case 37: case 48: case 70: case 71: out = d1; break;
+        case 38: case 39: case 40: case 41: out = m_log((T)1.0f + m_exp(d1)); break;
         case 42: out = d1 * ((T)1.0 - d1); break;
         case 45: {
             bool known;
@@ -600,8 +604,192 @@ template <typename T> static void specialTransform(int op, T *x, Long *xi, T *z,
     }
 }
 
+
+// ---- the other whole-array transforms (include/ops/special_ops.h) ------------------------------------------------
+static inline bool inRange(int a, int b) { return (unsigned)a < (unsigned)b; }   // special_ops.h:409-411
+static bool stridesDescend(const Long *info) {                                    // shape::strideDescendingCAscendingF
+    const int rank = siRank(info);
+    const Long *st = siStride(info);
+    if (siOrder(info) == 'c') { for (int i = 1; i < rank; i++) if (st[i - 1] <= st[i]) return false; return true; }
+    for (int i = 1; i < rank; i++) if (st[i - 1] >= st[i]) return false;
+    return true;
+}
+
+// Reverse 70 (special_ops.h:1317-1414): the array read in its own order lands back to front.  In place: swaps for an
+// element-wise stride; without one only the first half is copied onto the mirrored positions.
+template <typename T> static void reverseWhole(T *x, Long *xi, T *z, Long *zi) {
+    const Long n = siNumel(xi), last = n - 1;
+    const Long xe = siEws(xi);
+    const char xo = siOrder(xi);
+    const int xr = siRank(xi);
+    Long cx[kMaxRank], cz[kMaxRank];
+    auto coords = [](char order, int rank, const Long *shape, Long idx, Long *c) {
+        if (order == 'c') { for (int d = rank - 1; d >= 0; d--) { c[d] = idx % shape[d]; idx /= shape[d]; } }
+        else { for (int d = 0; d < rank; d++) { c[d] = idx % shape[d]; idx /= shape[d]; } }
+    };
+    if (x == z) {
+        if (xe >= 1) {
+            for (Long e = 0; e < n / 2; e++) { T t = x[e * xe]; x[e * xe] = x[(last - e) * xe]; x[(last - e) * xe] = t; }
+        } else {
+            for (Long e = 0; e < n / 2; e++) {
+                coords(xo, xr, siShape(xi), e, cx);
+                coords(xo, xr, siShape(xi), last - e, cz);
+                z[getOffset(0, siShape(xi), siStride(xi), cz, xr)] = x[getOffset(0, siShape(xi), siStride(xi), cx, xr)];
+            }
+        }
+        return;
+    }
+    const Long ze = siEws(zi);
+    const char zo = siOrder(zi);
+    if (xe >= 1 && ze >= 1 && xo == zo) {
+        for (Long e = 0; e < n; e++) z[(last - e) * ze] = x[e * xe];
+        return;
+    }
+    for (Long e = 0; e < n; e++) {
+        coords(xo, xr, siShape(xi), e, cx);
+        coords(zo, siRank(zi), siShape(zi), last - e, cz);
+        z[getOffset(0, siShape(zi), siStride(zi), cz, siRank(zi))] = x[getOffset(0, siShape(xi), siStride(xi), cx, xr)];
+    }
+}
+
+// Histogram 48 (special_ops.h:811-882): extra = [numBins, min, max]; the first length(x) elements of the buffer are
+// binned by (x - min) / binSize, clamped to the outer bins, and the counts are ADDED to z.  The divisor is invariant in
+// the loop and the reference's release flags allow reciprocals: the compiled loop multiplies by 1 / binSize (and does
+// not fold the bin count into that reciprocal, hence the barrier: this file is built with the same flags).
+template <typename T> static inline T opaqueValue(T v) { asm volatile("" : "+m"(v)); return v; }
+template <typename T> static void histogramWhole(T *x, Long *xi, T *z, T *extra) {
+    const int length = (int)siNumel(xi);
+    const int numBins = toInt(extra[0]);
+    const T lo = extra[1], hi = extra[2];
+    const T binSize = opaqueValue<T>((hi - lo) / (T)numBins);
+    // for half the reciprocal stays in float: float16's operator/ divides two floats and rounds the quotient
+    typedef typename M<T>::C C;
+    const C perBin = opaqueValue<C>((C)1.0f / M<T>::up(binSize));
+    std::vector<int> bins(numBins > 0 ? numBins : 0, 0);
+    for (int i = 0; i < length; i++) {
+        int idx = toInt((T)(M<T>::up(x[i] - lo) * perBin));
+        if (idx < 0) idx = 0;
+        else if (idx >= numBins) idx = numBins - 1;
+        bins[idx]++;
+    }
+    for (int b = 0; b < numBins; b++) z[b] = (T)(M<T>::up(z[b]) + (C)bins[b]);  // T += int: the count is not rounded to T first
+}
+
+// Im2col 37 (special_ops.h:530-663): x [bS, iC, iH, iW] -> z [bS, iC, kH, kW, oH, oW]; extra = [kH, kW, sH, sW, pH, pW,
+// dH, dW]; positions outside the image are zero.  When both arrays are c-order with descending strides a batch entry
+// of the result is written as one dense run, whatever its inner strides say.
+template <typename T> static void im2colWhole(T *x, Long *xi, T *z, Long *zi, T *extra) {
+    const int kH = toInt(extra[0]), kW = toInt(extra[1]), sH = toInt(extra[2]), sW = toInt(extra[3]);
+    const int pH = toInt(extra[4]), pW = toInt(extra[5]), dH = toInt(extra[6]), dW = toInt(extra[7]);
+    const Long *is = siShape(xi), *ist = siStride(xi), *os = siShape(zi), *ost = siStride(zi);
+    const int bS = (int)is[0], iC = (int)is[1], iH = (int)is[2], iW = (int)is[3], oH = (int)os[4], oW = (int)os[5];
+    const bool dense = siOrder(xi) == 'c' && siOrder(zi) == 'c' && stridesDescend(xi) && stridesDescend(zi);
+    Long zs[6] = {ost[0], ost[1], ost[2], ost[3], ost[4], ost[5]};
+    if (dense) { zs[5] = 1; zs[4] = oW; zs[3] = (Long)oH * oW; zs[2] = zs[3] * kW; zs[1] = zs[2] * kH; }
+    for (int b = 0; b < bS; b++)
+        for (int c = 0; c < iC; c++)
+            for (int kr = 0; kr < kH; kr++)
+                for (int kc = 0; kc < kW; kc++)
+                    for (int orow = 0; orow < oH; orow++)
+                        for (int ocol = 0; ocol < oW; ocol++) {
+                            const int r = -pH + kr * dH + orow * sH, q = -pW + kc * dW + ocol * sW;
+                            T v = (T)0.0f;
+                            if (inRange(r, iH) && inRange(q, iW)) v = x[b * (int)ist[0] + c * (int)ist[1] + r * (int)ist[2] + q * (int)ist[3]];
+                            z[b * (int)zs[0] + c * zs[1] + kr * zs[2] + kc * zs[3] + orow * zs[4] + ocol * zs[5]] = v;
+                        }
+}
+
+// Col2Im 36 (special_ops.h:997-1129): x [bS, iC, kH, kW, oH, oW] -> z [bS, iC, iH, iW]; extra = [sH, sW, pH, pW, iH, iW,
+// dH, dW].  The first length(z) elements of z's buffer are cleared, then every column entry is added onto its pixel in
+// the order (kRow, kCol, oRow, oCol).  With c-order arrays of descending strides a batch entry of x is read as one run
+// of stride inStride[5].
+template <typename T> static void col2imWhole(T *x, Long *xi, T *z, Long *zi, T *extra) {
+    const Long *is = siShape(xi), *ist = siStride(xi), *ost = siStride(zi);
+    const int kH = (int)is[2], kW = (int)is[3], bS = (int)is[0], iC = (int)is[1], oH = (int)is[4], oW = (int)is[5];
+    const int sH = toInt(extra[0]), sW = toInt(extra[1]), pH = toInt(extra[2]), pW = toInt(extra[3]);
+    const int iH = toInt(extra[4]), iW = toInt(extra[5]), dH = toInt(extra[6]), dW = toInt(extra[7]);
+    const bool dense = siOrder(xi) == 'c' && siOrder(zi) == 'c' && stridesDescend(xi) && stridesDescend(zi);
+    Long xs[6] = {ist[0], ist[1], ist[2], ist[3], ist[4], ist[5]};
+    if (dense) { xs[4] = oW * xs[5]; xs[3] = oH * xs[4]; xs[2] = kW * xs[3]; xs[1] = kH * xs[2]; }
+    const Long zn = siNumel(zi);
+    for (Long i = 0; i < zn; i++) z[i] = (T)0.0f;
+    for (int b = 0; b < bS; b++)
+        for (int c = 0; c < iC; c++)
+            for (int kr = 0; kr < kH; kr++)
+                for (int kc = 0; kc < kW; kc++)
+                    for (int orow = 0; orow < oH; orow++) {
+                        const int r = -pH + kr * dH + orow * sH;
+                        if (!inRange(r, iH)) continue;
+                        for (int ocol = 0; ocol < oW; ocol++) {
+                            const int q = -pW + kc * dW + ocol * sW;
+                            if (!inRange(q, iW)) continue;
+                            T &o = z[b * (int)ost[0] + c * (int)ost[1] + r * (int)ost[2] + q * (int)ost[3]];
+                            o = o + x[b * (int)xs[0] + c * xs[1] + kr * xs[2] + kc * xs[3] + orow * xs[4] + ocol * xs[5]];
+                        }
+                    }
+}
+
+// Pooling2D 71 (special_ops.h:227-359): x [bS, iC, iH, iW] -> z [bS, iC, oH, oW]; extra = [kH, kW, sH, sW, pH, pW, dH, dW,
+// -, mode, p]: mode 0 max, 1 average (p == 0: divide by the cells inside the image, p == 1: by kH * kW), 2 p-norm.
+// A c-order result is written densely behind each (batch, channel) start; an f-order one through its strides.
+template <typename T> static void pooling2dWhole(T *x, Long *xi, T *z, Long *zi, T *extra) {
+    const int kH = toInt(extra[0]), kW = toInt(extra[1]), sH = toInt(extra[2]), sW = toInt(extra[3]);
+    const int pH = toInt(extra[4]), pW = toInt(extra[5]), dH = toInt(extra[6]), dW = toInt(extra[7]);
+    const int mode = toInt(extra[9]);
+    const T p0 = extra[10];
+    const int kHEff = kH + (kH - 1) * (dH - 1), kWEff = kW + (kW - 1) * (dW - 1);
+    const Long *is = siShape(xi), *ist = siStride(xi), *os = siShape(zi), *ost = siStride(zi);
+    const int bS = (int)is[0], iC = (int)is[1], iH = (int)is[2], iW = (int)is[3], oH = (int)os[2], oW = (int)os[3];
+    const bool fOrder = siOrder(zi) == 'f';
+    auto ceilDiv = [](int a, int b) { return toInt(m_ceil((T)a / (T)b)); };
+    for (int c = 0; c < iC; c++)
+        for (int b = 0; b < bS; b++) {
+            const int zb = b * (int)ost[0] + c * (int)ost[1];
+            const T *in = x + b * ist[0] + c * ist[1];
+            for (int yy = 0; yy < oH; yy++)
+                for (int xx = 0; xx < oW; xx++) {
+                    int hs = yy * sH - pH, ws = xx * sW - pW, he = hs + kHEff, we = ws + kWEff;
+                    if (hs < 0) hs += ceilDiv(-hs, dH) * dH;
+                    if (ws < 0) ws += ceilDiv(-ws, dW) * dW;
+                    if (he > iH) he -= ceilDiv(he - iH, dH) * dH;
+                    if (we > iW) we -= ceilDiv(we - iW, dW) * dW;
+                    const int poolSize = toInt(m_ceil((T)(he - hs) / (T)dH) * (T)toInt(m_ceil((T)(we - ws) / (T)dW)));
+                    T acc = mode == 0 ? (T)-1e37 : (T)0.0f;  // MAX_FLOAT is 1e37 (ops.h:12)
+                    for (long ky = hs; ky < he; ky += dH)
+                        for (long kx = ws; kx < we; kx += dW) {
+                            const T v = in[ky * ist[2] + kx * ist[3]];
+                            if (mode == 0) { if (v > acc) acc = v; }
+                            else if (mode == 1) acc = acc + v;
+                            else if (mode == 2) acc = acc + m_pow(m_abs(v), p0);
+                        }
+                    if (mode == 1) {
+                        int div = 0;
+                        if (toInt(p0) == 0) div = poolSize;
+                        else if (toInt(p0) == 1) div = kH * kW;
+                        acc = acc / (T)div;
+                    } else if (mode == 2) {
+                        acc = m_pow(acc, (T)1.0f / p0);
+                    }
+                    if (!fOrder) z[zb + yy * oW + xx] = acc;
+                    else z[zb + yy * (int)ost[2] + xx * (int)ost[3]] = acc;
+                }
+        }
+}
+
+template <typename T> static bool wholeArrayTransform(int op, T *x, Long *xi, T *z, Long *zi, T *extra) {
+    switch (op) {
+        case 36: col2imWhole<T>(x, xi, z, zi, extra); return true;
+        case 37: im2colWhole<T>(x, xi, z, zi, extra); return true;
+        case 48: histogramWhole<T>(x, xi, z, extra); return true;
+        case 70: reverseWhole<T>(x, xi, z, zi); return true;
+        case 71: pooling2dWhole<T>(x, xi, z, zi, extra); return true;
+        default: return false;
+    }
+}
+
 template <typename T> static void transformShaped(int op, T *x, Long *xi, T *z, Long *zi, T *extra) {
     if (op >= 38 && op <= 41) { specialTransform<T>(op, x, xi, z, zi, extra); return; }
+    if (wholeArrayTransform<T>(op, x, xi, z, zi, extra)) return;
     Long n = siNumel(xi);
     Long xe = siEws(xi), ze = siEws(zi);
     if (xe >= 1 && ze >= 1 && siOrder(xi) == siOrder(zi)) { transformStrided<T>(op, x, xe, z, ze, extra, n); return; }

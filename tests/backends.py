@@ -221,6 +221,12 @@ class _CpuRng(object):
         self.g.random_xyz(op, x.copy(), info, y.copy(), _vec_info(y.size), z, info, a)
         return z
 
+    def choice(self, values, v_info, probs, p_info, z_info):
+        """Choice (random op 5): z[i] = the value whose cumulative probability first reaches the i-th draw."""
+        z = np.zeros(_span(z_info), values.dtype)
+        self.g.random_xyz(5, values.copy(), v_info, probs.copy(), p_info, z, z_info, np.zeros(1, values.dtype))
+        return z
+
     def destroy(self):
         self.g.destroy()
 
@@ -639,6 +645,18 @@ class _GpuRng(object):
                    Z.info_ptr, a)
         out = Z.get()
         self.be._finish(X, Y, Z, A)
+        return out
+
+    def choice(self, values, v_info, probs, p_info, z_info):
+        X, Y = self.be._op(values, v_info), self.be._op(probs, p_info)
+        Z = self.be._op(np.zeros(_span(z_info), values.dtype), z_info)
+        A, a = self.be._up(np.zeros(1, values.dtype))
+        try:
+            self._exec(self.be._suffix(values), self.dev.extra(z_info), 5, self.ptr, X.ptr, X.info_ptr, Y.ptr,
+                       Y.info_ptr, Z.ptr, Z.info_ptr, a)
+            out = Z.get()
+        finally:
+            self.be._finish(X, Y, Z, A)
         return out
 
     def destroy(self):

@@ -671,3 +671,220 @@ def check_random_views(be, ref, seed, cases):
             assert np.array_equal(g[sel], c[sel]), ("scalar", op, list(xi), list(zi))
         done[what] = done.get(what, 0) + 1
     return done
+
+
+# ---- whole-array transforms: Col2Im 36, Im2col 37, Histogram 48, Reverse 70, Pooling2D 71 ------------------------------
+def _strided_info(rs, shape, kind):
+    """dense c (0), dense f (1), permuted dense strides (2) or permuted strides with padding (3) for `shape`."""
+    from libnd4j_amd import harness
+    shape = [int(v) for v in shape]
+    if kind < 2 or any(v == 1 for v in shape):
+        return harness.shape_info(shape, "c" if kind != 1 else "f")
+    strides = [0] * len(shape)
+    run = 1
+    for d in rs.permutation(len(shape)):
+        strides[d] = run
+        run *= shape[d] + (int(rs.randint(0, 3)) if kind == 3 else 0)
+    return harness.shape_info(shape, "c" if rs.rand() < 0.5 else "f", strides=strides)
+
+
+def _conv_geometry(rs):
+    kH, kW = int(rs.randint(1, 4)), int(rs.randint(1, 4))
+    sH, sW = int(rs.randint(1, 3)), int(rs.randint(1, 3))
+    dH, dW = int(rs.randint(1, 3)), int(rs.randint(1, 3))
+    pH, pW = int(rs.randint(0, 3)), int(rs.randint(0, 3))
+    kHe, kWe = kH + (kH - 1) * (dH - 1), kW + (kW - 1) * (dW - 1)
+    iH, iW = int(rs.randint(kHe, kHe + 9)), int(rs.randint(kWe, kWe + 9))
+    oH, oW = (iH + 2 * pH - kHe) // sH + 1, (iW + 2 * pW - kWe) // sW + 1
+    return kH, kW, sH, sW, pH, pW, dH, dW, iH, iW, oH, oW
+
+
+def check_whole_array_transforms(be, ref, seed, cases, dtypes=(np.float32, np.float64)):
+    """`be` against `ref` on generated calls of the five whole-array transforms.  Reverse, Im2col and Col2Im (sums in
+    the reference's order) exactly, over the whole result buffer; Histogram counts exactly; Pooling2D: max exactly,
+    average and p-norm within REDUCE_RTOL (the reference's window sums are re-associated by its build)."""
+    from libnd4j_amd import harness
+    rs = np.random.RandomState(seed)
+    done = {}
+    for it in range(cases):
+        dt = dtypes[it % len(dtypes)]
+        what = int(rs.randint(0, 5))
+        if what == 0:  # Reverse
+            shape = [int(rs.choice([1, 2, 3, 4, 5, 7, 8, 16, 33, 64])) for _ in range(int(rs.randint(1, 4)))]
+            if len(shape) == 1:
+                shape = [1] + shape
+            xi = _strided_info(rs, shape, int(rs.randint(0, 4)))
+            x = rs.uniform(-3, 3, harness.span_of(xi)).astype(dt)
+            if rs.rand() < 0.4:
+                g, c = be.transform_inplace(70, x, xi), ref.transform_inplace(70, x, xi)
+            else:
+                zi = _strided_info(rs, shape, int(rs.randint(0, 4)))
+                g, c = be.transform(70, x, xi, zi), ref.transform(70, x, xi, zi)
+            assert np.array_equal(g, c), ("reverse", list(xi), it)
+        elif what == 1:  # Histogram
+            # half holds counts up to 2048 exactly; beyond that the reference's result depends on which of its two
+            # threads adds its share first
+            n = int(rs.choice([1, 5, 64, 1000, 4099, 70001] if np.dtype(dt) != np.float16 else [1, 5, 64, 1000, 2000]))
+            bins = int(rs.choice([1, 2, 7, 64, 1000, 5000]))
+            x = rs.uniform(-3, 3, n).astype(dt)
+            lo, hi = (float(x.min()), float(x.max())) if rs.rand() < 0.5 else (-2.0, 2.5)
+            if lo == hi:
+                hi = lo + 1.0
+            extra = np.array([bins, lo, hi], dtype=dt)
+            z0 = np.floor(rs.uniform(0, 4, bins)).astype(dt)
+            xi, zi = harness.shape_info([1, n]), harness.shape_info([1, bins])
+            g, c = be.transform(48, x, xi, zi, extra, z=z0), ref.transform(48, x, xi, zi, extra, z=z0)
+            assert np.array_equal(g, c), ("histogram", n, bins, lo, hi, np.dtype(dt).name, it, np.nonzero(g != c)[0][:4])
+        else:
+            kH, kW, sH, sW, pH, pW, dH, dW, iH, iW, oH, oW = _conv_geometry(rs)
+            bS, iC = int(rs.randint(1, 4)), int(rs.randint(1, 5))
+            img, col, pooled = [bS, iC, iH, iW], [bS, iC, kH, kW, oH, oW], [bS, iC, oH, oW]
+            if what == 2:  # Im2col
+                xi, zi = _strided_info(rs, img, int(rs.randint(0, 4))), _strided_info(rs, col, int(rs.randint(0, 4)))
+                x = rs.uniform(-3, 3, harness.span_of(xi)).astype(dt)
+                extra = np.array([kH, kW, sH, sW, pH, pW, dH, dW, 0, 0], dtype=dt)
+                z0 = np.full(harness.span_of(zi), 9, dt)
+                g, c = be.transform(37, x, xi, zi, extra, z=z0), ref.transform(37, x, xi, zi, extra, z=z0)
+                assert np.array_equal(g, c), ("im2col", list(xi), list(zi), list(extra), it)
+            elif what == 3:  # Col2Im
+                xi, zi = _strided_info(rs, col, int(rs.randint(0, 4))), _strided_info(rs, img, int(rs.randint(0, 4)))
+                x = rs.uniform(-3, 3, harness.span_of(xi)).astype(dt)
+                extra = np.array([sH, sW, pH, pW, iH, iW, dH, dW], dtype=dt)
+                z0 = np.full(harness.span_of(zi), 9, dt)
+                g, c = be.transform(36, x, xi, zi, extra, z=z0), ref.transform(36, x, xi, zi, extra, z=z0)
+                assert np.array_equal(g, c), ("col2im", list(xi), list(zi), list(extra), it)
+            else:  # Pooling2D
+                mode = int(rs.randint(0, 3))
+                p0 = float(rs.randint(0, 2)) if mode == 1 else float(rs.choice([1.0, 2.0, 3.0]))
+                xi = _strided_info(rs, img, int(rs.randint(0, 4)))
+                zi = harness.shape_info(pooled, "c" if rs.rand() < 0.6 else "f")
+                x = rs.uniform(-3, 3, harness.span_of(xi)).astype(dt)
+                extra = np.array([kH, kW, sH, sW, pH, pW, dH, dW, 0, mode, p0], dtype=dt)
+                g, c = be.transform(71, x, xi, zi, extra), ref.transform(71, x, xi, zi, extra)
+                if mode == 0:
+                    assert np.array_equal(g, c), ("maxpool", list(xi), list(zi), list(extra), it)
+                else:
+                    ok = np.isclose(g, c, rtol=REDUCE_RTOL if np.dtype(dt) != np.float16 else HALF_RTOL, atol=1e-6, equal_nan=True)
+                    assert ok.all(), ("pool", mode, list(xi), list(zi), list(extra), it, g[~ok][:3], c[~ok][:3])
+        done[what] = done.get(what, 0) + 1
+    return done
+
+
+def check_whole_array_vectors(be):
+    """The fixed calls of golden_inputs.whole_array_cases against what the compiled reference wrote for them."""
+    from golden_inputs import whole_array_cases
+    vec = load_json("ref_vectors.json")["ops"]["whole_array_f32"]
+    for name, op, x, x_info, z_info, extra, z0 in whole_array_cases():
+        want = from_hexbits(vec[name], np.float32)
+        got = be.transform(op, x, x_info, z_info, extra, z=z0)
+        if name.startswith("pool_") and name != "pool_max":
+            assert np.allclose(got, want, rtol=REDUCE_RTOL, atol=0), name
+        else:
+            assert np.array_equal(got, want), name
+
+
+def check_whole_array_closed_forms(be):
+    """The whole-array transforms against plain numpy on integer-valued data (so that no sum depends on its order)."""
+    rs = np.random.RandomState(77)
+    f = np.float32
+    # Reverse
+    x = rs.randint(-50, 50, 24).astype(f)
+    vi, mi = shape_info_np([1, 24]), shape_info_np([4, 6])
+    assert np.array_equal(be.transform(70, x, vi, vi), x[::-1])
+    assert np.array_equal(be.transform(70, x, mi, mi), x[::-1])
+    assert np.array_equal(be.transform_inplace(70, x, vi), x[::-1])
+    assert np.array_equal(be.transform_inplace(70, x[:23].copy(), shape_info_np([1, 23])), x[:23][::-1])
+    # Histogram: values in the middle of their bins, two outliers clamped into the outer bins, counts added onto z
+    bins, lo, hi = 8, -4.0, 4.0
+    idx = rs.randint(0, bins, 500)
+    x = (lo + (idx + 0.5) * (hi - lo) / bins).astype(f)
+    x[:2] = [-100.0, 100.0]
+    idx[:2] = [0, bins - 1]
+    z0 = np.arange(bins, dtype=f)
+    got = be.transform(48, x, shape_info_np([1, 500]), shape_info_np([1, bins]), np.array([bins, lo, hi], f), z=z0)
+    assert np.array_equal(got, z0 + np.bincount(idx, minlength=bins)), "histogram"
+    # Im2col / Col2Im / Pooling2D
+    bS, iC, iH, iW, kH, kW, sH, sW, pH, pW, dH, dW = 2, 3, 8, 7, 3, 2, 2, 1, 1, 1, 1, 2
+    kHe, kWe = kH + (kH - 1) * (dH - 1), kW + (kW - 1) * (dW - 1)
+    oH, oW = (iH + 2 * pH - kHe) // sH + 1, (iW + 2 * pW - kWe) // sW + 1
+    img = rs.randint(-9, 10, (bS, iC, iH, iW)).astype(f)
+    padded = np.zeros((bS, iC, iH + 2 * pH + sH * oH + kHe, iW + 2 * pW + sW * oW + kWe), f)
+    padded[:, :, pH:pH + iH, pW:pW + iW] = img
+    col = np.zeros((bS, iC, kH, kW, oH, oW), f)
+    for kr in range(kH):
+        for kc in range(kW):
+            for r in range(oH):
+                for q in range(oW):
+                    col[:, :, kr, kc, r, q] = padded[:, :, kr * dH + r * sH, kc * dW + q * sW]
+    ii, ci = shape_info_np([bS, iC, iH, iW]), shape_info_np([bS, iC, kH, kW, oH, oW])
+    e = np.array([kH, kW, sH, sW, pH, pW, dH, dW, 0, 0], f)
+    assert np.array_equal(be.transform(37, img.ravel(), ii, ci, e), col.ravel()), "im2col"
+    cols = rs.randint(-9, 10, col.shape).astype(f)
+    back = np.zeros_like(padded)
+    for kr in range(kH):
+        for kc in range(kW):
+            for r in range(oH):
+                for q in range(oW):
+                    back[:, :, kr * dH + r * sH, kc * dW + q * sW] += cols[:, :, kr, kc, r, q]
+    e = np.array([sH, sW, pH, pW, iH, iW, dH, dW], f)
+    assert np.array_equal(be.transform(36, cols.ravel(), ci, ii, e, z=np.full(img.size, 5, f)),
+                          back[:, :, pH:pH + iH, pW:pW + iW].ravel()), "col2im"
+    pi = shape_info_np([bS, iC, oH, oW])
+    inside = np.zeros_like(padded)
+    inside[:, :, pH:pH + iH, pW:pW + iW] = 1
+    mx = np.full((bS, iC, oH, oW), -1e37, f)
+    sm = np.zeros((bS, iC, oH, oW), np.float64)
+    sq = np.zeros((bS, iC, oH, oW), np.float64)
+    cnt = np.zeros((bS, iC, oH, oW), np.float64)
+    for kr in range(kH):
+        for kc in range(kW):
+            for r in range(oH):
+                for q in range(oW):
+                    v, ok = padded[:, :, kr * dH + r * sH, kc * dW + q * sW], inside[:, :, kr * dH + r * sH, kc * dW + q * sW]
+                    mx[:, :, r, q] = np.where(ok > 0, np.maximum(mx[:, :, r, q], v), mx[:, :, r, q])
+                    sm[:, :, r, q] += v
+                    sq[:, :, r, q] += v.astype(np.float64) ** 2
+                    cnt[:, :, r, q] += ok
+
+    def pool(mode, p0):
+        return be.transform(71, img.ravel(), ii, pi, np.array([kH, kW, sH, sW, pH, pW, dH, dW, 0, mode, p0], f))
+    assert np.array_equal(pool(0, 0), mx.ravel()), "max pooling"
+    assert np.allclose(pool(1, 0), (sm / cnt).ravel(), rtol=1e-6, atol=0), "average over the cells inside the image"
+    assert np.allclose(pool(1, 1), (sm / (kH * kW)).ravel(), rtol=1e-6, atol=0), "average over the kernel"
+    assert np.allclose(pool(2, 2), np.sqrt(sq).ravel(), rtol=1e-6, atol=0), "2-norm pooling"
+
+
+# ---- Choice (random op 5) ---------------------------------------------------------------------------------------------
+def check_choice(be, ref, seed=5):
+    """Choice on `be` against `ref`: the element-wise-stride branch on dense and strided vectors, and the coordinate
+    branch (which indexes the probabilities with the result's index, so it is only defined while there are no more
+    results than probabilities).  Results and generator state exactly."""
+    from libnd4j_amd import harness
+    rs = np.random.RandomState(seed)
+    for dt in (np.float32, np.float64, np.float16):
+        a, b = be.rng(119, 1 << 12), ref.rng(119, 1 << 12)
+        for n_vals, n_out in ((4, 500), (1, 17), (37, 4099), (256, 70001)):
+            probs = rs.uniform(0.1, 1, n_vals)
+            probs = (probs / probs.sum()).astype(dt)
+            vals = (np.arange(n_vals) * 3 + 10).astype(dt)
+            vi, zi = harness.shape_info([1, n_vals]), harness.shape_info([1, n_out])
+            assert np.array_equal(a.choice(vals, vi, probs, vi, zi), b.choice(vals, vi, probs, vi, zi)), ("choice", n_vals, n_out, dt)
+            assert a.state() == b.state()
+        # strided vectors: values and probabilities every third / second element, results every second
+        n_vals, n_out = 9, 301
+        vi = harness.shape_info([1, n_vals], strides=[1, 3], ews=3)
+        pi = harness.shape_info([1, n_vals], strides=[1, 2], ews=2)
+        zi = harness.shape_info([1, n_out], strides=[1, 2], ews=2)
+        vals = rs.uniform(-5, 5, harness.span_of(vi)).astype(dt)
+        probs = np.full(harness.span_of(pi), 1.0 / n_vals, dt)
+        assert np.array_equal(a.choice(vals, vi, probs, pi, zi), b.choice(vals, vi, probs, pi, zi)), ("choice strided", dt)
+        # no element-wise stride on the result: the coordinate branch
+        zi = harness.shape_info([3, 4], "c", strides=[1, 5])
+        vi = harness.shape_info([4, 5], "f")
+        vals = rs.uniform(-5, 5, 20).astype(dt)
+        probs = rs.uniform(0.02, 0.2, 20).astype(dt)
+        assert harness.info_numel(zi) <= 20
+        assert np.array_equal(a.choice(vals, vi, probs, vi, zi), b.choice(vals, vi, probs, vi, zi)), ("choice by coordinates", dt)
+        assert a.state() == b.state()
+        a.destroy()
+        b.destroy()

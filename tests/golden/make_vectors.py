@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(HERE))
 import cpu_ref  # noqa: E402
 from golden_inputs import (BROADCAST_OPS, INDEX_OPS, PAIRWISE_OPS, REDUCE_OPS, SCALAR_OPS, SCALAR_VALUES, TRANSFORM_OPS,  # noqa: E402
-                           hexbits, op_extra, pairwise_inputs, reduce_input, shape_info_np, transform_input)
+                           hexbits, op_extra, pairwise_inputs, reduce_input, shape_info_np, transform_input, whole_array_cases)
 
 
 def main():
@@ -223,6 +223,13 @@ def main():
     h["broadcast_add_row"] = hexbits(z)
     h["reduce_sum_y"] = hexbits(np.array([ref.reduce_scalar(1, yh, hi, None)], np.float16))
     ops["f16_2x4"] = h
+    # whole-array transforms: Col2Im, Im2col, Histogram, Reverse, Pooling2D
+    wa = {}
+    for name, op, x, x_info, z_info, extra, z0 in whole_array_cases():
+        z = z0.copy()
+        ref.transform(op, x, x_info, z, z_info, extra)
+        wa[name] = hexbits(z)
+    ops["whole_array_f32"] = wa
     out["ops"] = ops
 
     with open(os.path.join(HERE, "ref_vectors.json"), "w") as f:

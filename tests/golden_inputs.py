@@ -129,3 +129,29 @@ def ulp_distance(a, b):
     d = np.abs(ia - ib)
     both_nan = np.isnan(a) & np.isnan(b)
     return np.where(both_nan, 0, d)
+
+
+def whole_array_cases():
+    """Fixed calls of the whole-array transforms (Col2Im 36, Im2col 37, Histogram 48, Reverse 70, Pooling2D 71):
+    (name, opNum, x, x_info, z_info, extraParams, initial z).  Dense c-order float32 arrays, values from the same
+    arithmetic sweep as the other inputs."""
+    def values(n, scale=6.0):
+        k = np.arange(n, dtype=np.float64)
+        return (((k * 0.7919) % scale) - scale / 2).astype(np.float32)
+
+    f = np.float32
+    cases = []
+    img, col, pooled = [2, 3, 7, 6], [2, 3, 3, 2, 4, 3], [2, 3, 4, 3]
+    ii, ci, pi = shape_info_np(img), shape_info_np(col), shape_info_np(pooled)
+    n_img, n_col, n_pool = int(np.prod(img)), int(np.prod(col)), int(np.prod(pooled))
+    # kH 3, kW 2, stride 2 x 2, padding 1 x 1, dilation 1 x 2: oH = (7 + 2 - 3) / 2 + 1 = 4, oW = (6 + 2 - 3) / 2 + 1 = 3
+    cases.append(("im2col", 37, values(n_img), ii, ci, np.array([3, 2, 2, 2, 1, 1, 1, 2, 0, 0], f), np.full(n_col, 9, f)))
+    cases.append(("col2im", 36, values(n_col), ci, ii, np.array([2, 2, 1, 1, 7, 6, 1, 2], f), np.full(n_img, 9, f)))
+    for name, mode, p0 in (("pool_max", 0, 0), ("pool_avg_inside", 1, 0), ("pool_avg_kernel", 1, 1), ("pool_pnorm2", 2, 2)):
+        cases.append((name, 71, values(n_img), ii, pi, np.array([3, 2, 2, 2, 1, 1, 1, 2, 0, mode, p0], f), np.zeros(n_pool, f)))
+    x = values(1000)
+    cases.append(("histogram", 48, x, shape_info_np([1, 1000]), shape_info_np([1, 16]), np.array([16, -2.5, 2.75], f),
+                  np.arange(16, dtype=f)))
+    cases.append(("reverse_vector", 70, values(37), shape_info_np([1, 37]), shape_info_np([1, 37]), None, np.zeros(37, f)))
+    cases.append(("reverse_matrix_c_to_f", 70, values(35), shape_info_np([5, 7]), shape_info_np([5, 7], "f"), None, np.zeros(35, f)))
+    return cases

@@ -618,9 +618,109 @@ def test_unknown_op_leaves_output_untouched(gpu, capfd):
     xi = shape_info_np([1, 64])
     got = gpu.transform(500, x, xi, xi, z=np.full(64, 9.0, np.float32))
     assert np.all(got == 9.0)
-    got = gpu.transform(36, x, xi, xi, z=np.full(64, 9.0, np.float32))  # Col2Im: a whole-array op that is not on this path
-    assert np.all(got == 9.0)
     assert float(gpu.reduce_scalar(2, x, xi)) == 0.0  # opNum 2 is a gap in the reduce table
+
+
+def test_whole_array_transforms_vectors_and_closed_forms(gpu):
+    checks.check_whole_array_vectors(gpu)
+    checks.check_whole_array_closed_forms(gpu)
+
+
+def test_whole_array_transforms(gpu, cpu):
+    # Col2Im 36, Im2col 37, Histogram 48, Reverse 70, Pooling2D 71 on generated shapes, strides and geometries
+    done = checks.check_whole_array_transforms(gpu, cpu, 41, 500)
+    assert all(done.get(k, 0) >= 50 for k in range(5)), done
+    checks.check_whole_array_transforms(gpu, cpu, 42, 200, dtypes=(np.float16,))
+
+
+def test_whole_array_transforms_larger(gpu, cpu):
+    rs = np.random.RandomState(43)
+    f = np.float32
+    # Reverse of odd lengths (misaligned mirrored vectors), out of place and in place, three types
+    for n in (1, 2, 7, 4099, (1 << 20) + 3, (1 << 22)):
+        for dt in (np.float32, np.float64, np.float16):
+            x = rs.uniform(-3, 3, n).astype(dt)
+            vi = shape_info_np([1, n])
+            assert np.array_equal(gpu.transform(70, x, vi, vi), x[::-1]), ("reverse", n, dt)
+            assert np.array_equal(gpu.transform_inplace(70, x, vi), x[::-1]), ("reverse in place", n, dt)
+    # Histogram over a few million elements: bins in LDS and, beyond 8192 bins, in global memory
+    n = (1 << 22) + 5
+    x = rs.uniform(-3, 3, n).astype(f)
+    for bins in (10, 8192, 20000):
+        extra = np.array([bins, -2.5, 2.75], f)
+        xi, zi = shape_info_np([1, n]), shape_info_np([1, bins])
+        assert np.array_equal(gpu.transform(48, x, xi, zi, extra), cpu.transform(48, x, xi, zi, extra)), ("histogram", bins)
+    # a convolution-sized image through Im2col and back through Col2Im, and pooled
+    img, col, pooled = [4, 16, 56, 56], [4, 16, 3, 3, 56, 56], [4, 16, 28, 28]
+    ii, ci, pi = shape_info_np(img), shape_info_np(col), shape_info_np(pooled)
+    x = rs.uniform(-3, 3, int(np.prod(img))).astype(f)
+    e_im = np.array([3, 3, 1, 1, 1, 1, 1, 1, 0, 0], f)
+    g, c = gpu.transform(37, x, ii, ci, e_im), cpu.transform(37, x, ii, ci, e_im)
+    assert np.array_equal(g, c), "im2col"
+    e_col = np.array([1, 1, 1, 1, 56, 56, 1, 1], f)
+    assert np.array_equal(gpu.transform(36, g, ci, ii, e_col), cpu.transform(36, c, ci, ii, e_col)), "col2im"
+    for mode, p0 in ((0, 0.0), (1, 0.0), (1, 1.0), (2, 2.0)):
+        e_pool = np.array([2, 2, 2, 2, 0, 0, 1, 1, 0, mode, p0], f)
+        gp, cp = gpu.transform(71, x, ii, pi, e_pool), cpu.transform(71, x, ii, pi, e_pool)
+        if mode == 0:
+            assert np.array_equal(gp, cp), "max pooling"
+        else:
+            assert np.allclose(gp, cp, rtol=1e-5, atol=1e-6), ("pooling", mode, p0)
+
+
+def test_whole_array_transforms_strided_form_and_errors(gpu, cpu):
+    # the strided entry point runs the ops' per-element op(): identity, and softplus for the softmax family
+    x = np.linspace(-3, 3, 257).astype(np.float32)
+    for op in (36, 37, 48, 70, 71):
+        assert np.array_equal(gpu.transform_strided(op, x, 1, 1, None, x.size), x), op
+    for op in (38, 39, 40, 41):
+        assert ulp_distance(gpu.transform_strided(op, x, 1, 1, None, x.size), cpu.transform_strided(op, x, 1, 1, None, x.size)).max() <= 2, op
+    # arguments the whole-array routines cannot take are reported, not ignored
+    vi = shape_info_np([1, 257])
+    for op in (36, 37, 71):
+        with pytest.raises(Exception):
+            gpu.transform(op, x, vi, vi, np.zeros(11, np.float32))
+
+
+def test_choice(gpu, cpu):
+    checks.check_choice(gpu, cpu)
+    # more results than probabilities without element-wise strides: the reference reads outside the probabilities;
+    # the device refuses
+    zi = harness.shape_info([5, 6], "c", strides=[1, 7])
+    vi = shape_info_np([1, 4])
+    g = gpu.rng(1, 64)
+    with pytest.raises(Exception, match="Choice"):
+        g.choice(np.arange(4, dtype=np.float32), vi, np.full(4, 0.25, np.float32), vi, zi)
+    g.destroy()
+
+
+def test_dropout_transforms(gpu):
+    # DropOut 43 / DropOutInverted 44: the reference draws from an unseeded generator (rand() / the clock), so only the
+    # distribution can be held to it: survivors keep x (or x / p), the rest is zero, about p of the elements survive,
+    # and two calls do not drop the same elements
+    n, p = 1 << 20, 0.3
+    x = np.random.RandomState(3).uniform(1, 2, n).astype(np.float32)
+    vi = shape_info_np([1, n])
+    e = np.array([p, 0], np.float32)
+    a, b = gpu.transform(43, x, vi, vi, e), gpu.transform(43, x, vi, vi, e)
+    for z in (a, b):
+        kept = z != 0
+        assert np.array_equal(z[kept], x[kept])
+        assert abs(kept.mean() - p) < 5 * np.sqrt(p * (1 - p) / n)
+    both = ((a != 0) & (b != 0)).mean()
+    assert abs(both - p * p) < 0.01, both
+    inv = gpu.transform(44, x, vi, vi, e)
+    kept = inv != 0
+    assert np.array_equal(inv[kept], (x[kept] / np.float32(p)).astype(np.float32))
+    assert abs(kept.mean() - p) < 5 * np.sqrt(p * (1 - p) / n)
+    # a strided view: nothing outside it is written, and the strided entry point takes the same ops
+    xi = harness.shape_info([64, 50], "c", strides=[100, 2])
+    xs = np.ones(harness.span_of(xi), np.float32)
+    z = gpu.transform(43, xs, xi, xi, e)
+    sel = harness.element_offsets(xi)
+    assert np.all(np.delete(z, sel) == 0) and 0.2 < (z[sel] != 0).mean() < 0.4
+    z = gpu.transform_strided(44, xs, 2, 3, e, 1000)
+    assert np.all(np.delete(z, np.arange(1000) * 3) == 0) and 0.2 < (z[::3] != 0).mean() < 0.4
 
 
 def test_half_families(gpu, cpu):

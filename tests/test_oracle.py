@@ -40,6 +40,22 @@ def test_rng_closed_forms(oracle):
     checks.check_rng_closed_forms(oracle)
 
 
+def test_whole_array_transforms_vectors_and_closed_forms(oracle):
+    checks.check_whole_array_vectors(oracle)
+    checks.check_whole_array_closed_forms(oracle)
+
+
+def test_whole_array_transforms_match_compiled_reference(oracle, reference_lib):
+    ref = backends.CpuBackend(reference_lib)
+    done = checks.check_whole_array_transforms(oracle, ref, 11, 600)
+    assert all(done.get(k, 0) >= 60 for k in range(5)), done
+    checks.check_whole_array_transforms(oracle, ref, 12, 300, dtypes=(np.float16,))
+
+
+def test_choice_matches_compiled_reference(oracle, reference_lib):
+    checks.check_choice(oracle, backends.CpuBackend(reference_lib))
+
+
 def test_tad_fixtures(oracle):
     checks.check_tad_fixtures(oracle.tad)
 
