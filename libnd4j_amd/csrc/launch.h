@@ -69,11 +69,24 @@ struct TadPlan {
 struct Workspace {
     void *ptr;
     size_t bytes;
-    // Optional completion signal of a scalar-result launch: the thread that stores the result then stores `ticket`
-    // into `*signal` (host memory the device can write), behind a system-scope fence, so that the host may wait for
-    // the value itself instead of for the stream.  Null for array results.
-    unsigned *signal = nullptr;
+    // Optional hand-over of a scalar result to a waiting host: the thread that stores the result also stores it, 32 bits
+    // a word, into the 8-byte words at `signal` (host memory the device can write), each word tagged with `ticket` in
+    // its upper half, so that the host may wait for the value itself instead of for the stream.  Null for array results.
+    unsigned long long *signal = nullptr;
     unsigned ticket = 0;
+    // Optional: what the whole-array reductions need to finish in one launch - `slotBytes` bytes of 8-byte slots that no
+    // other kernel writes (zero when allocated), 16 KiB of block counters that are zero between calls, and tickets that differ
+    // from launch to launch on this stream (never zero).  Without them the reduction takes a second, merging launch.
+    unsigned long long *slots = nullptr;
+    size_t slotBytes = 0;
+    unsigned *counter = nullptr;
+    unsigned *slotTicketSource = nullptr;  // host memory: the last ticket handed out for these slots
+    // the next ticket: every launch that uses the slots takes its own
+    unsigned nextSlotTicket() const {
+        unsigned t = ++*slotTicketSource;
+        if (t == 0) t = ++*slotTicketSource;
+        return t;
+    }
 };
 
 // Full-array view for scalar reductions: either 1-D strided (ews >= 1) or a C-order coordinate map.

@@ -31,11 +31,12 @@ Scratch scratchFor(hipStream_t s, size_t wantRest = 0) {
     sc.scalars = w.ptr;
     sc.rest.ptr = reinterpret_cast<char *>(w.ptr) + kScalarArea;
     sc.rest.bytes = w.bytes - kScalarArea;
+    addFlatSlots(sc.rest, s);
     return sc;
 }
 
 Workspace withSignal(Workspace w, const ScalarSignal &sig) {
-    w.signal = sig.flag;
+    w.signal = sig.words;
     w.ticket = sig.ticket;
     return w;
 }
@@ -106,10 +107,9 @@ template <> struct ScalarOut<double> { typedef double R; static R get(double v) 
 template <> struct ScalarOut<float16> { typedef float R; static R get(float16 v) { return halfBitsToFloatHost(v.x); } };
 
 template <typename T>
-typename ScalarOut<T>::R readScalar(const void *pinnedSlot, hipStream_t s, const char *what, const ScalarSignal &sig) {
-    waitForScalar(sig, s, what);
+typename ScalarOut<T>::R readScalar(const void *, hipStream_t s, const char *what, const ScalarSignal &sig) {
     T v;
-    std::memcpy(&v, pinnedSlot, sizeof(T));
+    takeScalar(sig, s, what, &v, sizeof(T));
     return ScalarOut<T>::get(v);
 }
 

@@ -76,7 +76,7 @@ struct Reduce3Plan {
 template <typename T, int OP, int GROUP>
 __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, T *z, const T *extra, Reduce3Plan pl,
                                                         Acc3<typename Compute<T>::type> *partials, Long sliceLength, Long slices,
-                                                        unsigned *signal, unsigned ticket) {
+                                                        unsigned long long *signal, unsigned ticket) {
     typedef typename Compute<T>::type C;
     typedef Acc3<C> Acc;
     constexpr int GROUPS = kBlock / GROUP;
@@ -153,8 +153,9 @@ __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, 
             if (sliced) {
                 partials[u] = acc;
             } else {
-                z[u] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, pl.runLength));
-                signalResult(signal, ticket);  // set only for a launch with a single result
+                const T r = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, pl.runLength));
+                z[u] = r;
+                signalResult(signal, ticket, r);  // set only for a launch with a single result
             }
         }
     }
@@ -162,7 +163,7 @@ __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, 
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kBlock) reduce3Finish(T *z, const Acc3<typename Compute<T>::type> *partials, int count,
-                                                        Long runLength, unsigned *signal, unsigned ticket) {
+                                                        Long runLength, unsigned long long *signal, unsigned ticket) {
     typedef typename Compute<T>::type C;
     typedef Acc3<C> Acc;
     __shared__ Acc smem[kBlock / kWave];
@@ -174,8 +175,9 @@ __global__ void __launch_bounds__(kBlock) reduce3Finish(T *z, const Acc3<typenam
     Acc3Merge<C> mg;
     acc = blockMerge<Acc3Merge<C>>(mg, acc, smem);
     if (threadIdx.x == 0) {
-        z[blockIdx.x] = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, runLength));
-        signalResult(signal, ticket);  // set only for a launch with a single result
+        const T r = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, runLength));
+        z[blockIdx.x] = r;
+        signalResult(signal, ticket, r);  // set only for a launch with a single result
     }
 }
 
@@ -331,14 +333,14 @@ template <typename T> struct Reduce3Body {
                 if (slices >= 2) {  // a single slice needs no second launch: the per-result kernels below do it in one
                     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
                     hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)(slices * pl.numOut)), dim3(kBlock), 0, s, x, y, z,
-                                       extra, pl, partials, sliceLength, slices, (unsigned *)nullptr, 0u);
+                                       extra, pl, partials, sliceLength, slices, (unsigned long long *)nullptr, 0u);
                     hipLaunchKernelGGL((reduce3Finish<T, OP>), dim3((unsigned)pl.numOut), dim3(kBlock), 0, s, z, partials, (int)slices,
                                        pl.runLength, pl.numOut == 1 ? ws.signal : nullptr, ws.ticket);
                     return true;
                 }
             }
             Acc *none = nullptr;
-            unsigned *signal = pl.numOut == 1 ? ws.signal : nullptr;
+            unsigned long long *signal = pl.numOut == 1 ? ws.signal : nullptr;
             const unsigned ticket = ws.ticket;
             if (pl.runLength >= 4096) {
                 int grid = gridFor(pl.numOut, 1, kGridCap);

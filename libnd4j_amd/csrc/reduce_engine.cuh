@@ -17,7 +17,8 @@
 //   tadColKernel<Pol>         other strided TADs and short contiguous ones: one lane per TAD; the TAD length
 //                             is split over blockIdx.y and merged by tadColFinish when split.
 //   tadGeneralKernel<Pol>     block per TAD with a coordinate map.
-//   flatKernel<Pol> + flatFinish<Pol>  two-stage grid reduction over the whole array.
+//   flatKernel<Pol>           grid reduction over the whole array; the block that finishes last merges the blocks'
+//                             results (flatFinish<Pol>: the same merge as a second launch, for callers without slots).
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -354,23 +355,92 @@ __global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typena
     }
 }
 
-// After a scalar result has been stored by this thread: make it visible to the host, then raise the caller's ticket.
-__device__ __forceinline__ void signalResult(unsigned *signal, unsigned ticket) {
+// Hands a scalar result to a host that is waiting for it: the value goes out in 8-byte words of pinned host memory, each
+// the call's ticket (upper half) with 32 bits of the value (lower half), each one system-scope store.  The host takes
+// the value once every word shows the ticket; a word is complete or absent, so no fence (on this chip: a write-back of
+// the whole L2) has to separate value and signal.
+template <typename T> __device__ __forceinline__ void signalResult(unsigned long long *signal, unsigned ticket, T value) {
     if (signal == nullptr) return;
-    __threadfence_system();
-    __hip_atomic_store(signal, ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    constexpr int W = (sizeof(T) + 3) / 4;
+    struct Words { unsigned w[W]; };
+    Words in;
+    if constexpr (sizeof(T) == 2) in.w[0] = __builtin_bit_cast(unsigned short, value);
+    else in = __builtin_bit_cast(Words, value);
+#pragma unroll
+    for (int i = 0; i < W; i++)
+        __hip_atomic_store(signal + i, ((unsigned long long)ticket << 32) | in.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
-// Stage 1 of the full-array reduction: block b folds the chunks b, b+grid, ... of kBlock*kUnroll vectors.
-// A one-block launch (small arrays) is handed the result pointer and finishes by itself.
+static constexpr unsigned kFlatGroup = 32;          // blocks per first-level counter
+static constexpr unsigned kFlatCounterStride = 32;  // counters are this many 32-bit words (128 bytes) apart
+static constexpr unsigned kFlatMaxBlocks = 2048;    // 1 + kFlatMaxBlocks / kFlatGroup counters exist
+template <typename A> __device__ __forceinline__ void publishSlots(unsigned long long *slot, const A &a, unsigned ticket) {
+    static_assert(sizeof(A) % 4 == 0, "accumulator must be a multiple of 4 bytes");
+    constexpr int W = sizeof(A) / 4;
+    struct Words { unsigned w[W]; };
+    const Words in = __builtin_bit_cast(Words, a);
+#pragma unroll
+    for (int i = 0; i < W; i++)
+        __hip_atomic_store(slot + i, ((unsigned long long)ticket << 32) | in.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// One word of a slot group: waits (bounded) until it carries `ticket`, starting from the value `v` already loaded.  Only
+// called for groups whose writer has already issued its stores, so the wait ends as soon as they land.
+__device__ __forceinline__ unsigned awaitSlot(const unsigned long long *slot, unsigned long long v, unsigned ticket) {
+    for (int tries = 0; (unsigned)(v >> 32) != ticket && tries < (1 << 22); tries++) {
+        __builtin_amdgcn_s_sleep(1);
+        v = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return (unsigned)v;
+}
+// Merges the slot groups first, first + stride, ... (count of them in all) into acc, in that order.  The loads of
+// several groups are issued together: they bypass the caches, and one after the other their latencies would add up to
+// more than the second launch they replace.
+template <class Pol>
+__device__ __forceinline__ void mergeSlots(const Pol &pol, typename Pol::Acc &acc, const unsigned long long *slots, int first,
+                                           int stride, int count, unsigned ticket) {
+    typedef typename Pol::Acc Acc;
+    constexpr int W = sizeof(Acc) / 4;
+    constexpr int G = W <= 2 ? 8 : (W <= 4 ? 4 : 2);
+    struct Words { unsigned w[W]; };
+    for (int i0 = first; i0 < count; i0 += stride * G) {
+        unsigned long long v[G][W];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const int i = i0 + g * stride;
+            if (i < count) {
+#pragma unroll
+                for (int w = 0; w < W; w++) v[g][w] = __hip_atomic_load(slots + (size_t)i * W + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const int i = i0 + g * stride;
+            if (i < count) {
+                Words out;
+#pragma unroll
+                for (int w = 0; w < W; w++) out.w[w] = awaitSlot(slots + (size_t)i * W + w, v[g][w], ticket);
+                acc = pol.combine(acc, __builtin_bit_cast(Acc, out));
+            }
+        }
+    }
+}
+
+// The full-array reduction: block b folds the chunks b, b+grid, ... of kBlock*kUnroll vectors.
+// A one-block launch (small arrays) finishes by itself.  With several blocks and `slots` given, every block publishes
+// its accumulator in its slot group and takes a number from `counter`; the block that draws the last number has seen
+// every other block issue its stores, waits for them to land, merges all groups in block order and writes the result
+// (the counters are back at zero by then): one launch.  Without `slots` the accumulators go to `partials` and flatFinish
+// merges them in a second launch.
 template <class Pol>
 __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol::T *x, typename Pol::Acc *partials,
-                                                     Long n, int strided, Long ews, DimMap xm, typename Pol::T *zDirect,
-                                                     unsigned *signal, unsigned ticket) {
+                                                     Long n, int strided, Long ews, DimMap xm, typename Pol::T *z,
+                                                     unsigned long long *signal, unsigned ticket, unsigned long long *slots,
+                                                     unsigned *counter, unsigned slotTicket) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
     __shared__ Acc smem[kBlock / kWave];
+    __shared__ int mergeHere;
     pol.setTad(0, nullptr);
     Acc acc = pol.init(x);
     if (strided && ews == 1) {
@@ -410,23 +480,52 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
             { pol.accumulate(acc, toCompute(x[mapOffsetAny(xm, i)]), i); pol.checkpoint(acc); }
     }
     acc = blockMerge<Pol>(pol, acc, smem);
-    if (threadIdx.x == 0) {
-        if (zDirect != nullptr) {
-            zDirect[0] = pol.finalize(acc, n);
-            signalResult(signal, ticket);
-        } else {
-            partials[blockIdx.x] = acc;
+    if (gridDim.x == 1) {
+        if (threadIdx.x == 0) {
+            const T r = pol.finalize(acc, n);
+            z[0] = r;
+            signalResult(signal, ticket, r);
         }
+        return;
+    }
+    if (slots == nullptr) {
+        if (threadIdx.x == 0) partials[blockIdx.x] = acc;
+        return;
+    }
+    constexpr int W = sizeof(Acc) / 4;
+    if (threadIdx.x == 0) {
+        publishSlots(slots + (size_t)blockIdx.x * W, acc, slotTicket);
+        // Atomics on one address are served one after the other, some 15 ns apiece: two thousand blocks on a single
+        // counter cost more than the reduction itself.  So blocks count in groups of kFlatGroup, each group on a counter
+        // of its own (in a memory channel of its own), and only the last block of each group goes on to the top counter.
+        const unsigned group = blockIdx.x / kFlatGroup, groups = (gridDim.x + kFlatGroup - 1) / kFlatGroup;
+        const unsigned members = group + 1 < groups ? kFlatGroup : gridDim.x - group * kFlatGroup;
+        unsigned *mine = counter + (size_t)(1 + group) * kFlatCounterStride;
+        bool last = __hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1;
+        if (last) {
+            __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1;
+            if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        mergeHere = last;
+    }
+    __syncthreads();
+    if (!mergeHere) return;
+    acc = pol.init(x);
+    mergeSlots<Pol>(pol, acc, slots, threadIdx.x, kBlock, (int)gridDim.x, slotTicket);
+    acc = blockMerge<Pol>(pol, acc, smem);
+    if (threadIdx.x == 0) {
+        const typename Pol::T r = pol.finalize(acc, n);
+        z[0] = r;
+        signalResult(signal, ticket, r);
     }
 }
 
-// Stage 2: one block merges the per-block partials.  (Doing this in the first launch, by the block that
-// arrives last at a ticket counter, needs a device-scope fence in every block; on this chip those fences cost
-// the streaming kernel more than twice its run time, a second launch costs a few microseconds.)
+// Second launch of the two-launch form: one block merges the per-block partials.
 template <class Pol>
 __global__ void __launch_bounds__(kBlock) flatFinish(Pol pol, const typename Pol::T *x, typename Pol::T *z,
-                                                     const typename Pol::Acc *partials, int count, Long n, unsigned *signal,
-                                                     unsigned ticket) {
+                                                     const typename Pol::Acc *partials, int count, Long n,
+                                                     unsigned long long *signal, unsigned ticket) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::Acc Acc;
     __shared__ Acc smem[kBlock / kWave];
@@ -435,8 +534,9 @@ __global__ void __launch_bounds__(kBlock) flatFinish(Pol pol, const typename Pol
     for (int i = threadIdx.x; i < count; i += kBlock) acc = pol.combine(acc, partials[i]);
     acc = blockMerge<Pol>(pol, acc, smem);
     if (threadIdx.x == 0) {
-        z[0] = pol.finalize(acc, n);
-        signalResult(signal, ticket);
+        const typename Pol::T r = pol.finalize(acc, n);
+        z[0] = r;
+        signalResult(signal, ticket, r);
     }
 }
 
@@ -540,14 +640,16 @@ inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, type
     typedef typename Pol::Acc Acc;
     typedef typename Pol::T T;
     Long perBlock = (Long)kBlock * kUnroll * Pack<T>::N;
-    int grid = gridFor(pl.n, perBlock, 2048);
-    size_t maxByWs = ws.bytes / sizeof(Acc);
-    if ((size_t)grid > maxByWs) grid = (int)maxByWs;
+    int grid = gridFor(pl.n, perBlock, (int)kFlatMaxBlocks);
+    const bool oneLaunch = ws.slots != nullptr && ws.counter != nullptr && ws.slotTicketSource != nullptr;
+    size_t maxBlocks = oneLaunch ? ws.slotBytes / (sizeof(Acc) / 4 * sizeof(unsigned long long)) : ws.bytes / sizeof(Acc);
+    if ((size_t)grid > maxBlocks) grid = (int)maxBlocks;
     if (grid < 1) grid = 1;
     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
     hipLaunchKernelGGL((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
-                       pl.ews, pl.xm, grid == 1 ? z : nullptr, ws.signal, ws.ticket);
-    if (grid > 1)
+                       pl.ews, pl.xm, z, ws.signal, ws.ticket, oneLaunch ? ws.slots : nullptr, ws.counter,
+                       oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u);
+    if (grid > 1 && !oneLaunch)
         hipLaunchKernelGGL((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n, ws.signal, ws.ticket);
 }
 

@@ -140,6 +140,33 @@ Workspace workspaceFor(hipStream_t s, size_t minBytes) {
 }
 
 namespace {
+struct FlatSlots {
+    void *block = nullptr;  // kFlatSlotBytes of slots, then kFlatCounterBytes of block counters
+    unsigned ticket = 0;
+};
+const size_t kFlatSlotBytes = 256u << 10;  // 2048 blocks x 16 accumulator words x 8 bytes
+const size_t kFlatCounterBytes = 16u << 10;  // 65 counters, 128 bytes apart
+std::map<std::pair<int, hipStream_t>, FlatSlots> gFlatSlots;
+}  // namespace
+
+void addFlatSlots(Workspace &w, hipStream_t s) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    std::lock_guard<std::mutex> lock(gMutex);
+    FlatSlots &f = gFlatSlots[std::make_pair(dev, s)];
+    if (f.block == nullptr) {
+        hipError_t e = hipMalloc(&f.block, kFlatSlotBytes + kFlatCounterBytes);
+        if (e != hipSuccess) { f.block = nullptr; throwHip("reduction slots allocation", e); }
+        e = hipMemset(f.block, 0, kFlatSlotBytes + kFlatCounterBytes);
+        if (e != hipSuccess) throwHip("reduction slots clearing", e);
+    }
+    w.slots = reinterpret_cast<unsigned long long *>(f.block);
+    w.slotBytes = kFlatSlotBytes;
+    w.counter = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(f.block) + kFlatSlotBytes);
+    w.slotTicketSource = &f.ticket;  // map nodes stay where they are
+}
+
+namespace {
 struct PinnedSlot {
     void *block = nullptr;  // 256 bytes: value at 0, flag word at 128
     unsigned ticket = 0;
@@ -168,44 +195,60 @@ ScalarSignal nextScalarSignal(hipStream_t s) {
     std::lock_guard<std::mutex> lock(gMutex);
     PinnedSlot &p = pinnedSlotLocked(s);
     ScalarSignal sig;
-    sig.flag = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(p.block) + 128);
+    sig.words = reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.block) + 128);
     sig.ticket = ++p.ticket;
     if (sig.ticket == 0) sig.ticket = ++p.ticket;  // zero is what a fresh slot holds
     return sig;
 }
 
-void waitForScalar(const ScalarSignal &sig, hipStream_t s, const char *what) {
+void takeScalar(const ScalarSignal &sig, hipStream_t s, const char *what, void *value, size_t bytes) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) throwHip(what, e);
-    if (sig.flag == nullptr || environment().debug.load()) {
+    const int words = (int)((bytes + 3) / 4);
+    const volatile unsigned long long *tagged = sig.words;
+    auto arrived = [&]() {
+        for (int i = 0; i < words; i++)
+            if ((unsigned)(tagged[i] >> 32) != sig.ticket) return false;
+        return true;
+    };
+    bool have = false;
+    if (sig.words == nullptr || environment().debug.load()) {
         e = hipStreamSynchronize(s);
         if (e != hipSuccess) throwHip(what, e);
-        return;
-    }
-    const volatile unsigned *flag = sig.flag;
-    // Spin on the flag alone at first (asking the runtime about the stream costs microseconds and delays the answer);
-    // a launch that failed or wrote nothing never raises the flag, so from 50 us on the stream is asked as well.
-    const auto start = std::chrono::steady_clock::now();
-    auto nextQuery = start + std::chrono::microseconds(50);
-    for (unsigned spins = 1; *flag != sig.ticket; spins++) {
+    } else {
+        // Spin on the words alone at first (asking the runtime about the stream costs microseconds and delays the answer);
+        // a launch that failed or wrote nothing never tags them, so from 50 us on the stream is asked as well.
+        const auto start = std::chrono::steady_clock::now();
+        auto nextQuery = start + std::chrono::microseconds(50);
+        for (unsigned spins = 1; !(have = arrived()); spins++) {
 #if defined(__x86_64__)
-        __builtin_ia32_pause();  // leaves the core's shared resources to a sibling thread while this one spins
+            __builtin_ia32_pause();  // leaves the core's shared resources to a sibling thread while this one spins
 #endif
-        if ((spins & 0xff) != 0) continue;
-        const auto now = std::chrono::steady_clock::now();
-        if (now < nextQuery) continue;
-        if (now - start > std::chrono::microseconds(300)) {
-            // a long kernel: wait the runtime's way (which may yield the core) rather than spin on
-            e = hipStreamSynchronize(s);
-            if (e != hipSuccess) throwHip(what, e);
-            break;
+            if ((spins & 0xff) != 0) continue;
+            const auto now = std::chrono::steady_clock::now();
+            if (now < nextQuery) continue;
+            if (now - start > std::chrono::microseconds(300)) {
+                // a long kernel: wait the runtime's way (which may yield the core) rather than spin on
+                e = hipStreamSynchronize(s);
+                if (e != hipSuccess) throwHip(what, e);
+                break;
+            }
+            e = hipStreamQuery(s);
+            if (e == hipSuccess) break;
+            if (e != hipErrorNotReady) throwHip(what, e);
+            nextQuery = now + std::chrono::microseconds(20);
         }
-        e = hipStreamQuery(s);
-        if (e == hipSuccess) break;
-        if (e != hipErrorNotReady) throwHip(what, e);
-        nextQuery = now + std::chrono::microseconds(20);
     }
     std::atomic_thread_fence(std::memory_order_acquire);
+    if (!have && sig.words != nullptr) have = arrived();  // the stream has drained: the words are there if they were written
+    if (have) {
+        unsigned w[4] = {0, 0, 0, 0};
+        for (int i = 0; i < words && i < 4; i++) w[i] = (unsigned)tagged[i];
+        std::memcpy(value, w, bytes);
+    } else {
+        // no kernel of this call tagged the words: take the plain copy at the start of the block
+        std::memcpy(value, reinterpret_cast<const char *>(sig.words) - 128, bytes);
+    }
 }
 
 bool resolveTad(Nd4jPointer *extra, int hostSlot, int offsetSlot, const Long *hostXInfo, const int *dimension,

@@ -74,20 +74,26 @@ void reportUnknownOp(const char *family, int opNum);
 
 // Device scratch owned by the library, one per (device, stream), allocated on first use and kept.
 Workspace workspaceFor(hipStream_t s, size_t minBytes);
-// 256 bytes of pinned, device-visible host memory per (device, stream): the kernels of the scalar-returning
-// entry points write their result there, so the host reads it after the stream synchronisation without a copy.
+// Adds the slots, counter and ticket of the one-launch whole-array reduction to `w`: a block of device memory per
+// (device, stream) that only those reductions use, cleared when it is allocated.  Calls on one stream run one after the
+// other, so they may share it (one host thread per stream: the ticket source is not synchronised).
+void addFlatSlots(Workspace &w, hipStream_t s);
+// 256 bytes of pinned, device-visible host memory per (device, stream): the kernels of the scalar-returning entry
+// points write their result there (plainly at offset 0, and as ticket-tagged words at offset 128), so the host reads
+// it without a copy.
 void *pinnedScalarFor(hipStream_t s);
-// The completion signal that goes with that slot: a flag word in the same pinned block and the next ticket of this
-// (device, stream).  waitForScalar returns once the flag shows the ticket (the kernel stores it after the value,
-// behind a system-scope fence) or the stream has drained, whichever the host sees first, and throws on a HIP error:
-// the host gets the value a few microseconds before the stream's own completion would reach it.  In debug mode it
-// synchronises the stream instead.
+// The hand-over that goes with that slot: the tagged words and the next ticket of this (device, stream).  The kernel
+// stores every 32 bits of the value together with the ticket in one 8-byte word; takeScalar returns once `bytes` bytes
+// of the value have arrived that way, or, failing that, once the stream has drained (then it reads the plain copy), and
+// throws on a HIP error: the host gets the value a few microseconds before the stream's own completion would reach it.
+// Everything enqueued earlier on the stream has completed by then (stream order).  In debug mode it synchronises the
+// stream instead.  One host thread per stream: two threads on one stream would share the slot and the tickets.
 struct ScalarSignal {
-    unsigned *flag = nullptr;
+    unsigned long long *words = nullptr;
     unsigned ticket = 0;
 };
 ScalarSignal nextScalarSignal(hipStream_t s);
-void waitForScalar(const ScalarSignal &sig, hipStream_t s, const char *what);
+void takeScalar(const ScalarSignal &sig, hipStream_t s, const char *what, void *value, size_t bytes);
 
 // TAD tables resolved for a call: host shapeInfo of one TAD + device offsets.
 struct ResolvedTad {
