@@ -2,21 +2,27 @@
 // Reference: include/loops/cpu/summarystatsreduce.cpp:24-196; moment merge
 // include/loops/summarystatsreduce.h:221-257 (Chan et al. parallel update); getValue include/ops/ops.h:3471-3509.
 //
-// Each lane gathers short runs of samples as shifted sums (count, sum(x-c), sum((x-c)^2) around the run's
-// first sample c), turns a full run into (n, mean, M2) and merges it with the pairwise formula the
-// reference applies sample by sample.  Only n, mean and M2 are carried: min/max/M3/M4 never reach
-// variance or standard deviation.
+// Each lane gathers runs of samples as shifted sums (count, sum(x-c), sum((x-c)^2) around a shift c), turns a closed
+// run into (n, mean, M2) and merges it with the pairwise formula the reference applies sample by sample.  Only n,
+// mean and M2 are carried: min/max/M3/M4 never reach variance or standard deviation.
+//
+// The shift is a sample of the same TAD (its first one) until a lane closes a run, the merged mean afterwards.  With
+// M2 = sum(e^2) - (sum e)^2 / n the cancellation is 1 + (mean(e) / sigma)^2, at worst the run length + 1 (every sample
+// equal but the one that became the shift): runs of up to kStatsRun samples lose at most 2^17 of double precision's
+// 2^53.  So a lane rarely closes a run before the merge, and lanes that have not merge by adding their sums.
 #include "launch.h"
 #include "reduce_engine.cuh"
 
 namespace nd4j_amd {
 
 struct StatsAcc {
-    double n, mean, m2;      // merged so far
-    double cn, cs1, cs2, cp; // current run: count, shifted sums, shift
+    double n, mean, m2;  // merged so far
+    double cs1, cs2;     // current run: sum(x - cp), sum((x - cp)^2)
+    double cp;           // current shift (a value the data type holds exactly)
+    int cn, pad;         // current run: count
 };
 
-static constexpr double kStatsRun = 128.0;
+static constexpr int kStatsRun = 65536;
 
 __device__ __forceinline__ void statsMerge(double &n, double &mean, double &m2, double nb, double meanb, double m2b) {
     if (nb == 0.0) return;
@@ -27,13 +33,16 @@ __device__ __forceinline__ void statsMerge(double &n, double &mean, double &m2, 
     m2 = m2 + m2b + delta * delta * n * nb / tot;
     n = tot;
 }
-__device__ __forceinline__ void statsFlush(StatsAcc &a) {
-    if (a.cn == 0.0) return;
-    double meanb = a.cp + a.cs1 / a.cn;
-    double m2b = a.cs2 - a.cs1 * a.cs1 / a.cn;
+// closes the current run; the next one is shifted by the merged mean, rounded to what the data type holds
+template <typename C> __device__ __forceinline__ void statsFlush(StatsAcc &a) {
+    if (a.cn == 0) return;
+    const double cn = (double)a.cn;
+    double meanb = a.cp + a.cs1 / cn;
+    double m2b = a.cs2 - a.cs1 * a.cs1 / cn;
     if (m2b < 0.0) m2b = 0.0;
-    statsMerge(a.n, a.mean, a.m2, a.cn, meanb, m2b);
-    a.cn = 0.0; a.cs1 = 0.0; a.cs2 = 0.0;
+    statsMerge(a.n, a.mean, a.m2, cn, meanb, m2b);
+    a.cn = 0; a.cs1 = 0.0; a.cs2 = 0.0;
+    a.cp = (double)(C)a.mean;
 }
 
 template <typename TT, int OP> struct StatsPol {
@@ -46,50 +55,51 @@ template <typename TT, int OP> struct StatsPol {
 
     __device__ __forceinline__ void setTad(Long, const TT *) {}
     // Every lane's first run is shifted by the same value, the first sample of the TAD (of the array): lanes that have
-    // not closed a run yet then merge by adding their three sums (combine), which is what the merge tree of a short
-    // TAD consists of.  A run opened after a merge is shifted by its own first sample, as before.
+    // not closed a run yet then merge by adding their sums (combine), which is what the merge tree consists of.
     __device__ __forceinline__ Acc init(const TT *first) const {
         Acc a;
         a.n = a.mean = a.m2 = 0.0;
-        a.cn = a.cs1 = a.cs2 = 0.0;
+        a.cs1 = a.cs2 = 0.0;
+        a.cn = a.pad = 0;
         a.cp = (double)toCompute(first[0]);
         return a;
     }
+    // The difference to the shift is taken in the compute type: shift and sample are both values of that type, and where
+    // the difference matters (samples close to the shift) it is exact; sums and squares are kept in double.
     __device__ __forceinline__ void accumulate(Acc &a, C v, Long) const {
-        double d = (double)v;
-        if (a.cn == 0.0 && a.n != 0.0) a.cp = d;
-        double e = d - a.cp;
+        const double e = (double)(v - (C)a.cp);
         a.cs1 += e;
-        a.cs2 += e * e;
-        a.cn += 1.0;
+        a.cs2 = __builtin_fma(e, e, a.cs2);
+        a.cn += 1;
     }
     // closes the current run once it holds kStatsRun samples or more (kept out of accumulate() so that the
     // per-sample code is straight-line)
     __device__ __forceinline__ void checkpoint(Acc &a) const {
-        if (a.cn >= kStatsRun) statsFlush(a);
+        if (a.cn >= kStatsRun) statsFlush<C>(a);
     }
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const {
-        if (a.n == 0.0 && b.n == 0.0 && a.cp == b.cp) {  // two open first runs around the common shift: no divisions
+        // two open first runs around the common shift: no divisions (the count is a 32-bit integer: longer runs are closed)
+        if (a.n == 0.0 && b.n == 0.0 && a.cp == b.cp && a.cn <= (1 << 29) && b.cn <= (1 << 29)) {
             a.cn += b.cn;
             a.cs1 += b.cs1;
             a.cs2 += b.cs2;
             return a;
         }
-        statsFlush(a);
-        statsFlush(b);
+        statsFlush<C>(a);
+        statsFlush<C>(b);
         statsMerge(a.n, a.mean, a.m2, b.n, b.mean, b.m2);
         return a;
     }
-    // While no lane of the wave has closed a run, every lane holds three sums around the TAD's common shift: those are
-    // all that has to travel (6 words per step instead of 14), and they merge by addition.
+    // While no lane of the wave has closed a run, every lane holds two sums and a count around the TAD's common shift:
+    // those are all that has to travel (5 words per step instead of 16), and they merge by addition.
     static constexpr bool ownWaveMerge = true;
     template <int WIDTH> __device__ __forceinline__ Acc waveMergeOwn(Acc a) const {
-        if (__all(a.n == 0.0)) {
+        if (__all(a.n == 0.0 && a.cn <= (1 << 24))) {
 #pragma unroll
             for (int d = WIDTH / 2; d >= 1; d >>= 1) {
                 // (lanes of one segment work on one TAD and share its shift; what arrives from beyond the segment's end
                 // lands in lanes whose result is not used)
-                a.cn += shflDownAny(a.cn, d);
+                a.cn += __shfl_down(a.cn, d, kWave);
                 a.cs1 += shflDownAny(a.cs1, d);
                 a.cs2 += shflDownAny(a.cs2, d);
             }
@@ -100,7 +110,7 @@ template <typename TT, int OP> struct StatsPol {
         return a;
     }
     __device__ __forceinline__ TT finalize(Acc a, Long) const {
-        statsFlush(a);
+        statsFlush<C>(a);
         if (phantomZero) {
             double n = 1.0, mean = 0.0, m2 = 0.0;
             statsMerge(n, mean, m2, a.n, a.mean, a.m2);
