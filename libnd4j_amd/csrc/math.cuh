@@ -41,6 +41,42 @@ __device__ __forceinline__ float cos_(float v) {
 }
 __device__ __forceinline__ double cos_(double v) { return ::cos(v); }
 
+// exp for the softmax family (arguments x - max <= 0): 2^(v log2 e) on the hardware's exp2 with the product carried as a
+// rounded part and its exact remainder, about 1.5 ULP.  Those ops are held to the 1e-5 of reductions (their row sums
+// are re-associated anyway), and the C library's algorithm, replayed bit for bit in exp_, costs four times as many
+// instructions - which is what bounded every softmax kernel.  Below -87 the result is a denormal, or zero from where
+// the C library's is (-103.972): it is computed 2^64 times too large and scaled down by a multiplication, which rounds
+// it into the denormal range once.  NaN stays NaN.
+__device__ __forceinline__ float expSoftCore_(float v) {
+    const float l2eHi = 1.44269502162933349609375f, l2eLo = 1.925963033500011e-8f, ln2 = 0.693147182464599609375f;
+    const float t = v * l2eHi;
+    float r = __builtin_fmaf(v, l2eHi, -t);
+    r = __builtin_fmaf(v, l2eLo, r);
+    const float p = __builtin_amdgcn_exp2f(t);
+    return __builtin_fmaf(p, r * ln2, p);
+}
+__device__ __forceinline__ float expSoft_(float v) {
+    const bool far = !(v >= -87.0f);
+    // a branch on the whole wave (so that it stays a branch): the shifted argument and the scale for the lanes that need them
+    float scale = 1.0f;
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(far) != 0ull, 0)) {
+        if (far) { v += 44.3614196f; scale = 0x1p-64f; }  // 64 ln 2; NaN stays NaN, what lies below -103.972 rounds to zero below
+        const float r = expSoftCore_(v) * scale;
+        return (far && v < -103.972084f + 44.3614196f) ? 0.0f : r;
+    }
+    return expSoftCore_(v);
+}
+__device__ __forceinline__ double expSoft_(double v) { return ::exp(v); }
+// log to go with it: the hardware's log2 (1 ULP) times ln 2; denormal arguments are scaled into the normal range first
+__device__ __forceinline__ float logSoft_(float v) {
+    const float ln2 = 0.693147182464599609375f;
+    const bool tiny = v < 1.17549435e-38f;
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(tiny) != 0ull, 0))  // 0 -> -inf, negative -> NaN
+        return (__builtin_amdgcn_logf(tiny ? v * 0x1p64f : v) - (tiny ? 64.0f : 0.0f)) * ln2;
+    return __builtin_amdgcn_logf(v) * ln2;
+}
+__device__ __forceinline__ double logSoft_(double v) { return ::log(v); }
+
 ND4J_VIA_DOUBLE(tan_, tan)
 ND4J_VIA_DOUBLE(cosh_, cosh)
 ND4J_VIA_DOUBLE(sinh_, sinh)

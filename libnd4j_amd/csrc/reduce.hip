@@ -169,7 +169,7 @@ template <typename TT> struct SoftmaxStatsPol {
     typedef TT T;
     typedef typename Compute<TT>::type C;
     struct Acc { C m, s; };
-    static constexpr bool tables = true;
+    static constexpr bool tables = false;  // its exp runs on the hardware's exp2
     C *sums;  // in the compute type: a row sum of a half array may exceed the range of half
     Long row;
 
@@ -182,7 +182,7 @@ template <typename TT> struct SoftmaxStatsPol {
     }
     __device__ __forceinline__ void accumulate(Acc &a, C v, Long) const {
         const C d = v - a.m;
-        const C e = m::exp_(-m::abs_(d));
+        const C e = m::expSoft_(-m::abs_(d));
         const bool rises = d > (C)0;
         a.s = rises ? a.s * e + (C)1 : a.s + e;
         a.m = rises ? v : a.m;
@@ -192,7 +192,7 @@ template <typename TT> struct SoftmaxStatsPol {
         Acc r;
         r.m = m::max_(a.m, b.m);
         // an accumulator that has seen nothing yet holds s == 0 and the row's first element as m
-        r.s = a.s * m::exp_(a.m - r.m) + b.s * m::exp_(b.m - r.m);
+        r.s = a.s * m::expSoft_(a.m - r.m) + b.s * m::expSoft_(b.m - r.m);
         return r;
     }
     __device__ __forceinline__ TT finalize(Acc a, Long) const {

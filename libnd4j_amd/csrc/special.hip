@@ -35,19 +35,68 @@ template <typename C> __device__ __forceinline__ C laneBroadcast(C v, int srcLan
 // MODE 0: softmax, 1: softmax * (1 - softmax), 2: log(softmax)
 // `inv` is 1 / sum, taken once per row: multiplying by it is within 1 ULP of dividing every element by the sum (what
 // the reference's loops say; its build allows the compiler the same substitution), far inside the tolerance that the
-// re-associated row sum already needs
+// re-associated row sum already needs.
 template <int MODE, typename C> __device__ __forceinline__ C softmaxFinish(C e, C inv) {
     C v = e * inv;
     if (MODE == 1) return v * ((C)1 - v);
-    if (MODE == 2) return m::log_(v);
+    if (MODE == 2) return m::logSoft_(v);
     return v;
+}
+// log(sum) where the logarithm needs it
+template <int MODE, typename C> __device__ __forceinline__ C rowLog(C sum) { return MODE == 2 ? m::logSoft_(sum) : (C)0; }
+// The result for an element d = x - max below its row's maximum.  The logarithm of exp(d) / sum is d - log(sum): one
+// logarithm a row (`logSum`) instead of one an element, and no exp.  Where exp(d) has left the normal range (d < -87)
+// the reference's quotient is a denormal or zero, and its logarithm is taken as the reference takes it.
+template <int MODE, typename C> __device__ __forceinline__ C softmaxAt(C d, C inv, C logSum) {
+    if (MODE == 2) {
+        const bool far = d < (C)-87;
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(far) != 0ull, 0)) {  // a branch on the whole wave, so that it stays a branch
+            const C viaExp = m::logSoft_(m::expSoft_(d) * inv);
+            return far ? viaExp : d - logSum;
+        }
+        return d - logSum;
+    }
+    return softmaxFinish<MODE, C>(m::expSoft_(d), inv);
+}
+// what the register-resident kernels keep of an element between the pass that sums and the pass that writes: e = exp(d),
+// or d itself for the logarithm (which needs e only for the sum)
+template <int MODE, typename C> __device__ __forceinline__ C softmaxKeep(C e, C d) { return MODE == 2 ? d : e; }
+template <int MODE, typename C> __device__ __forceinline__ C softmaxFromKept(C kept, C inv, C logSum) {
+    if (MODE == 2) return softmaxAt<2, C>(kept, inv, logSum);
+    return softmaxFinish<MODE, C>(kept, inv);
+}
+// A whole vector of kept values into results; inv and logSum per element (PER true: arrays) or one for all.  The
+// logarithm's rare detour (an element more than 87 below its maximum) is looked for once per vector, not per element.
+template <typename T, int MODE, bool PER, typename C>
+__device__ __forceinline__ Pack<T> softmaxPackFromKept(const Pack<T> &kept, const C *inv, const C *logSum) {
+    constexpr int N = Pack<T>::N;
+    Pack<T> o;
+    if (MODE != 2) {
+#pragma unroll
+        for (int e = 0; e < N; e++) o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(toCompute(kept.v[e]), inv[PER ? e : 0]));
+        return o;
+    }
+    bool far = false;
+#pragma unroll
+    for (int e = 0; e < N; e++) {
+        const C d = toCompute(kept.v[e]);
+        far = far || d < (C)-87;
+        o.v[e] = fromCompute<T>(d - logSum[PER ? e : 0]);
+    }
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(far) != 0ull, 0)) {
+#pragma unroll
+        for (int e = 0; e < N; e++) {
+            const C d = toCompute(kept.v[e]);
+            if (d < (C)-87) o.v[e] = fromCompute<T>(m::logSoft_(m::expSoft_(d) * inv[PER ? e : 0]));
+        }
+    }
+    return o;
 }
 
 // Rows whose elements are `xEl` / `zEl` apart, row r starting at r * xRow / r * zRow; GROUP lanes per row.
 template <typename T, int MODE, int GROUP>
 __global__ void __launch_bounds__(kBlock) softmaxRowKernel(const T *x, T *z, Long numRows, Long length, Long xRow, Long xEl,
                                                            Long zRow, Long zEl) {
-    lm::loadTables();
     typedef typename Compute<T>::type C;
     constexpr int GROUPS = kBlock / GROUP;
     __shared__ C smem[kBlock / kWave];
@@ -76,7 +125,7 @@ __global__ void __launch_bounds__(kBlock) softmaxRowKernel(const T *x, T *z, Lon
         }
         C sum = (C)0;
         if (live)
-            for (Long c = lane; c < length; c += GROUP) sum += m::exp_(toCompute(xr[c * xEl]) - mx);
+            for (Long c = lane; c < length; c += GROUP) sum += m::expSoft_(toCompute(xr[c * xEl]) - mx);
         if (GROUP == kBlock) {
             SumMerge<C> mg;
             sum = blockMerge<SumMerge<C>>(mg, sum, smem);
@@ -89,10 +138,11 @@ __global__ void __launch_bounds__(kBlock) softmaxRowKernel(const T *x, T *z, Lon
             sum = waveMerge<SumMerge<C>, GROUP>(mg, sum);
             sum = laneBroadcast(sum, 0, GROUP);
         }
+        const C logSum = rowLog<MODE, C>(sum);
         sum = (C)1 / sum;
         if (live)
             for (Long c = lane; c < length; c += GROUP)
-                zr[c * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(xr[c * xEl]) - mx), sum));
+                zr[c * zEl] = fromCompute<T>(softmaxAt<MODE, C>(toCompute(xr[c * xEl]) - mx, sum, logSum));
         if (GROUP == kBlock) __syncthreads();
     }
 }
@@ -102,7 +152,6 @@ __global__ void __launch_bounds__(kBlock) softmaxRowKernel(const T *x, T *z, Lon
 template <typename T, int MODE>
 __global__ void __launch_bounds__(kBlock) softmaxColKernel(const T *x, T *z, Long numRows, Long length, Long xRow, Long xEl,
                                                            Long zRow, Long zEl) {
-    lm::loadTables();
     typedef typename Compute<T>::type C;
     constexpr int WAVES = kBlock / kWave;
     __shared__ C smem[WAVES][kWave];
@@ -132,27 +181,28 @@ __global__ void __launch_bounds__(kBlock) softmaxColKernel(const T *x, T *z, Lon
         for (; c + 3 * WAVES < length; c += 4 * WAVES) {
             C v0 = toCompute(xr[c * xEl]), v1 = toCompute(xr[(c + WAVES) * xEl]), v2 = toCompute(xr[(c + 2 * WAVES) * xEl]),
               v3 = toCompute(xr[(c + 3 * WAVES) * xEl]);
-            sum += (m::exp_(v0 - mx) + m::exp_(v1 - mx)) + (m::exp_(v2 - mx) + m::exp_(v3 - mx));
+            sum += (m::expSoft_(v0 - mx) + m::expSoft_(v1 - mx)) + (m::expSoft_(v2 - mx) + m::expSoft_(v3 - mx));
         }
-        for (; c < length; c += WAVES) sum += m::exp_(toCompute(xr[c * xEl]) - mx);
+        for (; c < length; c += WAVES) sum += m::expSoft_(toCompute(xr[c * xEl]) - mx);
     }
     smem[wave][lane] = sum;
     __syncthreads();
     sum = (C)0;
 #pragma unroll
     for (int w = 0; w < WAVES; w++) sum += smem[w][lane];
+    const C logSum = rowLog<MODE, C>(sum);
     sum = (C)1 / sum;
     if (live) {
         Long c = wave;
         for (; c + 3 * WAVES < length; c += 4 * WAVES) {
             C v0 = toCompute(xr[c * xEl]), v1 = toCompute(xr[(c + WAVES) * xEl]), v2 = toCompute(xr[(c + 2 * WAVES) * xEl]),
               v3 = toCompute(xr[(c + 3 * WAVES) * xEl]);
-            zr[c * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(v0 - mx), sum));
-            zr[(c + WAVES) * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(v1 - mx), sum));
-            zr[(c + 2 * WAVES) * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(v2 - mx), sum));
-            zr[(c + 3 * WAVES) * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(v3 - mx), sum));
+            zr[c * zEl] = fromCompute<T>(softmaxAt<MODE, C>(v0 - mx, sum, logSum));
+            zr[(c + WAVES) * zEl] = fromCompute<T>(softmaxAt<MODE, C>(v1 - mx, sum, logSum));
+            zr[(c + 2 * WAVES) * zEl] = fromCompute<T>(softmaxAt<MODE, C>(v2 - mx, sum, logSum));
+            zr[(c + 3 * WAVES) * zEl] = fromCompute<T>(softmaxAt<MODE, C>(v3 - mx, sum, logSum));
         }
-        for (; c < length; c += WAVES) zr[c * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(xr[c * xEl]) - mx), sum));
+        for (; c < length; c += WAVES) zr[c * zEl] = fromCompute<T>(softmaxAt<MODE, C>(toCompute(xr[c * xEl]) - mx, sum, logSum));
     }
 }
 
@@ -194,7 +244,6 @@ template <class Merge, int GROUP, typename C> __device__ __forceinline__ C teamA
 // (BLOCK: threads of a block, a multiple of GROUP; the 1024-thread blocks serve the longest rows, one team a block.)
 template <typename T, int MODE, int GROUP, int PACKS, bool EDGES, int BLOCK = kBlock>
 __global__ void __launch_bounds__(BLOCK) softmaxRowRegKernel(const T *x, T *z, Long numRows, Long length, Long xRow, Long zRow) {
-    lm::loadTables();
     typedef typename Compute<T>::type C;
     constexpr int N = Pack<T>::N;
     constexpr int GROUPS = BLOCK / GROUP;
@@ -230,48 +279,62 @@ __global__ void __launch_bounds__(BLOCK) softmaxRowRegKernel(const T *x, T *z, L
         mx = teamAll<MaxMerge<C>, GROUP>(mx, smem);
         C sum = (C)0;
         if (hasEdge) {
-            edge = toCompute(fromCompute<T>(m::exp_(edge - mx)));  // rounded to T like the cached ones
-            sum = edge;
+            const C d = edge - mx, ex = m::expSoft_(d);
+            sum = toCompute(fromCompute<T>(ex));  // rounded to T like the cached ones
+            edge = toCompute(fromCompute<T>(softmaxKeep<MODE, C>(ex, d)));
         }
 #pragma unroll
         for (int j = 0; j < PACKS; j++)
             if (live && lane + j * GROUP < npack) {
 #pragma unroll
                 for (int e = 0; e < N; e++) {
-                    const C ex = m::exp_(toCompute(cache[j].v[e]) - mx);
+                    const C d = toCompute(cache[j].v[e]) - mx, ex = m::expSoft_(d);
                     sum += ex;
-                    cache[j].v[e] = fromCompute<T>(ex);
+                    cache[j].v[e] = fromCompute<T>(softmaxKeep<MODE, C>(ex, d));
                 }
             }
         sum = teamAll<SumMerge<C>, GROUP>(sum, smem);
+        const C logSum = rowLog<MODE, C>(sum);
         sum = (C)1 / sum;
 #pragma unroll
         for (int j = 0; j < PACKS; j++)
             if (live && lane + j * GROUP < npack) {
-                Pack<T> o;
-#pragma unroll
-                for (int e = 0; e < N; e++) o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(toCompute(cache[j].v[e]), sum));
-                storePack(zr + lane + j * GROUP, o);
+                storePack(zr + lane + j * GROUP, softmaxPackFromKept<T, MODE, false, C>(cache[j], &sum, &logSum));
             }
-        if (hasEdge) zrow[edgeAt] = fromCompute<T>(softmaxFinish<MODE, C>(edge, sum));
+        if (hasEdge) zrow[edgeAt] = fromCompute<T>(softmaxFromKept<MODE, C>(edge, sum, logSum));
     }
 }
 
 // Rows adjacent in memory (an f-order matrix) and at most kColCols * PACKS columns: a 1024-thread block owns
-// 8 * Pack::N neighbouring rows - eight row lanes, each loading Pack::N rows of one column as one 16-byte vector,
-// times 128 column groups - and keeps all of it in registers (PACKS vectors a thread).  Row maxima and sums are
-// merged over the column groups with three butterfly steps inside a wave and through LDS across the 16 waves.
+// 8 * Pack::N neighbouring rows at a time - eight row lanes, each loading Pack::N rows of one column as one 16-byte
+// vector (a whole 128-byte line between them), times 128 column groups - and keeps all of it in registers (PACKS vectors
+// a thread).  Row maxima and sums are merged over the column groups with three butterfly steps inside a wave and
+// through LDS across the 16 waves.
+//
+// Such a block fills a compute unit, and it loads, then computes, then stores, all 16 waves in step: the unit's memory
+// pipes idle while it computes.  Two smaller blocks per unit would overlap, but the registers of a unit hold 32 rows of
+// 2048 floats only once; 512-thread blocks of 16 rows (half a 128-byte line per request) were slower by a third even
+// with neighbouring groups of rows placed on one die, and persistent blocks that issue the next group's loads behind
+// the current group's stores were slower by a tenth.  What is left to this layout is to keep the arithmetic short.
 static constexpr int kColBlock = 1024, kColRowLanes = 8, kColCols = kColBlock / kColRowLanes;
 template <typename T, int MODE, int PACKS>
-__global__ void __launch_bounds__(kColBlock) softmaxColRegKernel(const T *x, T *z, Long numRows, Long length, Long xEl, Long zEl) {
-    lm::loadTables();
+__global__ void __launch_bounds__(kColBlock) softmaxColRegKernel(const T *x, T *z, Long numRows, Long length, Long xEl, Long zEl,
+                                                                 Long groups) {
     typedef typename Compute<T>::type C;
     constexpr int N = Pack<T>::N;
     constexpr int WAVES = kColBlock / kWave;
     __shared__ C smax[WAVES][kColRowLanes][N], ssum[WAVES][kColRowLanes][N];
     const int rl = threadIdx.x % kColRowLanes, cg = threadIdx.x / kColRowLanes;
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const Long row0 = ((Long)blockIdx.x * kColRowLanes + rl) * N;  // numRows is a multiple of N: a vector is all live or all dead
+    // (the LDS arrays need no barrier between two rounds: who writes smax again has passed the second barrier of the
+    // round before, behind which nobody reads it; who writes ssum again has passed the first barrier of this round)
+    const int cg0 = cg;
+    for (Long g = blockIdx.x; g < groups; g += gridDim.x) {
+    // (opaque to the optimiser, which would otherwise carry the sixteen column offsets through the loop in registers
+    // that the row data needs)
+    int cg = cg0;
+    asm volatile("" : "+v"(cg));
+    const Long row0 = (g * kColRowLanes + rl) * N;  // numRows is a multiple of N: a vector is all live or all dead
     const bool live = row0 < numRows;
     Pack<T> cache[PACKS];
 #pragma unroll
@@ -308,9 +371,9 @@ __global__ void __launch_bounds__(kColBlock) softmaxColRegKernel(const T *x, T *
         if (live && cg + j * kColCols < length) {
 #pragma unroll
             for (int e = 0; e < N; e++) {
-                const C ex = m::exp_(toCompute(cache[j].v[e]) - mx[e]);
+                const C d = toCompute(cache[j].v[e]) - mx[e], ex = m::expSoft_(d);
                 sum[e] += ex;
-                cache[j].v[e] = fromCompute<T>(ex);
+                cache[j].v[e] = fromCompute<T>(softmaxKeep<MODE, C>(ex, d));
             }
         }
 #pragma unroll
@@ -330,16 +393,16 @@ __global__ void __launch_bounds__(kColBlock) softmaxColRegKernel(const T *x, T *
 #pragma unroll
         for (int e = 0; e < N; e++) sum[e] += ssum[w][rl][e];
     }
+    C logSum[N];
 #pragma unroll
-    for (int e = 0; e < N; e++) sum[e] = (C)1 / sum[e];
+    for (int e = 0; e < N; e++) { logSum[e] = rowLog<MODE, C>(sum[e]); sum[e] = (C)1 / sum[e]; }
 #pragma unroll
     for (int j = 0; j < PACKS; j++)
         if (live && cg + j * kColCols < length) {
-            Pack<T> o;
-#pragma unroll
-            for (int e = 0; e < N; e++) o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(toCompute(cache[j].v[e]), sum[e]));
-            storePack(reinterpret_cast<Pack<T> *>(z + row0 + (Long)(cg + j * kColCols) * zEl), o);
+            storePack(reinterpret_cast<Pack<T> *>(z + row0 + (Long)(cg + j * kColCols) * zEl),
+                      softmaxPackFromKept<T, MODE, true, C>(cache[j], sum, logSum));
         }
+    }
 }
 
 template <typename T> static bool aligned16(const T *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -357,9 +420,10 @@ template <typename T, int MODE, int GROUP, int PACKS, int BLOCK = kBlock> void r
 }
 template <typename T, int MODE, int PACKS> void runColReg(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
     const Long rowsPerBlock = (Long)kColRowLanes * Pack<T>::N;
-    int grid = (int)((pl.numRows + rowsPerBlock - 1) / rowsPerBlock);
+    const Long groups = (pl.numRows + rowsPerBlock - 1) / rowsPerBlock;
+    const int grid = (int)(groups < (Long)kMaxGrid / 4 ? groups : (Long)kMaxGrid / 4);  // blocks of 1024 threads walk the rest
     hipLaunchKernelGGL((softmaxColRegKernel<T, MODE, PACKS>), dim3(grid), dim3(kColBlock), 0, s, x, z, pl.numRows, pl.length, pl.xEl,
-                       pl.zEl);
+                       pl.zEl, groups);
 }
 
 // The widest team of the rows-in-registers kernel, and the vectors each of its lanes keeps: a 1024-thread block leaves
@@ -388,7 +452,7 @@ template <typename T> SoftmaxRoute softmaxRoute(const T *x, const T *z, const So
     if (!(aligned16(x) && aligned16(z))) return SM_PASSES;
     // an f-order matrix whose column stride keeps the row vectors aligned
     if (pl.xRow == 1 && pl.zRow == 1 && pl.numRows % N == 0 && pl.xEl % N == 0 && pl.zEl % N == 0 && pl.numRows >= kWave &&
-        pl.length <= (Long)kColCols * kColPacks && (Long)((pl.numRows + 8 * N - 1) / (8 * N)) <= kMaxGrid / 4)  // blocks of 1024 threads
+        pl.length <= (Long)kColCols * kColPacks && true)
         return SM_COL_REGISTERS;
     return SM_PASSES;
 }
@@ -450,13 +514,12 @@ __global__ void __launch_bounds__(kBlock) softmaxFinishKernel(const T *x, T *z, 
                                                               const typename Compute<T>::type *sums, Long numRows,
                                                               Long length, Long xRow, Long xEl, Long zRow, Long zEl, int alongRows) {
     typedef typename Compute<T>::type C;
-    lm::loadTables();
     const Long fastLen = alongRows ? numRows : length, slowLen = alongRows ? length : numRows;
     for (Long sl = blockIdx.y; sl < slowLen; sl += gridDim.y) {
         for (Long f = (Long)blockIdx.x * kBlock + threadIdx.x; f < fastLen; f += (Long)gridDim.x * kBlock) {
             const Long r = alongRows ? f : sl, c = alongRows ? sl : f;
-            const C e = m::exp_(toCompute(x[r * xRow + c * xEl]) - toCompute(maxima[r]));
-            z[r * zRow + c * zEl] = fromCompute<T>(softmaxFinish<MODE, C>(e, (C)1 / sums[r]));
+            const C d = toCompute(x[r * xRow + c * xEl]) - toCompute(maxima[r]);
+            z[r * zRow + c * zEl] = fromCompute<T>(softmaxAt<MODE, C>(d, (C)1 / sums[r], rowLog<MODE, C>(sums[r])));
         }
     }
 }
@@ -486,12 +549,13 @@ template <typename T, int MODE, int ALONG> struct SoftmaxFinishItem {
     __device__ __forceinline__ void finish(T *z, Long zSlow) const {
         constexpr int N = Pack<T>::N;
         Pack<T> o;
-        const C inv = ALONG == 1 ? (C)0 : (C)1 / sum;
+        const C inv = ALONG == 1 ? (C)0 : (C)1 / sum, logInv = ALONG == 1 ? (C)0 : rowLog<MODE, C>(sum);
 #pragma unroll
         for (int e = 0; e < N; e++) {
             const C m1 = ALONG == 1 ? toCompute(pm.v[e]) : mx;
             const C i1 = ALONG == 1 ? (C)1 / ps[e] : inv;
-            o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(a.v[e]) - m1), i1));
+            const C logSum = ALONG == 1 ? rowLog<MODE, C>(ps[e]) : logInv;
+            o.v[e] = fromCompute<T>(softmaxAt<MODE, C>(toCompute(a.v[e]) - m1, i1, logSum));
         }
         storePack(reinterpret_cast<Pack<T> *>(z + sl * zSlow) + v, o);
     }
@@ -506,7 +570,6 @@ __global__ void __launch_bounds__(kBlock) softmaxFinishVecKernel(const T *x, T *
     SoftmaxFinishItem<T, MODE, ALONG> cur, next;
     bool have = id < total;
     if (have) cur.load(id, small, x, maxima, sums, fastVecs, xSlow);
-    lm::loadTables();
     while (have) {
         id += stride;
         const bool more = id < total;
@@ -526,11 +589,10 @@ __global__ void __launch_bounds__(kBlock) softmaxFinishRowsKernel(const T *x, T 
                                                                   Long xRow, Long zRow) {
     typedef typename Compute<T>::type C;
     constexpr int N = Pack<T>::N;
-    lm::loadTables();
     for (Long r = blockIdx.y; r < numRows; r += gridDim.y) {
         const T *xr = x + r * xRow;
         T *zr = z + r * zRow;
-        const C mx = toCompute(maxima[r]), inv = (C)1 / sums[r];
+        const C mx = toCompute(maxima[r]), inv = (C)1 / sums[r], logSum = rowLog<MODE, C>(sums[r]);
         Long head = (Long)(((16 - (reinterpret_cast<uintptr_t>(xr) & 15)) & 15) / sizeof(T));
         if (head > length) head = length;
         const Long nvec = (length - head) / N;
@@ -540,7 +602,7 @@ __global__ void __launch_bounds__(kBlock) softmaxFinishRowsKernel(const T *x, T 
             const Pack<T> a = loadPack(xv + v);
             Pack<T> o;
 #pragma unroll
-            for (int e = 0; e < N; e++) o.v[e] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(a.v[e]) - mx), inv));
+            for (int e = 0; e < N; e++) o.v[e] = fromCompute<T>(softmaxAt<MODE, C>(toCompute(a.v[e]) - mx, inv, logSum));
             storePack(zv + v, o);
         }
         if (blockIdx.x == 0) {
@@ -548,7 +610,7 @@ __global__ void __launch_bounds__(kBlock) softmaxFinishRowsKernel(const T *x, T 
             const Long tail0 = head + nvec * N;
             for (Long f = threadIdx.x; f < head + (length - tail0); f += kBlock) {
                 const Long c = f < head ? f : tail0 + (f - head);
-                zr[c] = fromCompute<T>(softmaxFinish<MODE, C>(m::exp_(toCompute(xr[c]) - mx), inv));
+                zr[c] = fromCompute<T>(softmaxAt<MODE, C>(toCompute(xr[c]) - mx, inv, logSum));
             }
         }
     }
