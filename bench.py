@@ -229,7 +229,7 @@ def main():
                     ("half", lambda d: workloads.pairwise_broadcast(d, dtype="float16")),
                     ("reductions", workloads.reductions), ("reduce3", workloads.reduce3_pairs),
                     ("stats", workloads.stats_softmax), ("random", workloads.random_fills),
-                    ("movement", workloads.data_movement)]
+                    ("movement", workloads.data_movement), ("whole", workloads.whole_array_transforms)]
         only = [o for o in args.only.split(",") if o]
         for key, build in builders:
             if only and key not in only:

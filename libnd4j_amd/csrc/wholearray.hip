@@ -171,23 +171,29 @@ __global__ void __launch_bounds__(kBlock) clearCountsKernel(unsigned *counts, in
 }
 
 // Counts per block in LDS (when the bins fit), flushed with one atomic per non-empty bin; otherwise atomics on the
-// global counters directly.
+// global counters directly.  LDS atomics of one wave on one address are served one after the other, and with few bins
+// most lanes of a wave meet in the same few: the block then keeps several copies of the bins (as many as fit, up to
+// 32), lane l counting in copy l % copies, and adds the copies up when it flushes.
 constexpr int kLdsBins = 8192;
 template <typename T, bool LDS>
 __global__ void __launch_bounds__(kBlock) histogramCountKernel(const T *x, Long n, const T *extra, unsigned *counts, int capacity) {
     __shared__ unsigned local[LDS ? kLdsBins : 1];
     const HistogramBins<T> bins(extra, capacity);
     if (bins.numBins <= 0) return;
+    int copies = 1;
     if (LDS) {
-        for (int b = threadIdx.x; b < bins.numBins; b += kBlock) local[b] = 0u;
+        copies = kLdsBins / bins.numBins;
+        copies = copies > 32 ? 32 : (copies < 1 ? 1 : copies);
+        for (int b = threadIdx.x; b < bins.numBins * copies; b += kBlock) local[b] = 0u;
         __syncthreads();
     }
+    unsigned *myBins = local + (LDS ? (threadIdx.x % copies) * bins.numBins : 0);
     constexpr int N = Pack<T>::N;
     const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(x) & 15)) & 15) / sizeof(T));
     const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
     auto count = [&](T v) {
         const int idx = bins(v);
-        if (LDS) atomicAdd(&local[idx], 1u);
+        if (LDS) atomicAdd(&myBins[idx], 1u);
         else atomicAdd(&counts[idx], 1u);
     };
     const Long lead = head < n ? head : n;
@@ -204,7 +210,8 @@ __global__ void __launch_bounds__(kBlock) histogramCountKernel(const T *x, Long 
     if (LDS) {
         __syncthreads();
         for (int b = threadIdx.x; b < bins.numBins; b += kBlock) {
-            const unsigned c = local[b];
+            unsigned c = 0u;
+            for (int k = 0; k < copies; k++) c += local[k * bins.numBins + b];
             if (c != 0u) atomicAdd(&counts[b], c);
         }
     }
@@ -257,9 +264,53 @@ __global__ void __launch_bounds__(kBlock) im2colKernel(const T *x, T *z, const T
     }
 }
 
+// The same for a dense c-order result whose rows hold whole 16-byte vectors: a block owns one (b, c, kr, kc) plane of
+// oH x oW results at a time, so the five-fold index decomposition happens once per plane, and a thread fills one aligned
+// vector of the plane (N neighbouring columns of one row) from N image elements a stride sW apart.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) im2colPlaneKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned planes) {
+    constexpr int N = Pack<T>::N;
+    const int sH = paramInt(extra, 2), sW = paramInt(extra, 3), pH = paramInt(extra, 4), pW = paramInt(extra, 5);
+    const int dH = paramInt(extra, 6), dW = paramInt(extra, 7);
+    const unsigned vecsPerRow = (unsigned)g.oW / N, vecs = vecsPerRow * (unsigned)g.oH;
+    const FastDiv dRow = g.dAux;
+    for (unsigned plane = blockIdx.x; plane < planes; plane += gridDim.x) {
+        unsigned t = plane, kc, kr, c;
+        t = g.dKW.divmod(t, kc);
+        t = g.dKH.divmod(t, kr);
+        const unsigned b = g.dIC.divmod(t, c);
+        const T *image = x + (b * g.imS[0] + c * g.imS[1]);
+        Pack<T> *out = reinterpret_cast<Pack<T> *>(z + (Long)plane * g.oH * g.oW);
+        const int r0 = (int)kr * dH - pH, q0 = (int)kc * dW - pW;
+        for (unsigned v = threadIdx.x; v < vecs; v += kBlock) {
+            unsigned vc;
+            const unsigned orow = dRow.divmod(v, vc);
+            const int r = r0 + (int)orow * sH;
+            Pack<T> o;
+#pragma unroll
+            for (int k = 0; k < N; k++) {
+                const int q = q0 + ((int)vc * N + k) * sW;
+                o.v[k] = (inRange(r, g.iH) && inRange(q, g.iW)) ? image[r * g.imS[2] + q * g.imS[3]] : fromCompute<T>(0);
+            }
+            storePack(out + v, o);
+        }
+    }
+}
+
 template <typename T> void launchIm2col(hipStream_t s, const T *x, T *z, const T *extra, const ConvGeometry &g) {
     const Long total = (Long)g.bS * g.iC * g.kH * g.kW * g.oH * g.oW;
     if (total <= 0) return;
+    constexpr int N = Pack<T>::N;
+    const Long plane = (Long)g.oH * g.oW;
+    const bool dense = g.colS[5] == 1 && g.colS[4] == g.oW && g.colS[3] == plane && g.colS[2] == plane * g.kW &&
+                       g.colS[1] == plane * g.kW * g.kH && g.colS[0] == plane * g.kW * g.kH * g.iC;
+    if (dense && g.oW % N == 0 && (reinterpret_cast<uintptr_t>(z) & 15) == 0) {
+        const Long planes = total / plane;
+        ConvGeometry gv = g;
+        gv.dAux = FastDiv((unsigned)(g.oW / N));
+        hipLaunchKernelGGL(im2colPlaneKernel<T>, dim3(gridFor(planes, 1)), dim3(kBlock), 0, s, x, z, extra, gv, (unsigned)planes);
+        return;
+    }
     hipLaunchKernelGGL(im2colKernel<T>, dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
 }
 

@@ -230,6 +230,22 @@ def reductions(dev, rows=16384, cols=4096, seed=11, copies=None):
 
             cases.append(Case("%s_full" % opname, fam, n, 4 * n + 4, gpu, cpu, True,
                               lambda opname=opname: np.array([scalar_out[opname]], F32)))
+            cases[-1].note = "returns the scalar to the host: launch and hand-over latency included"
+        # the same whole-array reductions with the result left on the device (the array-result overload, all
+        # dimensions named): nothing waits for the call, so successive calls queue up as the per-dimension ones do
+        z1 = _vec(1)
+        Z1 = w.operand(np.zeros(1, F32), z1)
+        ex_d = dev.extra(xi, z_info=z1)
+        D01 = w.raw(np.array([0, 1], np.int32))
+        for fam, member, cpu_name, op, opname in (("reduce", ops.execReduceFloat, "reduce_scalar", R_SUM, "sum"),
+                                                  ("indexreduce", ops.execIndexReduceFloat, "indexreduce_scalar", I_MAX, "argmax")):
+            def gpu(member=member, op=op):
+                member(ex_d, op, X.ptr, X.info_ptr, None, Z1.ptr, Z1.info_ptr, D01.ptr, 2)
+
+            def cpu(lib, cpu_name=cpu_name, op=op):
+                return getattr(lib, cpu_name)(op, x, xi, None)
+
+            cases.append(Case("%s_full_to_device" % opname, fam, n, 4 * n + 4, gpu, cpu, True, Z1.get))
         return cases
 
     return _replicated(dev, "reduce sum/max/mean + argmax; fp32 [%d,%d] c-order; dim 1, dim 0, full" % (rows, cols),
@@ -558,6 +574,62 @@ def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data
 
     w.free = free
     return w
+
+
+# ---- the whole-array transforms: Reverse, Histogram, Im2col, Col2Im, Pooling2D ------------------------------------------
+def whole_array_transforms(dev, n=1 << 26, seed=41, copies=None):
+    """Reverse and Histogram over 2^26 floats; Im2col / Col2Im / Pooling2D on a [32, 64, 56, 56] image (3 x 3 kernel,
+    stride 1, padding 1 for the column forms; 2 x 2 / stride 2 max and average pooling)."""
+    rs = np.random.default_rng(seed)
+    x = _uniform(rs, n, -3, 3)
+    vi = _vec(n)
+    bins = 256
+    bi = _vec(bins)
+    img, col, pooled = [32, 64, 56, 56], [32, 64, 3, 3, 56, 56], [32, 64, 28, 28]
+    ii, ci, pi = harness.shape_info(img), harness.shape_info(col), harness.shape_info(pooled)
+    n_img, n_col, n_pool = int(np.prod(img)), int(np.prod(col)), int(np.prod(pooled))
+    image = _uniform(rs, n_img, -3, 3)
+    e_hist = np.array([bins, -2.5, 2.75], F32)
+    e_im2col = np.array([3, 3, 1, 1, 1, 1, 1, 1, 0, 0], F32)
+    e_col2im = np.array([1, 1, 1, 1, 56, 56, 1, 1], F32)
+    e_pool = {0: np.array([2, 2, 2, 2, 0, 0, 1, 1, 0, 0, 0], F32), 1: np.array([2, 2, 2, 2, 0, 0, 1, 1, 0, 1, 0], F32)}
+    ops = dev.ops
+    zc, hc, colc, imgc, poolc = np.zeros(n, F32), np.zeros(bins, F32), np.zeros(n_col, F32), np.zeros(n_img, F32), np.zeros(n_pool, F32)
+
+    def device_set(w):
+        X, Z = w.operand(x, vi), w.operand(np.zeros(n, F32), vi)
+        H = w.operand(np.zeros(bins, F32), bi)
+        I, C, P = w.operand(image, ii), w.operand(np.zeros(n_col, F32), ci), w.operand(np.zeros(n_pool, F32), pi)
+        I2 = w.operand(np.zeros(n_img, F32), ii)
+        EH, EI, EC = w.raw(e_hist), w.raw(e_im2col), w.raw(e_col2im)
+        EP = {k: w.raw(v) for k, v in e_pool.items()}
+        cases = []
+        ex = dev.extra(vi, z_info=vi)
+        cases.append(Case("reverse", "transform", n, 8 * n,
+                          lambda: ops.execTransformFloat(ex, 70, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, None),
+                          lambda lib: (lib.transform(70, x, vi, zc, vi, None), zc)[1], True, Z.get))
+        exh = dev.extra(vi, z_info=bi)
+        cases.append(Case("histogram_256_bins", "transform", n, 4 * n + 8 * bins,
+                          lambda: ops.execTransformFloat(exh, 48, X.ptr, X.info_ptr, H.ptr, H.info_ptr, EH.ptr),
+                          lambda lib: (hc.fill(0), lib.transform(48, x, vi, hc, bi, e_hist), hc)[2], True, H.get))
+        cases[-1].note = "counts accumulate over the calls of a timing loop"
+        exi = dev.extra(ii, z_info=ci)
+        cases.append(Case("im2col_3x3", "transform", n_col, 4 * n_img + 4 * n_col,
+                          lambda: ops.execTransformFloat(exi, 37, I.ptr, I.info_ptr, C.ptr, C.info_ptr, EI.ptr),
+                          lambda lib: (lib.transform(37, image, ii, colc, ci, e_im2col), colc)[1], True, C.get))
+        exc = dev.extra(ci, z_info=ii)
+        cases.append(Case("col2im_3x3", "transform", n_col, 4 * n_img + 4 * n_col,
+                          lambda: ops.execTransformFloat(exc, 36, C.ptr, C.info_ptr, I2.ptr, I2.info_ptr, EC.ptr),
+                          None, True, I2.get))
+        exp_ = dev.extra(ii, z_info=pi)
+        for mode, name in ((0, "maxpool_2x2"), (1, "avgpool_2x2")):
+            cases.append(Case(name, "transform", n_img, 4 * n_img + 4 * n_pool,
+                              lambda mode=mode: ops.execTransformFloat(exp_, 71, I.ptr, I.info_ptr, P.ptr, P.info_ptr, EP[mode].ptr),
+                              lambda lib, mode=mode: (lib.transform(71, image, ii, poolc, pi, e_pool[mode]), poolc)[1], True, P.get))
+        return cases
+
+    return _replicated(dev, "whole-array transforms: reverse / histogram 2^26; im2col, col2im, pooling on [32,64,56,56]",
+                       8 * n + 8 * n_col, dict(x=x, image=image), device_set, copies)
 
 
 BUILDERS = [transform_tanh, pairwise_broadcast, reductions, reduce3_pairs, stats_softmax, random_fills]
