@@ -48,7 +48,7 @@ def parse():
     ap.add_argument("--counters", action="store_true",
                     help="for hardware-counter runs: launch the yardstick copy kernel (256 MiB) and each headline kernel "
                          "3 times and exit")
-    ap.add_argument("--traffic", default=os.path.join(ROOT, "profiles", "headline_step_hbm_traffic.txt"),
+    ap.add_argument("--traffic", default=os.path.join(ROOT, "profiles", "all_families_hbm_traffic.txt"),
                     help="rocprofv3 counter summary holding the measured HBM bytes per launch of the dominant kernel")
     return ap.parse_args()
 
@@ -90,19 +90,47 @@ def time_case(dev, case, steps, warmup):
     return ms
 
 
-def measured_traffic(path, kernel):
-    """HBM bytes per launch of `kernel` from the committed counter summary (FETCH_SIZE and WRITE_SIZE runs of
-    `bench.py --counters`, scaled by a copy kernel of known size); None when the summary is not there."""
+def kernel_sources_digest():
+    """Digest of the kernel and host sources the library is built from: a counter summary under profiles/ records the
+    digest it was measured on, and its figures are only quoted while the sources still are what they were then."""
+    import hashlib
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "libnd4j_amd", "csrc")
+    for name in sorted(os.listdir(src)):
+        path = os.path.join(src, name)
+        if os.path.isfile(path) and name.rsplit(".", 1)[-1] in ("hip", "cuh", "h", "cpp"):
+            h.update(name.encode())
+            with open(path, "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(path, key):
+    """HBM bytes per launch (or per call) of the line that starts with `key` in a committed counter summary (FETCH_SIZE
+    and WRITE_SIZE runs of `bench.py --counters`, scaled by a copy kernel of known size).  None when the summary is not
+    there, has no such line, or was measured on other sources than the ones in this tree (its `sources:` line)."""
     if not path or not os.path.exists(path):
         return None
     with open(path) as f:
-        for line in f:
-            if kernel in line:
-                try:
-                    return int(line.split()[-1])
-                except ValueError:
-                    return None
+        lines = f.read().splitlines()
+    for line in lines:
+        if line.startswith("sources:") and line.split()[1] != kernel_sources_digest():
+            return None
+    for line in lines:
+        if line.startswith(key):
+            try:
+                return int(line.split()[-1])
+            except ValueError:
+                return None
     return None
+
+
+def family_builders(workloads):
+    return [("transform", workloads.transform_tanh), ("pairwise", lambda d: workloads.pairwise_broadcast(d, copies=2)),
+            ("half", lambda d: workloads.pairwise_broadcast(d, dtype="float16")),
+            ("reductions", workloads.reductions), ("reduce3", workloads.reduce3_pairs),
+            ("stats", workloads.stats_softmax), ("random", workloads.random_fills),
+            ("movement", workloads.data_movement), ("whole", workloads.whole_array_transforms)]
 
 
 def load_cpu():
@@ -144,15 +172,32 @@ def main():
     step_bytes = sum(c.bytes for c in step_cases)
     step_elems = sum(c.elements for c in step_cases)
     if args.counters:
+        # For a `rocprofv3 --pmc` run: the yardstick copy kernel (256 MiB read, 256 MiB written) 3 times, then every case
+        # 3 times, each case behind a small copy whose size (4096 bytes times the case's number) marks it in the trace.
         src, dst = dev.empty(1 << 28), dev.empty(1 << 28)
         for _ in range(3):
             dev.ops.amd_copyKernel(dev.extra(), dst.ptr, src.ptr, 1 << 28)
-        for c in step_cases:
-            for _ in range(3):
-                c.gpu()
-        dev.sync()
-        print(json.dumps({"counters_run": {"copy_bytes_read": 1 << 28, "copy_bytes_written": 1 << 28,
-                                           "kernels": {c.name: c.bytes for c in step_cases}}}))
+        listed = []
+
+        def run(cases):
+            for c in cases:
+                listed.append({"case": c.name, "bytes": c.bytes, "marker_bytes": 4096 * (len(listed) + 1)})
+                dev.ops.amd_copyKernel(dev.extra(), dst.ptr, src.ptr, listed[-1]["marker_bytes"])
+                for k in range(3):
+                    c.gpu(k)
+                dev.sync()
+
+        run(step_cases)
+        w.free()
+        only = [o for o in args.only.split(",") if o]
+        for key, build in family_builders(workloads):
+            if key == "pairwise" or (only and key not in only):
+                continue
+            wl = build(dev)
+            run(wl.cases)
+            wl.free()
+        print(json.dumps({"counters_run": {"copy_bytes_read": 1 << 28, "copy_bytes_written": 1 << 28, "sources": kernel_sources_digest(),
+                                           "cases": listed}}))
         return 0
     for k in range(W):
         for c in step_cases:
@@ -175,7 +220,7 @@ def main():
     ms_per_step = wall * 1e3 / K
     value = step_bytes / (wall / K) / 1e9
 
-    traffic = measured_traffic(args.traffic, "ewVecKernel<float, nd4j_amd::Pairwise3F<0>")
+    traffic = measured_traffic(args.traffic, "pairwise_add ")
     achieved = add.bytes / (per_kernel_ms[0] * 1e-3) / 1e9
     out = {
         "metric": "achieved HBM GB/s (algorithmic bytes) of the legacy op path: pairwise add + pairwise multiply + broadcast add row",
@@ -225,13 +270,8 @@ def main():
     if not args.no_families:
         fam = []
         cpu_left = args.families_cpu_seconds
-        builders = [("transform", workloads.transform_tanh), ("pairwise", lambda d: workloads.pairwise_broadcast(d, copies=2)),
-                    ("half", lambda d: workloads.pairwise_broadcast(d, dtype="float16")),
-                    ("reductions", workloads.reductions), ("reduce3", workloads.reduce3_pairs),
-                    ("stats", workloads.stats_softmax), ("random", workloads.random_fills),
-                    ("movement", workloads.data_movement), ("whole", workloads.whole_array_transforms)]
         only = [o for o in args.only.split(",") if o]
-        for key, build in builders:
+        for key, build in family_builders(workloads):
             if only and key not in only:
                 continue
             wl = build(dev)
@@ -244,6 +284,10 @@ def main():
                 if fetched:  # shapeInfo / dimension read-backs (each one a stream synchronisation)
                     row["host_fetches"] = int(fetched)
                 row["bound"] = getattr(c, "bound", "hbm")
+                t = measured_traffic(args.traffic, c.name + " ")
+                if t is not None:  # HBM bytes the call moved, by the chip's counters (profiles/): well above `bytes` = re-reads
+                    row["traffic"] = t
+                    row["traffic_over_algorithmic"] = round(t / float(c.bytes), 3)
                 # one warm-up and up to three timed passes of the compiled reference, while the budget lasts; a case whose
                 # single pass is known to take seconds (note "cpu once") is run once, cold
                 if cpu_lib is not None and c.cpu is not None and not (c.name.endswith("float16")) and cpu_left > 0:

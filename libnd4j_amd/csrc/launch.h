@@ -182,7 +182,7 @@ struct ConvGeometry {
     int bS, iC, iH, iW, kH, kW, oH, oW;
     Long imS[4], colS[6];
     FastDiv dOW, dOH, dKW, dKH, dIC, dIW, dIH;
-    FastDiv dAux;  // a launcher's own divisor (Im2col: 16-byte vectors per result row)
+    FastDiv dAux, dAux2;  // a launcher's own divisors (Im2col: 16-byte vectors per result row, planes per channel)
 };
 template <typename T> void launchIm2col(hipStream_t stream, const T *x, T *z, const T *extra, const ConvGeometry &g);
 // clearFirst > 0: that many leading elements of z's buffer are cleared first and the sums are added onto what z holds

@@ -14,12 +14,12 @@ namespace nd4j_amd {
 
 namespace {
 
-constexpr int kMaxGrid = 1 << 20;
+constexpr int kWholeGrid = 1 << 20;
 
 inline int gridFor(Long items, int perBlock = kBlock) {
     Long blocks = (items + perBlock - 1) / perBlock;
     if (blocks < 1) blocks = 1;
-    return (int)(blocks > kMaxGrid ? kMaxGrid : blocks);
+    return (int)(blocks > kWholeGrid ? kWholeGrid : blocks);
 }
 
 template <typename T> __device__ __forceinline__ int paramInt(const T *extra, int i) { return (int)toCompute(extra[i]); }
@@ -268,13 +268,27 @@ __global__ void __launch_bounds__(kBlock) im2colKernel(const T *x, T *z, const T
 // oH x oW results at a time, so the five-fold index decomposition happens once per plane, and a thread fills one aligned
 // vector of the plane (N neighbouring columns of one row) from N image elements a stride sW apart.
 template <typename T>
-__global__ void __launch_bounds__(kBlock) im2colPlaneKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned planes) {
+__global__ void __launch_bounds__(kBlock) im2colPlaneKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned planes,
+                                                            unsigned launched, int byDie) {
     constexpr int N = Pack<T>::N;
     const int sH = paramInt(extra, 2), sW = paramInt(extra, 3), pH = paramInt(extra, 4), pW = paramInt(extra, 5);
     const int dH = paramInt(extra, 6), dW = paramInt(extra, 7);
     const unsigned vecsPerRow = (unsigned)g.oW / N, vecs = vecsPerRow * (unsigned)g.oH;
     const FastDiv dRow = g.dAux;
-    for (unsigned plane = blockIdx.x; plane < planes; plane += gridDim.x) {
+    // The kH * kW planes of one image channel all read that channel.  Workgroups go to the chip's eight dies in turn, each
+    // die with a cache of its own, so in plain order the planes of a channel land on different dies and each die fetches
+    // the channel again.  `byDie`: workgroup w serves die w % 8, and the w / 8 -th plane of that die's channels (the
+    // channels die, die + 8, ...), so that a channel is fetched by one die only.
+    const unsigned perChannel = (unsigned)(g.kH * g.kW);
+    for (unsigned w = blockIdx.x; w < launched; w += gridDim.x) {
+        unsigned plane = w;
+        if (byDie) {
+            const unsigned die = w & 7u, local = w >> 3;
+            unsigned k;
+            const unsigned channel = g.dAux2.divmod(local, k) * 8u + die;
+            plane = channel * perChannel + k;
+        }
+        if (plane >= planes) continue;
         unsigned t = plane, kc, kr, c;
         t = g.dKW.divmod(t, kc);
         t = g.dKH.divmod(t, kr);
@@ -308,7 +322,16 @@ template <typename T> void launchIm2col(hipStream_t s, const T *x, T *z, const T
         const Long planes = total / plane;
         ConvGeometry gv = g;
         gv.dAux = FastDiv((unsigned)(g.oW / N));
-        hipLaunchKernelGGL(im2colPlaneKernel<T>, dim3(gridFor(planes, 1)), dim3(kBlock), 0, s, x, z, extra, gv, (unsigned)planes);
+        const Long perChannel = (Long)g.kH * g.kW, channels = planes / perChannel;
+        gv.dAux2 = FastDiv((unsigned)perChannel);
+        // workgroups for whole rounds of eight channels; in one launch when that fits, else in plain order
+        const Long byDie = (channels + 7) / 8 * 8 * perChannel;
+        if (byDie <= kWholeGrid)
+            hipLaunchKernelGGL(im2colPlaneKernel<T>, dim3((unsigned)byDie), dim3(kBlock), 0, s, x, z, extra, gv, (unsigned)planes,
+                               (unsigned)byDie, 1);
+        else
+            hipLaunchKernelGGL(im2colPlaneKernel<T>, dim3(gridFor(planes, 1)), dim3(kBlock), 0, s, x, z, extra, gv, (unsigned)planes,
+                               (unsigned)planes, 0);
         return;
     }
     hipLaunchKernelGGL(im2colKernel<T>, dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
