@@ -50,6 +50,8 @@ def parse():
                          "3 times and exit")
     ap.add_argument("--traffic", default=os.path.join(ROOT, "profiles", "all_families_hbm_traffic.txt"),
                     help="rocprofv3 counter summary holding the measured HBM bytes per launch of the dominant kernel")
+    ap.add_argument("--instructions", default=os.path.join(ROOT, "profiles", "all_families_instruction_counters.txt"),
+                    help="rocprofv3 counter summary holding the vector instructions per element of the benchmark cases")
     return ap.parse_args()
 
 
@@ -133,6 +135,25 @@ def family_builders(workloads):
             ("movement", workloads.data_movement), ("whole", workloads.whole_array_transforms)]
 
 
+def valu_per_element(path, case):
+    """VALU instructions per element of `case` from the committed instruction-counter summary (its line
+    "<case> ... VALU/element <v>"), or None: as measured_traffic, only while the sources are what they were."""
+    if not path or not os.path.exists(path):
+        return None
+    with open(path) as f:
+        lines = f.read().splitlines()
+    for line in lines:
+        if line.startswith("sources:") and line.split()[1] != kernel_sources_digest():
+            return None
+    for line in lines:
+        if line.startswith(case + " ") and "VALU/element" in line:
+            try:
+                return float(line.split("VALU/element")[1].split()[0])
+            except (ValueError, IndexError):
+                return None
+    return None
+
+
 def load_cpu():
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import cpu_ref
@@ -181,7 +202,7 @@ def main():
 
         def run(cases):
             for c in cases:
-                listed.append({"case": c.name, "bytes": c.bytes, "marker_bytes": 4096 * (len(listed) + 1)})
+                listed.append({"case": c.name, "bytes": c.bytes, "elements": c.elements, "marker_bytes": 4096 * (len(listed) + 1)})
                 dev.ops.amd_copyKernel(dev.extra(), dst.ptr, src.ptr, listed[-1]["marker_bytes"])
                 for k in range(3):
                     c.gpu(k)
@@ -284,6 +305,12 @@ def main():
                 if fetched:  # shapeInfo / dimension read-backs (each one a stream synchronisation)
                     row["host_fetches"] = int(fetched)
                 row["bound"] = getattr(c, "bound", "hbm")
+                v = valu_per_element(args.instructions, c.name)
+                if v is not None:
+                    # a wave64 vector instruction holds its 16-lane SIMD for 4 cycles: the time the chip's 1024 SIMDs need
+                    # to issue the call's vector instructions at 2.4 GHz, against the time measured
+                    issue_ms = v * c.elements / 64.0 * 4.0 / (1024 * 2.4e9) * 1e3
+                    row["valu"] = {"instructions_per_element": v, "issue_ms": round(issue_ms, 4), "frac": round(issue_ms / ms, 4)}
                 t = measured_traffic(args.traffic, c.name + " ")
                 if t is not None:  # HBM bytes the call moved, by the chip's counters (profiles/): well above `bytes` = re-reads
                     row["traffic"] = t

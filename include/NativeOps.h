@@ -11,11 +11,21 @@
 //   * data pointers, shapeInfo arguments, `dimension` and `extraParams` are DEVICE pointers;
 //   * extraPointers[0] host xShapeInfo, [1] the HIP stream handle by value, [2] device id,
 //     [3] allocation scratch (unused here), [4] reduction scratch (unused here), [5] host-visible scalar
-//     result (unused: scalars are returned by value after a stream synchronise), [7] host yShapeInfo,
+//     result (unused: scalars are returned by value; the library hands them over through pinned host memory
+//     of its own, see below), [7] host yShapeInfo,
 //     [8] host zShapeInfo, [9] host TAD shapeInfo, [10] device TAD shapeInfo, [11] device TAD offsets,
 //     [12]/[13] device TAD shapeInfo/offsets of the result (broadcast);
-//   * array results are enqueued on the stream and the call returns; scalar-returning members
-//     synchronise the stream.
+//   * array results are enqueued on the stream and the call returns; scalar-returning members return once the
+//     value has arrived: the last kernel writes it, tagged with the call's ticket, into pinned host memory that
+//     the library keeps per (device, stream), and the host waits for those words (asking the stream as well after
+//     50 us, and handing over to a stream synchronisation after 300 us, or at once in debug mode).  Everything
+//     enqueued earlier on the stream has completed by then, as after a synchronisation.
+//   * one host thread per stream at a time: the scalar slot, its tickets and the stream's scratch memory are per
+//     (device, stream) and not shared safely between threads that use one stream (the null stream included).
+//   * enableDebugMode synchronises after every launch and reports asynchronous errors; with enableVerboseMode on
+//     as well every kernel launch prints its name and launch dimensions.  setOmpNumThreads / setOmpMinThreads,
+//     setGridLimit, setElementThreshold and setTADThreshold store their values for the getters and tune nothing:
+//     launch geometry here follows the operand shapes.
 //   Missing host copies ([0],[7],[8],[9] null) are fetched from the device pointers, and missing TAD
 //   tables are computed and cached by the library, at the price of a stream synchronise.
 #pragma once

@@ -12,13 +12,13 @@ template <typename T> struct BroadcastBody {
             if (pl.kind == BroadcastPlan::ROW && pl.consecutive && pl.tadLength % Pack<T>::N == 0 &&
                 pl.tadLength / Pack<T>::N < 0xffffffffLL && (((uintptr_t)x | (uintptr_t)y | (uintptr_t)z) & 15) == 0) {
                 const Long nvec = pl.numTads * (pl.tadLength / Pack<T>::N);
-                hipLaunchKernelGGL((bcFlatKernel<T, F>), dim3(gridFor(nvec, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0,
+                ND4J_LAUNCH((bcFlatKernel<T, F>), dim3(gridFor(nvec, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0,
                                    s, x, y, z, nvec, (unsigned)(pl.tadLength / Pack<T>::N), Params<T>{nullptr});
             } else if (pl.kind == BroadcastPlan::ROW && pl.consecutive && pl.tadLength >= Pack<T>::N && pl.tadLength < 0xffffffffLL &&
                        (((uintptr_t)x | (uintptr_t)z) & 15) == 0) {
                 // gap-free rows whose length is not a multiple of the vector width
                 const Long n = pl.numTads * pl.tadLength;
-                hipLaunchKernelGGL((bcFlatAnyKernel<T, F>), dim3(gridFor(n / Pack<T>::N + 1, kBlock, F::tables ? kGridCap : kMaxGrid)),
+                ND4J_LAUNCH((bcFlatAnyKernel<T, F>), dim3(gridFor(n / Pack<T>::N + 1, kBlock, F::tables ? kGridCap : kMaxGrid)),
                                    dim3(kBlock), 0, s, x, y, z, n, pl.tadLength, Params<T>{nullptr});
             } else if (pl.kind == BroadcastPlan::ROW) {
                 constexpr int VEC = Pack<T>::N;
@@ -33,13 +33,13 @@ template <typename T> struct BroadcastBody {
                 if ((pl.numTads / (perBlock * 4)) * gy >= 4096) perBlock *= 4;
                 int gx = gridFor(pl.numTads, perBlock, kMaxGrid);
                 int aligned = (((uintptr_t)x | (uintptr_t)z) & 15) == 0 ? 1 : 0;
-                hipLaunchKernelGGL((bcRowKernel<T, F, false>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
+                ND4J_LAUNCH((bcRowKernel<T, F, false>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
                                    pl.zOffsets, pl.tadLength, pl.numTads, aligned, colShift, Params<T>{nullptr});
             } else if (pl.kind == BroadcastPlan::COL && pl.denseAlike && pl.tadEws >= 1 && pl.tadEws < 0xffffffffLL &&
                        pl.tadLength < 0xffffffffLL && (((uintptr_t)x | (uintptr_t)z) & 15) == 0) {
                 // any single dimension of a dense array: runs of tadEws consecutive elements share one y
                 const Long n = pl.numTads * pl.tadLength;
-                hipLaunchKernelGGL((bcFlatInnerKernel<T, F>), dim3(gridFor(n / Pack<T>::N + 1, kBlock, F::tables ? kGridCap : kMaxGrid)),
+                ND4J_LAUNCH((bcFlatInnerKernel<T, F>), dim3(gridFor(n / Pack<T>::N + 1, kBlock, F::tables ? kGridCap : kMaxGrid)),
                                    dim3(kBlock), 0, s, x, y, z, n, pl.tadEws, pl.tadLength, Params<T>{nullptr});
             } else if (pl.kind == BroadcastPlan::COL) {
                 int gx = (int)((pl.numTads + kBlock - 1) / kBlock);
@@ -47,11 +47,11 @@ template <typename T> struct BroadcastBody {
                 if (gy < 1) gy = 1;
                 if (gy > pl.tadLength) gy = pl.tadLength;
                 if (gy > 65535) gy = 65535;
-                hipLaunchKernelGGL((bcColKernel<T, F, false>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
+                ND4J_LAUNCH((bcColKernel<T, F, false>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
                                    pl.zOffsets, pl.tadLength, pl.numTads, pl.tadEws, pl.yEws, pl.zEws, Params<T>{nullptr});
             } else {
                 int grid = gridFor(pl.numTads, 1, kGridCap);
-                hipLaunchKernelGGL((bcGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, pl.xm, y, pl.ym, z, pl.zm,
+                ND4J_LAUNCH((bcGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, pl.xm, y, pl.ym, z, pl.zm,
                                    pl.xOffsets, pl.zOffsets, pl.tadLength, pl.numTads);
             }
             return true;

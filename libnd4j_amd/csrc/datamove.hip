@@ -334,7 +334,7 @@ __global__ void __launch_bounds__(kBlock) copyToEwsKernel(const T *x, Long xe, T
 }
 template <typename T> void launchCopyToEws(hipStream_t s, const T *x, Long xe, T *z, const Long *zInfo, Long n) {
     if (n <= 0) return;
-    hipLaunchKernelGGL((copyToEwsKernel<T>), dim3(gridFor(n, (Long)kBlock * Pack<T>::N, 1 << 22)), dim3(kBlock), 0, s, x, xe, z,
+    ND4J_LAUNCH((copyToEwsKernel<T>), dim3(gridFor(n, (Long)kBlock * Pack<T>::N, 1 << 22)), dim3(kBlock), 0, s, x, xe, z,
                        zInfo, n);
 }
 
@@ -403,8 +403,8 @@ void launchTransposeCopy(hipStream_t s, const T *x, T *z, Long rows, Long cols, 
     const dim3 grid((unsigned)(tiles < kMaxGrid ? tiles : kMaxGrid));
     const bool vec = rows % N == 0 && cols % N == 0 && xColStride % N == 0 && zRowStride % N == 0 &&
                      (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(z) & 15) == 0;
-    if (vec) hipLaunchKernelGGL((transposeCopyKernel<T, N, TR, TC>), grid, dim3(kBlock), 0, s, x, z, rows, cols, xColStride, zRowStride);
-    else hipLaunchKernelGGL((transposeCopyKernel<T, 1, TR, TC>), grid, dim3(kBlock), 0, s, x, z, rows, cols, xColStride, zRowStride);
+    if (vec) ND4J_LAUNCH((transposeCopyKernel<T, N, TR, TC>), grid, dim3(kBlock), 0, s, x, z, rows, cols, xColStride, zRowStride);
+    else ND4J_LAUNCH((transposeCopyKernel<T, 1, TR, TC>), grid, dim3(kBlock), 0, s, x, z, rows, cols, xColStride, zRowStride);
 }
 
 template <typename T>
@@ -412,13 +412,13 @@ void launchPullRows(hipStream_t s, const T *x, T *z, Long n, const Long *indexes
                     const Long *zTadInfo, const Long *zTadOffsets) {
     if (n <= 0) return;
     // (a launch with few rows gets the full grid: the kernel cuts long rows into pieces, and idle blocks leave at once)
-    hipLaunchKernelGGL((pullRowsKernel<T>), dim3(n >= kGridCap ? gridFor(n, 1, kGridCap * 4) : kGridCap), dim3(kBlock), 0, s, x, z, n,
+    ND4J_LAUNCH((pullRowsKernel<T>), dim3(n >= kGridCap ? gridFor(n, 1, kGridCap * 4) : kGridCap), dim3(kBlock), 0, s, x, z, n,
                        indexes, tadInfo, tadOffsets, zTadInfo, zTadOffsets);
 }
 template <typename T>
 void launchTear(hipStream_t s, const T *x, const Long *xInfo, T *const *targets, const Long *zInfo, const Long *tadInfo,
                 const Long *tadOffsets, Long numTadsHint) {
-    hipLaunchKernelGGL((tearKernel<T>), dim3(gridFor(numTadsHint > 0 ? numTadsHint : kGridCap, 1, kGridCap * 4)), dim3(kBlock), 0, s,
+    ND4J_LAUNCH((tearKernel<T>), dim3(gridFor(numTadsHint > 0 ? numTadsHint : kGridCap, 1, kGridCap * 4)), dim3(kBlock), 0, s,
                        x, xInfo, targets, zInfo, tadInfo, tadOffsets);
 }
 template <typename T>
@@ -426,7 +426,7 @@ void launchShuffle(hipStream_t s, T *const *xs, const Long *const *xInfos, T *co
                    const Long *const *tadInfos, const Long *const *tadOffsets, Long numTadsHint) {
     if (N <= 0) return;
     const int gy = N < 64 ? N : 64;
-    hipLaunchKernelGGL((shuffleKernel<T>), dim3(gridFor(numTadsHint > 0 ? numTadsHint : 4096, 1, kGridCap), gy), dim3(kBlock), 0, s,
+    ND4J_LAUNCH((shuffleKernel<T>), dim3(gridFor(numTadsHint > 0 ? numTadsHint : 4096, 1, kGridCap), gy), dim3(kBlock), 0, s,
                        xs, xInfos, zs, N, map, tadInfos, tadOffsets);
 }
 template <typename T>
@@ -434,7 +434,7 @@ void launchConcat(hipStream_t s, const T *const *data, const Long *const *infos,
                   void *scratch) {
     if (n <= 0) return;
     ConcatDesc *desc = reinterpret_cast<ConcatDesc *>(scratch);
-    hipLaunchKernelGGL(concatPrepareKernel, dim3(1), dim3(kBlock), 0, s, reinterpret_cast<const void *const *>(data), infos, n, v, desc);
+    ND4J_LAUNCH(concatPrepareKernel, dim3(1), dim3(kBlock), 0, s, reinterpret_cast<const void *const *>(data), infos, n, v, desc);
     const int gy = n < 65535 ? n : 65535;
     // four 16-byte vectors per thread while that keeps the grid below 2^22 blocks
     int budget = (1 << 22) / gy;
@@ -443,8 +443,8 @@ void launchConcat(hipStream_t s, const T *const *data, const Long *const *infos,
     // Short runs (the inputs' slabs alternate in z every few KB): blocks that run together should fill neighbouring
     // runs, so the input index varies fastest.  Long runs: one input after the other.
     const bool inputFastest = v.dim > 0 && n > 1 && gx <= 65535;
-    if (inputFastest) hipLaunchKernelGGL((concatKernel<T>), dim3(gy, gx), dim3(kBlock), 0, s, infos, z, v, desc, n, 1);
-    else hipLaunchKernelGGL((concatKernel<T>), dim3(gx, gy), dim3(kBlock), 0, s, infos, z, v, desc, n, 0);
+    if (inputFastest) ND4J_LAUNCH((concatKernel<T>), dim3(gy, gx), dim3(kBlock), 0, s, infos, z, v, desc, n, 1);
+    else ND4J_LAUNCH((concatKernel<T>), dim3(gx, gy), dim3(kBlock), 0, s, infos, z, v, desc, n, 0);
 }
 size_t concatScratchBytes(int numArrays) { return (size_t)(numArrays > 0 ? numArrays : 1) * sizeof(ConcatDesc); }
 
@@ -487,7 +487,7 @@ __global__ void __launch_bounds__(kBlock) averageKernel(T *const *xs, T *z, int 
 template <typename T> void launchAverage(hipStream_t s, T *const *xs, T *z, int n, Long length, bool average, bool propagate) {
     if (n <= 0 || length <= 0) return;
     const int grid = gridFor(length, (Long)kBlock * Pack<T>::N, kGridCap * 4);
-    hipLaunchKernelGGL((averageKernel<T>), dim3(grid), dim3(kBlock), 0, s, xs, z, n, length, average ? 1 : 0, propagate ? 1 : 0);
+    ND4J_LAUNCH((averageKernel<T>), dim3(grid), dim3(kBlock), 0, s, xs, z, n, length, average ? 1 : 0, propagate ? 1 : 0);
 }
 
 // ---- conversions between half, float and double: z[i] = (D)(float)x[i] (type_conversions.h:38-49) -----------------
@@ -549,7 +549,7 @@ template <typename S, typename D> void runConvert(hipStream_t s, const void *x, 
     const int vectors = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(z)) & 15) == 0 ? 1 : 0;
     // elements per block and pass: 8 per thread when narrowing, four output vectors per thread when widening
     const Long perBlock = sizeof(D) > sizeof(S) ? (Long)kBlock * 4 * (16 / (Long)sizeof(D)) : (Long)kBlock * 8;
-    hipLaunchKernelGGL((convertKernel<S, D>), dim3(gridFor(n, perBlock, kMaxGrid)), dim3(kBlock), 0, s,
+    ND4J_LAUNCH((convertKernel<S, D>), dim3(gridFor(n, perBlock, kMaxGrid)), dim3(kBlock), 0, s,
                        reinterpret_cast<const S *>(x), reinterpret_cast<D *>(z), n, vectors);
 }
 // type codes of type_conversions.h:11-18: 3 half, 6 float, 7 double

@@ -14,6 +14,7 @@
 
 #include <utility>
 
+#include "launch.h"
 #include "ops_elementwise.cuh"
 #include "types.h"
 #include "view.h"
@@ -466,7 +467,7 @@ inline void launchStrided(hipStream_t s, const T *x, Long xs, const T *y, Long y
             Long nvec = (n - head) / Pack<T>::N;
             // kernels that stage the lookup tables run several passes per block, so the staging is paid less often
             int grid = gridFor(nvec > 0 ? nvec : 1, (Long)kBlock, F::tables ? kGridCap : kMaxGrid);
-            hipLaunchKernelGGL((ewVecKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, two ? y : x, z, p, n, head,
+            ND4J_LAUNCH((ewVecKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, two ? y : x, z, p, n, head,
                                (two && ys == 0) ? 1 : 0);
             return;
         }
@@ -476,7 +477,7 @@ inline void launchStrided(hipStream_t s, const T *x, Long xs, const T *y, Long y
     xm.shape[0] = ym.shape[0] = zm.shape[0] = (unsigned)(n > 0xffffffffLL ? 0xffffffffu : n);
     xm.stride[0] = xs; ym.stride[0] = ys; zm.stride[0] = zs;
     int grid = gridFor(n, kBlock * 4, kGridCap);
-    hipLaunchKernelGGL((ewGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, xm, two ? y : x, ym, z, zm, p, n);
+    ND4J_LAUNCH((ewGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, xm, two ? y : x, ym, z, zm, p, n);
 }
 
 // Dense matrices in mixed orders (z = op(x, y) with x or y laid out the other way round than z: a + b.transpose()): in
@@ -567,12 +568,12 @@ inline void launchMixedOrder(hipStream_t s, const T *x, const T *y, T *z, Long r
     const Long tiles = ((rows + 31) / 32) * ((cols + 63) / 64);
     const dim3 grid((unsigned)(tiles < kMaxGrid ? tiles : kMaxGrid));
     if constexpr (F::nin == 2) {
-        if (xt && yt) hipLaunchKernelGGL((ewMixedOrderKernel<T, F, ACC, true, true>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
-        else if (xt) hipLaunchKernelGGL((ewMixedOrderKernel<T, F, ACC, true, false>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
-        else hipLaunchKernelGGL((ewMixedOrderKernel<T, F, ACC, false, true>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
+        if (xt && yt) ND4J_LAUNCH((ewMixedOrderKernel<T, F, ACC, true, true>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
+        else if (xt) ND4J_LAUNCH((ewMixedOrderKernel<T, F, ACC, true, false>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
+        else ND4J_LAUNCH((ewMixedOrderKernel<T, F, ACC, false, true>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
     } else {
         (void)yt;  // one input: it is the transposed one
-        hipLaunchKernelGGL((ewMixedOrderKernel<T, F, ACC, true, false>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
+        ND4J_LAUNCH((ewMixedOrderKernel<T, F, ACC, true, false>), grid, dim3(kBlock), 0, s, x, y, z, rows, cols, p);
     }
 }
 
@@ -604,7 +605,7 @@ inline void launchGeneral(hipStream_t s, const T *x, const DimMap &xm, const T *
     Params<T> p{extra};
     p.scalar = scalar;
     int grid = gridFor(n, kBlock * 4, kGridCap);
-    hipLaunchKernelGGL((ewGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, xm, two ? y : x, two ? ym : xm, z, zm,
+    ND4J_LAUNCH((ewGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, xm, two ? y : x, two ? ym : xm, z, zm,
                        p, n);
 }
 

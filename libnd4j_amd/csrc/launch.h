@@ -10,6 +10,17 @@
 
 namespace nd4j_amd {
 
+// Every kernel launch of the library goes through this macro: with debug and verbose mode both on (enableDebugMode,
+// enableVerboseMode) it prints the kernel and its launch dimensions first, as the reference's CUDA back end prints its
+// launch parameters (blas/cuda/NativeOps.cu:195-196, 257, 282).
+bool launchesAreVerbose();
+void printLaunch(const char *kernel, dim3 grid, dim3 block, size_t ldsBytes);
+#define ND4J_LAUNCH(kernel, grid, block, lds, stream, ...)                                        \
+    do {                                                                                          \
+        if (::nd4j_amd::launchesAreVerbose()) ::nd4j_amd::printLaunch(#kernel, grid, block, lds); \
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                        \
+    } while (0)
+
 // ---- elementwise -----------------------------------------------------------------------------------
 template <typename T>
 bool launchTransformStrided(hipStream_t stream, int opNum, const T *x, Long xs, T *z, Long zs, const T *extra, Long n);

@@ -411,7 +411,7 @@ template <typename T> struct RandomPlainBody {
         static bool run(hipStream_t s, const RandomCtx<T> &c, const T *x, const T *y, T *z, const RandomPlan &pl,
                         int operands) {
             int grid = gridFor(pl.n, kBlock * kRngIter, kMaxGrid);
-            hipLaunchKernelGGL((randomPlainKernel<T, OP>), dim3(grid), dim3(kBlock), 0, s, c, x, y, z, operands,
+            ND4J_LAUNCH((randomPlainKernel<T, OP>), dim3(grid), dim3(kBlock), 0, s, c, x, y, z, operands,
                                pl.strided ? 1 : 0, pl.xEws, pl.yEws, pl.zEws, pl.xm, pl.ym, pl.zm);
             return true;
         }
@@ -433,33 +433,33 @@ bool launchRandom(hipStream_t s, int opNum, const RngState &rng, const T *x, con
         switch (opNum) {
             case 5: {
                 int grid = gridFor(pl.n, kBlock, kGridCap);
-                hipLaunchKernelGGL((choiceKernel<T>), dim3(grid), dim3(kBlock), 0, s, c, x, y, z, pl.strided ? 1 : 0, pl.xEws,
+                ND4J_LAUNCH((choiceKernel<T>), dim3(grid), dim3(kBlock), 0, s, c, x, y, z, pl.strided ? 1 : 0, pl.xEws,
                                    pl.yEws, pl.zEws, pl.xm, pl.ym, pl.zm, pl.yLength);
                 break;
             }
             case 6: {
                 int grid = gridFor((pl.n + 1) / 2, kBlock * kRngIter, kMaxGrid);
-                hipLaunchKernelGGL((gaussianKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                ND4J_LAUNCH((gaussianKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
                 break;
             }
             case 10: {
                 int grid = gridFor((pl.n + 1) / 2, kBlock * kRngIter, kMaxGrid);
-                hipLaunchKernelGGL((gaussianKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                ND4J_LAUNCH((gaussianKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
                 break;
             }
             case 8: {
                 int grid = gridFor(pl.n, kBlock, kGridCap);
-                hipLaunchKernelGGL((binomialKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                ND4J_LAUNCH((binomialKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
                 break;
             }
             case 9: {
                 int grid = gridFor(pl.n, kBlock, kGridCap);
-                hipLaunchKernelGGL((binomialKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                ND4J_LAUNCH((binomialKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
                 break;
             }
             case 11: {
                 int grid = gridFor((pl.n + 1) / 2, kBlock, kGridCap);
-                hipLaunchKernelGGL((truncatedNormalKernel<T>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                ND4J_LAUNCH((truncatedNormalKernel<T>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
                 break;
             }
         }
@@ -472,7 +472,7 @@ bool launchRandom(hipStream_t s, int opNum, const RngState &rng, const T *x, con
 void launchRngDump(hipStream_t s, const RngState &rng, Long start, Long n, unsigned long long *out) {
     if (n <= 0) return;
     int grid = gridFor(n, kBlock * 4, kGridCap);
-    hipLaunchKernelGGL(rngDumpKernel, dim3(grid), dim3(kBlock), 0, s, rng, start, n, out);
+    ND4J_LAUNCH(rngDumpKernel, dim3(grid), dim3(kBlock), 0, s, rng, start, n, out);
 }
 
 void launchCopy(hipStream_t s, void *dst, const void *src, Long bytes) {
@@ -480,7 +480,7 @@ void launchCopy(hipStream_t s, void *dst, const void *src, Long bytes) {
     Long nvec = bytes / 16;
     int tail = (int)(bytes - nvec * 16);
     int grid = gridFor(nvec > 0 ? nvec : 1, kBlock * 4, kGridCap);
-    hipLaunchKernelGGL(copyKernel, dim3(grid), dim3(kBlock), 0, s, reinterpret_cast<uint4 *>(dst),
+    ND4J_LAUNCH(copyKernel, dim3(grid), dim3(kBlock), 0, s, reinterpret_cast<uint4 *>(dst),
                        reinterpret_cast<const uint4 *>(src), nvec, reinterpret_cast<unsigned char *>(dst) + nvec * 16,
                        reinterpret_cast<const unsigned char *>(src) + nvec * 16, tail);
 }

@@ -308,12 +308,12 @@ template <typename T> struct Reduce3Body {
                 const Long nx = pl.numOut / pl.yMod, ny = pl.yMod;
                 const Long tiles64 = ((nx + 63) / 64) * ((ny + 63) / 64), tiles32 = ((nx + 31) / 32) * ((ny + 31) / 32);
                 if (tiles64 >= 512 && tiles64 <= kMaxGrid) {
-                    hipLaunchKernelGGL((reduce3AllTileKernel<T, OP, 64>), dim3((unsigned)tiles64), dim3(kBlock), 0, s, x, y, z, extra,
+                    ND4J_LAUNCH((reduce3AllTileKernel<T, OP, 64>), dim3((unsigned)tiles64), dim3(kBlock), 0, s, x, y, z, extra,
                                        pl.xOffsets, pl.yOffsets, nx, ny, pl.runLength);
                     return true;
                 }
                 if (tiles32 <= kMaxGrid) {
-                    hipLaunchKernelGGL((reduce3AllTileKernel<T, OP, 32>), dim3((unsigned)tiles32), dim3(kBlock), 0, s, x, y, z, extra,
+                    ND4J_LAUNCH((reduce3AllTileKernel<T, OP, 32>), dim3((unsigned)tiles32), dim3(kBlock), 0, s, x, y, z, extra,
                                        pl.xOffsets, pl.yOffsets, nx, ny, pl.runLength);
                     return true;
                 }
@@ -332,9 +332,9 @@ template <typename T> struct Reduce3Body {
                 slices = (pl.runLength + sliceLength - 1) / sliceLength;
                 if (slices >= 2) {  // a single slice needs no second launch: the per-result kernels below do it in one
                     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
-                    hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)(slices * pl.numOut)), dim3(kBlock), 0, s, x, y, z,
+                    ND4J_LAUNCH((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)(slices * pl.numOut)), dim3(kBlock), 0, s, x, y, z,
                                        extra, pl, partials, sliceLength, slices, (unsigned long long *)nullptr, 0u);
-                    hipLaunchKernelGGL((reduce3Finish<T, OP>), dim3((unsigned)pl.numOut), dim3(kBlock), 0, s, z, partials, (int)slices,
+                    ND4J_LAUNCH((reduce3Finish<T, OP>), dim3((unsigned)pl.numOut), dim3(kBlock), 0, s, z, partials, (int)slices,
                                        pl.runLength, pl.numOut == 1 ? ws.signal : nullptr, ws.ticket);
                     return true;
                 }
@@ -344,13 +344,13 @@ template <typename T> struct Reduce3Body {
             const unsigned ticket = ws.ticket;
             if (pl.runLength >= 4096) {
                 int grid = gridFor(pl.numOut, 1, kGridCap);
-                hipLaunchKernelGGL((reduce3Kernel<T, OP, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
+                ND4J_LAUNCH((reduce3Kernel<T, OP, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
             } else if (pl.runLength >= 128) {
                 int grid = gridFor(pl.numOut, kBlock / 64, kGridCap);
-                hipLaunchKernelGGL((reduce3Kernel<T, OP, 64>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
+                ND4J_LAUNCH((reduce3Kernel<T, OP, 64>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
             } else {
                 int grid = gridFor(pl.numOut, kBlock / 16, kGridCap);
-                hipLaunchKernelGGL((reduce3Kernel<T, OP, 16>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
+                ND4J_LAUNCH((reduce3Kernel<T, OP, 16>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
             }
             return true;
         }

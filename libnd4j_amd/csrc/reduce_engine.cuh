@@ -558,9 +558,9 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
             sliceLength = (sliceLength + 63) / 64 * 64;  // slices start on 16-byte boundaries whenever the TAD does
             slices = (pl.tadLength + sliceLength - 1) / sliceLength;
             Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
-            hipLaunchKernelGGL((tadRowSliceKernel<Pol>), dim3((unsigned)pl.numTads, (unsigned)slices), dim3(kBlock), 0, s, pol, x, z,
+            ND4J_LAUNCH((tadRowSliceKernel<Pol>), dim3((unsigned)pl.numTads, (unsigned)slices), dim3(kBlock), 0, s, pol, x, z,
                                partials, pl.offsets, pl.tadLength, pl.numTads, sliceLength);
-            hipLaunchKernelGGL((tadSliceFinish<Pol>), dim3((unsigned)pl.numTads), dim3(kBlock), 0, s, pol, x, z, partials,
+            ND4J_LAUNCH((tadSliceFinish<Pol>), dim3((unsigned)pl.numTads), dim3(kBlock), 0, s, pol, x, z, partials,
                                pl.offsets, pl.tadLength, pl.numTads, (int)slices);
             return;
         }
@@ -568,15 +568,15 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
     if (pl.kind == TadPlan::ROW && pl.tadLength >= 32) {
         if (pl.tadLength >= 8192) {
             int grid = gridFor(pl.numTads, 1, kGridCap);
-            hipLaunchKernelGGL((tadRowKernel<Pol, kBlock>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets,
+            ND4J_LAUNCH((tadRowKernel<Pol, kBlock>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets,
                                pl.tadLength, pl.numTads);
         } else if (pl.tadLength >= 256) {
             int grid = gridFor(pl.numTads, kBlock / 64, kGridCap);
-            hipLaunchKernelGGL((tadRowKernel<Pol, 64>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets,
+            ND4J_LAUNCH((tadRowKernel<Pol, 64>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets,
                                pl.tadLength, pl.numTads);
         } else {
             int grid = gridFor(pl.numTads, kBlock / 16, kGridCap);
-            hipLaunchKernelGGL((tadRowKernel<Pol, 16>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets,
+            ND4J_LAUNCH((tadRowKernel<Pol, 16>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets,
                                pl.tadLength, pl.numTads);
         }
         return;
@@ -601,10 +601,10 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         splits = (pl.tadLength + rowsPerSplit - 1) / rowsPerSplit;
         if (splits < 1) splits = 1;
         Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
-        hipLaunchKernelGGL((tadColVecKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
+        ND4J_LAUNCH((tadColVecKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
                            pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit);
         if (splits > 1)
-            hipLaunchKernelGGL((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kWave - 1) / kWave)), dim3(kBlock), 0, s, pol,
+            ND4J_LAUNCH((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kWave - 1) / kWave)), dim3(kBlock), 0, s, pol,
                                z, partials, pl.tadLength, pl.numTads, (int)splits);
         return;
     }
@@ -622,15 +622,15 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         splits = (pl.tadLength + rowsPerSplit - 1) / rowsPerSplit;
         if (splits < 1) splits = 1;
         Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
-        hipLaunchKernelGGL((tadColKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
+        ND4J_LAUNCH((tadColKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
                            pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit);
         if (splits > 1)
-            hipLaunchKernelGGL((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kWave - 1) / kWave)), dim3(kBlock), 0, s, pol,
+            ND4J_LAUNCH((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kWave - 1) / kWave)), dim3(kBlock), 0, s, pol,
                                z, partials, pl.tadLength, pl.numTads, (int)splits);
         return;
     }
     int grid = gridFor(pl.numTads, 1, kGridCap);
-    hipLaunchKernelGGL((tadGeneralKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets, pl.tm, pl.tadLength,
+    ND4J_LAUNCH((tadGeneralKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, z, pl.offsets, pl.tm, pl.tadLength,
                        pl.numTads);
 }
 
@@ -646,11 +646,11 @@ inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, type
     if ((size_t)grid > maxBlocks) grid = (int)maxBlocks;
     if (grid < 1) grid = 1;
     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
-    hipLaunchKernelGGL((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
+    ND4J_LAUNCH((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
                        pl.ews, pl.xm, z, ws.signal, ws.ticket, oneLaunch ? ws.slots : nullptr, ws.counter,
                        oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u);
     if (grid > 1 && !oneLaunch)
-        hipLaunchKernelGGL((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n, ws.signal, ws.ticket);
+        ND4J_LAUNCH((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n, ws.signal, ws.ticket);
 }
 
 }  // namespace nd4j_amd

@@ -14,6 +14,13 @@ Environment &environment() {
     return env;
 }
 
+bool launchesAreVerbose() { return environment().verbose.load(std::memory_order_relaxed) && environment().debug.load(std::memory_order_relaxed); }
+void printLaunch(const char *kernel, dim3 grid, dim3 block, size_t ldsBytes) {
+    std::printf("Launch: %s gridSize: [%u, %u, %u], blockSize: [%u], dynamic shmem: [%zu]\n", kernel, grid.x, grid.y, grid.z, block.x,
+                ldsBytes);
+    std::fflush(stdout);
+}
+
 bool isDeviceMemory(const void *p) {
     if (p == nullptr) return false;
     hipPointerAttribute_t attr;
@@ -112,7 +119,9 @@ void dropTadCacheLocked() {
         if (hipSetDevice(d) == hipSuccess) (void)hipDeviceSynchronize();
     }
     (void)hipSetDevice(current);
-    gTadCache.clear();  // a call that still holds an entry keeps it (and its device table) until it returns
+    // A call that still holds an entry keeps it (and its device table) until it returns; its kernel may still be queued
+    // then, which is safe because ~CachedTad's hipFree waits for the device's outstanding work before it releases memory.
+    gTadCache.clear();
     gTadCacheBytes = 0;
 }
 }  // namespace

@@ -33,7 +33,7 @@ template <typename T> struct ScalarTadBody {
             if (pl.flatInner > 0 && pl.flatInner < 0xffffffffLL && pl.flatExtent < 0xffffffffLL &&
                 (((uintptr_t)x | (uintptr_t)z) & 15) == 0) {
                 const Long n = pl.numTads * pl.tadLength;
-                hipLaunchKernelGGL((bcFlatInnerKernel<T, F>), dim3(gridFor(n / Pack<T>::N + 1, kBlock, F::tables ? kGridCap : kMaxGrid)),
+                ND4J_LAUNCH((bcFlatInnerKernel<T, F>), dim3(gridFor(n / Pack<T>::N + 1, kBlock, F::tables ? kGridCap : kMaxGrid)),
                                    dim3(kBlock), 0, s, x, scalars, z, n, pl.flatInner, pl.flatExtent, p);
                 return true;
             }
@@ -47,7 +47,7 @@ template <typename T> struct ScalarTadBody {
                 if (gy > 65535) gy = 65535;
                 int gx = gridFor(pl.numTads, (Long)rowsPerBlock * kBcRows, kMaxGrid);
                 int aligned = (((uintptr_t)x | (uintptr_t)z) & 15) == 0 ? 1 : 0;
-                hipLaunchKernelGGL((bcRowKernel<T, F, true>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, scalars, z,
+                ND4J_LAUNCH((bcRowKernel<T, F, true>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, scalars, z,
                                    pl.xOffsets, pl.zOffsets, pl.tadLength, pl.numTads, aligned, colShift, p);
             } else {
                 int gx = (int)((pl.numTads + kBlock - 1) / kBlock);
@@ -55,7 +55,7 @@ template <typename T> struct ScalarTadBody {
                 if (gy < 1) gy = 1;
                 if (gy > pl.tadLength) gy = pl.tadLength;
                 if (gy > 65535) gy = 65535;
-                hipLaunchKernelGGL((bcColKernel<T, F, true>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, scalars, z,
+                ND4J_LAUNCH((bcColKernel<T, F, true>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, scalars, z,
                                    pl.xOffsets, pl.zOffsets, pl.tadLength, pl.numTads, pl.tadEws, (Long)0, pl.zEws, p);
             }
             return true;

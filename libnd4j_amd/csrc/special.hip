@@ -412,17 +412,17 @@ template <typename T, int MODE, int GROUP, int PACKS, int BLOCK = kBlock> void r
     constexpr int N = Pack<T>::N;
     const bool whole = aligned16(x) && aligned16(z) && pl.length % N == 0 && (pl.numRows == 1 || (pl.xRow % N == 0 && pl.zRow % N == 0));
     if (whole)
-        hipLaunchKernelGGL((softmaxRowRegKernel<T, MODE, GROUP, PACKS, false, BLOCK>), dim3(grid), dim3(BLOCK), 0, s, x, z, pl.numRows,
+        ND4J_LAUNCH((softmaxRowRegKernel<T, MODE, GROUP, PACKS, false, BLOCK>), dim3(grid), dim3(BLOCK), 0, s, x, z, pl.numRows,
                            pl.length, pl.xRow, pl.zRow);
     else
-        hipLaunchKernelGGL((softmaxRowRegKernel<T, MODE, GROUP, PACKS, true, BLOCK>), dim3(grid), dim3(BLOCK), 0, s, x, z, pl.numRows,
+        ND4J_LAUNCH((softmaxRowRegKernel<T, MODE, GROUP, PACKS, true, BLOCK>), dim3(grid), dim3(BLOCK), 0, s, x, z, pl.numRows,
                            pl.length, pl.xRow, pl.zRow);
 }
 template <typename T, int MODE, int PACKS> void runColReg(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
     const Long rowsPerBlock = (Long)kColRowLanes * Pack<T>::N;
     const Long groups = (pl.numRows + rowsPerBlock - 1) / rowsPerBlock;
     const int grid = (int)(groups < (Long)kMaxGrid / 4 ? groups : (Long)kMaxGrid / 4);  // blocks of 1024 threads walk the rest
-    hipLaunchKernelGGL((softmaxColRegKernel<T, MODE, PACKS>), dim3(grid), dim3(kColBlock), 0, s, x, z, pl.numRows, pl.length, pl.xEl,
+    ND4J_LAUNCH((softmaxColRegKernel<T, MODE, PACKS>), dim3(grid), dim3(kColBlock), 0, s, x, z, pl.numRows, pl.length, pl.xEl,
                        pl.zEl, groups);
 }
 
@@ -481,21 +481,21 @@ template <typename T, int MODE> void runSoftmax(hipStream_t s, const T *x, T *z,
     }
     if (pl.xRow == 1 && pl.zRow == 1 && pl.numRows >= kWave) {
         int grid = (int)((pl.numRows + kWave - 1) / kWave);
-        hipLaunchKernelGGL((softmaxColKernel<T, MODE>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows, pl.length, pl.xRow, pl.xEl,
+        ND4J_LAUNCH((softmaxColKernel<T, MODE>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows, pl.length, pl.xRow, pl.xEl,
                            pl.zRow, pl.zEl);
         return;
     }
     if (pl.length >= 2048 || pl.numRows < 4) {
         int grid = gridFor(pl.numRows, 1, kGridCap);
-        hipLaunchKernelGGL((softmaxRowKernel<T, MODE, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows, pl.length, pl.xRow,
+        ND4J_LAUNCH((softmaxRowKernel<T, MODE, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows, pl.length, pl.xRow,
                            pl.xEl, pl.zRow, pl.zEl);
     } else if (pl.length >= 128) {
         int grid = gridFor(pl.numRows, kBlock / 64, kGridCap);
-        hipLaunchKernelGGL((softmaxRowKernel<T, MODE, 64>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows, pl.length, pl.xRow,
+        ND4J_LAUNCH((softmaxRowKernel<T, MODE, 64>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows, pl.length, pl.xRow,
                            pl.xEl, pl.zRow, pl.zEl);
     } else {
         int grid = gridFor(pl.numRows, kBlock / 16, kGridCap);
-        hipLaunchKernelGGL((softmaxRowKernel<T, MODE, 16>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows, pl.length, pl.xRow,
+        ND4J_LAUNCH((softmaxRowKernel<T, MODE, 16>), dim3(grid), dim3(kBlock), 0, s, x, z, pl.numRows, pl.length, pl.xRow,
                            pl.xEl, pl.zRow, pl.zEl);
     }
 }
@@ -632,10 +632,10 @@ bool launchSoftmaxFinish(hipStream_t s, int opNum, const T *x, T *z, const T *ma
 #define ND4J_FINISH_VEC(MODE)                                                                                              \
     do {                                                                                                                   \
         if (alongRows)                                                                                                     \
-            hipLaunchKernelGGL((softmaxFinishVecKernel<T, MODE, 1>), vgrid, dim3(kBlock), 0, s, x, z, maxima, sums, vecs,   \
+            ND4J_LAUNCH((softmaxFinishVecKernel<T, MODE, 1>), vgrid, dim3(kBlock), 0, s, x, z, maxima, sums, vecs,   \
                                slowLen, xSlow, zSlow);                                                                     \
         else                                                                                                               \
-            hipLaunchKernelGGL((softmaxFinishVecKernel<T, MODE, 0>), vgrid, dim3(kBlock), 0, s, x, z, maxima, sums, vecs,   \
+            ND4J_LAUNCH((softmaxFinishVecKernel<T, MODE, 0>), vgrid, dim3(kBlock), 0, s, x, z, maxima, sums, vecs,   \
                                slowLen, xSlow, zSlow);                                                                     \
     } while (0)
         switch (opNum) {
@@ -655,7 +655,7 @@ bool launchSoftmaxFinish(hipStream_t s, int opNum, const T *x, T *z, const T *ma
         if (gx > budget) gx = budget;
         const dim3 rgrid((unsigned)gx, (unsigned)gy);
 #define ND4J_FINISH_ROWS(MODE)                                                                                                \
-    hipLaunchKernelGGL((softmaxFinishRowsKernel<T, MODE>), rgrid, dim3(kBlock), 0, s, x, z, maxima, sums, pl.numRows, pl.length, \
+    ND4J_LAUNCH((softmaxFinishRowsKernel<T, MODE>), rgrid, dim3(kBlock), 0, s, x, z, maxima, sums, pl.numRows, pl.length, \
                        pl.xRow, pl.zRow)
         switch (opNum) {
             case 38: ND4J_FINISH_ROWS(0); return true;
@@ -667,7 +667,7 @@ bool launchSoftmaxFinish(hipStream_t s, int opNum, const T *x, T *z, const T *ma
     }
     const dim3 grid((unsigned)gridFor(fastLen, kBlock, 4096), (unsigned)(slowLen < 65535 ? slowLen : 65535));
 #define ND4J_FINISH(MODE)                                                                                                 \
-    hipLaunchKernelGGL((softmaxFinishKernel<T, MODE>), grid, dim3(kBlock), 0, s, x, z, maxima, sums, pl.numRows, pl.length, \
+    ND4J_LAUNCH((softmaxFinishKernel<T, MODE>), grid, dim3(kBlock), 0, s, x, z, maxima, sums, pl.numRows, pl.length, \
                        pl.xRow, pl.xEl, pl.zRow, pl.zEl, alongRows)
     switch (opNum) {
         case 38: ND4J_FINISH(0); return true;
@@ -776,20 +776,20 @@ __global__ void __launch_bounds__(kBlock) isMaxColFillKernel(T *z, const T *inde
 template <typename T> void launchIsMaxFill(hipStream_t s, T *z, const T *index, const FlatPlan &zp) {
     if (zp.n <= 0) return;
     int grid = gridFor(zp.n, kBlock * 4, kGridCap);
-    hipLaunchKernelGGL((isMaxFillKernel<T>), dim3(grid), dim3(kBlock), 0, s, z, index, zp.n, zp.strided ? 1 : 0, zp.ews, zp.xm);
+    ND4J_LAUNCH((isMaxFillKernel<T>), dim3(grid), dim3(kBlock), 0, s, z, index, zp.n, zp.strided ? 1 : 0, zp.ews, zp.xm);
 }
 template <typename T> void launchIsMaxTadFill(hipStream_t s, T *z, const T *index, const TadPlan &zt) {
     if (zt.numTads <= 0 || zt.tadLength <= 0) return;
     if (zt.kind == TadPlan::ROW) {
         if (zt.tadLength >= 2048) {
             const Long pieces = (zt.tadLength + (Long)kBlock * 4 * Pack<T>::N - 1) / ((Long)kBlock * 4 * Pack<T>::N);
-            hipLaunchKernelGGL((isMaxRowFillKernel<T, kBlock>), dim3(gridFor(zt.numTads * pieces, 1, kMaxGrid)), dim3(kBlock), 0, s, z,
+            ND4J_LAUNCH((isMaxRowFillKernel<T, kBlock>), dim3(gridFor(zt.numTads * pieces, 1, kMaxGrid)), dim3(kBlock), 0, s, z,
                                index, zt.offsets, zt.tadLength, zt.numTads);
         } else if (zt.tadLength >= 256) {
-            hipLaunchKernelGGL((isMaxRowFillKernel<T, 64>), dim3(gridFor(zt.numTads, kBlock / 64, kMaxGrid)), dim3(kBlock), 0, s, z,
+            ND4J_LAUNCH((isMaxRowFillKernel<T, 64>), dim3(gridFor(zt.numTads, kBlock / 64, kMaxGrid)), dim3(kBlock), 0, s, z,
                                index, zt.offsets, zt.tadLength, zt.numTads);
         } else {
-            hipLaunchKernelGGL((isMaxRowFillKernel<T, 16>), dim3(gridFor(zt.numTads, kBlock / 16, kMaxGrid)), dim3(kBlock), 0, s, z,
+            ND4J_LAUNCH((isMaxRowFillKernel<T, 16>), dim3(gridFor(zt.numTads, kBlock / 16, kMaxGrid)), dim3(kBlock), 0, s, z,
                                index, zt.offsets, zt.tadLength, zt.numTads);
         }
         return;
@@ -802,13 +802,13 @@ template <typename T> void launchIsMaxTadFill(hipStream_t s, T *z, const T *inde
         const Long per = (zt.tadLength + splits - 1) / splits;
         splits = (zt.tadLength + per - 1) / per;
         if (gx <= kMaxGrid) {
-            hipLaunchKernelGGL((isMaxColFillKernel<T>), dim3((unsigned)gx, (unsigned)splits), dim3(kBlock), 0, s, z, index, zt.offsets,
+            ND4J_LAUNCH((isMaxColFillKernel<T>), dim3((unsigned)gx, (unsigned)splits), dim3(kBlock), 0, s, z, index, zt.offsets,
                                zt.tadLength, zt.numTads, zt.tadEws, per);
             return;
         }
     }
     int grid = gridFor(zt.numTads * zt.tadLength, kBlock * 4, kGridCap);
-    hipLaunchKernelGGL((isMaxTadFillKernel<T>), dim3(grid), dim3(kBlock), 0, s, z, index, zt.offsets, zt.tadLength, zt.numTads,
+    ND4J_LAUNCH((isMaxTadFillKernel<T>), dim3(grid), dim3(kBlock), 0, s, z, index, zt.offsets, zt.tadLength, zt.numTads,
                        zt.kind == TadPlan::GENERAL ? 0 : 1, zt.tadEws, zt.tm);
 }
 

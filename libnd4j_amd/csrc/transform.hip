@@ -107,7 +107,7 @@ template <typename T> bool launchTanhVec(hipStream_t s, const T *x, Long xs, T *
         if (head > n) head = (int)n;
         const Long nvec = (n - head) / Pack<T>::N;
         const int grid = gridFor(nvec > 0 ? nvec : 1, (Long)kBlock * kTanhPacks, kMaxGrid);
-        hipLaunchKernelGGL((tanhVecKernel<T>), dim3(grid), dim3(kBlock), 0, s, x, z, n, head);
+        ND4J_LAUNCH((tanhVecKernel<T>), dim3(grid), dim3(kBlock), 0, s, x, z, n, head);
         return true;
     }
 }

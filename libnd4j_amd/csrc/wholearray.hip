@@ -129,16 +129,16 @@ template <typename T> void launchReverse(hipStream_t s, const T *x, T *z, const 
     if (p.contiguous) {
         const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(z) & 15)) & 15) / sizeof(T));
         if (p.swap) {
-            hipLaunchKernelGGL(reverseSwapVecKernel<T>, dim3(gridFor(p.n / 2 / N + 1)), dim3(kBlock), 0, s, z, p.n, head);
+            ND4J_LAUNCH(reverseSwapVecKernel<T>, dim3(gridFor(p.n / 2 / N + 1)), dim3(kBlock), 0, s, z, p.n, head);
         } else {
-            hipLaunchKernelGGL(reverseVecKernel<T>, dim3(gridFor(p.n / N + 1)), dim3(kBlock), 0, s, x, z, p.n, head);
+            ND4J_LAUNCH(reverseVecKernel<T>, dim3(gridFor(p.n / N + 1)), dim3(kBlock), 0, s, x, z, p.n, head);
         }
         return;
     }
     if (p.swap) {
-        hipLaunchKernelGGL((reverseMapKernel<T, true>), dim3(gridFor(p.count)), dim3(kBlock), 0, s, x, p.xm, z, p.zm, p.n, p.count);
+        ND4J_LAUNCH((reverseMapKernel<T, true>), dim3(gridFor(p.count)), dim3(kBlock), 0, s, x, p.xm, z, p.zm, p.n, p.count);
     } else {
-        hipLaunchKernelGGL((reverseMapKernel<T, false>), dim3(gridFor(p.count)), dim3(kBlock), 0, s, x, p.xm, z, p.zm, p.n, p.count);
+        ND4J_LAUNCH((reverseMapKernel<T, false>), dim3(gridFor(p.count)), dim3(kBlock), 0, s, x, p.xm, z, p.zm, p.n, p.count);
     }
 }
 
@@ -231,16 +231,16 @@ __global__ void __launch_bounds__(kBlock) histogramAddKernel(T *z, const T *extr
 template <typename T>
 void launchHistogram(hipStream_t s, const T *x, Long n, T *z, int capacity, const T *extra, unsigned *counts) {
     if (capacity <= 0) return;
-    hipLaunchKernelGGL(clearCountsKernel, dim3(gridFor(capacity)), dim3(kBlock), 0, s, counts, capacity);
+    ND4J_LAUNCH(clearCountsKernel, dim3(gridFor(capacity)), dim3(kBlock), 0, s, counts, capacity);
     if (n > 0) {
         // enough blocks to fill the chip, few enough that the flushes of the per-block counts stay cheap
         const int grid = gridFor(n / Pack<T>::N + 1) > 2048 ? 2048 : gridFor(n / Pack<T>::N + 1);
         if (capacity <= kLdsBins)
-            hipLaunchKernelGGL((histogramCountKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
+            ND4J_LAUNCH((histogramCountKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
         else
-            hipLaunchKernelGGL((histogramCountKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
+            ND4J_LAUNCH((histogramCountKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
     }
-    hipLaunchKernelGGL(histogramAddKernel<T>, dim3(gridFor(capacity)), dim3(kBlock), 0, s, z, extra, counts, capacity);
+    ND4J_LAUNCH(histogramAddKernel<T>, dim3(gridFor(capacity)), dim3(kBlock), 0, s, z, extra, counts, capacity);
 }
 
 // ---- Im2col ----------------------------------------------------------------------------------------------------
@@ -327,14 +327,14 @@ template <typename T> void launchIm2col(hipStream_t s, const T *x, T *z, const T
         // workgroups for whole rounds of eight channels; in one launch when that fits, else in plain order
         const Long byDie = (channels + 7) / 8 * 8 * perChannel;
         if (byDie <= kWholeGrid)
-            hipLaunchKernelGGL(im2colPlaneKernel<T>, dim3((unsigned)byDie), dim3(kBlock), 0, s, x, z, extra, gv, (unsigned)planes,
+            ND4J_LAUNCH(im2colPlaneKernel<T>, dim3((unsigned)byDie), dim3(kBlock), 0, s, x, z, extra, gv, (unsigned)planes,
                                (unsigned)byDie, 1);
         else
-            hipLaunchKernelGGL(im2colPlaneKernel<T>, dim3(gridFor(planes, 1)), dim3(kBlock), 0, s, x, z, extra, gv, (unsigned)planes,
+            ND4J_LAUNCH(im2colPlaneKernel<T>, dim3(gridFor(planes, 1)), dim3(kBlock), 0, s, x, z, extra, gv, (unsigned)planes,
                                (unsigned)planes, 0);
         return;
     }
-    hipLaunchKernelGGL(im2colKernel<T>, dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
+    ND4J_LAUNCH(im2colKernel<T>, dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
 }
 
 // ---- Col2Im ----------------------------------------------------------------------------------------------------
@@ -389,14 +389,14 @@ template <typename T> void launchCol2im(hipStream_t s, const T *x, T *z, const T
         Long bytes = clearFirst * (Long)sizeof(T);
         Long lead = (Long)((16 - (reinterpret_cast<uintptr_t>(base) & 15)) & 15);
         if (lead > bytes) lead = bytes;
-        if (lead > 0) hipLaunchKernelGGL(clearBytesKernel, dim3(1), dim3(kBlock), 0, s, nullptr, 0, base, (int)lead);
+        if (lead > 0) ND4J_LAUNCH(clearBytesKernel, dim3(1), dim3(kBlock), 0, s, nullptr, 0, base, (int)lead);
         const Long vectors = (bytes - lead) / 16;
         const int tailBytes = (int)(bytes - lead - vectors * 16);
-        hipLaunchKernelGGL(clearBytesKernel, dim3(gridFor(vectors + 1)), dim3(kBlock), 0, s, reinterpret_cast<U32x4 *>(base + lead), vectors,
+        ND4J_LAUNCH(clearBytesKernel, dim3(gridFor(vectors + 1)), dim3(kBlock), 0, s, reinterpret_cast<U32x4 *>(base + lead), vectors,
                            base + lead + vectors * 16, tailBytes);
-        hipLaunchKernelGGL((col2imKernel<T, true>), dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
+        ND4J_LAUNCH((col2imKernel<T, true>), dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
     } else {
-        hipLaunchKernelGGL((col2imKernel<T, false>), dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
+        ND4J_LAUNCH((col2imKernel<T, false>), dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
     }
 }
 
@@ -450,7 +450,7 @@ __global__ void __launch_bounds__(kBlock) pooling2dKernel(const T *x, T *z, cons
 template <typename T> void launchPooling2d(hipStream_t s, const T *x, T *z, const T *extra, const ConvGeometry &g) {
     const Long total = (Long)g.bS * g.iC * g.oH * g.oW;
     if (total <= 0) return;
-    hipLaunchKernelGGL(pooling2dKernel<T>, dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
+    ND4J_LAUNCH(pooling2dKernel<T>, dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
 }
 
 // ---- DropOut 43 / DropOutInverted 44 as transforms ---------------------------------------------------------------
@@ -480,9 +480,9 @@ void launchDropoutTransform(hipStream_t s, bool inverted, const T *x, const DimM
                             Long n, unsigned long long seed) {
     if (n <= 0) return;
     if (inverted)
-        hipLaunchKernelGGL((dropoutTransformKernel<T, true>), dim3(gridFor(n)), dim3(kBlock), 0, s, x, xm, z, zm, extra, n, seed);
+        ND4J_LAUNCH((dropoutTransformKernel<T, true>), dim3(gridFor(n)), dim3(kBlock), 0, s, x, xm, z, zm, extra, n, seed);
     else
-        hipLaunchKernelGGL((dropoutTransformKernel<T, false>), dim3(gridFor(n)), dim3(kBlock), 0, s, x, xm, z, zm, extra, n, seed);
+        ND4J_LAUNCH((dropoutTransformKernel<T, false>), dim3(gridFor(n)), dim3(kBlock), 0, s, x, xm, z, zm, extra, n, seed);
 }
 
 #define INST(T)                                                                                                   \

@@ -15,7 +15,7 @@ from . import harness
 F32 = np.float32
 
 # opNums (reference: include/loops/legacy_ops.h)
-T_EXP, T_TANH = 3, 15
+T_EXP, T_TANH, T_TANH_DERIVATIVE = 3, 15, 23
 T_SOFTMAX, T_LOGSOFTMAX, T_ISMAX = 38, 40, 41
 P_ADD, P_MUL = 0, 6
 S_MUL = 2  # scalar family
@@ -137,9 +137,16 @@ def transform_tanh(dev, n=1 << 24, seed=42, copies=None):
     def device_set(w):
         X, Z = w.operand(x, xi), w.operand(np.zeros(n, F32), xi)
         ex = dev.extra(xi, z_info=xi)
-        return [Case("transform_tanh", "transform", n, 8 * n,
-                     lambda: ops.execTransformFloat(ex, T_TANH, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, None),
-                     lambda lib: (lib.transform(T_TANH, x, xi, zc, xi, None), zc)[1], True, Z.get)]
+        cases = [Case("transform_tanh", "transform", n, 8 * n,
+                      lambda: ops.execTransformFloat(ex, T_TANH, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, None),
+                      lambda lib: (lib.transform(T_TANH, x, xi, zc, xi, None), zc)[1], True, Z.get),
+                 # 1 - tanh^2 keeps the C library's tanhf, replayed bit for bit, for every element: what tanh itself cost
+                 # before its arguments of 1 and above took a cheaper route
+                 Case("transform_tanh_derivative", "transform", n, 8 * n,
+                      lambda: ops.execTransformFloat(ex, T_TANH_DERIVATIVE, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, None),
+                      lambda lib: (lib.transform(T_TANH_DERIVATIVE, x, xi, zc, xi, None), zc)[1], True, Z.get)]
+        cases[1].bound = "valu"
+        return cases
 
     return _replicated(dev, "transform tanh fp32 1-D 2^%d" % int(np.log2(n)), 8 * n, dict(x=x, xi=xi, z_cpu=zc),
                        device_set, copies)
@@ -560,6 +567,14 @@ def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data
                  lambda lib: (cpu_gen(lib).random_xz(RND_DROPOUT, cpu_state["x"], di, cpu_state["x"], di, np.array([0.5], F32)), cpu_state["x"])[1],
                  True, Xd.get)]
 
+    def valu_bound(cases):
+        # bound by the instruction count of the reference's 64-bit integer stream, not by HBM
+        for c in cases:
+            c.bound = "valu"
+        return cases
+
+    inner_set = device_set
+    device_set = lambda w: valu_bound(inner_set(w))
     host_cpu_state = cpu_state
     w = _replicated(dev, "random uniform / gaussian fill 2^%d fp32, dropout p=0.5 in place [%d,%d]" % (int(np.log2(n)), side, side),
                     4 * n + 4 * m, dict(rng_buffer=host_buf, generator=gen, seed=seed, buffer_longs=buffer_longs,

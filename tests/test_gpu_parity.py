@@ -723,6 +723,24 @@ def test_dropout_transforms(gpu):
     assert np.all(np.delete(z, np.arange(1000) * 3) == 0) and 0.2 < (z[::3] != 0).mean() < 0.4
 
 
+def test_debug_and_verbose_mode_print_the_launches(gpu, capfd):
+    x = np.linspace(-1, 1, 1000).astype(np.float32)
+    vi = shape_info_np([1, 1000])
+    gpu.ops.enableDebugMode(True)
+    gpu.ops.enableVerboseMode(True)
+    try:
+        got = gpu.transform(0, x, vi, vi)
+        total = gpu.reduce_scalar(1, np.ones(1000, np.float32), vi)
+    finally:
+        gpu.ops.enableDebugMode(False)
+        gpu.ops.enableVerboseMode(False)
+    out = capfd.readouterr().out
+    assert np.array_equal(got, np.abs(x)) and float(total) == 1000.0
+    assert "Launch:" in out and "ewVecKernel" in out and "flatKernel" in out and "gridSize" in out
+    gpu.transform(0, x, vi, vi)
+    assert "Launch:" not in capfd.readouterr().out
+
+
 def test_half_families(gpu, cpu):
     rs = np.random.RandomState(28)
     h = np.float16
