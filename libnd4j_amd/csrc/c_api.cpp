@@ -275,6 +275,7 @@ void nd4j_amd_execReduceFloatNoAlloc(Nd4jPointer *extraPointers, int opNum, floa
     guardVoid([&] { nd4j_amd::reduceFloatNoAlloc(extraPointers, opNum, x, xShapeInfo, extraParams, result); });
 }
 Nd4jLong nd4j_amd_hostFetchCount(void) { return (Nd4jLong)nd4j_amd::hostFetchCount(); }
+void nd4j_amd_setCooperativeWaitLimit(int tries) { nd4j_amd::setCooperativeWaitLimit(tries); }
 void nd4j_amd_copyKernel(Nd4jPointer *extraPointers, void *dst, const void *src, Nd4jLong bytes) {
     guardVoid([&] {
         hipStream_t s = nd4j_amd::streamOf(extraPointers);

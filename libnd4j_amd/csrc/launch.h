@@ -91,6 +91,8 @@ struct Workspace {
     unsigned long long *slots = nullptr;
     size_t slotBytes = 0;
     unsigned *counter = nullptr;
+    unsigned *rowStates = nullptr;         // rowStateCount 32-bit words beside the slots, for launches that decide per row
+    size_t rowStateCount = 0;
     unsigned *slotTicketSource = nullptr;  // host memory: the last ticket handed out for these slots
     // the next ticket: every launch that uses the slots takes its own
     unsigned nextSlotTicket() const {
@@ -165,6 +167,14 @@ template <typename T> bool launchSoftmax(hipStream_t stream, int opNum, const T 
 // row sums of exp(x - max) (these in the compute type) in two per-row arrays, and launchSoftmaxFinish writes exp(x - max) / sum (38), its
 // derivative p (1 - p) (39) or its logarithm (40)
 template <typename T> bool softmaxFitsRegisters(const T *x, const T *z, const SoftmaxPlan &plan);
+// The softmax family over contiguous rows (misaligned alike in x and z) that do not fit the register-resident kernels, in one pass:
+// the blocks that hold the slices of a row exchange their maxima and sums through ws.slots.  False when the operands
+// (or a workspace without slots) do not allow it; the caller then takes launchSoftmaxStats + launchSoftmaxFinish.
+// How many polls a block of that kernel spends on a slice of its row that has not been published yet before it votes to
+// abort the row (which the repair kernel then computes).  For tests of that path: 0 makes whatever is not there at the
+// first look count as missing.  Default 5000.
+void setCooperativeWaitLimit(int tries);
+template <typename T> bool launchSoftmaxCooperative(hipStream_t stream, int opNum, const T *x, T *z, const SoftmaxPlan &plan, Workspace ws);
 template <typename T>
 bool launchSoftmaxStats(hipStream_t stream, const T *x, T *maxima, typename Compute<T>::type *sums, const TadPlan &plan, Workspace ws);
 template <typename T>

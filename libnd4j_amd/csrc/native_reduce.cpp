@@ -526,6 +526,14 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
         const bool rowMajor = pl.xEl == 1 && pl.zEl == 1 && (pl.length >= 16384 || (pl.length >= 4096 && pl.numRows <= 512));
         const bool colMajor = pl.xRow == 1 && pl.zRow == 1 && pl.numRows >= 256 && pl.length >= 256;
         if (rank >= 1 && (rowMajor || colMajor) && !softmaxFitsRegisters<T>(x, z, pl)) {
+            if (rowMajor) {
+                // aligned rows: one pass, the blocks of a row exchanging their maxima and sums
+                Scratch coop = scratchFor(s);
+                if (launchSoftmaxCooperative<T>(s, opNum, x, z, pl, coop.rest)) {
+                    checkLaunch("execTransform(softmax)", s);
+                    return true;
+                }
+            }
             ResolvedTad tx;
             if (!resolveTad(nullptr, 0, 0, hx, &walked, 1, tx, s)) return true;
             typedef typename Compute<T>::type C;  // the row sums stay in the compute type: those of half rows may exceed half

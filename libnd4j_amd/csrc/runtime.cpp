@@ -150,11 +150,12 @@ Workspace workspaceFor(hipStream_t s, size_t minBytes) {
 
 namespace {
 struct FlatSlots {
-    void *block = nullptr;  // kFlatSlotBytes of slots, then kFlatCounterBytes of block counters
+    void *block = nullptr;  // kFlatSlotBytes of slots, then kFlatCounterBytes of block counters, then kFlatStateBytes of row states
     unsigned ticket = 0;
 };
 const size_t kFlatSlotBytes = 256u << 10;  // 2048 blocks x 16 accumulator words x 8 bytes
 const size_t kFlatCounterBytes = 16u << 10;  // 65 counters, 128 bytes apart
+const size_t kFlatStateBytes = 64u << 10;    // 16384 per-row state words
 std::map<std::pair<int, hipStream_t>, FlatSlots> gFlatSlots;
 }  // namespace
 
@@ -164,14 +165,16 @@ void addFlatSlots(Workspace &w, hipStream_t s) {
     std::lock_guard<std::mutex> lock(gMutex);
     FlatSlots &f = gFlatSlots[std::make_pair(dev, s)];
     if (f.block == nullptr) {
-        hipError_t e = hipMalloc(&f.block, kFlatSlotBytes + kFlatCounterBytes);
+        hipError_t e = hipMalloc(&f.block, kFlatSlotBytes + kFlatCounterBytes + kFlatStateBytes);
         if (e != hipSuccess) { f.block = nullptr; throwHip("reduction slots allocation", e); }
-        e = hipMemset(f.block, 0, kFlatSlotBytes + kFlatCounterBytes);
+        e = hipMemset(f.block, 0, kFlatSlotBytes + kFlatCounterBytes + kFlatStateBytes);
         if (e != hipSuccess) throwHip("reduction slots clearing", e);
     }
     w.slots = reinterpret_cast<unsigned long long *>(f.block);
     w.slotBytes = kFlatSlotBytes;
     w.counter = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(f.block) + kFlatSlotBytes);
+    w.rowStates = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(f.block) + kFlatSlotBytes + kFlatCounterBytes);
+    w.rowStateCount = kFlatStateBytes / sizeof(unsigned);
     w.slotTicketSource = &f.ticket;  // map nodes stay where they are
 }
 

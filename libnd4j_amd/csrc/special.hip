@@ -7,6 +7,8 @@
 // Here one launch does a row: maximum, sum of exp(x - max), then the result - exp is evaluated twice instead of
 // being stored and read back, so a row costs one read of x from HBM (the second and third pass hit the caches
 // for rows of ordinary length) and one write of z: 8 bytes per element instead of the chain's 32.
+#include <atomic>
+
 #include "elementwise.cuh"
 #include "launch.h"
 #include "reduce_engine.cuh"
@@ -403,6 +405,236 @@ __global__ void __launch_bounds__(kColBlock) softmaxColRegKernel(const T *x, T *
                       softmaxPackFromKept<T, MODE, true, C>(cache[j], sum, logSum));
         }
     }
+}
+
+// ---- rows too long for one block's registers, in one pass: the blocks of a row cooperate ------------------------------
+// A row is cut into slices of kCoopPacks * 256 vectors; a block keeps one slice in registers, takes the slice's maximum
+// m and its sum s of exp(x - m), and publishes (m, s) in the row's slot group (8-byte words tagged with the launch's
+// ticket, one relaxed device-scope store each: complete or absent, no fence).  Then it waits until every slice of its
+// row has published, merges the pairs (M = max m_i, S = sum s_i exp(m_i - M)) and finishes its slice from the
+// registers: exp(x - m) exp(m - M) / S.  x is read once and z written once, where maxima and sums from a reduction
+// pass followed by an elementwise pass read x twice.
+//
+// Waiting for other blocks needs them to be running.  The blocks of a row have consecutive numbers, and workgroups are
+// handed out in order (per die as well), so when a block waits, the blocks before it are running or done, and the
+// first row that is not finished has all its blocks on the chip: it completes and makes room.  That order is how the
+// chip behaves, not a promise of the programming model, and two such launches on two streams could block each other.
+// So every wait is bounded, and what a row does is decided once, by a compare-and-swap on the row's state word (the
+// words lie 128 bytes apart: device-scope atomics on one 128-byte line are served one after the other, and with the
+// rows' words side by side the kernel took twice as long): the
+// first block that has seen all the row's slices commits the row; a block whose wait ran out first aborts it.  After a
+// commit every slice is known to be there, so late blocks just read them; after an abort no block of the row writes
+// anything, and the repair kernel behind the launch computes such rows the slow way, from x, which nobody has touched
+// (z may be x).
+static constexpr int kCoopPacks = 8;
+static constexpr unsigned kCoopCommit = 1u, kCoopAbort = 2u;
+static constexpr int kCoopStateStride = 32;  // the rows' state words are 128 bytes apart
+static constexpr int kCoopLateTries = 5000;   // polls (a microsecond or two each) for a slice that is known to have been published
+// polls a block spends on a slice that may not have been published yet before it votes to abort its row; a test may
+// set it to zero, so that whatever is not there at the first look counts as missing
+static std::atomic<int> gCoopWaitTries{5000};
+void setCooperativeWaitLimit(int tries) { gCoopWaitTries.store(tries < 0 ? 0 : tries); }
+
+template <typename C> struct CoopPair { C m, s; };
+
+// one word of a slot group, waiting at most `tries` polls for the ticket; false when it did not come
+__device__ __forceinline__ bool tryAwaitSlot(const unsigned long long *slot, unsigned ticket, int tries, unsigned &payload) {
+    unsigned long long v = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int t = 0; (unsigned)(v >> 32) != ticket && t < tries; t++) {
+        __builtin_amdgcn_s_sleep(8);
+        v = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    payload = (unsigned)v;
+    return (unsigned)(v >> 32) == ticket;
+}
+template <typename C> __device__ __forceinline__ bool tryAwaitPair(const unsigned long long *slot, unsigned ticket, int tries, CoopPair<C> &out) {
+    constexpr int W = sizeof(CoopPair<C>) / 4;
+    struct Words { unsigned w[W]; };
+    Words in;
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < W; i++) ok = tryAwaitSlot(slot + i, ticket, tries, in.w[i]) && ok;
+    out = __builtin_bit_cast(CoopPair<C>, in);
+    return ok;
+}
+
+template <typename T, int MODE>
+__global__ void __launch_bounds__(kBlock) softmaxRowCoopKernel(const T *x, T *z, Long row0, Long numRows, Long length, Long xRow, Long zRow,
+                                                               int slices, unsigned long long *slots, unsigned *rowState, unsigned ticket, int waitTries) {
+    typedef typename Compute<T>::type C;
+    constexpr int N = Pack<T>::N, PACKS = kCoopPacks;
+    constexpr int W = sizeof(CoopPair<C>) / 4;
+    __shared__ C smem[kBlock / kWave];
+    __shared__ unsigned decision;
+    __shared__ int allThere;
+    const Long local = (Long)blockIdx.x / slices;   // row within this launch
+    const int sl = (int)((Long)blockIdx.x - local * slices);
+    const Long r = row0 + local;
+    if (r >= numRows) return;
+    const T *xrow = x + r * xRow;
+    T *zrow = z + r * zRow;
+    // A row need not start on a 16-byte boundary nor hold whole vectors: the elements before its first aligned vector
+    // are kept, one per lane, by the first lanes of its first slice, those behind its last whole vector by the first
+    // lanes of its last slice (x and z are misaligned alike in every row: the host checks it).
+    Long head = (Long)(((16 - (reinterpret_cast<uintptr_t>(xrow) & 15)) & 15) / sizeof(T));
+    if (head > length) head = length;
+    const Long nvecRow = (length - head) / N;
+    const Long tail0 = head + nvecRow * N;
+    const Long v0 = (Long)sl * PACKS * kBlock;       // first vector of the slice
+    const bool holdsHead = sl == 0 && (Long)threadIdx.x < head;
+    const bool holdsTail = sl == slices - 1 && (Long)threadIdx.x < length - tail0;
+    const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(xrow + head);
+    Pack<T> cache[PACKS];
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (v0 + j * kBlock + threadIdx.x < nvecRow) cache[j] = loadPack(xv + v0 + j * kBlock + threadIdx.x);
+    C edge = holdsTail ? toCompute(xrow[tail0 + threadIdx.x]) : (C)0;
+    C front = holdsHead ? toCompute(xrow[threadIdx.x]) : (C)0;
+    C mx = holdsTail ? edge : (C)-3.4028235e38;
+    if (holdsHead) mx = m::max_(mx, front);
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (v0 + j * kBlock + threadIdx.x < nvecRow) {
+#pragma unroll
+            for (int e = 0; e < N; e++) mx = m::max_(mx, toCompute(cache[j].v[e]));
+        }
+    mx = teamAll<MaxMerge<C>, kBlock>(mx, smem);
+    C sum = (C)0;
+    if (holdsTail) {
+        const C d = edge - mx, ex = m::expSoft_(d);
+        sum = toCompute(fromCompute<T>(ex));
+        edge = toCompute(fromCompute<T>(softmaxKeep<MODE, C>(ex, d)));
+    }
+    if (holdsHead) {
+        const C d = front - mx, ex = m::expSoft_(d);
+        sum += toCompute(fromCompute<T>(ex));
+        front = toCompute(fromCompute<T>(softmaxKeep<MODE, C>(ex, d)));
+    }
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (v0 + j * kBlock + threadIdx.x < nvecRow) {
+#pragma unroll
+            for (int e = 0; e < N; e++) {
+                const C d = toCompute(cache[j].v[e]) - mx, ex = m::expSoft_(d);
+                sum += ex;
+                cache[j].v[e] = fromCompute<T>(softmaxKeep<MODE, C>(ex, d));
+            }
+        }
+    sum = teamAll<SumMerge<C>, kBlock>(sum, smem);
+    unsigned long long *group = slots + (size_t)local * slices * W;
+    if (threadIdx.x == 0) {
+        CoopPair<C> mine;
+        mine.m = mx;
+        mine.s = sum;
+        publishSlots(group + (size_t)sl * W, mine, ticket);
+        allThere = 1;
+    }
+    __syncthreads();
+    // thread t collects slice t of the row (a row has at most 256 slices)
+    CoopPair<C> theirs;
+    theirs.m = (C)-3.4028235e38;
+    theirs.s = (C)0;
+    bool have = true;
+    if ((int)threadIdx.x < slices) {
+        have = tryAwaitPair<C>(group + (size_t)threadIdx.x * W, ticket, waitTries, theirs);
+        if (!have) allThere = 0;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        // the row's decision: the first block to get here makes it for all
+        const unsigned want = (ticket << 2) | (allThere ? kCoopCommit : kCoopAbort);
+        unsigned seen = __hip_atomic_load(rowState + local * kCoopStateStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        while ((seen >> 2) != ticket) {
+            if (__hip_atomic_compare_exchange_strong(rowState + local * kCoopStateStride, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+                seen = want;
+                break;
+            }
+        }
+        decision = seen & 3u;
+    }
+    __syncthreads();
+    if (decision != kCoopCommit) return;  // aborted: the repair kernel computes this row
+    // committed: every slice of the row has been published (a thread that gave up waiting finds its slice now)
+    if (!have) tryAwaitPair<C>(group + (size_t)threadIdx.x * W, ticket, kCoopLateTries, theirs);
+    const C rowMax = teamAll<MaxMerge<C>, kBlock>(theirs.m, smem);
+    const C rowSum = teamAll<SumMerge<C>, kBlock>((int)threadIdx.x < slices ? theirs.s * m::expSoft_(theirs.m - rowMax) : (C)0, smem);
+    // this slice's exp(x - mx) -> exp(x - rowMax) / rowSum; for the logarithm (x - mx) + (mx - rowMax) - log(rowSum)
+    const C shift = mx - rowMax;
+    const C scale = m::expSoft_(shift) / rowSum;
+    const C logSum = rowLog<MODE, C>(rowSum) - shift;
+    Pack<T> *zv = reinterpret_cast<Pack<T> *>(zrow + head);
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (v0 + j * kBlock + threadIdx.x < nvecRow)
+            storePack(zv + v0 + j * kBlock + threadIdx.x, softmaxPackFromKept<T, MODE, false, C>(cache[j], &scale, &logSum));
+    if (holdsTail) zrow[tail0 + threadIdx.x] = fromCompute<T>(softmaxFromKept<MODE, C>(edge, scale, logSum));
+    if (holdsHead) zrow[threadIdx.x] = fromCompute<T>(softmaxFromKept<MODE, C>(front, scale, logSum));
+}
+
+// Rows that softmaxRowCoopKernel aborted (none, unless the chip handed out workgroups in an unexpected order or two such
+// launches got in each other's way): a block per aborted row, three passes over the row, which nobody has written.
+template <typename T, int MODE>
+__global__ void __launch_bounds__(kBlock) softmaxRowRepairKernel(const T *x, T *z, Long row0, Long rowsHere, Long length, Long xRow, Long zRow,
+                                                                 const unsigned *rowState, unsigned ticket) {
+    typedef typename Compute<T>::type C;
+    __shared__ C smem[kBlock / kWave];
+    for (Long local = blockIdx.x; local < rowsHere; local += gridDim.x) {
+        const unsigned st = __hip_atomic_load(rowState + local * kCoopStateStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (st == ((ticket << 2) | kCoopCommit)) continue;  // (a block-uniform decision)
+        const T *xr = x + (row0 + local) * xRow;
+        T *zr = z + (row0 + local) * zRow;
+        C mx = (C)-3.4028235e38;
+        for (Long c = threadIdx.x; c < length; c += kBlock) mx = m::max_(mx, toCompute(xr[c]));
+        mx = teamAll<MaxMerge<C>, kBlock>(mx, smem);
+        C sum = (C)0;
+        for (Long c = threadIdx.x; c < length; c += kBlock) sum += m::expSoft_(toCompute(xr[c]) - mx);
+        sum = teamAll<SumMerge<C>, kBlock>(sum, smem);
+        const C logSum = rowLog<MODE, C>(sum), inv = (C)1 / sum;
+        __syncthreads();  // in place: every thread has read its part of the row in both passes before any writes
+        for (Long c = threadIdx.x; c < length; c += kBlock) zr[c] = fromCompute<T>(softmaxAt<MODE, C>(toCompute(xr[c]) - mx, inv, logSum));
+        __syncthreads();
+    }
+}
+
+// true when the call was taken: contiguous rows, misaligned alike in x and z, too long for the register-resident kernels
+template <typename T> bool launchSoftmaxCooperative(hipStream_t s, int opNum, const T *x, T *z, const SoftmaxPlan &pl, Workspace ws) {
+    typedef typename Compute<T>::type C;
+    constexpr int N = Pack<T>::N;
+    constexpr int W = sizeof(CoopPair<C>) / 4;
+    if (opNum < 38 || opNum > 40) return false;
+    if (pl.xEl != 1 || pl.zEl != 1 || pl.numRows <= 0 || pl.length < (Long)kCoopPacks * kBlock * N) return false;
+    // x and z misaligned alike in every row: equal distance of the bases and of the row pitches from a 16-byte boundary
+    const uintptr_t xa = reinterpret_cast<uintptr_t>(x), za = reinterpret_cast<uintptr_t>(z);
+    if (xa % sizeof(T) != 0 || (xa & 15) != (za & 15)) return false;
+    if (pl.numRows > 1 && ((pl.xRow - pl.zRow) * (Long)sizeof(T)) % 16 != 0) return false;
+    if (ws.slots == nullptr || ws.rowStates == nullptr || ws.slotTicketSource == nullptr) return false;
+    const Long perSlice = (Long)kCoopPacks * kBlock * N;
+    // (a row that starts off a boundary has up to N - 1 elements before its first vector; they travel with slice 0)
+    const Long slices = (pl.length + perSlice - 1) / perSlice;
+    if (slices > kBlock) return false;  // a thread per slice collects the row's pairs
+    // rows per launch: what the slot groups and the state words hold (and a grid may number)
+    Long rowsPer = (Long)(ws.slotBytes / sizeof(unsigned long long)) / (slices * W);
+    if (rowsPer > (Long)ws.rowStateCount / kCoopStateStride) rowsPer = (Long)ws.rowStateCount / kCoopStateStride;
+    if (rowsPer * slices > (Long)kMaxGrid) rowsPer = (Long)kMaxGrid / slices;
+    if (rowsPer < 1) return false;
+    for (Long row0 = 0; row0 < pl.numRows; row0 += rowsPer) {
+        const Long rowsHere = pl.numRows - row0 < rowsPer ? pl.numRows - row0 : rowsPer;
+        const unsigned ticket = ws.nextSlotTicket() & 0x3fffffffu;
+        const dim3 grid((unsigned)(rowsHere * slices));
+        const dim3 repair((unsigned)(rowsHere < 1024 ? rowsHere : 1024));
+#define ND4J_COOP(MODE)                                                                                                         \
+    do {                                                                                                                        \
+        ND4J_LAUNCH((softmaxRowCoopKernel<T, MODE>), grid, dim3(kBlock), 0, s, x, z, row0, pl.numRows, pl.length, pl.xRow, pl.zRow, \
+                    (int)slices, ws.slots, ws.rowStates, ticket, gCoopWaitTries.load());                                          \
+        ND4J_LAUNCH((softmaxRowRepairKernel<T, MODE>), repair, dim3(kBlock), 0, s, x, z, row0, rowsHere, pl.length, pl.xRow,   \
+                    pl.zRow, ws.rowStates, ticket);                                                                             \
+    } while (0)
+        if (opNum == 38) ND4J_COOP(0);
+        else if (opNum == 39) ND4J_COOP(1);
+        else ND4J_COOP(2);
+#undef ND4J_COOP
+    }
+    return true;
 }
 
 template <typename T> static bool aligned16(const T *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -814,6 +1046,7 @@ template <typename T> void launchIsMaxTadFill(hipStream_t s, T *z, const T *inde
 
 #define INST(T)                                                                                           \
     template bool launchSoftmax<T>(hipStream_t, int, const T *, T *, const SoftmaxPlan &);                \
+    template bool launchSoftmaxCooperative<T>(hipStream_t, int, const T *, T *, const SoftmaxPlan &, Workspace);  \
     template bool softmaxFitsRegisters<T>(const T *, const T *, const SoftmaxPlan &);                     \
     template bool launchSoftmaxFinish<T>(hipStream_t, int, const T *, T *, const T *, const Compute<T>::type *, const SoftmaxPlan &); \
     template void launchIsMaxFill<T>(hipStream_t, T *, const T *, const FlatPlan &);                      \

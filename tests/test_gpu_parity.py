@@ -741,6 +741,47 @@ def test_debug_and_verbose_mode_print_the_launches(gpu, capfd):
     assert "Launch:" not in capfd.readouterr().out
 
 
+def test_softmax_of_long_rows_cooperating_blocks(gpu, cpu):
+    # contiguous, 16-byte aligned rows too long for one block's registers: the blocks that hold the slices of a row
+    # exchange maxima and sums.  Checked against float64 and the CPU checker, out of place and in place, for the three
+    # ops and types; then again with the blocks' patience set to zero from the host, so that every row whose slices are
+    # not all there at the first look is aborted and computed by the repair kernel - same results.
+    rs = np.random.RandomState(37)
+
+    def run(limit):
+        gpu.ops.amd_setCooperativeWaitLimit(limit)
+        for shape, dt in (([6, 40000], np.float32), ([1, 300001], np.float32), ([700, 8192 + 4 * 7], np.float32),
+                          ([3, 16384 * 3 + 8], np.float16), ([5, 20002], np.float64), ([40, 262144], np.float32),
+                          # rows of odd length: every row starts at another distance from a 16-byte boundary
+                          ([33, 50257], np.float32), ([7, 20001], np.float16), ([9, 9001], np.float64)):
+            n = shape[0] * shape[1]
+            info = harness.shape_info(shape, "c")
+            x = rs.uniform(-6, 6, n).astype(dt)
+            rows = x.astype(np.float64).reshape(shape)
+            truth = np.exp(rows - rows.max(axis=1, keepdims=True))
+            truth /= truth.sum(axis=1, keepdims=True)
+            rtol = {np.float32: 2e-5, np.float16: 1e-2, np.float64: 1e-12}[dt]
+            atol = {np.float32: 1e-7, np.float16: 1e-4, np.float64: 1e-300}[dt]
+            for op, f in ((38, lambda v: v), (39, lambda v: v * (1 - v)), (40, np.log)):
+                got = gpu.transform(op, x, info, info).astype(np.float64).reshape(shape)
+                assert np.all(np.abs(got - f(truth)) <= rtol * np.abs(f(truth)) + atol), (shape, dt, op, limit)
+                inplace = gpu.transform_inplace(op, x, info).astype(np.float64).reshape(shape)
+                if limit > 0:
+                    assert np.array_equal(inplace, got), (shape, dt, op, limit, "in place")
+                else:
+                    # with no patience, which rows the slow kernel redoes (it sums in another order) is a matter of timing
+                    assert np.all(np.abs(inplace - f(truth)) <= rtol * np.abs(f(truth)) + atol), (shape, dt, op, limit, "in place")
+            if dt == np.float32 and n <= 300001:
+                c = cpu.transform(38, x, info, info)
+                assert np.all(np.abs(gpu.transform(38, x, info, info).astype(np.float64) - c) <= 1e-5 * np.abs(c) + 1e-7)
+
+    try:
+        run(5000)
+        run(0)
+    finally:
+        gpu.ops.amd_setCooperativeWaitLimit(5000)
+
+
 def test_half_families(gpu, cpu):
     rs = np.random.RandomState(28)
     h = np.float16
