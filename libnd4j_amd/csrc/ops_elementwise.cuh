@@ -80,7 +80,7 @@ ND4J_TRANSFORM(11, Sign, return (C)((d1 > (C)0) - (d1 < (C)0));)
 ND4J_TRANSFORM(12, Sin, return m::sin_(d1);)
 ND4J_TRANSFORM(13, SoftPlus, return m::log_((C)1 + m::exp_(d1));)
 ND4J_TRANSFORM(14, Sqrt, return m::sqrt_(d1);)
-ND4J_TRANSFORM(15, Tanh, return m::tanh_(d1);)
+ND4J_TRANSFORM(15, Tanh, return m::tanhNear_(d1);)
 ND4J_TRANSFORM(16, ACos, return m::acos_(d1);)
 ND4J_TRANSFORM(17, ASin, return m::asin_(d1);)
 ND4J_TRANSFORM(18, ATan, return m::atan_(d1);)
@@ -99,6 +99,7 @@ ND4J_TRANSFORM(22, ELUDerivative, {
     return m::exp_(d1);
 })
 ND4J_TRANSFORM(23, TanhDerivative, {
+    // the C library's tanhf bit for bit, not the cheaper tanhNear_: near saturation one ULP of tanh is many of 1 - tanh^2
     C t = m::tanh_(d1);
     return (C)1 - t * t;
 })

@@ -140,8 +140,8 @@ def transform_tanh(dev, n=1 << 24, seed=42, copies=None):
         cases = [Case("transform_tanh", "transform", n, 8 * n,
                       lambda: ops.execTransformFloat(ex, T_TANH, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, None),
                       lambda lib: (lib.transform(T_TANH, x, xi, zc, xi, None), zc)[1], True, Z.get),
-                 # 1 - tanh^2 keeps the C library's tanhf, replayed bit for bit, for every element: what tanh itself cost
-                 # before its arguments of 1 and above took a cheaper route
+                 # 1 - tanh^2 keeps the C library's tanhf, replayed bit for bit, for every element (near saturation one
+                 # ULP of tanh is a multiple of the result): what tanh itself cost while it did the same
                  Case("transform_tanh_derivative", "transform", n, 8 * n,
                       lambda: ops.execTransformFloat(ex, T_TANH_DERIVATIVE, X.ptr, X.info_ptr, Z.ptr, Z.info_ptr, None),
                       lambda lib: (lib.transform(T_TANH_DERIVATIVE, x, xi, zc, xi, None), zc)[1], True, Z.get)]

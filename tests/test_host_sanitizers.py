@@ -16,7 +16,6 @@ def test_shape_and_view_logic_under_sanitizers(tmp_path):
     subprocess.check_call(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
                            "-fno-omit-frame-pointer", os.path.join(HERE, "host_sanitize.cpp"), "-o", exe])
     env = dict(os.environ)
-    env.pop("LD_PRELOAD", None)  # the sanitizer runtime wants to come first
     env["ASAN_OPTIONS"] = "detect_leaks=1:abort_on_error=0:verify_asan_link_order=0"
     env["UBSAN_OPTIONS"] = "print_stacktrace=1:halt_on_error=1"
     out = subprocess.run([exe], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=600)
