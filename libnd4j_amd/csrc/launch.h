@@ -175,6 +175,9 @@ template <typename T> bool softmaxFitsRegisters(const T *x, const T *z, const So
 // first look count as missing.  Default 5000.
 void setCooperativeWaitLimit(int tries);
 template <typename T> bool launchSoftmaxCooperative(hipStream_t stream, int opNum, const T *x, T *z, const SoftmaxPlan &plan, Workspace ws);
+// The same exchange for an f-order matrix (rows adjacent in memory) with more columns than one block's slice of a group of
+// rows: the blocks that share a group's columns cooperate.  True when the call was taken.
+template <typename T> bool launchSoftmaxColCooperative(hipStream_t stream, int opNum, const T *x, T *z, const SoftmaxPlan &plan, Workspace ws);
 template <typename T>
 bool launchSoftmaxStats(hipStream_t stream, const T *x, T *maxima, typename Compute<T>::type *sums, const TadPlan &plan, Workspace ws);
 template <typename T>

@@ -523,6 +523,15 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
         // exp(x - max) come from one pass of the reduction kernels instead, which cut long rows into slices, and one
         // elementwise pass finishes: 12 bytes per element.  Measured against the per-row kernels this wins for rows of
         // 16384 elements or more, for shorter rows when they are few, and always for f-order matrices.
+        if (rank >= 1 && pl.xRow == 1 && pl.zRow == 1 && pl.numRows >= 256) {
+            // an f-order matrix with more columns than half a compute unit's registers hold of a group of rows: one
+            // pass, the blocks that share the group's columns exchanging the rows' maxima and sums
+            Scratch coop = scratchFor(s);
+            if (launchSoftmaxColCooperative<T>(s, opNum, x, z, pl, coop.rest)) {
+                checkLaunch("execTransform(softmax)", s);
+                return true;
+            }
+        }
         const bool rowMajor = pl.xEl == 1 && pl.zEl == 1 && (pl.length >= 16384 || (pl.length >= 4096 && pl.numRows <= 512));
         const bool colMajor = pl.xRow == 1 && pl.zRow == 1 && pl.numRows >= 256 && pl.length >= 256;
         if (rank >= 1 && (rowMajor || colMajor) && !softmaxFitsRegisters<T>(x, z, pl)) {

@@ -153,9 +153,10 @@ struct FlatSlots {
     void *block = nullptr;  // kFlatSlotBytes of slots, then kFlatCounterBytes of block counters, then kFlatStateBytes of row states
     unsigned ticket = 0;
 };
-const size_t kFlatSlotBytes = 256u << 10;  // 2048 blocks x 16 accumulator words x 8 bytes
+const size_t kFlatSlotBytes = 2u << 20;      // 2048 blocks x 16 accumulator words x 8 bytes for a whole-array reduction; the
+                                             // rest so that a cooperative softmax over a few thousand rows is one launch
 const size_t kFlatCounterBytes = 16u << 10;  // 65 counters, 128 bytes apart
-const size_t kFlatStateBytes = 64u << 10;    // 16384 per-row state words
+const size_t kFlatStateBytes = 256u << 10;   // 2048 row (or row group) states, 128 bytes apart
 std::map<std::pair<int, hipStream_t>, FlatSlots> gFlatSlots;
 }  // namespace
 

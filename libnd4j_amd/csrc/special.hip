@@ -639,6 +639,253 @@ template <typename T> bool launchSoftmaxCooperative(hipStream_t s, int opNum, co
 
 template <typename T> static bool aligned16(const T *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// ---- rows adjacent in memory (f-order) whose columns are shared out over cooperating blocks ---------------------------
+// softmaxColRegKernel keeps 8 * Pack::N whole rows in the registers of a 1024-thread block: a 128-byte piece of every
+// column, and no row longer than 2048 floats.  Here the columns of a group of rows are cut into slices of
+// (block / RL) * PACKS; a 512-thread block keeps one slice of RL * Pack::N rows, two blocks to a compute unit.  With
+// RL = 16 a block asks for 256 contiguous bytes of each of its columns, which the memory serves better than 128, and
+// rows may be as long as the threads of a block can collect pairs for.  The blocks of a group exchange the rows' maxima
+// and sums the way the blocks of a long row do (softmaxRowCoopKernel): pairs in ticket-tagged slots, bounded waits, the
+// group's fate decided once by a compare-and-swap on its state word, a repair kernel behind the launch.
+//
+// Measured on 32768 x 2048 floats (the one-block kernel: 125 us): 8 row lanes and 2 slices 132 us, 16 and 4 117 us,
+// 32 and 8 138 us, 16 and 8 with 256-thread blocks 137 us - wider pieces help, more slices to exchange cost more than
+// they help.  Letting every lane start its exponentials from the maximum of its own columns, before the block has
+// agreed on the rows' maxima, gained nothing (122 us), nor did late starts for the first blocks (151 us); handing
+// neighbouring groups to blocks that do not run at the same time cost a third (152 us): what the memory likes here is
+// that the blocks running together sweep the same columns of adjacent rows.
+static constexpr int kCCCollect = 1;  // pairs each thread of a block collects
+template <typename T, int MODE, int PACKS, int RL, int kCCBlock>
+__global__ void __launch_bounds__(kCCBlock) __attribute__((amdgpu_waves_per_eu(4)))  // two blocks to a compute unit: 128 registers a lane
+softmaxColCoopKernel(const T *x, T *z, Long group0, Long numRows, Long length, Long xEl, Long zEl,
+                                                                 int slices, unsigned long long *slots, unsigned *groupState, unsigned ticket,
+                                                                 int waitTries) {
+    typedef typename Compute<T>::type C;
+    constexpr int N = Pack<T>::N, WAVES = kCCBlock / kWave, R = RL * N;  // RL row lanes, R rows to a group
+    constexpr int kCCCols = kCCBlock / RL;
+    constexpr int W = sizeof(CoopPair<C>) / 4;
+    __shared__ C smax[WAVES][RL][N], ssum[WAVES][RL][N];
+    __shared__ C allM[kCCBlock * kCCCollect], allS[kCCBlock * kCCCollect];  // the pairs of all slices: slice i, row r at [i * R + r]
+    __shared__ unsigned decision;
+    __shared__ int allThere;
+    const int rl = threadIdx.x % RL, cg = threadIdx.x / RL;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const Long local = (Long)blockIdx.x / slices;  // group within this launch
+    const int sl = (int)((Long)blockIdx.x - local * slices);
+    const Long row0 = ((group0 + local) * RL + rl) * N;  // numRows is a multiple of N: a vector is all live or all dead
+    const bool live = row0 < numRows;
+    // this lane's columns are colFirst + j * kCCCols for j < mine (none when its rows are beyond the matrix)
+    const int colFirst = sl * PACKS * kCCCols + cg;
+    int mine = live && colFirst < length ? (int)((length - colFirst + kCCCols - 1) / kCCCols) : 0;
+    if (mine > PACKS) mine = PACKS;
+    Pack<T> cache[PACKS];
+    {
+        const T *px = x + row0 + (Long)colFirst * xEl;
+#pragma unroll
+        for (int j = 0; j < PACKS; j++)
+            if (j < mine) cache[j] = loadPack(reinterpret_cast<const Pack<T> *>(px + (Long)j * kCCCols * xEl));
+    }
+    C mx[N], sum[N];
+#pragma unroll
+    for (int e = 0; e < N; e++) mx[e] = (C)-3.4028235e38;
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (j < mine) {
+#pragma unroll
+            for (int e = 0; e < N; e++) mx[e] = m::max_(mx[e], toCompute(cache[j].v[e]));
+        }
+#pragma unroll
+    for (int d = RL; d < kWave; d <<= 1) {
+#pragma unroll
+        for (int e = 0; e < N; e++) mx[e] = m::max_(mx[e], laneXor(mx[e], d));
+    }
+    if (lane < RL) {
+#pragma unroll
+        for (int e = 0; e < N; e++) smax[wave][lane][e] = mx[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < WAVES; w++) {
+#pragma unroll
+        for (int e = 0; e < N; e++) mx[e] = m::max_(mx[e], smax[w][rl][e]);
+    }
+#pragma unroll
+    for (int e = 0; e < N; e++) sum[e] = (C)0;
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (j < mine) {
+#pragma unroll
+            for (int e = 0; e < N; e++) {
+                const C d = toCompute(cache[j].v[e]) - mx[e], ex = m::expSoft_(d);
+                sum[e] += ex;
+                cache[j].v[e] = fromCompute<T>(softmaxKeep<MODE, C>(ex, d));
+            }
+        }
+#pragma unroll
+    for (int d = RL; d < kWave; d <<= 1) {
+#pragma unroll
+        for (int e = 0; e < N; e++) sum[e] += laneXor(sum[e], d);
+    }
+    if (lane < RL) {
+#pragma unroll
+        for (int e = 0; e < N; e++) ssum[wave][lane][e] = sum[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < N; e++) sum[e] = ssum[0][rl][e];
+#pragma unroll
+    for (int w = 1; w < WAVES; w++) {
+#pragma unroll
+        for (int e = 0; e < N; e++) sum[e] += ssum[w][rl][e];
+    }
+    // the slice's pairs, one per row, go out from the first eight lanes; thread t then collects pair t of the group
+    unsigned long long *group = slots + (size_t)local * slices * R * W;
+    if (threadIdx.x < RL) {
+#pragma unroll
+        for (int e = 0; e < N; e++) {
+            CoopPair<C> mine;
+            mine.m = mx[e];
+            mine.s = sum[e];
+            publishSlots(group + ((size_t)sl * R + rl * N + e) * W, mine, ticket);
+        }
+    }
+    if (threadIdx.x == 0) allThere = 1;
+    __syncthreads();
+    // thread t collects pair t (t + the block size, .. when kCCCollect is more than one) of the group's slices * R
+    CoopPair<C> theirs[kCCCollect];
+    bool have[kCCCollect];
+    const int pairs = slices * R;
+#pragma unroll
+    for (int k = 0; k < kCCCollect; k++) {
+        theirs[k].m = (C)-3.4028235e38;
+        theirs[k].s = (C)0;
+        have[k] = true;
+        const int at = threadIdx.x + k * kCCBlock;
+        if (at < pairs) {
+            have[k] = tryAwaitPair<C>(group + (size_t)at * W, ticket, waitTries, theirs[k]);
+            if (!have[k]) allThere = 0;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned want = (ticket << 2) | (allThere ? kCoopCommit : kCoopAbort);
+        unsigned seen = __hip_atomic_load(groupState + local * kCoopStateStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        while ((seen >> 2) != ticket) {
+            if (__hip_atomic_compare_exchange_strong(groupState + local * kCoopStateStride, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+                seen = want;
+                break;
+            }
+        }
+        decision = seen & 3u;
+    }
+    __syncthreads();
+    if (decision != kCoopCommit) return;  // aborted: the repair kernel computes this group, which nobody has written
+#pragma unroll
+    for (int k = 0; k < kCCCollect; k++) {
+        const int at = threadIdx.x + k * kCCBlock;
+        if (!have[k]) tryAwaitPair<C>(group + (size_t)at * W, ticket, kCoopLateTries, theirs[k]);
+        allM[at] = theirs[k].m;
+        allS[at] = theirs[k].s;
+    }
+    __syncthreads();
+    C scale[N], logSum[N];
+#pragma unroll
+    for (int e = 0; e < N; e++) {
+        const int r = rl * N + e;
+        C rowMax = allM[r];
+        for (int i = 1; i < slices; i++) rowMax = m::max_(rowMax, allM[i * R + r]);
+        C rowSum = (C)0;
+        for (int i = 0; i < slices; i++) rowSum += allS[i * R + r] * m::expSoft_(allM[i * R + r] - rowMax);
+        // this slice's exp(x - mx) -> exp(x - rowMax) / rowSum; for the logarithm (x - mx) + (mx - rowMax) - log(rowSum)
+        const C shift = mx[e] - rowMax;
+        scale[e] = m::expSoft_(shift) / rowSum;
+        logSum[e] = rowLog<MODE, C>(rowSum) - shift;
+    }
+    // (opaque to the optimiser, which would otherwise work out the sixteen addresses early and hold them in registers
+    // that the row data needs)
+    int colAgain = colFirst;
+    asm volatile("" : "+v"(colAgain));
+    T *pz = z + row0 + (Long)colAgain * zEl;
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (j < mine) storePack(reinterpret_cast<Pack<T> *>(pz + (Long)j * kCCCols * zEl), softmaxPackFromKept<T, MODE, true, C>(cache[j], scale, logSum));
+}
+
+// Groups of rows that softmaxColCoopKernel aborted: a block per such group, a lane per row and some columns, three passes.
+template <typename T, int MODE, int RL>
+__global__ void __launch_bounds__(kBlock) softmaxColRepairKernel(const T *x, T *z, Long group0, Long groupsHere, Long numRows, Long length,
+                                                                 Long xEl, Long zEl, const unsigned *groupState, unsigned ticket) {
+    typedef typename Compute<T>::type C;
+    constexpr int R = RL * Pack<T>::N, CL = kBlock / R;
+    __shared__ C part[CL][R];
+    const int r = threadIdx.x % R, cl = threadIdx.x / R;
+    for (Long local = blockIdx.x; local < groupsHere; local += gridDim.x) {
+        const unsigned st = __hip_atomic_load(groupState + local * kCoopStateStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (st == ((ticket << 2) | kCoopCommit)) continue;  // (a block-uniform decision)
+        const Long row = (group0 + local) * R + r;
+        const bool live = row < numRows;
+        C mx = (C)-3.4028235e38;
+        if (live) for (Long c = cl; c < length; c += CL) mx = m::max_(mx, toCompute(x[row + c * xEl]));
+        part[cl][r] = mx;
+        __syncthreads();
+        for (int k = 0; k < CL; k++) mx = m::max_(mx, part[k][r]);
+        __syncthreads();
+        C sum = (C)0;
+        if (live) for (Long c = cl; c < length; c += CL) sum += m::expSoft_(toCompute(x[row + c * xEl]) - mx);
+        part[cl][r] = sum;
+        __syncthreads();  // (in place: every lane has read its share of the rows in both passes before any writes)
+        sum = (C)0;
+        for (int k = 0; k < CL; k++) sum += part[k][r];
+        const C logSum = rowLog<MODE, C>(sum), inv = (C)1 / sum;
+        if (live) for (Long c = cl; c < length; c += CL) z[row + c * zEl] = fromCompute<T>(softmaxAt<MODE, C>(toCompute(x[row + c * xEl]) - mx, inv, logSum));
+        __syncthreads();
+    }
+}
+
+// true when the call was taken: an f-order matrix whose column pitch keeps the row vectors aligned, with more columns than
+// one block's slice and no more than the threads of a block can collect pairs for
+template <typename T, int MODE, int RL, int kCCBlock> static bool runColCooperative(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl, Workspace ws) {
+    typedef typename Compute<T>::type C;
+    constexpr int N = Pack<T>::N, R = RL * N, kCCCols = kCCBlock / RL;
+    // vectors a lane keeps: a half vector unpacks to eight float maxima and sums (and eight shifts for the logarithm), so
+    // fewer of them fit beside
+    constexpr int PACKS = sizeof(T) == 2 ? (MODE == 2 ? 4 : 8) : 16;
+    constexpr int W = sizeof(CoopPair<C>) / 4;
+    const Long perSlice = (Long)PACKS * kCCCols;
+    const Long slices = (pl.length + perSlice - 1) / perSlice;
+    if (slices < 2 || slices * R > kCCBlock * kCCCollect) return false;
+    const Long groups = (pl.numRows + R - 1) / R;
+    Long groupsPer = (Long)(ws.slotBytes / sizeof(unsigned long long)) / (slices * R * W);
+    if (groupsPer > (Long)ws.rowStateCount / kCoopStateStride) groupsPer = (Long)ws.rowStateCount / kCoopStateStride;
+    if (groupsPer * slices > (Long)kMaxGrid) groupsPer = (Long)kMaxGrid / slices;
+    if (groupsPer < 1) return false;
+    for (Long group0 = 0; group0 < groups; group0 += groupsPer) {
+        const Long groupsHere = groups - group0 < groupsPer ? groups - group0 : groupsPer;
+        const unsigned ticket = ws.nextSlotTicket() & 0x3fffffffu;
+        const dim3 grid((unsigned)(groupsHere * slices));
+        const dim3 repair((unsigned)(groupsHere < 1024 ? groupsHere : 1024));
+        ND4J_LAUNCH((softmaxColCoopKernel<T, MODE, PACKS, RL, kCCBlock>), grid, dim3(kCCBlock), 0, s, x, z, group0, pl.numRows, pl.length, pl.xEl,
+                    pl.zEl, (int)slices, ws.slots, ws.rowStates, ticket, gCoopWaitTries.load());
+        ND4J_LAUNCH((softmaxColRepairKernel<T, MODE, RL>), repair, dim3(kBlock), 0, s, x, z, group0, groupsHere, pl.numRows, pl.length,
+                    pl.xEl, pl.zEl, ws.rowStates, ticket);
+    }
+    return true;
+}
+template <typename T> bool launchSoftmaxColCooperative(hipStream_t s, int opNum, const T *x, T *z, const SoftmaxPlan &pl, Workspace ws) {
+    constexpr int N = Pack<T>::N;
+    if (opNum < 38 || opNum > 40) return false;
+    if (pl.xRow != 1 || pl.zRow != 1 || pl.numRows < 256 || pl.numRows % N != 0 || pl.xEl % N != 0 || pl.zEl % N != 0) return false;
+    if (!aligned16(x) || !aligned16(z)) return false;
+    if (ws.slots == nullptr || ws.rowStates == nullptr || ws.slotTicketSource == nullptr) return false;
+    // Sixteen row lanes (256 bytes of each column to a block, half as many columns) where the row count and the pairs to
+    // collect allow it, else eight (a 128-byte line)
+    constexpr int kWideLanes = sizeof(T) == 2 ? 8 : 16;
+    constexpr int kWideBlock = 512;  // (64 rows of halves to a group are the most a repair block seats)
+    if (opNum == 38) return runColCooperative<T, 0, kWideLanes, kWideBlock>(s, x, z, pl, ws) || runColCooperative<T, 0, 8, 512>(s, x, z, pl, ws);
+    if (opNum == 39) return runColCooperative<T, 1, kWideLanes, kWideBlock>(s, x, z, pl, ws) || runColCooperative<T, 1, 8, 512>(s, x, z, pl, ws);
+    return runColCooperative<T, 2, kWideLanes, kWideBlock>(s, x, z, pl, ws) || runColCooperative<T, 2, 8, 512>(s, x, z, pl, ws);
+}
+
 template <typename T, int MODE, int GROUP, int PACKS, int BLOCK = kBlock> void runRowReg(hipStream_t s, const T *x, T *z, const SoftmaxPlan &pl) {
     int grid = gridFor(pl.numRows, BLOCK / GROUP, kMaxGrid / (BLOCK / kBlock));
     constexpr int N = Pack<T>::N;
@@ -1047,6 +1294,7 @@ template <typename T> void launchIsMaxTadFill(hipStream_t s, T *z, const T *inde
 #define INST(T)                                                                                           \
     template bool launchSoftmax<T>(hipStream_t, int, const T *, T *, const SoftmaxPlan &);                \
     template bool launchSoftmaxCooperative<T>(hipStream_t, int, const T *, T *, const SoftmaxPlan &, Workspace);  \
+    template bool launchSoftmaxColCooperative<T>(hipStream_t, int, const T *, T *, const SoftmaxPlan &, Workspace);  \
     template bool softmaxFitsRegisters<T>(const T *, const T *, const SoftmaxPlan &);                     \
     template bool launchSoftmaxFinish<T>(hipStream_t, int, const T *, T *, const T *, const Compute<T>::type *, const SoftmaxPlan &); \
     template void launchIsMaxFill<T>(hipStream_t, T *, const T *, const FlatPlan &);                      \

@@ -782,6 +782,43 @@ def test_softmax_of_long_rows_cooperating_blocks(gpu, cpu):
         gpu.ops.amd_setCooperativeWaitLimit(5000)
 
 
+def test_softmax_of_f_order_matrices_cooperating_blocks(gpu, cpu):
+    # f-order matrices with more columns than one block keeps of a group of rows: the blocks that share a group's columns
+    # exchange the rows' maxima and sums.  Against float64, out of place and in place, the three ops and types, ragged
+    # last groups and last slices; then with no patience, so that the repair kernel does what was not there at once.
+    rs = np.random.RandomState(41)
+
+    def run(limit):
+        gpu.ops.amd_setCooperativeWaitLimit(limit)
+        for shape, dt in (([512, 2048], np.float32), ([260, 1500], np.float32), ([1024, 5001], np.float32),
+                          ([512, 1100], np.float16), ([264, 3000], np.float64), ([4100, 1025], np.float32)):
+            info = harness.shape_info(shape, "f")
+            a = rs.uniform(-6, 6, shape).astype(dt)
+            x = np.ascontiguousarray(a.flatten(order="F"))
+            rows = a.astype(np.float64)
+            truth = np.exp(rows - rows.max(axis=1, keepdims=True))
+            truth /= truth.sum(axis=1, keepdims=True)
+            rtol = {np.float32: 2e-5, np.float16: 1e-2, np.float64: 1e-12}[dt]
+            atol = {np.float32: 1e-7, np.float16: 1e-4, np.float64: 1e-300}[dt]
+            for op, f in ((38, lambda v: v), (39, lambda v: v * (1 - v)), (40, np.log)):
+                got = gpu.transform(op, x, info, info).astype(np.float64).reshape(shape, order="F")
+                assert np.all(np.abs(got - f(truth)) <= rtol * np.abs(f(truth)) + atol), (shape, dt, op, limit)
+                inplace = gpu.transform_inplace(op, x, info).astype(np.float64).reshape(shape, order="F")
+                if limit > 0:
+                    assert np.array_equal(inplace, got), (shape, dt, op, limit, "in place")
+                else:
+                    assert np.all(np.abs(inplace - f(truth)) <= rtol * np.abs(f(truth)) + atol), (shape, dt, op, limit, "in place")
+            if dt == np.float32 and shape[0] * shape[1] <= 1 << 20:
+                c = cpu.transform(38, x, info, info)
+                assert np.all(np.abs(gpu.transform(38, x, info, info).astype(np.float64) - c) <= 1e-5 * np.abs(c) + 1e-7)
+
+    try:
+        run(5000)
+        run(0)
+    finally:
+        gpu.ops.amd_setCooperativeWaitLimit(5000)
+
+
 def test_half_families(gpu, cpu):
     rs = np.random.RandomState(28)
     h = np.float16
