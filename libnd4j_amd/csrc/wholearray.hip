@@ -341,33 +341,62 @@ template <typename T> void launchIm2col(hipStream_t s, const T *x, T *z, const T
 // z[b, c, h, w] = sum of the column entries that im2col would have read from (h, w), added one after the other in the
 // order (kr, kc) the reference's scatter loop reaches them (for one (kr, kc) at most one output position maps to a
 // pixel).  extra = [sH, sW, pH, pW, iH, iW, dH, dW].  ACCUMULATE: start from what z holds instead of from zero.
+// The output position that reads a pixel through kernel cell (kr, kc) is (pixel + padding - cell * dilation) / stride when
+// that divides.  The strides sit in device memory, so the compiler sees divisions by unknowns, a dozen per pixel, which
+// cost more than the memory traffic: strides that are powers of two (1 included) go by shifts instead - the kernel picks
+// its loop once, the same for every lane.
+// The cells of the kernel window are taken kCellBatch at a time: first the loads of a batch, all of them in flight
+// together, then the additions in the reference's order.  (One load per trip of a loop whose bounds the compiler does not
+// know waits for each value before it asks for the next: a pixel then costs nine memory latencies in a row.)
+// Offsets are 32-bit: the host has checked that both arrays span fewer than 2^31 elements, and 64-bit products of a
+// lane's index and a stride are what this kernel would otherwise spend its time on.
+static constexpr int kCellBatch = 16;
+template <typename T, bool SHIFTS>
+__device__ __forceinline__ typename Compute<T>::type col2imPixel(typename Compute<T>::type acc, const T *col, const ConvGeometry &g, int h, int w,
+                                                                 int sH, int sW, int pH, int pW, int dH, int dW, int shH, int shW) {
+    typedef typename Compute<T>::type C;
+    const int cells = g.kH * g.kW;
+    const int cs2 = (int)g.colS[2], cs3 = (int)g.colS[3], cs4 = (int)g.colS[4], cs5 = (int)g.colS[5];
+    int kr = 0, kc = 0;  // the cell's row and column in the window (the same for every lane)
+    for (int cell0 = 0; cell0 < cells; cell0 += kCellBatch) {
+        C v[kCellBatch];
+        bool ok[kCellBatch];
+#pragma unroll
+        for (int u = 0; u < kCellBatch; u++) {
+            ok[u] = false;
+            v[u] = (C)0;
+            if (cell0 + u < cells) {  // (a branch of the whole wave)
+                const int hh = h + pH - kr * dH, ww = w + pW - kc * dW;
+                const int orow = SHIFTS ? hh >> shH : (hh >= 0 ? hh / sH : 0), ocol = SHIFTS ? ww >> shW : (ww >= 0 ? ww / sW : 0);
+                ok[u] = hh >= 0 && ww >= 0 && orow * sH == hh && ocol * sW == ww && orow < g.oH && ocol < g.oW;
+                if (ok[u]) v[u] = toCompute(col[kr * cs2 + kc * cs3 + orow * cs4 + ocol * cs5]);
+                if (++kc == g.kW) { kc = 0; kr++; }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kCellBatch; u++)
+            if (ok[u]) acc = stored<T>(acc + v[u]);
+    }
+    return acc;
+}
 template <typename T, bool ACCUMULATE>
 __global__ void __launch_bounds__(kBlock) col2imKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned total) {
     typedef typename Compute<T>::type C;
     const int sH = paramInt(extra, 0), sW = paramInt(extra, 1), pH = paramInt(extra, 2), pW = paramInt(extra, 3);
     const int iH = paramInt(extra, 4), iW = paramInt(extra, 5), dH = paramInt(extra, 6), dW = paramInt(extra, 7);
+    const bool shifts = sH > 0 && sW > 0 && (sH & (sH - 1)) == 0 && (sW & (sW - 1)) == 0;
+    const int shH = shifts ? __builtin_ctz((unsigned)sH) : 0, shW = shifts ? __builtin_ctz((unsigned)sW) : 0;
     for (unsigned i = blockIdx.x * kBlock + threadIdx.x; i < total; i += gridDim.x * kBlock) {
         unsigned t = i, w, h, c;
         t = g.dIW.divmod(t, w);
         t = g.dIH.divmod(t, h);
         const unsigned b = g.dIC.divmod(t, c);
-        T *out = z + (b * g.imS[0] + c * g.imS[1] + h * g.imS[2] + w * g.imS[3]);
+        T *out = z + (int)(b * (unsigned)g.imS[0] + c * (unsigned)g.imS[1] + h * (unsigned)g.imS[2] + w * (unsigned)g.imS[3]);
         C acc = ACCUMULATE ? toCompute(*out) : (C)0;
         if ((int)h < iH && (int)w < iW) {
-            const T *col = x + (b * g.colS[0] + c * g.colS[1]);
-            for (int kr = 0; kr < g.kH; kr++) {
-                const int hh = (int)h + pH - kr * dH;
-                if (hh < 0) break;
-                const int orow = hh / sH;
-                if (orow * sH != hh || orow >= g.oH) continue;
-                for (int kc = 0; kc < g.kW; kc++) {
-                    const int ww = (int)w + pW - kc * dW;
-                    if (ww < 0) break;
-                    const int ocol = ww / sW;
-                    if (ocol * sW != ww || ocol >= g.oW) continue;
-                    acc = stored<T>(acc + toCompute(col[kr * g.colS[2] + kc * g.colS[3] + orow * g.colS[4] + ocol * g.colS[5]]));
-                }
-            }
+            const T *col = x + (int)(b * (unsigned)g.colS[0] + c * (unsigned)g.colS[1]);
+            if (shifts) acc = col2imPixel<T, true>(acc, col, g, (int)h, (int)w, sH, sW, pH, pW, dH, dW, shH, shW);
+            else acc = col2imPixel<T, false>(acc, col, g, (int)h, (int)w, sH, sW, pH, pW, dH, dW, shH, shW);
         }
         *out = fromCompute<T>(acc);
     }
@@ -407,10 +436,10 @@ template <typename T> void launchCol2im(hipStream_t s, const T *x, T *z, const T
 template <typename T>
 __global__ void __launch_bounds__(kBlock) pooling2dKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned total) {
     typedef typename Compute<T>::type C;
-    lm::loadTables();  // the p-norm's powf
     const int kH = paramInt(extra, 0), kW = paramInt(extra, 1), sH = paramInt(extra, 2), sW = paramInt(extra, 3);
     const int pH = paramInt(extra, 4), pW = paramInt(extra, 5), dH = paramInt(extra, 6), dW = paramInt(extra, 7);
     const int mode = paramInt(extra, 9);
+    if (mode == 2) lm::loadTables();  // the p-norm's powf (the same decision in every thread of the grid)
     const C p0 = toCompute(extra[10]);
     const int kHEff = kH + (kH - 1) * (dH - 1), kWEff = kW + (kW - 1) * (dW - 1);
     for (unsigned i = blockIdx.x * kBlock + threadIdx.x; i < total; i += gridDim.x * kBlock) {
@@ -419,23 +448,32 @@ __global__ void __launch_bounds__(kBlock) pooling2dKernel(const T *x, T *z, cons
         t = g.dOH.divmod(t, yy);
         const unsigned b = g.dIC.divmod(t, c);
         int hs = (int)yy * sH - pH, ws = (int)xx * sW - pW, he = hs + kHEff, we = ws + kWEff;
-        if (hs < 0) hs += ((-hs + dH - 1) / dH) * dH;
-        if (ws < 0) ws += ((-ws + dW - 1) / dW) * dW;
-        if (he > g.iH) he -= ((he - g.iH + dH - 1) / dH) * dH;
-        if (we > g.iW) we -= ((we - g.iW + dW - 1) / dW) * dW;
-        const T *in = x + (b * g.imS[0] + c * g.imS[1]);
+        // (without dilation, the usual case and the same for every lane, the clipping needs no division)
+        if (dH == 1) { hs = hs < 0 ? 0 : hs; he = he > g.iH ? g.iH : he; }
+        else {
+            if (hs < 0) hs += ((-hs + dH - 1) / dH) * dH;
+            if (he > g.iH) he -= ((he - g.iH + dH - 1) / dH) * dH;
+        }
+        if (dW == 1) { ws = ws < 0 ? 0 : ws; we = we > g.iW ? g.iW : we; }
+        else {
+            if (ws < 0) ws += ((-ws + dW - 1) / dW) * dW;
+            if (we > g.iW) we -= ((we - g.iW + dW - 1) / dW) * dW;
+        }
+        const T *in = x + (int)(b * (unsigned)g.imS[0] + c * (unsigned)g.imS[1]);  // (offsets fit 32 bits: the host has checked the spans)
         C acc = mode == 0 ? (C)-1e37 : (C)0;
+        const int is2 = (int)g.imS[2], is3 = (int)g.imS[3];
         for (int ky = hs; ky < he; ky += dH)
             for (int kx = ws; kx < we; kx += dW) {
-                const C v = toCompute(in[ky * g.imS[2] + kx * g.imS[3]]);
+                const C v = toCompute(in[ky * is2 + kx * is3]);
                 if (mode == 0) { if (v > acc) acc = v; }
                 else if (mode == 1) acc = stored<T>(acc + v);
                 else if (mode == 2) acc = stored<T>(acc + stored<T>(m::pow_(m::abs_(v), p0)));
             }
         if (mode == 1) {
             // ceil((he - hs) / dH) * ceil((we - ws) / dW), also where clipping has turned a window inside out
-            const int rowsIn = he >= hs ? (he - hs + dH - 1) / dH : -((hs - he) / dH);
-            const int colsIn = we >= ws ? (we - ws + dW - 1) / dW : -((ws - we) / dW);
+            int rowsIn = he - hs, colsIn = we - ws;
+            if (dH != 1) rowsIn = he >= hs ? (he - hs + dH - 1) / dH : -((hs - he) / dH);
+            if (dW != 1) colsIn = we >= ws ? (we - ws + dW - 1) / dW : -((ws - we) / dW);
             int div = 0;
             if ((int)p0 == 0) div = rowsIn * colsIn;
             else if ((int)p0 == 1) div = kH * kW;
@@ -443,7 +481,7 @@ __global__ void __launch_bounds__(kBlock) pooling2dKernel(const T *x, T *z, cons
         } else if (mode == 2) {
             acc = m::pow_(acc, stored<T>((C)1 / p0));
         }
-        z[b * g.colS[0] + c * g.colS[1] + yy * g.colS[2] + xx * g.colS[3]] = fromCompute<T>(acc);
+        z[(int)(b * (unsigned)g.colS[0] + c * (unsigned)g.colS[1] + yy * (unsigned)g.colS[2] + xx * (unsigned)g.colS[3])] = fromCompute<T>(acc);
     }
 }
 
