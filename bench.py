@@ -135,9 +135,10 @@ def family_builders(workloads):
             ("movement", workloads.data_movement), ("whole", workloads.whole_array_transforms)]
 
 
-def valu_per_element(path, case):
+def valu_per_element(path, case, field="VALU/element"):
     """VALU instructions per element of `case` from the committed instruction-counter summary (its line
-    "<case> ... VALU/element <v>"), or None: as measured_traffic, only while the sources are what they were."""
+    "<case> ... VALU/element <v>"; `field` names another figure of that line), or None: as measured_traffic, only while
+    the sources are what they were."""
     if not path or not os.path.exists(path):
         return None
     with open(path) as f:
@@ -146,9 +147,9 @@ def valu_per_element(path, case):
         if line.startswith("sources:") and line.split()[1] != kernel_sources_digest():
             return None
     for line in lines:
-        if line.startswith(case + " ") and "VALU/element" in line:
+        if line.startswith(case + " ") and field in line:
             try:
-                return float(line.split("VALU/element")[1].split()[0])
+                return float(line.split(field)[1].split()[0])
             except (ValueError, IndexError):
                 return None
     return None
@@ -307,10 +308,18 @@ def main():
                 row["bound"] = getattr(c, "bound", "hbm")
                 v = valu_per_element(args.instructions, c.name)
                 if v is not None:
-                    # a wave64 vector instruction holds its 16-lane SIMD for 4 cycles: the time the chip's 1024 SIMDs need
-                    # to issue the call's vector instructions at 2.4 GHz, against the time measured
-                    issue_ms = v * c.elements / 64.0 * 4.0 / (1024 * 2.4e9) * 1e3
+                    # a SIMD retires a wave64 fp32 instruction every 2 cycles at best (157.3 TFLOP/s of vector fp32 = 256 CUs x
+                    # 4 SIMDs x 32 lanes x 2 flops x 2.4 GHz): the time the chip's 1024 SIMDs need for the call's vector
+                    # instructions if each went at that rate (integer multiplies, transcendentals and doubles take longer),
+                    # against the time measured - a lower bound of the arithmetic's share
+                    issue_ms = v * c.elements / 64.0 * 2.0 / (1024 * 2.4e9) * 1e3
                     row["valu"] = {"instructions_per_element": v, "issue_ms": round(issue_ms, 4), "frac": round(issue_ms / ms, 4)}
+                    # the time the vector units were held, by the chip's own count (SQ_ACTIVE_INST_VALU; like the issue
+                    # time it prices every instruction at one slot, so both are lower bounds)
+                    busy = valu_per_element(args.instructions, c.name, "VALU busy time")
+                    if busy is not None:
+                        row["valu"]["busy_ms"] = busy
+                        row["valu"]["busy_frac"] = round(busy / ms, 4)
                 t = measured_traffic(args.traffic, c.name + " ")
                 if t is not None:  # HBM bytes the call moved, by the chip's counters (profiles/): well above `bytes` = re-reads
                     row["traffic"] = t
