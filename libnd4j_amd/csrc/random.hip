@@ -111,6 +111,7 @@ struct RngWalk {
     u64 y, m;
     bool valid;
     __device__ __forceinline__ RngWalk() : lastP(0), q(0), rem(0), y(0), m(0), valid(false) {}
+    __device__ __forceinline__ u64 element(const RngState &st, Long position);
 };
 
 // RandomBuffer::getElement (helper_generator.h:185-220)
@@ -146,6 +147,55 @@ __device__ __forceinline__ u64 rngElement(const RngState &st, Long position) {
     RngWalk w;
     return rngElement(st, position, w);
 }
+__device__ __forceinline__ u64 RngWalk::element(const RngState &st, Long position) { return rngElement(st, position, *this); }
+
+// getElement for a block whose elements lie within one trip round the buffer of each other: the block's first position
+// is divided by the buffer size once (by its first thread, through LDS), after which an element's index is an addition
+// with at most one wrap, its buffer round is the block's or the next, and the multipliers of both rounds' divisors are
+// the block's too.  Needs size < 2^31 and generation + round + 1 < 2^31 (the host checks both).
+struct RngBlockWalk {
+    Long first;   // index of the block's first element in the draw
+    Long q0, r0;  // buffer round and index of position + first
+    u64 mA, mB;   // floor((2^64 - 1) / (generation + q0)) and the same for the next round
+    __device__ __forceinline__ u64 element(const RngState &st, Long i) const {
+        Long r = r0 + (i - first);
+        const bool wrapped = r >= st.size;
+        if (wrapped) r -= st.size;
+        const Long q = q0 + (wrapped ? 1 : 0);
+        u64 x = st.buffer[r];
+        const bool genDiffers = q != 0;
+        if (genDiffers) {
+            const u64 tempGen = (u64)(st.generation + q);
+            __builtin_assume(tempGen != 0 && (tempGen >> 31) == 0);
+            x = safeShiftDev(x, tempGen, wrapped ? mB : mA);
+        }
+        if (st.generation > 1) x = safeShiftDev(x, (u64)st.generation, st.mGeneration);
+        if (st.amplifier != st.seed) x = safeShiftDev(x, (u64)st.amplifier, st.mAmplifier);
+        if (st.amplifier != st.seed || st.generation > 1 || genDiffers) x = next64Dev(seedConvDev(x));
+        return x;
+    }
+};
+// all threads of the block call this together (it holds a barrier)
+__device__ __forceinline__ RngBlockWalk rngBlockWalk(const RngState &st, Long first) {
+    __shared__ unsigned long long shared[4];
+    if (threadIdx.x == 0) {
+        const Long p = st.position + first;
+        Long q = 0;
+        if (p >= st.size) q = ((u64)p >> 32) < (u64)st.size ? (Long)quot32((u64)p, (unsigned)st.size, st.rSize) : (Long)((u64)p / (u64)st.size);
+        shared[0] = (u64)q;
+        shared[1] = (u64)(p - q * st.size);
+        shared[2] = magicFor((u64)(st.generation + q));
+        shared[3] = magicFor((u64)(st.generation + q + 1));
+    }
+    __syncthreads();
+    RngBlockWalk w;
+    w.first = first;
+    w.q0 = (Long)shared[0];
+    w.r0 = (Long)shared[1];
+    w.mA = shared[2];
+    w.mB = shared[3];
+    return w;
+}
 
 // relativeT<T>(index): u64 -> [0, 1] (helper_generator.h:481-486).  (T)MAX_UINT is exactly 2^64.
 template <typename C> __device__ __forceinline__ C toUnit(u64 r);
@@ -157,8 +207,8 @@ template <typename TT> struct RandomCtx {
     RngState st;
     Params<TT> args;
     Long length;
-    __device__ __forceinline__ C unit(Long i, RngWalk &w) const {
-        C u = toUnit<C>(rngElement(st, i, w));
+    template <class Walk> __device__ __forceinline__ C unit(Long i, Walk &w) const {
+        C u = toUnit<C>(w.element(st, i));
         // storage types narrower than float round the draw to the storage type first (481-484)
         if (sizeof(TT) < 4) u = toCompute(fromCompute<TT>(u));
         return u;
@@ -167,16 +217,16 @@ template <typename TT> struct RandomCtx {
         RngWalk w;
         return unit(i, w);
     }
-    __device__ __forceinline__ C unit(Long i, C from, C to, RngWalk &w) const { return from + (unit(i, w) * (to - from)); }
+    template <class Walk> __device__ __forceinline__ C unit(Long i, C from, C to, Walk &w) const { return from + (unit(i, w) * (to - from)); }
     __device__ __forceinline__ C unit(Long i, C from, C to) const { return from + (unit(i) * (to - from)); }
 };
 
 // Plain (non-special) ops.  nOperands: 1 = (z), 2 = (x, z), 3 = (x, y, z).  Overloads an op does not define
 // return the reference's marker values -1 / -2 / -3 (random_ops.h:15-17).
-template <int OP, typename TT>
+template <int OP, typename TT, class Walk>
 __device__ __forceinline__ typename Compute<TT>::type randomOp(const RandomCtx<TT> &c, int nOperands,
                                                                typename Compute<TT>::type x,
-                                                               typename Compute<TT>::type y, Long i, RngWalk &w) {
+                                                               typename Compute<TT>::type y, Long i, Walk &w) {
     typedef typename Compute<TT>::type C;
     const C undefinedValue = nOperands == 1 ? (C)-1 : (nOperands == 2 ? (C)-2 : (C)-3);
     switch (OP) {
@@ -265,16 +315,64 @@ __global__ void __launch_bounds__(kBlock) randomPlainKernel(RandomCtx<TT> c, con
     }
 }
 
+// The same ops for the usual call: operands with element-wise strides, a buffer of fewer than 2^31 words, generations
+// below 2^31.  A block takes `perBlock` consecutive elements (no more than the buffer holds), so its elements' buffer
+// rounds and divisor multipliers are the block's (RngBlockWalk); the operand count and unit strides are compile-time.
+template <typename TT, int OP, int NOPS, bool UNIT>
+__global__ void __launch_bounds__(kBlock) randomLeanKernel(RandomCtx<TT> c, const TT *x, const TT *y, TT *z, Long xEws, Long yEws,
+                                                           Long zEws, Long perBlock) {
+    if (OP == 13) lm::loadTables();  // ExponentialDistribution's pow
+    typedef typename Compute<TT>::type C;
+    const Long first = (Long)blockIdx.x * perBlock;
+    RngBlockWalk w = rngBlockWalk(c.st, first);
+    Long last = first + perBlock;
+    if (last > c.length) last = c.length;
+    for (Long i = first + threadIdx.x; i < last; i += kBlock) {
+        const C xv = NOPS >= 2 ? toCompute(x[UNIT ? i : i * xEws]) : (C)0;
+        const C yv = NOPS >= 3 ? toCompute(y[UNIT ? i : i * yEws]) : (C)0;
+        z[UNIT ? i : i * zEws] = fromCompute<TT>(randomOp<OP, TT>(c, NOPS, xv, yv, i, w));
+    }
+}
+
 // Box-Muller pairs (2k, 2k+1) sharing u0 = draw(2k), u1 = draw(2k+1) (special_random_ops.h:333-396):
 // z[2k] = sqrt(-2 ln u0) cos(2 pi u1) * stddev + mean, z[2k+1] = ... sin(...).  EXP applies exp() on top
 // (LogNormal, 900-969).
-template <typename TT, bool EXP>
-__global__ void __launch_bounds__(kBlock) gaussianKernel(RandomCtx<TT> c, const TT *y, TT *z, int yIsZ, Long yEws, Long zEws) {
-    lm::loadTables();
+template <typename TT, bool EXP, class Walk>
+__device__ __forceinline__ void gaussianPair(const RandomCtx<TT> &c, const TT *y, TT *z, int yIsZ, Long yEws, Long zEws, bool pairStores,
+                                             Long k, Walk &w) {
     typedef typename Compute<TT>::type C;
     const C twoPi = (C)(2.0 * 3.14159265358979323846);
     const C mean = c.args[0];
     const C stddev = c.args[1];
+    const Long e = 2 * k;
+    C u0 = c.unit(e, (C)1e-5f, (C)1, w);
+    C u1 = c.unit(e + 1, (C)1e-5f, (C)1, w);
+    C r = m::sqrt_((C)-2 * m::log_(u0));
+    C ang = twoPi * u1;
+    C z0 = r * m::cos_(ang);
+    C z1 = r * m::sin_(ang);
+    C m0 = yIsZ ? mean : toCompute(y[e * yEws]);
+    C v0 = z0 * stddev + m0;
+    const TT r0 = fromCompute<TT>(EXP ? m::exp_(v0) : v0);
+    if (e + 1 < c.length) {
+        C m1 = yIsZ ? mean : toCompute(y[(e + 1) * yEws]);
+        C v1 = z1 * stddev + m1;
+        const TT r1 = fromCompute<TT>(EXP ? m::exp_(v1) : v1);
+        if (pairStores) {
+            // one store per pair: a wave's store then covers one contiguous stretch instead of every other element
+            struct alignas(2 * sizeof(TT)) Two { TT a, b; } two = {r0, r1};
+            *reinterpret_cast<Two *>(z + e) = two;
+        } else {
+            z[e * zEws] = r0;
+            z[(e + 1) * zEws] = r1;
+        }
+    } else {
+        z[e * zEws] = r0;
+    }
+}
+template <typename TT, bool EXP>
+__global__ void __launch_bounds__(kBlock) gaussianKernel(RandomCtx<TT> c, const TT *y, TT *z, int yIsZ, Long yEws, Long zEws) {
+    lm::loadTables();
     const Long pairs = (c.length + 1) / 2;
     const Long chunk = (Long)kBlock * kRngIter;
     const bool pairStores = zEws == 1 && (reinterpret_cast<uintptr_t>(z) & (2 * sizeof(TT) - 1)) == 0;
@@ -287,32 +385,21 @@ __global__ void __launch_bounds__(kBlock) gaussianKernel(RandomCtx<TT> c, const 
     for (int it = 0; it < kRngIter; it++) {
         const Long k = base + (Long)it * kBlock + threadIdx.x;
         if (k >= pairs) break;
-        const Long e = 2 * k;
-        C u0 = c.unit(e, (C)1e-5f, (C)1, w);
-        C u1 = c.unit(e + 1, (C)1e-5f, (C)1, w);
-        C r = m::sqrt_((C)-2 * m::log_(u0));
-        C ang = twoPi * u1;
-        C z0 = r * m::cos_(ang);
-        C z1 = r * m::sin_(ang);
-        C m0 = yIsZ ? mean : toCompute(y[e * yEws]);
-        C v0 = z0 * stddev + m0;
-        const TT r0 = fromCompute<TT>(EXP ? m::exp_(v0) : v0);
-        if (e + 1 < c.length) {
-            C m1 = yIsZ ? mean : toCompute(y[(e + 1) * yEws]);
-            C v1 = z1 * stddev + m1;
-            const TT r1 = fromCompute<TT>(EXP ? m::exp_(v1) : v1);
-            if (pairStores) {
-                // one store per pair: a wave's store then covers one contiguous stretch instead of every other element
-                struct alignas(2 * sizeof(TT)) Two { TT a, b; } two = {r0, r1};
-                *reinterpret_cast<Two *>(z + e) = two;
-            } else {
-                z[e * zEws] = r0;
-                z[(e + 1) * zEws] = r1;
-            }
-        } else {
-            z[e * zEws] = r0;
-        }
+        gaussianPair<TT, EXP>(c, y, z, yIsZ, yEws, zEws, pairStores, k, w);
     }
+}
+// the usual call (see randomLeanKernel): a block takes `pairsPerBlock` consecutive pairs, twice as many positions
+template <typename TT, bool EXP>
+__global__ void __launch_bounds__(kBlock) gaussianLeanKernel(RandomCtx<TT> c, const TT *y, TT *z, int yIsZ, Long yEws, Long zEws,
+                                                             Long pairsPerBlock) {
+    lm::loadTables();
+    const Long pairs = (c.length + 1) / 2;
+    const bool pairStores = zEws == 1 && (reinterpret_cast<uintptr_t>(z) & (2 * sizeof(TT) - 1)) == 0;
+    const Long first = (Long)blockIdx.x * pairsPerBlock;
+    RngBlockWalk w = rngBlockWalk(c.st, 2 * first);
+    Long last = first + pairsPerBlock;
+    if (last > pairs) last = pairs;
+    for (Long k = first + threadIdx.x; k < last; k += kBlock) gaussianPair<TT, EXP>(c, y, z, yIsZ, yEws, zEws, pairStores, k, w);
 }
 
 // TruncatedNormal (special_random_ops.h:731-790): pairs (e, e + middle), redrawn with the index advanced
@@ -406,10 +493,38 @@ __global__ void __launch_bounds__(kBlock) copyKernel(uint4 *dst, const uint4 *sr
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dtail[threadIdx.x] = stail[threadIdx.x];
 }
 
+// Elements a block of the lean kernels takes (`positions` draws in all), or 0 when the call does not qualify: operands
+// with element-wise strides, a buffer of at least one block's and fewer than 2^31 words, and every generation the
+// draw can reach (the generator's own plus the buffer rounds up to its last position, plus one) below 2^31.
+static Long leanElementsPerBlock(const RngState &st, const RandomPlan &pl, Long positions) {
+    if (!pl.strided || st.size < kBlock || st.size >= (1LL << 31) || st.position < 0 || st.generation < 0) return 0;
+    if (positions < 0 || st.position > (1LL << 62) - positions) return 0;
+    const Long rounds = (st.position + positions) / st.size;
+    if (st.generation > (1LL << 31) - 3 - rounds) return 0;
+    const Long most = 8192;
+    const Long fit = st.size / kBlock * kBlock;
+    return fit < most ? fit : most;
+}
+
 template <typename T> struct RandomPlainBody {
     template <int OP> struct Run {
         static bool run(hipStream_t s, const RandomCtx<T> &c, const T *x, const T *y, T *z, const RandomPlan &pl,
                         int operands) {
+            const Long perBlock = leanElementsPerBlock(c.st, pl, pl.n);
+            if (perBlock > 0 && (pl.n + perBlock - 1) / perBlock <= 0x7fffffffLL) {
+                const dim3 lean((unsigned)((pl.n + perBlock - 1) / perBlock));
+                const bool unit = pl.xEws == 1 && pl.yEws == 1 && pl.zEws == 1;
+#define ND4J_LEAN(NOPS)                                                                                                          \
+    do {                                                                                                                         \
+        if (unit) ND4J_LAUNCH((randomLeanKernel<T, OP, NOPS, true>), lean, dim3(kBlock), 0, s, c, x, y, z, pl.xEws, pl.yEws, pl.zEws, perBlock); \
+        else ND4J_LAUNCH((randomLeanKernel<T, OP, NOPS, false>), lean, dim3(kBlock), 0, s, c, x, y, z, pl.xEws, pl.yEws, pl.zEws, perBlock);     \
+    } while (0)
+                if (operands == 1) ND4J_LEAN(1);
+                else if (operands == 2) ND4J_LEAN(2);
+                else ND4J_LEAN(3);
+#undef ND4J_LEAN
+                return true;
+            }
             int grid = gridFor(pl.n, kBlock * kRngIter, kMaxGrid);
             ND4J_LAUNCH((randomPlainKernel<T, OP>), dim3(grid), dim3(kBlock), 0, s, c, x, y, z, operands,
                                pl.strided ? 1 : 0, pl.xEws, pl.yEws, pl.zEws, pl.xm, pl.ym, pl.zm);
@@ -437,14 +552,20 @@ bool launchRandom(hipStream_t s, int opNum, const RngState &rng, const T *x, con
                                    pl.yEws, pl.zEws, pl.xm, pl.ym, pl.zm, pl.yLength);
                 break;
             }
-            case 6: {
-                int grid = gridFor((pl.n + 1) / 2, kBlock * kRngIter, kMaxGrid);
-                ND4J_LAUNCH((gaussianKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
-                break;
-            }
+            case 6:
             case 10: {
-                int grid = gridFor((pl.n + 1) / 2, kBlock * kRngIter, kMaxGrid);
-                ND4J_LAUNCH((gaussianKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                const Long pairs = (pl.n + 1) / 2;
+                // (an odd length draws one position beyond its last element's, like the reference)
+                const Long perBlock = leanElementsPerBlock(c.st, pl, 2 * pairs) / 2 / kBlock * kBlock;
+                if (perBlock > 0 && (pairs + perBlock - 1) / perBlock <= 0x7fffffffLL) {
+                    const dim3 lean((unsigned)((pairs + perBlock - 1) / perBlock));
+                    if (opNum == 6) ND4J_LAUNCH((gaussianLeanKernel<T, false>), lean, dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws, perBlock);
+                    else ND4J_LAUNCH((gaussianLeanKernel<T, true>), lean, dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws, perBlock);
+                    break;
+                }
+                int grid = gridFor(pairs, kBlock * kRngIter, kMaxGrid);
+                if (opNum == 6) ND4J_LAUNCH((gaussianKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
+                else ND4J_LAUNCH((gaussianKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, c, y, z, yz, pl.yEws, pl.zEws);
                 break;
             }
             case 8: {
