@@ -16,6 +16,7 @@
 
 #include "libm_float.cuh"
 #include "tanh_poly.h"
+#include "log_poly.h"
 
 namespace nd4j_amd {
 namespace m {
@@ -53,6 +54,10 @@ __device__ __forceinline__ float tanhNear_(float v) {
     return __builtin_copysignf(ax >= 1.0f ? tanhAboveOne_(ax) : tanhBelowOneMagnitude(ax), v);
 }
 __device__ __forceinline__ double tanhNear_(double v) { return ::tanh(v); }
+// log for the Log transform itself: log_poly.h, at most 1 ULP from the C library's logf over every float (the bar is 2),
+// some 25 instructions and no lookup table against the replay's 45 and its table in LDS
+__device__ __forceinline__ float logNear_(float v) { return logNear(v); }
+__device__ __forceinline__ double logNear_(double v) { return ::log(v); }
 __device__ __forceinline__ float sin_(float v) {
     if (((lm::asU32(v) >> 20) & 0x7ff) < 0x42f) return lm::sincosCore(v, false);
     return (float)::sin((double)v);

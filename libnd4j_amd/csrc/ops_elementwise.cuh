@@ -61,7 +61,7 @@ ND4J_TRANSFORM(1, Ceiling, return m::ceil_(d1);)
 ND4J_TRANSFORM(2, Cosine, return m::cos_(d1);)
 ND4J_TRANSFORM(3, Exp, return m::exp_(d1);)
 ND4J_TRANSFORM(4, Floor, return m::floor_(d1);)
-ND4J_TRANSFORM(5, Log, return m::log_(d1);)
+ND4J_TRANSFORM(5, Log, return m::logNear_(d1);)
 ND4J_TRANSFORM(6, Neg, return -d1;)
 ND4J_TRANSFORM(7, Pow, return m::pow_(d1, p[0]);)
 ND4J_TRANSFORM(8, Round, return m::round_(d1);)
@@ -180,7 +180,8 @@ ND4J_TRANSFORM(54, RationalTanhDerivative, {
 })
 ND4J_TRANSFORM(55, LogX, return m::log_(d1) / m::log_((C)p[0]);)
 ND4J_TRANSFORM(59, Not, return d1 == p[0] ? (C)1 : (C)0;)
-ND4J_TRANSFORM(61, RectifiedTanh, return m::max_((C)0, m::tanh_(d1));)
+// (the Tanh transform's routine, within 2 ULP of the C library's tanhf: the maximum with 0 keeps that distance)
+ND4J_TRANSFORM(61, RectifiedTanh, return m::max_((C)0, m::tanhNear_(d1));)
 ND4J_TRANSFORM(62, RectifiedTanhDerivative, {
     if (!(d1 > (C)0)) return (C)0;
     C t = m::tanh_(d1);
@@ -258,7 +259,7 @@ static constexpr int kTransformOpCount = 97;
 // kernels skip loading the lookup tables of those routines.  Anything not listed loads them.
 __host__ __device__ constexpr bool transformIsPlain(int op) {
     switch (op) {
-        case 0: case 1: case 2: case 4: case 6: case 8: case 11: case 12: case 14: case 15: case 19: case 20: case 23: case 24:
+        case 0: case 1: case 2: case 4: case 5: case 6: case 8: case 11: case 12: case 14: case 15: case 19: case 20: case 23: case 24:
         case 25: case 26: case 27: case 61: case 62:
         case 31: case 32: case 33: case 34: case 35: case 42: case 49: case 50: case 51: case 52: case 76: case 79:
         case 80: case 81: case 87: case 94: case 96:

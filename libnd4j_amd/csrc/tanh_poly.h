@@ -3,7 +3,7 @@
 //   tanh(x) = x + x t R(t),  t = x^2,  R = a degree-7 fit of (tanh(x) / x - 1) / t over t in [0, 1]
 // (0.01 ULP of tanh).  Over every float of magnitude below 1 the result is at most 1 ULP from the correctly rounded
 // value and at most 2 ULP from the C library's tanhf (glibc 2.35, itself up to 2 ULP off there); the host test
-// tests/test_tanh_host.py runs these lines against the library over a strided sample, or over all of them on request.
+// tests/test_host_math.py runs these lines against the library over a strided sample, or over all of them on request.
 #pragma once
 
 #if defined(__HIPCC__)
