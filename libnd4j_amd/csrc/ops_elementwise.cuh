@@ -78,7 +78,8 @@ ND4J_TRANSFORM(9, SetRange, {
 ND4J_TRANSFORM(10, Sigmoid, return m::sigmoid_(d1);)
 ND4J_TRANSFORM(11, Sign, return (C)((d1 > (C)0) - (d1 < (C)0));)
 ND4J_TRANSFORM(12, Sin, return m::sin_(d1);)
-ND4J_TRANSFORM(13, SoftPlus, return m::log_((C)1 + m::exp_(d1));)
+// (the logarithm of these is the Log transform's routine, at most 1 ULP from logf on the same argument; exp stays the replay)
+ND4J_TRANSFORM(13, SoftPlus, return m::logNear_((C)1 + m::exp_(d1));)
 ND4J_TRANSFORM(14, Sqrt, return m::sqrt_(d1);)
 ND4J_TRANSFORM(15, Tanh, return m::tanhNear_(d1);)
 ND4J_TRANSFORM(16, ACos, return m::acos_(d1);)
@@ -142,10 +143,10 @@ ND4J_TRANSFORM(35, OneMinus, return (C)1 - d1;)
 // routes these opNums to their own routines before it gets here.
 ND4J_TRANSFORM(36, Col2Im, return d1;)
 ND4J_TRANSFORM(37, Im2col, return d1;)
-ND4J_TRANSFORM(38, SoftMax, return m::log_((C)1 + m::exp_(d1));)
-ND4J_TRANSFORM(39, SoftMaxDerivative, return m::log_((C)1 + m::exp_(d1));)
-ND4J_TRANSFORM(40, LogSoftMax, return m::log_((C)1 + m::exp_(d1));)
-ND4J_TRANSFORM(41, IsMax, return m::log_((C)1 + m::exp_(d1));)
+ND4J_TRANSFORM(38, SoftMax, return m::logNear_((C)1 + m::exp_(d1));)
+ND4J_TRANSFORM(39, SoftMaxDerivative, return m::logNear_((C)1 + m::exp_(d1));)
+ND4J_TRANSFORM(40, LogSoftMax, return m::logNear_((C)1 + m::exp_(d1));)
+ND4J_TRANSFORM(41, IsMax, return m::logNear_((C)1 + m::exp_(d1));)
 ND4J_TRANSFORM(48, Histogram, return d1;)
 ND4J_TRANSFORM(70, Reverse, return d1;)
 ND4J_TRANSFORM(71, Pooling2D, return d1;)
@@ -221,7 +222,7 @@ ND4J_TRANSFORM(75, SwishDerivative, {
     return (C)(num / (double)den);
 })
 ND4J_TRANSFORM(76, RSqrt, return (C)1 / m::sqrt_(d1);)
-ND4J_TRANSFORM(77, Log1p, return m::log_((C)1 + d1);)
+ND4J_TRANSFORM(77, Log1p, return m::logNear_((C)1 + d1);)
 ND4J_TRANSFORM(78, Erf, return m::erf_(d1);)
 ND4J_TRANSFORM(79, IsInf, return m::isinf_(d1) ? (C)1 : (C)0;)
 ND4J_TRANSFORM(80, IsNan, return m::isnan_(d1) ? (C)1 : (C)0;)
@@ -232,7 +233,7 @@ ND4J_TRANSFORM(84, ASinh, return m::log_(m::sqrt_(m::pow_(d1, (C)2) + (C)1) + d1
 ND4J_TRANSFORM(85, ASinhDerivative, return (C)1 / m::sqrt_(m::pow_(d1, (C)2) + (C)1);)
 ND4J_TRANSFORM(86, SinhDerivative, return m::cosh_(d1);)
 ND4J_TRANSFORM(87, Rint, return m::rint_(d1);)
-ND4J_TRANSFORM(88, LogSigmoid, return m::log_(m::sigmoid_(d1));)
+ND4J_TRANSFORM(88, LogSigmoid, return m::logNear_(m::sigmoid_(d1));)
 ND4J_TRANSFORM(89, LogSigmoidDerivative, {
     C ex = m::pow_((C)2.718281828459045, d1);
     return (C)1 / (ex + (C)1);
