@@ -200,7 +200,20 @@ __global__ void __launch_bounds__(kBlock) histogramCountKernel(const T *x, Long 
     if (gtid < lead) count(x[gtid]);
     const Long nvec = (n - lead) / N;
     const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x + lead);
-    for (Long v = gtid; v < nvec; v += (Long)gridDim.x * kBlock) {
+    // four vectors in flight per lane: the counting of one batch then overlaps the memory latency of the next lanes'
+    const Long step = (Long)gridDim.x * kBlock;
+    Long v = gtid;
+    for (; v + 3 * step < nvec; v += 4 * step) {
+        Pack<T> a[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) a[u] = loadPack(xv + v + u * step);
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+            for (int k = 0; k < N; k++) count(a[u].v[k]);
+        }
+    }
+    for (; v < nvec; v += step) {
         const Pack<T> a = loadPack(xv + v);
 #pragma unroll
         for (int k = 0; k < N; k++) count(a.v[k]);
@@ -311,6 +324,60 @@ __global__ void __launch_bounds__(kBlock) im2colPlaneKernel(const T *x, T *z, co
     }
 }
 
+// With many (batch, channel) pairs a block takes a whole channel: its kH * kW result planes as one list of vectors (a
+// plane alone is rarely a whole number of rounds of the block: 784 vectors of a 56 x 56 plane leave the fourth round of
+// 256 threads nearly empty), all of them reading the one image plane, which stays in the unit's cache.  Offsets are
+// 32-bit (the host has checked the spans).  dAux: vectors per result row, dAux2: vectors per plane.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) im2colChannelKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned channels) {
+    constexpr int N = Pack<T>::N;
+    const int sH = paramInt(extra, 2), sW = paramInt(extra, 3), pH = paramInt(extra, 4), pW = paramInt(extra, 5);
+    const int dH = paramInt(extra, 6), dW = paramInt(extra, 7);
+    const unsigned vecsPerRow = (unsigned)g.oW / N, vecs = vecsPerRow * (unsigned)g.oH;
+    const unsigned all = vecs * (unsigned)(g.kH * g.kW);
+    const int is2 = (int)g.imS[2], is3 = (int)g.imS[3];
+    for (unsigned ch = blockIdx.x; ch < channels; ch += gridDim.x) {
+        unsigned c;
+        const unsigned b = g.dIC.divmod(ch, c);
+        const T *image = x + (int)(b * (unsigned)g.imS[0] + c * (unsigned)g.imS[1]);
+        Pack<T> *out = reinterpret_cast<Pack<T> *>(z + (Long)ch * all * N);
+        // four vectors per thread and round, all their loads before the first store (the compiler must assume that a store
+        // to z changes the image, so it does not start the next vector's loads by itself: one vector per trip waits out a
+        // memory latency per trip)
+        for (unsigned v0 = threadIdx.x; v0 < all; v0 += 4 * kBlock) {
+            Pack<T> o[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const unsigned v = v0 + u * kBlock;
+                if (v < all) {
+                    unsigned within, kc, vc;
+                    const unsigned cell = g.dAux2.divmod(v, within);
+                    const unsigned kr = g.dKW.divmod(cell, kc);
+                    const unsigned orow = g.dAux.divmod(within, vc);
+                    const int r = (int)kr * dH - pH + (int)orow * sH;
+                    const int q0 = (int)kc * dW - pW + (int)(vc * N) * sW;
+                    const bool rowIn = inRange(r, g.iH);
+                    const T *line = image + r * is2;
+                    if (sW == 1 && is3 == 1 && rowIn && q0 >= 0 && q0 + N <= g.iW) {
+                        // the vector's N image elements lie side by side: one 16-byte load at whatever alignment they have
+                        // (element by element the vector cache serves four requests a vector, and sets the pace)
+                        o[u] = loadPackAnywhere(line + q0);
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < N; k++) {
+                            const int q = q0 + k * sW;
+                            o[u].v[k] = (rowIn && inRange(q, g.iW)) ? line[q * is3] : fromCompute<T>(0);
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (v0 + u * kBlock < all) storePack(out + v0 + u * kBlock, o[u]);
+        }
+    }
+}
+
 template <typename T> void launchIm2col(hipStream_t s, const T *x, T *z, const T *extra, const ConvGeometry &g) {
     const Long total = (Long)g.bS * g.iC * g.kH * g.kW * g.oH * g.oW;
     if (total <= 0) return;
@@ -323,6 +390,11 @@ template <typename T> void launchIm2col(hipStream_t s, const T *x, T *z, const T
         ConvGeometry gv = g;
         gv.dAux = FastDiv((unsigned)(g.oW / N));
         const Long perChannel = (Long)g.kH * g.kW, channels = planes / perChannel;
+        if (channels >= 1024 && plane / N * perChannel < (1LL << 31)) {
+            gv.dAux2 = FastDiv((unsigned)(plane / N));
+            ND4J_LAUNCH(im2colChannelKernel<T>, dim3(gridFor(channels, 1)), dim3(kBlock), 0, s, x, z, extra, gv, (unsigned)channels);
+            return;
+        }
         gv.dAux2 = FastDiv((unsigned)perChannel);
         // workgroups for whole rounds of eight channels; in one launch when that fits, else in plain order
         const Long byDie = (channels + 7) / 8 * 8 * perChannel;
