@@ -158,16 +158,18 @@ struct RngBlockWalk {
     Long q0, r0;  // buffer round and index of position + first
     u64 mA, mB;   // floor((2^64 - 1) / (generation + q0)) and the same for the next round
     __device__ __forceinline__ u64 element(const RngState &st, Long i) const {
-        Long r = r0 + (i - first);
-        const bool wrapped = r >= st.size;
-        if (wrapped) r -= st.size;
-        const Long q = q0 + (wrapped ? 1 : 0);
+        // (32-bit arithmetic: the block's elements span no more than the buffer, which holds fewer than 2^31 words, and the
+        // generations stay below 2^31)
+        const unsigned size = (unsigned)st.size;
+        unsigned r = (unsigned)r0 + (unsigned)(i - first);
+        const bool wrapped = r >= size;
+        if (wrapped) r -= size;
         u64 x = st.buffer[r];
-        const bool genDiffers = q != 0;
+        const bool genDiffers = q0 != 0 || wrapped;
         if (genDiffers) {
-            const u64 tempGen = (u64)(st.generation + q);
-            __builtin_assume(tempGen != 0 && (tempGen >> 31) == 0);
-            x = safeShiftDev(x, tempGen, wrapped ? mB : mA);
+            const unsigned gen = (unsigned)(st.generation + q0) + (wrapped ? 1u : 0u);
+            __builtin_assume(gen != 0 && (gen >> 31) == 0);
+            x = safeShiftDev(x, (u64)gen, wrapped ? mB : mA);
         }
         if (st.generation > 1) x = safeShiftDev(x, (u64)st.generation, st.mGeneration);
         if (st.amplifier != st.seed) x = safeShiftDev(x, (u64)st.amplifier, st.mAmplifier);
@@ -325,9 +327,9 @@ __global__ void __launch_bounds__(kBlock) randomLeanKernel(RandomCtx<TT> c, cons
     typedef typename Compute<TT>::type C;
     const Long first = (Long)blockIdx.x * perBlock;
     RngBlockWalk w = rngBlockWalk(c.st, first);
-    Long last = first + perBlock;
-    if (last > c.length) last = c.length;
-    for (Long i = first + threadIdx.x; i < last; i += kBlock) {
+    const unsigned count = (unsigned)(c.length - first < perBlock ? c.length - first : perBlock);
+    for (unsigned o = threadIdx.x; o < count; o += kBlock) {
+        const Long i = first + o;
         const C xv = NOPS >= 2 ? toCompute(x[UNIT ? i : i * xEws]) : (C)0;
         const C yv = NOPS >= 3 ? toCompute(y[UNIT ? i : i * yEws]) : (C)0;
         z[UNIT ? i : i * zEws] = fromCompute<TT>(randomOp<OP, TT>(c, NOPS, xv, yv, i, w));
