@@ -422,36 +422,58 @@ template <typename T> void launchIm2col(hipStream_t s, const T *x, T *z, const T
 // know waits for each value before it asks for the next: a pixel then costs nine memory latencies in a row.)
 // Offsets are 32-bit: the host has checked that both arrays span fewer than 2^31 elements, and 64-bit products of a
 // lane's index and a stride are what this kernel would otherwise spend its time on.
+// A compute unit has one scalar unit, and with window extents that are only known at run time the bookkeeping of the
+// window (cell counters, their comparisons and branches, all the same for every lane, so all scalar) came to 48 scalar
+// instructions per element and set the pace.  The usual windows (1x1, 2x2, 3x3, 5x5) are therefore compiled in (KH, KW > 0):
+// their cells are constants and the batch is the whole window.
 static constexpr int kCellBatch = 16;
-template <typename T, bool SHIFTS>
+template <typename T, bool SHIFTS, int KH, int KW>
 __device__ __forceinline__ typename Compute<T>::type col2imPixel(typename Compute<T>::type acc, const T *col, const ConvGeometry &g, int h, int w,
                                                                  int sH, int sW, int pH, int pW, int dH, int dW, int shH, int shW) {
     typedef typename Compute<T>::type C;
-    const int cells = g.kH * g.kW;
     const int cs2 = (int)g.colS[2], cs3 = (int)g.colS[3], cs4 = (int)g.colS[4], cs5 = (int)g.colS[5];
-    int kr = 0, kc = 0;  // the cell's row and column in the window (the same for every lane)
-    for (int cell0 = 0; cell0 < cells; cell0 += kCellBatch) {
-        C v[kCellBatch];
-        bool ok[kCellBatch];
+    if constexpr (KH > 0) {
+        constexpr int CELLS = KH * KW;
+        C v[CELLS];
+        bool ok[CELLS];
 #pragma unroll
-        for (int u = 0; u < kCellBatch; u++) {
-            ok[u] = false;
-            v[u] = (C)0;
-            if (cell0 + u < cells) {  // (a branch of the whole wave)
-                const int hh = h + pH - kr * dH, ww = w + pW - kc * dW;
-                const int orow = SHIFTS ? hh >> shH : (hh >= 0 ? hh / sH : 0), ocol = SHIFTS ? ww >> shW : (ww >= 0 ? ww / sW : 0);
-                ok[u] = hh >= 0 && ww >= 0 && orow * sH == hh && ocol * sW == ww && orow < g.oH && ocol < g.oW;
-                if (ok[u]) v[u] = toCompute(col[kr * cs2 + kc * cs3 + orow * cs4 + ocol * cs5]);
-                if (++kc == g.kW) { kc = 0; kr++; }
-            }
+        for (int u = 0; u < CELLS; u++) {
+            const int kr = u / KW, kc = u % KW;
+            const int hh = h + pH - kr * dH, ww = w + pW - kc * dW;
+            const int orow = SHIFTS ? hh >> shH : (hh >= 0 ? hh / sH : 0), ocol = SHIFTS ? ww >> shW : (ww >= 0 ? ww / sW : 0);
+            ok[u] = hh >= 0 && ww >= 0 && orow * sH == hh && ocol * sW == ww && orow < g.oH && ocol < g.oW;
+            v[u] = ok[u] ? toCompute(col[kr * cs2 + kc * cs3 + orow * cs4 + ocol * cs5]) : (C)0;
         }
 #pragma unroll
-        for (int u = 0; u < kCellBatch; u++)
+        for (int u = 0; u < CELLS; u++)
             if (ok[u]) acc = stored<T>(acc + v[u]);
+        return acc;
+    } else {
+        const int cells = g.kH * g.kW;
+        int kr = 0, kc = 0;  // the cell's row and column in the window (the same for every lane)
+        for (int cell0 = 0; cell0 < cells; cell0 += kCellBatch) {
+            C v[kCellBatch];
+            bool ok[kCellBatch];
+#pragma unroll
+            for (int u = 0; u < kCellBatch; u++) {
+                ok[u] = false;
+                v[u] = (C)0;
+                if (cell0 + u < cells) {  // (a branch of the whole wave)
+                    const int hh = h + pH - kr * dH, ww = w + pW - kc * dW;
+                    const int orow = SHIFTS ? hh >> shH : (hh >= 0 ? hh / sH : 0), ocol = SHIFTS ? ww >> shW : (ww >= 0 ? ww / sW : 0);
+                    ok[u] = hh >= 0 && ww >= 0 && orow * sH == hh && ocol * sW == ww && orow < g.oH && ocol < g.oW;
+                    if (ok[u]) v[u] = toCompute(col[kr * cs2 + kc * cs3 + orow * cs4 + ocol * cs5]);
+                    if (++kc == g.kW) { kc = 0; kr++; }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kCellBatch; u++)
+                if (ok[u]) acc = stored<T>(acc + v[u]);
+        }
+        return acc;
     }
-    return acc;
 }
-template <typename T, bool ACCUMULATE>
+template <typename T, bool ACCUMULATE, int KH, int KW>
 __global__ void __launch_bounds__(kBlock) col2imKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned total) {
     typedef typename Compute<T>::type C;
     const int sH = paramInt(extra, 0), sW = paramInt(extra, 1), pH = paramInt(extra, 2), pW = paramInt(extra, 3);
@@ -467,8 +489,8 @@ __global__ void __launch_bounds__(kBlock) col2imKernel(const T *x, T *z, const T
         C acc = ACCUMULATE ? toCompute(*out) : (C)0;
         if ((int)h < iH && (int)w < iW) {
             const T *col = x + (int)(b * (unsigned)g.colS[0] + c * (unsigned)g.colS[1]);
-            if (shifts) acc = col2imPixel<T, true>(acc, col, g, (int)h, (int)w, sH, sW, pH, pW, dH, dW, shH, shW);
-            else acc = col2imPixel<T, false>(acc, col, g, (int)h, (int)w, sH, sW, pH, pW, dH, dW, shH, shW);
+            if (shifts) acc = col2imPixel<T, true, KH, KW>(acc, col, g, (int)h, (int)w, sH, sW, pH, pW, dH, dW, shH, shW);
+            else acc = col2imPixel<T, false, KH, KW>(acc, col, g, (int)h, (int)w, sH, sW, pH, pW, dH, dW, shH, shW);
         }
         *out = fromCompute<T>(acc);
     }
@@ -495,10 +517,19 @@ template <typename T> void launchCol2im(hipStream_t s, const T *x, T *z, const T
         const int tailBytes = (int)(bytes - lead - vectors * 16);
         ND4J_LAUNCH(clearBytesKernel, dim3(gridFor(vectors + 1)), dim3(kBlock), 0, s, reinterpret_cast<U32x4 *>(base + lead), vectors,
                            base + lead + vectors * 16, tailBytes);
-        ND4J_LAUNCH((col2imKernel<T, true>), dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
-    } else {
-        ND4J_LAUNCH((col2imKernel<T, false>), dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
     }
+    const dim3 grid(gridFor(total));
+#define ND4J_COL2IM(KH, KW)                                                                                                   \
+    do {                                                                                                                      \
+        if (clearFirst > 0) ND4J_LAUNCH((col2imKernel<T, true, KH, KW>), grid, dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);  \
+        else ND4J_LAUNCH((col2imKernel<T, false, KH, KW>), grid, dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);                \
+    } while (0)
+    if (g.kH == 3 && g.kW == 3) ND4J_COL2IM(3, 3);
+    else if (g.kH == 1 && g.kW == 1) ND4J_COL2IM(1, 1);
+    else if (g.kH == 2 && g.kW == 2) ND4J_COL2IM(2, 2);
+    else if (g.kH == 5 && g.kW == 5) ND4J_COL2IM(5, 5);
+    else ND4J_COL2IM(0, 0);
+#undef ND4J_COL2IM
 }
 
 // ---- Pooling2D -------------------------------------------------------------------------------------------------
