@@ -536,6 +536,46 @@ template <typename T> void launchCol2im(hipStream_t s, const T *x, T *z, const T
 // extra = [kH, kW, sH, sW, pH, pW, dH, dW, -, mode, p]: mode 0 maximum (from -1e37, the reference's MAX_FLOAT), 1 average
 // (p == 0: over the cells inside the image, p == 1: over kH * kW), 2 p-norm.  One thread per result element; the window
 // is clipped to the image in steps of the dilation, as the reference clips it.
+// The window's cells for the usual 2x2 and 3x3 windows without dilation, compiled in (see col2imPixel: loops whose bounds
+// differ from lane to lane cost a round of exec-mask bookkeeping on the one scalar unit per trip): all loads first, a
+// cell counting when it lies inside the image, which is what the clipped bounds select; then the reference's order.
+template <typename T, int KH, int KW>
+__device__ __forceinline__ typename Compute<T>::type poolCells(typename Compute<T>::type acc, const T *in, int hs0, int ws0, int iH, int iW,
+                                                               int is2, int is3, int mode, typename Compute<T>::type p0) {
+    typedef typename Compute<T>::type C;
+    C v[KH * KW];
+    bool ok[KH * KW];
+    if (KW == 2 && is3 == 1 && ws0 >= 0 && ws0 + 2 <= iW) {
+        // both cells of a window row lie side by side inside the image: one load of two elements (element by element a
+        // wave asks the vector cache for every line twice, and its request rate sets the pace)
+        struct __attribute__((packed, aligned(sizeof(T)))) Two { T a, b; };
+#pragma unroll
+        for (int r = 0; r < KH; r++) {
+            const int ky = hs0 + r;
+            ok[2 * r] = ok[2 * r + 1] = inRange(ky, iH);
+            Two t = {fromCompute<T>(0), fromCompute<T>(0)};
+            if (ok[2 * r]) t = *reinterpret_cast<const Two *>(in + ky * is2 + ws0);
+            v[2 * r] = toCompute(t.a);
+            v[2 * r + 1] = toCompute(t.b);
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < KH * KW; u++) {
+            const int ky = hs0 + u / KW, kx = ws0 + u % KW;
+            ok[u] = inRange(ky, iH) && inRange(kx, iW);
+            v[u] = ok[u] ? toCompute(in[ky * is2 + kx * is3]) : (C)0;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < KH * KW; u++)
+        if (ok[u]) {
+            if (mode == 0) { if (v[u] > acc) acc = v[u]; }
+            else if (mode == 1) acc = stored<T>(acc + v[u]);
+            else if (mode == 2) acc = stored<T>(acc + stored<T>(m::pow_(m::abs_(v[u]), p0)));
+        }
+    return acc;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kBlock) pooling2dKernel(const T *x, T *z, const T *extra, ConvGeometry g, unsigned total) {
     typedef typename Compute<T>::type C;
@@ -545,6 +585,42 @@ __global__ void __launch_bounds__(kBlock) pooling2dKernel(const T *x, T *z, cons
     if (mode == 2) lm::loadTables();  // the p-norm's powf (the same decision in every thread of the grid)
     const C p0 = toCompute(extra[10]);
     const int kHEff = kH + (kH - 1) * (dH - 1), kWEff = kW + (kW - 1) * (dW - 1);
+    constexpr int N = Pack<T>::N, OUT = N / 2;
+    if (OUT >= 1 && mode != 2 && kH == 2 && kW == 2 && sH == 2 && sW == 2 && pH == 0 && pW == 0 && dH == 1 && dW == 1 && g.imS[3] == 1 &&
+        g.colS[3] == 1 && g.oW % OUT == 0 && 2 * g.oW <= g.iW && 2 * g.oH <= g.iH) {
+        // The everyday case, 2 x 2 windows side by side: a thread takes N / 2 neighbouring results, whose 2 x N inputs are
+        // two 16-byte loads (at whatever alignment the rows have), and stores them together.  Same order of operations per
+        // result as below: upper row left, right, lower row left, right.
+        const int is2 = (int)g.imS[2];
+        const C div = ((int)p0 == 0 || (int)p0 == 1) ? (C)4 : (C)0;
+        for (unsigned j = blockIdx.x * kBlock + threadIdx.x; j < total / OUT; j += gridDim.x * kBlock) {
+            unsigned t = j * OUT, xx, yy, c;
+            t = g.dOW.divmod(t, xx);
+            t = g.dOH.divmod(t, yy);
+            const unsigned b = g.dIC.divmod(t, c);
+            const T *in = x + (int)(b * (unsigned)g.imS[0] + c * (unsigned)g.imS[1]) + (int)(2 * yy) * is2 + (int)(2 * xx);
+            const Pack<T> up = loadPackAnywhere(in), low = loadPackAnywhere(in + is2);
+            T *out = z + (int)(b * (unsigned)g.colS[0] + c * (unsigned)g.colS[1] + yy * (unsigned)g.colS[2] + xx);
+#pragma unroll
+            for (int k = 0; k < OUT; k++) {
+                const C v0 = toCompute(up.v[2 * k]), v1 = toCompute(up.v[2 * k + 1]), v2 = toCompute(low.v[2 * k]), v3 = toCompute(low.v[2 * k + 1]);
+                C acc;
+                if (mode == 0) {
+                    acc = (C)-1e37;
+                    if (v0 > acc) acc = v0;
+                    if (v1 > acc) acc = v1;
+                    if (v2 > acc) acc = v2;
+                    if (v3 > acc) acc = v3;
+                } else if (mode == 1) {
+                    acc = stored<T>(stored<T>(stored<T>(stored<T>((C)0 + v0) + v1) + v2) + v3) / div;
+                } else {
+                    acc = (C)0;  // (what the general path leaves for a mode it does not know)
+                }
+                out[k] = fromCompute<T>(acc);
+            }
+        }
+        return;
+    }
     for (unsigned i = blockIdx.x * kBlock + threadIdx.x; i < total; i += gridDim.x * kBlock) {
         unsigned t = i, xx, yy, c;
         t = g.dOW.divmod(t, xx);
@@ -565,6 +641,10 @@ __global__ void __launch_bounds__(kBlock) pooling2dKernel(const T *x, T *z, cons
         const T *in = x + (int)(b * (unsigned)g.imS[0] + c * (unsigned)g.imS[1]);  // (offsets fit 32 bits: the host has checked the spans)
         C acc = mode == 0 ? (C)-1e37 : (C)0;
         const int is2 = (int)g.imS[2], is3 = (int)g.imS[3];
+        const int hs0 = (int)yy * sH - pH, ws0 = (int)xx * sW - pW;
+        if (dH == 1 && dW == 1 && kH == 2 && kW == 2) acc = poolCells<T, 2, 2>(acc, in, hs0, ws0, g.iH, g.iW, is2, is3, mode, p0);
+        else if (dH == 1 && dW == 1 && kH == 3 && kW == 3) acc = poolCells<T, 3, 3>(acc, in, hs0, ws0, g.iH, g.iW, is2, is3, mode, p0);
+        else
         for (int ky = hs; ky < he; ky += dH)
             for (int kx = ws; kx < we; kx += dW) {
                 const C v = toCompute(in[ky * is2 + kx * is3]);

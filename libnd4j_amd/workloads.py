@@ -593,17 +593,20 @@ def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data
 
 # ---- the whole-array transforms: Reverse, Histogram, Im2col, Col2Im, Pooling2D ------------------------------------------
 def whole_array_transforms(dev, n=1 << 26, seed=41, copies=None):
-    """Reverse and Histogram over 2^26 floats; Im2col / Col2Im / Pooling2D on a [32, 64, 56, 56] image (3 x 3 kernel,
-    stride 1, padding 1 for the column forms; 2 x 2 / stride 2 max and average pooling)."""
+    """Reverse and Histogram over 2^26 floats; Im2col / Col2Im on a [32, 64, 56, 56] image (3 x 3 kernel, stride 1,
+    padding 1); 2 x 2 / stride 2 max and average pooling of a [64, 64, 112, 112] image (205 MB: the 26 MB of the other
+    image are gone in the time a launch takes)."""
     rs = np.random.default_rng(seed)
     x = _uniform(rs, n, -3, 3)
     vi = _vec(n)
     bins = 256
     bi = _vec(bins)
-    img, col, pooled = [32, 64, 56, 56], [32, 64, 3, 3, 56, 56], [32, 64, 28, 28]
-    ii, ci, pi = harness.shape_info(img), harness.shape_info(col), harness.shape_info(pooled)
-    n_img, n_col, n_pool = int(np.prod(img)), int(np.prod(col)), int(np.prod(pooled))
+    img, col = [32, 64, 56, 56], [32, 64, 3, 3, 56, 56]
+    big, pooled = [64, 64, 112, 112], [64, 64, 56, 56]
+    ii, ci, bgi, pi = harness.shape_info(img), harness.shape_info(col), harness.shape_info(big), harness.shape_info(pooled)
+    n_img, n_col, n_big, n_pool = int(np.prod(img)), int(np.prod(col)), int(np.prod(big)), int(np.prod(pooled))
     image = _uniform(rs, n_img, -3, 3)
+    big_image = _uniform(rs, n_big, -3, 3)
     e_hist = np.array([bins, -2.5, 2.75], F32)
     e_im2col = np.array([3, 3, 1, 1, 1, 1, 1, 1, 0, 0], F32)
     e_col2im = np.array([1, 1, 1, 1, 56, 56, 1, 1], F32)
@@ -615,6 +618,7 @@ def whole_array_transforms(dev, n=1 << 26, seed=41, copies=None):
         X, Z = w.operand(x, vi), w.operand(np.zeros(n, F32), vi)
         H = w.operand(np.zeros(bins, F32), bi)
         I, C, P = w.operand(image, ii), w.operand(np.zeros(n_col, F32), ci), w.operand(np.zeros(n_pool, F32), pi)
+        B = w.operand(big_image, bgi)
         I2 = w.operand(np.zeros(n_img, F32), ii)
         EH, EI, EC = w.raw(e_hist), w.raw(e_im2col), w.raw(e_col2im)
         EP = {k: w.raw(v) for k, v in e_pool.items()}
@@ -636,15 +640,15 @@ def whole_array_transforms(dev, n=1 << 26, seed=41, copies=None):
         cases.append(Case("col2im_3x3", "transform", n_col, 4 * n_img + 4 * n_col,
                           lambda: ops.execTransformFloat(exc, 36, C.ptr, C.info_ptr, I2.ptr, I2.info_ptr, EC.ptr),
                           None, True, I2.get))
-        exp_ = dev.extra(ii, z_info=pi)
+        exp_ = dev.extra(bgi, z_info=pi)
         for mode, name in ((0, "maxpool_2x2"), (1, "avgpool_2x2")):
-            cases.append(Case(name, "transform", n_img, 4 * n_img + 4 * n_pool,
-                              lambda mode=mode: ops.execTransformFloat(exp_, 71, I.ptr, I.info_ptr, P.ptr, P.info_ptr, EP[mode].ptr),
-                              lambda lib, mode=mode: (lib.transform(71, image, ii, poolc, pi, e_pool[mode]), poolc)[1], True, P.get))
+            cases.append(Case(name, "transform", n_big, 4 * n_big + 4 * n_pool,
+                              lambda mode=mode: ops.execTransformFloat(exp_, 71, B.ptr, B.info_ptr, P.ptr, P.info_ptr, EP[mode].ptr),
+                              lambda lib, mode=mode: (lib.transform(71, big_image, bgi, poolc, pi, e_pool[mode]), poolc)[1], True, P.get))
         return cases
 
-    return _replicated(dev, "whole-array transforms: reverse / histogram 2^26; im2col, col2im, pooling on [32,64,56,56]",
-                       8 * n + 8 * n_col, dict(x=x, image=image), device_set, copies)
+    return _replicated(dev, "whole-array transforms: reverse / histogram 2^26; im2col, col2im on [32,64,56,56]; pooling on [64,64,112,112]",
+                       8 * n + 8 * n_col + 4 * n_big, dict(x=x, image=image, big_image=big_image), device_set, copies)
 
 
 BUILDERS = [transform_tanh, pairwise_broadcast, reductions, reduce3_pairs, stats_softmax, random_fills]

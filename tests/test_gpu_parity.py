@@ -668,6 +668,36 @@ def test_whole_array_transforms_larger(gpu, cpu):
             assert np.allclose(gp, cp, rtol=1e-5, atol=1e-6), ("pooling", mode, p0)
 
 
+def test_whole_array_transforms_usual_windows(gpu, cpu):
+    # The shapes that have kernels of their own: Im2col with a block per channel (1024 (batch, channel) pairs or more),
+    # Col2Im with the window compiled in (1x1, 2x2, 3x3, 5x5) and with a run-time window (3x2, 7x7), 2x2 / stride 2
+    # pooling with its paired loads (even and odd row pitches, result rows of even and odd length), for the three types.
+    rs = np.random.RandomState(47)
+    for dt in (np.float32, np.float64, np.float16):
+        for (kH, kW, pad) in ((3, 3, 1), (1, 1, 0), (2, 2, 0), (5, 5, 2), (3, 2, 1), (7, 7, 3)):
+            bS, iC, iH, iW = 16, 64, 14, 12
+            oH, oW = iH + 2 * pad - kH + 1, iW + 2 * pad - kW + 1
+            img, col = [bS, iC, iH, iW], [bS, iC, kH, kW, oH, oW]
+            ii, ci = shape_info_np(img), shape_info_np(col)
+            x = rs.randint(-8, 9, int(np.prod(img))).astype(dt)  # small integers: every sum is exact in every type
+            e_im = np.array([kH, kW, 1, 1, pad, pad, 1, 1, 0, 0], dt)
+            g, c = gpu.transform(37, x, ii, ci, e_im), cpu.transform(37, x, ii, ci, e_im)
+            assert np.array_equal(g, c), ("im2col", dt, kH, kW)
+            e_col = np.array([1, 1, pad, pad, iH, iW, 1, 1], dt)
+            assert np.array_equal(gpu.transform(36, g, ci, ii, e_col), cpu.transform(36, c, ci, ii, e_col)), ("col2im", dt, kH, kW)
+        for iH, iW in ((56, 56), (9, 57), (10, 54), (7, 7)):
+            img, pooled = [3, 5, iH, iW], [3, 5, iH // 2, iW // 2]
+            ii, pi = shape_info_np(img), shape_info_np(pooled)
+            x = rs.randint(-8, 9, int(np.prod(img))).astype(dt)
+            for mode, p0 in ((0, 0.0), (1, 0.0), (1, 1.0), (1, 2.0), (2, 2.0), (3, 0.0)):
+                e_pool = np.array([2, 2, 2, 2, 0, 0, 1, 1, 0, mode, p0], dt)
+                gp, cp = gpu.transform(71, x, ii, pi, e_pool), cpu.transform(71, x, ii, pi, e_pool)
+                if mode == 2:
+                    assert np.allclose(gp.astype(np.float64), cp.astype(np.float64), rtol=1e-2 if dt == np.float16 else 1e-5), ("pooling", dt, iH, iW, mode)
+                else:
+                    assert np.array_equal(gp, cp, equal_nan=True), ("pooling", dt, iH, iW, mode, p0)
+
+
 def test_whole_array_transforms_strided_form_and_errors(gpu, cpu):
     # the strided entry point runs the ops' per-element op(): identity, and softplus for the softmax family
     x = np.linspace(-3, 3, 257).astype(np.float32)
