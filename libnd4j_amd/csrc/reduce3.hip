@@ -76,7 +76,8 @@ struct Reduce3Plan {
 template <typename T, int OP, int GROUP>
 __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, T *z, const T *extra, Reduce3Plan pl,
                                                         Acc3<typename Compute<T>::type> *partials, Long sliceLength, Long slices,
-                                                        unsigned long long *signal, unsigned ticket) {
+                                                        unsigned long long *signal, unsigned ticket, unsigned long long *slots,
+                                                        unsigned *counter, unsigned slotTicket) {
     typedef typename Compute<T>::type C;
     typedef Acc3<C> Acc;
     constexpr int GROUPS = kBlock / GROUP;
@@ -151,12 +152,31 @@ __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, 
         }
         if (live && lane == 0) {
             if (sliced) {
-                partials[u] = acc;
+                if (slots != nullptr) publishSlots(slots + (size_t)u * (sizeof(Acc) / 4), acc, slotTicket);
+                else partials[u] = acc;
             } else {
                 const T r = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, pl.runLength));
                 z[u] = r;
                 signalResult(signal, ticket, r);  // set only for a launch with a single result
             }
+        }
+    }
+    if (GROUP == kBlock && slots != nullptr) {
+        // A single result cut into one slice per block (`slots` is only given then): the block that counts itself in last
+        // merges the slices, as the whole-array reductions do, instead of a second launch.
+        __shared__ int mergeHere;
+        if (threadIdx.x == 0) mergeHere = countedInLast(counter);
+        __syncthreads();
+        if (!mergeHere) return;
+        Acc3Merge<C> mg;
+        Acc acc;
+        acc.r = acc.e0 = acc.e1 = (C)0;
+        mergeSlots<Acc3Merge<C>>(mg, acc, slots, threadIdx.x, kBlock, (int)gridDim.x, slotTicket);
+        acc = blockMerge<Acc3Merge<C>>(mg, acc, smem);
+        if (threadIdx.x == 0) {
+            const T r = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, pl.runLength));
+            z[0] = r;
+            signalResult(signal, ticket, r);
         }
     }
 }
@@ -332,8 +352,16 @@ template <typename T> struct Reduce3Body {
                 slices = (pl.runLength + sliceLength - 1) / sliceLength;
                 if (slices >= 2) {  // a single slice needs no second launch: the per-result kernels below do it in one
                     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+                    if (pl.numOut == 1 && ws.slots != nullptr && ws.counter != nullptr && ws.slotTicketSource != nullptr &&
+                        slices <= (Long)kFlatMaxBlocks && (size_t)slices * sizeof(Acc) * 2 <= ws.slotBytes) {
+                        // one result: one launch, the last block merging the slices
+                        ND4J_LAUNCH((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)slices), dim3(kBlock), 0, s, x, y, z, extra, pl,
+                                    partials, sliceLength, slices, ws.signal, ws.ticket, ws.slots, ws.counter, ws.nextSlotTicket());
+                        return true;
+                    }
                     ND4J_LAUNCH((reduce3Kernel<T, OP, kBlock>), dim3((unsigned)(slices * pl.numOut)), dim3(kBlock), 0, s, x, y, z,
-                                       extra, pl, partials, sliceLength, slices, (unsigned long long *)nullptr, 0u);
+                                       extra, pl, partials, sliceLength, slices, (unsigned long long *)nullptr, 0u,
+                                       (unsigned long long *)nullptr, (unsigned *)nullptr, 0u);
                     ND4J_LAUNCH((reduce3Finish<T, OP>), dim3((unsigned)pl.numOut), dim3(kBlock), 0, s, z, partials, (int)slices,
                                        pl.runLength, pl.numOut == 1 ? ws.signal : nullptr, ws.ticket);
                     return true;
@@ -344,13 +372,13 @@ template <typename T> struct Reduce3Body {
             const unsigned ticket = ws.ticket;
             if (pl.runLength >= 4096) {
                 int grid = gridFor(pl.numOut, 1, kGridCap);
-                ND4J_LAUNCH((reduce3Kernel<T, OP, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
+                ND4J_LAUNCH((reduce3Kernel<T, OP, kBlock>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket, (unsigned long long *)nullptr, (unsigned *)nullptr, 0u);
             } else if (pl.runLength >= 128) {
                 int grid = gridFor(pl.numOut, kBlock / 64, kGridCap);
-                ND4J_LAUNCH((reduce3Kernel<T, OP, 64>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
+                ND4J_LAUNCH((reduce3Kernel<T, OP, 64>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket, (unsigned long long *)nullptr, (unsigned *)nullptr, 0u);
             } else {
                 int grid = gridFor(pl.numOut, kBlock / 16, kGridCap);
-                ND4J_LAUNCH((reduce3Kernel<T, OP, 16>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket);
+                ND4J_LAUNCH((reduce3Kernel<T, OP, 16>), dim3(grid), dim3(kBlock), 0, s, x, y, z, extra, pl, none, (Long)0, (Long)1, signal, ticket, (unsigned long long *)nullptr, (unsigned *)nullptr, 0u);
             }
             return true;
         }

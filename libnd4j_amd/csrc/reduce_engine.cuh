@@ -425,6 +425,24 @@ __device__ __forceinline__ void mergeSlots(const Pol &pol, typename Pol::Acc &ac
     }
 }
 
+// One thread of every block of a one-dimensional grid (of at most kFlatMaxBlocks blocks) calls this once, after it has
+// published the block's slots: true in the block that counts itself in last.  The counters are back at zero by then.
+// Atomics on one address are served one after the other, some 15 ns apiece: two thousand blocks on a single counter
+// cost more than the reduction itself.  So blocks count in groups of kFlatGroup, each group on a counter of its own (in
+// a memory channel of its own), and only the last block of each group goes on to the top counter.
+__device__ __forceinline__ bool countedInLast(unsigned *counter) {
+    const unsigned group = blockIdx.x / kFlatGroup, groups = (gridDim.x + kFlatGroup - 1) / kFlatGroup;
+    const unsigned members = group + 1 < groups ? kFlatGroup : gridDim.x - group * kFlatGroup;
+    unsigned *mine = counter + (size_t)(1 + group) * kFlatCounterStride;
+    bool last = __hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1;
+    if (last) {
+        __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1;
+        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return last;
+}
+
 // The full-array reduction: block b folds the chunks b, b+grid, ... of kBlock*kUnroll vectors.
 // A one-block launch (small arrays) finishes by itself.  With several blocks and `slots` given, every block publishes
 // its accumulator in its slot group and takes a number from `counter`; the block that draws the last number has seen
@@ -495,19 +513,7 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
     constexpr int W = sizeof(Acc) / 4;
     if (threadIdx.x == 0) {
         publishSlots(slots + (size_t)blockIdx.x * W, acc, slotTicket);
-        // Atomics on one address are served one after the other, some 15 ns apiece: two thousand blocks on a single
-        // counter cost more than the reduction itself.  So blocks count in groups of kFlatGroup, each group on a counter
-        // of its own (in a memory channel of its own), and only the last block of each group goes on to the top counter.
-        const unsigned group = blockIdx.x / kFlatGroup, groups = (gridDim.x + kFlatGroup - 1) / kFlatGroup;
-        const unsigned members = group + 1 < groups ? kFlatGroup : gridDim.x - group * kFlatGroup;
-        unsigned *mine = counter + (size_t)(1 + group) * kFlatCounterStride;
-        bool last = __hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1;
-        if (last) {
-            __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            last = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1;
-            if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        mergeHere = last;
+        mergeHere = countedInLast(counter);
     }
     __syncthreads();
     if (!mergeHere) return;

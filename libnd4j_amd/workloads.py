@@ -293,6 +293,7 @@ def reduce3_pairs(dev, rows=16384, cols=4096, seed=12, copies=None):
 
         cases.append(Case("dot_full", "reduce3", n, 8 * n + 4, gpu_dot, lambda lib: lib.reduce3_scalar(3, x, xi, y, xi, None), True,
                           lambda: np.array([out["dot"]], F32)))
+        cases[-1].note = "returns the scalar to the host: launch and hand-over latency included"
         # every row of a [2048,1024] piece of x (its first 2 Mi elements) against every row of the same piece of y: 2048 x 2048
         # dot products.
         # Not a streaming case: each operand is read from HBM once and reused from LDS (its "bytes" are the 16 MiB of
