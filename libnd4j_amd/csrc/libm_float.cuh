@@ -137,11 +137,9 @@ __device__ __forceinline__ float sincosPoly(double x, double x2, int n, bool neg
 __device__ __forceinline__ float sincosCore(float y, bool wantCos) {
     const double hpiInv = 0x1.45F306DC9C883p+23, hpi = 0x1.921FB54442D18p0;
     double x = (double)y;
-    const unsigned top = (asU32(y) >> 20) & 0x7ff;
-    if (top < 0x3f4) {  // |y| < pi/4
-        if (top < 0x398) return wantCos ? 1.0f : y;  // |y| < 2^-12
-        return sincosPoly(x, x * x, wantCos ? 1 : 0, false);
-    }
+    // (The C library returns early below pi/4 - the polynomial on the argument itself - and below 2^-12 - the argument,
+    // or 1.  The general path gives the same bits there: the quadrant comes out as 0 exactly, and the polynomial of so
+    // small an argument rounds to the argument, or to 1.  Without the early returns the lanes of a wave stay together.)
     double r = x * hpiInv;
     int n = ((int)r + 0x800000) >> 24;
     x = x - (double)n * hpi;
