@@ -936,6 +936,29 @@ def test_random_ops_against_cpu(gpu, cpu):
         b.destroy()
 
 
+def test_random_blocks_across_the_ends_of_the_buffer(gpu, cpu):
+    # Draws far longer than the buffer, whose size is no multiple of what a block takes: blocks straddle the buffer's end,
+    # where the generation (and with it the divisor of the first shift) changes inside a block; started at several
+    # positions, after a reseed too.  Uniform and dropout bit for bit, Gaussian within 2 ULP.
+    n = 50000
+    x = np.linspace(-2, 2, n).astype(np.float32)
+    for seed, size, pre in ((7, 1000, 0), (8, 4099, 123456), (9, 10000, 9999), (10, 300, 77)):
+        a, b = gpu.rng(seed, size), cpu.rng(seed, size)
+        a.rewind(pre)
+        b.rewind(pre)
+        for round_ in range(2):
+            assert np.array_equal(a.random_z(0, n, [-1, 3]), b.random_z(0, n, [-1, 3])), (size, pre, round_)
+            assert np.array_equal(a.random_xz(1, x, [0.5]), b.random_xz(1, x, [0.5])), (size, pre, round_)
+            g = a.random_xyz(6, None, None, [0.5, 2.0], mode="inplace_all", n=n - 1)
+            c = b.random_xyz(6, None, None, [0.5, 2.0], mode="inplace_all", n=n - 1)
+            assert ulp_distance(g, c).max() <= 2, (size, pre, round_)
+            assert a.state() == b.state()
+            a.reseed(31337)
+            b.reseed(31337)
+        a.destroy()
+        b.destroy()
+
+
 def test_random_on_strided_output(gpu, cpu):
     # a non-EWS output is filled in Fortran order of its shape (the reference's ind2sub branch)
     zi = harness.shape_info([7, 9], "f")  # EWS -1
