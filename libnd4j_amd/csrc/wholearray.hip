@@ -518,7 +518,7 @@ template <typename T> void launchCol2im(hipStream_t s, const T *x, T *z, const T
         ND4J_LAUNCH(clearBytesKernel, dim3(gridFor(vectors + 1)), dim3(kBlock), 0, s, reinterpret_cast<U32x4 *>(base + lead), vectors,
                            base + lead + vectors * 16, tailBytes);
     }
-    const dim3 grid(gridFor(total));
+    const dim3 grid(gridFor(total, kBlock * 2));  // two pixels to a thread, one after the other
 #define ND4J_COL2IM(KH, KW)                                                                                                   \
     do {                                                                                                                      \
         if (clearFirst > 0) ND4J_LAUNCH((col2imKernel<T, true, KH, KW>), grid, dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);  \
@@ -671,7 +671,9 @@ __global__ void __launch_bounds__(kBlock) pooling2dKernel(const T *x, T *z, cons
 template <typename T> void launchPooling2d(hipStream_t s, const T *x, T *z, const T *extra, const ConvGeometry &g) {
     const Long total = (Long)g.bS * g.iC * g.oH * g.oW;
     if (total <= 0) return;
-    ND4J_LAUNCH(pooling2dKernel<T>, dim3(gridFor(total)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
+    // (two results to a thread: what the 2 x 2 path takes per thread for floats, so that none of its blocks starts for nothing;
+    // the general path walks its two in a loop)
+    ND4J_LAUNCH(pooling2dKernel<T>, dim3(gridFor(total, kBlock * 2)), dim3(kBlock), 0, s, x, z, extra, g, (unsigned)total);
 }
 
 // ---- DropOut 43 / DropOutInverted 44 as transforms ---------------------------------------------------------------
