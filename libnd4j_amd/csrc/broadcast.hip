@@ -12,7 +12,7 @@ template <typename T> struct BroadcastBody {
             if (pl.kind == BroadcastPlan::ROW && pl.consecutive && pl.tadLength % Pack<T>::N == 0 &&
                 pl.tadLength / Pack<T>::N < 0xffffffffLL && (((uintptr_t)x | (uintptr_t)y | (uintptr_t)z) & 15) == 0) {
                 const Long nvec = pl.numTads * (pl.tadLength / Pack<T>::N);
-                ND4J_LAUNCH((bcFlatKernel<T, F>), dim3(gridFor(nvec, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0,
+                ND4J_LAUNCH((bcFlatKernel<T, F>), dim3(gridFor(nvec, kBlock * 2, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0,
                                    s, x, y, z, nvec, (unsigned)(pl.tadLength / Pack<T>::N), Params<T>{nullptr});
             } else if (pl.kind == BroadcastPlan::ROW && pl.consecutive && pl.tadLength >= Pack<T>::N && pl.tadLength < 0xffffffffLL &&
                        (((uintptr_t)x | (uintptr_t)z) & 15) == 0) {
