@@ -21,6 +21,7 @@ template <typename TT, int OP> struct IndexPol {
     typedef typename Compute<TT>::type C;
     typedef IndexAcc<C> Acc;
     static constexpr bool tables = false;  // no exp / log / pow in these accumulators
+    static constexpr int kChains = 4;      // accumulators of one lane may be kept apart and combined (ties go to the lower index)
     Params<TT> p;
 
     __device__ __forceinline__ void setTad(Long, const TT *) {}

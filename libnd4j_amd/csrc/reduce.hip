@@ -93,6 +93,9 @@ template <typename TT, int OP> struct ReducePol {
     // ops whose functor or post-processing evaluates exp / log / pow (variance and standard deviation square their
     // bias term with pow); 20-23 have no functor
     static constexpr bool tables = OP == 9 || OP == 10 || (OP >= 16 && OP <= 24);
+    static constexpr int kChains = 4;  // accumulators of one lane may be kept apart and combined (combine is the update)
+    // Mean, Sum, Norm1, Norm2, SquaredNorm: plain running sums
+    static constexpr int kFlatBlocks = (OP == 0 || OP == 1 || OP == 5 || OP == 6 || OP == 25) ? 1024 : 2048;
     Params<TT> p;
     const TT *shiftSource;  // LogSumExp: per-TAD (TAD calls) or single (scalar calls) maximum; else null
     int shiftPerTad;

@@ -47,6 +47,14 @@ template <typename A> __device__ __forceinline__ A shflDownAny(A v, int delta) {
 template <class Pol, typename = void> struct HasOwnWaveMerge { static constexpr bool value = false; };
 template <class Pol> struct HasOwnWaveMerge<Pol, decltype((void)Pol::ownWaveMerge)> { static constexpr bool value = Pol::ownWaveMerge; };
 
+// A policy announces with a member constant kChains > 1 that a lane may keep several accumulators and combine() them.
+template <class Pol, typename = void> struct PolChains { static constexpr int value = 1; };
+template <class Pol> struct PolChains<Pol, decltype((void)Pol::kChains)> { static constexpr int value = Pol::kChains; };
+
+// The most blocks a policy wants for the whole-array kernel (a member constant kFlatBlocks; kFlatMaxBlocks otherwise).
+template <class Pol, typename = void> struct PolFlatBlocks { static constexpr int value = 2048; };
+template <class Pol> struct PolFlatBlocks<Pol, decltype((void)Pol::kFlatBlocks)> { static constexpr int value = Pol::kFlatBlocks; };
+
 // Merge over the lanes of one wave; lane 0 (of each WIDTH-lane segment) ends up with the result.
 template <class Pol, int WIDTH = kWave>
 __device__ __forceinline__ typename Pol::Acc waveMerge(const Pol &pol, typename Pol::Acc a) {
@@ -472,6 +480,16 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
         const Long nvec = (n - head) / VEC;
         const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x + head);
         const Long chunk = (Long)kBlock * kUnroll;
+        // A policy whose accumulators may be regrouped freely (kChains > 1: its combine() is its update) gets one
+        // accumulator per vector in flight: one accumulator makes every element wait for the one before it (a compare and a
+        // select for a maximum, three selects for an index), and with the few waves per SIMD of this launch nothing else
+        // fills the gaps - the maximum over 2^26 floats took 85 us with 512 blocks where the sum took 48.
+        constexpr int CH = PolChains<Pol>::value > 1 ? 4 : 1;
+        Acc more[CH > 1 ? CH - 1 : 1];
+        if (CH > 1) {
+#pragma unroll
+            for (int c = 0; c < CH - 1; c++) more[c] = pol.init(x);
+        }
         for (Long b = (Long)blockIdx.x * chunk; b < nvec; b += (Long)gridDim.x * chunk) {
             Pack<T> pk[kUnroll];
 #pragma unroll
@@ -483,11 +501,16 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
             for (int u = 0; u < kUnroll; u++) {
                 Long v = b + u * kBlock + threadIdx.x;
                 if (v < nvec) {
+                    Acc &to = (CH > 1 && u % CH > 0) ? more[u % CH - 1] : acc;
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[u].v[e]), head + v * VEC + e);
-                    pol.checkpoint(acc);
+                    for (int e = 0; e < VEC; e++) pol.accumulate(to, toCompute(pk[u].v[e]), head + v * VEC + e);
+                    pol.checkpoint(to);
                 }
             }
+        }
+        if (CH > 1) {
+#pragma unroll
+            for (int c = 0; c < CH - 1; c++) acc = pol.combine(acc, more[c]);
         }
         if (blockIdx.x == 0) {
             for (Long i = threadIdx.x; i < head; i += kBlock) { pol.accumulate(acc, toCompute(x[i]), i); pol.checkpoint(acc); }
@@ -649,7 +672,9 @@ inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, type
     typedef typename Pol::Acc Acc;
     typedef typename Pol::T T;
     Long perBlock = (Long)kBlock * kUnroll * Pack<T>::N;
-    int grid = gridFor(pl.n, perBlock, (int)kFlatMaxBlocks);
+    // (plain sums run a little faster - 49.5 against 51.4 us over 2^26 floats - with half as many blocks, each streaming
+    // longer; maxima and index reductions lose a third that way, so a policy asks for it: kFlatBlocks)
+    int grid = gridFor(pl.n, perBlock, PolFlatBlocks<Pol>::value);
     const bool oneLaunch = ws.slots != nullptr && ws.counter != nullptr && ws.slotTicketSource != nullptr;
     size_t maxBlocks = oneLaunch ? ws.slotBytes / (sizeof(Acc) / 4 * sizeof(unsigned long long)) : ws.bytes / sizeof(Acc);
     if ((size_t)grid > maxBlocks) grid = (int)maxBlocks;
