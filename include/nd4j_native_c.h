@@ -214,10 +214,10 @@ int nd4j_amd_timerDestroy(Nd4jPointer timer);
  * the device because the host copy / TAD tables of the CUDA convention were not passed: each one synchronises the
  * stream, so a caller that wants asynchronous array-result calls keeps this from growing */
 Nd4jLong nd4j_amd_hostFetchCount(void);
-/* No counterpart in the reference.  SoftMax / SoftMaxDerivative / LogSoftMax over long contiguous rows run as one pass in
- * which the blocks that hold the slices of a row wait for each other; every such wait is bounded, and a row whose
- * blocks could not all see each other in time is left untouched by them and computed by a repair kernel behind the
- * launch.  `tries` is the number of polls a block spends on a slice that is not there yet (default 5000, each a
+/* No counterpart in the reference.  SoftMax / SoftMaxDerivative / LogSoftMax over long contiguous rows, and over f-order
+ * matrices of more than 1024 columns, run as one pass in which the blocks that hold the slices of a row (of a group of
+ * rows) wait for each other; every such wait is bounded, and a row whose blocks could not all see each other in time is
+ * left untouched by them and computed by a repair kernel behind the launch.  `tries` is the number of polls a block spends on a slice that is not there yet (default 5000, each a
  * microsecond or two); 0 makes everything that is not there at the first look count as missing, which is how the tests
  * drive rows through the repair kernel. */
 void nd4j_amd_setCooperativeWaitLimit(int tries);
