@@ -642,7 +642,11 @@ def check_random_views(be, ref, seed, cases):
                 g = be.reduce(op, x, xi, None, dims, out_len, **kw(pass_tads=bool(rs.randint(0, 2))))
                 c = ref.reduce(op, x, xi, None, dims, out_len)
                 scale = np.abs(x).sum() / max(1, out_len)
-                assert np.all(np.abs(g.astype(np.float64) - c) <= 2 * REDUCE_RTOL * np.abs(c) + 2e-6 * scale), ("reduce", op, dims, list(xi))
+                # (the reference adds a TAD up in float, one element after the other: over millions of elements its own
+                # result is off by some sqrt(length) roundings - 4e-5 was seen on 2.9 M elements where the device's sum was
+                # within 5e-8 of the float64 one - so the bar widens with the TAD's length)
+                drift = 2.0 * np.sqrt(n / max(1, out_len)) * 6e-8
+                assert np.all(np.abs(g.astype(np.float64) - c) <= (2 * REDUCE_RTOL + drift) * np.abs(c) + (2e-6 + drift) * scale), ("reduce", op, dims, list(xi))
             elif what == 3:
                 xu = rs.permutation(harness.span_of(xi)).astype(np.float32)  # distinct values: no ties to resolve
                 op = int(rs.choice([0, 1]))
