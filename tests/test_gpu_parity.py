@@ -849,6 +849,42 @@ def test_softmax_of_f_order_matrices_cooperating_blocks(gpu, cpu):
         gpu.ops.amd_setCooperativeWaitLimit(5000)
 
 
+def test_softmax_family_over_generated_shapes(gpu):
+    # SoftMax / SoftMaxDerivative / LogSoftMax over generated matrices whose row lengths sit on and around the sizes where
+    # the kernels change (16, 64, 256, 1024, 2048, 8192, 16384, 65536 columns; few and many rows), both orders, three types,
+    # in place or not, now and then with the cooperative kernels' patience at zero: against float64.
+    rs = np.random.RandomState(53)
+    col_choices = [2, 3, 15, 16, 17, 63, 64, 65, 255, 256, 257, 1000, 1023, 1024, 1025, 1026, 1500, 2047, 2048, 2049, 2052, 3000, 4096,
+                   4100, 5001, 8191, 8192, 8193, 8200, 10000, 16383, 16384, 16388, 20000, 32768, 50257, 65536, 65540, 100003, 300001]
+    row_choices = [1, 2, 3, 4, 7, 8, 31, 32, 33, 64, 100, 255, 256, 257, 260, 264, 300, 512, 1000, 1024, 2048, 4100]
+    try:
+        for it in range(160):
+            cols = int(rs.choice(col_choices))
+            rows = min(int(rs.choice(row_choices)), max(1, (4 << 20) // cols))
+            order = "c" if rs.rand() < 0.5 else "f"
+            dt = [np.float32, np.float32, np.float16, np.float64][int(rs.randint(0, 4))]
+            op = int(rs.choice([38, 39, 40]))
+            limit = 5000 if rs.rand() < 0.8 else 0
+            gpu.ops.amd_setCooperativeWaitLimit(limit)
+            shape = [rows, cols]
+            info = harness.shape_info(shape, order)
+            a = rs.uniform(-6, 6, shape).astype(dt)
+            memory_order = "F" if order == "f" else "C"
+            x = np.ascontiguousarray(a.flatten(order=memory_order))
+            r64 = a.astype(np.float64)
+            truth = np.exp(r64 - r64.max(axis=1, keepdims=True))
+            truth /= truth.sum(axis=1, keepdims=True)
+            want = {38: lambda v: v, 39: lambda v: v * (1 - v), 40: np.log}[op](truth)
+            rtol = {np.float32: 3e-5, np.float16: 2e-2, np.float64: 1e-11}[dt]
+            atol = {np.float32: 2e-7, np.float16: 2e-4, np.float64: 1e-300}[dt]
+            in_place = rs.rand() < 0.4
+            got = gpu.transform_inplace(op, x, info) if in_place else gpu.transform(op, x, info, info)
+            got = got.astype(np.float64).reshape(shape, order=memory_order)
+            assert np.all(np.abs(got - want) <= rtol * np.abs(want) + atol), (shape, order, dt, op, limit, in_place)
+    finally:
+        gpu.ops.amd_setCooperativeWaitLimit(5000)
+
+
 def test_half_families(gpu, cpu):
     rs = np.random.RandomState(28)
     h = np.float16
