@@ -849,6 +849,70 @@ def test_softmax_of_f_order_matrices_cooperating_blocks(gpu, cpu):
         gpu.ops.amd_setCooperativeWaitLimit(5000)
 
 
+def test_reductions_over_generated_shapes(gpu):
+    # Sum / Mean / Max, IndexMax, bias-corrected variance and the scalar-returning calls over generated matrices whose
+    # extents sit on and around the sizes where the reduction kernels change (lanes per TAD, slices of long TADs, vector
+    # widths, the whole-array grid), both orders, three types, along either dimension or both, with and without the
+    # caller's TAD tables: against float64.
+    rs = np.random.RandomState(59)
+    sizes = [1, 2, 3, 7, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1000, 1023, 1024, 1025, 2048, 4095, 4096,
+             4100, 8192, 16383, 16384, 16385, 20000, 65536, 100003, 262144, 1 << 20, (1 << 20) + 3]
+    for it in range(200):
+        rows, cols = int(rs.choice(sizes)), int(rs.choice(sizes))
+        while rows * cols > (4 << 20):
+            if rows > cols:
+                rows = int(rs.choice([v for v in sizes if v < rows]))
+            else:
+                cols = int(rs.choice([v for v in sizes if v < cols]))
+        order = "c" if rs.rand() < 0.5 else "f"
+        dt = [np.float32, np.float32, np.float64, np.float16][int(rs.randint(0, 4))]
+        shape = [rows, cols]
+        info = harness.shape_info(shape, order)
+        a = rs.uniform(-1, 1, shape).astype(dt) if dt == np.float16 else rs.uniform(-3, 3, shape).astype(dt)
+        memory_order = "F" if order == "f" else "C"
+        x = np.ascontiguousarray(a.flatten(order=memory_order))
+        a64 = a.astype(np.float64)
+        which = int(rs.randint(0, 4))
+        dims = [[0], [1], [0, 1]][int(rs.randint(0, 3))]
+        pass_tads = bool(rs.randint(0, 2))
+        axis = tuple(dims)
+        out_len = int(np.prod([shape[d] for d in range(2) if d not in dims])) if len(dims) < 2 else 1
+        rtol = {np.float32: 2e-5, np.float64: 1e-12, np.float16: 2e-2}[dt]
+        tag = (shape, order, dt.__name__, which, dims, pass_tads)
+        if which == 0:
+            op = int(rs.choice([0, 1, 3]))
+            got = gpu.reduce(op, x, info, None, dims, out_len, pass_tads=pass_tads).astype(np.float64)
+            want = {0: a64.mean(axis=axis), 1: a64.sum(axis=axis), 3: a64.max(axis=axis)}[op].reshape(-1)
+            scale = np.abs(a64).sum(axis=axis).reshape(-1) if op != 3 else np.abs(want)
+            if op == 0:
+                scale = scale / np.prod([shape[d] for d in dims])
+            if dt == np.float16 and op != 3 and np.abs(want).max() > 60000:
+                continue
+            assert np.all(np.abs(got - want) <= rtol * scale + 1e-30), tag
+        elif which == 1:
+            if (dt == np.float16 and rows * cols > 2000) or len(dims) == 2 and order == "f":
+                continue
+            perm = rs.permutation(rows * cols).astype(dt)  # distinct values: no ties to resolve
+            got = gpu.indexreduce(0, perm, info, None, dims, out_len, pass_tads=pass_tads).astype(np.int64)
+            p2 = perm.reshape(shape, order=memory_order).astype(np.float64)
+            want = np.array([int(np.argmax(p2.reshape(-1)))]) if len(dims) == 2 else p2.argmax(axis=dims[0]).reshape(-1)
+            assert np.array_equal(got, want), tag
+        elif which == 2:
+            if dt == np.float16 or int(np.prod([shape[d] for d in dims])) < 2:
+                continue
+            got = gpu.summarystats(0, True, x, info, dims, out_len, pass_tads=pass_tads).astype(np.float64)
+            want = a64.var(axis=axis, ddof=1).reshape(-1)
+            assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-12), tag
+        else:
+            op = int(rs.choice([0, 1, 3]))
+            got = float(gpu.reduce_scalar(op, x, info))
+            want = {0: a64.mean(), 1: a64.sum(), 3: a64.max()}[op]
+            scale = np.abs(a64).sum() if op == 1 else (np.abs(a64).mean() if op == 0 else abs(want))
+            if dt == np.float16 and op == 1 and abs(want) > 60000:
+                continue
+            assert abs(got - want) <= rtol * scale + 1e-30, tag
+
+
 def test_softmax_family_over_generated_shapes(gpu):
     # SoftMax / SoftMaxDerivative / LogSoftMax over generated matrices whose row lengths sit on and around the sizes where
     # the kernels change (16, 64, 256, 1024, 2048, 8192, 16384, 65536 columns; few and many rows), both orders, three types,
