@@ -197,9 +197,11 @@ struct ReversePlan {
     DimMap xm, zm;            // element e of x -> offset, element of z -> offset (each in its own order)
 };
 template <typename T> void launchReverse(hipStream_t stream, const T *x, T *z, const ReversePlan &plan);
-// counts: capacity 32-bit counters of scratch; capacity = length of z (the bins that can be written)
+// counts: histogramScratchBytes(..) of scratch; capacity = length of z (the bins that can be written)
 template <typename T>
 void launchHistogram(hipStream_t stream, const T *x, Long n, T *z, int capacity, const T *extra, unsigned *counts);
+// bytes of `counts` that launchHistogram uses for n elements of the given size and a result of `capacity` bins
+size_t histogramScratchBytes(Long n, int elementBytes, int capacity);
 // An image [bS, iC, iH, iW] with strides imS, and either its column form [bS, iC, kH, kW, oH, oW] with strides colS
 // (Im2col, Col2Im) or its pooled form [bS, iC, oH, oW] with strides colS[0..3] (Pooling2D).  Element counts stay below 2^31.
 struct ConvGeometry {

@@ -99,7 +99,7 @@ template <typename T> void histogramWhole(const T *x, const Long *hx, T *z, cons
     const Long capacity = siNumel(hz);
     requireSmall(capacity, "Histogram");
     if (capacity <= 0) return;
-    Workspace w = workspaceFor(s, (size_t)capacity * sizeof(unsigned));
+    Workspace w = workspaceFor(s, histogramScratchBytes(n, (int)sizeof(T), (int)capacity));
     launchHistogram<T>(s, x, n, z, (int)capacity, params, reinterpret_cast<unsigned *>(w.ptr));
 }
 

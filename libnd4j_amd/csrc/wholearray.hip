@@ -170,30 +170,43 @@ __global__ void __launch_bounds__(kBlock) clearCountsKernel(unsigned *counts, in
     for (int i = blockIdx.x * kBlock + threadIdx.x; i < n; i += gridDim.x * kBlock) counts[i] = 0u;
 }
 
-// Counts per block in LDS (when the bins fit), flushed with one atomic per non-empty bin; otherwise atomics on the
-// global counters directly.  LDS atomics of one wave on one address are served one after the other, and with few bins
-// most lanes of a wave meet in the same few: the block then keeps several copies of the bins (as many as fit, up to
-// 32), lane l counting in copy l % copies, and adds the copies up when it flushes.
+// Counts per block in LDS (when the bins fit); otherwise atomics on the global counters directly.  LDS atomics of one
+// wave that meet in one bank are served one after the other, whether they name the same word or not, so the bank should
+// follow from the lane and not from the bin: the block keeps `copies` (a power of two, as many as fit, up to 32)
+// counters per bin side by side, lane l counting in word bin * copies + l % copies.  With 32 copies the word's bank is
+// the lane's number modulo 32, which no two lanes of a half wave share.
+// A block hands its counts over in one of two ways.  ROWS: it stores them, zeros included, as row blockIdx of a
+// [blocks, capacity] table that the adding kernel sums; nothing needs clearing, and no two blocks touch the same word.
+// Otherwise it adds them to one shared row, cleared first, with an atomic per non-empty bin: atomics of many blocks on
+// the same few hundred words are served one after the other, so this way is kept for bin counts whose table would be too
+// large.  Either way a block costs its share of clearing and adding up 32 KiB of LDS and of the hand-over, whatever it
+// counts: two blocks per compute unit are the measured optimum (2^26 floats, 256 bins, whole call: 256 blocks 72 us,
+// 384 58, 512 49, 768 51, 1024 56, 2048 64; of the 49, the counting kernel is 44 and the adding kernel 5).
 constexpr int kLdsBins = 8192;
-template <typename T, bool LDS>
+constexpr Long kHistogramTableWords = 1 << 20;
+constexpr int kHistogramBlocks = 512;
+constexpr int kHistogramInFlight = 4;  // vectors a lane loads before it counts them (8 measured slower)
+template <typename T, bool LDS, bool ROWS>
 __global__ void __launch_bounds__(kBlock) histogramCountKernel(const T *x, Long n, const T *extra, unsigned *counts, int capacity) {
+    static_assert(LDS || !ROWS, "a table of rows is filled from the block's counts in LDS");
     __shared__ unsigned local[LDS ? kLdsBins : 1];
     const HistogramBins<T> bins(extra, capacity);
     if (bins.numBins <= 0) return;
     int copies = 1;
     if (LDS) {
-        copies = kLdsBins / bins.numBins;
-        copies = copies > 32 ? 32 : (copies < 1 ? 1 : copies);
+        const int fit = kLdsBins / bins.numBins;
+        while (copies < 32 && copies * 2 <= fit) copies *= 2;
         for (int b = threadIdx.x; b < bins.numBins * copies; b += kBlock) local[b] = 0u;
         __syncthreads();
     }
-    unsigned *myBins = local + (LDS ? (threadIdx.x % copies) * bins.numBins : 0);
+    const int shift = __builtin_ctz(copies);
+    unsigned *myBins = local + (LDS ? (threadIdx.x & (copies - 1)) : 0);
     constexpr int N = Pack<T>::N;
     const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(x) & 15)) & 15) / sizeof(T));
     const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
     auto count = [&](T v) {
         const int idx = bins(v);
-        if (LDS) atomicAdd(&myBins[idx], 1u);
+        if (LDS) atomicAdd(&myBins[idx << shift], 1u);
         else atomicAdd(&counts[idx], 1u);
     };
     const Long lead = head < n ? head : n;
@@ -203,12 +216,12 @@ __global__ void __launch_bounds__(kBlock) histogramCountKernel(const T *x, Long 
     // four vectors in flight per lane: the counting of one batch then overlaps the memory latency of the next lanes'
     const Long step = (Long)gridDim.x * kBlock;
     Long v = gtid;
-    for (; v + 3 * step < nvec; v += 4 * step) {
-        Pack<T> a[4];
+    for (; v + (kHistogramInFlight - 1) * step < nvec; v += kHistogramInFlight * step) {
+        Pack<T> a[kHistogramInFlight];
 #pragma unroll
-        for (int u = 0; u < 4; u++) a[u] = loadPack(xv + v + u * step);
+        for (int u = 0; u < kHistogramInFlight; u++) a[u] = loadPack(xv + v + u * step);
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kHistogramInFlight; u++) {
 #pragma unroll
             for (int k = 0; k < N; k++) count(a[u].v[k]);
         }
@@ -224,36 +237,60 @@ __global__ void __launch_bounds__(kBlock) histogramCountKernel(const T *x, Long 
         __syncthreads();
         for (int b = threadIdx.x; b < bins.numBins; b += kBlock) {
             unsigned c = 0u;
-            for (int k = 0; k < copies; k++) c += local[k * bins.numBins + b];
-            if (c != 0u) atomicAdd(&counts[b], c);
+            // thread b starts at copy b % copies, so that the lanes of a wave read different banks
+            for (int k = 0; k < copies; k++) c += local[(b << shift) + ((k + b) & (copies - 1))];
+            if (ROWS) counts[(Long)blockIdx.x * capacity + b] = c;
+            else if (c != 0u) atomicAdd(&counts[b], c);
         }
     }
 }
 
-// z[b] += count[b], as the reference adds its counts onto what the result holds
+// z[b] += the counts of bin b over the table's rows, as the reference adds its counts onto what the result holds; one
+// wave per bin
 template <typename T>
-__global__ void __launch_bounds__(kBlock) histogramAddKernel(T *z, const T *extra, const unsigned *counts, int capacity) {
+__global__ void __launch_bounds__(kBlock) histogramAddKernel(T *z, const T *extra, const unsigned *counts, int capacity, int rows) {
     int numBins = paramInt(extra, 0);
     if (numBins > capacity) numBins = capacity;
-    for (int b = blockIdx.x * kBlock + threadIdx.x; b < numBins; b += gridDim.x * kBlock) {
+    const int lane = threadIdx.x & 63, wavesPerBlock = kBlock / 64;
+    for (int b = blockIdx.x * wavesPerBlock + (threadIdx.x >> 6); b < numBins; b += gridDim.x * wavesPerBlock) {
+        unsigned c = 0u;
+        for (int r = lane; r < rows; r += 64) c += counts[(Long)r * capacity + b];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
         typedef typename Compute<T>::type C;
-        z[b] = fromCompute<T>(toCompute(z[b]) + (C)(int)counts[b]);
+        if (lane == 0) z[b] = fromCompute<T>(toCompute(z[b]) + (C)(int)c);
     }
+}
+
+// blocks of the counting launch, and rows of the table it fills (0: one shared row, cleared first and added to with atomics)
+inline void histogramLaunchShape(Long vectors, int capacity, int &grid, int &rows) {
+    grid = gridFor(vectors + 1) > kHistogramBlocks ? kHistogramBlocks : gridFor(vectors + 1);
+    rows = (capacity <= kLdsBins && (Long)grid * capacity <= kHistogramTableWords) ? grid : 0;
+}
+size_t histogramScratchBytes(Long n, int elementBytes, int capacity) {
+    int grid, rows;
+    histogramLaunchShape(n / (16 / elementBytes), capacity, grid, rows);
+    return (size_t)(rows > 0 ? rows : 1) * (size_t)capacity * sizeof(unsigned);
 }
 
 template <typename T>
 void launchHistogram(hipStream_t s, const T *x, Long n, T *z, int capacity, const T *extra, unsigned *counts) {
     if (capacity <= 0) return;
-    ND4J_LAUNCH(clearCountsKernel, dim3(gridFor(capacity)), dim3(kBlock), 0, s, counts, capacity);
+    int grid, rows;
+    histogramLaunchShape(n / Pack<T>::N, capacity, grid, rows);
+    if (n <= 0) rows = 0;
+    if (rows == 0) ND4J_LAUNCH(clearCountsKernel, dim3(gridFor(capacity)), dim3(kBlock), 0, s, counts, capacity);
     if (n > 0) {
-        // enough blocks to fill the chip, few enough that the flushes of the per-block counts stay cheap
-        const int grid = gridFor(n / Pack<T>::N + 1) > 2048 ? 2048 : gridFor(n / Pack<T>::N + 1);
-        if (capacity <= kLdsBins)
-            ND4J_LAUNCH((histogramCountKernel<T, true>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
+        if (rows > 0)
+            ND4J_LAUNCH((histogramCountKernel<T, true, true>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
+        else if (capacity <= kLdsBins)
+            ND4J_LAUNCH((histogramCountKernel<T, true, false>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
         else
-            ND4J_LAUNCH((histogramCountKernel<T, false>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
+            ND4J_LAUNCH((histogramCountKernel<T, false, false>), dim3(grid), dim3(kBlock), 0, s, x, n, extra, counts, capacity);
     }
-    ND4J_LAUNCH(histogramAddKernel<T>, dim3(gridFor(capacity)), dim3(kBlock), 0, s, z, extra, counts, capacity);
+    const int addGrid = (capacity + kBlock / 64 - 1) / (kBlock / 64);
+    ND4J_LAUNCH(histogramAddKernel<T>, dim3(addGrid > 2048 ? 2048 : addGrid), dim3(kBlock), 0, s, z, extra, counts, capacity,
+                rows > 0 ? rows : 1);
 }
 
 // ---- Im2col ----------------------------------------------------------------------------------------------------

@@ -643,10 +643,11 @@ def test_whole_array_transforms_larger(gpu, cpu):
             vi = shape_info_np([1, n])
             assert np.array_equal(gpu.transform(70, x, vi, vi), x[::-1]), ("reverse", n, dt)
             assert np.array_equal(gpu.transform_inplace(70, x, vi), x[::-1]), ("reverse in place", n, dt)
-    # Histogram over a few million elements: bins in LDS and, beyond 8192 bins, in global memory
+    # Histogram over a few million elements: bins in LDS, handed over as a table of one row per block (up to 2048 bins) or
+    # with atomics on one row, and, beyond 8192 bins, counted in global memory
     n = (1 << 22) + 5
     x = rs.uniform(-3, 3, n).astype(f)
-    for bins in (10, 8192, 20000):
+    for bins in (10, 300, 2048, 2049, 8192, 20000):
         extra = np.array([bins, -2.5, 2.75], f)
         xi, zi = shape_info_np([1, n]), shape_info_np([1, bins])
         assert np.array_equal(gpu.transform(48, x, xi, zi, extra), cpu.transform(48, x, xi, zi, extra)), ("histogram", bins)
