@@ -55,6 +55,10 @@ template <class Pol> struct PolChains<Pol, decltype((void)Pol::kChains)> { stati
 template <class Pol, typename = void> struct PolFlatBlocks { static constexpr int value = 2048; };
 template <class Pol> struct PolFlatBlocks<Pol, decltype((void)Pol::kFlatBlocks)> { static constexpr int value = Pol::kFlatBlocks; };
 
+// Whether the clearing form of the whole-array kernel is built for a policy (a member constant kClears).
+template <class Pol, typename = void> struct PolClears { static constexpr bool value = false; };
+template <class Pol> struct PolClears<Pol, decltype((void)Pol::kClears)> { static constexpr bool value = Pol::kClears; };
+
 // Merge over the lanes of one wave; lane 0 (of each WIDTH-lane segment) ends up with the result.
 template <class Pol, int WIDTH = kWave>
 __device__ __forceinline__ typename Pol::Acc waveMerge(const Pol &pol, typename Pol::Acc a) {
@@ -460,11 +464,14 @@ __device__ __forceinline__ bool countedInLast(unsigned *counter) {
 // every other block issue its stores, waits for them to land, merges all groups in block order and writes the result
 // (the counters are back at zero by then): one launch.  Without `slots` the accumulators go to `partials` and flatFinish
 // merges them in a second launch.
-template <class Pol>
+// CLEAR (dense x only): every element that has been read is overwritten with zero in `cleared`, an array laid out like x
+// and on the same offset from a 16-byte boundary (x itself, or one that does not overlap it): each thread clears exactly
+// the elements it has loaded itself, so clearing in place is safe.
+template <class Pol, bool CLEAR = false>
 __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol::T *x, typename Pol::Acc *partials,
                                                      Long n, int strided, Long ews, DimMap xm, typename Pol::T *z,
                                                      unsigned long long *signal, unsigned ticket, unsigned long long *slots,
-                                                     unsigned *counter, unsigned slotTicket) {
+                                                     unsigned *counter, unsigned slotTicket, typename Pol::T *cleared = nullptr) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
@@ -507,14 +514,32 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
                     pol.checkpoint(to);
                 }
             }
+            if (CLEAR) {
+                Pack<T> zeros;
+#pragma unroll
+                for (int e = 0; e < VEC; e++) zeros.v[e] = fromCompute<T>((typename Pol::C)0);
+#pragma unroll
+                for (int u = 0; u < kUnroll; u++) {
+                    Long v = b + u * kBlock + threadIdx.x;
+                    if (v < nvec) storePack(reinterpret_cast<Pack<T> *>(cleared + head) + v, zeros);
+                }
+            }
         }
         if (CH > 1) {
 #pragma unroll
             for (int c = 0; c < CH - 1; c++) acc = pol.combine(acc, more[c]);
         }
         if (blockIdx.x == 0) {
-            for (Long i = threadIdx.x; i < head; i += kBlock) { pol.accumulate(acc, toCompute(x[i]), i); pol.checkpoint(acc); }
-            for (Long i = head + nvec * VEC + threadIdx.x; i < n; i += kBlock) { pol.accumulate(acc, toCompute(x[i]), i); pol.checkpoint(acc); }
+            for (Long i = threadIdx.x; i < head; i += kBlock) {
+                pol.accumulate(acc, toCompute(x[i]), i);
+                pol.checkpoint(acc);
+                if (CLEAR) cleared[i] = fromCompute<T>((typename Pol::C)0);
+            }
+            for (Long i = head + nvec * VEC + threadIdx.x; i < n; i += kBlock) {
+                pol.accumulate(acc, toCompute(x[i]), i);
+                pol.checkpoint(acc);
+                if (CLEAR) cleared[i] = fromCompute<T>((typename Pol::C)0);
+            }
         }
     } else if (strided) {
         for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock)
@@ -666,9 +691,10 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
                        pl.numTads);
 }
 
+// `cleared` (optional; only for a dense x, see flatKernel): an array like x that is overwritten with zeros on the way
 template <class Pol>
 inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typename Pol::T *z, const FlatPlan &pl,
-                          Workspace ws) {
+                          Workspace ws, typename Pol::T *cleared = nullptr) {
     typedef typename Pol::Acc Acc;
     typedef typename Pol::T T;
     Long perBlock = (Long)kBlock * kUnroll * Pack<T>::N;
@@ -680,9 +706,16 @@ inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, type
     if ((size_t)grid > maxBlocks) grid = (int)maxBlocks;
     if (grid < 1) grid = 1;
     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
-    ND4J_LAUNCH((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
-                       pl.ews, pl.xm, z, ws.signal, ws.ticket, oneLaunch ? ws.slots : nullptr, ws.counter,
-                       oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u);
+    if (cleared != nullptr) {
+        if constexpr (PolClears<Pol>::value)
+            ND4J_LAUNCH((flatKernel<Pol, true>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, 1, (Long)1, pl.xm, z,
+                               ws.signal, ws.ticket, oneLaunch ? ws.slots : nullptr, ws.counter,
+                               oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u, cleared);
+    } else {
+        ND4J_LAUNCH((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
+                           pl.ews, pl.xm, z, ws.signal, ws.ticket, oneLaunch ? ws.slots : nullptr, ws.counter,
+                           oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u, (typename Pol::T *)nullptr);
+    }
     if (grid > 1 && !oneLaunch)
         ND4J_LAUNCH((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n, ws.signal, ws.ticket);
 }

@@ -1172,10 +1172,37 @@ template <typename T>
 __global__ void __launch_bounds__(kBlock) isMaxFillKernel(T *z, const T *index, Long n, int strided, Long ews, DimMap zm) {
     typedef typename Compute<T>::type C;
     const Long hit = (Long)toCompute(index[0]);
+    if (strided && ews == 1) {
+        // a dense result: 16-byte stores between a head and a tail of single elements
+        constexpr int N = Pack<T>::N;
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(z);
+        Long head = ((addr & (sizeof(T) - 1)) == 0) ? (Long)(((16 - (addr & 15)) & 15) / sizeof(T)) : n;
+        if (head > n) head = n;
+        const Long nvec = (n - head) / N, gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
+        const T one = fromCompute<T>((C)1), zero = fromCompute<T>((C)0);
+        if (gtid < head) z[gtid] = gtid == hit ? one : zero;
+        Pack<T> *zv = reinterpret_cast<Pack<T> *>(z + head);
+        for (Long v = gtid; v < nvec; v += (Long)gridDim.x * kBlock) {
+            const Long i0 = head + v * N;
+            Pack<T> o;
+#pragma unroll
+            for (int e = 0; e < N; e++) o.v[e] = (i0 + e == hit) ? one : zero;
+            storePack(zv + v, o);
+        }
+        const Long tail = head + nvec * N;
+        if (gtid < n - tail) z[tail + gtid] = (tail + gtid == hit) ? one : zero;
+        return;
+    }
     for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock) {
         const Long o = strided ? i * ews : mapOffset64(zm, (unsigned long long)i);
         z[o] = fromCompute<T>(i == hit ? (C)1 : (C)0);
     }
+}
+// the second step after a clearing index reduction: the one element that is not zero
+template <typename T> __global__ void isMaxMarkKernel(T *z, const T *index, Long n) {
+    typedef typename Compute<T>::type C;
+    const Long hit = (Long)toCompute(index[0]);
+    if (threadIdx.x == 0 && blockIdx.x == 0 && hit >= 0 && hit < n) z[hit] = fromCompute<T>((C)1);
 }
 template <typename T>
 __global__ void __launch_bounds__(kBlock) isMaxTadFillKernel(T *z, const T *index, const Long *offsets, Long tadLength, Long numTads,
@@ -1254,8 +1281,13 @@ __global__ void __launch_bounds__(kBlock) isMaxColFillKernel(T *z, const T *inde
 
 template <typename T> void launchIsMaxFill(hipStream_t s, T *z, const T *index, const FlatPlan &zp) {
     if (zp.n <= 0) return;
+    // (the head and the tail of a dense result are written by the first threads of the grid: it never has fewer than 16)
     int grid = gridFor(zp.n, kBlock * 4, kGridCap);
     ND4J_LAUNCH((isMaxFillKernel<T>), dim3(grid), dim3(kBlock), 0, s, z, index, zp.n, zp.strided ? 1 : 0, zp.ews, zp.xm);
+}
+template <typename T> void launchIsMaxMark(hipStream_t s, T *z, const T *index, Long n) {
+    if (n <= 0) return;
+    ND4J_LAUNCH((isMaxMarkKernel<T>), dim3(1), dim3(64), 0, s, z, index, n);
 }
 template <typename T> void launchIsMaxTadFill(hipStream_t s, T *z, const T *index, const TadPlan &zt) {
     if (zt.numTads <= 0 || zt.tadLength <= 0) return;
@@ -1298,6 +1330,7 @@ template <typename T> void launchIsMaxTadFill(hipStream_t s, T *z, const T *inde
     template bool softmaxFitsRegisters<T>(const T *, const T *, const SoftmaxPlan &);                     \
     template bool launchSoftmaxFinish<T>(hipStream_t, int, const T *, T *, const T *, const Compute<T>::type *, const SoftmaxPlan &); \
     template void launchIsMaxFill<T>(hipStream_t, T *, const T *, const FlatPlan &);                      \
+    template void launchIsMaxMark<T>(hipStream_t, T *, const T *, Long);                                  \
     template void launchIsMaxTadFill<T>(hipStream_t, T *, const T *, const TadPlan &);
 INST(float)
 INST(float16)

@@ -146,6 +146,46 @@ def test_misaligned_buffers(gpu, cpu):
     dev.release()
 
 
+def test_ismax_whole_array_dense_operands(gpu, cpu):
+    # IsMax over a whole dense array finds the maximum and clears the result in one pass when x and z start on the same
+    # offset from a 16-byte boundary and are one array or two apart; otherwise in two.  Lengths around the vector and
+    # block sizes, operands 0..3 elements past a boundary, in place and out of place, ties, three types.
+    rs = np.random.RandomState(77)
+    dev = gpu.dev
+    pad = 16
+    for dt, name in ((np.float32, "Float"), (np.float64, "Double"), (np.float16, "Half")):
+        item = np.dtype(dt).itemsize
+        # (the winning index travels in the data type, as the index reductions store it: a half holds it up to 2048)
+        for n in ((1, 3, 4, 5, 8, 9, 1023, 2047) if dt == np.float16 else (1, 3, 4, 5, 1023, 4099, 70001, (1 << 20) + 7)):
+            # values the type holds exactly, the maximum twice: the first one wins
+            base = rs.randint(-1000, 1000, n + pad).astype(dt)
+            info = dev.upload(shape_info_np([1, n]))
+            for xo, zo, inplace in ((0, 0, False), (1, 1, False), (3, 3, False), (1, 2, False), (0, 3, False), (0, 0, True),
+                                    (2, 2, True)):
+                x = base.copy()
+                first = int(rs.randint(0, n))
+                x[xo + first] = 1500
+                if first + 2 < n:
+                    x[xo + first + 2] = 1500
+                X = dev.upload(x)
+                Z = X if inplace else dev.upload(np.full(n + pad, 7, dt))
+                getattr(gpu.ops, "execTransform" + name)(dev.extra(shape_info_np([1, n]), z_info=shape_info_np([1, n])), 41,
+                                                         X.ptr + item * xo, info.ptr, Z.ptr + item * zo, info.ptr, None)
+                got = Z.download(dt)
+                want = np.zeros(n, dt)
+                want[first] = 1
+                assert np.array_equal(got[zo:zo + n], want), (name, n, xo, zo, inplace)
+                if inplace:
+                    assert np.array_equal(got[:zo], x[:zo]) and np.array_equal(got[zo + n:], x[zo + n:]), (name, n, xo, zo)
+                else:
+                    assert np.all(got[:zo] == 7) and np.all(got[zo + n:] == 7), (name, n, xo, zo)
+                    assert np.array_equal(X.download(dt), x), ("input untouched", name, n, xo, zo)
+                    Z.free()
+                X.free()
+            info.free()
+    dev.release()
+
+
 def _dims_of(rank):
     for k in range(1, rank):
         for dims in itertools.combinations(range(rank), k):
