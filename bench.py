@@ -29,6 +29,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_FP32_PEAK_TFLOPS = 157.3  # dense fp32 on the matrix unit
 
 
 def parse():
@@ -307,6 +308,10 @@ def main():
                 if fetched:  # shapeInfo / dimension read-backs (each one a stream synchronisation)
                     row["host_fetches"] = int(fetched)
                 row["bound"] = getattr(c, "bound", "hbm")
+                if row["bound"] == "mfma":  # against the chip's dense fp32 matrix peak
+                    tflops = getattr(c, "flops", 0) / ms / 1e9
+                    row["mfma"] = {"achieved": round(tflops, 1), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                   "frac": round(tflops / MFMA_FP32_PEAK_TFLOPS, 4)}
                 v = valu_per_element(args.instructions, c.name)
                 if v is not None:
                     # a SIMD retires a wave64 fp32 instruction every 2 cycles at best (157.3 TFLOP/s of vector fp32 = 256 CUs x

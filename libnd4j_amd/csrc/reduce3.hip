@@ -10,6 +10,8 @@
 // run of y that starts at yOffsets[r % yMod] (null tables mean offset 0); element f of a run sits at
 // map(xm, f) / map(ym, f).  A whole-array call is a single output whose run is cut into slices that a second
 // kernel merges.
+#include <type_traits>
+
 #include "elementwise.cuh"
 #include "launch.h"
 #include "reduce_engine.cuh"
@@ -317,6 +319,110 @@ __global__ void __launch_bounds__(kBlock) reduce3AllTileKernel(const T *x, const
     }
 }
 
+// The dot product of every pair of runs is a matrix product, and so is the cross term of the two cosine ops: for float
+// arithmetic a block's four waves each keep a 32 x 32 quadrant of the 64 x 64 tile in the accumulator of the matrix
+// unit (v_mfma_f32_32x32x2_f32: lane l supplies x[row l % 32][k + l / 32] and y[col l % 32][k + l / 32], and holds the
+// results of column l % 32 in rows 8 * (v / 4) + 4 * (l / 32) + v % 4, v = 0 .. 15).  LDS holds the staged step with the
+// 64 runs' values of one k side by side, so that a wave's operand loads fall in consecutive banks; a staged element is
+// read from LDS once per quadrant instead of once per 4 x 4 patch, which is what bounded the vector-ALU tile kernel.
+// The operands of a step's 16 matrix instructions are fetched from LDS first, then the instructions follow each other.
+// The cosines' norms are sums per run, not per pair: every lane squares the operands it feeds, and the two lanes that
+// hold a run's even and odd k add up at the end.  A result sums its pairs in the matrix unit's order (pairs of k),
+// not one after the other as the reference's loop does: within the reductions' tolerance, not bit for bit.
+typedef float MfmaAcc __attribute__((ext_vector_type(16)));
+template <typename T, int OP>
+__global__ void __launch_bounds__(kBlock) reduce3AllMfmaKernel(const T *x, const T *y, T *z, const Long *xOffsets,
+                                                               const Long *yOffsets, Long nx, Long ny, Long length) {
+    static_assert(OP == 2 || OP == 3 || OP == 5, "dot and the cosines");
+    static_assert(kTileK == 32, "a step feeds 16 matrix instructions of two k each");
+    constexpr int TR = 64, S = TR + 2;             // 66 words per k: the four k groups of a staging wave fall on two bank halves
+    constexpr int PER = TR * kTileK / kBlock;      // staged elements per thread, run and step
+    constexpr int LANES_K = kTileK / PER;          // threads along a staged run
+    constexpr int N = Pack<T>::N, NP = PER / N;    // 16-byte vectors per thread, run and step
+    constexpr bool NORMS = OP != 3;
+    __shared__ float xs[kTileK][S];
+    __shared__ float ys[kTileK][S];
+    const Long tilesY = (ny + TR - 1) / TR;
+    const Long tileX = blockIdx.x / tilesY, tileY = blockIdx.x - tileX * tilesY;
+    const Long row0 = tileX * TR, col0 = tileY * TR;
+    const int sRun = threadIdx.x / LANES_K, sK = (threadIdx.x % LANES_K) * PER;
+    const T *xRun = row0 + sRun < nx ? x + xOffsets[row0 + sRun] : nullptr;
+    const T *yRun = col0 + sRun < ny ? y + yOffsets[col0 + sRun] : nullptr;
+    // A tile whose 128 runs all exist, start on 16-byte boundaries and hold whole steps is staged with plain vector
+    // loads.  The general staging decides per thread and step between zeros, a vector and single elements, and those
+    // decisions run on the compute unit's one scalar unit, which its sixteen waves share.
+    const bool plainRun = xRun != nullptr && yRun != nullptr && (reinterpret_cast<uintptr_t>(xRun) & 15) == 0 &&
+                          (reinterpret_cast<uintptr_t>(yRun) & 15) == 0;
+    const bool plain = __builtin_amdgcn_readfirstlane(__syncthreads_and(plainRun && length % kTileK == 0 ? 1 : 0)) != 0;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int wi = wave / 2, wj = wave % 2, half = lane / 32, col = lane % 32;
+    MfmaAcc acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+    float e0 = 0.0f, e1 = 0.0f;
+
+    TileStage<T, PER> sx, sy;
+    auto fetch = [&](Long k) {
+        if (plain) {
+            const Pack<T> *px = reinterpret_cast<const Pack<T> *>(xRun + k + sK), *py = reinterpret_cast<const Pack<T> *>(yRun + k + sK);
+#pragma unroll
+            for (int q = 0; q < NP; q++) {
+                const Pack<T> vx = px[q], vy = py[q];
+#pragma unroll
+                for (int e = 0; e < N; e++) {
+                    sx.v[q * N + e] = toCompute(vx.v[e]);
+                    sy.v[q * N + e] = toCompute(vy.v[e]);
+                }
+            }
+        } else {
+            // (elements beyond the end of a run, and runs beyond the last, come as zeros: they add nothing)
+            sx.load(xRun, k + sK, length);
+            sy.load(yRun, k + sK, length);
+        }
+    };
+    fetch(0);
+    for (Long k0 = 0; k0 < length; k0 += kTileK) {
+#pragma unroll
+        for (int e = 0; e < PER; e++) {
+            xs[sK + e][sRun] = sx.v[e];
+            ys[sK + e][sRun] = sy.v[e];
+        }
+        __syncthreads();
+        if (k0 + kTileK < length) fetch(k0 + kTileK);  // the next step's elements travel while this step is computed
+        float a[16], b[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            a[i] = xs[2 * i + half][wi * 32 + col];
+            b[i] = ys[2 * i + half][wj * 32 + col];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[i], acc, 0, 0, 0);
+            if (NORMS) {
+                e0 = __builtin_fmaf(a[i], a[i], e0);
+                e1 = __builtin_fmaf(b[i], b[i], e1);
+            }
+        }
+        __syncthreads();
+    }
+    if (NORMS) {
+        e0 += __shfl_xor(e0, 32, kWave);  // row wi * 32 + lane % 32 of x
+        e1 += __shfl_xor(e1, 32, kWave);  // column wj * 32 + lane % 32 of y
+    }
+    const Long g = col0 + wj * 32 + col;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const int m = 8 * (v / 4) + 4 * half + v % 4;
+        Acc3<float> a3;
+        a3.r = acc[v];
+        a3.e0 = NORMS ? __shfl(e0, m, kWave) : 0.0f;
+        a3.e1 = e1;
+        const Long r = row0 + wi * 32 + m;
+        if (r < nx && g < ny) z[r * ny + g] = fromCompute<T>(Reduce3Op<float, OP>::finalize(a3, length));
+    }
+}
+
 template <typename T> struct Reduce3Body {
     template <int OP> struct Run {
         static bool run(hipStream_t s, const T *x, const T *y, T *z, const T *extra, const Reduce3Plan &pl, Workspace ws) {
@@ -327,6 +433,13 @@ template <typename T> struct Reduce3Body {
                 pl.numOut / pl.yMod >= 16 && pl.runLength >= 8) {
                 const Long nx = pl.numOut / pl.yMod, ny = pl.yMod;
                 const Long tiles64 = ((nx + 63) / 64) * ((ny + 63) / 64), tiles32 = ((nx + 31) / 32) * ((ny + 31) / 32);
+                if constexpr ((OP == 2 || OP == 3 || OP == 5) && std::is_same<typename Compute<T>::type, float>::value) {
+                    if (tiles64 >= 512 && tiles64 <= kMaxGrid) {
+                        ND4J_LAUNCH((reduce3AllMfmaKernel<T, OP>), dim3((unsigned)tiles64), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
+                                           pl.yOffsets, nx, ny, pl.runLength);
+                        return true;
+                    }
+                }
                 if (tiles64 >= 512 && tiles64 <= kMaxGrid) {
                     ND4J_LAUNCH((reduce3AllTileKernel<T, OP, 64>), dim3((unsigned)tiles64), dim3(kBlock), 0, s, x, y, z, extra,
                                        pl.xOffsets, pl.yOffsets, nx, ny, pl.runLength);

@@ -44,7 +44,7 @@ class Case(object):
         self.cpu = cpu
         self.contiguous = contiguous
         self.note = None  # printed beside the case by the benchmark
-        self.bound = "hbm"  # what limits the case: "hbm", or "valu" when instruction issue does
+        self.bound = "hbm"  # what limits the case: "hbm", "valu" when instruction issue does, "mfma" (with `flops` set) for the matrix unit
         self.cpu_once = False  # the benchmark times a single cold CPU pass of this case
 
     @property
@@ -297,7 +297,7 @@ def reduce3_pairs(dev, rows=16384, cols=4096, seed=12, copies=None):
         # every row of a [2048,1024] piece of x (its first 2 Mi elements) against every row of the same piece of y: 2048 x 2048
         # dot products.
         # Not a streaming case: each operand is read from HBM once and reused from LDS (its "bytes" are the 16 MiB of
-        # operands and the 16 MiB of results), so what bounds it is the vector ALUs; `elements` counts the pairs.
+        # operands and the 16 MiB of results): a matrix product, bound by the matrix unit; `elements` counts the pairs.
         ar, al = min(2048, rows), min(1024, cols)
         ai, azi = harness.shape_info([ar, al]), harness.shape_info([ar, ar])
         ZA = w.operand(np.zeros(ar * ar, F32), azi)
@@ -308,8 +308,9 @@ def reduce3_pairs(dev, rows=16384, cols=4096, seed=12, copies=None):
                     lambda: ops.execReduce3AllFloat(ex_a, 3, X.ptr, AI.ptr, None, Y.ptr, AI.ptr, ZA.ptr, ZA.info_ptr, D.ptr, 1, ex_a[10],
                                                     ex_a[11], ex_a[10], ex_a[11]),
                     lambda lib: (lib.reduce3_all(3, x[:ar * al], ai, y[:ar * al], ai, za, azi, [1], None), za)[1], True, ZA.get)
-        case.note = "compute-bound: %.0f G pairs, fp32 FMA on the vector ALUs" % (ar * ar * al / 1e9)
-        case.bound = "valu"
+        case.note = "compute-bound: %.0f G pairs, fp32 on the matrix unit (v_mfma_f32_32x32x2_f32)" % (ar * ar * al / 1e9)
+        case.bound = "mfma"
+        case.flops = 2 * ar * ar * al  # a multiplication and an addition per pair
         case.cpu_once = True  # one pass of the reference takes seconds
         cases.append(case)
         return cases

@@ -391,7 +391,10 @@ def test_reduce3_family(gpu, cpu):
         close(gpu.reduce3_all(op, x, xi, y, yi, None, [1], 6), cpu.reduce3_all(op, x, xi, y, yi, None, [1], 6), ("long all", op))
     # enough pairs for the tiled kernel: ragged tile edges, a run length that ends inside a staged step, misaligned runs
     # (the last shape has enough 64 x 64 tiles for the larger tile; the others run 32 x 32 ones)
-    for (nx, ny, length) in ((70, 33, 100), (64, 128, 256), (17, 16, 9), (130, 65, 1027), (1450, 1420, 43)):
+    # (the last three shapes have enough 64 x 64 tiles for the larger tile, which for dot and the cosines is the matrix-unit
+    # kernel: ragged runs that end inside a step, whole aligned runs, and whole runs with ragged tile edges)
+    for (nx, ny, length) in ((70, 33, 100), (64, 128, 256), (17, 16, 9), (130, 65, 1027), (1450, 1420, 43), (1536, 1408, 96),
+                             (1500, 1480, 64)):
         xi, yi = shape_info_np([nx, length]), shape_info_np([ny, length])
         x, y = rs.uniform(0.1, 2, nx * length).astype(np.float32), rs.uniform(0.1, 2, ny * length).astype(np.float32)
         x64, y64 = x.astype(np.float64).reshape(nx, length), y.astype(np.float64).reshape(ny, length)
@@ -400,6 +403,14 @@ def test_reduce3_family(gpu, cpu):
             close(got, cpu.reduce3_all(op, x, xi, y, yi, None, [1], nx * ny), ("tiled all", nx, ny, length, op))
         dots = x64 @ y64.T
         assert np.allclose(gpu.reduce3_all(3, x, xi, y, yi, None, [1], nx * ny).reshape(nx, ny), dots, rtol=1e-5)
+        norms = np.sqrt((x64 * x64).sum(axis=1))[:, None] * np.sqrt((y64 * y64).sum(axis=1))[None, :]
+        assert np.allclose(gpu.reduce3_all(2, x, xi, y, yi, None, [1], nx * ny).reshape(nx, ny), dots / norms, rtol=1e-5)
+        assert np.allclose(gpu.reduce3_all(5, x, xi, y, yi, None, [1], nx * ny).reshape(nx, ny), 1 - dots / norms, rtol=1e-4, atol=1e-6)
+        if nx * ny > 100000:
+            xh, yh = x.astype(np.float16), y.astype(np.float16)
+            doth = xh.astype(np.float64).reshape(nx, length) @ yh.astype(np.float64).reshape(ny, length).T
+            goth = gpu.reduce3_all(3, xh, xi, yh, yi, None, [1], nx * ny).astype(np.float64).reshape(nx, ny)
+            assert np.allclose(goth, doth, rtol=2e-3), ("half dots", nx, ny, length)
         # with the caller's TAD tables (nothing is read back from the device then)
         before = gpu.ops.amd_hostFetchCount()
         assert np.allclose(gpu.reduce3_all(3, x, xi, y, yi, None, [1], nx * ny, pass_tads=True).reshape(nx, ny), dots, rtol=1e-5)
