@@ -328,6 +328,31 @@ __global__ void __launch_bounds__(kBlock) randomLeanKernel(RandomCtx<TT> c, cons
     const Long first = (Long)blockIdx.x * perBlock;
     RngBlockWalk w = rngBlockWalk(c.st, first);
     const unsigned count = (unsigned)(c.length - first < perBlock ? c.length - first : perBlock);
+    if constexpr (UNIT && sizeof(TT) == 4) {
+        // dense 4-byte operands on 16-byte boundaries: a thread draws four neighbouring elements and moves them as one vector
+        const bool aligned = ((reinterpret_cast<uintptr_t>(z) | (NOPS >= 2 ? reinterpret_cast<uintptr_t>(x) : 0) |
+                               (NOPS >= 3 ? reinterpret_cast<uintptr_t>(y) : 0)) & 15) == 0 && perBlock % 4 == 0;
+        if (aligned) {
+            for (unsigned o = threadIdx.x * 4; o < count; o += kBlock * 4) {
+                const Long i = first + o;
+                if (o + 4 <= count) {
+                    Pack<TT> xv, yv, out;
+                    if (NOPS >= 2) xv = loadPack(reinterpret_cast<const Pack<TT> *>(x + i));
+                    if (NOPS >= 3) yv = loadPack(reinterpret_cast<const Pack<TT> *>(y + i));
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        out.v[e] = fromCompute<TT>(randomOp<OP, TT>(c, NOPS, NOPS >= 2 ? toCompute(xv.v[e]) : (C)0,
+                                                                    NOPS >= 3 ? toCompute(yv.v[e]) : (C)0, i + e, w));
+                    storePack(reinterpret_cast<Pack<TT> *>(z + i), out);
+                } else {
+                    for (unsigned e = o; e < count; e++)
+                        z[first + e] = fromCompute<TT>(randomOp<OP, TT>(c, NOPS, NOPS >= 2 ? toCompute(x[first + e]) : (C)0,
+                                                                        NOPS >= 3 ? toCompute(y[first + e]) : (C)0, first + e, w));
+                }
+            }
+            return;
+        }
+    }
     for (unsigned o = threadIdx.x; o < count; o += kBlock) {
         const Long i = first + o;
         const C xv = NOPS >= 2 ? toCompute(x[UNIT ? i : i * xEws]) : (C)0;
