@@ -391,10 +391,11 @@ def test_reduce3_family(gpu, cpu):
         close(gpu.reduce3_all(op, x, xi, y, yi, None, [1], 6), cpu.reduce3_all(op, x, xi, y, yi, None, [1], 6), ("long all", op))
     # enough pairs for the tiled kernel: ragged tile edges, a run length that ends inside a staged step, misaligned runs
     # (the last shape has enough 64 x 64 tiles for the larger tile; the others run 32 x 32 ones)
-    # (the last three shapes have enough 64 x 64 tiles for the larger tile, which for dot and the cosines is the matrix-unit
-    # kernel: ragged runs that end inside a step, whole aligned runs, and whole runs with ragged tile edges)
+    # (from the fifth shape on there are enough 64 x 64 tiles for the larger tile, which for dot and the cosines is the
+    # matrix-unit kernel: ragged runs that end inside a step, whole aligned runs, and whole runs with ragged tile edges; the
+    # last two have enough 64 x 128 tiles for its wider form, ragged and whole)
     for (nx, ny, length) in ((70, 33, 100), (64, 128, 256), (17, 16, 9), (130, 65, 1027), (1450, 1420, 43), (1536, 1408, 96),
-                             (1500, 1480, 64)):
+                             (1500, 1480, 64), (2100, 2000, 70), (2048, 2048, 64)):
         xi, yi = shape_info_np([nx, length]), shape_info_np([ny, length])
         x, y = rs.uniform(0.1, 2, nx * length).astype(np.float32), rs.uniform(0.1, 2, ny * length).astype(np.float32)
         x64, y64 = x.astype(np.float64).reshape(nx, length), y.astype(np.float64).reshape(ny, length)
@@ -416,9 +417,10 @@ def test_reduce3_family(gpu, cpu):
         assert np.allclose(gpu.reduce3_all(3, x, xi, y, yi, None, [1], nx * ny, pass_tads=True).reshape(nx, ny), dots, rtol=1e-5)
         assert gpu.ops.amd_hostFetchCount() == before
         if nx * ny > 100000:
-            xd, yd = rs.randn(nx * length), rs.randn(ny * length)
-            assert np.allclose(gpu.reduce3_all(1, xd, xi, yd, yi, None, [1], nx * ny).reshape(nx, ny),
-                               np.sqrt(((xd.reshape(nx, 1, length) - yd.reshape(1, ny, length)) ** 2).sum(axis=2)), rtol=1e-12)
+            if nx * ny * length < 100000000:  # (the check's own temporary holds nx * ny * length doubles)
+                xd, yd = rs.randn(nx * length), rs.randn(ny * length)
+                assert np.allclose(gpu.reduce3_all(1, xd, xi, yd, yi, None, [1], nx * ny).reshape(nx, ny),
+                                   np.sqrt(((xd.reshape(nx, 1, length) - yd.reshape(1, ny, length)) ** 2).sum(axis=2)), rtol=1e-12)
             continue
         # EqualsWithEps counts the pairs that differ: elements staged beyond the end of a run must not be counted
         y2 = x[:ny * length].copy() if nx >= ny else np.resize(x, ny * length)
