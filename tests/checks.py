@@ -46,7 +46,8 @@ def assert_reduction_close(got, want, scale, what, rtol=REDUCE_RTOL):
     want = np.asarray(want, dtype=np.float64)
     assert np.array_equal(np.isnan(got), np.isnan(want)), "%s: NaN pattern differs" % what
     bound = rtol * np.maximum(np.abs(want), scale)
-    err = np.abs(got - want)
+    with np.errstate(invalid="ignore"):  # equal infinities subtract to NaN; `got == want` accepts them below
+        err = np.abs(got - want)
     ok = (err <= bound) | (np.isnan(want)) | (got == want)
     assert ok.all(), "%s: |err| %g > bound %g at %d (got %r want %r)" % (
         what, err[~ok].max(), bound[~ok][0], int(np.nonzero(~ok)[0][0]), got[~ok][0], want[~ok][0])
