@@ -14,8 +14,11 @@ last-level cache).  The line printed at the end is one JSON object:
              the timed loop, against 8 TB/s
   cpu_baseline  the same step on the host cores (compiled reference loops when oracle/_ref is present, else
              this repository's CPU restatement), a bounded sample
-  families   (with --families) every op family of the other configurations, each timed with HIP events over
-             K back-to-back launches, with its CPU time next to it
+  families   every case of the other configurations as {case: [ms per launch, fraction of 8 TB/s]}, each timed with
+             HIP events over K back-to-back launches (--no-families leaves them out)
+
+The printed line stays under 4 KB.  The full family rows (GB/s, elements/s, CPU time of the same case, measured HBM
+traffic, vector-instruction figures, notes) go to stderr as a table and to the file named by --families-out.
 
 Inputs are synthetic (seeded numpy generators); nothing is read from disk.
 """
@@ -42,8 +45,10 @@ def parse():
     ap.add_argument("--families-cpu-seconds", type=float, default=25.0,
                     help="total budget of the CPU passes beside the family rows; cases left over when it is spent get no "
                          "CPU column")
+    ap.add_argument("--families-out", default=os.path.join(ROOT, "gpurun_out", "bench_families.json"),
+                    help="file that receives the full family rows (the printed line carries [ms, frac] per case only)")
     ap.add_argument("--only", default="", help="with --families: comma-separated workload builders to run "
-                                               "(transform,pairwise,half,reductions,reduce3,stats,random,movement)")
+                                               "(transform,pairwise,half,reductions,reduce3,stats,views,random,movement,whole)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU sample of the headline step")
     ap.add_argument("--counters", action="store_true",
@@ -132,7 +137,7 @@ def family_builders(workloads):
     return [("transform", workloads.transform_tanh), ("pairwise", lambda d: workloads.pairwise_broadcast(d, copies=2)),
             ("half", lambda d: workloads.pairwise_broadcast(d, dtype="float16")),
             ("reductions", workloads.reductions), ("reduce3", workloads.reduce3_pairs),
-            ("stats", workloads.stats_softmax), ("random", workloads.random_fills),
+            ("stats", workloads.stats_softmax), ("views", workloads.general_views), ("random", workloads.random_fills),
             ("movement", workloads.data_movement), ("whole", workloads.whole_array_transforms)]
 
 
@@ -175,6 +180,31 @@ def cpu_time(fn, lib, budget_s, min_runs=3, max_runs=5000):
         times.append(time.perf_counter() - t0)
     times.sort()
     return times[len(times) // 2], len(times)
+
+
+MAX_LINE_BYTES = 6000  # whoever runs this keeps only the last 8000 bytes of stdout: the result line must fit with room to spare
+
+
+def result_line(out, family_rows):
+    """The one line printed on stdout: the headline object plus, per family case, [ms per launch, fraction of the HBM
+    peak].  Raises when it would not fit in MAX_LINE_BYTES."""
+    line = dict(out)
+    if family_rows is not None:
+        line["families"] = {r["case"]: [r["ms"], round(r["frac"], 3)] for r in family_rows}
+    text = json.dumps(line, separators=(",", ":"))
+    if len(text) >= MAX_LINE_BYTES:
+        raise RuntimeError("the result line has grown to %d bytes (limit %d)" % (len(text), MAX_LINE_BYTES))
+    return text
+
+
+def write_family_rows(path, out, family_rows):
+    """The full rows, beside the headline they belong to; a directory that cannot be written is reported, not fatal."""
+    try:
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        with open(path, "w") as f:
+            json.dump({"headline": out, "families": family_rows}, f, indent=1)
+    except OSError as e:
+        print("bench.py: could not write %s: %s" % (path, e), file=sys.stderr)
 
 
 def main():
@@ -354,8 +384,10 @@ def main():
                     "   (%d read-backs from the device)" % fetched if fetched else "") + ("   [%s]" % c.note if c.note else ""),
                     file=sys.stderr, flush=True)
             wl.free()
-        out["families"] = fam
-    print(json.dumps(out), flush=True)
+        write_family_rows(args.families_out, out, fam)
+        print(result_line(out, fam), flush=True)
+        return 0
+    print(result_line(out, None), flush=True)
     return 0
 
 

@@ -427,6 +427,80 @@ def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
                        dict(x=x, xi=xi, softmax_cpu=tc), device_set, copies)
 
 
+# ---- general views: multi-dimensional TADs, broadcasts over several dimensions, padded views --------------------------
+def general_views(dev, seed=61, copies=None):
+    """What nd4j's everyday multi-dimensional calls look like to the loops: TADs over several dimensions (their
+    shapeInfo carries no element-wise stride, whatever their layout), broadcasts of a sub-array, and views with a row
+    pitch.  A batch-norm style sum / variance over dimensions {0,2,3} of an NCHW array [128,128,56,56]; argmax over
+    dimensions {1,2} of [4096,128,128]; add of a [56,56] plane along dimensions {2,3} of the NCHW array and of a
+    [256,256] matrix along dimensions {0,2} of [256,1024,256]; pairwise add and exp on a [65536,1024] view whose rows
+    are 1032 elements apart."""
+    rs = np.random.default_rng(seed)
+    ops = dev.ops
+    nchw, cube, slab = [128, 128, 56, 56], [4096, 128, 128], [256, 1024, 256]
+    n1, n2, n3 = int(np.prod(nchw)), int(np.prod(cube)), int(np.prod(slab))
+    x1, x2, x3 = _normal(rs, n1, F32), _normal(rs, n2, F32), _normal(rs, n3, F32)
+    i1, i2, i3 = harness.shape_info(nchw), harness.shape_info(cube), harness.shape_info(slab)
+    plane, mat = _uniform(rs, 56 * 56, -1, 1), _uniform(rs, 256 * 256, -1, 1)
+    pi, mi = harness.shape_info([56, 56]), harness.shape_info([256, 256])
+    rows, cols, pitch = 65536, 1024, 1032
+    vi = harness.shape_info([rows, cols], strides=[pitch, 1])
+    nv, span = rows * cols, harness.span_of(vi)
+    xv, yv = _normal(rs, span, F32), _normal(rs, span, F32)
+    tad1_023, tad1_23 = dev.tad(i1, [0, 2, 3]), dev.tad(i1, [2, 3])
+    tad2_12, tad3_02 = dev.tad(i2, [1, 2]), dev.tad(i3, [0, 2])
+    c_out, r_out = _vec(nchw[1]), _vec(cube[0])
+    zc1, zc2, zc3 = np.zeros(n1, F32), np.zeros(n3, F32), np.zeros(span, F32)
+    oc1, oc2 = np.zeros(nchw[1], F32), np.zeros(cube[0], F32)
+
+    def device_set(w):
+        cases = []
+        X1, Z1 = w.operand(x1, i1), w.operand(np.zeros(n1, F32), i1)
+        C = w.operand(np.zeros(nchw[1], F32), c_out)
+        D023, D23 = w.raw(np.array([0, 2, 3], np.int32)), w.raw(np.array([2, 3], np.int32))
+        ex = dev.extra(i1, z_info=c_out, tad=tad1_023)
+        cases.append(Case("sum_nchw_dims023", "reduce", n1, 4 * n1 + 4 * nchw[1],
+                          lambda: ops.execReduceFloat(ex, R_SUM, X1.ptr, X1.info_ptr, None, C.ptr, C.info_ptr, D023.ptr, 3),
+                          lambda lib: (lib.reduce(R_SUM, x1, i1, None, oc1, c_out, [0, 2, 3]), oc1)[1], False, C.get))
+        cases.append(Case("variance_nchw_dims023", "summarystats", n1, 4 * n1 + 4 * nchw[1],
+                          lambda: ops.execSummaryStatsFloat(ex, S_VAR, X1.ptr, X1.info_ptr, None, C.ptr, C.info_ptr, D023.ptr, 3, 1),
+                          lambda lib: (lib.summarystats(S_VAR, 1, x1, i1, oc1, c_out, [0, 2, 3]), oc1)[1], False, C.get))
+        P = w.operand(plane, pi)
+        ex_b = dev.extra(i1, pi, i1, tad=tad1_23, tad_z=tad1_23)
+        cases.append(Case("broadcast_add_nchw_dims23", "broadcast", n1, 8 * n1 + 4 * plane.size,
+                          lambda: ops.execBroadcastFloat(ex_b, B_ADD, X1.ptr, X1.info_ptr, P.ptr, P.info_ptr, Z1.ptr, Z1.info_ptr, D23.ptr, 2),
+                          lambda lib: (lib.broadcast(B_ADD, x1, i1, plane, pi, zc1, i1, [2, 3]), zc1)[1], False, Z1.get))
+        X2 = w.operand(x2, i2)
+        R = w.operand(np.zeros(cube[0], F32), r_out)
+        D12 = w.raw(np.array([1, 2], np.int32))
+        ex2 = dev.extra(i2, z_info=r_out, tad=tad2_12)
+        cases.append(Case("argmax_cube_dims12", "indexreduce", n2, 4 * n2 + 4 * cube[0],
+                          lambda: ops.execIndexReduceFloat(ex2, I_MAX, X2.ptr, X2.info_ptr, None, R.ptr, R.info_ptr, D12.ptr, 2),
+                          lambda lib: (lib.indexreduce(I_MAX, x2, i2, None, oc2, r_out, [1, 2]), oc2)[1], False, R.get))
+        X3, Z3 = w.operand(x3, i3), w.operand(np.zeros(n3, F32), i3)
+        M = w.operand(mat, mi)
+        D02 = w.raw(np.array([0, 2], np.int32))
+        ex3 = dev.extra(i3, mi, i3, tad=tad3_02, tad_z=tad3_02)
+        cases.append(Case("broadcast_add_slab_dims02", "broadcast", n3, 8 * n3 + 4 * mat.size,
+                          lambda: ops.execBroadcastFloat(ex3, B_ADD, X3.ptr, X3.info_ptr, M.ptr, M.info_ptr, Z3.ptr, Z3.info_ptr, D02.ptr, 2),
+                          lambda lib: (lib.broadcast(B_ADD, x3, i3, mat, mi, zc2, i3, [0, 2]), zc2)[1], False, Z3.get))
+        XV, YV, ZV = w.operand(xv, vi), w.operand(yv, vi), w.operand(np.zeros(span, F32), vi)
+        exv = dev.extra(vi, vi, vi)
+        cases.append(Case("pairwise_add_padded_rows", "pairwise", nv, 12 * nv,
+                          lambda: ops.execPairwiseTransformFloat(exv, P_ADD, XV.ptr, XV.info_ptr, YV.ptr, YV.info_ptr, ZV.ptr, ZV.info_ptr, None),
+                          lambda lib: (lib.pairwise(P_ADD, xv, vi, yv, vi, zc3, vi, None), zc3)[1], False, ZV.get))
+        cases.append(Case("transform_exp_padded_rows", "transform", nv, 8 * nv,
+                          lambda: ops.execTransformFloat(exv, T_EXP, XV.ptr, XV.info_ptr, ZV.ptr, ZV.info_ptr, None),
+                          lambda lib: (lib.transform(T_EXP, xv, vi, zc3, vi, None), zc3)[1], False, ZV.get))
+        for c in cases:
+            c.cpu_once = True  # the reference walks these element by element through coordinate arithmetic: a pass takes long
+        return cases
+
+    return _replicated(dev, "general views: multi-dimensional TADs on [128,128,56,56] / [4096,128,128] / [256,1024,256], rows with a pitch",
+                       4 * n1 + 4 * n2 + 8 * n3, dict(x1=x1, i1=i1, x2=x2, i2=i2, x3=x3, i3=i3, plane=plane, pi=pi, mat=mat, mi=mi,
+                                                      xv=xv, yv=yv, vi=vi), device_set, copies)
+
+
 # ---- data-movement specials: gathers, concatenations, reorders, conversions ---------------------------------
 def data_movement(dev, rows=65536, cols=1024, seed=31, copies=None):
     import ctypes
