@@ -41,6 +41,39 @@ template <typename T> __device__ __forceinline__ void storePack(Pack<T> *p, cons
     __builtin_nontemporal_store(__builtin_bit_cast(U32x4, v), reinterpret_cast<U32x4 *>(p));
 }
 
+// 16 bytes at an address that is only aligned to the element size: the hardware serves misaligned global accesses
+// (slower than aligned ones where they straddle cache lines, far faster than element-wise accesses).
+typedef U32x4 U32x4A2 __attribute__((aligned(2)));
+typedef U32x4 U32x4A4 __attribute__((aligned(4)));
+typedef U32x4 U32x4A8 __attribute__((aligned(8)));
+template <typename T> __device__ __forceinline__ Pack<T> loadPackAnywhere(const T *p) {
+    U32x4 v;
+    if (sizeof(T) == 2) v = *reinterpret_cast<const U32x4A2 *>(p);
+    else if (sizeof(T) == 4) v = *reinterpret_cast<const U32x4A4 *>(p);
+    else v = *reinterpret_cast<const U32x4A8 *>(p);
+    return __builtin_bit_cast(Pack<T>, v);
+}
+template <typename T> __device__ __forceinline__ void storePackAnywhere(T *p, const Pack<T> &a) {
+    const U32x4 v = __builtin_bit_cast(U32x4, a);
+    if (sizeof(T) == 2) *reinterpret_cast<U32x4A2 *>(p) = v;
+    else if (sizeof(T) == 4) *reinterpret_cast<U32x4A4 *>(p) = v;
+    else *reinterpret_cast<U32x4A8 *>(p) = v;
+}
+// the same with the streaming cache policy of loadPack / storePack
+template <typename T> __device__ __forceinline__ Pack<T> streamPackAnywhere(const T *p) {
+    U32x4 v;
+    if (sizeof(T) == 2) v = __builtin_nontemporal_load(reinterpret_cast<const U32x4A2 *>(p));
+    else if (sizeof(T) == 4) v = __builtin_nontemporal_load(reinterpret_cast<const U32x4A4 *>(p));
+    else v = __builtin_nontemporal_load(reinterpret_cast<const U32x4A8 *>(p));
+    return __builtin_bit_cast(Pack<T>, v);
+}
+template <typename T> __device__ __forceinline__ void streamPackAnywhere(T *p, const Pack<T> &a) {
+    const U32x4 v = __builtin_bit_cast(U32x4, a);
+    if (sizeof(T) == 2) __builtin_nontemporal_store(v, reinterpret_cast<U32x4A2 *>(p));
+    else if (sizeof(T) == 4) __builtin_nontemporal_store(v, reinterpret_cast<U32x4A4 *>(p));
+    else __builtin_nontemporal_store(v, reinterpret_cast<U32x4A8 *>(p));
+}
+
 // Functor adapters: apply(a, b, params)
 template <int OP> struct TransformF {
     static constexpr int nin = 1;
@@ -430,6 +463,61 @@ __global__ void __launch_bounds__(kBlock) bcGeneralKernel(const T *x, DimMap xm,
     }
 }
 
+// Views that are made of contiguous runs: every operand's index -> offset map ends in a dimension of stride 1 whose extent
+// is a multiple of runLength (the padded rows of a view with a pitch; the TADs of a broadcast over several dimensions).
+// The element space is cut into units of one 16-byte vector inside a run (the last unit of a run is shorter when
+// runLength is not a multiple of the vector width); a thread takes one unit, finds its place through each operand's map
+// once - divisions per vector, not per element - and moves it with 16-byte accesses that need no alignment beyond the
+// element's own.  xOffsets / zOffsets (null: one "TAD" at offset 0) add a per-TAD offset, y is shared by all TADs.
+// Units are numbered run by run inside a TAD (runMajor 0), or with the same run of all TADs side by side (runMajor 1):
+// whichever makes neighbouring threads touch neighbouring memory.
+template <typename T, typename F>
+__global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, const T *y, DimMap ym, T *z, DimMap zm,
+                                                       const Long *xOffsets, const Long *zOffsets, Params<T> p, Long numTads,
+                                                       unsigned tadLength, unsigned runLength, int runMajor) {
+    typedef typename Compute<T>::type C;
+    if (F::tables) lm::loadTables();
+    constexpr int VEC = Pack<T>::N;
+    const unsigned unitsPerRun = (runLength + VEC - 1) / VEC;
+    const unsigned runsPerTad = tadLength / runLength;
+    const Long total = numTads * ((Long)runsPerTad * unitsPerRun);
+    const bool small = total <= 0xffffffffLL;
+    for (Long g = (Long)blockIdx.x * kBlock + threadIdx.x; g < total; g += (Long)gridDim.x * kBlock) {
+        // g -> (TAD r, run m of the TAD, unit c of the run)
+        Long r;
+        unsigned m, c;
+        if (small) {
+            const unsigned t = (unsigned)g / unitsPerRun;
+            c = (unsigned)g - t * unitsPerRun;
+            if (runMajor) { m = t / (unsigned)numTads; r = t - m * (unsigned)numTads; }
+            else { const unsigned q = t / runsPerTad; m = t - q * runsPerTad; r = q; }
+        } else {
+            const Long t = g / unitsPerRun;
+            c = (unsigned)(g - t * unitsPerRun);
+            if (runMajor) { m = (unsigned)(t / numTads); r = t - (Long)m * numTads; }
+            else { r = t / runsPerTad; m = (unsigned)(t - r * runsPerTad); }
+        }
+        const unsigned f0 = m * runLength + c * VEC;  // index of the unit's first element inside its TAD
+        const unsigned count = runLength - c * VEC;   // elements left in the run from there on
+        const T *xp = x + (xOffsets != nullptr ? xOffsets[r] : 0) + mapOffset32(xm, f0);
+        T *zp = z + (zOffsets != nullptr ? zOffsets[r] : 0) + mapOffset32(zm, f0);
+        const T *yp = F::nin == 2 ? y + mapOffset32(ym, f0) : nullptr;
+        if (count >= VEC) {
+            const Pack<T> a = streamPackAnywhere(xp);
+            Pack<T> b;
+            if (F::nin == 2) b = loadPackAnywhere(yp);
+            Pack<T> o;
+#pragma unroll
+            for (int e = 0; e < VEC; e++)
+                o.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), F::nin == 2 ? toCompute(b.v[e]) : (C)0, p));
+            streamPackAnywhere(zp, o);
+        } else {
+            for (unsigned e = 0; e < count; e++)
+                zp[e] = fromCompute<T>(F::template apply<C>(toCompute(xp[e]), F::nin == 2 ? toCompute(yp[e]) : (C)0, p));
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Host-side launch helpers.
 
@@ -607,6 +695,16 @@ inline void launchGeneral(hipStream_t s, const T *x, const DimMap &xm, const T *
     }
     Params<T> p{extra};
     p.scalar = scalar;
+    // rows with a pitch and the like: contiguous runs along the innermost dimension of every operand
+    const DimMap *const maps[3] = {&xm, two ? &ym : nullptr, &zm};
+    const unsigned run = commonRunLength(maps);
+    if (run >= (unsigned)Pack<T>::N && n <= 0x7fffffffLL) {
+        const Long units = n / run * ((run + Pack<T>::N - 1) / Pack<T>::N);
+        ND4J_LAUNCH((ewRunsKernel<T, F>), dim3(gridFor(units, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0, s, x, xm,
+                           two ? y : x, two ? ym : xm, z, zm, (const Long *)nullptr, (const Long *)nullptr, p, (Long)1, (unsigned)n,
+                           run, 0);
+        return;
+    }
     int grid = gridFor(n, kBlock * 4, kGridCap);
     ND4J_LAUNCH((ewGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, xm, two ? y : x, two ? ym : xm, z, zm,
                        p, n);

@@ -45,6 +45,8 @@ struct BroadcastPlan {
     bool consecutive = false;    // ROW only: TAD r starts at r * tadLength in x and in z (rows of a dense c-order array)
     bool denseAlike = false;     // ROW / COL: x and z are dense arrays of one layout, y is contiguous: memory position i of
                                  // either takes y[(i / tadEws) % tadLength]
+    unsigned runLength = 0;      // GENERAL only, 0 = not applicable: the three maps end in contiguous runs of this many elements
+    bool runMajor = false;       //   ... and the same run of neighbouring TADs is nearer in memory than the next run of one TAD
     Long flatInner = 0, flatExtent = 0;  // per-TAD scalars over dense x and z of one layout: memory position i takes
                                          // scalars[(i / flatInner) % flatExtent]; 0 = not applicable
 };
@@ -73,6 +75,7 @@ struct TadPlan {
     } kind;
     Long tadLength, numTads, tadEws;
     DimMap tm;               // GENERAL
+    unsigned runLength = 0;  // GENERAL: extent of the map's innermost dimension when its stride is 1 (contiguous runs), else 0
     const Long *offsets;     // device, numTads entries
 };
 

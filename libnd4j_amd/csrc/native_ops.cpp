@@ -222,7 +222,27 @@ void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Lon
     pl.tadEws = siEws(tx.hostInfo);
     pl.yEws = siEws(hy);
     pl.zEws = siEws(zTadInfo);
-    if (pl.tadEws > 0 && pl.yEws > 0 && pl.zEws > 0 && dimLen == 1) {
+    // The reference takes its strided loop only for a single dimension whose TAD, y and result TAD all carry an
+    // element-wise stride (cpu/broadcasting.cpp:95), and coordinate arithmetic per element otherwise.  Both visit element f
+    // of every TAD with element f of y, so what decides the kernel here is the layout: TADs over several dimensions
+    // (whose shapeInfo never carries an element-wise stride) that are one strided run all the same take the strided
+    // kernels too.
+    bool stridedWalk = pl.tadEws > 0 && pl.yEws > 0 && pl.zEws > 0 && dimLen == 1;
+    if (!stridedWalk) {
+        char xo = siOrder(tx.hostInfo) == 'c' ? 'c' : 'f';
+        char zo = siOrder(zTadInfo) == 'c' ? 'c' : 'f';
+        linearMap(siShape(tx.hostInfo), siStride(tx.hostInfo), siRank(tx.hostInfo), xo, pl.xm);
+        linearMap(siShape(hy), siStride(hy), siRank(hy), xo, pl.ym);
+        linearMap(siShape(zTadInfo), siStride(zTadInfo), siRank(zTadInfo), zo, pl.zm);
+        if (pl.xm.rank == 1 && pl.ym.rank == 1 && pl.zm.rank == 1 && pl.xm.stride[0] > 0 && pl.ym.stride[0] > 0 &&
+            pl.zm.stride[0] > 0 && siNumel(hy) >= tx.tadLength) {
+            pl.tadEws = pl.xm.stride[0];
+            pl.yEws = pl.ym.stride[0];
+            pl.zEws = pl.zm.stride[0];
+            stridedWalk = true;
+        }
+    }
+    if (stridedWalk) {
         pl.kind = (pl.tadEws == 1 && pl.yEws == 1 && pl.zEws == 1) ? BroadcastPlan::ROW : BroadcastPlan::COL;
         // contiguous TADs of a dense array are its trailing (c order) or leading (f order) block, so they follow one
         // another without gaps;
@@ -235,11 +255,17 @@ void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Lon
         }
     } else {
         pl.kind = BroadcastPlan::GENERAL;
-        char xo = siOrder(tx.hostInfo) == 'c' ? 'c' : 'f';
-        char zo = siOrder(zTadInfo) == 'c' ? 'c' : 'f';
-        linearMap(siShape(tx.hostInfo), siStride(tx.hostInfo), siRank(tx.hostInfo), xo, pl.xm);
-        linearMap(siShape(hy), siStride(hy), siRank(hy), xo, pl.ym);
-        linearMap(siShape(zTadInfo), siStride(zTadInfo), siRank(zTadInfo), zo, pl.zm);
+        if (tx.tadLength > 0x7fffffffLL) throw std::invalid_argument("execBroadcast: a TAD without an element-wise stride holds 2^31 elements or more");
+        // contiguous runs along the innermost dimension of all three walks: one 16-byte vector per thread.  Consecutive
+        // runs of one TAD lie xm.stride[rank - 2] apart; when that leaves room for the same run of other TADs in between
+        // (a dense array's TADs interleave), those are walked side by side.
+        const DimMap *const maps[3] = {&pl.xm, &pl.ym, &pl.zm};
+        const unsigned run = commonRunLength(maps);
+        if (run >= 2 && siNumel(hy) >= tx.tadLength) {
+            pl.runLength = run;
+            const Long next = pl.xm.rank >= 2 && pl.xm.shape[pl.xm.rank - 1] == run ? pl.xm.stride[pl.xm.rank - 2] : (Long)run;
+            pl.runMajor = tx.numTads > 1 && (next >= 2 * (Long)run || next < 0);
+        }
     }
     if (!launchBroadcast<T>(s, opNum, x, y, z, pl)) { reportUnknownOp("broadcast", opNum); return; }
     checkLaunch("execBroadcast", s);

@@ -81,7 +81,22 @@ TadPlan tadPlanFrom(const ResolvedTad &t) {
     pl.tm.rank = 0;
     if (pl.tadEws == 1) pl.kind = TadPlan::ROW;
     else if (pl.tadEws > 1) pl.kind = TadPlan::COL;
-    else { pl.kind = TadPlan::GENERAL; cLinearMap(t.hostInfo, pl.tm); }
+    else {
+        // No element-wise stride in the shapeInfo: the reference walks such a TAD by the C-order coordinates of its
+        // elements (cpu/reduce.cpp:173-188, cpu/indexreduce.cpp:197-205).  TADs over several dimensions never carry
+        // one (shape::TAD leaves it at -1), whatever their layout, so the layout decides here: a TAD whose dimensions merge
+        // into one strided run is walked as the strided kinds walk theirs (same elements, same numbering).
+        pl.kind = TadPlan::GENERAL;
+        cLinearMap(t.hostInfo, pl.tm);
+        if (pl.tm.rank == 1 && pl.tm.stride[0] >= 1) {
+            pl.tadEws = pl.tm.stride[0];
+            pl.kind = pl.tadEws == 1 ? TadPlan::ROW : TadPlan::COL;
+        } else {
+            if (pl.tadLength > 0x7fffffffLL)
+                throw std::invalid_argument("a TAD without an element-wise stride holds 2^31 elements or more");
+            if (pl.tm.stride[pl.tm.rank - 1] == 1 && pl.tm.shape[pl.tm.rank - 1] >= 2) pl.runLength = pl.tm.shape[pl.tm.rank - 1];
+        }
+    }
     return pl;
 }
 

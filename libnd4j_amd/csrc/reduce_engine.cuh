@@ -353,6 +353,88 @@ __global__ void __launch_bounds__(kBlock) tadColFinish(Pol pol, typename Pol::T 
     }
 }
 
+// TADs over several dimensions (their shapeInfo carries no element-wise stride) whose innermost dimension, after the
+// map has been canonicalised, is contiguous: a TAD is a set of runs of runLength elements, placed by the outer dimensions
+// of the map.  TEAM lanes share a TAD - or a slice of one (blockIdx.y) when the TADs are few and long - and take its
+// 16-byte vectors in turn, four in flight per lane; a vector's place costs one division by the number of vectors in a
+// run plus one per outer dimension beyond the first: divisions per vector, none per element.  The last vector of a run
+// is short when runLength is not a multiple of the vector width; vectors need no alignment beyond the element's own.
+template <class Pol, int TEAM>
+__global__ void __launch_bounds__(kBlock) tadRunsKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
+                                                        typename Pol::Acc *partials, const Long *offsets, DimMap tm,
+                                                        Long tadLength, Long numTads, unsigned runLength, FastDiv perRun,
+                                                        unsigned unitsPerTad, unsigned unitsPerSlice) {
+    if (Pol::tables) lm::loadTables();
+    typedef typename Pol::T T;
+    typedef typename Pol::Acc Acc;
+    constexpr int VEC = Pack<T>::N;
+    constexpr int TEAMS = kBlock / TEAM;
+    __shared__ Acc smem[kBlock / kWave];
+    const int team = threadIdx.x / TEAM, lane = threadIdx.x % TEAM;
+    const unsigned u0 = blockIdx.y * unitsPerSlice;
+    const unsigned u1 = unitsPerTad - u0 < unitsPerSlice ? unitsPerTad : u0 + unitsPerSlice;
+    const int outer = tm.rank - 1;  // dimensions that place a run
+    for (Long r0 = (Long)blockIdx.x * TEAMS; r0 < numTads; r0 += (Long)gridDim.x * TEAMS) {
+        const Long r = r0 + team;
+        const bool live = r < numTads;
+        Acc acc;
+        if (live) {
+            pol.setTad(r, z);
+            const T *tx = x + offsets[r];
+            acc = pol.init(tx);
+            for (unsigned u = u0 + lane; u < u1; u += 4 * TEAM) {
+                Pack<T> pk[4];
+                unsigned first[4], count[4];
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const unsigned uu = u + k * TEAM;
+                    count[k] = 0;
+                    if (uu < u1) {
+                        unsigned c;
+                        unsigned m = perRun.divmod(uu, c);
+                        first[k] = m * runLength + c * VEC;
+                        count[k] = runLength - c * VEC;
+                        Long off = (Long)(c * VEC);
+                        for (int d = outer - 1; d > 0; d--) {
+                            const unsigned q = m / tm.shape[d];
+                            off += (Long)(m - q * tm.shape[d]) * tm.stride[d];
+                            m = q;
+                        }
+                        off += (Long)m * tm.stride[0];
+                        if (count[k] >= (unsigned)VEC) {
+                            pk[k] = streamPackAnywhere(tx + off);
+                        } else {
+                            for (unsigned e = 0; e < count[k]; e++) pk[k].v[e] = tx[off + e];
+                        }
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    if (count[k] >= (unsigned)VEC) {
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[k].v[e]), (Long)first[k] + e);
+                        pol.checkpoint(acc);
+                    } else if (count[k] > 0) {
+#pragma unroll
+                        for (int e = 0; e < VEC; e++)
+                            if ((unsigned)e < count[k]) pol.accumulate(acc, toCompute(pk[k].v[e]), (Long)first[k] + e);
+                        pol.checkpoint(acc);
+                    }
+                }
+            }
+        }
+        if (TEAM == kBlock) {
+            acc = blockMerge<Pol>(pol, acc, smem);  // one TAD per block: every thread runs the same trips
+        } else {
+            if (live) acc = waveMerge<Pol, TEAM>(pol, acc);
+        }
+        if (live && lane == 0) {
+            if (gridDim.y == 1) z[r] = pol.finalize(acc, tadLength);
+            else partials[(Long)blockIdx.y * numTads + r] = acc;
+        }
+    }
+}
+
 template <class Pol>
 __global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
                                                            const Long *offsets, DimMap tm, Long tadLength, Long numTads) {
@@ -684,6 +766,38 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         if (splits > 1)
             ND4J_LAUNCH((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kWave - 1) / kWave)), dim3(kBlock), 0, s, pol,
                                z, partials, pl.tadLength, pl.numTads, (int)splits);
+        return;
+    }
+    if (pl.runLength > 0 && pl.tm.rank >= 2) {
+        // several dimensions, the innermost contiguous: vectors along the runs
+        constexpr int VEC = Pack<typename Pol::T>::N;
+        const unsigned unitsPerRun = (pl.runLength + VEC - 1) / VEC;
+        const unsigned unitsPerTad = (unsigned)(pl.tadLength / pl.runLength) * unitsPerRun;
+        const FastDiv perRun(unitsPerRun);
+        Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+        if (unitsPerTad >= 2048) {
+            // a block per TAD; few TADs are cut into slices of at least four vectors per thread and round, about 4096 blocks
+            Long slices = pl.numTads < 2048 ? (4096 + pl.numTads - 1) / pl.numTads : 1;
+            const Long maxSlices = unitsPerTad / (4 * kBlock);
+            if (slices > maxSlices) slices = maxSlices;
+            if (slices > 65535) slices = 65535;
+            while (slices > 1 && (size_t)slices * (size_t)pl.numTads * sizeof(Acc) > ws.bytes) slices /= 2;
+            if (slices < 1) slices = 1;
+            unsigned perSlice = (unsigned)((unitsPerTad + slices - 1) / slices);
+            slices = (unitsPerTad + perSlice - 1) / perSlice;
+            const int gx = (int)(pl.numTads < kGridCap ? pl.numTads : kGridCap);
+            ND4J_LAUNCH((tadRunsKernel<Pol, kBlock>), dim3(gx, (unsigned)slices), dim3(kBlock), 0, s, pol, x, z, partials, pl.offsets,
+                               pl.tm, pl.tadLength, pl.numTads, pl.runLength, perRun, unitsPerTad, perSlice);
+            if (slices > 1)
+                ND4J_LAUNCH((tadSliceFinish<Pol>), dim3((unsigned)pl.numTads), dim3(kBlock), 0, s, pol, x, z, partials, pl.offsets,
+                                   pl.tadLength, pl.numTads, (int)slices);
+        } else if (unitsPerTad >= 64) {
+            ND4J_LAUNCH((tadRunsKernel<Pol, 64>), dim3(gridFor(pl.numTads, kBlock / 64, kGridCap)), dim3(kBlock), 0, s, pol, x, z,
+                               partials, pl.offsets, pl.tm, pl.tadLength, pl.numTads, pl.runLength, perRun, unitsPerTad, unitsPerTad);
+        } else {
+            ND4J_LAUNCH((tadRunsKernel<Pol, 16>), dim3(gridFor(pl.numTads, kBlock / 16, kGridCap)), dim3(kBlock), 0, s, pol, x, z,
+                               partials, pl.offsets, pl.tm, pl.tadLength, pl.numTads, pl.runLength, perRun, unitsPerTad, unitsPerTad);
+        }
         return;
     }
     int grid = gridFor(pl.numTads, 1, kGridCap);

@@ -12,6 +12,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <stdexcept>
 
 #include "shape_host.h"
 
@@ -58,6 +59,17 @@ struct FastDiv {
     }
 };
 
+// An extent as a DimMap stores it.  A map of one dimension is walked by multiplying the index with the stride and never
+// looks at its extent (which may exceed 32 bits: whole arrays of more than 2^32 elements); with two dimensions or more the
+// kernels divide by the extents in 32-bit arithmetic, so one that does not fit is refused instead of wrapping round.
+inline unsigned mapExtent(Long extent, int rank) {
+    if (extent > 0xffffffffLL) {
+        if (rank > 1) throw std::invalid_argument("a view with a (merged) dimension of 2^32 elements or more next to other dimensions is not supported");
+        return 0xffffffffu;
+    }
+    return (unsigned)extent;
+}
+
 // C-order merge of one operand (drop unit dims, fuse dims d,d+1 when stride[d] == shape[d+1]*stride[d+1]).
 inline void ownCanon(int rank, const Long *shape, const Long *stride, DimMap &out) {
     Long shp[kMaxDims], str[kMaxDims];
@@ -75,7 +87,7 @@ inline void ownCanon(int rank, const Long *shape, const Long *stride, DimMap &ou
     }
     if (m == 0) { shp[0] = 1; str[0] = 1; m = 1; }
     out.rank = m;
-    for (int i = 0; i < m; i++) { out.shape[i] = (unsigned)shp[i]; out.stride[i] = str[i]; }
+    for (int i = 0; i < m; i++) { out.shape[i] = mapExtent(shp[i], m); out.stride[i] = str[i]; }
 }
 
 // Joint canonicalisation of up to three operands sharing one shape.  `strides[k]` may be null for an
@@ -108,8 +120,24 @@ inline void jointCanon(int rank, const Long *shape, const Long *const strides[3]
     if (m == 0) { d[0].shp = 1; for (int k = 0; k < 3; k++) d[0].s[k] = 1; m = 1; }
     for (int k = 0; k < 3; k++) {
         out[k].rank = m;
-        for (int i = 0; i < m; i++) { out[k].shape[i] = (unsigned)d[i].shp; out[k].stride[i] = d[i].s[k]; }
+        for (int i = 0; i < m; i++) { out[k].shape[i] = mapExtent(d[i].shp, m); out[k].stride[i] = d[i].s[k]; }
     }
+}
+
+// Largest run length the contiguous-run kernel can use for these maps: the greatest common divisor of the innermost
+// extents when every present map ends in a stride of 1, else 0.  (A run of that many elements starting at a multiple of
+// it lies inside the innermost dimension of every operand.)
+inline unsigned commonRunLength(const DimMap *const maps[3]) {
+    unsigned long long g = 0;
+    for (int k = 0; k < 3; k++) {
+        const DimMap *m = maps[k];
+        if (m == nullptr) continue;
+        if (m->rank < 1 || m->stride[m->rank - 1] != 1) return 0;
+        unsigned long long a = m->shape[m->rank - 1], b = g;
+        while (b != 0) { const unsigned long long t = a % b; a = b; b = t; }
+        g = a;
+    }
+    return (unsigned)g;
 }
 
 }  // namespace nd4j_amd

@@ -32,24 +32,6 @@ template <typename T> __device__ __forceinline__ typename Compute<T>::type store
 
 __device__ __forceinline__ bool inRange(int a, int b) { return (unsigned)a < (unsigned)b; }
 
-// 16 bytes at an address that is only aligned to the element size: the hardware serves misaligned global accesses
-typedef U32x4 U32x4A2 __attribute__((aligned(2)));
-typedef U32x4 U32x4A4 __attribute__((aligned(4)));
-typedef U32x4 U32x4A8 __attribute__((aligned(8)));
-template <typename T> __device__ __forceinline__ Pack<T> loadPackAnywhere(const T *p) {
-    U32x4 v;
-    if (sizeof(T) == 2) v = *reinterpret_cast<const U32x4A2 *>(p);
-    else if (sizeof(T) == 4) v = *reinterpret_cast<const U32x4A4 *>(p);
-    else v = *reinterpret_cast<const U32x4A8 *>(p);
-    return __builtin_bit_cast(Pack<T>, v);
-}
-template <typename T> __device__ __forceinline__ void storePackAnywhere(T *p, const Pack<T> &a) {
-    const U32x4 v = __builtin_bit_cast(U32x4, a);
-    if (sizeof(T) == 2) *reinterpret_cast<U32x4A2 *>(p) = v;
-    else if (sizeof(T) == 4) *reinterpret_cast<U32x4A4 *>(p) = v;
-    else *reinterpret_cast<U32x4A8 *>(p) = v;
-}
-
 }  // namespace
 
 // ---- Reverse ---------------------------------------------------------------------------------------------------

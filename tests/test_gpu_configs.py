@@ -159,6 +159,59 @@ def test_config3_summary_stats_and_softmax_chain(gpu, lib):
         w.free()
 
 
+def test_general_views_at_benchmark_size(gpu, lib):
+    """TADs over several dimensions, broadcasts of sub-arrays and rows with a pitch: against the compiled reference and
+    against numpy on the same inputs."""
+    w = workloads.general_views(gpu.dev, copies=1)
+    try:
+        h = w.host
+        x1 = h["x1"].reshape(128, 128, 56, 56)
+        x64 = x1.astype(np.float64)
+        truth = x64.sum(axis=(0, 2, 3))
+        scale = np.abs(x64).sum(axis=(0, 2, 3)) / np.sqrt(x1.size // 128)
+        c = w.case("sum_nchw_dims023")
+        got, cpu = _run(c).astype(np.float64), c.cpu(lib).astype(np.float64)
+        assert np.all(np.abs(got - truth) <= 1e-5 * np.maximum(np.abs(truth), scale))
+        assert np.all(np.abs(got - cpu) <= np.abs(cpu - truth) + 1e-5 * np.maximum(np.abs(truth), scale))
+        c = w.case("variance_nchw_dims023")
+        var = x64.var(axis=(0, 2, 3), ddof=1)
+        got, cpu = _run(c).astype(np.float64), c.cpu(lib).astype(np.float64)
+        assert np.all(np.abs(got - var) <= 1e-5 * var)
+        assert np.all(np.abs(got - cpu) <= 1e-5 * np.abs(cpu))
+        c = w.case("broadcast_add_nchw_dims23")
+        got = _run(c)
+        assert np.array_equal(got, (x1 + h["plane"].reshape(1, 1, 56, 56)).ravel())
+        assert np.array_equal(got, c.cpu(lib))
+        c = w.case("argmax_cube_dims12")
+        got = _run(c)
+        assert np.array_equal(got, np.argmax(h["x2"].reshape(4096, -1), axis=1).astype(np.float32))
+        assert np.array_equal(got, c.cpu(lib))
+        c = w.case("broadcast_add_slab_dims02")
+        got = _run(c)
+        assert np.array_equal(got, (h["x3"].reshape(256, 1024, 256) + h["mat"].reshape(256, 1, 256)).ravel())
+        assert np.array_equal(got, c.cpu(lib))
+        # the view's rows: 1024 of every 1032 elements; the 8 between two rows are never written
+        rows, cols, pitch = 65536, 1024, 1032
+
+        def view(a):
+            return np.lib.stride_tricks.as_strided(a, (rows, cols), (4 * pitch, 4))
+
+        def gaps(a):
+            return np.lib.stride_tricks.as_strided(a[cols:], (rows - 1, pitch - cols), (4 * pitch, 4))
+
+        c = w.case("pairwise_add_padded_rows")
+        got = _run(c)
+        assert np.array_equal(view(got), view(h["xv"]) + view(h["yv"]))
+        assert np.array_equal(view(got), view(c.cpu(lib)))
+        assert not gaps(got).any()
+        c = w.case("transform_exp_padded_rows")
+        got = _run(c)
+        assert ulp_distance(view(got), view(c.cpu(lib))).max() <= 2
+        assert not gaps(got).any()
+    finally:
+        w.free()
+
+
 def test_data_movement_at_benchmark_size(gpu, lib):
     w = workloads.data_movement(gpu.dev, copies=1)
     try:
