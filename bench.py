@@ -344,11 +344,11 @@ def main():
                                    "frac": round(tflops / MFMA_FP32_PEAK_TFLOPS, 4)}
                 v = valu_per_element(args.instructions, c.name)
                 if v is not None:
-                    # the data sheet's 157.3 TFLOP/s of vector fp32 are 256 CUs x 4 SIMDs x 32 lanes x 2 flops x 2.4 GHz: a
-                    # wave64 instruction every 2 cycles per SIMD, which takes the packed forms; plain fp32 and integer
-                    # instructions measure 3 to 4.5 cycles here.  Priced at 2 cycles apiece, the call's vector instructions
-                    # need at least this long on the chip's 1024 SIMDs: a floor of the arithmetic's share, not its size
-                    issue_ms = v * c.elements / 64.0 * 2.0 / (1024 * 2.4e9) * 1e3
+                    # A SIMD is 16 lanes wide: a wave64 vector instruction holds it for 4 cycles (plain fp32 and integer
+                    # instructions measure 2.9 to 4.7 on this chip; the data sheet's 157.3 TFLOP/s take the packed forms,
+                    # two results per lane and cycle, which this build does not use).  At 4 cycles apiece the call's vector
+                    # instructions need this long on the chip's 1024 SIMDs
+                    issue_ms = v * c.elements / 64.0 * 4.0 / (1024 * 2.4e9) * 1e3
                     row["valu"] = {"instructions_per_element": v, "issue_ms": round(issue_ms, 4), "frac": round(issue_ms / ms, 4)}
                     # the time the vector units were held, by the chip's own count (SQ_ACTIVE_INST_VALU; like the issue
                     # time it prices every instruction at one slot, so both are lower bounds)

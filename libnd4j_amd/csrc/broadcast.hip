@@ -51,10 +51,8 @@ template <typename T> struct BroadcastBody {
                                    pl.zOffsets, pl.tadLength, pl.numTads, pl.tadEws, pl.yEws, pl.zEws, Params<T>{nullptr});
             } else if (pl.runLength > 0) {
                 // TADs over several dimensions whose innermost one is contiguous in x, y and z
-                const Long units = pl.numTads * (pl.tadLength / pl.runLength) * ((pl.runLength + Pack<T>::N - 1) / Pack<T>::N);
-                ND4J_LAUNCH((ewRunsKernel<T, F>), dim3(gridFor(units, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0, s, x,
-                                   pl.xm, y, pl.ym, z, pl.zm, pl.xOffsets, pl.zOffsets, Params<T>{nullptr}, pl.numTads,
-                                   (unsigned)pl.tadLength, pl.runLength, pl.runMajor ? 1 : 0);
+                launchRuns<T, F, true>(s, x, pl.xm, y, pl.ym, z, pl.zm, pl.xOffsets, pl.zOffsets, Params<T>{nullptr}, pl.numTads,
+                                 pl.tadLength, pl.runLength, pl.runMajor);
             } else {
                 int grid = gridFor(pl.numTads, 1, kGridCap);
                 ND4J_LAUNCH((bcGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, pl.xm, y, pl.ym, z, pl.zm,

@@ -21,11 +21,13 @@ OBJS := \$(addsuffix .o,\$(basename $SRCS))
 all: ../$OUT
 ../$OUT: \$(OBJS)
 	hipcc --offload-arch=gfx950 -shared -fPIC -o \$@ \$(OBJS)
-%.o: ../%.hip \$(wildcard ../*.h ../*.cuh ../../../include/*.h)
-	hipcc $HIPFLAGS -c \$< -o \$@ 2>&1 | grep -v "packed-fp32-ops' is not a recognized feature" || true
+# an object is rebuilt when a header it includes has changed (the compiler writes the list beside it: -MMD)
+%.o: ../%.hip
+	hipcc $HIPFLAGS -MMD -MP -c \$< -o \$@ 2>&1 | grep -v "packed-fp32-ops' is not a recognized feature" || true
 	test -f \$@
-%.o: ../%.cpp \$(wildcard ../*.h ../*.cuh ../../../include/*.h)
-	hipcc $HIPFLAGS -x hip -c \$< -o \$@ 2>&1 | grep -v "packed-fp32-ops' is not a recognized feature" || true
+%.o: ../%.cpp
+	hipcc $HIPFLAGS -MMD -MP -x hip -c \$< -o \$@ 2>&1 | grep -v "packed-fp32-ops' is not a recognized feature" || true
 	test -f \$@
+-include \$(OBJS:.o=.d)
 MK
 make -C $OBJ $JOBS $FORCE all

@@ -463,58 +463,159 @@ __global__ void __launch_bounds__(kBlock) bcGeneralKernel(const T *x, DimMap xm,
     }
 }
 
+// Offset of the vector that starts `inner` elements into run m (runs of runLength elements, numbered in C order) of a
+// map whose innermost dimension is contiguous and holds whole runs.  When a run is that whole dimension - the usual case -
+// m counts the outer dimensions directly and the first of them costs no division.
+__device__ __forceinline__ Long runOffset(const DimMap &mp, unsigned m, unsigned inner, unsigned runLength) {
+    const int last = mp.rank - 1;
+    if (last > 0 && mp.shape[last] == runLength) {
+        Long off = inner;
+        for (int d = last - 1; d > 0; d--) {
+            const unsigned q = m / mp.shape[d];
+            off += (Long)(m - q * mp.shape[d]) * mp.stride[d];
+            m = q;
+        }
+        return off + (Long)m * mp.stride[0];
+    }
+    return mapOffset32(mp, m * runLength + inner);
+}
+
 // Views that are made of contiguous runs: every operand's index -> offset map ends in a dimension of stride 1 whose extent
 // is a multiple of runLength (the padded rows of a view with a pitch; the TADs of a broadcast over several dimensions).
 // The element space is cut into units of one 16-byte vector inside a run (the last unit of a run is shorter when
-// runLength is not a multiple of the vector width); a thread takes one unit, finds its place through each operand's map
+// runLength is not a multiple of the vector width); a thread takes a unit, finds its place through each operand's map
 // once - divisions per vector, not per element - and moves it with 16-byte accesses that need no alignment beyond the
-// element's own.  xOffsets / zOffsets (null: one "TAD" at offset 0) add a per-TAD offset, y is shared by all TADs.
-// Units are numbered run by run inside a TAD (runMajor 0), or with the same run of all TADs side by side (runMajor 1):
-// whichever makes neighbouring threads touch neighbouring memory.
-template <typename T, typename F>
+// element's own; the next unit's loads are issued before the current one is worked on.  xOffsets / zOffsets (null: one
+// "TAD" at offset 0) add a per-TAD offset, y is shared by all TADs.  Units are numbered run by run inside a TAD
+// (runMajor 0), or with the same run of all TADs side by side (runMajor 1): whichever makes neighbouring threads touch
+// neighbouring memory.  perRun divides by the units of a run, second by the TAD count (runMajor) or the runs of a TAD;
+// both serve totals below 2^31 units, larger ones take 64-bit divisions.
+template <typename T, typename F, int U>
 __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, const T *y, DimMap ym, T *z, DimMap zm,
                                                        const Long *xOffsets, const Long *zOffsets, Params<T> p, Long numTads,
-                                                       unsigned tadLength, unsigned runLength, int runMajor) {
+                                                       unsigned tadLength, unsigned runLength, int runMajor, FastDiv perRun,
+                                                       FastDiv second) {
     typedef typename Compute<T>::type C;
-    if (F::tables) lm::loadTables();
     constexpr int VEC = Pack<T>::N;
+    constexpr bool two = F::nin == 2;
     const unsigned unitsPerRun = (runLength + VEC - 1) / VEC;
     const unsigned runsPerTad = tadLength / runLength;
     const Long total = numTads * ((Long)runsPerTad * unitsPerRun);
-    const bool small = total <= 0xffffffffLL;
-    for (Long g = (Long)blockIdx.x * kBlock + threadIdx.x; g < total; g += (Long)gridDim.x * kBlock) {
-        // g -> (TAD r, run m of the TAD, unit c of the run)
-        Long r;
-        unsigned m, c;
+    const bool small = total <= 0x7fffffffLL;
+    const Long step = (Long)gridDim.x * kBlock;
+
+    // g -> (TAD r, run m of the TAD, unit c of the run)
+    auto locate = [&](Long g, Long &r, unsigned &m, unsigned &c) {
         if (small) {
-            const unsigned t = (unsigned)g / unitsPerRun;
-            c = (unsigned)g - t * unitsPerRun;
-            if (runMajor) { m = t / (unsigned)numTads; r = t - m * (unsigned)numTads; }
-            else { const unsigned q = t / runsPerTad; m = t - q * runsPerTad; r = q; }
+            const unsigned t = perRun.divmod((unsigned)g, c);
+            unsigned rem;
+            const unsigned q = second.divmod(t, rem);
+            if (runMajor) { m = q; r = rem; }
+            else { r = q; m = rem; }
         } else {
             const Long t = g / unitsPerRun;
             c = (unsigned)(g - t * unitsPerRun);
             if (runMajor) { m = (unsigned)(t / numTads); r = t - (Long)m * numTads; }
             else { r = t / runsPerTad; m = (unsigned)(t - r * runsPerTad); }
         }
-        const unsigned f0 = m * runLength + c * VEC;  // index of the unit's first element inside its TAD
-        const unsigned count = runLength - c * VEC;   // elements left in the run from there on
-        const T *xp = x + (xOffsets != nullptr ? xOffsets[r] : 0) + mapOffset32(xm, f0);
-        T *zp = z + (zOffsets != nullptr ? zOffsets[r] : 0) + mapOffset32(zm, f0);
-        const T *yp = F::nin == 2 ? y + mapOffset32(ym, f0) : nullptr;
-        if (count >= VEC) {
-            const Pack<T> a = streamPackAnywhere(xp);
-            Pack<T> b;
-            if (F::nin == 2) b = loadPackAnywhere(yp);
+    };
+    if constexpr (U > 1) {
+        // With offset tables a unit costs two trips to memory, one after the other (its TAD's offsets, then its vectors): U
+        // units per thread go through each stage together, so that what is in flight stays ahead of the memory's latency.
+        if (F::tables) lm::loadTables();
+        for (Long g0 = (Long)blockIdx.x * kBlock + threadIdx.x; g0 < total; g0 += step * U) {
+            unsigned m[U], c[U];
+            Long xo[U], zo[U];
+            bool live[U];
+#pragma unroll
+            for (int k = 0; k < U; k++) {
+                const Long g = g0 + k * step;
+                live[k] = g < total;
+                xo[k] = zo[k] = 0;
+                if (live[k]) {
+                    Long r;
+                    locate(g, r, m[k], c[k]);
+                    if (xOffsets != nullptr) xo[k] = xOffsets[r];
+                    if (zOffsets != nullptr) zo[k] = zOffsets[r];
+                }
+            }
+            const T *xp[U], *yp[U];
+            T *zp[U];
+            Pack<T> a[U], b[U];
+            bool whole[U];
+#pragma unroll
+            for (int k = 0; k < U; k++) {
+                whole[k] = false;
+                if (live[k]) {
+                    xp[k] = x + xo[k] + runOffset(xm, m[k], c[k] * VEC, runLength);
+                    zp[k] = z + zo[k] + runOffset(zm, m[k], c[k] * VEC, runLength);
+                    if (two) yp[k] = y + runOffset(ym, m[k], c[k] * VEC, runLength);
+                    whole[k] = runLength - c[k] * VEC >= (unsigned)VEC;
+                    if (whole[k]) {
+                        a[k] = streamPackAnywhere(xp[k]);
+                        if (two) b[k] = loadPackAnywhere(yp[k]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < U; k++) {
+                if (whole[k]) {
+                    Pack<T> o;
+#pragma unroll
+                    for (int e = 0; e < VEC; e++)
+                        o.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a[k].v[e]), two ? toCompute(b[k].v[e]) : (C)0, p));
+                    streamPackAnywhere(zp[k], o);
+                } else if (live[k]) {
+                    const unsigned count = runLength - c[k] * VEC;
+                    for (unsigned e = 0; e < count; e++)
+                        zp[k][e] = fromCompute<T>(F::template apply<C>(toCompute(xp[k][e]), two ? toCompute(yp[k][e]) : (C)0, p));
+                }
+            }
+        }
+        return;
+    }
+    const T *xp = nullptr, *yp = nullptr;
+    T *zp = nullptr;
+    unsigned count = 0;
+    Pack<T> a, b;
+    // the three addresses of unit g; requests the unit's vectors
+    auto fetch = [&](Long g, const T *&ux, const T *&uy, T *&uz, unsigned &ucount, Pack<T> &ua, Pack<T> &ub) {
+        Long r;
+        unsigned m, c;
+        locate(g, r, m, c);
+        ucount = runLength - c * VEC;  // elements left in the run from the unit's first one on
+        ux = x + (xOffsets != nullptr ? xOffsets[r] : 0) + runOffset(xm, m, c * VEC, runLength);
+        uz = z + (zOffsets != nullptr ? zOffsets[r] : 0) + runOffset(zm, m, c * VEC, runLength);
+        if (two) uy = y + runOffset(ym, m, c * VEC, runLength);
+        if (ucount >= (unsigned)VEC) {
+            ua = streamPackAnywhere(ux);
+            if (two) ub = loadPackAnywhere(uy);  // through the caches: every TAD reads it again
+        }
+    };
+    Long g = (Long)blockIdx.x * kBlock + threadIdx.x;
+    bool have = g < total;
+    if (have) fetch(g, xp, yp, zp, count, a, b);
+    if (F::tables) lm::loadTables();  // staged while the first vectors are on their way
+    while (have) {
+        const Long gn = g + step;
+        const bool haveNext = gn < total;
+        const T *nxp = nullptr, *nyp = nullptr;
+        T *nzp = nullptr;
+        unsigned ncount = 0;
+        Pack<T> na, nb;
+        if (haveNext) fetch(gn, nxp, nyp, nzp, ncount, na, nb);
+        if (count >= (unsigned)VEC) {
             Pack<T> o;
 #pragma unroll
             for (int e = 0; e < VEC; e++)
-                o.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), F::nin == 2 ? toCompute(b.v[e]) : (C)0, p));
+                o.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), two ? toCompute(b.v[e]) : (C)0, p));
             streamPackAnywhere(zp, o);
         } else {
             for (unsigned e = 0; e < count; e++)
-                zp[e] = fromCompute<T>(F::template apply<C>(toCompute(xp[e]), F::nin == 2 ? toCompute(yp[e]) : (C)0, p));
+                zp[e] = fromCompute<T>(F::template apply<C>(toCompute(xp[e]), two ? toCompute(yp[e]) : (C)0, p));
         }
+        g = gn; have = haveNext;
+        xp = nxp; yp = nyp; zp = nzp; count = ncount; a = na; b = nb;
     }
 }
 
@@ -538,6 +639,31 @@ template <typename T> inline int commonHead(const void *a, const void *b, const 
     if ((pa & 15) != (pb & 15) || (pa & 15) != (pc & 15)) return -1;
     if ((pa & (sizeof(T) - 1)) != 0) return -1;
     return (int)(((16 - (pa & 15)) & 15) / sizeof(T));
+}
+
+// grid and divisors of ewRunsKernel for `numTads` TADs of tadLength elements in runs of runLength; OFFSETS: the call
+// carries per-TAD offset tables (a compile-time choice, so that each family builds only the form it launches)
+template <typename T, typename F, bool OFFSETS>
+inline void launchRuns(hipStream_t s, const T *x, const DimMap &xm, const T *y, const DimMap &ym, T *z, const DimMap &zm,
+                       const Long *xOffsets, const Long *zOffsets, Params<T> p, Long numTads, Long tadLength, unsigned runLength,
+                       bool runMajor) {
+    const unsigned unitsPerRun = (runLength + Pack<T>::N - 1) / Pack<T>::N;
+    const Long runsPerTad = tadLength / runLength;
+    const Long units = numTads * runsPerTad * unitsPerRun;
+    const FastDiv perRun(unitsPerRun);
+    const Long by = runMajor ? numTads : runsPerTad;
+    const FastDiv second((unsigned)(by > 0x7fffffffLL ? 0x7fffffffLL : by));
+    // with offset tables: two units per thread and round (one: 54-63 % of the HBM peak on a [256,1024,256] array broadcast
+    // along dimensions {0,2}, two: 68 %, four: 60 %); without, one unit per thread and the next one's loads ahead
+    if constexpr (OFFSETS) {
+        ND4J_LAUNCH((ewRunsKernel<T, F, 2>), dim3(gridFor(units, kBlock * 2, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0, s,
+                           x, xm, y, ym, z, zm, xOffsets, zOffsets, p, numTads, (unsigned)tadLength, runLength, runMajor ? 1 : 0, perRun,
+                           second);
+    } else {
+        ND4J_LAUNCH((ewRunsKernel<T, F, 1>), dim3(gridFor(units, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0, s,
+                           x, xm, y, ym, z, zm, xOffsets, zOffsets, p, numTads, (unsigned)tadLength, runLength, runMajor ? 1 : 0, perRun,
+                           second);
+    }
 }
 
 template <typename T, typename F>
@@ -699,10 +825,7 @@ inline void launchGeneral(hipStream_t s, const T *x, const DimMap &xm, const T *
     const DimMap *const maps[3] = {&xm, two ? &ym : nullptr, &zm};
     const unsigned run = commonRunLength(maps);
     if (run >= (unsigned)Pack<T>::N && n <= 0x7fffffffLL) {
-        const Long units = n / run * ((run + Pack<T>::N - 1) / Pack<T>::N);
-        ND4J_LAUNCH((ewRunsKernel<T, F>), dim3(gridFor(units, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0, s, x, xm,
-                           two ? y : x, two ? ym : xm, z, zm, (const Long *)nullptr, (const Long *)nullptr, p, (Long)1, (unsigned)n,
-                           run, 0);
+        launchRuns<T, F, false>(s, x, xm, two ? y : x, two ? ym : xm, z, zm, nullptr, nullptr, p, 1, n, run, false);
         return;
     }
     int grid = gridFor(n, kBlock * 4, kGridCap);

@@ -55,6 +55,18 @@ template <typename TT, int OP> struct IndexPol {
             }
         }
     }
+    // the same for an element that lies behind everything the accumulator has seen: a tie never replaces
+    static constexpr bool hasAscending = true;
+    __device__ __forceinline__ void accumulateAscending(Acc &a, C v, Long i) const {
+        if (OP <= 3) {
+            C c = (OP == 2 || OP == 3) ? m::abs_(v) : v;
+            const bool wins = (OP == 0 || OP == 2) ? c > a.value : c < a.value;
+            a.value = wins ? c : a.value;
+            a.index = wins ? i : a.index;
+        } else if (matchConditionOp<C>(v, p) != (C)0) {
+            if (OP == 5 || a.index < 0) { a.index = i; a.value = v; }
+        }
+    }
     __device__ __forceinline__ void checkpoint(Acc &) const {}
     __device__ __forceinline__ Acc combine(Acc a, Acc b) const {
         if (OP <= 3) {

@@ -59,6 +59,19 @@ template <class Pol> struct PolFlatBlocks<Pol, decltype((void)Pol::kFlatBlocks)>
 template <class Pol, typename = void> struct PolClears { static constexpr bool value = false; };
 template <class Pol> struct PolClears<Pol, decltype((void)Pol::kClears)> { static constexpr bool value = Pol::kClears; };
 
+// Folds an element whose index is higher than that of every element the accumulator has seen (the kernels walk their
+// elements in ascending order wherever they can).  A policy may exploit that with a member accumulateAscending(): an
+// index reduction then needs one comparison per element, where the general rule (better value, or the same value at a
+// lower index) takes three and a handful of mask operations on the compute unit's one scalar unit - these kernels issued
+// five scalar instructions per element of a wave that way, as many as a sum issues in all.
+template <class Pol, typename = void> struct HasAscending { static constexpr bool value = false; };
+template <class Pol> struct HasAscending<Pol, decltype((void)Pol::hasAscending)> { static constexpr bool value = Pol::hasAscending; };
+template <class Pol>
+__device__ __forceinline__ void foldNext(const Pol &pol, typename Pol::Acc &acc, typename Pol::C v, Long i) {
+    if constexpr (HasAscending<Pol>::value) pol.accumulateAscending(acc, v, i);
+    else pol.accumulate(acc, v, i);
+}
+
 // Merge over the lanes of one wave; lane 0 (of each WIDTH-lane segment) ends up with the result.
 template <class Pol, int WIDTH = kWave>
 __device__ __forceinline__ typename Pol::Acc waveMerge(const Pol &pol, typename Pol::Acc a) {
@@ -113,6 +126,8 @@ __device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc
     if (!oneEach) {
         for (Long i = lane; i < head; i += lanes) { pol.accumulate(acc, toCompute(p[i]), base + i); pol.checkpoint(acc); }
     }
+    // (a lane's elements are folded in ascending order: its head element first, its tail element last)
+    if (hasEdge && lane < head) { foldNext(pol, acc, toCompute(edge), base + edgeAt); pol.checkpoint(acc); }
     const Pack<T> *pv = reinterpret_cast<const Pack<T> *>(p + head);
     Long v = lane;
     // Four independent 16-byte loads in flight per lane, then the arithmetic.  Each of the four is guarded on its own: a
@@ -128,14 +143,14 @@ __device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc
         for (int u = 0; u < 4; u++) {
             if (v + u * (Long)lanes < nvec) {
 #pragma unroll
-                for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[u].v[e]), base + head + (v + u * (Long)lanes) * VEC + e);
+                for (int e = 0; e < VEC; e++) foldNext(pol, acc, toCompute(pk[u].v[e]), base + head + (v + u * (Long)lanes) * VEC + e);
                 pol.checkpoint(acc);
             }
         }
     }
-    if (hasEdge) { pol.accumulate(acc, toCompute(edge), base + edgeAt); pol.checkpoint(acc); }
+    if (hasEdge && lane >= head) { foldNext(pol, acc, toCompute(edge), base + edgeAt); pol.checkpoint(acc); }
     if (!oneEach) {
-        for (Long i = tail0 + lane; i < n; i += lanes) { pol.accumulate(acc, toCompute(p[i]), base + i); pol.checkpoint(acc); }
+        for (Long i = tail0 + lane; i < n; i += lanes) { foldNext(pol, acc, toCompute(p[i]), base + i); pol.checkpoint(acc); }
     }
 }
 
@@ -189,10 +204,10 @@ __global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename P
 #pragma unroll
         for (int u = 0; u < 8; u++) v[u] = base[(j + u * S) * tadEws];
 #pragma unroll
-        for (int u = 0; u < 8; u++) pol.accumulate(acc, toCompute(v[u]), j + u * S);
+        for (int u = 0; u < 8; u++) foldNext(pol, acc, toCompute(v[u]), j + u * S);
         pol.checkpoint(acc);
     }
-    for (; j < tadLength; j += S) { pol.accumulate(acc, toCompute(base[j * tadEws]), j); pol.checkpoint(acc); }
+    for (; j < tadLength; j += S) { foldNext(pol, acc, toCompute(base[j * tadEws]), j); pol.checkpoint(acc); }
     if (gridDim.y == 1) z[t] = pol.finalize(acc, tadLength);
     else partials[(Long)blockIdx.y * numTads + t] = acc;
 }
@@ -243,6 +258,11 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
             const Long turn = span >= 8 * WAVES ? (((Long)blockIdx.y * 3) % (span / (4 * WAVES))) * (4 * WAVES) : 0;
             for (int part = 0; part < 2; part++) {
                 const Long a = part == 0 ? j0 + turn : j0, b = part == 0 ? j1 : j0 + turn;
+                // (each part is walked in ascending order with accumulators of its own; the second part's rows lie before
+                // the first's)
+                Acc cur[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; e++) cur[e] = pe[e].init(x + off[e]);
                 Long j = a + wave;
                 for (; j + 3 * WAVES < b; j += 4 * WAVES) {
                     Pack<T> pk[4];
@@ -251,23 +271,25 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
 #pragma unroll
                     for (int u = 0; u < 4; u++) {
 #pragma unroll
-                        for (int e = 0; e < VEC; e++) pe[e].accumulate(acc[e], toCompute(pk[u].v[e]), j + u * WAVES);
+                        for (int e = 0; e < VEC; e++) foldNext(pe[e], cur[e], toCompute(pk[u].v[e]), j + u * WAVES);
                     }
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) pe[e].checkpoint(acc[e]);
+                    for (int e = 0; e < VEC; e++) pe[e].checkpoint(cur[e]);
                 }
                 for (; j < b; j += WAVES) {
                     Pack<T> pk = loadPack(reinterpret_cast<const Pack<T> *>(base + j * tadEws));
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) { pe[e].accumulate(acc[e], toCompute(pk.v[e]), j); pe[e].checkpoint(acc[e]); }
+                    for (int e = 0; e < VEC; e++) { foldNext(pe[e], cur[e], toCompute(pk.v[e]), j); pe[e].checkpoint(cur[e]); }
                 }
+#pragma unroll
+                for (int e = 0; e < VEC; e++) acc[e] = part == 0 ? cur[e] : pe[e].combine(acc[e], cur[e]);
             }
         } else {
 #pragma unroll
             for (int e = 0; e < VEC; e++) {
                 if (t0 + e >= numTads) continue;
                 const T *base = x + off[e];
-                for (Long j = j0 + wave; j < j1; j += WAVES) { pe[e].accumulate(acc[e], toCompute(base[j * tadEws]), j); pe[e].checkpoint(acc[e]); }
+                for (Long j = j0 + wave; j < j1; j += WAVES) { foldNext(pe[e], acc[e], toCompute(base[j * tadEws]), j); pe[e].checkpoint(acc[e]); }
             }
         }
     }
@@ -404,7 +426,11 @@ __global__ void __launch_bounds__(kBlock) tadRunsKernel(Pol pol, const typename 
                         if (count[k] >= (unsigned)VEC) {
                             pk[k] = streamPackAnywhere(tx + off);
                         } else {
-                            for (unsigned e = 0; e < count[k]; e++) pk[k].v[e] = tx[off + e];
+                            // (a loop with a run-time bound would index the vectors dynamically, and the compiler would
+                            // move all four of them from registers to LDS)
+#pragma unroll
+                            for (int e = 0; e < VEC; e++)
+                                if ((unsigned)e < count[k]) pk[k].v[e] = tx[off + e];
                         }
                     }
                 }
@@ -412,12 +438,12 @@ __global__ void __launch_bounds__(kBlock) tadRunsKernel(Pol pol, const typename 
                 for (int k = 0; k < 4; k++) {
                     if (count[k] >= (unsigned)VEC) {
 #pragma unroll
-                        for (int e = 0; e < VEC; e++) pol.accumulate(acc, toCompute(pk[k].v[e]), (Long)first[k] + e);
+                        for (int e = 0; e < VEC; e++) foldNext(pol, acc, toCompute(pk[k].v[e]), (Long)first[k] + e);
                         pol.checkpoint(acc);
                     } else if (count[k] > 0) {
 #pragma unroll
                         for (int e = 0; e < VEC; e++)
-                            if ((unsigned)e < count[k]) pol.accumulate(acc, toCompute(pk[k].v[e]), (Long)first[k] + e);
+                            if ((unsigned)e < count[k]) foldNext(pol, acc, toCompute(pk[k].v[e]), (Long)first[k] + e);
                         pol.checkpoint(acc);
                     }
                 }
@@ -446,7 +472,7 @@ __global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typena
         const typename Pol::T *tx = x + offsets[r];
         Acc acc = pol.init(tx);
         for (Long f = threadIdx.x; f < tadLength; f += kBlock)
-            { pol.accumulate(acc, toCompute(tx[mapOffset32(tm, (unsigned)f)]), f); pol.checkpoint(acc); }
+            { foldNext(pol, acc, toCompute(tx[mapOffset32(tm, (unsigned)f)]), f); pol.checkpoint(acc); }
         acc = blockMerge<Pol>(pol, acc, smem);
         if (threadIdx.x == 0) z[r] = pol.finalize(acc, tadLength);
     }
@@ -592,7 +618,7 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
                 if (v < nvec) {
                     Acc &to = (CH > 1 && u % CH > 0) ? more[u % CH - 1] : acc;
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) pol.accumulate(to, toCompute(pk[u].v[e]), head + v * VEC + e);
+                    for (int e = 0; e < VEC; e++) foldNext(pol, to, toCompute(pk[u].v[e]), head + v * VEC + e);
                     pol.checkpoint(to);
                 }
             }
@@ -625,10 +651,10 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
         }
     } else if (strided) {
         for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock)
-            { pol.accumulate(acc, toCompute(x[i * ews]), i); pol.checkpoint(acc); }
+            { foldNext(pol, acc, toCompute(x[i * ews]), i); pol.checkpoint(acc); }
     } else {
         for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < n; i += (Long)gridDim.x * kBlock)
-            { pol.accumulate(acc, toCompute(x[mapOffsetAny(xm, i)]), i); pol.checkpoint(acc); }
+            { foldNext(pol, acc, toCompute(x[mapOffsetAny(xm, i)]), i); pol.checkpoint(acc); }
     }
     acc = blockMerge<Pol>(pol, acc, smem);
     if (gridDim.x == 1) {
@@ -776,14 +802,19 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         const FastDiv perRun(unitsPerRun);
         Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
         if (unitsPerTad >= 2048) {
-            // a block per TAD; few TADs are cut into slices of at least four vectors per thread and round, about 4096 blocks
-            Long slices = pl.numTads < 2048 ? (4096 + pl.numTads - 1) / pl.numTads : 1;
-            const Long maxSlices = unitsPerTad / (4 * kBlock);
+            // a block per TAD; few TADs are cut into slices of whole rounds (four vectors per thread), four rounds or more
+            // each, about 2048 blocks in all (4096 or 8192 blocks and slices of one or two rounds measured the same for sums
+            // and 10 % slower for the summary statistics, whose accumulators cost more to merge)
+            const int tuneRounds = 4, tuneBlocks = 2048;
+            const unsigned round = 4 * kBlock;
+            Long slices = pl.numTads < tuneBlocks ? (tuneBlocks + pl.numTads - 1) / pl.numTads : 1;
+            const Long maxSlices = unitsPerTad / (tuneRounds * round);
             if (slices > maxSlices) slices = maxSlices;
             if (slices > 65535) slices = 65535;
             while (slices > 1 && (size_t)slices * (size_t)pl.numTads * sizeof(Acc) > ws.bytes) slices /= 2;
             if (slices < 1) slices = 1;
             unsigned perSlice = (unsigned)((unitsPerTad + slices - 1) / slices);
+            if (slices > 1) perSlice = (perSlice + round - 1) / round * round;
             slices = (unitsPerTad + perSlice - 1) / perSlice;
             const int gx = (int)(pl.numTads < kGridCap ? pl.numTads : kGridCap);
             ND4J_LAUNCH((tadRunsKernel<Pol, kBlock>), dim3(gx, (unsigned)slices), dim3(kBlock), 0, s, pol, x, z, partials, pl.offsets,

@@ -647,8 +647,7 @@ def random_fills(dev, n=1 << 26, side=8192, seed=119, buffer_longs=1 << 20, data
         # bound by the instruction count of the reference's 64-bit integer stream, not by HBM
         for c in cases:
             c.bound = "valu"
-            c.note = ("the arithmetic of the reference's u64 stream: valu.issue_ms prices an instruction at 2 cycles, plain fp32 and "
-                      "integer instructions measure 3 to 4.5 on this chip")
+            c.note = "the arithmetic of the reference's u64 stream: valu.issue_ms prices a wave64 vector instruction at 4 cycles of its SIMD"
         return cases
 
     inner_set = device_set
