@@ -225,6 +225,16 @@ void nd4j_amd_setCooperativeWaitLimit(int tries);
  * hardware traffic counters are scaled */
 void nd4j_amd_copyKernel(Nd4jPointer *extraPointers, void *dst, const void *src, Nd4jLong bytes);
 
+/* No counterpart in the reference (its scratch belongs to the caller).  The library keeps a workspace, reduction slots
+ * and a pinned scalar block per (device, stream), allocated at the stream's first call that needs them.  A host that
+ * destroys a stream calls this first, with the stream's device current: it waits for the stream to drain and frees them
+ * (13 MiB of device memory and 256 bytes of pinned host memory a stream); a later call on the same handle allocates
+ * afresh.  Without it they stay until the process ends. */
+void nd4j_amd_releaseStream(Nd4jPointer stream);
+/* test aid: sets the counter from which the launches on extraPointers[1]'s stream draw the tickets that tag their
+ * exchange slots, so that a test can walk it across the points where the library clears the slots */
+void nd4j_amd_setSlotTicket(Nd4jPointer *extraPointers, unsigned int value);
+
 /* ---- for callers that cannot allocate: no counterpart in the reference ------------------------------- */
 /* execReduceFloat over the whole array (no dimensions): result[0], a device pointer, receives what
  * nd4j_execReduceFloatFull leaves there, bit for bit.  For callers that may not call hipMalloc while they run

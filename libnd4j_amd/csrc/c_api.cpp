@@ -274,6 +274,12 @@ void nd4j_amd_execReduceFloatNoAlloc(Nd4jPointer *extraPointers, int opNum, floa
                                      float *result) {
     guardVoid([&] { nd4j_amd::reduceFloatNoAlloc(extraPointers, opNum, x, xShapeInfo, extraParams, result); });
 }
+void nd4j_amd_releaseStream(Nd4jPointer stream) {
+    guardVoid([&] { nd4j_amd::releaseStreamResources(reinterpret_cast<hipStream_t>(stream)); });
+}
+void nd4j_amd_setSlotTicket(Nd4jPointer *extraPointers, unsigned int value) {
+    guardVoid([&] { nd4j_amd::setSlotTicketForTesting(nd4j_amd::streamOf(extraPointers), value); });
+}
 Nd4jLong nd4j_amd_hostFetchCount(void) { return (Nd4jLong)nd4j_amd::hostFetchCount(); }
 void nd4j_amd_setCooperativeWaitLimit(int tries) { nd4j_amd::setCooperativeWaitLimit(tries); }
 void nd4j_amd_copyKernel(Nd4jPointer *extraPointers, void *dst, const void *src, Nd4jLong bytes) {

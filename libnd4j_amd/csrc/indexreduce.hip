@@ -22,6 +22,7 @@ template <typename TT, int OP> struct IndexPol {
     typedef IndexAcc<C> Acc;
     static constexpr bool tables = false;  // no exp / log / pow in these accumulators
     static constexpr int kChains = 4;      // accumulators of one lane may be kept apart and combined (ties go to the lower index)
+    static constexpr int kSlotWords = 2 + sizeof(C) / 4;  // index and value; the float accumulator's padding word stays behind
     static constexpr bool kClears = OP == 0;  // IsMax over a whole array looks for the maximum and clears the result in one pass
     Params<TT> p;
 

@@ -97,6 +97,9 @@ struct Workspace {
     unsigned *rowStates = nullptr;         // rowStateCount 32-bit words beside the slots, for launches that decide per row
     size_t rowStateCount = 0;
     unsigned *slotTicketSource = nullptr;  // host memory: the last ticket handed out for these slots
+    // pinned host word the device can write: a merging block that gave up waiting for a slot stores 1 here (and NaN as
+    // the result), which the host reports at its next look (null: nobody looks)
+    unsigned *fault = nullptr;
     // the next ticket: every launch that uses the slots takes its own
     unsigned nextSlotTicket() const {
         unsigned t = ++*slotTicketSource;
@@ -294,5 +297,7 @@ bool launchRandom(hipStream_t stream, int opNum, const RngState &rng, const T *x
 void launchRngDump(hipStream_t stream, const RngState &rng, Long start, Long n, unsigned long long *out);
 // plain copy with 16-byte vectors (bytes is rounded down to a multiple of 16 plus a byte tail)
 void launchCopy(hipStream_t stream, void *dst, const void *src, Long bytes);
+// zero fill of `bytes` bytes (a multiple of 16, at a 16-byte boundary) by a kernel: safe to record where a memset node is not
+void launchFill(hipStream_t stream, void *dst, size_t bytes);
 
 }  // namespace nd4j_amd

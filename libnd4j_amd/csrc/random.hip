@@ -661,6 +661,15 @@ void launchCopy(hipStream_t s, void *dst, const void *src, Long bytes) {
                        reinterpret_cast<const unsigned char *>(src) + nvec * 16, tail);
 }
 
+__global__ void __launch_bounds__(kBlock) fillZeroKernel(uint4 *dst, Long nvec) {
+    for (Long i = (Long)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (Long)gridDim.x * kBlock) dst[i] = make_uint4(0, 0, 0, 0);
+}
+void launchFill(hipStream_t s, void *dst, size_t bytes) {
+    const Long nvec = (Long)(bytes / 16);
+    if (nvec <= 0) return;
+    ND4J_LAUNCH(fillZeroKernel, dim3(gridFor(nvec, kBlock, kGridCap)), dim3(kBlock), 0, s, reinterpret_cast<uint4 *>(dst), nvec);
+}
+
 #define INST(T)                                                                                                   \
     template bool launchRandom<T>(hipStream_t, int, const RngState &, const T *, const T *, T *, const T *,        \
                                   const RandomPlan &, int, bool);

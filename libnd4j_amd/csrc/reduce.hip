@@ -239,6 +239,12 @@ void *scratchOnCurrentDevice() {
 
 void prepareNoAllocScratch() { (void)scratchOnCurrentDevice(); }
 
+// The two-launch form this entry point takes (flatKernel into partials, flatFinish over them) and the one-launch form of
+// execReduceFloat fold the same blocks in the same order only while every block's accumulator fits the scratch array:
+// the "bit for bit" promise of the header rests on that.
+static_assert((kNoAllocScratchBytes - kNoAllocPartialsOffset) / sizeof(float) >= kFlatMaxBlocks,
+              "the no-allocation scratch must hold one float accumulator per block of the largest whole-array grid");
+
 bool launchReduceScalarNoAlloc(hipStream_t s, int opNum, const float *x, const float *extra, float *z, const FlatPlan &plan) {
     char *base = reinterpret_cast<char *>(scratchOnCurrentDevice());
     Workspace ws;

@@ -173,10 +173,12 @@ __global__ void __launch_bounds__(kBlock) reduce3Kernel(const T *x, const T *y, 
         Acc3Merge<C> mg;
         Acc acc;
         acc.r = acc.e0 = acc.e1 = (C)0;
-        mergeSlots<Acc3Merge<C>>(mg, acc, slots, threadIdx.x, kBlock, (int)gridDim.x, slotTicket);
+        // (the stream's fault word lies 64 bytes behind the tagged words of its pinned block)
+        unsigned *fault = signal != nullptr ? reinterpret_cast<unsigned *>(signal + 8) : nullptr;
+        const bool missing = slotsWereMissing(mergeSlots<Acc3Merge<C>>(mg, acc, slots, threadIdx.x, kBlock, (int)gridDim.x, slotTicket), fault);
         acc = blockMerge<Acc3Merge<C>>(mg, acc, smem);
         if (threadIdx.x == 0) {
-            const T r = fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, pl.runLength));
+            const T r = missing ? notANumber<T>() : fromCompute<T>(Reduce3Op<C, OP>::finalize(acc, pl.runLength));
             z[0] = r;
             signalResult(signal, ticket, r);
         }

@@ -23,6 +23,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "elementwise.cuh"
 #include "types.h"
 #include "view.h"
@@ -256,13 +258,9 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
             // would keep hitting the same few memory channels: each range is walked from a different row, wrapping round.
             const Long span = j1 - j0;
             const Long turn = span >= 8 * WAVES ? (((Long)blockIdx.y * 3) % (span / (4 * WAVES))) * (4 * WAVES) : 0;
-            for (int part = 0; part < 2; part++) {
-                const Long a = part == 0 ? j0 + turn : j0, b = part == 0 ? j1 : j0 + turn;
-                // (each part is walked in ascending order with accumulators of its own; the second part's rows lie before
-                // the first's)
-                Acc cur[VEC];
-#pragma unroll
-                for (int e = 0; e < VEC; e++) cur[e] = pe[e].init(x + off[e]);
+            // (the first part is walked in ascending order from fresh accumulators; the second part's rows lie before the
+            // first's, so its elements are folded by the general rule)
+            auto walk = [&](Long a, Long b, auto ascending) {
                 Long j = a + wave;
                 for (; j + 3 * WAVES < b; j += 4 * WAVES) {
                     Pack<T> pk[4];
@@ -271,18 +269,29 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
 #pragma unroll
                     for (int u = 0; u < 4; u++) {
 #pragma unroll
-                        for (int e = 0; e < VEC; e++) foldNext(pe[e], cur[e], toCompute(pk[u].v[e]), j + u * WAVES);
+                        for (int e = 0; e < VEC; e++) {
+                            if constexpr (decltype(ascending)::value) foldNext(pe[e], acc[e], toCompute(pk[u].v[e]), j + u * WAVES);
+                            else pe[e].accumulate(acc[e], toCompute(pk[u].v[e]), j + u * WAVES);
+                        }
                     }
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) pe[e].checkpoint(cur[e]);
+                    for (int e = 0; e < VEC; e++) pe[e].checkpoint(acc[e]);
                 }
                 for (; j < b; j += WAVES) {
                     Pack<T> pk = loadPack(reinterpret_cast<const Pack<T> *>(base + j * tadEws));
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) { foldNext(pe[e], cur[e], toCompute(pk.v[e]), j); pe[e].checkpoint(cur[e]); }
+                    for (int e = 0; e < VEC; e++) {
+                        if constexpr (decltype(ascending)::value) foldNext(pe[e], acc[e], toCompute(pk.v[e]), j);
+                        else pe[e].accumulate(acc[e], toCompute(pk.v[e]), j);
+                        pe[e].checkpoint(acc[e]);
+                    }
                 }
-#pragma unroll
-                for (int e = 0; e < VEC; e++) acc[e] = part == 0 ? cur[e] : pe[e].combine(acc[e], cur[e]);
+            };
+            if constexpr (HasAscending<Pol>::value) {
+                walk(j0 + turn, j1, std::true_type());
+                walk(j0, j0 + turn, std::false_type());
+            } else {
+                for (int part = 0; part < 2; part++) walk(part == 0 ? j0 + turn : j0, part == 0 ? j1 : j0 + turn, std::false_type());
             }
         } else {
 #pragma unroll
@@ -497,10 +506,15 @@ template <typename T> __device__ __forceinline__ void signalResult(unsigned long
 static constexpr unsigned kFlatGroup = 32;          // blocks per first-level counter
 static constexpr unsigned kFlatCounterStride = 32;  // counters are this many 32-bit words (128 bytes) apart
 static constexpr unsigned kFlatMaxBlocks = 2048;    // 1 + kFlatMaxBlocks / kFlatGroup counters exist
-template <typename A> __device__ __forceinline__ void publishSlots(unsigned long long *slot, const A &a, unsigned ticket) {
+// How many 32-bit words of a policy's accumulator travel through the slots: all of them, unless the policy says that
+// only the first kSlotWords matter (trailing padding stays at home; the receiver fills it with zeros).
+template <class Pol, typename = void> struct SlotWords { static constexpr int value = sizeof(typename Pol::Acc) / 4; };
+template <class Pol> struct SlotWords<Pol, decltype((void)Pol::kSlotWords)> { static constexpr int value = Pol::kSlotWords; };
+
+template <typename A, int W = sizeof(A) / 4>
+__device__ __forceinline__ void publishSlots(unsigned long long *slot, const A &a, unsigned ticket) {
     static_assert(sizeof(A) % 4 == 0, "accumulator must be a multiple of 4 bytes");
-    constexpr int W = sizeof(A) / 4;
-    struct Words { unsigned w[W]; };
+    struct Words { unsigned w[sizeof(A) / 4]; };
     const Words in = __builtin_bit_cast(Words, a);
 #pragma unroll
     for (int i = 0; i < W; i++)
@@ -508,23 +522,34 @@ template <typename A> __device__ __forceinline__ void publishSlots(unsigned long
 }
 // One word of a slot group: waits (bounded) until it carries `ticket`, starting from the value `v` already loaded.  Only
 // called for groups whose writer has already issued its stores, so the wait ends as soon as they land.
-__device__ __forceinline__ unsigned awaitSlot(const unsigned long long *slot, unsigned long long v, unsigned ticket) {
+// `missing` is set when the wait ran out (seconds: only a launch that has gone wrong gets there).
+__device__ __forceinline__ unsigned awaitSlot(const unsigned long long *slot, unsigned long long v, unsigned ticket, bool &missing) {
     for (int tries = 0; (unsigned)(v >> 32) != ticket && tries < (1 << 22); tries++) {
         __builtin_amdgcn_s_sleep(1);
         v = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    if ((unsigned)(v >> 32) != ticket) missing = true;
     return (unsigned)v;
 }
+// What the merging block does when a slot never arrived (all its threads call this together): true tells the caller to
+// store NaN instead of a number made of stale words; the stream's fault word, when there is one, lets the host report it.
+__device__ __forceinline__ bool slotsWereMissing(bool missing, unsigned *fault) {
+    const bool any = __syncthreads_or(missing ? 1 : 0) != 0;
+    if (any && threadIdx.x == 0 && fault != nullptr) __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    return any;
+}
+template <typename T> __device__ __forceinline__ T notANumber() { return fromCompute<T>((typename Compute<T>::type)__builtin_nanf("")); }
 // Merges the slot groups first, first + stride, ... (count of them in all) into acc, in that order.  The loads of
 // several groups are issued together: they bypass the caches, and one after the other their latencies would add up to
 // more than the second launch they replace.
 template <class Pol>
-__device__ __forceinline__ void mergeSlots(const Pol &pol, typename Pol::Acc &acc, const unsigned long long *slots, int first,
+__device__ __forceinline__ bool mergeSlots(const Pol &pol, typename Pol::Acc &acc, const unsigned long long *slots, int first,
                                            int stride, int count, unsigned ticket) {
+    bool missing = false;
     typedef typename Pol::Acc Acc;
-    constexpr int W = sizeof(Acc) / 4;
+    constexpr int W = SlotWords<Pol>::value;
     constexpr int G = W <= 2 ? 8 : (W <= 4 ? 4 : 2);
-    struct Words { unsigned w[W]; };
+    struct Words { unsigned w[sizeof(Acc) / 4]; };
     for (int i0 = first; i0 < count; i0 += stride * G) {
         unsigned long long v[G][W];
 #pragma unroll
@@ -539,13 +564,14 @@ __device__ __forceinline__ void mergeSlots(const Pol &pol, typename Pol::Acc &ac
         for (int g = 0; g < G; g++) {
             const int i = i0 + g * stride;
             if (i < count) {
-                Words out;
+                Words out = {};
 #pragma unroll
-                for (int w = 0; w < W; w++) out.w[w] = awaitSlot(slots + (size_t)i * W + w, v[g][w], ticket);
+                for (int w = 0; w < W; w++) out.w[w] = awaitSlot(slots + (size_t)i * W + w, v[g][w], ticket, missing);
                 acc = pol.combine(acc, __builtin_bit_cast(Acc, out));
             }
         }
     }
+    return missing;
 }
 
 // One thread of every block of a one-dimensional grid (of at most kFlatMaxBlocks blocks) calls this once, after it has
@@ -579,7 +605,8 @@ template <class Pol, bool CLEAR = false>
 __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol::T *x, typename Pol::Acc *partials,
                                                      Long n, int strided, Long ews, DimMap xm, typename Pol::T *z,
                                                      unsigned long long *signal, unsigned ticket, unsigned long long *slots,
-                                                     unsigned *counter, unsigned slotTicket, typename Pol::T *cleared = nullptr) {
+                                                     unsigned *counter, unsigned slotTicket, typename Pol::T *cleared = nullptr,
+                                                     unsigned *fault = nullptr) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
@@ -669,18 +696,18 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
         if (threadIdx.x == 0) partials[blockIdx.x] = acc;
         return;
     }
-    constexpr int W = sizeof(Acc) / 4;
+    constexpr int W = SlotWords<Pol>::value;
     if (threadIdx.x == 0) {
-        publishSlots(slots + (size_t)blockIdx.x * W, acc, slotTicket);
+        publishSlots<Acc, W>(slots + (size_t)blockIdx.x * W, acc, slotTicket);
         mergeHere = countedInLast(counter);
     }
     __syncthreads();
     if (!mergeHere) return;
     acc = pol.init(x);
-    mergeSlots<Pol>(pol, acc, slots, threadIdx.x, kBlock, (int)gridDim.x, slotTicket);
+    const bool missing = slotsWereMissing(mergeSlots<Pol>(pol, acc, slots, threadIdx.x, kBlock, (int)gridDim.x, slotTicket), fault);
     acc = blockMerge<Pol>(pol, acc, smem);
     if (threadIdx.x == 0) {
-        const typename Pol::T r = pol.finalize(acc, n);
+        const typename Pol::T r = missing ? notANumber<T>() : pol.finalize(acc, n);
         z[0] = r;
         signalResult(signal, ticket, r);
     }
@@ -847,7 +874,7 @@ inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, type
     // longer; maxima and index reductions lose a third that way, so a policy asks for it: kFlatBlocks)
     int grid = gridFor(pl.n, perBlock, PolFlatBlocks<Pol>::value);
     const bool oneLaunch = ws.slots != nullptr && ws.counter != nullptr && ws.slotTicketSource != nullptr;
-    size_t maxBlocks = oneLaunch ? ws.slotBytes / (sizeof(Acc) / 4 * sizeof(unsigned long long)) : ws.bytes / sizeof(Acc);
+    size_t maxBlocks = oneLaunch ? ws.slotBytes / (SlotWords<Pol>::value * sizeof(unsigned long long)) : ws.bytes / sizeof(Acc);
     if ((size_t)grid > maxBlocks) grid = (int)maxBlocks;
     if (grid < 1) grid = 1;
     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
@@ -855,11 +882,11 @@ inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, type
         if constexpr (PolClears<Pol>::value)
             ND4J_LAUNCH((flatKernel<Pol, true>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, 1, (Long)1, pl.xm, z,
                                ws.signal, ws.ticket, oneLaunch ? ws.slots : nullptr, ws.counter,
-                               oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u, cleared);
+                               oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u, cleared, ws.fault);
     } else {
         ND4J_LAUNCH((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
                            pl.ews, pl.xm, z, ws.signal, ws.ticket, oneLaunch ? ws.slots : nullptr, ws.counter,
-                           oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u, (typename Pol::T *)nullptr);
+                           oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u, (typename Pol::T *)nullptr, ws.fault);
     }
     if (grid > 1 && !oneLaunch)
         ND4J_LAUNCH((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n, ws.signal, ws.ticket);

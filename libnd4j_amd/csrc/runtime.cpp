@@ -72,12 +72,26 @@ bool hostInts(const int *arg, int count, std::vector<int> &out, hipStream_t s) {
     return true;
 }
 
+// A kernel whose merging block gave up waiting for another block's partial result stores a non-zero word in the stream's
+// pinned block (and NaN as its result): reported by the next call on the stream that looks (scalar-returning calls, and
+// every call in debug mode).
+static void throwOnFault(unsigned *fault, const char *what) {
+    if (fault == nullptr) return;
+    volatile unsigned *f = fault;
+    if (*f == 0) return;
+    *f = 0;
+    throw std::runtime_error(std::string(what) + ": a block's partial result did not reach the block that merges them "
+                             "(a whole-array reduction on this stream gave up after its bounded wait); its result is NaN");
+}
+static unsigned *faultWordIfAny(hipStream_t s);
+
 void checkLaunch(const char *what, hipStream_t s) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) throwHip(what, e);
     if (environment().debug.load()) {
         e = hipStreamSynchronize(s);
         if (e != hipSuccess) throwHip(what, e);
+        throwOnFault(faultWordIfAny(s), what);
     }
 }
 
@@ -111,17 +125,12 @@ size_t gTadCacheBytes = 0;
 const size_t kTadCacheLimitBytes = (size_t)1 << 30;
 const size_t kTadCacheLimitEntries = 16384;
 
-void dropTadCacheLocked() {
-    int current = 0, count = 0;
-    (void)hipGetDevice(&current);
-    (void)hipGetDeviceCount(&count);
-    for (int d = 0; d < count; d++) {
-        if (hipSetDevice(d) == hipSuccess) (void)hipDeviceSynchronize();
-    }
-    (void)hipSetDevice(current);
-    // A call that still holds an entry keeps it (and its device table) until it returns; its kernel may still be queued
-    // then, which is safe because ~CachedTad's hipFree waits for the device's outstanding work before it releases memory.
-    gTadCache.clear();
+// Empties the cache into `old`, which the caller destroys after it has let go of gMutex: an entry's device table is
+// released by hipFree, which waits for the device's outstanding work first (kernels queued by calls that have already
+// returned may still read the table), and that wait must not hold up every other thread of the library.  A call that
+// still holds an entry keeps it alive until it returns.
+void takeTadCacheLocked(std::map<std::vector<Long>, std::shared_ptr<CachedTad> > &old) {
+    old.swap(gTadCache);
     gTadCacheBytes = 0;
 }
 }  // namespace
@@ -149,6 +158,27 @@ Workspace workspaceFor(hipStream_t s, size_t minBytes) {
 }
 
 namespace {
+struct PinnedSlot {
+    void *block = nullptr;  // 256 bytes: value at 0, tagged words at 128, fault word at kPinnedFaultOffset
+    unsigned ticket = 0;
+};
+const size_t kPinnedFaultOffset = 192;
+std::map<std::pair<int, hipStream_t>, PinnedSlot> gPinnedSlots;
+PinnedSlot &pinnedSlotLocked(hipStream_t s) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    PinnedSlot &p = gPinnedSlots[std::make_pair(dev, s)];
+    if (p.block == nullptr) {
+        // coherent: the device's stores reach host memory while the kernel runs, not only when it has ended
+        hipError_t e = hipHostMalloc(&p.block, 256, hipHostMallocCoherent);
+        if (e != hipSuccess) { p.block = nullptr; throwHip("pinned scalar slot", e); }
+        std::memset(p.block, 0, 256);
+    }
+    return p;
+}
+}  // namespace
+
+namespace {
 struct FlatSlots {
     void *block = nullptr;  // kFlatSlotBytes of slots, then kFlatCounterBytes of block counters, then kFlatStateBytes of row states
     unsigned ticket = 0;
@@ -159,6 +189,12 @@ const size_t kFlatCounterBytes = 16u << 10;  // 65 counters, 128 bytes apart
 const size_t kFlatStateBytes = 256u << 10;   // 2048 row (or row group) states, 128 bytes apart
 std::map<std::pair<int, hipStream_t>, FlatSlots> gFlatSlots;
 }  // namespace
+
+// Tickets tag the slot words and row states of one launch; the cooperative softmax kernels keep 30 bits of them.  Slots
+// are never cleared between launches, so a word left behind 2^30 tickets ago would pass for a fresh one: shortly before
+// the counter crosses a multiple of 2^30 (a call takes a handful of tickets) the slots and states are cleared on the
+// stream - behind everything that still uses them - and the counter is moved past the boundary.
+const unsigned kTicketPeriod = 1u << 30, kTicketMargin = 256;
 
 void addFlatSlots(Workspace &w, hipStream_t s) {
     int dev = 0;
@@ -171,6 +207,12 @@ void addFlatSlots(Workspace &w, hipStream_t s) {
         e = hipMemset(f.block, 0, kFlatSlotBytes + kFlatCounterBytes + kFlatStateBytes);
         if (e != hipSuccess) throwHip("reduction slots clearing", e);
     }
+    if ((f.ticket & (kTicketPeriod - 1)) >= kTicketPeriod - kTicketMargin) {
+        launchFill(s, f.block, kFlatSlotBytes);
+        launchFill(s, reinterpret_cast<char *>(f.block) + kFlatSlotBytes + kFlatCounterBytes, kFlatStateBytes);
+        f.ticket = (f.ticket | (kTicketPeriod - 1)) + 1;  // the next ticket is this + 1 (zero is skipped by nextSlotTicket)
+    }
+    w.fault = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(pinnedSlotLocked(s).block) + kPinnedFaultOffset);
     w.slots = reinterpret_cast<unsigned long long *>(f.block);
     w.slotBytes = kFlatSlotBytes;
     w.counter = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(f.block) + kFlatSlotBytes);
@@ -179,25 +221,14 @@ void addFlatSlots(Workspace &w, hipStream_t s) {
     w.slotTicketSource = &f.ticket;  // map nodes stay where they are
 }
 
-namespace {
-struct PinnedSlot {
-    void *block = nullptr;  // 256 bytes: value at 0, flag word at 128
-    unsigned ticket = 0;
-};
-PinnedSlot &pinnedSlotLocked(hipStream_t s) {
-    static std::map<std::pair<int, hipStream_t>, PinnedSlot> slots;
+static unsigned *faultWordIfAny(hipStream_t s) {
     int dev = 0;
     (void)hipGetDevice(&dev);
-    PinnedSlot &p = slots[std::make_pair(dev, s)];
-    if (p.block == nullptr) {
-        // coherent: the device's stores reach host memory while the kernel runs, not only when it has ended
-        hipError_t e = hipHostMalloc(&p.block, 256, hipHostMallocCoherent);
-        if (e != hipSuccess) { p.block = nullptr; throwHip("pinned scalar slot", e); }
-        std::memset(p.block, 0, 256);
-    }
-    return p;
+    std::lock_guard<std::mutex> lock(gMutex);
+    auto it = gPinnedSlots.find(std::make_pair(dev, s));
+    if (it == gPinnedSlots.end() || it->second.block == nullptr) return nullptr;
+    return reinterpret_cast<unsigned *>(reinterpret_cast<char *>(it->second.block) + kPinnedFaultOffset);
 }
-}  // namespace
 
 void *pinnedScalarFor(hipStream_t s) {
     std::lock_guard<std::mutex> lock(gMutex);
@@ -209,6 +240,8 @@ ScalarSignal nextScalarSignal(hipStream_t s) {
     PinnedSlot &p = pinnedSlotLocked(s);
     ScalarSignal sig;
     sig.words = reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.block) + 128);
+    sig.plain = p.block;
+    sig.fault = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(p.block) + kPinnedFaultOffset);
     sig.ticket = ++p.ticket;
     if (sig.ticket == 0) sig.ticket = ++p.ticket;  // zero is what a fresh slot holds
     return sig;
@@ -254,14 +287,48 @@ void takeScalar(const ScalarSignal &sig, hipStream_t s, const char *what, void *
     }
     std::atomic_thread_fence(std::memory_order_acquire);
     if (!have && sig.words != nullptr) have = arrived();  // the stream has drained: the words are there if they were written
+    throwOnFault(sig.fault, what);
     if (have) {
         unsigned w[4] = {0, 0, 0, 0};
         for (int i = 0; i < words && i < 4; i++) w[i] = (unsigned)tagged[i];
         std::memcpy(value, w, bytes);
-    } else {
+    } else if (sig.plain != nullptr) {
         // no kernel of this call tagged the words: take the plain copy at the start of the block
-        std::memcpy(value, reinterpret_cast<const char *>(sig.words) - 128, bytes);
+        std::memcpy(value, sig.plain, bytes);
+    } else {
+        throw std::runtime_error(std::string(what) + ": no scalar slot to read the result from");
     }
+}
+
+void releaseStreamResources(hipStream_t s) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const auto key = std::make_pair(dev, s);
+    Workspace w;
+    w.ptr = nullptr;
+    void *slots = nullptr, *pinned = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(gMutex);
+        auto wi = gWorkspaces.find(key);
+        if (wi != gWorkspaces.end()) { w = wi->second; gWorkspaces.erase(wi); }
+        auto fi = gFlatSlots.find(key);
+        if (fi != gFlatSlots.end()) { slots = fi->second.block; gFlatSlots.erase(fi); }
+        auto pi = gPinnedSlots.find(key);
+        if (pi != gPinnedSlots.end()) { pinned = pi->second.block; gPinnedSlots.erase(pi); }
+    }
+    if (w.ptr == nullptr && slots == nullptr && pinned == nullptr) return;
+    hipError_t e = hipStreamSynchronize(s);  // what is queued on the stream may still use them
+    if (e != hipSuccess) throwHip("releaseStreamResources", e);
+    if (w.ptr != nullptr) (void)hipFree(w.ptr);
+    if (slots != nullptr) (void)hipFree(slots);
+    if (pinned != nullptr) (void)hipHostFree(pinned);
+}
+
+void setSlotTicketForTesting(hipStream_t s, unsigned value) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    std::lock_guard<std::mutex> lock(gMutex);
+    gFlatSlots[std::make_pair(dev, s)].ticket = value;
 }
 
 bool resolveTad(Nd4jPointer *extra, int hostSlot, int offsetSlot, const Long *hostXInfo, const int *dimension,
@@ -289,13 +356,14 @@ bool resolveTad(Nd4jPointer *extra, int hostSlot, int offsetSlot, const Long *ho
     (void)hipGetDevice(&dev);
     key.push_back(dev);  // the offsets live in this device's memory
 
-    std::lock_guard<std::mutex> lock(gMutex);
+    std::map<std::vector<Long>, std::shared_ptr<CachedTad> > dropped;  // destroyed after the lock below is gone
+    std::unique_lock<std::mutex> lock(gMutex);
     auto it = gTadCache.find(key);
     std::shared_ptr<CachedTad> c;
     if (it != gTadCache.end()) {
         c = it->second;
     } else {
-        if (gTadCache.size() >= kTadCacheLimitEntries || gTadCacheBytes >= kTadCacheLimitBytes) dropTadCacheLocked();
+        if (gTadCache.size() >= kTadCacheLimitEntries || gTadCacheBytes >= kTadCacheLimitBytes) takeTadCacheLocked(dropped);
         c = std::make_shared<CachedTad>();
         computeTad(hostXInfo, dims.data(), dimLen, c->pack, true);
         c->tadLength = tadLengthOf(hostXInfo, dims.data(), dimLen);
@@ -314,6 +382,8 @@ bool resolveTad(Nd4jPointer *extra, int hostSlot, int offsetSlot, const Long *ho
     out.devOffsets = c->devOffsets;
     out.numTads = c->pack.numTads;
     out.tadLength = c->tadLength;
+    lock.unlock();
+    dropped.clear();
     return true;
 }
 

@@ -91,9 +91,17 @@ void *pinnedScalarFor(hipStream_t s);
 struct ScalarSignal {
     unsigned long long *words = nullptr;
     unsigned ticket = 0;
+    const void *plain = nullptr;  // the start of the pinned block: the plainly stored copy of the value
+    unsigned *fault = nullptr;    // the stream's fault word (see Workspace::fault)
 };
 ScalarSignal nextScalarSignal(hipStream_t s);
 void takeScalar(const ScalarSignal &sig, hipStream_t s, const char *what, void *value, size_t bytes);
+
+// Frees what the library keeps for a stream of the current device (workspace, reduction slots, pinned scalar block) once
+// the stream has drained; a later call on the stream allocates afresh.  For hosts that create and destroy streams.
+void releaseStreamResources(hipStream_t s);
+// test aid: the last ticket handed out for the stream's reduction slots
+void setSlotTicketForTesting(hipStream_t s, unsigned value);
 
 // TAD tables resolved for a call: host shapeInfo of one TAD + device offsets.
 struct ResolvedTad {

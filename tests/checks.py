@@ -254,6 +254,45 @@ def check_half_vectors(be, exact):
     cmp(np.array([be.reduce_scalar(1, yh, hi)], h), "reduce_sum_y")
 
 
+def check_half_reduction_vectors(be, exact):
+    """fp16 reductions, index reductions and summary statistics against what the reference's own float16 loops return
+    (they accumulate in fp16, cpu/reduce.cpp:150-156 with T = float16).  `exact`: the CPU checkers reproduce them bit for
+    bit; the HIP path accumulates in fp32 (statistics in double) and rounds once, and is held to the 1e-2 of fp16 -
+    index reductions bit for bit."""
+    from golden_inputs import half_reduction_input
+    vec = load_json("ref_vectors.json")["ops"]["f16_reductions_12x16"]
+    h = np.float16
+    x = half_reduction_input()
+    assert np.array_equal(x.view(np.uint16), from_hexbits(vec["x"], h).view(np.uint16))
+    info = shape_info_np([12, 16])
+
+    def cmp(got, want_hex, what, bitwise):
+        want = from_hexbits(want_hex, h)
+        got = np.asarray(got, h).reshape(want.shape)
+        if bitwise:
+            assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), what
+        else:
+            g, w = got.astype(np.float64), want.astype(np.float64)
+            assert np.all(np.abs(g - w) <= HALF_RTOL * np.abs(w)), (what, np.abs(g - w).max())
+
+    for op in (0, 1, 3, 4, 5, 6):
+        v = vec["reduce_%d" % op]
+        cmp(be.reduce(op, x, info, None, [1], 12), v["dim1"], ("reduce", op, 1), exact)
+        cmp(be.reduce(op, x, info, None, [0], 16), v["dim0"], ("reduce", op, 0), exact)
+        cmp([be.reduce_scalar(op, x, info)], v["scalar"], ("reduce", op, "scalar"), exact)
+    for op in (0, 1):
+        v = vec["indexreduce_%d" % op]
+        cmp(be.indexreduce(op, x, info, None, [1], 12), v["dim1"], ("indexreduce", op, 1), True)
+        cmp(be.indexreduce(op, x, info, None, [0], 16), v["dim0"], ("indexreduce", op, 0), True)
+        cmp([be.indexreduce_scalar(op, x, info)], v["scalar"], ("indexreduce", op, "scalar"), True)
+    for op in (0, 1):
+        for bias in (0, 1):
+            v = vec["summarystats_%d_%d" % (op, bias)]
+            cmp(be.summarystats(op, bias, x, info, [1], 12), v["dim1"], ("summarystats", op, bias, 1), exact)
+            cmp(be.summarystats(op, bias, x, info, [0], 16), v["dim0"], ("summarystats", op, bias, 0), exact)
+            cmp([be.summarystats_scalar(op, bias, x, info)], v["scalar"], ("summarystats", op, bias, "scalar"), exact)
+
+
 def check_rng_vectors(be, float_ulp=ELEMENTWISE_ULP, big=True):
     vec = load_json("ref_vectors.json")["rng"]
     u64 = np.uint64

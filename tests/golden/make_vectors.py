@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(HERE))
 import cpu_ref  # noqa: E402
 from golden_inputs import (BROADCAST_OPS, INDEX_OPS, PAIRWISE_OPS, REDUCE_OPS, SCALAR_OPS, SCALAR_VALUES, TRANSFORM_OPS,  # noqa: E402
-                           hexbits, op_extra, pairwise_inputs, reduce_input, shape_info_np, transform_input, whole_array_cases)
+                           half_reduction_input, hexbits, op_extra, pairwise_inputs, reduce_input, shape_info_np, transform_input, whole_array_cases)
 
 
 def main():
@@ -223,6 +223,32 @@ def main():
     h["broadcast_add_row"] = hexbits(z)
     h["reduce_sum_y"] = hexbits(np.array([ref.reduce_scalar(1, yh, hi, None)], np.float16))
     ops["f16_2x4"] = h
+    # fp16 reductions at a size where the reference's accumulation in fp16 (every update rounds to half,
+    # cpu/reduce.cpp:150-156, types/float16.h:391-394) is still within a few 1e-3 of the exact value: rows of 16, columns
+    # of 12, 192 elements in all, values in [0.5, 1.5)
+    xr = half_reduction_input()
+    ri = shape_info_np([12, 16])
+    hr = {"x": hexbits(xr)}
+    for op in (0, 1, 3, 4, 5, 6):
+        z1, z0 = np.zeros(12, np.float16), np.zeros(16, np.float16)
+        ref.reduce(op, xr, ri, None, z1, shape_info_np([1, 12]), [1])
+        ref.reduce(op, xr, ri, None, z0, shape_info_np([1, 16]), [0])
+        hr["reduce_%d" % op] = {"dim1": hexbits(z1), "dim0": hexbits(z0),
+                                "scalar": hexbits(np.array([ref.reduce_scalar(op, xr, ri, None)], np.float16))}
+    for op in (0, 1):
+        z1, z0 = np.zeros(12, np.float16), np.zeros(16, np.float16)
+        ref.indexreduce(op, xr, ri, None, z1, shape_info_np([1, 12]), [1])
+        ref.indexreduce(op, xr, ri, None, z0, shape_info_np([1, 16]), [0])
+        hr["indexreduce_%d" % op] = {"dim1": hexbits(z1), "dim0": hexbits(z0),
+                                     "scalar": hexbits(np.array([ref.indexreduce_scalar(op, xr, ri, None)], np.float16))}
+    for op in (0, 1):
+        for bias in (0, 1):
+            z1, z0 = np.zeros(12, np.float16), np.zeros(16, np.float16)
+            ref.summarystats(op, bias, xr, ri, z1, shape_info_np([1, 12]), [1])
+            ref.summarystats(op, bias, xr, ri, z0, shape_info_np([1, 16]), [0])
+            hr["summarystats_%d_%d" % (op, bias)] = {"dim1": hexbits(z1), "dim0": hexbits(z0),
+                                                     "scalar": hexbits(np.array([ref.summarystats_scalar(op, bias, xr, ri)], np.float16))}
+    ops["f16_reductions_12x16"] = hr
     # whole-array transforms: Col2Im, Im2col, Histogram, Reverse, Pooling2D
     wa = {}
     for name, op, x, x_info, z_info, extra, z0 in whole_array_cases():

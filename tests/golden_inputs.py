@@ -155,3 +155,9 @@ def whole_array_cases():
     cases.append(("reverse_vector", 70, values(37), shape_info_np([1, 37]), shape_info_np([1, 37]), None, np.zeros(37, f)))
     cases.append(("reverse_matrix_c_to_f", 70, values(35), shape_info_np([5, 7]), shape_info_np([5, 7], "f"), None, np.zeros(35, f)))
     return cases
+
+
+def half_reduction_input():
+    """192 fp16 values in [0.5, 1.5) (a [12, 16] matrix): short enough that sums accumulated in fp16, as the reference's
+    float16 loops accumulate them, stay within a few 1e-3 of the exact ones."""
+    return (0.5 + np.random.RandomState(5).rand(192)).astype(np.float16)

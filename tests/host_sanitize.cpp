@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <set>
+#include <stdexcept>
 #include <vector>
 
 typedef long long Long;
@@ -111,6 +112,37 @@ int main() {
         const FastDiv f(d);
         unsigned rem;
         if (f.div(v) != v / d || f.divmod(v, rem) != v / d || rem != v % d) return fail("FastDiv", it);
+    }
+    // Extents that do not fit 32 bits: a map of one dimension clamps its extent (the kernels never divide by it), one of
+    // several dimensions refuses instead of wrapping round
+    {
+        const Long big = (Long)1 << 33;
+        Long shape1[1] = {big}, stride1[1] = {1};
+        DimMap m1;
+        ownCanon(1, shape1, stride1, m1);
+        if (m1.rank != 1 || m1.shape[0] != 0xffffffffu) return fail("one long dimension", 0);
+        Long shape2[2] = {big, 3}, dense2[2] = {3, 1}, padded2[2] = {4, 1};
+        ownCanon(2, shape2, dense2, m1);  // merges into one run of 3 * 2^33 elements
+        if (m1.rank != 1 || m1.shape[0] != 0xffffffffu || m1.stride[0] != 1) return fail("merged long dimension", 0);
+        bool threw = false;
+        try { ownCanon(2, shape2, padded2, m1); } catch (const std::invalid_argument &) { threw = true; }
+        if (!threw) return fail("a long dimension beside another one was not refused", 0);
+        const Long *strides[3] = {padded2, nullptr, padded2};
+        DimMap joint[3];
+        threw = false;
+        try { jointCanon(2, shape2, strides, joint); } catch (const std::invalid_argument &) { threw = true; }
+        if (!threw) return fail("jointCanon: a long dimension beside another one was not refused", 0);
+    }
+    // the common run length of up to three maps
+    {
+        DimMap a, b, c;
+        a.rank = 2; a.shape[0] = 7; a.shape[1] = 24; a.stride[0] = 100; a.stride[1] = 1;
+        b.rank = 1; b.shape[0] = 7 * 24; b.stride[0] = 1;
+        c.rank = 3; c.shape[0] = 7; c.shape[1] = 2; c.shape[2] = 12; c.stride[0] = 50; c.stride[1] = 20; c.stride[2] = 1;
+        const DimMap *abc[3] = {&a, &b, &c}, *ab[3] = {&a, &b, nullptr};
+        if (commonRunLength(abc) != 12 || commonRunLength(ab) != 24) return fail("commonRunLength", 0);
+        c.stride[2] = 2;
+        if (commonRunLength(abc) != 0) return fail("commonRunLength with a strided innermost dimension", 0);
     }
     std::printf("host sanitize run: ok\n");
     return 0;

@@ -120,31 +120,41 @@ def test_config3_summary_stats_and_softmax_chain(gpu, lib):
         sm = got.astype(np.float64).reshape(cols, rows).T
         assert np.all(got >= 0) and np.all(got <= 1)
         assert np.all(np.abs(sm.sum(axis=1) - 1.0) <= 1e-5)
-        # exp and the row sums differ by rounding only; 2 ULP on each factor and 1e-5 on the sum
+        # exp and the row sums differ by rounding only: 2 ULP on the exponential (2.4e-7), 1e-5 on the row sum and half
+        # an ULP on the quotient add up to 1.03e-5; the measured maxima are printed (pytest -s shows them)
+        bar = 1.0e-5 + 3 * 2.0 ** -23
         denom = np.maximum(np.abs(want.astype(np.float64)), 1e-30)
-        assert np.all(np.abs(got.astype(np.float64) - want) / denom <= 2e-5)
+        worst = {"chain vs reference": (np.abs(got.astype(np.float64) - want) / denom).max()}
+        assert worst["chain vs reference"] <= bar
         truth = np.exp(m - m.max(axis=1, keepdims=True))
         truth /= truth.sum(axis=1, keepdims=True)
-        assert np.all(np.abs(sm - truth) <= 2e-5 * truth + 1e-30)
+        worst["chain vs float64"] = (np.abs(sm - truth) / np.maximum(truth, 1e-30)).max()
+        assert worst["chain vs float64"] <= bar
         # the same softmax as one call, on the f-order matrix and on the same memory read as a c-order matrix
         fused = _run(w.case("softmax_fused_forder")).astype(np.float64).reshape(cols, rows).T
-        assert np.all(np.abs(fused - truth) <= 2e-5 * truth + 1e-30)
+        worst["fused f-order vs float64"] = (np.abs(fused - truth) / np.maximum(truth, 1e-30)).max()
+        assert worst["fused f-order vs float64"] <= bar
         assert np.all(np.abs(fused.sum(axis=1) - 1.0) <= 1e-5)
         mc = x.astype(np.float64).reshape(rows, cols)
         truth_c = np.exp(mc - mc.max(axis=1, keepdims=True))
         truth_c /= truth_c.sum(axis=1, keepdims=True)
         fused = _run(w.case("softmax_fused_corder")).astype(np.float64).reshape(rows, cols)
-        assert np.all(np.abs(fused - truth_c) <= 2e-5 * truth_c + 1e-30)
+        worst["fused c-order vs float64"] = (np.abs(fused - truth_c) / np.maximum(truth_c, 1e-30)).max()
+        assert worst["fused c-order vs float64"] <= bar
         want = w.case("softmax_fused_corder").cpu(lib).astype(np.float64).reshape(rows, cols)
-        assert np.all(np.abs(fused - want) <= 2e-5 * np.maximum(want, 1e-30))
+        worst["fused c-order vs reference"] = (np.abs(fused - want) / np.maximum(want, 1e-30)).max()
+        assert worst["fused c-order vs reference"] <= bar
         logsm = _run(w.case("logsoftmax_fused_corder")).astype(np.float64).reshape(rows, cols)
-        assert np.all(np.abs(logsm - np.log(truth_c)) <= 2e-5 * np.abs(np.log(truth_c)) + 1e-6)
+        # (a logarithm near zero has no relative accuracy to speak of: 1e-5 relative plus 1e-6 absolute)
+        assert np.all(np.abs(logsm - np.log(truth_c)) <= 1e-5 * np.abs(np.log(truth_c)) + 1e-6)
         # few long rows: the same memory read as [rows / 64, cols * 64]
         ml = x.astype(np.float64).reshape(rows // 64, cols * 64)
         truth_l = np.exp(ml - ml.max(axis=1, keepdims=True))
         truth_l /= truth_l.sum(axis=1, keepdims=True)
         fused = _run(w.case("softmax_fused_long_rows")).astype(np.float64).reshape(rows // 64, cols * 64)
-        assert np.all(np.abs(fused - truth_l) <= 2e-5 * truth_l + 1e-30)
+        worst["fused long rows vs float64"] = (np.abs(fused - truth_l) / np.maximum(truth_l, 1e-30)).max()
+        assert worst["fused long rows vs float64"] <= bar
+        print("softmax, largest relative differences:", ", ".join("%s %.3g" % kv for kv in sorted(worst.items())))
         assert np.all(np.abs(fused.sum(axis=1) - 1.0) <= 1e-5)
         # IsMax: one-hot of the first maximum, whole array and per row; bit-exact
         xf = x.reshape(rows, cols)

@@ -42,6 +42,8 @@ def test_op_vectors(gpu):
 
 def test_half_vectors(gpu):
     checks.check_half_vectors(gpu, exact=False)
+    # reductions against the reference's own fp16-accumulating loops: within 1e-2, index reductions bit for bit
+    checks.check_half_reduction_vectors(gpu, exact=False)
 
 
 def test_rng_vectors(gpu):
@@ -1042,6 +1044,81 @@ def test_half_families(gpu, cpu):
     nan_in = np.array([np.nan, 1.0], h)
     out = gpu.transform(6, nan_in, shape_info_np([1, 2]), shape_info_np([1, 2]))
     assert out.view(np.uint16)[0] == 0x7fff
+
+
+def test_half_reductions_against_the_reference_loops(gpu, cpu):
+    """The reference's float16 reductions accumulate in fp16; this path in fp32.  On TADs short enough for the fp16
+    accumulation to stay inside the bar the two are compared directly, 1e-2, over several shapes and dimensions."""
+    rs = np.random.RandomState(29)
+    h = np.float16
+    for shape, dims in (([40, 16], [1]), ([16, 40], [0]), ([6, 12, 5], [1]), ([8, 3, 6], [0, 2]), ([5, 24], [1])):
+        n = int(np.prod(shape))
+        x = (0.5 + rs.rand(n)).astype(h)
+        info = shape_info_np(shape)
+        out_len = n // int(np.prod([shape[d] for d in dims]))
+        for op in (0, 1, 3, 5, 6):
+            g = gpu.reduce(op, x, info, None, dims, out_len).astype(np.float64)
+            c = cpu.reduce(op, x, info, None, dims, out_len).astype(np.float64)
+            assert np.all(np.abs(g - c) <= 1e-2 * np.abs(c)), (shape, dims, op, np.abs(g - c).max())
+        assert np.array_equal(gpu.indexreduce(0, x, info, None, dims, out_len), cpu.indexreduce(0, x, info, None, dims, out_len)), (shape, dims)
+        for op in (0, 1):
+            g = gpu.summarystats(op, 1, x, info, dims, out_len).astype(np.float64)
+            c = cpu.summarystats(op, 1, x, info, dims, out_len).astype(np.float64)
+            assert np.all(np.abs(g - c) <= 1e-2 * np.abs(c)), (shape, dims, op, "stats")
+
+
+def test_slot_tickets_across_the_points_where_the_slots_are_cleared(gpu):
+    """Whole-array reductions, the whole-array reduce3 and the cooperative softmax kernels tag what their blocks exchange
+    with a per-stream launch ticket (30 bits of it for the softmax), and the exchange area is not cleared between launches.
+    Data set A is run on the tickets just behind a multiple of 2^30; then the counter is put back to just before that
+    multiple - where a long-running process arrives 2^30 launches later - and data set B is run: it draws the same tickets
+    again, and must not see what A left behind (the library clears the area when the counter nears the boundary)."""
+    rs = np.random.RandomState(41)
+    n = 1 << 20
+    xi = shape_info_np([1, n])
+    rows = shape_info_np([4, 40000])
+    ex = gpu.dev.extra(xi)
+
+    def data():
+        x, y = rs.randn(n).astype(np.float32), rs.randn(n).astype(np.float32)
+        xr = rs.uniform(-5, 5, 4 * 40000).astype(np.float32)
+        r64 = xr.astype(np.float64).reshape(4, 40000)
+        soft = np.exp(r64 - r64.max(axis=1, keepdims=True))
+        return x, y, xr, soft / soft.sum(axis=1, keepdims=True)
+
+    def run(d, what):
+        x, y, xr, soft = d
+        total, dot = x.astype(np.float64).sum(), (x.astype(np.float64) * y).sum()
+        scale = np.abs(x).astype(np.float64).sum() / np.sqrt(n)
+        for k in range(6):
+            assert abs(float(gpu.reduce_scalar(1, x, xi)) - total) <= 1e-5 * max(abs(total), scale), (what, k)
+            assert float(gpu.indexreduce_scalar(0, x, xi)) == float(np.argmax(x)), (what, k)
+            assert abs(float(gpu.reduce3_scalar(3, x, xi, y, xi)) - dot) <= 1e-4 * np.sqrt(n), (what, k)
+            got = gpu.transform(38, xr, rows, rows).astype(np.float64).reshape(4, 40000)
+            assert np.all(np.abs(got - soft) <= 2e-5 * soft + 1e-30), (what, k)
+
+    a, b = data(), data()
+    try:
+        for boundary in (0x40000000, 0x80000000, 0):
+            gpu.ops.amd_setSlotTicket(ex, boundary)
+            run(a, ("A", hex(boundary)))
+            gpu.ops.amd_setSlotTicket(ex, (boundary - 16) & 0xffffffff)
+            run(b, ("B", hex(boundary)))
+    finally:
+        gpu.ops.amd_setSlotTicket(ex, 5)
+
+
+def test_releasing_a_streams_resources(gpu):
+    """A stream's workspace, exchange slots and pinned scalar block are freed on request and come back at the next call."""
+    rs = np.random.RandomState(43)
+    x = rs.randn(1 << 18).astype(np.float32)
+    xi = shape_info_np([512, 512])
+    want = x.astype(np.float64).reshape(512, 512)
+    for _ in range(3):
+        assert abs(float(gpu.reduce_scalar(1, x, xi)) - want.sum()) <= 1e-5 * np.abs(want).sum()
+        assert np.array_equal(gpu.reduce(3, x, xi, None, [0], 512), want.max(axis=0).astype(np.float32))
+        gpu.ops.amd_releaseStream(gpu.dev.stream)
+    gpu.ops.amd_releaseStream(gpu.dev.stream)  # nothing left to free: a no-op
 
 
 def test_double_family_smoke(gpu, cpu):

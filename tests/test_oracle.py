@@ -26,6 +26,7 @@ def test_op_vectors_bit_exact(oracle):
 
 def test_half_vectors(oracle):
     checks.check_half_vectors(oracle, exact=True)
+    checks.check_half_reduction_vectors(oracle, exact=True)
 
 
 def test_rng_vectors(oracle):
