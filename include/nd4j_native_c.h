@@ -225,6 +225,11 @@ void nd4j_amd_setCooperativeWaitLimit(int tries);
  * hardware traffic counters are scaled */
 void nd4j_amd_copyKernel(Nd4jPointer *extraPointers, void *dst, const void *src, Nd4jLong bytes);
 
+/* yardstick for the fused softmax over f-order matrices: copies the f-order float matrix src [rows, cols] (rows adjacent in
+ * memory, a multiple of 4 of them, 16-byte aligned) to dst in exactly the tiles and block order of that kernel - 64 rows
+ * x 512 columns to a 512-thread block, 256 contiguous bytes of each column at a time - with no arithmetic and no exchange
+ * between blocks */
+void nd4j_amd_forderTileCopy(Nd4jPointer *extraPointers, float *dst, const float *src, Nd4jLong rows, Nd4jLong cols);
 /* No counterpart in the reference (its scratch belongs to the caller).  The library keeps a workspace, reduction slots
  * and a pinned scalar block per (device, stream), allocated at the stream's first call that needs them.  A host that
  * destroys a stream calls this first, with the stream's device current: it waits for the stream to drain and frees them

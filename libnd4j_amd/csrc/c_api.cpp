@@ -274,6 +274,12 @@ void nd4j_amd_execReduceFloatNoAlloc(Nd4jPointer *extraPointers, int opNum, floa
                                      float *result) {
     guardVoid([&] { nd4j_amd::reduceFloatNoAlloc(extraPointers, opNum, x, xShapeInfo, extraParams, result); });
 }
+void nd4j_amd_forderTileCopy(Nd4jPointer *extraPointers, float *dst, const float *src, Nd4jLong rows, Nd4jLong cols) {
+    guardVoid([&] {
+        nd4j_amd::launchForderTileCopy(nd4j_amd::streamOf(extraPointers), src, dst, rows, cols);
+        nd4j_amd::checkLaunch("forderTileCopy", nd4j_amd::streamOf(extraPointers));
+    });
+}
 void nd4j_amd_releaseStream(Nd4jPointer stream) {
     guardVoid([&] { nd4j_amd::releaseStreamResources(reinterpret_cast<hipStream_t>(stream)); });
 }

@@ -297,6 +297,8 @@ bool launchRandom(hipStream_t stream, int opNum, const RngState &rng, const T *x
 void launchRngDump(hipStream_t stream, const RngState &rng, Long start, Long n, unsigned long long *out);
 // plain copy with 16-byte vectors (bytes is rounded down to a multiple of 16 plus a byte tail)
 void launchCopy(hipStream_t stream, void *dst, const void *src, Long bytes);
+// measurement aid: copies an f-order float matrix in the tiles and block order of the cooperative f-order softmax kernel
+void launchForderTileCopy(hipStream_t stream, const float *x, float *z, Long numRows, Long length);
 // zero fill of `bytes` bytes (a multiple of 16, at a 16-byte boundary) by a kernel: safe to record where a memset node is not
 void launchFill(hipStream_t stream, void *dst, size_t bytes);
 

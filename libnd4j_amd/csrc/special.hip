@@ -10,6 +10,8 @@
 #include <atomic>
 
 #include "elementwise.cuh"
+#include <stdexcept>
+
 #include "launch.h"
 #include "reduce_engine.cuh"
 
@@ -871,6 +873,38 @@ template <typename T, int MODE, int RL, int kCCBlock> static bool runColCooperat
     }
     return true;
 }
+// Measurement aid: a copy of an f-order float matrix (rows adjacent in memory, columns `rows` elements apart) that moves
+// exactly the tiles softmaxColCoopKernel moves, in its block order - a 512-thread block takes 64 rows x 512 columns as
+// 16 row lanes x 32 column lanes, 16 vectors a lane, asking for 256 contiguous bytes of each column - with no arithmetic
+// and no exchange between blocks: what that access pattern costs on its own.
+__global__ void __launch_bounds__(512) forderTileCopyKernel(const float *x, float *z, Long numRows, Long length, int slices) {
+    constexpr int N = 4, RL = 16, PACKS = 16, kCols = 512 / RL;
+    const int rl = threadIdx.x % RL, cg = threadIdx.x / RL;
+    const Long group = (Long)blockIdx.x / slices;
+    const int sl = (int)((Long)blockIdx.x - group * slices);
+    const Long row0 = (group * RL + rl) * N;
+    if (row0 >= numRows) return;
+    const int colFirst = sl * PACKS * kCols + cg;
+    int mine = colFirst < length ? (int)((length - colFirst + kCols - 1) / kCols) : 0;
+    if (mine > PACKS) mine = PACKS;
+    Pack<float> cache[PACKS];
+    const float *px = x + row0 + (Long)colFirst * numRows;
+    float *pz = z + row0 + (Long)colFirst * numRows;
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (j < mine) cache[j] = loadPack(reinterpret_cast<const Pack<float> *>(px + (Long)j * kCols * numRows));
+#pragma unroll
+    for (int j = 0; j < PACKS; j++)
+        if (j < mine) storePack(reinterpret_cast<Pack<float> *>(pz + (Long)j * kCols * numRows), cache[j]);
+}
+void launchForderTileCopy(hipStream_t s, const float *x, float *z, Long numRows, Long length) {
+    if (numRows <= 0 || length <= 0 || numRows % 4 != 0 || !aligned16(x) || !aligned16(z))
+        throw std::invalid_argument("forderTileCopy: needs 16-byte aligned operands and a row count that is a multiple of 4");
+    const Long groups = (numRows + 63) / 64, slices = (length + 511) / 512;
+    if (groups * slices > kMaxGrid) throw std::invalid_argument("forderTileCopy: matrix too large for one launch");
+    ND4J_LAUNCH(forderTileCopyKernel, dim3((unsigned)(groups * slices)), dim3(512), 0, s, x, z, numRows, length, (int)slices);
+}
+
 template <typename T> bool launchSoftmaxColCooperative(hipStream_t s, int opNum, const T *x, T *z, const SoftmaxPlan &pl, Workspace ws) {
     constexpr int N = Pack<T>::N;
     if (opNum < 38 || opNum > 40) return false;

@@ -112,6 +112,7 @@ _PLAIN_SIGNATURES = {
     "nd4j_amd_copyKernel": ([_P, _P, _P, c_ll], None),
     "nd4j_amd_hostFetchCount": ([], c_ll),
     "nd4j_amd_setCooperativeWaitLimit": ([c_int], None),
+    "nd4j_amd_forderTileCopy": ([_P, _P, _P, c_ll, c_ll], None),
     "nd4j_amd_releaseStream": ([_P], None),
     "nd4j_amd_setSlotTicket": ([_P, ctypes.c_uint], None),
     "nd4j_amd_execReduceFloatNoAlloc": ([_P, c_int, _P, _P, _P, _P], None),

@@ -396,6 +396,12 @@ def stats_softmax(dev, rows=32768, cols=2048, seed=23, copies=None):
         cases.append(Case("softmax_fused_forder", "special", n, 8 * n,
                           lambda: ops.execTransformFloat(ex_t, T_SOFTMAX, X.ptr, X.info_ptr, T.ptr, T.info_ptr, None),
                           lambda lib: (lib.transform(T_SOFTMAX, x, xi, tc, xi, None), tc)[1], False, T.get))
+        # yardstick: a plain copy of the same matrix in the fused f-order kernel's tiles and block order (no arithmetic, no
+        # exchange between blocks) - what its access pattern, 256-byte pieces of columns 128 KiB apart, costs by itself
+        cases.append(Case("yardstick_copy_forder_tiles", "yardstick", n, 8 * n,
+                          lambda: ops.amd_forderTileCopy(ex_t, T.ptr, X.ptr, rows, cols),
+                          None, False, T.get))
+        cases[-1].note = "not an op: the fused f-order softmax's memory accesses without its arithmetic"
         cases.append(Case("softmax_fused_corder", "special", n, 8 * n,
                           lambda: ops.execTransformFloat(ex_c, T_SOFTMAX, X.ptr, XCI.ptr, T.ptr, XCI.ptr, None),
                           lambda lib: (lib.transform(T_SOFTMAX, x, xci, tc, xci, None), tc)[1], True, T.get))

@@ -156,6 +156,8 @@ def test_config3_summary_stats_and_softmax_chain(gpu, lib):
         assert worst["fused long rows vs float64"] <= bar
         print("softmax, largest relative differences:", ", ".join("%s %.3g" % kv for kv in sorted(worst.items())))
         assert np.all(np.abs(fused.sum(axis=1) - 1.0) <= 1e-5)
+        # the copy that serves as the f-order kernel's yardstick moves every element
+        assert np.array_equal(_run(w.case("yardstick_copy_forder_tiles")), x)
         # IsMax: one-hot of the first maximum, whole array and per row; bit-exact
         xf = x.reshape(rows, cols)
         # (the winning index travels as a value of the data type, in the reference too - execIndexReduceScalarFloat
