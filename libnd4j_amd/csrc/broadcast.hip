@@ -53,6 +53,16 @@ template <typename T> struct BroadcastBody {
                 // TADs over several dimensions whose innermost one is contiguous in x, y and z
                 launchRuns<T, F, true>(s, x, pl.xm, y, pl.ym, z, pl.zm, pl.xOffsets, pl.zOffsets, Params<T>{nullptr}, pl.numTads,
                                  pl.tadLength, pl.runLength, pl.runMajor);
+            } else if (pl.numTads >= 64) {
+                // several dimensions, no contiguous runs: a lane per TAD, so that neighbouring TADs coalesce
+                int gx = (int)((pl.numTads + kBlock - 1) / kBlock);
+                Long gy = (Long)kGridCap / gx;
+                if (gy < 1) gy = 1;
+                if (gy > pl.tadLength) gy = pl.tadLength;
+                if (gy > 65535) gy = 65535;
+                ND4J_LAUNCH((bcColKernel<T, F, false, true>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
+                                   pl.zOffsets, pl.tadLength, pl.numTads, (Long)0, (Long)0, (Long)0, Params<T>{nullptr}, pl.xm, pl.ym,
+                                   pl.zm);
             } else {
                 int grid = gridFor(pl.numTads, 1, kGridCap);
                 ND4J_LAUNCH((bcGeneralKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, pl.xm, y, pl.ym, z, pl.zm,

@@ -426,10 +426,13 @@ __global__ void __launch_bounds__(kBlock) bcFlatInnerKernel(const T *x, const T 
 
 // Broadcast over strided TADs: thread <-> TAD, loop over the TAD's elements.  When neighbouring TADs
 // are neighbours in memory (a column of a c-order matrix) each wave reads and writes full lines.
-template <typename T, typename F, bool BYTAD>
+// MAPPED: TADs over several dimensions without contiguous runs: element f of a TAD (of y, of the result's TAD) lies where
+// the operand's coordinate map puts it; f is the same for all lanes of a wave, so the maps are worked out once per wave.
+template <typename T, typename F, bool BYTAD, bool MAPPED = false>
 __global__ void __launch_bounds__(kBlock) bcColKernel(const T *x, const T *y, T *z, const Long *xOffsets,
                                                       const Long *zOffsets, Long tadLength, Long numTads,
-                                                      Long tadEws, Long yEws, Long zEws, Params<T> p) {
+                                                      Long tadEws, Long yEws, Long zEws, Params<T> p, DimMap xm = DimMap(),
+                                                      DimMap ym = DimMap(), DimMap zm = DimMap()) {
     typedef typename Compute<T>::type C;
     if (F::tables) lm::loadTables();
     const Long t = (Long)blockIdx.x * kBlock + threadIdx.x;
@@ -439,8 +442,13 @@ __global__ void __launch_bounds__(kBlock) bcColKernel(const T *x, const T *y, T 
     const C yt = BYTAD ? toCompute(y[t]) : (C)0;
     const Long f0 = (Long)blockIdx.y;
     for (Long f = f0; f < tadLength; f += gridDim.y) {
-        C bv = BYTAD ? yt : toCompute(y[f * yEws]);
-        zr[f * zEws] = fromCompute<T>(F::template apply<C>(toCompute(xr[f * tadEws]), bv, p));
+        if (MAPPED) {
+            const unsigned ff = (unsigned)f;
+            zr[mapOffset32(zm, ff)] = fromCompute<T>(F::template apply<C>(toCompute(xr[mapOffset32(xm, ff)]), toCompute(y[mapOffset32(ym, ff)]), p));
+        } else {
+            C bv = BYTAD ? yt : toCompute(y[f * yEws]);
+            zr[f * zEws] = fromCompute<T>(F::template apply<C>(toCompute(xr[f * tadEws]), bv, p));
+        }
     }
 }
 

@@ -185,10 +185,13 @@ __global__ void __launch_bounds__(kBlock) tadRowKernel(Pol pol, const typename P
 }
 
 // Strided TADs: thread t <-> TAD t, rows [rowsPerSplit * blockIdx.y, ...) of each TAD.
-template <class Pol>
+// MAPPED: TADs over several dimensions whose innermost one is strided (no vectors to be had along a TAD): element j of a
+// TAD lies at the offset the coordinate map gives - the same for every lane, so one division chain serves the 64 TADs
+// of a wave - and neighbouring TADs still coalesce wherever they are neighbours in memory.
+template <class Pol, bool MAPPED = false>
 __global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
                                                        typename Pol::Acc *partials, const Long *offsets, Long tadLength,
-                                                       Long numTads, Long tadEws, Long rowsPerSplit) {
+                                                       Long numTads, Long tadEws, Long rowsPerSplit, DimMap tm = DimMap()) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::Acc Acc;
     const Long t = (Long)blockIdx.x * kBlock + threadIdx.x;
@@ -201,15 +204,16 @@ __global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename P
     (void)rowsPerSplit;
     const Long S = gridDim.y;
     Long j = blockIdx.y;
+    auto at = [&](Long row) -> Long { return MAPPED ? mapOffset32(tm, (unsigned)row) : row * tadEws; };
     for (; j + 7 * S < tadLength; j += 8 * S) {
         typename Pol::T v[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = base[(j + u * S) * tadEws];
+        for (int u = 0; u < 8; u++) v[u] = base[at(j + u * S)];
 #pragma unroll
         for (int u = 0; u < 8; u++) foldNext(pol, acc, toCompute(v[u]), j + u * S);
         pol.checkpoint(acc);
     }
-    for (; j < tadLength; j += S) { foldNext(pol, acc, toCompute(base[j * tadEws]), j); pol.checkpoint(acc); }
+    for (; j < tadLength; j += S) { foldNext(pol, acc, toCompute(base[at(j)]), j); pol.checkpoint(acc); }
     if (gridDim.y == 1) z[t] = pol.finalize(acc, tadLength);
     else partials[(Long)blockIdx.y * numTads + t] = acc;
 }
@@ -803,7 +807,8 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
                                z, partials, pl.tadLength, pl.numTads, (int)splits);
         return;
     }
-    if (pl.kind == TadPlan::ROW || pl.kind == TadPlan::COL) {
+    const bool mappedLanes = pl.kind == TadPlan::GENERAL && pl.runLength == 0 && pl.numTads >= kWave;
+    if (pl.kind == TadPlan::ROW || pl.kind == TadPlan::COL || mappedLanes) {
         // one lane per TAD; split the TAD length so that the grid fills the chip
         int gx = (int)((pl.numTads + kBlock - 1) / kBlock);
         Long splits = 2048 / gx;
@@ -817,8 +822,12 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         splits = (pl.tadLength + rowsPerSplit - 1) / rowsPerSplit;
         if (splits < 1) splits = 1;
         Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+        if (mappedLanes)
+            ND4J_LAUNCH((tadColKernel<Pol, true>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
+                               pl.offsets, pl.tadLength, pl.numTads, (Long)0, rowsPerSplit, pl.tm);
+        else
         ND4J_LAUNCH((tadColKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
-                           pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit);
+                           pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit, DimMap());
         if (splits > 1)
             ND4J_LAUNCH((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kFinishLanes - 1) / kFinishLanes)), dim3(kBlock), 0, s, pol,
                                z, partials, pl.tadLength, pl.numTads, (int)splits);

@@ -267,6 +267,53 @@ def test_tad_shapes_of_every_kernel_variant(gpu, cpu):
         assert float(gpu.indexreduce_scalar(0, x, xi)) == float(cpu.indexreduce_scalar(0, x, xi))
 
 
+def test_tads_over_several_dimensions(gpu, cpu):
+    """TADs over several dimensions carry no element-wise stride; which kernel walks them follows from their layout.  Shapes
+    for each: dimensions that merge into one contiguous or strided run, contiguous runs placed by outer dimensions (long
+    TADs cut into slices, TADs a wave or sixteen lanes share, runs whose length is no multiple of the vector width), and
+    a strided innermost dimension (a lane per TAD)."""
+    rs = np.random.RandomState(52)
+    for shape, dims in (([12, 9, 16, 8], [2, 3]), ([12, 9, 16, 8], [0, 1]), ([130, 7, 300], [0, 2]), ([40, 50, 24], [0, 2]),
+                        ([9, 400, 6], [0, 2]), ([33, 20, 5, 7], [0, 2, 3]), ([6, 40, 5, 8], [0, 2]), ([3, 70, 4, 9], [0, 2]),
+                        ([5, 1100, 3, 2], [0, 2]), ([64, 3, 4100], [0, 2]), ([2, 3, 70000], [0, 2])):
+        n = int(np.prod(shape))
+        x = rs.randn(n).astype(np.float32)
+        xi = shape_info_np(shape)
+        x64 = x.astype(np.float64).reshape(shape)
+        axes = tuple(dims)
+        out_len = n // int(np.prod([shape[d] for d in dims]))
+        tad_len = n // out_len
+        what = "%s dims %s" % (shape, dims)
+        scale = np.abs(x64).sum(axis=axes).ravel() / np.sqrt(tad_len)
+        g, c = gpu.reduce(1, x, xi, None, dims, out_len).astype(np.float64), cpu.reduce(1, x, xi, None, dims, out_len).astype(np.float64)
+        truth = x64.sum(axis=axes).ravel()
+        bound = 1e-5 * np.maximum(np.abs(truth), scale)
+        assert np.all(np.abs(g - truth) <= bound), what
+        # (the reference's sequential fp32 sum of a long TAD drifts from the exact value by more than the bar: allow it its drift)
+        assert np.all(np.abs(g - c) <= np.abs(c - truth) + bound), what
+        assert np.array_equal(gpu.reduce(3, x, xi, None, dims, out_len), cpu.reduce(3, x, xi, None, dims, out_len)), what
+        for op in (0, 1):
+            assert np.array_equal(gpu.indexreduce(op, x, xi, None, dims, out_len), cpu.indexreduce(op, x, xi, None, dims, out_len)), what
+        checks.assert_reduction_close(gpu.summarystats(0, 1, x, xi, dims, out_len), cpu.summarystats(0, 1, x, xi, dims, out_len), 0, "var " + what)
+        if n <= 2000000:
+            yshape = [shape[d] for d in dims]
+            y = rs.uniform(1, 2, tad_len).astype(np.float32)
+            yi = shape_info_np(yshape)
+            for op in (0, 3):
+                assert np.array_equal(gpu.broadcast(op, x, xi, y, yi, xi, dims), cpu.broadcast(op, x, xi, y, yi, xi, dims)), ("broadcast", op, what)
+    # ties and half / double storage through the run-wise kernel
+    shape, dims = [8, 5, 64], [0, 2]
+    xi = shape_info_np(shape)
+    for dt in (np.float16, np.float64):
+        x = rs.randint(0, 4, int(np.prod(shape))).astype(dt)
+        assert np.array_equal(gpu.indexreduce(0, x, xi, None, dims, 5), cpu.indexreduce(0, x, xi, None, dims, 5)), dt
+        if dt == np.float64:
+            assert np.array_equal(gpu.reduce(1, x, xi, None, dims, 5), cpu.reduce(1, x, xi, None, dims, 5))
+        y = rs.uniform(1, 2, 8 * 64).astype(dt)
+        g, c = gpu.broadcast(0, x, xi, y, shape_info_np([8, 64]), xi, dims), cpu.broadcast(0, x, xi, y, shape_info_np([8, 64]), xi, dims)
+        assert np.array_equal(g, c), dt
+
+
 def test_broadcast_on_views_all_ops(gpu, cpu):
     rs = np.random.RandomState(27)
     for shape, order, dims in (([17, 33], "c", [1]), ([17, 33], "c", [0]), ([17, 33], "f", [0]), ([17, 33], "f", [1]),
