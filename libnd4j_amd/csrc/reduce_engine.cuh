@@ -226,10 +226,13 @@ __global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename P
 // (The four waves side by side instead - 4 KiB of every row to a block, each wave walking all the rows of the range, no
 // merge through LDS - was slower: 52.6 against 48.6 us for sums along dim 0 of [16384, 4096], twice as slow for the
 // summary statistics.)
-template <class Pol>
+// MAPPED: the same for TADs over several dimensions whose innermost one is strided: row j of the TADs lies where the
+// coordinate map puts it (every stride of the map a multiple of the vector width, so that the vectors stay aligned);
+// a row's divisions are shared by the Pack::N TADs of a lane.
+template <class Pol, bool MAPPED = false>
 __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
                                                           typename Pol::Acc *partials, const Long *offsets, Long tadLength,
-                                                          Long numTads, Long tadEws, Long rowsPerSplit) {
+                                                          Long numTads, Long tadEws, Long rowsPerSplit, DimMap tm = DimMap()) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
@@ -255,7 +258,8 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
             acc[e] = pe[e].init(x + off[e]);
             if (e > 0 && off[e] != off[0] + e) vec = false;
         }
-        if ((reinterpret_cast<uintptr_t>(x + off[0]) & 15) != 0 || (tadEws % VEC) != 0) vec = false;
+        if ((reinterpret_cast<uintptr_t>(x + off[0]) & 15) != 0 || (!MAPPED && (tadEws % VEC) != 0)) vec = false;
+        auto rowAt = [&](Long row) -> Long { return MAPPED ? mapOffset32(tm, (unsigned)row) : row * tadEws; };
         if (vec) {
             const T *base = x + off[0];
             // Row ranges start a power-of-two number of bytes apart, so blocks that all began at the top of their range
@@ -269,7 +273,7 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
                 for (; j + 3 * WAVES < b; j += 4 * WAVES) {
                     Pack<T> pk[4];
 #pragma unroll
-                    for (int u = 0; u < 4; u++) pk[u] = loadPack(reinterpret_cast<const Pack<T> *>(base + (j + u * WAVES) * tadEws));
+                    for (int u = 0; u < 4; u++) pk[u] = loadPack(reinterpret_cast<const Pack<T> *>(base + rowAt(j + u * WAVES)));
 #pragma unroll
                     for (int u = 0; u < 4; u++) {
 #pragma unroll
@@ -282,7 +286,7 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
                     for (int e = 0; e < VEC; e++) pe[e].checkpoint(acc[e]);
                 }
                 for (; j < b; j += WAVES) {
-                    Pack<T> pk = loadPack(reinterpret_cast<const Pack<T> *>(base + j * tadEws));
+                    Pack<T> pk = loadPack(reinterpret_cast<const Pack<T> *>(base + rowAt(j)));
 #pragma unroll
                     for (int e = 0; e < VEC; e++) {
                         if constexpr (decltype(ascending)::value) foldNext(pe[e], acc[e], toCompute(pk.v[e]), j);
@@ -302,7 +306,7 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
             for (int e = 0; e < VEC; e++) {
                 if (t0 + e >= numTads) continue;
                 const T *base = x + off[e];
-                for (Long j = j0 + wave; j < j1; j += WAVES) { foldNext(pe[e], acc[e], toCompute(base[j * tadEws]), j); pe[e].checkpoint(acc[e]); }
+                for (Long j = j0 + wave; j < j1; j += WAVES) { foldNext(pe[e], acc[e], toCompute(base[rowAt(j)]), j); pe[e].checkpoint(acc[e]); }
             }
         }
     }
@@ -783,8 +787,11 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
     // (the vector loads need every row of the TADs' common pitch to start on a 16-byte boundary: a pitch that is not a
     // multiple of the vector width goes to the lane-per-TAD kernel below, whose neighbouring lanes read neighbouring
     // elements)
-    if (pl.kind == TadPlan::COL && pl.numTads >= 2 * kWave * Pack<typename Pol::T>::N &&
-        pl.tadEws % Pack<typename Pol::T>::N == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    bool mappedVec = pl.kind == TadPlan::GENERAL && pl.runLength == 0 && pl.numTads >= 2 * kWave * Pack<typename Pol::T>::N &&
+                     (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    for (int d = 0; mappedVec && d < pl.tm.rank; d++) mappedVec = pl.tm.stride[d] % Pack<typename Pol::T>::N == 0;
+    if (mappedVec || (pl.kind == TadPlan::COL && pl.numTads >= 2 * kWave * Pack<typename Pol::T>::N &&
+        pl.tadEws % Pack<typename Pol::T>::N == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0)) {
         // lane per Pack::N adjacent TADs, 64 lanes per block column, rows split over the block's waves and blockIdx.y
         constexpr int VEC = Pack<typename Pol::T>::N;
         int gx = (int)((pl.numTads + (Long)kWave * VEC - 1) / ((Long)kWave * VEC));
@@ -800,8 +807,12 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         splits = (pl.tadLength + rowsPerSplit - 1) / rowsPerSplit;
         if (splits < 1) splits = 1;
         Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+        if (mappedVec)
+            ND4J_LAUNCH((tadColVecKernel<Pol, true>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
+                               pl.offsets, pl.tadLength, pl.numTads, (Long)0, rowsPerSplit, pl.tm);
+        else
         ND4J_LAUNCH((tadColVecKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
-                           pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit);
+                           pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit, DimMap());
         if (splits > 1)
             ND4J_LAUNCH((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kFinishLanes - 1) / kFinishLanes)), dim3(kBlock), 0, s, pol,
                                z, partials, pl.tadLength, pl.numTads, (int)splits);

@@ -455,6 +455,8 @@ def general_views(dev, seed=61, copies=None):
     xv, yv = _normal(rs, span, F32), _normal(rs, span, F32)
     tad1_023, tad1_23 = dev.tad(i1, [0, 2, 3]), dev.tad(i1, [2, 3])
     tad2_12, tad3_02 = dev.tad(i2, [1, 2]), dev.tad(i3, [0, 2])
+    tad1_02 = dev.tad(i1, [0, 2])
+    cw_out, ocw = _vec(nchw[1] * nchw[3]), np.zeros(nchw[1] * nchw[3], F32)
     c_out, r_out = _vec(nchw[1]), _vec(cube[0])
     zc1, zc2, zc3 = np.zeros(n1, F32), np.zeros(n3, F32), np.zeros(span, F32)
     oc1, oc2 = np.zeros(nchw[1], F32), np.zeros(cube[0], F32)
@@ -471,6 +473,13 @@ def general_views(dev, seed=61, copies=None):
         cases.append(Case("variance_nchw_dims023", "summarystats", n1, 4 * n1 + 4 * nchw[1],
                           lambda: ops.execSummaryStatsFloat(ex, S_VAR, X1.ptr, X1.info_ptr, None, C.ptr, C.info_ptr, D023.ptr, 3, 1),
                           lambda lib: (lib.summarystats(S_VAR, 1, x1, i1, oc1, c_out, [0, 2, 3]), oc1)[1], False, C.get))
+        # dimensions {0, 2}: the TADs' innermost dimension is strided (56 elements apart), neighbouring TADs are neighbours
+        CW = w.operand(np.zeros(nchw[1] * nchw[3], F32), cw_out)
+        D02n = w.raw(np.array([0, 2], np.int32))
+        ex02 = dev.extra(i1, z_info=cw_out, tad=tad1_02)
+        cases.append(Case("sum_nchw_dims02", "reduce", n1, 4 * n1 + 4 * nchw[1] * nchw[3],
+                          lambda: ops.execReduceFloat(ex02, R_SUM, X1.ptr, X1.info_ptr, None, CW.ptr, CW.info_ptr, D02n.ptr, 2),
+                          lambda lib: (lib.reduce(R_SUM, x1, i1, None, ocw, cw_out, [0, 2]), ocw)[1], False, CW.get))
         P = w.operand(plane, pi)
         ex_b = dev.extra(i1, pi, i1, tad=tad1_23, tad_z=tad1_23)
         cases.append(Case("broadcast_add_nchw_dims23", "broadcast", n1, 8 * n1 + 4 * plane.size,

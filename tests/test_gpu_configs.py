@@ -185,6 +185,12 @@ def test_general_views_at_benchmark_size(gpu, lib):
         got, cpu = _run(c).astype(np.float64), c.cpu(lib).astype(np.float64)
         assert np.all(np.abs(got - truth) <= 1e-5 * np.maximum(np.abs(truth), scale))
         assert np.all(np.abs(got - cpu) <= np.abs(cpu - truth) + 1e-5 * np.maximum(np.abs(truth), scale))
+        c = w.case("sum_nchw_dims02")
+        truth2 = x64.sum(axis=(0, 2)).ravel()
+        scale2 = np.abs(x64).sum(axis=(0, 2)).ravel() / np.sqrt(128 * 56)
+        got, cpu = _run(c).astype(np.float64), c.cpu(lib).astype(np.float64)
+        assert np.all(np.abs(got - truth2) <= 1e-5 * np.maximum(np.abs(truth2), scale2))
+        assert np.all(np.abs(got - cpu) <= np.abs(cpu - truth2) + 1e-5 * np.maximum(np.abs(truth2), scale2))
         c = w.case("variance_nchw_dims023")
         var = x64.var(axis=(0, 2, 3), ddof=1)
         got, cpu = _run(c).astype(np.float64), c.cpu(lib).astype(np.float64)

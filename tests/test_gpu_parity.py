@@ -274,7 +274,7 @@ def test_tads_over_several_dimensions(gpu, cpu):
     a strided innermost dimension (a lane per TAD)."""
     rs = np.random.RandomState(52)
     for shape, dims in (([12, 9, 16, 8], [2, 3]), ([12, 9, 16, 8], [0, 1]), ([130, 7, 300], [0, 2]), ([40, 50, 24], [0, 2]),
-                        ([9, 400, 6], [0, 2]), ([33, 20, 5, 7], [0, 2, 3]), ([6, 40, 5, 8], [0, 2]), ([3, 70, 4, 9], [0, 2]),
+                        ([9, 400, 6], [0, 2]), ([33, 20, 5, 7], [0, 2, 3]), ([6, 40, 5, 8], [0, 2]), ([3, 70, 4, 9], [0, 2]), ([6, 150, 5, 8], [0, 2]), ([40, 9, 30, 64], [0, 2]),
                         ([5, 1100, 3, 2], [0, 2]), ([64, 3, 4100], [0, 2]), ([2, 3, 70000], [0, 2])):
         n = int(np.prod(shape))
         x = rs.randn(n).astype(np.float32)
