@@ -659,8 +659,23 @@ def check_random_views(be, ref, seed, cases):
         shape = [int(v) for v in harness.info_shape(xi)]
         n, rank = int(np.prod(shape)), len(shape)
         x = rs.uniform(-3, 3, harness.span_of(xi)).astype(np.float32)
-        what = int(rs.randint(0, 7))
-        if what == 0:
+        what = int(rs.randint(0, 8))
+        if what == 7:
+            # broadcast of a dense sub-array along several dimensions
+            if rank < 3:
+                continue
+            k = int(rs.randint(2, rank))
+            dims = sorted(int(d) for d in rs.choice(rank, size=k, replace=False))
+            yshape = [shape[d] for d in dims]
+            yi = harness.shape_info(yshape, "c")
+            y = rs.uniform(-3, 3, int(np.prod(yshape))).astype(np.float32)
+            op = int(rs.choice([0, 1, 2, 3]))
+            g = be.broadcast(op, x, xi, y, yi, xi, dims, **kw(pass_tads=bool(rs.randint(0, 2))))
+            c = ref.broadcast(op, x, xi, y, yi, xi, dims)
+            sel = harness.element_offsets(xi)
+            assert ulp_distance(g[sel], c[sel]).max() <= 1, ("broadcast", op, dims, list(xi))
+            assert np.array_equal(np.delete(g, sel), np.delete(c, sel)), ("broadcast wrote outside its view", dims, list(xi))
+        elif what == 0:
             zi, op = random_view(rs, shape), int(rs.choice([0, 3, 15, 6, 10, 23, 42]))
             g, c = be.transform(op, x, xi, zi), ref.transform(op, x, xi, zi)
             sel = harness.element_offsets(zi)

@@ -1295,7 +1295,7 @@ def test_random_views_against_the_cpu_checker(gpu, cpu):
     """Generated shapes, strides and dimensions through every loop family (tests/checks.py: check_random_views), with and
     without the caller's TAD tables.  Fixed seed: the same few thousand calls every run."""
     done = checks.check_random_views(gpu, cpu, seed=7, cases=4000)
-    assert len(done) == 7 and min(done.values()) > 200
+    assert len(done) == 8 and min(done.values()) > 200
 
 
 def test_dense_matrices_in_mixed_orders(gpu):

@@ -320,4 +320,4 @@ def test_random_views_match_compiled_reference(oracle_lib, reference_lib):
     """Generated shapes, strides and dimensions through every loop family: this repository's restatement against the
     reference's own loops (elementwise exactly or within 2 ULP, reductions to 1e-5, index reductions exactly)."""
     done = checks.check_random_views(backends.CpuBackend(oracle_lib), backends.CpuBackend(reference_lib), seed=2, cases=2500)
-    assert len(done) == 7 and min(done.values()) > 100
+    assert len(done) == 8 and min(done.values()) > 100
