@@ -535,35 +535,36 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
             unsigned m[U], c[U];
             Long xo[U], zo[U];
             bool live[U];
+            // (a unit beyond the end is placed on the last one, so that no load sits in a branch of its own - the compiler
+            // would make each such load wait for those before it - and is neither worked on nor stored)
 #pragma unroll
             for (int k = 0; k < U; k++) {
                 const Long g = g0 + k * step;
                 live[k] = g < total;
-                xo[k] = zo[k] = 0;
-                if (live[k]) {
-                    Long r;
-                    locate(g, r, m[k], c[k]);
-                    if (xOffsets != nullptr) xo[k] = xOffsets[r];
-                    if (zOffsets != nullptr) zo[k] = zOffsets[r];
-                }
+                Long r;
+                locate(live[k] ? g : total - 1, r, m[k], c[k]);
+                xo[k] = xOffsets != nullptr ? xOffsets[r] : 0;
+                zo[k] = zOffsets != nullptr ? zOffsets[r] : 0;
             }
             const T *xp[U], *yp[U];
             T *zp[U];
             Pack<T> a[U], b[U];
             bool whole[U];
+            const bool shortRuns = runLength % VEC != 0;  // some units hold fewer elements than a vector
 #pragma unroll
             for (int k = 0; k < U; k++) {
-                whole[k] = false;
-                if (live[k]) {
-                    xp[k] = x + xo[k] + runOffset(xm, m[k], c[k] * VEC, runLength);
-                    zp[k] = z + zo[k] + runOffset(zm, m[k], c[k] * VEC, runLength);
-                    if (two) yp[k] = y + runOffset(ym, m[k], c[k] * VEC, runLength);
-                    whole[k] = runLength - c[k] * VEC >= (unsigned)VEC;
-                    if (whole[k]) {
-                        a[k] = streamPackAnywhere(xp[k]);
-                        if (two) b[k] = loadPackAnywhere(yp[k]);
-                    }
+                xp[k] = x + xo[k] + runOffset(xm, m[k], c[k] * VEC, runLength);
+                zp[k] = z + zo[k] + runOffset(zm, m[k], c[k] * VEC, runLength);
+                if (two) yp[k] = y + runOffset(ym, m[k], c[k] * VEC, runLength);
+                whole[k] = !shortRuns || runLength - c[k] * VEC >= (unsigned)VEC;
+                if (!shortRuns) {
+                    a[k] = streamPackAnywhere(xp[k]);
+                    if (two) b[k] = loadPackAnywhere(yp[k]);
+                } else if (whole[k]) {
+                    a[k] = streamPackAnywhere(xp[k]);
+                    if (two) b[k] = loadPackAnywhere(yp[k]);
                 }
+                whole[k] = whole[k] && live[k];
             }
 #pragma unroll
             for (int k = 0; k < U; k++) {

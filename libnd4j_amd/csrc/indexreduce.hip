@@ -23,6 +23,7 @@ template <typename TT, int OP> struct IndexPol {
     static constexpr bool tables = false;  // no exp / log / pow in these accumulators
     static constexpr int kChains = 4;      // accumulators of one lane may be kept apart and combined (ties go to the lower index)
     static constexpr int kSlotWords = 2 + sizeof(C) / 4;  // index and value; the float accumulator's padding word stays behind
+    static constexpr int kFlatBlocks = 768;   // blocks of the whole-array kernel: three per compute unit (see runFlatReduce)
     static constexpr bool kClears = OP == 0;  // IsMax over a whole array looks for the maximum and clears the result in one pass
     Params<TT> p;
 

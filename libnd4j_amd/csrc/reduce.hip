@@ -94,8 +94,7 @@ template <typename TT, int OP> struct ReducePol {
     // bias term with pow); 20-23 have no functor
     static constexpr bool tables = OP == 9 || OP == 10 || (OP >= 16 && OP <= 24);
     static constexpr int kChains = 4;  // accumulators of one lane may be kept apart and combined (combine is the update)
-    // Mean, Sum, Norm1, Norm2, SquaredNorm: plain running sums
-    static constexpr int kFlatBlocks = (OP == 0 || OP == 1 || OP == 5 || OP == 6 || OP == 25) ? 1024 : 2048;
+    static constexpr int kFlatBlocks = 512;  // blocks of the whole-array kernel: two per compute unit (see runFlatReduce)
     Params<TT> p;
     const TT *shiftSource;  // LogSumExp: per-TAD (TAD calls) or single (scalar calls) maximum; else null
     int shiftPerTad;

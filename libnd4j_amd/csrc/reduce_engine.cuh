@@ -138,9 +138,13 @@ __device__ __forceinline__ void foldContiguous(const Pol &pol, typename Pol::Acc
     // batch for the full ones measured slower again, for the code it adds).
     for (; v < nvec; v += 4 * (Long)lanes) {
         Pack<T> pk[4];
+        // (the loads themselves are unconditional - a vector beyond the end re-reads the last one and is not folded: a
+        // load inside a branch of its own makes the compiler wait for the loads before it, one round trip after the other)
 #pragma unroll
-        for (int u = 0; u < 4; u++)
-            if (v + u * (Long)lanes < nvec) pk[u] = loadPack(pv + v + u * (Long)lanes);
+        for (int u = 0; u < 4; u++) {
+            const Long vu = v + u * (Long)lanes;
+            pk[u] = loadPack(pv + (vu < nvec ? vu : nvec - 1));
+        }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             if (v + u * (Long)lanes < nvec) {
@@ -424,48 +428,60 @@ __global__ void __launch_bounds__(kBlock) tadRunsKernel(Pol pol, const typename 
             pol.setTad(r, z);
             const T *tx = x + offsets[r];
             acc = pol.init(tx);
-            for (unsigned u = u0 + lane; u < u1; u += 4 * TEAM) {
-                Pack<T> pk[4];
-                unsigned first[4], count[4];
+            if (runLength >= (unsigned)VEC) {
+                // Every unit is one 16-byte load, requested unconditionally (a load inside a branch of its own would make the
+                // compiler wait for the loads before it): a unit beyond the slice re-reads the slice's last one and is not
+                // folded, and the short last unit of a run loads the VEC elements that END with the run and skips those
+                // that the unit before it has folded.
+                for (unsigned u = u0 + lane; u < u1; u += 4 * TEAM) {
+                    Pack<T> pk[4];
+                    unsigned first[4], skip[4];
 #pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const unsigned uu = u + k * TEAM;
-                    count[k] = 0;
-                    if (uu < u1) {
+                    for (int k = 0; k < 4; k++) {
+                        const unsigned uu = u + k * TEAM;
                         unsigned c;
-                        unsigned m = perRun.divmod(uu, c);
-                        first[k] = m * runLength + c * VEC;
-                        count[k] = runLength - c * VEC;
-                        Long off = (Long)(c * VEC);
+                        unsigned m = perRun.divmod(uu < u1 ? uu : u1 - 1, c);
+                        const unsigned begin = c * VEC + VEC <= runLength ? c * VEC : runLength - VEC;
+                        skip[k] = uu < u1 ? c * VEC - begin : (unsigned)VEC;
+                        first[k] = m * runLength + begin;
+                        Long off = (Long)begin;
                         for (int d = outer - 1; d > 0; d--) {
                             const unsigned q = m / tm.shape[d];
                             off += (Long)(m - q * tm.shape[d]) * tm.stride[d];
                             m = q;
                         }
                         off += (Long)m * tm.stride[0];
-                        if (count[k] >= (unsigned)VEC) {
-                            pk[k] = streamPackAnywhere(tx + off);
-                        } else {
-                            // (a loop with a run-time bound would index the vectors dynamically, and the compiler would
-                            // move all four of them from registers to LDS)
+                        pk[k] = streamPackAnywhere(tx + off);
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        if (skip[k] == 0) {
+#pragma unroll
+                            for (int e = 0; e < VEC; e++) foldNext(pol, acc, toCompute(pk[k].v[e]), (Long)first[k] + e);
+                            pol.checkpoint(acc);
+                        } else if (skip[k] < (unsigned)VEC) {
 #pragma unroll
                             for (int e = 0; e < VEC; e++)
-                                if ((unsigned)e < count[k]) pk[k].v[e] = tx[off + e];
+                                if ((unsigned)e >= skip[k]) foldNext(pol, acc, toCompute(pk[k].v[e]), (Long)first[k] + e);
+                            pol.checkpoint(acc);
                         }
                     }
                 }
-#pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    if (count[k] >= (unsigned)VEC) {
-#pragma unroll
-                        for (int e = 0; e < VEC; e++) foldNext(pol, acc, toCompute(pk[k].v[e]), (Long)first[k] + e);
-                        pol.checkpoint(acc);
-                    } else if (count[k] > 0) {
-#pragma unroll
-                        for (int e = 0; e < VEC; e++)
-                            if ((unsigned)e < count[k]) foldNext(pol, acc, toCompute(pk[k].v[e]), (Long)first[k] + e);
-                        pol.checkpoint(acc);
+            } else {
+                // runs shorter than a vector: element by element
+                for (unsigned u = u0 + lane; u < u1; u += TEAM) {
+                    unsigned c;
+                    unsigned m = perRun.divmod(u, c);  // (one unit per run: c == 0)
+                    const unsigned first = m * runLength;
+                    Long off = 0;
+                    for (int d = outer - 1; d > 0; d--) {
+                        const unsigned q = m / tm.shape[d];
+                        off += (Long)(m - q * tm.shape[d]) * tm.stride[d];
+                        m = q;
                     }
+                    off += (Long)m * tm.stride[0];
+                    for (unsigned e = 0; e < runLength; e++) foldNext(pol, acc, toCompute(tx[off + e]), (Long)first + e);
+                    pol.checkpoint(acc);
                 }
             }
         }
@@ -643,12 +659,15 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
 #pragma unroll
             for (int c = 0; c < CH - 1; c++) more[c] = pol.init(x);
         }
-        for (Long b = (Long)blockIdx.x * chunk; b < nvec; b += (Long)gridDim.x * chunk) {
+        // (every block takes every gridDim.x-th chunk; one contiguous range per block measured 1 to 2 % slower)
+        const Long bFirst = (Long)blockIdx.x * chunk, bEnd = nvec, bStep = (Long)gridDim.x * chunk;
+        for (Long b = bFirst; b < bEnd; b += bStep) {
             Pack<T> pk[kUnroll];
+            // (unconditional loads, see foldContiguous: out-of-range lanes re-read the last vector and do not fold it)
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
                 Long v = b + u * kBlock + threadIdx.x;
-                if (v < nvec) pk[u] = loadPack(xv + v);
+                pk[u] = loadPack(xv + (v < nvec ? v : nvec - 1));
             }
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
@@ -893,8 +912,10 @@ inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, type
     typedef typename Pol::Acc Acc;
     typedef typename Pol::T T;
     Long perBlock = (Long)kBlock * kUnroll * Pack<T>::N;
-    // (plain sums run a little faster - 49.5 against 51.4 us over 2^26 floats - with half as many blocks, each streaming
-    // longer; maxima and index reductions lose a third that way, so a policy asks for it: kFlatBlocks)
+    // (how many blocks serve best differs by policy - kFlatBlocks: with a thread's four loads in flight together, two
+    // blocks per compute unit stream 2^26 floats as fast as eight do, and every block less is a slot less for the last
+    // block to collect: sums and maxima 49 us per synchronous call with 512 blocks, 50 to 52 with 1024 or 2048; index
+    // reductions, whose accumulators are three slot words, 53 us with 768, 54 with 1024, 56 with 2048, 71 with 512)
     int grid = gridFor(pl.n, perBlock, PolFlatBlocks<Pol>::value);
     const bool oneLaunch = ws.slots != nullptr && ws.counter != nullptr && ws.slotTicketSource != nullptr;
     size_t maxBlocks = oneLaunch ? ws.slotBytes / (SlotWords<Pol>::value * sizeof(unsigned long long)) : ws.bytes / sizeof(Acc);

@@ -269,9 +269,16 @@ __global__ void __launch_bounds__(BLOCK) softmaxRowRegKernel(const T *x, T *z, L
         const Pack<T> *xr = reinterpret_cast<const Pack<T> *>(xrow + head);
         Pack<T> *zr = reinterpret_cast<Pack<T> *>(zrow + head);
         Pack<T> cache[PACKS];
+        // (one branch round all the loads, none round each: a load inside a branch of its own makes the compiler wait for
+        // the loads before it, and a lane's vectors then arrive one round trip after the other instead of together; a
+        // vector beyond the row re-reads the row's last one and is not used - a dead row reads the first row)
+        if (npack > 0) {
 #pragma unroll
-        for (int j = 0; j < PACKS; j++)
-            if (live && lane + j * GROUP < npack) cache[j] = loadPack(xr + lane + j * GROUP);
+            for (int j = 0; j < PACKS; j++) {
+                const Long at = lane + j * GROUP;
+                cache[j] = loadPack(xr + (at < npack ? at : npack - 1));
+            }
+        }
         C edge = hasEdge ? toCompute(xrow[edgeAt]) : (C)0;
         C mx = hasEdge ? edge : (C)-3.4028235e38;
 #pragma unroll
@@ -341,9 +348,16 @@ __global__ void __launch_bounds__(kColBlock) softmaxColRegKernel(const T *x, T *
     const Long row0 = (g * kColRowLanes + rl) * N;  // numRows is a multiple of N: a vector is all live or all dead
     const bool live = row0 < numRows;
     Pack<T> cache[PACKS];
+    // (unconditional loads, see softmaxRowRegKernel: a column beyond the matrix re-reads the lane's first one, a dead lane
+    // the matrix's first rows; neither is used.  cg < kColCols <= length wherever this kernel is chosen)
+    {
+        const Long liveRow = live ? row0 : 0;
 #pragma unroll
-    for (int j = 0; j < PACKS; j++)
-        if (live && cg + j * kColCols < length) cache[j] = loadPack(reinterpret_cast<const Pack<T> *>(x + row0 + (Long)(cg + j * kColCols) * xEl));
+        for (int j = 0; j < PACKS; j++) {
+            const int col = cg + j * kColCols < length ? cg + j * kColCols : (cg < length ? cg : 0);
+            cache[j] = loadPack(reinterpret_cast<const Pack<T> *>(x + liveRow + (Long)col * xEl));
+        }
+    }
     C mx[N], sum[N];
 #pragma unroll
     for (int e = 0; e < N; e++) mx[e] = (C)-3.4028235e38;
