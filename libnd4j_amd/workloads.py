@@ -455,6 +455,7 @@ def general_views(dev, seed=61, copies=None):
     xv, yv = _normal(rs, span, F32), _normal(rs, span, F32)
     tad1_023, tad1_23 = dev.tad(i1, [0, 2, 3]), dev.tad(i1, [2, 3])
     tad2_12, tad3_02 = dev.tad(i2, [1, 2]), dev.tad(i3, [0, 2])
+    bias_v, bvi, tad_v = _uniform(rs, cols, -1, 1), _vec(cols), dev.tad(vi, [1])
     tad1_02 = dev.tad(i1, [0, 2])
     cw_out, ocw = _vec(nchw[1] * nchw[3]), np.zeros(nchw[1] * nchw[3], F32)
     c_out, r_out = _vec(nchw[1]), _vec(cube[0])
@@ -504,6 +505,12 @@ def general_views(dev, seed=61, copies=None):
         cases.append(Case("pairwise_add_padded_rows", "pairwise", nv, 12 * nv,
                           lambda: ops.execPairwiseTransformFloat(exv, P_ADD, XV.ptr, XV.info_ptr, YV.ptr, YV.info_ptr, ZV.ptr, ZV.info_ptr, None),
                           lambda lib: (lib.pairwise(P_ADD, xv, vi, yv, vi, zc3, vi, None), zc3)[1], False, ZV.get))
+        BV = w.operand(bias_v, bvi)
+        DV = w.raw(np.array([1], np.int32))
+        exbv = dev.extra(vi, bvi, vi, tad=tad_v, tad_z=tad_v)
+        cases.append(Case("broadcast_add_row_padded_rows", "broadcast", nv, 8 * nv + 4 * cols,
+                          lambda: ops.execBroadcastFloat(exbv, B_ADD, XV.ptr, XV.info_ptr, BV.ptr, BV.info_ptr, ZV.ptr, ZV.info_ptr, DV.ptr, 1),
+                          lambda lib: (lib.broadcast(B_ADD, xv, vi, bias_v, bvi, zc3, vi, [1]), zc3)[1], False, ZV.get))
         cases.append(Case("transform_exp_padded_rows", "transform", nv, 8 * nv,
                           lambda: ops.execTransformFloat(exv, T_EXP, XV.ptr, XV.info_ptr, ZV.ptr, ZV.info_ptr, None),
                           lambda lib: (lib.transform(T_EXP, xv, vi, zc3, vi, None), zc3)[1], False, ZV.get))
@@ -513,7 +520,7 @@ def general_views(dev, seed=61, copies=None):
 
     return _replicated(dev, "general views: multi-dimensional TADs on [128,128,56,56] / [4096,128,128] / [256,1024,256], rows with a pitch",
                        4 * n1 + 4 * n2 + 8 * n3, dict(x1=x1, i1=i1, x2=x2, i2=i2, x3=x3, i3=i3, plane=plane, pi=pi, mat=mat, mi=mi,
-                                                      xv=xv, yv=yv, vi=vi), device_set, copies)
+                                                      xv=xv, yv=yv, vi=vi, bias_v=bias_v), device_set, copies)
 
 
 # ---- data-movement specials: gathers, concatenations, reorders, conversions ---------------------------------

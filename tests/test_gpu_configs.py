@@ -222,6 +222,11 @@ def test_general_views_at_benchmark_size(gpu, lib):
         assert np.array_equal(view(got), view(h["xv"]) + view(h["yv"]))
         assert np.array_equal(view(got), view(c.cpu(lib)))
         assert not gaps(got).any()
+        c = w.case("broadcast_add_row_padded_rows")
+        got = _run(c)
+        assert np.array_equal(view(got), view(h["xv"]) + h["bias_v"][None, :])
+        assert np.array_equal(view(got), view(c.cpu(lib)))
+        assert not gaps(got).any()
         c = w.case("transform_exp_padded_rows")
         got = _run(c)
         assert ulp_distance(view(got), view(c.cpu(lib))).max() <= 2
