@@ -57,6 +57,10 @@ template <class Pol> struct PolChains<Pol, decltype((void)Pol::kChains)> { stati
 template <class Pol, typename = void> struct PolFlatBlocks { static constexpr int value = 2048; };
 template <class Pol> struct PolFlatBlocks<Pol, decltype((void)Pol::kFlatBlocks)> { static constexpr int value = Pol::kFlatBlocks; };
 
+// The blocks a policy wants in all for the strided vector kernel (a member constant kColBlocks; 2048 otherwise).
+template <class Pol, typename = void> struct PolColBlocks { static constexpr int value = 2048; };
+template <class Pol> struct PolColBlocks<Pol, decltype((void)Pol::kColBlocks)> { static constexpr int value = Pol::kColBlocks; };
+
 // Whether the clearing form of the whole-array kernel is built for a policy (a member constant kClears).
 template <class Pol, typename = void> struct PolClears { static constexpr bool value = false; };
 template <class Pol> struct PolClears<Pol, decltype((void)Pol::kClears)> { static constexpr bool value = Pol::kClears; };
@@ -814,7 +818,11 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         // lane per Pack::N adjacent TADs, 64 lanes per block column, rows split over the block's waves and blockIdx.y
         constexpr int VEC = Pack<typename Pol::T>::N;
         int gx = (int)((pl.numTads + (Long)kWave * VEC - 1) / ((Long)kWave * VEC));
-        Long splits = 2048 / gx;
+        // (blocks in all - kColBlocks of the policy: sums and maxima over [16384, 4096] along dimension 0 take 45.5 us with
+        // 512 or 384 blocks, 46.3 with 1024, 47.5 with 2048, 53 with 4096 - every block less is a row of partial results less
+        // to write and merge, and four 16-byte loads in flight per lane keep the memory busy from two blocks a compute unit;
+        // index reductions, with more arithmetic per element, want 2048 (49.3 us, 51 with 512))
+        Long splits = PolColBlocks<Pol>::value / gx;
         if (splits < 1) splits = 1;
         Long maxSplitsByRows = (pl.tadLength + 63) / 64;  // at least 16 rows per wave
         if (splits > maxSplitsByRows) splits = maxSplitsByRows;

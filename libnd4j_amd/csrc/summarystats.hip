@@ -50,6 +50,7 @@ template <typename TT, int OP> struct StatsPol {
     typedef typename Compute<TT>::type C;
     typedef StatsAcc Acc;
     static constexpr bool tables = false;  // no exp / log / pow in these accumulators
+    static constexpr int kColBlocks = 1024;  // blocks of the strided vector kernel (see runTadReduce)
     int biasCorrected;
     int phantomZero;  // the reference's single-dimension non-EWS branch starts from a zero sample
 
