@@ -354,12 +354,6 @@ def main():
                     # instructions need this long on the chip's 1024 SIMDs
                     issue_ms = v * c.elements / 64.0 * 4.0 / (1024 * 2.4e9) * 1e3
                     row["valu"] = {"instructions_per_element": v, "issue_ms": round(issue_ms, 4), "frac": round(issue_ms / ms, 4)}
-                    # the time the vector units were held, by the chip's own count (SQ_ACTIVE_INST_VALU; like the issue
-                    # time it prices every instruction at one slot, so both are lower bounds)
-                    busy = valu_per_element(args.instructions, c.name, "VALU busy time")
-                    if busy is not None:
-                        row["valu"]["busy_ms"] = busy
-                        row["valu"]["busy_frac"] = round(busy / ms, 4)
                 t = measured_traffic(args.traffic, c.name + " ")
                 if t is not None:  # HBM bytes the call moved, by the chip's counters (profiles/): well above `bytes` = re-reads
                     row["traffic"] = t

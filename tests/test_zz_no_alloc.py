@@ -52,10 +52,15 @@ def test_no_alloc_reduce_matches_the_allocating_entry_point():
         x = rs.randn(3 * n).astype(np.float32)
         want, got = _both(dev, MAX, x, harness.shape_info([1, n], strides=[3, 3], ews=3))
         assert want == got
-    # agreement with numpy on top of agreement with the other entry point
+    # agreement with float64 numpy on top of agreement with the other entry point (which shares the kernels)
     x = rs.uniform(-1, 1, 123457).astype(np.float32)
-    _, got = _both(dev, SUM, x, harness.shape_info([1, x.size]))
-    assert abs(float(np.uint32(got).view(np.float32)) - x.astype(np.float64).sum()) < 1e-5 * np.abs(x).sum()
+    x64 = x.astype(np.float64)
+    truth = {SUM: x64.sum(), MAX: x64.max(), NORM2: np.sqrt((x64 * x64).sum()), LOGSUMEXP: np.log(np.exp(x64 - x64.max()).sum()) + x64.max()}
+    for op, want in truth.items():
+        _, got = _both(dev, op, x, harness.shape_info([1, x.size]))
+        value = float(np.uint32(got).view(np.float32))
+        bound = 1e-5 * (np.abs(x64).sum() if op == SUM else abs(want))
+        assert value == want if op == MAX else abs(value - want) <= bound, (op, value, want)
 
 
 def test_no_alloc_reduce_refuses_what_it_cannot_do():
