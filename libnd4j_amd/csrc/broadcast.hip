@@ -49,7 +49,7 @@ template <typename T> struct BroadcastBody {
                 if (gy > 65535) gy = 65535;
                 ND4J_LAUNCH((bcColKernel<T, F, false>), dim3(gx, (unsigned)gy), dim3(kBlock), 0, s, x, y, z, pl.xOffsets,
                                    pl.zOffsets, pl.tadLength, pl.numTads, pl.tadEws, pl.yEws, pl.zEws, Params<T>{nullptr});
-            } else if (pl.runLength > 0) {
+            } else if (pl.runLength > 0 && runUnits<T>(pl.numTads, pl.tadLength, pl.runLength) <= kMaxRunUnits) {
                 // TADs over several dimensions whose innermost one is contiguous in x, y and z
                 launchRuns<T, F, true>(s, x, pl.xm, y, pl.ym, z, pl.zm, pl.xOffsets, pl.zOffsets, Params<T>{nullptr}, pl.numTads,
                                  pl.tadLength, pl.runLength, pl.runMajor);

@@ -500,38 +500,30 @@ __device__ __forceinline__ Long runOffset(const DimMap &mp, unsigned m, unsigned
 // both serve totals below 2^31 units, larger ones take 64-bit divisions.
 template <typename T, typename F, int U>
 __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, const T *y, DimMap ym, T *z, DimMap zm,
-                                                       const Long *xOffsets, const Long *zOffsets, Params<T> p, Long numTads,
-                                                       unsigned tadLength, unsigned runLength, int runMajor, FastDiv perRun,
-                                                       FastDiv second) {
+                                                       const Long *xOffsets, const Long *zOffsets, Params<T> p, unsigned total,
+                                                       unsigned runLength, int runMajor, FastDiv perRun, FastDiv second) {
     typedef typename Compute<T>::type C;
     constexpr int VEC = Pack<T>::N;
     constexpr bool two = F::nin == 2;
-    const unsigned unitsPerRun = (runLength + VEC - 1) / VEC;
-    const unsigned runsPerTad = tadLength / runLength;
-    const Long total = numTads * ((Long)runsPerTad * unitsPerRun);
-    const bool small = total <= 0x7fffffffLL;
-    const Long step = (Long)gridDim.x * kBlock;
+    // (everything that numbers units is 32-bit - the host sends calls of 2^31 units or more elsewhere: with 64-bit
+    // counters and the divisions they bring, a wave spent 200 instructions of its compute unit's one scalar unit on a
+    // single vector, which set the pace)
+    const unsigned step = gridDim.x * kBlock;
 
     // g -> (TAD r, run m of the TAD, unit c of the run)
-    auto locate = [&](Long g, Long &r, unsigned &m, unsigned &c) {
-        if (small) {
-            const unsigned t = perRun.divmod((unsigned)g, c);
-            unsigned rem;
-            const unsigned q = second.divmod(t, rem);
-            if (runMajor) { m = q; r = rem; }
-            else { r = q; m = rem; }
-        } else {
-            const Long t = g / unitsPerRun;
-            c = (unsigned)(g - t * unitsPerRun);
-            if (runMajor) { m = (unsigned)(t / numTads); r = t - (Long)m * numTads; }
-            else { r = t / runsPerTad; m = (unsigned)(t - r * runsPerTad); }
-        }
+    auto locate = [&](unsigned g, unsigned &r, unsigned &m, unsigned &c) {
+        const unsigned t = perRun.divmod(g, c);
+        unsigned rem;
+        const unsigned q = second.divmod(t, rem);
+        if (runMajor) { m = q; r = rem; }
+        else { r = q; m = rem; }
     };
     if constexpr (U > 1) {
         // With offset tables a unit costs two trips to memory, one after the other (its TAD's offsets, then its vectors): U
         // units per thread go through each stage together, so that what is in flight stays ahead of the memory's latency.
         if (F::tables) lm::loadTables();
-        for (Long g0 = (Long)blockIdx.x * kBlock + threadIdx.x; g0 < total; g0 += step * U) {
+        const bool shortRuns = runLength % VEC != 0;  // some units hold fewer elements than a vector
+        for (unsigned g0 = blockIdx.x * kBlock + threadIdx.x; g0 < total; g0 += step * U) {
             unsigned m[U], c[U];
             Long xo[U], zo[U];
             bool live[U];
@@ -539,9 +531,9 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
             // would make each such load wait for those before it - and is neither worked on nor stored)
 #pragma unroll
             for (int k = 0; k < U; k++) {
-                const Long g = g0 + k * step;
-                live[k] = g < total;
-                Long r;
+                const unsigned g = g0 + k * step;
+                live[k] = g < total && g >= g0;  // (g >= g0: no wrap of the 32-bit sum)
+                unsigned r;
                 locate(live[k] ? g : total - 1, r, m[k], c[k]);
                 xo[k] = xOffsets != nullptr ? xOffsets[r] : 0;
                 zo[k] = zOffsets != nullptr ? zOffsets[r] : 0;
@@ -550,7 +542,6 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
             T *zp[U];
             Pack<T> a[U], b[U];
             bool whole[U];
-            const bool shortRuns = runLength % VEC != 0;  // some units hold fewer elements than a vector
 #pragma unroll
             for (int k = 0; k < U; k++) {
                 xp[k] = x + xo[k] + runOffset(xm, m[k], c[k] * VEC, runLength);
@@ -580,6 +571,7 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
                         zp[k][e] = fromCompute<T>(F::template apply<C>(toCompute(xp[k][e]), two ? toCompute(yp[k][e]) : (C)0, p));
                 }
             }
+            if (g0 + step * U < g0) break;  // the next round's first unit would wrap round
         }
         return;
     }
@@ -588,9 +580,8 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
     unsigned count = 0;
     Pack<T> a, b;
     // the three addresses of unit g; requests the unit's vectors
-    auto fetch = [&](Long g, const T *&ux, const T *&uy, T *&uz, unsigned &ucount, Pack<T> &ua, Pack<T> &ub) {
-        Long r;
-        unsigned m, c;
+    auto fetch = [&](unsigned g, const T *&ux, const T *&uy, T *&uz, unsigned &ucount, Pack<T> &ua, Pack<T> &ub) {
+        unsigned r, m, c;
         locate(g, r, m, c);
         ucount = runLength - c * VEC;  // elements left in the run from the unit's first one on
         ux = x + (xOffsets != nullptr ? xOffsets[r] : 0) + runOffset(xm, m, c * VEC, runLength);
@@ -601,13 +592,13 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
             if (two) ub = loadPackAnywhere(uy);  // through the caches: every TAD reads it again
         }
     };
-    Long g = (Long)blockIdx.x * kBlock + threadIdx.x;
+    unsigned g = blockIdx.x * kBlock + threadIdx.x;
     bool have = g < total;
     if (have) fetch(g, xp, yp, zp, count, a, b);
     if (F::tables) lm::loadTables();  // staged while the first vectors are on their way
     while (have) {
-        const Long gn = g + step;
-        const bool haveNext = gn < total;
+        const unsigned gn = g + step;
+        const bool haveNext = gn < total && gn > g;
         const T *nxp = nullptr, *nyp = nullptr;
         T *nzp = nullptr;
         unsigned ncount = 0;
@@ -650,28 +641,33 @@ template <typename T> inline int commonHead(const void *a, const void *b, const 
     return (int)(((16 - (pa & 15)) & 15) / sizeof(T));
 }
 
-// grid and divisors of ewRunsKernel for `numTads` TADs of tadLength elements in runs of runLength; OFFSETS: the call
-// carries per-TAD offset tables (a compile-time choice, so that each family builds only the form it launches)
+// The most units (vectors inside runs) a call of ewRunsKernel may have, and their number for `numTads` TADs of tadLength
+// elements in runs of runLength; callers send larger calls to the element-wise kernels.
+static constexpr Long kMaxRunUnits = 0x7fffffffLL;
+template <typename T> inline Long runUnits(Long numTads, Long tadLength, unsigned runLength) {
+    const Long perTad = tadLength / runLength * ((runLength + Pack<T>::N - 1) / Pack<T>::N);
+    if (perTad <= 0 || numTads > kMaxRunUnits / perTad) return kMaxRunUnits + 1;
+    return numTads * perTad;
+}
+// grid and divisors of ewRunsKernel; OFFSETS: the call carries per-TAD offset tables (a compile-time choice, so that each
+// family builds only the form it launches)
 template <typename T, typename F, bool OFFSETS>
 inline void launchRuns(hipStream_t s, const T *x, const DimMap &xm, const T *y, const DimMap &ym, T *z, const DimMap &zm,
                        const Long *xOffsets, const Long *zOffsets, Params<T> p, Long numTads, Long tadLength, unsigned runLength,
                        bool runMajor) {
     const unsigned unitsPerRun = (runLength + Pack<T>::N - 1) / Pack<T>::N;
     const Long runsPerTad = tadLength / runLength;
-    const Long units = numTads * runsPerTad * unitsPerRun;
+    const Long units = runUnits<T>(numTads, tadLength, runLength);
     const FastDiv perRun(unitsPerRun);
-    const Long by = runMajor ? numTads : runsPerTad;
-    const FastDiv second((unsigned)(by > 0x7fffffffLL ? 0x7fffffffLL : by));
+    const FastDiv second((unsigned)(runMajor ? numTads : runsPerTad));
     // with offset tables: two units per thread and round (one: 54-63 % of the HBM peak on a [256,1024,256] array broadcast
     // along dimensions {0,2}, two: 68 %, four: 60 %); without, one unit per thread and the next one's loads ahead
     if constexpr (OFFSETS) {
         ND4J_LAUNCH((ewRunsKernel<T, F, 2>), dim3(gridFor(units, kBlock * 2, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0, s,
-                           x, xm, y, ym, z, zm, xOffsets, zOffsets, p, numTads, (unsigned)tadLength, runLength, runMajor ? 1 : 0, perRun,
-                           second);
+                           x, xm, y, ym, z, zm, xOffsets, zOffsets, p, (unsigned)units, runLength, runMajor ? 1 : 0, perRun, second);
     } else {
         ND4J_LAUNCH((ewRunsKernel<T, F, 1>), dim3(gridFor(units, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0, s,
-                           x, xm, y, ym, z, zm, xOffsets, zOffsets, p, numTads, (unsigned)tadLength, runLength, runMajor ? 1 : 0, perRun,
-                           second);
+                           x, xm, y, ym, z, zm, xOffsets, zOffsets, p, (unsigned)units, runLength, runMajor ? 1 : 0, perRun, second);
     }
 }
 
@@ -833,7 +829,7 @@ inline void launchGeneral(hipStream_t s, const T *x, const DimMap &xm, const T *
     // rows with a pitch and the like: contiguous runs along the innermost dimension of every operand
     const DimMap *const maps[3] = {&xm, two ? &ym : nullptr, &zm};
     const unsigned run = commonRunLength(maps);
-    if (run >= (unsigned)Pack<T>::N && n <= 0x7fffffffLL) {
+    if (run >= (unsigned)Pack<T>::N && n <= 0x7fffffffLL && runUnits<T>(1, n, run) <= kMaxRunUnits) {
         launchRuns<T, F, false>(s, x, xm, two ? y : x, two ? ym : xm, z, zm, nullptr, nullptr, p, 1, n, run, false);
         return;
     }
