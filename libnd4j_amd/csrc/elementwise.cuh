@@ -501,20 +501,31 @@ __device__ __forceinline__ Long runOffset(const DimMap &mp, unsigned m, unsigned
 template <typename T, typename F, int U>
 __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, const T *y, DimMap ym, T *z, DimMap zm,
                                                        const Long *xOffsets, const Long *zOffsets, Params<T> p, unsigned total,
-                                                       unsigned runLength, int runMajor, FastDiv perRun, FastDiv second) {
+                                                       unsigned runLength, int runMajor, FastDiv perRun, FastDiv second,
+                                                       unsigned unitStep, unsigned runStep) {
     typedef typename Compute<T>::type C;
     constexpr int VEC = Pack<T>::N;
     constexpr bool two = F::nin == 2;
     // (everything that numbers units is 32-bit - the host sends calls of 2^31 units or more elsewhere: with 64-bit
     // counters and the divisions they bring, a wave spent 200 instructions of its compute unit's one scalar unit on a
-    // single vector, which set the pace)
+    // single vector)
     const unsigned step = gridDim.x * kBlock;
-
-    // g -> (TAD r, run m of the TAD, unit c of the run)
-    auto locate = [&](unsigned g, unsigned &r, unsigned &m, unsigned &c) {
-        const unsigned t = perRun.divmod(g, c);
+    const unsigned unitsPerRun = perRun.d;
+    // A thread's units lie `step` apart: the first one's run t (counted over all TADs) and place c in it come from a
+    // division, the later ones from adding step / unitsPerRun and step % unitsPerRun (unitStep, runStep: from the host).
+    unsigned g = blockIdx.x * kBlock + threadIdx.x;
+    unsigned c, t;
+    t = perRun.divmod(g, c);
+    auto advance = [&]() {
+        g += step;
+        c += unitStep;
+        t += runStep;
+        if (c >= unitsPerRun) { c -= unitsPerRun; t++; }
+    };
+    // run t -> (TAD r, run m of the TAD)
+    auto split = [&](unsigned run, unsigned &r, unsigned &m) {
         unsigned rem;
-        const unsigned q = second.divmod(t, rem);
+        const unsigned q = second.divmod(run, rem);
         if (runMajor) { m = q; r = rem; }
         else { r = q; m = rem; }
     };
@@ -523,20 +534,23 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
         // units per thread go through each stage together, so that what is in flight stays ahead of the memory's latency.
         if (F::tables) lm::loadTables();
         const bool shortRuns = runLength % VEC != 0;  // some units hold fewer elements than a vector
-        for (unsigned g0 = blockIdx.x * kBlock + threadIdx.x; g0 < total; g0 += step * U) {
-            unsigned m[U], c[U];
+        while (g < total) {
+            unsigned m[U], first[U];
             Long xo[U], zo[U];
             bool live[U];
-            // (a unit beyond the end is placed on the last one, so that no load sits in a branch of its own - the compiler
-            // would make each such load wait for those before it - and is neither worked on nor stored)
+            // (a unit beyond the end is placed on the array's first one, so that no load sits in a branch of its own - the
+            // compiler would make each such load wait for those before it - and is neither worked on nor stored)
 #pragma unroll
             for (int k = 0; k < U; k++) {
-                const unsigned g = g0 + k * step;
-                live[k] = g < total && g >= g0;  // (g >= g0: no wrap of the 32-bit sum)
+                live[k] = g < total;
                 unsigned r;
-                locate(live[k] ? g : total - 1, r, m[k], c[k]);
+                split(live[k] ? t : 0, r, m[k]);
+                first[k] = live[k] ? c * VEC : 0;
                 xo[k] = xOffsets != nullptr ? xOffsets[r] : 0;
                 zo[k] = zOffsets != nullptr ? zOffsets[r] : 0;
+                const unsigned before = g;
+                advance();
+                if (g < before) g = total;  // (the 32-bit sum wrapped round: past the end)
             }
             const T *xp[U], *yp[U];
             T *zp[U];
@@ -544,10 +558,10 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
             bool whole[U];
 #pragma unroll
             for (int k = 0; k < U; k++) {
-                xp[k] = x + xo[k] + runOffset(xm, m[k], c[k] * VEC, runLength);
-                zp[k] = z + zo[k] + runOffset(zm, m[k], c[k] * VEC, runLength);
-                if (two) yp[k] = y + runOffset(ym, m[k], c[k] * VEC, runLength);
-                whole[k] = !shortRuns || runLength - c[k] * VEC >= (unsigned)VEC;
+                xp[k] = x + xo[k] + runOffset(xm, m[k], first[k], runLength);
+                zp[k] = z + zo[k] + runOffset(zm, m[k], first[k], runLength);
+                if (two) yp[k] = y + runOffset(ym, m[k], first[k], runLength);
+                whole[k] = !shortRuns || runLength - first[k] >= (unsigned)VEC;
                 if (!shortRuns) {
                     a[k] = streamPackAnywhere(xp[k]);
                     if (two) b[k] = loadPackAnywhere(yp[k]);
@@ -566,12 +580,11 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
                         o.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a[k].v[e]), two ? toCompute(b[k].v[e]) : (C)0, p));
                     streamPackAnywhere(zp[k], o);
                 } else if (live[k]) {
-                    const unsigned count = runLength - c[k] * VEC;
+                    const unsigned count = runLength - first[k];
                     for (unsigned e = 0; e < count; e++)
                         zp[k][e] = fromCompute<T>(F::template apply<C>(toCompute(xp[k][e]), two ? toCompute(yp[k][e]) : (C)0, p));
                 }
             }
-            if (g0 + step * U < g0) break;  // the next round's first unit would wrap round
         }
         return;
     }
@@ -579,10 +592,10 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
     T *zp = nullptr;
     unsigned count = 0;
     Pack<T> a, b;
-    // the three addresses of unit g; requests the unit's vectors
-    auto fetch = [&](unsigned g, const T *&ux, const T *&uy, T *&uz, unsigned &ucount, Pack<T> &ua, Pack<T> &ub) {
-        unsigned r, m, c;
-        locate(g, r, m, c);
+    // the three addresses of the unit the walk stands on; requests the unit's vectors
+    auto fetch = [&](const T *&ux, const T *&uy, T *&uz, unsigned &ucount, Pack<T> &ua, Pack<T> &ub) {
+        unsigned r, m;
+        split(t, r, m);
         ucount = runLength - c * VEC;  // elements left in the run from the unit's first one on
         ux = x + (xOffsets != nullptr ? xOffsets[r] : 0) + runOffset(xm, m, c * VEC, runLength);
         uz = z + (zOffsets != nullptr ? zOffsets[r] : 0) + runOffset(zm, m, c * VEC, runLength);
@@ -592,18 +605,18 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
             if (two) ub = loadPackAnywhere(uy);  // through the caches: every TAD reads it again
         }
     };
-    unsigned g = blockIdx.x * kBlock + threadIdx.x;
     bool have = g < total;
-    if (have) fetch(g, xp, yp, zp, count, a, b);
+    if (have) fetch(xp, yp, zp, count, a, b);
     if (F::tables) lm::loadTables();  // staged while the first vectors are on their way
     while (have) {
-        const unsigned gn = g + step;
-        const bool haveNext = gn < total && gn > g;
+        const unsigned before = g;
+        advance();
+        const bool haveNext = g < total && g > before;
         const T *nxp = nullptr, *nyp = nullptr;
         T *nzp = nullptr;
         unsigned ncount = 0;
         Pack<T> na, nb;
-        if (haveNext) fetch(gn, nxp, nyp, nzp, ncount, na, nb);
+        if (haveNext) fetch(nxp, nyp, nzp, ncount, na, nb);
         if (count >= (unsigned)VEC) {
             Pack<T> o;
 #pragma unroll
@@ -614,7 +627,7 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
             for (unsigned e = 0; e < count; e++)
                 zp[e] = fromCompute<T>(F::template apply<C>(toCompute(xp[e]), two ? toCompute(yp[e]) : (C)0, p));
         }
-        g = gn; have = haveNext;
+        have = haveNext;
         xp = nxp; yp = nyp; zp = nzp; count = ncount; a = na; b = nb;
     }
 }
@@ -662,13 +675,11 @@ inline void launchRuns(hipStream_t s, const T *x, const DimMap &xm, const T *y, 
     const FastDiv second((unsigned)(runMajor ? numTads : runsPerTad));
     // with offset tables: two units per thread and round (one: 54-63 % of the HBM peak on a [256,1024,256] array broadcast
     // along dimensions {0,2}, two: 68 %, four: 60 %); without, one unit per thread and the next one's loads ahead
-    if constexpr (OFFSETS) {
-        ND4J_LAUNCH((ewRunsKernel<T, F, 2>), dim3(gridFor(units, kBlock * 2, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0, s,
-                           x, xm, y, ym, z, zm, xOffsets, zOffsets, p, (unsigned)units, runLength, runMajor ? 1 : 0, perRun, second);
-    } else {
-        ND4J_LAUNCH((ewRunsKernel<T, F, 1>), dim3(gridFor(units, kBlock, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0, s,
-                           x, xm, y, ym, z, zm, xOffsets, zOffsets, p, (unsigned)units, runLength, runMajor ? 1 : 0, perRun, second);
-    }
+    const unsigned grid = gridFor(units, OFFSETS ? kBlock * 2 : kBlock, F::tables ? kGridCap : kMaxGrid);
+    const unsigned long long step = (unsigned long long)grid * kBlock;  // at most 2^32 - 256
+    const unsigned unitStep = (unsigned)(step % unitsPerRun), runStep = (unsigned)(step / unitsPerRun);
+    ND4J_LAUNCH((ewRunsKernel<T, F, OFFSETS ? 2 : 1>), dim3(grid), dim3(kBlock), 0, s, x, xm, y, ym, z, zm, xOffsets, zOffsets, p,
+                       (unsigned)units, runLength, runMajor ? 1 : 0, perRun, second, unitStep, runStep);
 }
 
 template <typename T, typename F>
