@@ -62,6 +62,9 @@ template <class Pol, typename = void> struct PolColBlocks { static constexpr int
 template <class Pol> struct PolColBlocks<Pol, decltype((void)Pol::kColBlocks)> { static constexpr int value = Pol::kColBlocks; };
 
 // Whether the clearing form of the whole-array kernel is built for a policy (a member constant kClears).
+// and whether many column tiles (64 or more: TADs by the ten thousand) are better served by 256 blocks of 512 threads
+template <class Pol, typename = void> struct PolColWide { static constexpr bool value = false; };
+template <class Pol> struct PolColWide<Pol, decltype((void)Pol::kColWide)> { static constexpr bool value = Pol::kColWide; };
 template <class Pol, typename = void> struct PolClears { static constexpr bool value = false; };
 template <class Pol> struct PolClears<Pol, decltype((void)Pol::kClears)> { static constexpr bool value = Pol::kClears; };
 
@@ -226,9 +229,114 @@ __global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename P
     else partials[(Long)blockIdx.y * numTads + t] = acc;
 }
 
+// Hands a scalar result to a host that is waiting for it: the value goes out in 8-byte words of pinned host memory, each
+// the call's ticket (upper half) with 32 bits of the value (lower half), each one system-scope store.  The host takes
+// the value once every word shows the ticket; a word is complete or absent, so no fence (on this chip: a write-back of
+// the whole L2) has to separate value and signal.
+template <typename T> __device__ __forceinline__ void signalResult(unsigned long long *signal, unsigned ticket, T value) {
+    if (signal == nullptr) return;
+    constexpr int W = (sizeof(T) + 3) / 4;
+    struct Words { unsigned w[W]; };
+    Words in;
+    if constexpr (sizeof(T) == 2) in.w[0] = __builtin_bit_cast(unsigned short, value);
+    else in = __builtin_bit_cast(Words, value);
+#pragma unroll
+    for (int i = 0; i < W; i++)
+        __hip_atomic_store(signal + i, ((unsigned long long)ticket << 32) | in.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+static constexpr unsigned kFlatGroup = 32;          // blocks per first-level counter
+static constexpr unsigned kFlatCounterStride = 32;  // counters are this many 32-bit words (128 bytes) apart
+static constexpr unsigned kFlatMaxBlocks = 2048;    // 1 + kFlatMaxBlocks / kFlatGroup counters exist
+// How many 32-bit words of a policy's accumulator travel through the slots: all of them, unless the policy says that
+// only the first kSlotWords matter (trailing padding stays at home; the receiver fills it with zeros).
+template <class Pol, typename = void> struct SlotWords { static constexpr int value = sizeof(typename Pol::Acc) / 4; };
+template <class Pol> struct SlotWords<Pol, decltype((void)Pol::kSlotWords)> { static constexpr int value = Pol::kSlotWords; };
+
+template <typename A, int W = sizeof(A) / 4>
+__device__ __forceinline__ void publishSlots(unsigned long long *slot, const A &a, unsigned ticket) {
+    static_assert(sizeof(A) % 4 == 0, "accumulator must be a multiple of 4 bytes");
+    struct Words { unsigned w[sizeof(A) / 4]; };
+    const Words in = __builtin_bit_cast(Words, a);
+#pragma unroll
+    for (int i = 0; i < W; i++)
+        __hip_atomic_store(slot + i, ((unsigned long long)ticket << 32) | in.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// One word of a slot group: waits (bounded) until it carries `ticket`, starting from the value `v` already loaded.  Only
+// called for groups whose writer has already issued its stores, so the wait ends as soon as they land.
+// `missing` is set when the wait ran out (seconds: only a launch that has gone wrong gets there).
+__device__ __forceinline__ unsigned awaitSlot(const unsigned long long *slot, unsigned long long v, unsigned ticket, bool &missing) {
+    for (int tries = 0; (unsigned)(v >> 32) != ticket && tries < (1 << 22); tries++) {
+        __builtin_amdgcn_s_sleep(1);
+        v = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if ((unsigned)(v >> 32) != ticket) missing = true;
+    return (unsigned)v;
+}
+// What the merging block does when a slot never arrived (all its threads call this together): true tells the caller to
+// store NaN instead of a number made of stale words; the stream's fault word, when there is one, lets the host report it.
+__device__ __forceinline__ bool slotsWereMissing(bool missing, unsigned *fault) {
+    const bool any = __syncthreads_or(missing ? 1 : 0) != 0;
+    if (any && threadIdx.x == 0 && fault != nullptr) __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    return any;
+}
+template <typename T> __device__ __forceinline__ T notANumber() { return fromCompute<T>((typename Compute<T>::type)__builtin_nanf("")); }
+// Merges the slot groups first, first + stride, ... (count of them in all) into acc, in that order.  The loads of
+// several groups are issued together: they bypass the caches, and one after the other their latencies would add up to
+// more than the second launch they replace.
+template <class Pol>
+__device__ __forceinline__ bool mergeSlots(const Pol &pol, typename Pol::Acc &acc, const unsigned long long *slots, int first,
+                                           int stride, int count, unsigned ticket) {
+    bool missing = false;
+    typedef typename Pol::Acc Acc;
+    constexpr int W = SlotWords<Pol>::value;
+    constexpr int G = W <= 2 ? 8 : (W <= 4 ? 4 : 2);
+    struct Words { unsigned w[sizeof(Acc) / 4]; };
+    for (int i0 = first; i0 < count; i0 += stride * G) {
+        unsigned long long v[G][W];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const int i = i0 + g * stride;
+            if (i < count) {
+#pragma unroll
+                for (int w = 0; w < W; w++) v[g][w] = __hip_atomic_load(slots + (size_t)i * W + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const int i = i0 + g * stride;
+            if (i < count) {
+                Words out = {};
+#pragma unroll
+                for (int w = 0; w < W; w++) out.w[w] = awaitSlot(slots + (size_t)i * W + w, v[g][w], ticket, missing);
+                acc = pol.combine(acc, __builtin_bit_cast(Acc, out));
+            }
+        }
+    }
+    return missing;
+}
+
+// One thread of every block of a one-dimensional grid (of at most kFlatMaxBlocks blocks) calls this once, after it has
+// published the block's slots: true in the block that counts itself in last.  The counters are back at zero by then.
+// Atomics on one address are served one after the other, some 15 ns apiece: two thousand blocks on a single counter
+// cost more than the reduction itself.  So blocks count in groups of kFlatGroup, each group on a counter of its own (in
+// a memory channel of its own), and only the last block of each group goes on to the top counter.
+__device__ __forceinline__ bool countedInLast(unsigned *counter) {
+    const unsigned group = blockIdx.x / kFlatGroup, groups = (gridDim.x + kFlatGroup - 1) / kFlatGroup;
+    const unsigned members = group + 1 < groups ? kFlatGroup : gridDim.x - group * kFlatGroup;
+    unsigned *mine = counter + (size_t)(1 + group) * kFlatCounterStride;
+    bool last = __hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1;
+    if (last) {
+        __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1;
+        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return last;
+}
+
 // Strided TADs whose neighbours are neighbours in memory (columns of a c-order matrix, rows of an f-order
 // one): every lane owns Pack<T>::N adjacent TADs and reads them with one 16-byte load per row, so a wave
-// covers a contiguous kilobyte per row.  The four waves of a block take every fourth row of the block's row
+// covers a contiguous kilobyte per row.  The waves of a block (four, or eight) take the rows of the block's row
 // range [rowsPerSplit * blockIdx.y, ...) and merge through LDS; row ranges are merged by tadColFinish.
 // Lanes whose TADs are not adjacent / aligned (checked against the offsets table) walk them one by one.
 // (The four waves side by side instead - 4 KiB of every row to a block, each wave walking all the rows of the range, no
@@ -237,16 +345,22 @@ __global__ void __launch_bounds__(kBlock) tadColKernel(Pol pol, const typename P
 // MAPPED: the same for TADs over several dimensions whose innermost one is strided: row j of the TADs lies where the
 // coordinate map puts it (every stride of the map a multiple of the vector width, so that the vectors stay aligned);
 // a row's divisions are shared by the Pack::N TADs of a lane.
-template <class Pol, bool MAPPED = false>
-__global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
-                                                          typename Pol::Acc *partials, const Long *offsets, Long tadLength,
-                                                          Long numTads, Long tadEws, Long rowsPerSplit, DimMap tm = DimMap()) {
+// BLK: threads of a block (256, or 512 where the host finds that to pay).
+template <class Pol, bool MAPPED = false, int BLK = kBlock>
+__global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
+                                                       typename Pol::Acc *partials, const Long *offsets, Long tadLength,
+                                                       Long numTads, Long tadEws, Long rowsPerSplit, DimMap tm = DimMap(),
+                                                       unsigned long long *slots = nullptr, unsigned *counter = nullptr,
+                                                       unsigned slotTicket = 0, unsigned *fault = nullptr) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
     constexpr int VEC = Pack<T>::N;
-    constexpr int WAVES = kBlock / kWave;
+    constexpr int WAVES = BLK / kWave;
+    constexpr int W = SlotWords<Pol>::value;
+    constexpr int TILE = VEC * kWave;  // TADs of a column tile
     __shared__ Acc smem[(WAVES - 1) * kWave];
+    __shared__ int mergeHere;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const Long t0 = ((Long)blockIdx.x * kWave + lane) * VEC;
     const bool live = t0 < numTads;
@@ -318,7 +432,7 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
             }
         }
     }
-    // merge the four waves, one owned TAD at a time (keeps the LDS footprint at three waves of accumulators)
+    // merge the waves, one owned TAD at a time (keeps the LDS footprint at one accumulator per lane of the other waves)
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
         __syncthreads();
@@ -329,8 +443,55 @@ __global__ void __launch_bounds__(kBlock) tadColVecKernel(Pol pol, const typenam
 #pragma unroll
             for (int w = 0; w < WAVES - 1; w++) a = pe[e].combine(a, smem[w * kWave + lane]);
             if (gridDim.y == 1) z[t0 + e] = pe[e].finalize(a, tadLength);
+            else if (slots != nullptr)
+                publishSlots<Acc, W>(slots + (((size_t)blockIdx.x * gridDim.y + blockIdx.y) * TILE + e * kWave + lane) * W, a, slotTicket);
             else partials[(Long)blockIdx.y * numTads + t0 + e] = a;
         }
+    }
+    if (gridDim.y == 1 || slots == nullptr) return;
+    // One launch: the row ranges of a column tile count themselves in on the tile's counter once their slots are on the
+    // way, and the block that comes last merges the tile - a thread per TAD, the ranges in order, 16 slot groups in
+    // flight - and writes its results.  (Tiles finish at different times: only the last one's merge is not hidden.)
+    if (threadIdx.x == 0) {
+        unsigned *mine = counter + (size_t)blockIdx.x * kFlatCounterStride;
+        const bool last = __hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.y - 1;
+        if (last) __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        mergeHere = last ? 1 : 0;
+    }
+    __syncthreads();
+    if (!mergeHere) return;
+    struct Words { unsigned w[sizeof(Acc) / 4]; };
+    constexpr int G = W <= 1 ? 16 : (W <= 2 ? 8 : 4);
+    const int splits = (int)gridDim.y;
+    for (int k = threadIdx.x; k < TILE; k += BLK) {
+        const Long t = ((Long)blockIdx.x * kWave + k % kWave) * VEC + k / kWave;
+        if (t >= numTads) continue;
+        const unsigned long long *mine = slots + ((size_t)blockIdx.x * splits * TILE + k) * W;
+        Pol pm = pol;
+        pm.setTad(t, z);
+        Acc a;
+        bool missing = false;
+        for (int b0 = 0; b0 < splits; b0 += G) {
+            unsigned long long v[G][W];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const int b = b0 + g < splits ? b0 + g : splits - 1;
+#pragma unroll
+                for (int w = 0; w < W; w++) v[g][w] = __hip_atomic_load(mine + (size_t)b * TILE * W + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                if (b0 + g < splits) {
+                    Words out = {};
+#pragma unroll
+                    for (int w = 0; w < W; w++) out.w[w] = awaitSlot(mine + (size_t)(b0 + g) * TILE * W + w, v[g][w], slotTicket, missing);
+                    const Acc piece = __builtin_bit_cast(Acc, out);
+                    a = (b0 + g == 0) ? piece : pm.combine(a, piece);
+                }
+            }
+        }
+        if (missing && fault != nullptr) __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        z[t] = missing ? notANumber<T>() : pm.finalize(a, tadLength);
     }
 }
 
@@ -516,111 +677,6 @@ __global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typena
         acc = blockMerge<Pol>(pol, acc, smem);
         if (threadIdx.x == 0) z[r] = pol.finalize(acc, tadLength);
     }
-}
-
-// Hands a scalar result to a host that is waiting for it: the value goes out in 8-byte words of pinned host memory, each
-// the call's ticket (upper half) with 32 bits of the value (lower half), each one system-scope store.  The host takes
-// the value once every word shows the ticket; a word is complete or absent, so no fence (on this chip: a write-back of
-// the whole L2) has to separate value and signal.
-template <typename T> __device__ __forceinline__ void signalResult(unsigned long long *signal, unsigned ticket, T value) {
-    if (signal == nullptr) return;
-    constexpr int W = (sizeof(T) + 3) / 4;
-    struct Words { unsigned w[W]; };
-    Words in;
-    if constexpr (sizeof(T) == 2) in.w[0] = __builtin_bit_cast(unsigned short, value);
-    else in = __builtin_bit_cast(Words, value);
-#pragma unroll
-    for (int i = 0; i < W; i++)
-        __hip_atomic_store(signal + i, ((unsigned long long)ticket << 32) | in.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-}
-
-static constexpr unsigned kFlatGroup = 32;          // blocks per first-level counter
-static constexpr unsigned kFlatCounterStride = 32;  // counters are this many 32-bit words (128 bytes) apart
-static constexpr unsigned kFlatMaxBlocks = 2048;    // 1 + kFlatMaxBlocks / kFlatGroup counters exist
-// How many 32-bit words of a policy's accumulator travel through the slots: all of them, unless the policy says that
-// only the first kSlotWords matter (trailing padding stays at home; the receiver fills it with zeros).
-template <class Pol, typename = void> struct SlotWords { static constexpr int value = sizeof(typename Pol::Acc) / 4; };
-template <class Pol> struct SlotWords<Pol, decltype((void)Pol::kSlotWords)> { static constexpr int value = Pol::kSlotWords; };
-
-template <typename A, int W = sizeof(A) / 4>
-__device__ __forceinline__ void publishSlots(unsigned long long *slot, const A &a, unsigned ticket) {
-    static_assert(sizeof(A) % 4 == 0, "accumulator must be a multiple of 4 bytes");
-    struct Words { unsigned w[sizeof(A) / 4]; };
-    const Words in = __builtin_bit_cast(Words, a);
-#pragma unroll
-    for (int i = 0; i < W; i++)
-        __hip_atomic_store(slot + i, ((unsigned long long)ticket << 32) | in.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// One word of a slot group: waits (bounded) until it carries `ticket`, starting from the value `v` already loaded.  Only
-// called for groups whose writer has already issued its stores, so the wait ends as soon as they land.
-// `missing` is set when the wait ran out (seconds: only a launch that has gone wrong gets there).
-__device__ __forceinline__ unsigned awaitSlot(const unsigned long long *slot, unsigned long long v, unsigned ticket, bool &missing) {
-    for (int tries = 0; (unsigned)(v >> 32) != ticket && tries < (1 << 22); tries++) {
-        __builtin_amdgcn_s_sleep(1);
-        v = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if ((unsigned)(v >> 32) != ticket) missing = true;
-    return (unsigned)v;
-}
-// What the merging block does when a slot never arrived (all its threads call this together): true tells the caller to
-// store NaN instead of a number made of stale words; the stream's fault word, when there is one, lets the host report it.
-__device__ __forceinline__ bool slotsWereMissing(bool missing, unsigned *fault) {
-    const bool any = __syncthreads_or(missing ? 1 : 0) != 0;
-    if (any && threadIdx.x == 0 && fault != nullptr) __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    return any;
-}
-template <typename T> __device__ __forceinline__ T notANumber() { return fromCompute<T>((typename Compute<T>::type)__builtin_nanf("")); }
-// Merges the slot groups first, first + stride, ... (count of them in all) into acc, in that order.  The loads of
-// several groups are issued together: they bypass the caches, and one after the other their latencies would add up to
-// more than the second launch they replace.
-template <class Pol>
-__device__ __forceinline__ bool mergeSlots(const Pol &pol, typename Pol::Acc &acc, const unsigned long long *slots, int first,
-                                           int stride, int count, unsigned ticket) {
-    bool missing = false;
-    typedef typename Pol::Acc Acc;
-    constexpr int W = SlotWords<Pol>::value;
-    constexpr int G = W <= 2 ? 8 : (W <= 4 ? 4 : 2);
-    struct Words { unsigned w[sizeof(Acc) / 4]; };
-    for (int i0 = first; i0 < count; i0 += stride * G) {
-        unsigned long long v[G][W];
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            const int i = i0 + g * stride;
-            if (i < count) {
-#pragma unroll
-                for (int w = 0; w < W; w++) v[g][w] = __hip_atomic_load(slots + (size_t)i * W + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            const int i = i0 + g * stride;
-            if (i < count) {
-                Words out = {};
-#pragma unroll
-                for (int w = 0; w < W; w++) out.w[w] = awaitSlot(slots + (size_t)i * W + w, v[g][w], ticket, missing);
-                acc = pol.combine(acc, __builtin_bit_cast(Acc, out));
-            }
-        }
-    }
-    return missing;
-}
-
-// One thread of every block of a one-dimensional grid (of at most kFlatMaxBlocks blocks) calls this once, after it has
-// published the block's slots: true in the block that counts itself in last.  The counters are back at zero by then.
-// Atomics on one address are served one after the other, some 15 ns apiece: two thousand blocks on a single counter
-// cost more than the reduction itself.  So blocks count in groups of kFlatGroup, each group on a counter of its own (in
-// a memory channel of its own), and only the last block of each group goes on to the top counter.
-__device__ __forceinline__ bool countedInLast(unsigned *counter) {
-    const unsigned group = blockIdx.x / kFlatGroup, groups = (gridDim.x + kFlatGroup - 1) / kFlatGroup;
-    const unsigned members = group + 1 < groups ? kFlatGroup : gridDim.x - group * kFlatGroup;
-    unsigned *mine = counter + (size_t)(1 + group) * kFlatCounterStride;
-    bool last = __hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1;
-    if (last) {
-        __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        last = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1;
-        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    return last;
 }
 
 // The full-array reduction: block b folds the chunks b, b+grid, ... of kBlock*kUnroll vectors.
@@ -822,9 +878,14 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         // 512 or 384 blocks, 46.3 with 1024, 47.5 with 2048, 53 with 4096 - every block less is a row of partial results less
         // to write and merge, and four 16-byte loads in flight per lane keep the memory busy from two blocks a compute unit;
         // index reductions, with more arithmetic per element, want 2048 (49.3 us, 51 with 512))
-        Long splits = PolColBlocks<Pol>::value / gx;
+        // (with 64 column tiles or more - max / sum along dimension 1 of an f-order [32768, 2048] - 256 blocks of 512 threads
+        // take 42.5 us where 512 of 256 take 44: half as many rows of partial results for a merge that has 32768 results to
+        // write; with 16 tiles the two measure the same, with 256 threads and 256 blocks 50 us)
+        const bool wide = PolColWide<Pol>::value && !mappedVec && gx >= 64;
+        const int waves = wide ? 8 : kBlock / kWave;
+        Long splits = (wide ? 256 : PolColBlocks<Pol>::value) / gx;
         if (splits < 1) splits = 1;
-        Long maxSplitsByRows = (pl.tadLength + 63) / 64;  // at least 16 rows per wave
+        Long maxSplitsByRows = (pl.tadLength + 16 * waves - 1) / (16 * waves);  // at least 16 rows per wave
         if (splits > maxSplitsByRows) splits = maxSplitsByRows;
         if (splits > 65535) splits = 65535;
         size_t need = (size_t)splits * (size_t)pl.numTads * sizeof(Acc);
@@ -834,13 +895,29 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         splits = (pl.tadLength + rowsPerSplit - 1) / rowsPerSplit;
         if (splits < 1) splits = 1;
         Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+        // One launch when the accumulators are one or two slot words, the tiles' counters exist (128 of them) and the slots
+        // hold a group per (tile, row range, TAD); otherwise the row ranges are merged by a second launch.  (What the second
+        // launch costs is small: sums along dimension 0 of [16384, 4096] take 45.6 us either way, maxima along dimension 1
+        // of an f-order [32768, 2048] 41.9 in one launch and 42.5 in two.  Accumulators of more words - index pairs, the
+        // statistics' moments - would have a tile's last block collect hundreds of words per thread: they keep the second
+        // launch, which spreads that over the chip.)
+        constexpr int W = SlotWords<Pol>::value;
+        const bool oneLaunch = splits > 1 && W <= 2 && ws.slots != nullptr && ws.counter != nullptr && ws.slotTicketSource != nullptr &&
+                               gx <= 128 && (size_t)gx * (size_t)splits * kWave * VEC * W * sizeof(unsigned long long) <= ws.slotBytes;
+        unsigned long long *slots = oneLaunch ? ws.slots : nullptr;
+        const unsigned slotTicket = oneLaunch ? ws.nextSlotTicket() : 0u;
         if (mappedVec)
             ND4J_LAUNCH((tadColVecKernel<Pol, true>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
-                               pl.offsets, pl.tadLength, pl.numTads, (Long)0, rowsPerSplit, pl.tm);
+                               pl.offsets, pl.tadLength, pl.numTads, (Long)0, rowsPerSplit, pl.tm, slots, ws.counter, slotTicket, ws.fault);
+        else if (wide)
+            ND4J_LAUNCH((tadColVecKernel<Pol, false, PolColWide<Pol>::value ? 512 : kBlock>), dim3(gx, (unsigned)splits), dim3(512), 0, s,
+                               pol, x, z, partials, pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit, DimMap(), slots,
+                               ws.counter, slotTicket, ws.fault);
         else
-        ND4J_LAUNCH((tadColVecKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
-                           pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit, DimMap());
-        if (splits > 1)
+            ND4J_LAUNCH((tadColVecKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
+                               pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit, DimMap(), slots, ws.counter, slotTicket,
+                               ws.fault);
+        if (splits > 1 && !oneLaunch)
             ND4J_LAUNCH((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kFinishLanes - 1) / kFinishLanes)), dim3(kBlock), 0, s, pol,
                                z, partials, pl.tadLength, pl.numTads, (int)splits);
         return;

@@ -1115,8 +1115,8 @@ def test_half_reductions_against_the_reference_loops(gpu, cpu):
 
 
 def test_slot_tickets_across_the_points_where_the_slots_are_cleared(gpu):
-    """Whole-array reductions, the whole-array reduce3 and the cooperative softmax kernels tag what their blocks exchange
-    with a per-stream launch ticket (30 bits of it for the softmax), and the exchange area is not cleared between launches.
+    """Whole-array reductions, strided reductions that finish in one launch, the whole-array reduce3 and the cooperative
+    softmax kernels tag what their blocks exchange with a per-stream launch ticket (30 bits of it for the softmax), and the exchange area is not cleared between launches.
     Data set A is run on the tickets just behind a multiple of 2^30; then the counter is put back to just before that
     multiple - where a long-running process arrives 2^30 launches later - and data set B is run: it draws the same tickets
     again, and must not see what A left behind (the library clears the area when the counter nears the boundary)."""
@@ -1124,6 +1124,7 @@ def test_slot_tickets_across_the_points_where_the_slots_are_cleared(gpu):
     n = 1 << 20
     xi = shape_info_np([1, n])
     rows = shape_info_np([4, 40000])
+    square = shape_info_np([1024, 1024])
     ex = gpu.dev.extra(xi)
 
     def data():
@@ -1137,7 +1138,11 @@ def test_slot_tickets_across_the_points_where_the_slots_are_cleared(gpu):
         x, y, xr, soft = d
         total, dot = x.astype(np.float64).sum(), (x.astype(np.float64) * y).sum()
         scale = np.abs(x).astype(np.float64).sum() / np.sqrt(n)
+        columns = x.astype(np.float64).reshape(1024, 1024).sum(axis=0)
+        column_scale = np.abs(x).astype(np.float64).reshape(1024, 1024).sum(axis=0)
         for k in range(6):
+            got = gpu.reduce(1, x, square, None, [0], 1024).astype(np.float64)
+            assert np.all(np.abs(got - columns) <= 1e-5 * column_scale), (what, k)
             assert abs(float(gpu.reduce_scalar(1, x, xi)) - total) <= 1e-5 * max(abs(total), scale), (what, k)
             assert float(gpu.indexreduce_scalar(0, x, xi)) == float(np.argmax(x)), (what, k)
             assert abs(float(gpu.reduce3_scalar(3, x, xi, y, xi)) - dot) <= 1e-4 * np.sqrt(n), (what, k)
