@@ -96,7 +96,6 @@ template <typename TT, int OP> struct ReducePol {
     static constexpr int kChains = 4;  // accumulators of one lane may be kept apart and combined (combine is the update)
     static constexpr int kFlatBlocks = 512;  // blocks of the whole-array kernel: two per compute unit (see runFlatReduce)
     static constexpr int kColBlocks = 512;   // and of the strided vector kernel (see runTadReduce)
-    static constexpr bool kColWide = true;   // 512-thread blocks for many column tiles (see runTadReduce)
     Params<TT> p;
     const TT *shiftSource;  // LogSumExp: per-TAD (TAD calls) or single (scalar calls) maximum; else null
     int shiftPerTad;

@@ -20,6 +20,7 @@
 //   flatKernel<Pol>           grid reduction over the whole array; the block that finishes last merges the blocks'
 //                             results (flatFinish<Pol>: the same merge as a second launch, for callers without slots).
 #pragma once
+#include <cstdlib>
 
 #include <hip/hip_runtime.h>
 
@@ -62,9 +63,6 @@ template <class Pol, typename = void> struct PolColBlocks { static constexpr int
 template <class Pol> struct PolColBlocks<Pol, decltype((void)Pol::kColBlocks)> { static constexpr int value = Pol::kColBlocks; };
 
 // Whether the clearing form of the whole-array kernel is built for a policy (a member constant kClears).
-// and whether many column tiles (64 or more: TADs by the ten thousand) are better served by 256 blocks of 512 threads
-template <class Pol, typename = void> struct PolColWide { static constexpr bool value = false; };
-template <class Pol> struct PolColWide<Pol, decltype((void)Pol::kColWide)> { static constexpr bool value = Pol::kColWide; };
 template <class Pol, typename = void> struct PolClears { static constexpr bool value = false; };
 template <class Pol> struct PolClears<Pol, decltype((void)Pol::kClears)> { static constexpr bool value = Pol::kClears; };
 
@@ -337,7 +335,9 @@ __device__ __forceinline__ bool countedInLast(unsigned *counter) {
 // Strided TADs whose neighbours are neighbours in memory (columns of a c-order matrix, rows of an f-order
 // one): every lane owns Pack<T>::N adjacent TADs and reads them with one 16-byte load per row, so a wave
 // covers a contiguous kilobyte per row.  The waves of a block (four, or eight) take the rows of the block's row
-// range [rowsPerSplit * blockIdx.y, ...) and merge through LDS; row ranges are merged by tadColFinish.
+// range and merge through LDS.  A block's rows are [rowsPerSplit * blockIdx.y, ...) or, with `dealt` rows to a batch, the
+// batches blockIdx.y, blockIdx.y + gridDim.y, ... of the TAD; the row ranges are merged by the last block of the column
+// tile to finish (when `slots` are given: one launch) or by tadColFinish.
 // Lanes whose TADs are not adjacent / aligned (checked against the offsets table) walk them one by one.
 // (The four waves side by side instead - 4 KiB of every row to a block, each wave walking all the rows of the range, no
 // merge through LDS - was slower: 52.6 against 48.6 us for sums along dim 0 of [16384, 4096], twice as slow for the
@@ -351,7 +351,7 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
                                                        typename Pol::Acc *partials, const Long *offsets, Long tadLength,
                                                        Long numTads, Long tadEws, Long rowsPerSplit, DimMap tm = DimMap(),
                                                        unsigned long long *slots = nullptr, unsigned *counter = nullptr,
-                                                       unsigned slotTicket = 0, unsigned *fault = nullptr) {
+                                                       unsigned slotTicket = 0, unsigned *fault = nullptr, Long dealt = 0) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
@@ -417,7 +417,13 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
                     }
                 }
             };
-            if constexpr (HasAscending<Pol>::value) {
+            if (dealt > 0) {
+                for (Long q = blockIdx.y; q * dealt < tadLength; q += gridDim.y) {
+                    const Long a = q * dealt, b = a + dealt < tadLength ? a + dealt : tadLength;
+                    if constexpr (HasAscending<Pol>::value) walk(a, b, std::true_type());
+                    else walk(a, b, std::false_type());
+                }
+            } else if constexpr (HasAscending<Pol>::value) {
                 walk(j0 + turn, j1, std::true_type());
                 walk(j0, j0 + turn, std::false_type());
             } else {
@@ -428,6 +434,13 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
             for (int e = 0; e < VEC; e++) {
                 if (t0 + e >= numTads) continue;
                 const T *base = x + off[e];
+                if (dealt > 0) {
+                    for (Long q = blockIdx.y; q * dealt < tadLength; q += gridDim.y) {
+                        const Long a = q * dealt, b = a + dealt < tadLength ? a + dealt : tadLength;
+                        for (Long j = a + wave; j < b; j += WAVES) { foldNext(pe[e], acc[e], toCompute(base[rowAt(j)]), j); pe[e].checkpoint(acc[e]); }
+                    }
+                    continue;
+                }
                 for (Long j = j0 + wave; j < j1; j += WAVES) { foldNext(pe[e], acc[e], toCompute(base[rowAt(j)]), j); pe[e].checkpoint(acc[e]); }
             }
         }
@@ -462,36 +475,63 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
     if (!mergeHere) return;
     struct Words { unsigned w[sizeof(Acc) / 4]; };
     constexpr int G = W <= 1 ? 16 : (W <= 2 ? 8 : 4);
+    // PARTS threads share a TAD when the block has more threads than the tile has TADs: each takes every PARTS-th batch of
+    // G row ranges, the first of them merges what the others hand over through LDS
+    constexpr int PARTS = BLK > TILE ? BLK / TILE : 1;
+    static_assert(PARTS == 1 || (PARTS - 1) * TILE <= (WAVES - 1) * kWave, "the hand-over reuses the waves' merge area");
     const int splits = (int)gridDim.y;
-    for (int k = threadIdx.x; k < TILE; k += BLK) {
+    __syncthreads();  // (the waves' merge area is free from here on)
+    for (int k0 = 0; k0 < TILE * PARTS; k0 += BLK) {
+        const int k = (k0 + (int)threadIdx.x) % TILE, part = (k0 + (int)threadIdx.x) / TILE;
         const Long t = ((Long)blockIdx.x * kWave + k % kWave) * VEC + k / kWave;
-        if (t >= numTads) continue;
+        const bool mineLive = t < numTads && part < PARTS;
         const unsigned long long *mine = slots + ((size_t)blockIdx.x * splits * TILE + k) * W;
         Pol pm = pol;
-        pm.setTad(t, z);
+        if (mineLive) pm.setTad(t, z);
         Acc a;
-        bool missing = false;
-        for (int b0 = 0; b0 < splits; b0 += G) {
-            unsigned long long v[G][W];
+        bool have = false, missing = false;
+        if (mineLive) {
+            for (int b0 = part * G; b0 < splits; b0 += PARTS * G) {
+                unsigned long long v[G][W];
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                const int b = b0 + g < splits ? b0 + g : splits - 1;
+                for (int g = 0; g < G; g++) {
+                    const int b = b0 + g < splits ? b0 + g : splits - 1;
 #pragma unroll
-                for (int w = 0; w < W; w++) v[g][w] = __hip_atomic_load(mine + (size_t)b * TILE * W + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+                    for (int w = 0; w < W; w++) v[g][w] = __hip_atomic_load(mine + (size_t)b * TILE * W + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                if (b0 + g < splits) {
-                    Words out = {};
+                for (int g = 0; g < G; g++) {
+                    if (b0 + g < splits) {
+                        Words out = {};
 #pragma unroll
-                    for (int w = 0; w < W; w++) out.w[w] = awaitSlot(mine + (size_t)(b0 + g) * TILE * W + w, v[g][w], slotTicket, missing);
-                    const Acc piece = __builtin_bit_cast(Acc, out);
-                    a = (b0 + g == 0) ? piece : pm.combine(a, piece);
+                        for (int w = 0; w < W; w++) out.w[w] = awaitSlot(mine + (size_t)(b0 + g) * TILE * W + w, v[g][w], slotTicket, missing);
+                        const Acc piece = __builtin_bit_cast(Acc, out);
+                        a = have ? pm.combine(a, piece) : piece;
+                        have = true;
+                    }
                 }
             }
         }
-        if (missing && fault != nullptr) __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        z[t] = missing ? notANumber<T>() : pm.finalize(a, tadLength);
+        if constexpr (PARTS > 1) {
+            __shared__ int handed[(PARTS - 1) * TILE];  // 0: nothing, 1: an accumulator, 2: a slot was missing
+            if (mineLive && part > 0) {
+                if (have) smem[(part - 1) * TILE + k] = a;
+                handed[(part - 1) * TILE + k] = missing ? 2 : (have ? 1 : 0);
+            }
+            __syncthreads();
+            if (mineLive && part == 0) {
+#pragma unroll
+                for (int q = 1; q < PARTS; q++) {
+                    const int h = handed[(q - 1) * TILE + k];
+                    if (h == 2) missing = true;
+                    else if (h == 1) { a = have ? pm.combine(a, smem[(q - 1) * TILE + k]) : smem[(q - 1) * TILE + k]; have = true; }
+                }
+            }
+        }
+        if (mineLive && part == 0) {
+            if (missing && fault != nullptr) __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            z[t] = missing ? notANumber<T>() : pm.finalize(a, tadLength);
+        }
     }
 }
 
@@ -874,14 +914,13 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         // lane per Pack::N adjacent TADs, 64 lanes per block column, rows split over the block's waves and blockIdx.y
         constexpr int VEC = Pack<typename Pol::T>::N;
         int gx = (int)((pl.numTads + (Long)kWave * VEC - 1) / ((Long)kWave * VEC));
-        // (blocks in all - kColBlocks of the policy: sums and maxima over [16384, 4096] along dimension 0 take 45.5 us with
-        // 512 or 384 blocks, 46.3 with 1024, 47.5 with 2048, 53 with 4096 - every block less is a row of partial results less
-        // to write and merge, and four 16-byte loads in flight per lane keep the memory busy from two blocks a compute unit;
-        // index reductions, with more arithmetic per element, want 2048 (49.3 us, 51 with 512))
-        // (with 64 column tiles or more - max / sum along dimension 1 of an f-order [32768, 2048] - 256 blocks of 512 threads
-        // take 42.5 us where 512 of 256 take 44: half as many rows of partial results for a merge that has 32768 results to
-        // write; with 16 tiles the two measure the same, with 256 threads and 256 blocks 50 us)
-        const bool wide = PolColWide<Pol>::value && !mappedVec && gx >= 64;
+        // Plain strided TADs: 256 blocks of 512 threads, whatever the policy (one block per compute unit: eight waves with four
+        // 16-byte loads in flight each keep the memory busy, and every block less is a row of partial results less to merge).
+        // Measured on [16384, 4096] along dimension 0 (16 column tiles) and on an f-order [32768, 2048] along dimension 1
+        // (128 tiles), in us: sums 42.9 / 41.8, index of the maximum 46.0, variance - / 48.6; with 256 threads and 512
+        // (sums), 2048 (index) or 1024 (statistics) blocks 45.6 / 44.0, 49.3 and 49.1; 512 or 1024 blocks of 512 threads
+        // are slower for all of them.  Mapped TADs keep 256 threads and the policy's kColBlocks.
+        const bool wide = !mappedVec;
         const int waves = wide ? 8 : kBlock / kWave;
         Long splits = (wide ? 256 : PolColBlocks<Pol>::value) / gx;
         if (splits < 1) splits = 1;
@@ -904,19 +943,22 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         constexpr int W = SlotWords<Pol>::value;
         const bool oneLaunch = splits > 1 && W <= 2 && ws.slots != nullptr && ws.counter != nullptr && ws.slotTicketSource != nullptr &&
                                gx <= 128 && (size_t)gx * (size_t)splits * kWave * VEC * W * sizeof(unsigned long long) <= ws.slotBytes;
+        // With eight row ranges or more a tile's rows are dealt to them a batch at a time (what all blocks have in flight is
+        // then one stretch of memory): 45.6 -> 42.9 us for the sums over 16 tiles above, 51 -> 46 for the index of the
+        // maximum; with two ranges (128 tiles) it changes nothing for sums and costs the statistics 3 us, so few ranges keep
+        // a contiguous share each.
+        Long dealt = wide && splits >= 8 ? 4 * waves : 0;
+        if (const char *e = getenv("ND4J_AMD_TUNE_MAPDEALT")) { if (mappedVec) dealt = atoi(e); }
         unsigned long long *slots = oneLaunch ? ws.slots : nullptr;
         const unsigned slotTicket = oneLaunch ? ws.nextSlotTicket() : 0u;
         if (mappedVec)
             ND4J_LAUNCH((tadColVecKernel<Pol, true>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
-                               pl.offsets, pl.tadLength, pl.numTads, (Long)0, rowsPerSplit, pl.tm, slots, ws.counter, slotTicket, ws.fault);
-        else if (wide)
-            ND4J_LAUNCH((tadColVecKernel<Pol, false, PolColWide<Pol>::value ? 512 : kBlock>), dim3(gx, (unsigned)splits), dim3(512), 0, s,
-                               pol, x, z, partials, pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit, DimMap(), slots,
-                               ws.counter, slotTicket, ws.fault);
+                               pl.offsets, pl.tadLength, pl.numTads, (Long)0, rowsPerSplit, pl.tm, slots, ws.counter, slotTicket, ws.fault,
+                               dealt);
         else
-            ND4J_LAUNCH((tadColVecKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials,
+            ND4J_LAUNCH((tadColVecKernel<Pol, false, 512>), dim3(gx, (unsigned)splits), dim3(512), 0, s, pol, x, z, partials,
                                pl.offsets, pl.tadLength, pl.numTads, pl.tadEws, rowsPerSplit, DimMap(), slots, ws.counter, slotTicket,
-                               ws.fault);
+                               ws.fault, dealt);
         if (splits > 1 && !oneLaunch)
             ND4J_LAUNCH((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kFinishLanes - 1) / kFinishLanes)), dim3(kBlock), 0, s, pol,
                                z, partials, pl.tadLength, pl.numTads, (int)splits);
