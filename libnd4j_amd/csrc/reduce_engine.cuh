@@ -20,7 +20,6 @@
 //   flatKernel<Pol>           grid reduction over the whole array; the block that finishes last merges the blocks'
 //                             results (flatFinish<Pol>: the same merge as a second launch, for callers without slots).
 #pragma once
-#include <cstdlib>
 
 #include <hip/hip_runtime.h>
 
@@ -389,7 +388,8 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
             const Long span = j1 - j0;
             const Long turn = span >= 8 * WAVES ? (((Long)blockIdx.y * 3) % (span / (4 * WAVES))) * (4 * WAVES) : 0;
             // (the first part is walked in ascending order from fresh accumulators; the second part's rows lie before the
-            // first's, so its elements are folded by the general rule)
+            // first's, so its elements are folded by the general rule.  Issuing the next batch's loads before the current
+            // batch is folded measured no better: sums 42.9 -> 43.8 us, variance 48.6 -> 48.0, mapped TADs 44.9 -> 47.3)
             auto walk = [&](Long a, Long b, auto ascending) {
                 Long j = a + wave;
                 for (; j + 3 * WAVES < b; j += 4 * WAVES) {
@@ -948,7 +948,6 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         // maximum; with two ranges (128 tiles) it changes nothing for sums and costs the statistics 3 us, so few ranges keep
         // a contiguous share each.
         Long dealt = wide && splits >= 8 ? 4 * waves : 0;
-        if (const char *e = getenv("ND4J_AMD_TUNE_MAPDEALT")) { if (mappedVec) dealt = atoi(e); }
         unsigned long long *slots = oneLaunch ? ws.slots : nullptr;
         const unsigned slotTicket = oneLaunch ? ws.nextSlotTicket() : 0u;
         if (mappedVec)
