@@ -20,6 +20,13 @@ template <typename T> struct BroadcastBody {
                 const Long n = pl.numTads * pl.tadLength;
                 ND4J_LAUNCH((bcFlatAnyKernel<T, F>), dim3(gridFor(n / Pack<T>::N + 1, kBlock, F::tables ? kGridCap : kMaxGrid)),
                                    dim3(kBlock), 0, s, x, y, z, n, pl.tadLength, Params<T>{nullptr});
+            } else if (pl.wholeRun >= (unsigned)Pack<T>::N && runUnits<T>(1, pl.wholeN, pl.wholeRun) <= kMaxRunUnits) {
+                // contiguous TADs with gaps whose places follow from x's own strides: the call is an element-wise walk over x,
+                // y repeating along the dimensions that are not the TAD's; no offset tables (add a row to [65536, 1024] with
+                // a pitch of 1032: 69.5 % of the HBM peak with two units per thread, 62 % with one or four, 66.5 % through
+                // bcRowKernel; TADs over several dimensions are better off with their tables: 71 % against 64 %)
+                launchRuns<T, F, false, 2>(s, x, pl.wx, y, pl.wy, z, pl.wz, nullptr, nullptr, Params<T>{nullptr}, 1, pl.wholeN,
+                                           pl.wholeRun, false);
             } else if (pl.kind == BroadcastPlan::ROW) {
                 constexpr int VEC = Pack<T>::N;
                 Long vecsPerTad = (pl.tadLength + VEC - 1) / VEC;

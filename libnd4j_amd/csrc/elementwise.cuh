@@ -664,7 +664,7 @@ template <typename T> inline Long runUnits(Long numTads, Long tadLength, unsigne
 }
 // grid and divisors of ewRunsKernel; OFFSETS: the call carries per-TAD offset tables (a compile-time choice, so that each
 // family builds only the form it launches)
-template <typename T, typename F, bool OFFSETS>
+template <typename T, typename F, bool OFFSETS, int UNITS = 0>
 inline void launchRuns(hipStream_t s, const T *x, const DimMap &xm, const T *y, const DimMap &ym, T *z, const DimMap &zm,
                        const Long *xOffsets, const Long *zOffsets, Params<T> p, Long numTads, Long tadLength, unsigned runLength,
                        bool runMajor) {
@@ -676,10 +676,11 @@ inline void launchRuns(hipStream_t s, const T *x, const DimMap &xm, const T *y, 
     // with offset tables: two units per thread and round (one: 54-63 % of the HBM peak on a [256,1024,256] array broadcast
     // along dimensions {0,2}, two: 68 %, four: 60 %), and so for functors with lookup tables, whose capped grid gives a
     // thread several rounds (exp over rows with a pitch: 56 -> 62 %); otherwise one unit per thread
-    const unsigned grid = gridFor(units, (OFFSETS || F::tables) ? kBlock * 2 : kBlock, F::tables ? kGridCap : kMaxGrid);
+    constexpr int U = UNITS > 0 ? UNITS : ((OFFSETS || F::tables) ? 2 : 1);
+    const unsigned grid = gridFor(units, kBlock * U, F::tables ? kGridCap : kMaxGrid);
     const unsigned long long step = (unsigned long long)grid * kBlock;  // at most 2^32 - 256
     const unsigned unitStep = (unsigned)(step % unitsPerRun), runStep = (unsigned)(step / unitsPerRun);
-    ND4J_LAUNCH((ewRunsKernel<T, F, (OFFSETS || F::tables) ? 2 : 1>), dim3(grid), dim3(kBlock), 0, s, x, xm, y, ym, z, zm, xOffsets, zOffsets, p,
+    ND4J_LAUNCH((ewRunsKernel<T, F, U>), dim3(grid), dim3(kBlock), 0, s, x, xm, y, ym, z, zm, xOffsets, zOffsets, p,
                        (unsigned)units, runLength, runMajor ? 1 : 0, perRun, second, unitStep, runStep);
 }
 

@@ -47,6 +47,12 @@ struct BroadcastPlan {
                                  // either takes y[(i / tadEws) % tadLength]
     unsigned runLength = 0;      // GENERAL only, 0 = not applicable: the three maps end in contiguous runs of this many elements
     bool runMajor = false;       //   ... and the same run of neighbouring TADs is nearer in memory than the next run of one TAD
+    // The whole call as one element-wise walk, when the host could state it so (wholeRun > 0): maps over all of x's
+    // dimensions - y's with stride 0 along those that are not the TAD's - that end in contiguous runs of wholeRun elements;
+    // wholeN elements in all.  Needs no offset tables.
+    DimMap wx, wy, wz;
+    Long wholeN = 0;
+    unsigned wholeRun = 0;
     Long flatInner = 0, flatExtent = 0;  // per-TAD scalars over dense x and z of one layout: memory position i takes
                                          // scalars[(i / flatInner) % flatExtent]; 0 = not applicable
 };

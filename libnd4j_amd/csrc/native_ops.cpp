@@ -267,6 +267,48 @@ void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Lon
             pl.runMajor = tx.numTads > 1 && (next >= 2 * (Long)run || next < 0);
         }
     }
+    // Contiguous TADs that the flat kernels do not take (gaps between them): their places follow from x's own
+    // strides, so the call can be stated as one element-wise walk over x's shape in which y repeats along the dimensions
+    // that are not the TAD's.  The reference pairs element f of every TAD, f counting in the TAD's order, with element f of
+    // y; that is y[f * stride] here whenever y's own walk came out as one run (yLinear), and f counts in C order over the
+    // TAD's dimensions when the TAD's order is 'c' (or it has one dimension).  The TAD's dimensions are found in x's by
+    // extent and stride, in order (extents of 1 take no part); the result must be laid out over the same shape.
+    const Long yLinear = pl.kind == BroadcastPlan::GENERAL ? (pl.ym.rank == 1 ? pl.ym.stride[0] : 0) : pl.yEws;
+    if (!pl.consecutive && !pl.denseAlike && pl.kind == BroadcastPlan::ROW && yLinear > 0 &&
+        (siOrder(tx.hostInfo) == 'c' || dimLen == 1) && sameShape(hx, hz) && siNumel(hy) >= tx.tadLength &&
+        siNumel(hx) <= 0x7fffffffLL && siRank(hx) <= kMaxDims) {
+        const int rank = siRank(hx), tadRank = siRank(tx.hostInfo);
+        const Long *xs = siShape(hx), *xst = siStride(hx), *zst = siStride(hz);
+        const Long *ts = siShape(tx.hostInfo), *tst = siStride(tx.hostInfo);
+        Long ystr[kMaxDims];
+        bool inTad[kMaxDims];
+        int k = 0;
+        while (k < tadRank && ts[k] == 1) k++;
+        for (int d = 0; d < rank; d++) {
+            inTad[d] = xs[d] != 1 && k < tadRank && xs[d] == ts[k] && xst[d] == tst[k];
+            if (inTad[d]) {
+                k++;
+                while (k < tadRank && ts[k] == 1) k++;
+            }
+        }
+        if (k == tadRank) {
+            Long inner = yLinear;
+            for (int d = rank - 1; d >= 0; d--) {
+                ystr[d] = inTad[d] ? inner : 0;
+                if (inTad[d]) inner *= xs[d];
+            }
+            const Long *strides[3] = {xst, ystr, zst};
+            DimMap maps[3];
+            jointCanon(rank, xs, strides, maps);
+            const DimMap *const all[3] = {&maps[0], &maps[1], &maps[2]};
+            const unsigned run = commonRunLength(all);
+            if (run >= 2) {
+                pl.wx = maps[0]; pl.wy = maps[1]; pl.wz = maps[2];
+                pl.wholeN = siNumel(hx);
+                pl.wholeRun = run;
+            }
+        }
+    }
     if (!launchBroadcast<T>(s, opNum, x, y, z, pl)) { reportUnknownOp("broadcast", opNum); return; }
     checkLaunch("execBroadcast", s);
 }
