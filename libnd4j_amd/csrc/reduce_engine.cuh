@@ -358,7 +358,10 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
     constexpr int WAVES = BLK / kWave;
     constexpr int W = SlotWords<Pol>::value;
     constexpr int TILE = VEC * kWave;  // TADs of a column tile
-    __shared__ Acc smem[(WAVES - 1) * kWave];
+    // (accumulators of 16 bytes or more - index pairs, moments - are merged by halving the waves, all owned TADs at once:
+    // three rounds of combines side by side instead of seven on the first wave for each owned TAD in turn)
+    constexpr bool TREE = sizeof(Acc) >= 16 && WAVES >= 4 && (WAVES & (WAVES - 1)) == 0;
+    __shared__ Acc smem[TREE ? (WAVES / 2) * kWave * VEC : (WAVES - 1) * kWave];
     __shared__ int mergeHere;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const Long t0 = ((Long)blockIdx.x * kWave + lane) * VEC;
@@ -445,16 +448,35 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
             }
         }
     }
+    if constexpr (TREE) {
+        for (int half = WAVES / 2; half >= 1; half >>= 1) {
+            __syncthreads();
+            if (wave >= half && wave < 2 * half) {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) smem[((wave - half) * VEC + e) * kWave + lane] = acc[e];
+            }
+            __syncthreads();
+            if (wave < half && live) {
+#pragma unroll
+                for (int e = 0; e < VEC; e++)
+                    if (t0 + e < numTads) acc[e] = pe[e].combine(acc[e], smem[(wave * VEC + e) * kWave + lane]);
+            }
+        }
+    }
     // merge the waves, one owned TAD at a time (keeps the LDS footprint at one accumulator per lane of the other waves)
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
-        __syncthreads();
-        if (wave > 0) smem[(wave - 1) * kWave + lane] = acc[e];
-        __syncthreads();
+        if constexpr (!TREE) {
+            __syncthreads();
+            if (wave > 0) smem[(wave - 1) * kWave + lane] = acc[e];
+            __syncthreads();
+        }
         if (wave == 0 && live && t0 + e < numTads) {
             Acc a = acc[e];
+            if constexpr (!TREE) {
 #pragma unroll
-            for (int w = 0; w < WAVES - 1; w++) a = pe[e].combine(a, smem[w * kWave + lane]);
+                for (int w = 0; w < WAVES - 1; w++) a = pe[e].combine(a, smem[w * kWave + lane]);
+            }
             if (gridDim.y == 1) z[t0 + e] = pe[e].finalize(a, tadLength);
             else if (slots != nullptr)
                 publishSlots<Acc, W>(slots + (((size_t)blockIdx.x * gridDim.y + blockIdx.y) * TILE + e * kWave + lane) * W, a, slotTicket);
@@ -462,6 +484,7 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
         }
     }
     if (gridDim.y == 1 || slots == nullptr) return;
+    if constexpr (W <= 2) {  // (the host asks for this form only with accumulators of one or two words)
     // One launch: the row ranges of a column tile count themselves in on the tile's counter once their slots are on the
     // way, and the block that comes last merges the tile - a thread per TAD, the ranges in order, 16 slot groups in
     // flight - and writes its results.  (Tiles finish at different times: only the last one's merge is not hidden.)
@@ -478,7 +501,7 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
     // PARTS threads share a TAD when the block has more threads than the tile has TADs: each takes every PARTS-th batch of
     // G row ranges, the first of them merges what the others hand over through LDS
     constexpr int PARTS = BLK > TILE ? BLK / TILE : 1;
-    static_assert(PARTS == 1 || (PARTS - 1) * TILE <= (WAVES - 1) * kWave, "the hand-over reuses the waves' merge area");
+    static_assert(PARTS == 1 || (!TREE && (PARTS - 1) * TILE <= (WAVES - 1) * kWave), "the hand-over reuses the waves' merge area");
     const int splits = (int)gridDim.y;
     __syncthreads();  // (the waves' merge area is free from here on)
     for (int k0 = 0; k0 < TILE * PARTS; k0 += BLK) {
@@ -532,6 +555,7 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
             if (missing && fault != nullptr) __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             z[t] = missing ? notANumber<T>() : pm.finalize(a, tadLength);
         }
+    }
     }
 }
 
