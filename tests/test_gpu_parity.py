@@ -314,6 +314,31 @@ def test_tads_over_several_dimensions(gpu, cpu):
         assert np.array_equal(g, c), dt
 
 
+def test_strided_reductions_with_many_row_ranges(gpu, cpu):
+    """Reductions along dimension 0 of c-order matrices tall enough for the strided vector kernel to cut every column tile
+    into eight row ranges or more (rows dealt to the ranges a batch at a time, a last batch that is short, a last tile
+    that is not full): sums and maxima finish in one launch (the tile's last block merges the ranges), index pairs and
+    moments in two; all three storage types, ties included."""
+    rs = np.random.RandomState(57)
+    for dt, shape in ((np.float32, [3001, 1100]), (np.float32, [4096, 512]), (np.float64, [2050, 530]), (np.float16, [2300, 1032])):
+        rows, cols = shape
+        xi = shape_info_np(shape)
+        x = (rs.randint(-8, 9, rows * cols) / 4.0).astype(dt)  # many ties; sums of quarters are exact in every type's accumulator
+        x64 = x.astype(np.float64).reshape(shape)
+        what = "%s %s" % (np.dtype(dt).name, shape)
+        for k in range(2):  # (the second call meets the slots the first one left behind)
+            got = gpu.reduce(1, x, xi, None, [0], cols).astype(np.float64)
+            want = x64.sum(axis=0)
+            tol = 1e-2 * np.abs(x64).sum(axis=0) if dt == np.float16 else 0.0
+            assert np.all(np.abs(got - want) <= tol), what
+            assert np.array_equal(gpu.reduce(3, x, xi, None, [0], cols), cpu.reduce(3, x, xi, None, [0], cols)), what
+            for op in (0, 1):
+                assert np.array_equal(gpu.indexreduce(op, x, xi, None, [0], cols), cpu.indexreduce(op, x, xi, None, [0], cols)), what
+        var = gpu.summarystats(0, 1, x, xi, [0], cols).astype(np.float64)
+        truth = x64.var(axis=0, ddof=1)
+        assert np.all(np.abs(var - truth) <= (1e-2 if dt == np.float16 else 1e-5) * np.maximum(truth, 1e-30)), what
+
+
 def test_broadcast_on_views_all_ops(gpu, cpu):
     rs = np.random.RandomState(27)
     for shape, order, dims in (([17, 33], "c", [1]), ([17, 33], "c", [0]), ([17, 33], "f", [0]), ([17, 33], "f", [1]),
