@@ -1326,6 +1326,11 @@ def test_random_views_against_the_cpu_checker(gpu, cpu):
     without the caller's TAD tables.  Fixed seed: the same few thousand calls every run."""
     done = checks.check_random_views(gpu, cpu, seed=7, cases=4000)
     assert len(done) == 8 and min(done.values()) > 200
+    # the other two storage types: vectors of two and of eight elements through the same kernels
+    done = checks.check_random_views(gpu, cpu, seed=8, cases=1200, dtype=np.float64)
+    assert len(done) == 8 and min(done.values()) > 50
+    done = checks.check_random_views(gpu, cpu, seed=9, cases=1200, dtype=np.float16)
+    assert len(done) == 5 and min(done.values()) > 50
 
 
 def test_dense_matrices_in_mixed_orders(gpu):
