@@ -963,7 +963,8 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         // launch costs is small: sums along dimension 0 of [16384, 4096] take 45.6 us either way, maxima along dimension 1
         // of an f-order [32768, 2048] 41.9 in one launch and 42.5 in two.  Accumulators of more words - index pairs, the
         // statistics' moments - would have a tile's last block collect hundreds of words per thread: they keep the second
-        // launch, which spreads that over the chip.)
+        // launch, which spreads that over the chip - measured: index of the maximum 45.8 us in two launches, 46.7 in one;
+        // variance, with its moments cut down to the seven words of an open run, 47.3 against 49.8.)
         constexpr int W = SlotWords<Pol>::value;
         const bool oneLaunch = splits > 1 && W <= 2 && ws.slots != nullptr && ws.counter != nullptr && ws.slotTicketSource != nullptr &&
                                gx <= 128 && (size_t)gx * (size_t)splits * kWave * VEC * W * sizeof(unsigned long long) <= ws.slotBytes;
