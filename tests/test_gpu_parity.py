@@ -1185,6 +1185,64 @@ def test_slot_tickets_across_the_points_where_the_slots_are_cleared(gpu):
         gpu.ops.amd_setSlotTicket(ex, 5)
 
 
+def test_elementwise_calls_in_a_captured_graph(gpu):
+    """A pairwise add, an exp transform and a row broadcast are captured into a HIP graph on the caller's stream (after one
+    eager pass, which lets the stream allocate what it keeps) and replayed three times with new operand values, eager
+    work and synchronisations in between; every replay must give the bits of the same three calls made eagerly."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    dev, ops = gpu.dev, gpu.dev.ops
+    rs = np.random.RandomState(91)
+    rows, cols = 300, 1024
+    n = rows * cols
+    xi, bi = shape_info_np([rows, cols]), shape_info_np([1, cols])
+    tad = dev.tad(xi, [1])
+    X = harness.Operand(dev, rs.uniform(-2, 2, n).astype(np.float32), xi)
+    Y = harness.Operand(dev, rs.uniform(-2, 2, n).astype(np.float32), xi)
+    B = harness.Operand(dev, rs.uniform(-2, 2, cols).astype(np.float32), bi)
+    outs = [[harness.Operand(dev, np.zeros(n, np.float32), xi) for _ in range(3)] for _ in range(2)]  # graph, eager
+    dim = dev.upload(np.array([1], np.int32))
+    ex = dev.extra(xi, xi, xi)
+    exb = dev.extra(xi, bi, xi, tad=tad, tad_z=tad)
+
+    def calls(o):
+        ops.execPairwiseTransformFloat(ex, 0, X.ptr, X.info_ptr, Y.ptr, Y.info_ptr, o[0].ptr, o[0].info_ptr, None)
+        ops.execTransformFloat(ex, 3, o[0].ptr, o[0].info_ptr, o[1].ptr, o[1].info_ptr, None)
+        ops.execBroadcastFloat(exb, 0, o[1].ptr, o[1].info_ptr, B.ptr, B.info_ptr, o[2].ptr, o[2].info_ptr, dim.ptr, 1)
+
+    calls(outs[1])
+    dev.sync()
+    stream = ctypes.c_void_p(dev.stream)
+    graph, executable = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 1) == 0  # 1: thread-local capture mode
+    try:
+        calls(outs[0])
+    finally:
+        status = hip.hipStreamEndCapture(stream, ctypes.byref(graph))
+    assert status == 0 and graph.value
+    assert hip.hipGraphInstantiate(ctypes.byref(executable), graph, None, None, ctypes.c_size_t(0)) == 0
+    try:
+        for replay in range(3):
+            fresh = rs.uniform(-2, 2, n).astype(np.float32)
+            ops.memcpy(X.ptr, fresh.ctypes.data, fresh.nbytes, 1, None)
+            dev.sync()
+            assert hip.hipGraphLaunch(executable, stream) == 0
+            dev.sync()
+            calls(outs[1])
+            dev.sync()
+            e = np.exp((fresh + Y.get()).astype(np.float64)).reshape(rows, cols)
+            b = B.get().astype(np.float64)
+            for k in range(3):
+                assert np.array_equal(outs[0][k].get(), outs[1][k].get()), (replay, k)
+            assert np.all(np.abs(outs[0][2].get().reshape(rows, cols) - (e + b)) <= 1e-5 * (e + np.abs(b))), replay
+    finally:
+        hip.hipGraphExecDestroy(executable)
+        hip.hipGraphDestroy(graph)
+        for o in [X, Y, B] + outs[0] + outs[1]:
+            o.free()
+        dim.free()
+
+
 def test_releasing_a_streams_resources(gpu):
     """A stream's workspace, exchange slots and pinned scalar block are freed on request and come back at the next call."""
     rs = np.random.RandomState(43)
