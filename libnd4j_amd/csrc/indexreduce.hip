@@ -24,7 +24,6 @@ template <typename TT, int OP> struct IndexPol {
     static constexpr int kChains = 4;      // accumulators of one lane may be kept apart and combined (ties go to the lower index)
     static constexpr int kSlotWords = 2 + sizeof(C) / 4;  // index and value; the float accumulator's padding word stays behind
     static constexpr int kFlatBlocks = 768;   // blocks of the whole-array kernel: three per compute unit (see runFlatReduce)
-    static constexpr bool kClears = OP == 0;  // IsMax over a whole array looks for the maximum and clears the result in one pass
     Params<TT> p;
 
     __device__ __forceinline__ void setTad(Long, const TT *) {}
@@ -117,17 +116,7 @@ bool launchIndexReduceScalar(hipStream_t s, int opNum, const T *x, const T *extr
                                                        extra, z, plan, ws);
 }
 
-// IndexMax over a dense x that also overwrites `cleared` (laid out like x, the same offset from a 16-byte boundary; x
-// itself or an array apart from it) with zeros: the first of IsMax's two steps
-template <typename T>
-void launchIndexMaxClearing(hipStream_t s, const T *x, T *z, const FlatPlan &plan, Workspace ws, T *cleared) {
-    IndexPol<T, 0> pol;
-    pol.p.p = nullptr;
-    runFlatReduce(s, pol, x, z, plan, ws, cleared);
-}
-
 #define INST(T)                                                                                                       \
-    template void launchIndexMaxClearing<T>(hipStream_t, const T *, T *, const FlatPlan &, Workspace, T *);           \
     template bool launchIndexReduceTad<T>(hipStream_t, int, const T *, const T *, T *, const TadPlan &, Workspace);   \
     template bool launchIndexReduceScalar<T>(hipStream_t, int, const T *, const T *, T *, const FlatPlan &, Workspace);
 INST(float)

@@ -198,12 +198,6 @@ bool launchSoftmaxFinish(hipStream_t stream, int opNum, const T *x, T *z, const 
 // z = one-hot of the position stored (as a T) in index[0] / index[tad]; `zp` / `zt` walk z the way the index
 // reduction walked x
 template <typename T> void launchIsMaxFill(hipStream_t stream, T *z, const T *index, const FlatPlan &zp);
-// IsMax over a whole dense array in one pass: launchIndexMaxClearing finds the maximum's index (into `index`, as the
-// index reductions store it) while it clears `cleared`; launchIsMaxMark then sets the one element.  x and `cleared` are
-// dense, n elements each, on the same offset from a 16-byte boundary, and the same array or two that do not overlap.
-template <typename T>
-void launchIndexMaxClearing(hipStream_t stream, const T *x, T *index, const FlatPlan &plan, Workspace ws, T *cleared);
-template <typename T> void launchIsMaxMark(hipStream_t stream, T *z, const T *index, Long n);
 template <typename T> void launchIsMaxTadFill(hipStream_t stream, T *z, const T *index, const TadPlan &zt);
 
 // ---- whole-array transforms (Col2Im 36, Im2col 37, Histogram 48, Reverse 70, Pooling2D 71) ---------------------

@@ -503,14 +503,6 @@ namespace nd4j_amd {
 
 // IsMax over a whole array, both operands dense with the same number of elements, on the same offset from a 16-byte
 // boundary, and either the same array or two that do not overlap: the index reduction clears z while it reads x.
-template <typename T> bool isMaxInOnePass(const T *x, const FlatPlan &xp, const T *z, const FlatPlan &zp) {
-    if (!xp.strided || xp.ews != 1 || !zp.strided || zp.ews != 1 || xp.n != zp.n || xp.n <= 0) return false;
-    const uintptr_t xa = reinterpret_cast<uintptr_t>(x), za = reinterpret_cast<uintptr_t>(z);
-    if ((xa & 15) != (za & 15)) return false;
-    const uintptr_t bytes = (uintptr_t)xp.n * sizeof(T);
-    return xa == za || xa + bytes <= za || za + bytes <= xa;
-}
-
 template <typename T>
 bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z, const Long *hz, T *params, hipStream_t s) {
     if (opNum < 38 || opNum > 41) return false;
@@ -603,13 +595,10 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
         T *slot = reinterpret_cast<T *>(sc.scalars);
         FlatPlan xp = flatIndexed(hx);
         FlatPlan zp = flatIndexed(hz);
-        if (isMaxInOnePass<T>(x, xp, z, zp)) {
-            launchIndexMaxClearing<T>(s, x, slot, xp, sc.rest, z);
-            launchIsMaxMark<T>(s, z, slot, zp.n);
-        } else {
-            if (!launchIndexReduceScalar<T>(s, 0, x, nullptr, slot, xp, sc.rest)) return false;
-            launchIsMaxFill<T>(s, z, slot, zp);
-        }
+        // (two passes - the index of the maximum, then a fill - take 83 us over 2^26 floats; one pass that cleared the
+        // result while it looked for the maximum, and set the one element afterwards, took 96)
+        if (!launchIndexReduceScalar<T>(s, 0, x, nullptr, slot, xp, sc.rest)) return false;
+        launchIsMaxFill<T>(s, z, slot, zp);
         checkLaunch("execTransform(IsMax)", s);
         return true;
     }
@@ -629,20 +618,16 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
     rest.ptr = reinterpret_cast<char *>(rest.ptr) + used;
     rest.bytes -= used;
     TadPlan xp = tadPlanFrom(tx);
-    bool onePass = false;
     if (tx.numTads == 1) {
-        FlatPlan fp = flatIndexed(hx), fz = flatIndexed(hz);
-        onePass = isMaxInOnePass<T>(x, fp, z, fz);
-        if (onePass) launchIndexMaxClearing<T>(s, x, index, fp, rest, z);
-        else if (!launchIndexReduceScalar<T>(s, 0, x, nullptr, index, fp, rest)) return false;
+        FlatPlan fp = flatIndexed(hx);
+        if (!launchIndexReduceScalar<T>(s, 0, x, nullptr, index, fp, rest)) return false;
     } else if (!launchIndexReduceTad<T>(s, 0, x, nullptr, index, xp, rest)) {
         return false;
     }
     TadPlan zp = tadPlanFrom(tz);
     if (tx.numTads == 1) {
         FlatPlan fz = flatIndexed(hz);
-        if (onePass) launchIsMaxMark<T>(s, z, index, fz.n);
-        else launchIsMaxFill<T>(s, z, index, fz);
+        launchIsMaxFill<T>(s, z, index, fz);
     } else {
         launchIsMaxTadFill<T>(s, z, index, zp);
     }

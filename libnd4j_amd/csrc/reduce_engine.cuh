@@ -61,9 +61,6 @@ template <class Pol> struct PolFlatBlocks<Pol, decltype((void)Pol::kFlatBlocks)>
 template <class Pol, typename = void> struct PolColBlocks { static constexpr int value = 2048; };
 template <class Pol> struct PolColBlocks<Pol, decltype((void)Pol::kColBlocks)> { static constexpr int value = Pol::kColBlocks; };
 
-// Whether the clearing form of the whole-array kernel is built for a policy (a member constant kClears).
-template <class Pol, typename = void> struct PolClears { static constexpr bool value = false; };
-template <class Pol> struct PolClears<Pol, decltype((void)Pol::kClears)> { static constexpr bool value = Pol::kClears; };
 
 // Folds an element whose index is higher than that of every element the accumulator has seen (the kernels walk their
 // elements in ascending order wherever they can).  A policy may exploit that with a member accumulateAscending(): an
@@ -749,15 +746,11 @@ __global__ void __launch_bounds__(kBlock) tadGeneralKernel(Pol pol, const typena
 // every other block issue its stores, waits for them to land, merges all groups in block order and writes the result
 // (the counters are back at zero by then): one launch.  Without `slots` the accumulators go to `partials` and flatFinish
 // merges them in a second launch.
-// CLEAR (dense x only): every element that has been read is overwritten with zero in `cleared`, an array laid out like x
-// and on the same offset from a 16-byte boundary (x itself, or one that does not overlap it): each thread clears exactly
-// the elements it has loaded itself, so clearing in place is safe.
-template <class Pol, bool CLEAR = false>
+template <class Pol>
 __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol::T *x, typename Pol::Acc *partials,
                                                      Long n, int strided, Long ews, DimMap xm, typename Pol::T *z,
                                                      unsigned long long *signal, unsigned ticket, unsigned long long *slots,
-                                                     unsigned *counter, unsigned slotTicket, typename Pol::T *cleared = nullptr,
-                                                     unsigned *fault = nullptr) {
+                                                     unsigned *counter, unsigned slotTicket, unsigned *fault = nullptr) {
     if (Pol::tables) lm::loadTables();
     typedef typename Pol::T T;
     typedef typename Pol::Acc Acc;
@@ -803,16 +796,6 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
                     pol.checkpoint(to);
                 }
             }
-            if (CLEAR) {
-                Pack<T> zeros;
-#pragma unroll
-                for (int e = 0; e < VEC; e++) zeros.v[e] = fromCompute<T>((typename Pol::C)0);
-#pragma unroll
-                for (int u = 0; u < kUnroll; u++) {
-                    Long v = b + u * kBlock + threadIdx.x;
-                    if (v < nvec) storePack(reinterpret_cast<Pack<T> *>(cleared + head) + v, zeros);
-                }
-            }
         }
         if (CH > 1) {
 #pragma unroll
@@ -822,12 +805,10 @@ __global__ void __launch_bounds__(kBlock) flatKernel(Pol pol, const typename Pol
             for (Long i = threadIdx.x; i < head; i += kBlock) {
                 pol.accumulate(acc, toCompute(x[i]), i);
                 pol.checkpoint(acc);
-                if (CLEAR) cleared[i] = fromCompute<T>((typename Pol::C)0);
             }
             for (Long i = head + nvec * VEC + threadIdx.x; i < n; i += kBlock) {
                 pol.accumulate(acc, toCompute(x[i]), i);
                 pol.checkpoint(acc);
-                if (CLEAR) cleared[i] = fromCompute<T>((typename Pol::C)0);
             }
         }
     } else if (strided) {
@@ -1056,10 +1037,9 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
                        pl.numTads);
 }
 
-// `cleared` (optional; only for a dense x, see flatKernel): an array like x that is overwritten with zeros on the way
 template <class Pol>
 inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typename Pol::T *z, const FlatPlan &pl,
-                          Workspace ws, typename Pol::T *cleared = nullptr) {
+                          Workspace ws) {
     typedef typename Pol::Acc Acc;
     typedef typename Pol::T T;
     Long perBlock = (Long)kBlock * kUnroll * Pack<T>::N;
@@ -1073,16 +1053,9 @@ inline void runFlatReduce(hipStream_t s, Pol pol, const typename Pol::T *x, type
     if ((size_t)grid > maxBlocks) grid = (int)maxBlocks;
     if (grid < 1) grid = 1;
     Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
-    if (cleared != nullptr) {
-        if constexpr (PolClears<Pol>::value)
-            ND4J_LAUNCH((flatKernel<Pol, true>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, 1, (Long)1, pl.xm, z,
-                               ws.signal, ws.ticket, oneLaunch ? ws.slots : nullptr, ws.counter,
-                               oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u, cleared, ws.fault);
-    } else {
-        ND4J_LAUNCH((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
-                           pl.ews, pl.xm, z, ws.signal, ws.ticket, oneLaunch ? ws.slots : nullptr, ws.counter,
-                           oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u, (typename Pol::T *)nullptr, ws.fault);
-    }
+    ND4J_LAUNCH((flatKernel<Pol>), dim3(grid), dim3(kBlock), 0, s, pol, x, partials, pl.n, pl.strided ? 1 : 0,
+                       pl.ews, pl.xm, z, ws.signal, ws.ticket, oneLaunch ? ws.slots : nullptr, ws.counter,
+                       oneLaunch && grid > 1 ? ws.nextSlotTicket() : 0u, ws.fault);
     if (grid > 1 && !oneLaunch)
         ND4J_LAUNCH((flatFinish<Pol>), dim3(1), dim3(kBlock), 0, s, pol, x, z, partials, grid, pl.n, ws.signal, ws.ticket);
 }
