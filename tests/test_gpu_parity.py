@@ -813,6 +813,15 @@ def test_whole_array_transforms_usual_windows(gpu, cpu):
             assert np.array_equal(g, c), ("im2col", dt, kH, kW)
             e_col = np.array([1, 1, pad, pad, iH, iW, 1, 1], dt)
             assert np.array_equal(gpu.transform(36, g, ci, ii, e_col), cpu.transform(36, c, ci, ii, e_col)), ("col2im", dt, kH, kW)
+        # planes large enough for a channel's vectors to be spread over several blocks (two, and three)
+        for (iH, iW, kH, kW, pad) in ((40, 44, 3, 3, 1), (56, 56, 3, 3, 1)):
+            bS, iC = 8, 128
+            oH, oW = iH + 2 * pad - kH + 1, iW + 2 * pad - kW + 1
+            img, col = [bS, iC, iH, iW], [bS, iC, kH, kW, oH, oW]
+            ii, ci = shape_info_np(img), shape_info_np(col)
+            x = rs.randint(-8, 9, int(np.prod(img))).astype(dt)
+            e_im = np.array([kH, kW, 1, 1, pad, pad, 1, 1, 0, 0], dt)
+            assert np.array_equal(gpu.transform(37, x, ii, ci, e_im), cpu.transform(37, x, ii, ci, e_im)), ("im2col", dt, iH, iW)
         for iH, iW in ((56, 56), (9, 57), (10, 54), (7, 7)):
             img, pooled = [3, 5, iH, iW], [3, 5, iH // 2, iW // 2]
             ii, pi = shape_info_np(img), shape_info_np(pooled)
