@@ -94,8 +94,11 @@ __device__ __forceinline__ void copyRun(const T *src, Long se, const Long *sInfo
 
 // A block works on one long TAD, on four shorter ones (a wave each) or on sixteen short ones, sized so that a lane
 // keeps about four 16-byte vectors in flight
-template <typename T> __device__ __forceinline__ int lanesPerTad(Long tadLength) {
+template <typename T> __device__ __forceinline__ int lanesPerTad(Long tadLength, bool wide = false) {
     const Long vectors = tadLength / Pack<T>::N;
+    // (wide: a vector per lane from 256 vectors on - rows of 1024 floats torn into buffers of their own: 88 -> 85 us;
+    // the same rows gathered or swapped in place: 95 -> 127 us, so those keep a wave per row)
+    if (wide) return vectors >= 256 ? kBlock : (vectors >= 64 ? kWave : 16);
     return vectors >= 1024 ? kBlock : (vectors >= 256 ? kWave : 16);
 }
 
@@ -129,7 +132,7 @@ __global__ void __launch_bounds__(kBlock) tearKernel(const T *x, const Long *xIn
     const Long tadLength = dLength(tadInfo);
     const Long numTads = dLength(xInfo) / tadLength;
     const Long xe = dEws(tadInfo), ze = dEws(zInfo);
-    const int lanes = lanesPerTad<T>(tadLength), groups = kBlock / lanes;
+    const int lanes = lanesPerTad<T>(tadLength, true), groups = kBlock / lanes;
     const int g = threadIdx.x / lanes, lane = threadIdx.x % lanes;
     if (lanes == kBlock && xe == 1 && ze == 1) {
         // long contiguous TADs are cut into pieces of four vectors per lane, so that a few long TADs still fill the chip
