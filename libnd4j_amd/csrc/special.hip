@@ -993,7 +993,8 @@ template <typename T, int MODE> void runSoftmax(hipStream_t s, const T *x, T *z,
         const Long npack = pl.length / N;  // at most this many aligned vectors in a row (fewer when it starts off a boundary)
         if (npack <= 16 * 2) runRowReg<T, MODE, 16, 2>(s, x, z, pl);
         else if (npack <= 64 * 2) runRowReg<T, MODE, 64, 2>(s, x, z, pl);
-        else if (npack <= 64 * 8) runRowReg<T, MODE, 64, 8>(s, x, z, pl);
+        // (a wave per row up to 256 vectors, a block per row beyond: rows of 2048 floats 88 -> 86 us, log-softmax 90 -> 86)
+        else if (npack <= 64 * 4) runRowReg<T, MODE, 64, 8>(s, x, z, pl);
         else if (npack <= 256 * 4) runRowReg<T, MODE, kBlock, 4>(s, x, z, pl);
         else if (npack <= 256 * 8) runRowReg<T, MODE, kBlock, 8>(s, x, z, pl);
         else if (npack <= 256 * 16) runRowReg<T, MODE, kBlock, 16>(s, x, z, pl);
