@@ -926,10 +926,13 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
         // Measured on [16384, 4096] along dimension 0 (16 column tiles) and on an f-order [32768, 2048] along dimension 1
         // (128 tiles), in us: sums 42.9 / 41.8, index of the maximum 46.0, variance - / 48.6; with 256 threads and 512
         // (sums), 2048 (index) or 1024 (statistics) blocks 45.6 / 44.0, 49.3 and 49.1; 512 or 1024 blocks of 512 threads
-        // are slower for all of them.  Mapped TADs keep 256 threads and the policy's kColBlocks.
+        // are slower for all of them.  Mapped TADs keep 256 threads and the policy's kColBlocks (1024 at least).
         const bool wide = !mappedVec;
         const int waves = wide ? 8 : kBlock / kWave;
-        Long splits = (wide ? 256 : PolColBlocks<Pol>::value) / gx;
+        // (mapped TADs: at least 1024 blocks - sums over dimensions {0,2} of [128,128,56,56] 45.2 us with 512, 43.2 with 1024,
+        // 46.9 with 2048, 66 with 256)
+        constexpr int kMappedBlocks = PolColBlocks<Pol>::value < 1024 ? 1024 : PolColBlocks<Pol>::value;
+        Long splits = (wide ? 256 : kMappedBlocks) / gx;
         if (splits < 1) splits = 1;
         Long maxSplitsByRows = (pl.tadLength + 16 * waves - 1) / (16 * waves);  // at least 16 rows per wave
         if (splits > maxSplitsByRows) splits = maxSplitsByRows;
