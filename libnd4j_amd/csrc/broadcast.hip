@@ -12,7 +12,10 @@ template <typename T> struct BroadcastBody {
             if (pl.kind == BroadcastPlan::ROW && pl.consecutive && pl.tadLength % Pack<T>::N == 0 &&
                 pl.tadLength / Pack<T>::N < 0xffffffffLL && (((uintptr_t)x | (uintptr_t)y | (uintptr_t)z) & 15) == 0) {
                 const Long nvec = pl.numTads * (pl.tadLength / Pack<T>::N);
-                ND4J_LAUNCH((bcFlatKernel<T, F>), dim3(gridFor(nvec, kBlock * 2, F::tables ? kGridCap : kMaxGrid)), dim3(kBlock), 0,
+                // (blocks of 128 threads, as for two-operand element-wise calls: a row added to [65536, 1024] floats 85.7 -> 83 us;
+                // the functors with lookup tables keep the 256 threads their staging is written for)
+                const int blk = F::tables ? kBlock : kBlock / 2;
+                ND4J_LAUNCH((bcFlatKernel<T, F>), dim3(gridFor(nvec, blk * 2, F::tables ? kGridCap : kMaxGrid)), dim3(blk), 0,
                                    s, x, y, z, nvec, (unsigned)(pl.tadLength / Pack<T>::N), Params<T>{nullptr});
             } else if (pl.kind == BroadcastPlan::ROW && pl.consecutive && pl.tadLength >= Pack<T>::N && pl.tadLength < 0xffffffffLL &&
                        (((uintptr_t)x | (uintptr_t)z) & 15) == 0) {

@@ -126,7 +126,8 @@ template <int KIND> struct Broadcast2F {
 // ---------------------------------------------------------------------------------------------------
 // z[i] = F(x[i], y[i or 0]) over n contiguous elements.  `head` leading elements are done one by one so
 // that the vector part starts on a 16-byte boundary (the host guarantees all operands share the same
-// misalignment); yScalar selects y[0] for every element.
+// misalignment); yScalar selects y[0] for every element.  Launched with kBlock threads or fewer (the kernel goes by
+// blockDim.x; the lookup-table staging wants all kBlock).
 template <typename T, typename F>
 __global__ void __launch_bounds__(kBlock) ewVecKernel(const T *x, const T *y, T *z, Params<T> p, Long n, int head,
                                                       int yScalar) {
@@ -144,7 +145,7 @@ __global__ void __launch_bounds__(kBlock) ewVecKernel(const T *x, const T *y, T 
     // sustain a higher HBM rate on this chip than fewer blocks with several vectors in flight per thread
     if (F::tables) {
         // the first vectors are requested before the lookup tables are staged, so the two waits overlap
-        Long j = (Long)blockIdx.x * kBlock + threadIdx.x;
+        Long j = (Long)blockIdx.x * blockDim.x + threadIdx.x;
         bool have = j < nvec;
         Pack<T> a, b;
         if (have) {
@@ -160,7 +161,7 @@ __global__ void __launch_bounds__(kBlock) ewVecKernel(const T *x, const T *y, T 
                 r.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), bv, p));
             }
             storePack(zv + j, r);
-            j += (Long)gridDim.x * kBlock;
+            j += (Long)gridDim.x * blockDim.x;
             have = j < nvec;
             if (have) {
                 a = loadPack(xv + j);
@@ -168,7 +169,7 @@ __global__ void __launch_bounds__(kBlock) ewVecKernel(const T *x, const T *y, T 
             }
         }
     } else {
-        for (Long j = (Long)blockIdx.x * kBlock + threadIdx.x; j < nvec; j += (Long)gridDim.x * kBlock) {
+        for (Long j = (Long)blockIdx.x * blockDim.x + threadIdx.x; j < nvec; j += (Long)gridDim.x * blockDim.x) {
             Pack<T> a = loadPack(xv + j), b;
             if (F::nin == 2 && !yScalar) b = loadPack(yv + j);
             Pack<T> r;
@@ -181,7 +182,7 @@ __global__ void __launch_bounds__(kBlock) ewVecKernel(const T *x, const T *y, T 
         }
     }
     // head and tail elements
-    const Long gtid = (Long)blockIdx.x * kBlock + threadIdx.x;
+    const Long gtid = (Long)blockIdx.x * blockDim.x + threadIdx.x;
     const Long tailStart = head + nvec * VEC;
     const Long nScalar = head + (n - tailStart);
     if (gtid < nScalar) {
@@ -334,7 +335,7 @@ __global__ void __launch_bounds__(kBlock) bcFlatKernel(const T *x, const T *y, T
     const Pack<T> *yv = reinterpret_cast<const Pack<T> *>(y);
     Pack<T> *zv = reinterpret_cast<Pack<T> *>(z);
     const bool pow2 = (vecsPerTad & (vecsPerTad - 1)) == 0;
-    for (Long j = (Long)blockIdx.x * kBlock + threadIdx.x; j < nvec; j += (Long)gridDim.x * kBlock) {
+    for (Long j = (Long)blockIdx.x * blockDim.x + threadIdx.x; j < nvec; j += (Long)gridDim.x * blockDim.x) {
         const Pack<T> a = loadPack(xv + j);
         unsigned col;
         if (pow2) col = (unsigned)j & (vecsPerTad - 1);  // the usual case: no division
@@ -706,7 +707,15 @@ inline void launchStrided(hipStream_t s, const T *x, Long xs, const T *y, Long y
             // one operand: two passes per thread (a little better for the functors with some arithmetic to overlap - tanh
             // 89 -> 82 us per 2^26 - and no worse for copies); with two operands one pass per thread stays the faster
             if (!two && !F::tables && grid > 2) grid = (grid + 1) / 2;
-            ND4J_LAUNCH((ewVecKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, two ? y : x, z, p, n, head,
+            // Two operands: blocks of 128 threads (z = x + y over 2^26 floats 123.6 -> 119.1 us against 256, the same with 64,
+            // 124.4 with 192; one-operand calls measure the same with either).  The kernel takes its block size from the
+            // launch; the functors that stage lookup tables keep the 256 threads their staging is written for.
+            int blk = kBlock;
+            if (two && !F::tables) {
+                blk = kBlock / 2;
+                grid = gridFor(nvec > 0 ? nvec : 1, (Long)blk, kMaxGrid);
+            }
+            ND4J_LAUNCH((ewVecKernel<T, F>), dim3(grid), dim3(blk), 0, s, x, two ? y : x, z, p, n, head,
                                (two && ys == 0) ? 1 : 0);
             return;
         }
