@@ -105,6 +105,47 @@ def test_transform_and_pairwise_on_views(gpu, cpu):
         assert ulp_distance(g, c).max() <= 2, vx[0]
 
 
+def test_rows_with_a_pitch(gpu, cpu):
+    """Matrices whose rows lie a pitch apart (different pitches for the operand and the result, row lengths that are and are
+    not multiples of the 16-byte vector, odd pitches that leave most rows off a 16-byte boundary): one-operand calls, calls
+    with a scalar and a row added to every row take the kernel written for this layout; two full operands keep the general
+    walk."""
+    rs = np.random.RandomState(211)
+    for dtype, tol in ((np.float32, 2), (np.float64, 2), (np.float16, None)):
+        for rows, cols, px, pz in ((37, 41, 45, 43), (64, 128, 132, 128), (5, 1030, 1032, 1040), (300, 8, 9, 12), (3, 3, 5, 4)):
+            xi = harness.shape_info([rows, cols], "c", strides=[px, 1])
+            zi = harness.shape_info([rows, cols], "c", strides=[pz, 1])
+            sel = _touched(zi)
+            x = rs.uniform(-3, 3, harness.span_of(xi)).astype(dtype)
+            y = rs.uniform(-3, 3, harness.span_of(xi)).astype(dtype)
+            row = rs.uniform(-3, 3, cols).astype(dtype)
+
+            def same(g, c, what):
+                if tol is None:
+                    g64, c64 = g[sel].astype(np.float64), c[sel].astype(np.float64)
+                    assert np.all(np.abs(g64 - c64) <= 1e-2 * np.maximum(np.abs(c64), 1e-2)), what
+                elif dtype == np.float32:
+                    assert ulp_distance(g[sel], c[sel]).max() <= tol, what
+                else:
+                    assert np.allclose(g[sel], c[sel], rtol=1e-14, atol=0), what
+                untouched = np.setdiff1d(np.arange(g.size), sel)
+                assert np.all(g[untouched] == 0), ("wrote outside the view", what)
+
+            case = (dtype.__name__, rows, cols, px, pz)
+            for op in (3, 6, 0):  # exp (lookup tables), neg, abs
+                same(gpu.transform(op, x, xi, zi), cpu.transform(op, x, xi, zi), case + ("transform", op))
+            same(gpu.scalar(0, x, xi, zi, 1.5), cpu.scalar(0, x, xi, zi, 1.5), case + ("scalar",))
+            same(gpu.pairwise(0, x, xi, y, xi, zi), cpu.pairwise(0, x, xi, y, xi, zi), case + ("pairwise",))
+            # (handed no tables for the result, the reference walks it with the operand's: its answer exists for equal pitches
+            # only; with different ones the sum itself is the check - one rounding in every type)
+            g, c = gpu.broadcast(0, x, xi, row, shape_info_np([1, cols]), xi, [1]), cpu.broadcast(0, x, xi, row, shape_info_np([1, cols]), xi, [1])
+            at = _touched(xi)
+            assert np.array_equal(g[at], c[at]) and np.all(g[np.setdiff1d(np.arange(g.size), at)] == 0), case + ("broadcast",)
+            g = gpu.broadcast(0, x, xi, row, shape_info_np([1, cols]), zi, [1])
+            assert np.array_equal(g[sel].reshape(rows, cols), x[at].reshape(rows, cols) + row[None, :]), case + ("broadcast, own pitch",)
+            assert np.all(g[np.setdiff1d(np.arange(g.size), sel)] == 0), case + ("broadcast, own pitch",)
+
+
 def test_pairwise_branches(gpu, cpu):
     rs = np.random.RandomState(22)
     # scalar y
