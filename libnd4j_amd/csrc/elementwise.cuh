@@ -635,9 +635,8 @@ __global__ void __launch_bounds__(kBlock) ewRunsKernel(const T *x, DimMap xm, co
 
 // The plainest of those views: a matrix whose rows lie a pitch apart, one run per row, the same for every operand (a
 // pitch of 0 repeats y's one row).  Unit g is vector g % unitsPerRun of row g / unitsPerRun: one multiplication in place of
-// a division and three pointer sums, a third of the instructions the general walk spends on a unit.  U units per thread
-// and round, all loads first.
-template <typename T, typename F, int U>
+// a division and three pointer sums, a third of the instructions the general walk spends on a unit.
+template <typename T, typename F>
 __global__ void __launch_bounds__(kBlock) ewPitchKernel(const T *x, Long px, const T *y, Long py, T *z, Long pz, Params<T> p,
                                                         unsigned total, unsigned runLength, FastDiv perRun) {
     typedef typename Compute<T>::type C;
@@ -645,47 +644,30 @@ __global__ void __launch_bounds__(kBlock) ewPitchKernel(const T *x, Long px, con
     constexpr bool two = F::nin == 2;
     if (F::tables) lm::loadTables();
     const unsigned step = gridDim.x * kBlock;
-    const bool shortRuns = runLength % VEC != 0;
-    unsigned g = blockIdx.x * kBlock + threadIdx.x;
-    while (g < total) {
-        const T *xp[U], *yp[U];
-        T *zp[U];
-        Pack<T> a[U], b[U];
-        unsigned count[U];
-        bool live[U];
+    const bool shortRuns = runLength % VEC != 0;  // some units hold fewer elements than a vector
+    for (unsigned g = blockIdx.x * kBlock + threadIdx.x; g < total;) {
+        unsigned c;
+        const unsigned r = perRun.divmod(g, c);
+        const unsigned first = c * VEC, count = runLength - first;
+        const T *xp = x + (Long)r * px + first;
+        const T *yp = two ? y + (Long)r * py + first : nullptr;
+        T *zp = z + (Long)r * pz + first;
+        if (!shortRuns || count >= (unsigned)VEC) {
+            const Pack<T> a = streamPackAnywhere(xp);
+            Pack<T> b;
+            if (two) b = loadPackAnywhere(yp);  // through the caches: a repeated row is read again and again
+            Pack<T> o;
 #pragma unroll
-        for (int k = 0; k < U; k++) {
-            live[k] = g < total;
-            // (a unit beyond the end re-reads the first one and is dropped: no load in a branch of its own)
-            unsigned c;
-            const unsigned r = perRun.divmod(live[k] ? g : 0, c);
-            const unsigned first = c * VEC;
-            count[k] = runLength - first;
-            xp[k] = x + (Long)r * px + first;
-            zp[k] = z + (Long)r * pz + first;
-            if (two) yp[k] = y + (Long)r * py + first;
-            if (!shortRuns || count[k] >= (unsigned)VEC) {
-                a[k] = streamPackAnywhere(xp[k]);
-                if (two) b[k] = loadPackAnywhere(yp[k]);  // through the caches: a repeated row is read again and again
-            }
-            const unsigned before = g;
-            g += step;
-            if (g < before) g = total;  // (the 32-bit sum wrapped round: past the end)
+            for (int e = 0; e < VEC; e++)
+                o.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), two ? toCompute(b.v[e]) : (C)0, p));
+            streamPackAnywhere(zp, o);
+        } else {
+            for (unsigned e = 0; e < count; e++)
+                zp[e] = fromCompute<T>(F::template apply<C>(toCompute(xp[e]), two ? toCompute(yp[e]) : (C)0, p));
         }
-#pragma unroll
-        for (int k = 0; k < U; k++) {
-            if (!live[k]) continue;
-            if (!shortRuns || count[k] >= (unsigned)VEC) {
-                Pack<T> o;
-#pragma unroll
-                for (int e = 0; e < VEC; e++)
-                    o.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a[k].v[e]), two ? toCompute(b[k].v[e]) : (C)0, p));
-                streamPackAnywhere(zp[k], o);
-            } else {
-                for (unsigned e = 0; e < count[k]; e++)
-                    zp[k][e] = fromCompute<T>(F::template apply<C>(toCompute(xp[k][e]), two ? toCompute(yp[k][e]) : (C)0, p));
-            }
-        }
+        const unsigned before = g;
+        g += step;
+        if (g < before) break;  // (the 32-bit sum wrapped round: past the end)
     }
 }
 
@@ -740,13 +722,15 @@ inline void launchRuns(hipStream_t s, const T *x, const DimMap &xm, const T *y, 
     constexpr int U = UNITS > 0 ? UNITS : ((OFFSETS || F::tables) ? 2 : 1);
     if (!OFFSETS && numTads == 1 && xOffsets == nullptr && zOffsets == nullptr) {
         // rows with a pitch, y (if any) one repeated row: the plain kernel (a row added to [65536, 1024] floats with a pitch of
-        // 1032: 69 -> 74 % of the HBM peak, exp over them 61 -> 63.5 %; with a y of rows of its own the general walk is
+        // 1032: 69 -> 74 % of the HBM peak, exp over them 61 -> 71.5 %; with a y of rows of its own the general walk is
         // ahead, 79 % against 77 %, and keeps the call)
         auto pitched = [&](const DimMap &m) { return m.rank == 2 && m.shape[1] == runLength && m.stride[1] == 1; };
         if (pitched(xm) && pitched(zm) && (F::nin != 2 || (pitched(ym) && ym.stride[0] == 0))) {
-            constexpr int PU = F::tables ? 2 : 1;
-            const unsigned grid = gridFor(units, kBlock * PU, F::tables ? kGridCap : kMaxGrid);
-            ND4J_LAUNCH((ewPitchKernel<T, F, PU>), dim3(grid), dim3(kBlock), 0, s, x, xm.stride[0], y, (Long)0, z, zm.stride[0], p,
+            // (functors with lookup tables on up to 24576 blocks, a thread going round for the rest: exp over the 2^26 floats
+            // of such rows 71.5 % of the HBM peak; 65 / 70 / 71.4 / 68.5 / 66 % on 8192 / 16384 / 32768 / 40960 / 49152 blocks,
+            // 58 % uncapped, 64-67 % with two units per thread and round)
+            const unsigned grid = gridFor(units, kBlock, F::tables ? 256 * 96 : kMaxGrid);
+            ND4J_LAUNCH((ewPitchKernel<T, F>), dim3(grid), dim3(kBlock), 0, s, x, xm.stride[0], y, (Long)0, z, zm.stride[0], p,
                         (unsigned)units, runLength, perRun);
             return;
         }
