@@ -278,8 +278,13 @@ void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Lon
         (siOrder(tx.hostInfo) == 'c' || dimLen == 1) && sameShape(hx, hz) && siNumel(hy) >= tx.tadLength &&
         siNumel(hx) <= 0x7fffffffLL && siRank(hx) <= kMaxDims) {
         const int rank = siRank(hx), tadRank = siRank(tx.hostInfo);
-        const Long *xs = siShape(hx), *xst = siStride(hx), *zst = siStride(hz);
+        // (without tables of its own the result is walked with x's, whatever its shapeInfo says: cpu/broadcasting.cpp:79-82;
+        // with them, its TADs must be the ones its own strides give along the same dimensions)
+        const bool ownTables = zOffsets != tx.devOffsets;
+        const Long *xs = siShape(hx), *xst = siStride(hx), *zst = ownTables ? siStride(hz) : xst;
         const Long *ts = siShape(tx.hostInfo), *tst = siStride(tx.hostInfo);
+        const Long *zts = siStride(zTadInfo);
+        bool zNatural = siRank(zTadInfo) == tadRank;
         Long ystr[kMaxDims];
         bool inTad[kMaxDims];
         int k = 0;
@@ -287,11 +292,12 @@ void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Lon
         for (int d = 0; d < rank; d++) {
             inTad[d] = xs[d] != 1 && k < tadRank && xs[d] == ts[k] && xst[d] == tst[k];
             if (inTad[d]) {
+                if (zNatural && (siShape(zTadInfo)[k] != ts[k] || zts[k] != zst[d])) zNatural = false;
                 k++;
                 while (k < tadRank && ts[k] == 1) k++;
             }
         }
-        if (k == tadRank) {
+        if (k == tadRank && zNatural) {
             Long inner = yLinear;
             for (int d = rank - 1; d >= 0; d--) {
                 ystr[d] = inTad[d] ? inner : 0;

@@ -144,6 +144,12 @@ def test_rows_with_a_pitch(gpu, cpu):
             g = gpu.broadcast(0, x, xi, row, shape_info_np([1, cols]), zi, [1])
             assert np.array_equal(g[sel].reshape(rows, cols), x[at].reshape(rows, cols) + row[None, :]), case + ("broadcast, own pitch",)
             assert np.all(g[np.setdiff1d(np.arange(g.size), sel)] == 0), case + ("broadcast, own pitch",)
+            if pz >= px:
+                # no tables for the result: it is walked with the operand's pitch, whatever its own shapeInfo says
+                # (cpu/broadcasting.cpp:79-82) - the reference's answer, every element of the buffer compared
+                g = gpu.broadcast(0, x, xi, row, shape_info_np([1, cols]), zi, [1], pass_tads=False)
+                c = cpu.broadcast(0, x, xi, row, shape_info_np([1, cols]), zi, [1])
+                assert np.array_equal(g, c), case + ("broadcast, no tables for the result",)
 
 
 def test_pairwise_branches(gpu, cpu):
