@@ -552,19 +552,20 @@ bool specialTransform(Nd4jPointer *extra, int opNum, T *x, const Long *hx, T *z,
         const bool rowMajor = pl.xEl == 1 && pl.zEl == 1 && (pl.length >= 16384 || (pl.length >= 4096 && pl.numRows <= 512));
         const bool colMajor = pl.xRow == 1 && pl.zRow == 1 && pl.numRows >= 256 && pl.length >= 256;
         if (rank >= 1 && (rowMajor || colMajor) && !softmaxFitsRegisters<T>(x, z, pl)) {
-            if (rowMajor) {
-                // aligned rows: one pass, the blocks of a row exchanging their maxima and sums
-                Scratch coop = scratchFor(s);
-                if (launchSoftmaxCooperative<T>(s, opNum, x, z, pl, coop.rest)) {
-                    checkLaunch("execTransform(softmax)", s);
-                    return true;
-                }
-            }
+            // (the rows' table is looked up before the one-pass kernel is tried, which does not need it: a stream under
+            // capture, where that kernel is not available, then finds the table its eager calls left in the cache)
             ResolvedTad tx;
             if (!resolveTad(nullptr, 0, 0, hx, &walked, 1, tx, s)) return true;
             typedef typename Compute<T>::type C;  // the row sums stay in the compute type: those of half rows may exceed half
             const size_t perRow = ((size_t)pl.numRows * sizeof(C) + 255) / 256 * 256;
-            Scratch sc = scratchFor(s, 2 * perRow + kWorkspaceBytes);
+            Scratch sc = scratchFor(s, 2 * perRow + kWorkspaceBytes);  // (sized for the two-pass form in either case, for the same reason)
+            if (rowMajor) {
+                // aligned rows: one pass, the blocks of a row exchanging their maxima and sums
+                if (launchSoftmaxCooperative<T>(s, opNum, x, z, pl, sc.rest)) {
+                    checkLaunch("execTransform(softmax)", s);
+                    return true;
+                }
+            }
             T *maxima = reinterpret_cast<T *>(sc.rest.ptr);
             C *sums = reinterpret_cast<C *>(reinterpret_cast<char *>(sc.rest.ptr) + perRow);
             Workspace rest;

@@ -95,9 +95,19 @@ void checkLaunch(const char *what, hipStream_t s) {
     }
 }
 
+bool streamIsCapturing(hipStream_t s) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return capture != hipStreamCaptureStatusNone;
+}
+
 void syncAndCheck(const char *what, hipStream_t s) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) throwHip(what, e);
+    if (streamIsCapturing(s)) return;  // nothing runs yet that could be waited for; the graph's launch is what the caller waits on
     e = hipStreamSynchronize(s);
     if (e != hipSuccess) throwHip(what, e);
 }
@@ -141,6 +151,11 @@ Workspace workspaceFor(hipStream_t s, size_t minBytes) {
     std::lock_guard<std::mutex> lock(gMutex);
     Workspace &w = gWorkspaces[std::make_pair(dev, s)];
     if (w.ptr != nullptr && w.bytes >= minBytes) return w;
+    // (allocating - and waiting for the stream before the old block is freed - is not something a stream under capture
+    // can do: say so, instead of leaving the capture broken by the calls below)
+    if (streamIsCapturing(s))
+        throw std::runtime_error("the stream is being captured and its workspace does not exist yet or is too small: make the "
+                                 "same call once on this stream before the capture begins");
     size_t want = minBytes < (size_t)(8u << 20) ? (size_t)(8u << 20) : minBytes;
     if (w.ptr != nullptr) {
         // earlier work on this stream may still use the old block
@@ -197,6 +212,11 @@ std::map<std::pair<int, hipStream_t>, FlatSlots> gFlatSlots;
 const unsigned kTicketPeriod = 1u << 30, kTicketMargin = 256;
 
 void addFlatSlots(Workspace &w, hipStream_t s) {
+    // A stream that is being captured into a graph gets no slots: the tickets that keep one launch's partial results apart
+    // from the next one's are drawn here, on the host, and a graph would replay the one it was captured with.  Without
+    // slots every caller takes its path of two launches (partial results in the workspace, merged by a second kernel),
+    // which replays like any other pair of kernels.
+    if (streamIsCapturing(s)) return;
     int dev = 0;
     (void)hipGetDevice(&dev);
     std::lock_guard<std::mutex> lock(gMutex);

@@ -78,6 +78,8 @@ Workspace workspaceFor(hipStream_t s, size_t minBytes);
 // (device, stream) that only those reductions use, cleared when it is allocated.  Calls on one stream run one after the
 // other, so they may share it (one host thread per stream: the ticket source is not synchronised).
 void addFlatSlots(Workspace &w, hipStream_t s);
+// true while `s` is being captured into a HIP graph
+bool streamIsCapturing(hipStream_t s);
 // 256 bytes of pinned, device-visible host memory per (device, stream): the kernels of the scalar-returning entry
 // points write their result there (plainly at offset 0, and as ticket-tagged words at offset 128), so the host reads
 // it without a copy.

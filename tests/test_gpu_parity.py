@@ -1299,6 +1299,83 @@ def test_elementwise_calls_in_a_captured_graph(gpu):
         dim.free()
 
 
+def test_reductions_in_a_captured_graph(gpu):
+    """Calls whose blocks exchange partial results (sums along the strided dimension, the whole-array sum left on the
+    device, argmax along dimension 0, SoftMax over long rows) keep their launches apart by tickets drawn on the host, which a
+    graph would replay; on a stream under capture they take their two-launch forms instead.  Captured after one eager pass,
+    replayed three times with new values: every replay against float64 numpy (1e-5; indices exactly)."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    dev, ops = gpu.dev, gpu.dev.ops
+    rs = np.random.RandomState(92)
+    rows, cols = 4096, 512
+    n = rows * cols
+    xi = shape_info_np([rows, cols])
+    li = shape_info_np([8, n // 8])  # the same buffer as eight long rows
+    X = harness.Operand(dev, rs.uniform(0.5, 1.5, n).astype(np.float32), xi)
+    XL = harness.Operand(dev, np.zeros(n, np.float32), li)
+    ci, ri, si = shape_info_np([1, cols]), shape_info_np([1, rows]), shape_info_np([1, 1])
+    S0, M1, A0 = (harness.Operand(dev, np.zeros(cols, np.float32), ci), harness.Operand(dev, np.zeros(rows, np.float32), ri),
+                  harness.Operand(dev, np.zeros(cols, np.float32), ci))
+    F = harness.Operand(dev, np.zeros(1, np.float32), si)
+    P = harness.Operand(dev, np.zeros(n, np.float32), li)
+    d0, d1 = dev.upload(np.array([0], np.int32)), dev.upload(np.array([1], np.int32))
+    ex0 = dev.extra(xi, z_info=ci, tad=dev.tad(xi, [0]))
+    ex1 = dev.extra(xi, z_info=ri, tad=dev.tad(xi, [1]))
+    exf = dev.extra(xi, z_info=si)
+    exl = dev.extra(li, z_info=li, tad=dev.tad(li, [1]))  # (with the row tables a host passes: building them would allocate)
+
+    def calls():
+        ops.execReduceFloat(ex0, 1, X.ptr, X.info_ptr, None, S0.ptr, S0.info_ptr, d0.ptr, 1)
+        ops.execReduceFloat(ex1, 3, X.ptr, X.info_ptr, None, M1.ptr, M1.info_ptr, d1.ptr, 1)
+        ops.execIndexReduceFloat(ex0, 0, X.ptr, X.info_ptr, None, A0.ptr, A0.info_ptr, d0.ptr, 1)
+        ops.execReduceFloatFull(exf, 1, X.ptr, X.info_ptr, None, F.ptr, F.info_ptr)
+        ops.execTransformFloat(exl, 38, X.ptr, XL.info_ptr, P.ptr, P.info_ptr, None)
+
+    def check(values, what):
+        v = values.astype(np.float64).reshape(rows, cols)
+        close = lambda g, e: np.all(np.abs(g.astype(np.float64) - e) <= 1e-5 * np.abs(e) + 1e-12)
+        assert close(S0.get(), v.sum(axis=0)), (what, "sum along dimension 0")
+        assert np.array_equal(M1.get(), values.reshape(rows, cols).max(axis=1)), (what, "max along dimension 1")
+        assert np.array_equal(A0.get(), np.argmax(v, axis=0).astype(np.float32)), (what, "argmax along dimension 0")
+        assert close(F.get(), np.array([v.sum()])), (what, "whole-array sum")
+        long = values.astype(np.float64).reshape(8, n // 8)
+        e = np.exp(long - long.max(axis=1, keepdims=True))
+        assert np.all(np.abs(P.get().reshape(8, n // 8) - e / e.sum(axis=1, keepdims=True)) <= 1e-5 * e / e.sum(axis=1, keepdims=True) + 1e-12), (what, "softmax")
+
+    first = X.get().copy()
+    calls()
+    dev.sync()
+    check(first, "eager")
+    stream = ctypes.c_void_p(dev.stream)
+    graph, executable = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 1) == 0  # 1: thread-local capture mode
+    try:
+        calls()
+    finally:
+        status = hip.hipStreamEndCapture(stream, ctypes.byref(graph))
+    assert status == 0 and graph.value
+    assert hip.hipGraphInstantiate(ctypes.byref(executable), graph, None, None, ctypes.c_size_t(0)) == 0
+    try:
+        for replay in range(3):
+            fresh = rs.uniform(0.5, 1.5, n).astype(np.float32)
+            ops.memcpy(X.ptr, fresh.ctypes.data, fresh.nbytes, 1, None)
+            for o in (S0, M1, A0, F):
+                ops.memset(o.ptr, 0, 4, 0, None)
+            dev.sync()
+            assert hip.hipGraphLaunch(executable, stream) == 0
+            dev.sync()
+            check(fresh, ("replay", replay))
+            calls()  # eager work between the replays, on its one-launch paths
+            dev.sync()
+            check(fresh, ("eager after replay", replay))
+    finally:
+        hip.hipGraphExecDestroy(executable)
+        hip.hipGraphDestroy(graph)
+        for o in (X, XL, S0, M1, A0, F, P, d0, d1):
+            o.free()
+
+
 def test_releasing_a_streams_resources(gpu):
     """A stream's workspace, exchange slots and pinned scalar block are freed on request and come back at the next call."""
     rs = np.random.RandomState(43)
