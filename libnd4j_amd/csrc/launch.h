@@ -83,6 +83,11 @@ struct TadPlan {
     DimMap tm;               // GENERAL
     unsigned runLength = 0;  // GENERAL: extent of the map's innermost dimension when its stride is 1 (contiguous runs), else 0
     const Long *offsets;     // device, numTads entries
+    // When the last dimension of x that the TADs do not take is its contiguous one: that dimension's extent (TADs
+    // t .. t + keptInner - 1, t a multiple of keptInner, then start on consecutive elements), and the greatest common
+    // divisor of x's other strides (what decides whether rows of such a group start on 16-byte boundaries).  0: not so.
+    unsigned keptInner = 0;
+    Long otherStrides = 0;
 };
 
 // Scratch for multi-block stages.  `bytes` is what the pointer is known to hold.

@@ -100,6 +100,35 @@ TadPlan tadPlanFrom(const ResolvedTad &t) {
     return pl;
 }
 
+// The dimensions of the TAD are found among x's by extent and stride, in order (extents of 1 take no part); what is left
+// are the dimensions that number the TADs, the last of them varying fastest.
+TadPlan tadPlanFrom(const ResolvedTad &t, const Long *hx) {
+    TadPlan pl = tadPlanFrom(t);
+    const int rank = siRank(hx), tadRank = siRank(t.hostInfo);
+    if (rank > kMaxDims) return pl;
+    const Long *xs = siShape(hx), *xst = siStride(hx), *ts = siShape(t.hostInfo), *tst = siStride(t.hostInfo);
+    bool inTad[kMaxDims];
+    int k = 0, last = -1;
+    while (k < tadRank && ts[k] == 1) k++;
+    for (int d = 0; d < rank; d++) {
+        inTad[d] = xs[d] != 1 && k < tadRank && xs[d] == ts[k] && xst[d] == tst[k];
+        if (inTad[d]) {
+            k++;
+            while (k < tadRank && ts[k] == 1) k++;
+        } else if (xs[d] != 1) last = d;
+    }
+    if (k != tadRank || last < 0 || xst[last] != 1 || xs[last] > 0x7fffffffLL) return pl;
+    Long g = 0;
+    for (int d = 0; d < rank; d++) {
+        if (d == last || xs[d] == 1) continue;
+        Long a = xst[d] < 0 ? -xst[d] : xst[d];
+        while (a != 0) { const Long r = g % a; g = a; a = r; }
+    }
+    pl.keptInner = (unsigned)xs[last];
+    pl.otherStrides = g;
+    return pl;
+}
+
 float halfBitsToFloatHost(unsigned short h) {
     unsigned sign = (h >> 15) & 1u, exp = (h >> 10) & 0x1fu, man = h & 0x3ffu;
     unsigned bits;
@@ -183,7 +212,7 @@ void reduceDims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params, T *
         return;
     }
     Scratch sc = scratchFor(s);
-    TadPlan pl = tadPlanFrom(t);
+    TadPlan pl = tadPlanFrom(t, hx);
     bool ok = true;
     if (opNum == 19) ok = launchReduceTad<T>(s, 3, x, params, z, pl, sc.rest);  // maxima into z first
     ok = ok && launchReduceTad<T>(s, opNum, x, params, z, pl, sc.rest);
@@ -232,7 +261,7 @@ void indexReduceDims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *params
         return;
     }
     Scratch sc = scratchFor(s);
-    TadPlan pl = tadPlanFrom(t);
+    TadPlan pl = tadPlanFrom(t, hx);
     if (!launchIndexReduceTad<T>(s, opNum, x, params, z, pl, sc.rest)) { reportUnknownOp("indexreduce", opNum); return; }
     checkLaunch("execIndexReduce", s);
 }
@@ -300,7 +329,7 @@ void statsDims(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *z, Long *zIn
         return;
     }
     Scratch sc = scratchFor(s);
-    TadPlan pl = tadPlanFrom(t);
+    TadPlan pl = tadPlanFrom(t, hx);
     // single-dimension TADs without an element-wise stride start from a zero sample in the reference
     // (cpu/summarystatsreduce.cpp:92-146, `comp.initWithValue(0.0)`)
     bool phantomZero = dimLen == 1 && siEws(t.hostInfo) < 1;

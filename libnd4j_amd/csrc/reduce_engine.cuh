@@ -556,6 +556,115 @@ __global__ void __launch_bounds__(BLK) tadColVecKernel(Pol pol, const typename P
     }
 }
 
+// Strided TADs of which only a few are neighbours in memory: the last dimension that is kept is the contiguous one and
+// short (`inner` elements, fewer than a wave's 64 vectors), as when the rows of the 56 x 56 planes of an image batch are
+// summed.  A wave of the kernel above would straddle several such groups with every load.  Here a block takes one group -
+// TADs a * inner .. a * inner + inner - 1 - and walks it plane by plane: thread = (row lane, vector of the row), so that what
+// the block has in flight is one contiguous stretch wherever the rows of a plane follow one another.  Row j of a TAD (j
+// counts the TAD's elements in C order) lies at outer(j / planeRows) + (j % planeRows) * rowStride, the map's innermost
+// dimension being the plane's rows.  Row ranges (blockIdx.y) leave their accumulators in partials[range * numTads + tad]
+// for tadColFinish.  Nothing is assumed about the offsets table beyond what the vector loads need, which is checked here:
+// a thread whose TADs are not neighbours, or not aligned, reads them element by element.
+__device__ __forceinline__ Long outerRowsOffset(const DimMap &m, unsigned idx) {
+    if (m.rank < 2) return 0;
+    Long off = 0;
+    for (int d = m.rank - 2; d > 0; d--) {
+        const unsigned q = idx / m.shape[d];
+        off += (Long)(idx - q * m.shape[d]) * m.stride[d];
+        idx = q;
+    }
+    return off + (Long)idx * m.stride[0];
+}
+template <class Pol>
+__global__ void __launch_bounds__(kBlock) tadPlaneKernel(Pol pol, const typename Pol::T *x, typename Pol::T *z,
+                                                        typename Pol::Acc *partials, const Long *offsets, Long tadLength,
+                                                        Long numTads, unsigned inner, unsigned groups, DimMap tm,
+                                                        FastDiv planeRows, Long rowStride, Long rowsPerSplit) {
+    if (Pol::tables) lm::loadTables();
+    typedef typename Pol::T T;
+    typedef typename Pol::Acc Acc;
+    constexpr int VEC = Pack<T>::N;
+    static_assert(sizeof(Acc) * kBlock * VEC <= 32768, "the merge area holds every thread's accumulators");
+    __shared__ Acc smem[kBlock * VEC];
+    const unsigned vpr = inner / VEC;           // vectors of a row
+    const unsigned lanes = kBlock / vpr;        // rows in flight per round
+    const unsigned cv = threadIdx.x % vpr, rl = threadIdx.x / vpr;
+    const bool active = rl < lanes;
+    const Long j0 = (Long)blockIdx.y * rowsPerSplit;
+    Long j1 = j0 + rowsPerSplit;
+    if (j1 > tadLength) j1 = tadLength;
+    auto rowAt = [&](Long j) -> Long {
+        unsigned ji;
+        const unsigned jo = planeRows.divmod((unsigned)j, ji);
+        return outerRowsOffset(tm, jo) + (Long)ji * rowStride;
+    };
+    for (unsigned a = blockIdx.x; a < groups; a += gridDim.x) {
+        const Long t0 = (Long)a * inner + (Long)cv * VEC;
+        Acc acc[VEC];
+        Pol pe[VEC];
+        if (active) {
+            Long off[VEC];
+            bool vec = true;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                off[e] = offsets[t0 + e];
+                pe[e] = pol;
+                pe[e].setTad(t0 + e, z);
+                acc[e] = pe[e].init(x + off[e]);
+                if (e > 0 && off[e] != off[0] + e) vec = false;
+            }
+            if ((reinterpret_cast<uintptr_t>(x + off[0]) & 15) != 0) vec = false;
+            if (vec) {
+                const T *base = x + off[0];
+                Long j = j0 + rl;
+                for (; j < j1; j += 4 * (Long)lanes) {
+                    Pack<T> pk[4];
+                    // (unconditional loads on clamped rows, the guard at the use: a load in a branch of its own would wait for
+                    // the loads before it)
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const Long ju = j + u * (Long)lanes;
+                        pk[u] = loadPack(reinterpret_cast<const Pack<T> *>(base + rowAt(ju < j1 ? ju : j1 - 1)));
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const Long ju = j + u * (Long)lanes;
+                        if (ju < j1) {
+#pragma unroll
+                            for (int e = 0; e < VEC; e++) foldNext(pe[e], acc[e], toCompute(pk[u].v[e]), ju);
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) pe[e].checkpoint(acc[e]);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
+                    const T *base = x + off[e];
+                    for (Long j = j0 + rl; j < j1; j += lanes) { foldNext(pe[e], acc[e], toCompute(base[rowAt(j)]), j); pe[e].checkpoint(acc[e]); }
+                }
+            }
+        }
+        // every TAD of the group is merged by a thread of its own, over the row lanes that hold a part of it
+        __syncthreads();  // (the area may still be read for the group before)
+        if (active) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) smem[threadIdx.x * VEC + e] = acc[e];
+        }
+        __syncthreads();
+        if (threadIdx.x < inner) {
+            const Long t = (Long)a * inner + threadIdx.x;
+            Pol pm = pol;
+            pm.setTad(t, z);
+            // (lanes beyond the range's rows hold fresh accumulators, which merge like any other)
+            Acc m = smem[threadIdx.x];  // row lane 0: thread cv, element e at cv * VEC + e
+            for (unsigned r = 1; r < lanes; r++) m = pm.combine(m, smem[(size_t)r * inner + threadIdx.x]);
+            if (gridDim.y == 1) z[t] = pm.finalize(m, tadLength);
+            else partials[(Long)blockIdx.y * numTads + t] = m;
+        }
+    }
+}
+
 // A few very long contiguous TADs: blockIdx.x is the TAD, blockIdx.y one slice of it; the slices' accumulators go to
 // partials[slice * numTads + tad] and are merged by tadColFinish.  (One block per TAD would leave most of the chip idle.)
 template <class Pol>
@@ -913,6 +1022,46 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
     // (the vector loads need every row of the TADs' common pitch to start on a 16-byte boundary: a pitch that is not a
     // multiple of the vector width goes to the lane-per-TAD kernel below, whose neighbouring lanes read neighbouring
     // elements)
+    {
+        // Strided TADs in groups of fewer neighbours than a wave has vectors, and at least ten rounds of rows for the block:
+        // the plane kernel.  In us against the kernels below - sums over dimensions {0,2} of [128,128,56,56]: 36.1 / 43.4, index
+        // of the maximum 40.3 / 52.8; sums over dimension 1 of [4096,128,100]: 33.8 / 41.1, of [6000,40,252]: 42.0 / 49.7, of
+        // [8,100000,32]: 22.9 / 28.8, of [4096,128,128]: 42.3 / 42.9.  Shorter ranges lose (three rounds, dimension 2 of the
+        // first array: 43.0 against 42.5 for sums, 79 against 47 for the index; two rounds, [4096,128,16]: 21 against 9), and
+        // so do the statistics' moments (66 against 53-60), whose merge is the expensive part: both stay below.
+        constexpr int VEC = Pack<typename Pol::T>::N;
+        const bool stridedTads = pl.kind == TadPlan::COL || (pl.kind == TadPlan::GENERAL && pl.runLength == 0 && pl.tm.rank >= 1);
+        if constexpr (sizeof(Acc) <= 16)
+        if (stridedTads && pl.keptInner >= 4u * VEC && pl.keptInner % VEC == 0 && pl.keptInner / VEC < (unsigned)kWave &&
+            pl.otherStrides % VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && pl.numTads % pl.keptInner == 0 &&
+            pl.tadLength <= 0x7fffffffLL) {
+            const unsigned lanes = kBlock / (pl.keptInner / VEC);
+            DimMap tm = pl.tm;
+            if (pl.kind == TadPlan::COL) { tm.rank = 1; tm.shape[0] = (unsigned)pl.tadLength; tm.stride[0] = pl.tadEws; }
+            const unsigned planeRows = tm.shape[tm.rank - 1];
+            const Long rowStride = tm.stride[tm.rank - 1];
+            if (pl.tadLength >= 10 * (Long)lanes && rowStride % VEC == 0) {
+                const Long groups = pl.numTads / pl.keptInner;
+                // about 2048 blocks, a range no shorter than four rounds of the block's row lanes, whole planes where it has several
+                Long splits = groups >= 2048 ? 1 : (2048 + groups - 1) / groups;
+                const Long maxByRows = pl.tadLength / (10 * (Long)lanes) > 1 ? pl.tadLength / (10 * (Long)lanes) : 1;
+                if (splits > maxByRows) splits = maxByRows;
+                if (splits > 65535) splits = 65535;
+                while (splits > 1 && (size_t)splits * (size_t)pl.numTads * sizeof(Acc) > ws.bytes) splits /= 2;
+                Long rowsPerSplit = (pl.tadLength + splits - 1) / splits;
+                if (rowsPerSplit > (Long)planeRows) rowsPerSplit = (rowsPerSplit + planeRows - 1) / planeRows * planeRows;
+                splits = (pl.tadLength + rowsPerSplit - 1) / rowsPerSplit;
+                Acc *partials = reinterpret_cast<Acc *>(ws.ptr);
+                const unsigned gx = (unsigned)(groups < (1 << 20) ? groups : (1 << 20));
+                ND4J_LAUNCH((tadPlaneKernel<Pol>), dim3(gx, (unsigned)splits), dim3(kBlock), 0, s, pol, x, z, partials, pl.offsets,
+                            pl.tadLength, pl.numTads, pl.keptInner, (unsigned)groups, tm, FastDiv(planeRows), rowStride, rowsPerSplit);
+                if (splits > 1)
+                    ND4J_LAUNCH((tadColFinish<Pol>), dim3((unsigned)((pl.numTads + kFinishLanes - 1) / kFinishLanes)), dim3(kBlock), 0, s,
+                                pol, z, partials, pl.tadLength, pl.numTads, (int)splits);
+                return;
+            }
+        }
+    }
     bool mappedVec = pl.kind == TadPlan::GENERAL && pl.runLength == 0 && pl.numTads >= 2 * kWave * Pack<typename Pol::T>::N &&
                      (reinterpret_cast<uintptr_t>(x) & 15) == 0;
     for (int d = 0; mappedVec && d < pl.tm.rank; d++) mappedVec = pl.tm.stride[d] % Pack<typename Pol::T>::N == 0;

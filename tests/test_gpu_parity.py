@@ -386,6 +386,34 @@ def test_strided_reductions_with_many_row_ranges(gpu, cpu):
         assert np.all(np.abs(var - truth) <= (1e-2 if dt == np.float16 else 1e-5) * np.maximum(truth, 1e-30)), what
 
 
+def test_strided_reductions_in_short_groups(gpu, cpu):
+    """TADs that are strided while the last dimension they leave out is the contiguous one and short (the rows of image
+    planes summed, a sequence pooled over time): groups of a few neighbouring TADs, walked plane by plane.  Shapes on both
+    sides of that kernel's conditions (range lengths, group widths, a pitch, one or several row ranges, three types)."""
+    rs = np.random.RandomState(331)
+    cases = (([12, 5, 30, 40], None, [0, 2]), ([16, 500, 24], None, [1]), ([2, 4000, 24], None, [1]), ([3, 700, 252], None, [1]),
+             ([16, 500, 24], [500 * 32, 32, 1], [1]), ([20, 5, 30, 40], None, [0, 2]), ([4, 90, 16], None, [1]), ([5, 2000, 20], None, [1]),
+             ([7, 3, 400, 8], None, [2]))
+    for dtype in (np.float32, np.float64, np.float16):
+        for shape, strides, dims in cases:
+            xi = harness.shape_info(shape, "c", strides=strides)
+            lo, hi = (0.5, 1.5) if dtype == np.float16 else (-2, 2)
+            x = rs.uniform(lo, hi, harness.span_of(xi)).astype(dtype)
+            out = int(np.prod([shape[d] for d in range(len(shape)) if d not in dims]))
+            case = (dtype.__name__, shape, strides, dims)
+            g, c = gpu.indexreduce(0, x, xi, None, dims, out), cpu.indexreduce(0, x, xi, None, dims, out)
+            assert np.array_equal(g, c), case + ("index of the maximum",)
+            assert np.array_equal(gpu.reduce(3, x, xi, None, dims, out), cpu.reduce(3, x, xi, None, dims, out)), case + ("max",)
+            g = gpu.reduce(1, x, xi, None, dims, out).astype(np.float64)
+            kept = [d for d in range(len(shape)) if d not in dims]
+            v = x[harness.element_offsets(xi)].astype(np.float64).reshape(shape)
+            exact = np.transpose(v, kept + list(dims)).reshape(out, -1)
+            tol = (1e-2 if dtype == np.float16 else 1e-5) * np.abs(exact).sum(axis=1)
+            assert np.all(np.abs(g - exact.sum(axis=1)) <= tol), case + ("sum",)
+            if dtype != np.float16:
+                assert np.allclose(gpu.reduce(0, x, xi, None, dims, out), cpu.reduce(0, x, xi, None, dims, out), rtol=1e-5, atol=1e-6), case + ("mean",)
+
+
 def test_broadcast_on_views_all_ops(gpu, cpu):
     rs = np.random.RandomState(27)
     for shape, order, dims in (([17, 33], "c", [1]), ([17, 33], "c", [0]), ([17, 33], "f", [0]), ([17, 33], "f", [1]),
