@@ -348,6 +348,34 @@ __global__ void __launch_bounds__(kBlock) bcFlatKernel(const T *x, const T *y, T
     }
 }
 
+// TADs over the outer and the inner part of a dense array [A, B, C] (dimensions {0, 2}): x and z are still one vector after
+// the other; vector j lies in row j / (C / VEC) of the [A * B, C] matrix, whose y row is that of a = row / B.  Two divisions
+// by multiplication per vector, no tables.  Needs C % VEC == 0, 16-byte aligned x, y, z and fewer than 2^31 vectors.
+template <typename T, typename F>
+__global__ void __launch_bounds__(kBlock) bcFlatSlabKernel(const T *x, const T *y, T *z, unsigned nvec, FastDiv vecsPerRow,
+                                                           FastDiv mid, Params<T> p) {
+    typedef typename Compute<T>::type C;
+    if (F::tables) lm::loadTables();
+    constexpr int VEC = Pack<T>::N;
+    const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x);
+    const Pack<T> *yv = reinterpret_cast<const Pack<T> *>(y);
+    Pack<T> *zv = reinterpret_cast<Pack<T> *>(z);
+    const unsigned step = gridDim.x * blockDim.x;
+    for (unsigned j = blockIdx.x * blockDim.x + threadIdx.x; j < nvec;) {
+        const Pack<T> a = loadPack(xv + j);
+        unsigned col;
+        const unsigned row = vecsPerRow.divmod(j, col);
+        const Pack<T> b = yv[(size_t)mid.div(row) * vecsPerRow.d + col];
+        Pack<T> r;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) r.v[e] = fromCompute<T>(F::template apply<C>(toCompute(a.v[e]), toCompute(b.v[e]), p));
+        storePack(zv + j, r);
+        const unsigned before = j;
+        j += step;
+        if (j < before) break;
+    }
+}
+
 // The same walk when the TAD length is not a multiple of the vector width (rows of odd length: only every fourth row
 // of a float matrix then starts on a 16-byte boundary): x and z are still one aligned vector after the other, and a
 // vector's elements take their y one by one, from the position inside the row where the vector begins, wrapping into

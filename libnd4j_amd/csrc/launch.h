@@ -53,6 +53,8 @@ struct BroadcastPlan {
     DimMap wx, wy, wz;
     Long wholeN = 0;
     unsigned wholeRun = 0;
+    // GENERAL: x and z are dense arrays [A, slabMid, slabInner] walked as plain vectors, y a dense [A, slabInner]
+    unsigned slabInner = 0, slabMid = 0;
     Long flatInner = 0, flatExtent = 0;  // per-TAD scalars over dense x and z of one layout: memory position i takes
                                          // scalars[(i / flatInner) % flatExtent]; 0 = not applicable
 };

@@ -274,7 +274,7 @@ void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Lon
     // TAD's dimensions when the TAD's order is 'c' (or it has one dimension).  The TAD's dimensions are found in x's by
     // extent and stride, in order (extents of 1 take no part); the result must be laid out over the same shape.
     const Long yLinear = pl.kind == BroadcastPlan::GENERAL ? (pl.ym.rank == 1 ? pl.ym.stride[0] : 0) : pl.yEws;
-    if (!pl.consecutive && !pl.denseAlike && pl.kind == BroadcastPlan::ROW && yLinear > 0 &&
+    if (!pl.consecutive && !pl.denseAlike && (pl.kind == BroadcastPlan::ROW || pl.kind == BroadcastPlan::GENERAL) && yLinear > 0 &&
         (siOrder(tx.hostInfo) == 'c' || dimLen == 1) && sameShape(hx, hz) && siNumel(hy) >= tx.tadLength &&
         siNumel(hx) <= 0x7fffffffLL && siRank(hx) <= kMaxDims) {
         const int rank = siRank(hx), tadRank = siRank(tx.hostInfo);
@@ -308,10 +308,21 @@ void broadcastShaped(Nd4jPointer *extra, int opNum, T *x, Long *xInfo, T *y, Lon
             jointCanon(rank, xs, strides, maps);
             const DimMap *const all[3] = {&maps[0], &maps[1], &maps[2]};
             const unsigned run = commonRunLength(all);
-            if (run >= 2) {
+            if (run >= 2 && pl.kind == BroadcastPlan::ROW) {
                 pl.wx = maps[0]; pl.wy = maps[1]; pl.wz = maps[2];
                 pl.wholeN = siNumel(hx);
                 pl.wholeRun = run;
+            } else if (pl.kind == BroadcastPlan::GENERAL && maps[0].rank == 3) {
+                // TADs over the outer and the inner part of a dense array ([A, B, C] along {0, 2}): x and z are plain vectors,
+                // and position i takes y[(i / (B * C)) * C + i % C]
+                const Long B = maps[0].shape[1], C = maps[0].shape[2];
+                bool slab = yLinear == 1 && siNumel(hy) == tx.tadLength;
+                for (int m = 0; m < 3 && slab; m += 2)
+                    slab = maps[m].stride[0] == B * C && maps[m].stride[1] == C && maps[m].stride[2] == 1;
+                if (slab && maps[1].stride[0] == C && maps[1].stride[1] == 0 && maps[1].stride[2] == 1) {
+                    pl.slabInner = (unsigned)C;
+                    pl.slabMid = (unsigned)B;
+                }
             }
         }
     }

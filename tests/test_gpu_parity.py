@@ -428,6 +428,26 @@ def test_broadcast_on_views_all_ops(gpu, cpu):
             assert ulp_distance(g, c).max() <= 2, (shape, order, dims, op)
 
 
+def test_broadcast_over_outer_and_inner_dimensions(gpu, cpu):
+    """y spans the outer and the inner part of a dense array ([A, B, C] along {0, 2}, [A, B, C, D] along {0, 2, 3}): inner
+    extents that are multiples of the 16-byte vector take a kernel of their own, the others the general ones; three types."""
+    rs = np.random.RandomState(341)
+    for dtype in (np.float32, np.float64, np.float16):
+        for shape, dims in (([6, 7, 8], [0, 2]), ([2, 3, 4, 8], [0, 2, 3]), ([5, 300, 64], [0, 2]), ([3, 9, 6], [0, 2]), ([4, 1, 16], [0, 2]),
+                            ([40, 33, 24], [0, 2])):
+            xi = harness.shape_info(shape, "c")
+            x = rs.uniform(1.5, 4, int(np.prod(shape))).astype(dtype)
+            yshape = [shape[d] for d in dims]
+            yi = harness.shape_info(yshape, "c")
+            y = rs.uniform(1.5, 4, int(np.prod(yshape))).astype(dtype)
+            for op in (0, 1, 2, 3):
+                g, c = gpu.broadcast(op, x, xi, y, yi, xi, dims), cpu.broadcast(op, x, xi, y, yi, xi, dims)
+                if dtype == np.float32:
+                    assert ulp_distance(g, c).max() <= 2, (shape, dims, op)
+                else:
+                    assert np.allclose(g.astype(np.float64), c.astype(np.float64), rtol=1e-2 if dtype == np.float16 else 1e-14, atol=0), (dtype.__name__, shape, dims, op)
+
+
 def test_scalar_family(gpu, cpu):
     from golden_inputs import SCALAR_OPS
     rs = np.random.RandomState(32)
