@@ -285,8 +285,9 @@ __global__ void __launch_bounds__(kBlock) concatKernel(const Long *const *infos,
                 const Pack<T> *xv = reinterpret_cast<const Pack<T> *>(x);
                 Pack<T> *zv = reinterpret_cast<Pack<T> *>(zb);
                 const bool small = (nv >> 32) == 0;
-                // a block moves four vectors per thread, all four loads in flight before the first store
-                constexpr int STEPS = 4;
+                // a block moves two vectors per thread, both loads in flight before the first store (eight inputs of 2^23 floats
+                // each: 90.1 us; 90.9 with four, 106.9 with one)
+                constexpr int STEPS = 2;
                 for (Long j0 = bx * (kBlock * STEPS) + threadIdx.x; j0 < nv; j0 += gdx * (kBlock * STEPS)) {
                     Pack<T> a[STEPS];
 #pragma unroll
@@ -440,10 +441,10 @@ void launchConcat(hipStream_t s, const T *const *data, const Long *const *infos,
     ConcatDesc *desc = reinterpret_cast<ConcatDesc *>(scratch);
     ND4J_LAUNCH(concatPrepareKernel, dim3(1), dim3(kBlock), 0, s, reinterpret_cast<const void *const *>(data), infos, n, v, desc);
     const int gy = n < 65535 ? n : 65535;
-    // four 16-byte vectors per thread while that keeps the grid below 2^22 blocks
+    // two 16-byte vectors per thread while that keeps the grid below 2^22 blocks
     int budget = (1 << 22) / gy;
     if (budget < 1) budget = 1;
-    const int gx = gridFor(maxLength > 0 ? maxLength : 1, (Long)kBlock * 4 * Pack<T>::N, budget);
+    const int gx = gridFor(maxLength > 0 ? maxLength : 1, (Long)kBlock * 2 * Pack<T>::N, budget);
     // Short runs (the inputs' slabs alternate in z every few KB): blocks that run together should fill neighbouring
     // runs, so the input index varies fastest.  Long runs: one input after the other.
     const bool inputFastest = v.dim > 0 && n > 1 && gx <= 65535;
@@ -502,14 +503,14 @@ template <typename S, typename D> __device__ __forceinline__ D convertOne(S v) {
 // Narrowing (or equal width): a thread converts 8 elements per pass, reading two or four 16-byte vectors and writing
 // one or two.  Widening: every store instruction should cover one contiguous stretch per wave (stores of 16 bytes
 // that alternate between the lanes' halves of 32-byte pieces were a third slower), so a thread converts the
-// 16 / sizeof(D) elements of ONE output vector per step and takes four steps a block-width apart.
+// 16 / sizeof(D) elements of ONE output vector per step and takes two steps a block-width apart.
 template <typename S, typename D>
 __global__ void __launch_bounds__(kBlock) convertKernel(const S *x, D *z, Long n, int vectors) {
     constexpr bool widening = sizeof(D) > sizeof(S);
     constexpr int E = widening ? 16 / (int)sizeof(D) : 8;
     const Long chunks = vectors ? n / E : 0;
     if (widening) {
-        constexpr int STEPS = 4;
+        constexpr int STEPS = 2;  // (half -> float over 2^26 elements: 65.6 us; 67.3 with four steps, 68.2 with one)
         typedef typename std::conditional<E * sizeof(S) == 8, unsigned long long, unsigned>::type Word;  // E source elements
         for (Long c0 = (Long)blockIdx.x * (kBlock * STEPS) + threadIdx.x; c0 < chunks; c0 += (Long)gridDim.x * (kBlock * STEPS)) {
             Word w[STEPS];
@@ -551,8 +552,8 @@ __global__ void __launch_bounds__(kBlock) convertKernel(const S *x, D *z, Long n
 template <typename S, typename D> void runConvert(hipStream_t s, const void *x, void *z, Long n) {
     if (n <= 0) return;
     const int vectors = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(z)) & 15) == 0 ? 1 : 0;
-    // elements per block and pass: 8 per thread when narrowing, four output vectors per thread when widening
-    const Long perBlock = sizeof(D) > sizeof(S) ? (Long)kBlock * 4 * (16 / (Long)sizeof(D)) : (Long)kBlock * 8;
+    // elements per block and pass: 8 per thread when narrowing, two output vectors per thread when widening
+    const Long perBlock = sizeof(D) > sizeof(S) ? (Long)kBlock * 2 * (16 / (Long)sizeof(D)) : (Long)kBlock * 8;
     ND4J_LAUNCH((convertKernel<S, D>), dim3(gridFor(n, perBlock, kMaxGrid)), dim3(kBlock), 0, s,
                        reinterpret_cast<const S *>(x), reinterpret_cast<D *>(z), n, vectors);
 }
