@@ -1042,8 +1042,12 @@ inline void runTadReduce(hipStream_t s, Pol pol, const typename Pol::T *x, typen
             const Long rowStride = tm.stride[tm.rank - 1];
             if (pl.tadLength >= 10 * (Long)lanes && rowStride % VEC == 0) {
                 const Long groups = pl.numTads / pl.keptInner;
-                // about 2048 blocks, a range no shorter than four rounds of the block's row lanes, whole planes where it has several
-                Long splits = groups >= 2048 ? 1 : (2048 + groups - 1) / groups;
+                // 512 blocks or more (1024 for index pairs), a range no shorter than ten rounds of the block's row lanes, whole planes
+                // where it has several
+                // (sums over {0,2} of [128,128,56,56] with 256 / 512 / 1024 / 2048 / 4096 blocks: 50.0 / 34.1 / 34.8 / 36.5 / 34.9 us; the
+                // index of the maximum: 61.5 / 41.0 / 38.6 / 39.9)
+                const Long tgt = sizeof(Acc) <= 8 ? 512 : 1024;
+                Long splits = groups >= tgt ? 1 : (tgt + groups - 1) / groups;
                 const Long maxByRows = pl.tadLength / (10 * (Long)lanes) > 1 ? pl.tadLength / (10 * (Long)lanes) : 1;
                 if (splits > maxByRows) splits = maxByRows;
                 if (splits > 65535) splits = 65535;
